@@ -1,0 +1,210 @@
+// C ABI of libdlspm_hip: argument validation, launch-shape selection and the device-side CSR check.
+// The entry points and what each one replaces in the reference are documented in include/dlspm_hip.h.
+#include "../../include/dlspm_hip.h"
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace dlspm {
+
+static thread_local int t_last_hip_error = 0;
+
+static int fail_hip(hipError_t e)
+{
+    t_last_hip_error = (int)e;
+    return DLSPM_E_LAUNCH;
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Optional launch-shape override for tuning sweeps: DLSPM_SPLIT="W,R" read once per process.
+static bool split_override(int& W, int& R)
+{
+    static const struct Ov {
+        bool on = false;
+        int W = 0, R = 0;
+        Ov()
+        {
+            const char* e = std::getenv("DLSPM_SPLIT");
+            if (e && std::sscanf(e, "%d,%d", &W, &R) == 2) on = true;
+        }
+    } ov;
+    if (ov.on) {
+        W = ov.W;
+        R = ov.R;
+    }
+    return ov.on;
+}
+
+void choose_split(int M, long long col_tiles, int nnz, int target, int max_w, int& W, int& R)
+{
+    static const int kPairs[][2] = {{4, 16}, {4, 8}, {4, 4}, {4, 2}, {4, 1}, {8, 4}, {8, 2}, {8, 1}, {16, 1}};
+    if (split_override(W, R)) {
+        for (const auto& pr : kPairs)
+            if (pr[0] == W && pr[1] == R && W <= max_w) return;
+    }
+    const double avg = M > 0 ? (double)nnz / M : 0.0;
+    double best = 1e300;
+    W = 4;
+    R = 4;
+    for (const auto& pr : kPairs) {
+        const int w = pr[0], r = pr[1];
+        if (w > max_w) continue;
+        const double per = avg * r / w;  // nonzeros per wave
+        double cost = per > target ? std::log2(per / target) : std::log2((target + 1.0) / (per + 1.0)) * 0.75;
+        const double blocks = (double)((M + r - 1) / r) * (double)col_tiles;
+        const double want = 1024.0;  // 4 workgroups per CU keeps every SIMD busy while others drain
+        if (blocks < want && (M + r - 1) / r < M) cost += 0.5 * std::log2(want / (blocks < 1 ? 1 : blocks));
+        cost += 0.05 * (w / 4);  // prefer fewer waves per workgroup when otherwise equal (cheaper barrier)
+        if (cost < best) {
+            best = cost;
+            W = w;
+            R = r;
+        }
+    }
+}
+
+// ---- device-side CSR check ------------------------------------------------------------------------
+// flag bits: 1 nnz > M*K | 2 row_offsets[M] != nnz | 4 offsets decrease | 8 row longer than K
+//            16 column >= K | 32 row_offsets[0] != 0 | 64 negative column
+__global__ void csr_check_kernel(int M, int K, int nnz, const int* __restrict__ row_offsets,
+                                 const int* __restrict__ col_indices, int* __restrict__ flags)
+{
+    const int tid = blockIdx.x * blockDim.x + threadIdx.x;
+    const int stride = gridDim.x * blockDim.x;
+    int f = 0;
+    if (tid == 0) {
+        if (row_offsets[M] != nnz) f |= 2;
+        if (row_offsets[0] != 0) f |= 32;
+    }
+    for (int i = tid; i < M; i += stride) {
+        const int lo = row_offsets[i], hi = row_offsets[i + 1];
+        if (hi < lo) f |= 4;
+        if (hi - lo > K) f |= 8;
+    }
+    if (!(f & 2)) {
+        for (int i = tid; i < nnz; i += stride) {
+            const int c = col_indices[i];
+            if (c >= K) f |= 16;
+            if (c < 0) f |= 64;
+        }
+    }
+    if (f) atomicOr(flags, f);
+}
+
+}  // namespace dlspm
+
+using namespace dlspm;
+
+extern "C" {
+
+int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int* col_indices, const float* values,
+                 const float* B, float* C, void* workspace, size_t workspace_bytes, void* stream)
+{
+    (void)workspace;
+    (void)workspace_bytes;
+    if (M < 0 || K < 0 || N < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
+    if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
+    if (M == 0 || N == 0) return DLSPM_OK;
+    if (!row_offsets || !C) return DLSPM_E_INVALID_ARG;
+    if (nnz > 0 && (!col_indices || !values || !B)) return DLSPM_E_INVALID_ARG;
+    const bool vec4 = (N % 4 == 0) && aligned16(B) && aligned16(C);
+    const SpmmShape shape = spmm_choose(M, N, nnz, vec4);
+    const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C};
+    const hipError_t e = spmm_launch(args, shape, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+}
+
+int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* lhs,
+                  const float* rhs, float* out_values, void* workspace, size_t workspace_bytes, void* stream)
+{
+    (void)workspace;
+    (void)workspace_bytes;
+    if (M < 0 || K < 0 || D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
+    if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
+    if (M == 0 || nnz == 0) return DLSPM_OK;
+    if (!row_offsets || !col_indices || !out_values) return DLSPM_E_INVALID_ARG;
+    if (D > 0 && (!lhs || !rhs)) return DLSPM_E_INVALID_ARG;  // D == 0: every dot product is the empty sum, 0
+    const bool vec4 = (D % 4 == 0) && D > 0 && aligned16(lhs) && aligned16(rhs);
+    const SddmmShape shape = sddmm_choose(M, D, nnz, vec4);
+    const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values};
+    const hipError_t e = sddmm_launch(args, shape, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+}
+
+int fused_sddmm_spmm_f32(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* Q,
+                         const float* Kmat, const float* V, float scale, float* O, void* workspace,
+                         size_t workspace_bytes, void* stream)
+{
+    (void)workspace;
+    (void)workspace_bytes;
+    if (M < 0 || K < 0 || D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
+    if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
+    if (M == 0 || D == 0) return DLSPM_OK;
+    if (!row_offsets || !O) return DLSPM_E_INVALID_ARG;
+    if (nnz > 0 && (!col_indices || !Q || !Kmat || !V)) return DLSPM_E_INVALID_ARG;
+    const bool vec4 = (D % 4 == 0) && aligned16(Q) && aligned16(Kmat) && aligned16(V) && aligned16(O);
+    const FusedShape shape = fused_choose(M, D, nnz, vec4);
+    const FusedArgs args{M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O};
+    const hipError_t e = fused_launch(args, shape, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+}
+
+size_t dlspm_workspace_bytes(int op, int M, int K, int N_or_D, int nnz)
+{
+    // The kernels split work inside each workgroup from row_offsets alone and keep partial sums in LDS,
+    // so no launch needs device scratch.
+    (void)op; (void)M; (void)K; (void)N_or_D; (void)nnz;
+    return 0;
+}
+
+int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* col_indices, void* stream)
+{
+    if (M < 0 || K < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
+    if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_CSR;
+    if (!row_offsets) return DLSPM_E_INVALID_ARG;
+    if (nnz > 0 && !col_indices) return DLSPM_E_INVALID_ARG;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int* d_flags = nullptr;
+    hipError_t e = hipMalloc(&d_flags, sizeof(int));
+    if (e != hipSuccess) return fail_hip(e);
+    int h_flags = 0;
+    e = hipMemsetAsync(d_flags, 0, sizeof(int), s);
+    if (e == hipSuccess) {
+        const long long work = (long long)(M > nnz ? M : nnz);
+        int blocks = (int)((work + 255) / 256);
+        blocks = blocks < 1 ? 1 : blocks > 2048 ? 2048 : blocks;
+        hipLaunchKernelGGL(csr_check_kernel, dim3(blocks), dim3(256), 0, s, M, K, nnz, row_offsets, col_indices, d_flags);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(&h_flags, d_flags, sizeof(int), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    (void)hipFree(d_flags);
+    if (e != hipSuccess) return fail_hip(e);
+    return h_flags == 0 ? DLSPM_OK : DLSPM_E_INVALID_CSR;
+}
+
+const char* dlspm_status_string(int status)
+{
+    switch (status) {
+        case DLSPM_OK: return "ok";
+        case DLSPM_E_INVALID_ARG: return "invalid argument (negative size, NULL operand, or nnz larger than M*K)";
+        case DLSPM_E_WORKSPACE: return "workspace too small or misaligned";
+        case DLSPM_E_LAUNCH: return "HIP runtime error at launch (see dlspm_last_hip_error)";
+        case DLSPM_E_INVALID_CSR: return "malformed CSR structure";
+        case DLSPM_E_NO_DEVICE: return "no gfx950 device is current";
+        default: return "unknown status";
+    }
+}
+
+int dlspm_last_hip_error(void) { return t_last_hip_error; }
+
+const char* dlspm_version(void) { return "dlspm_hip 0.1 gfx950"; }
+
+}  // extern "C"

@@ -1,0 +1,285 @@
+// Shared device helpers for the gfx950 sparse kernels: vector load/store types, cross-lane moves
+// (DPP inside 16-lane rows, ds_bpermute across rows) and the work split used by every kernel.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace dlspm {
+
+constexpr int kWave = 64;
+
+// ---- VEC floats per lane: dwordx4 (VEC = 4) or dword (VEC = 1) global accesses --------------------
+template <int VEC> struct Vec;
+template <> struct Vec<4> {
+    float4 v;
+    __device__ __forceinline__ static Vec zero() { return Vec{make_float4(0.f, 0.f, 0.f, 0.f)}; }
+    __device__ __forceinline__ static Vec load(const float* p) { return Vec{*reinterpret_cast<const float4*>(p)}; }
+    __device__ __forceinline__ void store(float* p) const { *reinterpret_cast<float4*>(p) = v; }
+    __device__ __forceinline__ void fma(float a, const Vec& b)
+    {
+        v.x = fmaf(a, b.v.x, v.x); v.y = fmaf(a, b.v.y, v.y); v.z = fmaf(a, b.v.z, v.z); v.w = fmaf(a, b.v.w, v.w);
+    }
+    __device__ __forceinline__ void add(const Vec& b) { v.x += b.v.x; v.y += b.v.y; v.z += b.v.z; v.w += b.v.w; }
+    __device__ __forceinline__ float dot(const Vec& b, float acc) const
+    {
+        acc = fmaf(v.x, b.v.x, acc); acc = fmaf(v.y, b.v.y, acc); acc = fmaf(v.z, b.v.z, acc); acc = fmaf(v.w, b.v.w, acc);
+        return acc;
+    }
+};
+template <> struct Vec<1> {
+    float v;
+    __device__ __forceinline__ static Vec zero() { return Vec{0.f}; }
+    __device__ __forceinline__ static Vec load(const float* p) { return Vec{*p}; }
+    __device__ __forceinline__ void store(float* p) const { *p = v; }
+    __device__ __forceinline__ void fma(float a, const Vec& b) { v = fmaf(a, b.v, v); }
+    __device__ __forceinline__ void add(const Vec& b) { v += b.v; }
+    __device__ __forceinline__ float dot(const Vec& b, float acc) const { return fmaf(v, b.v, acc); }
+};
+
+// ---- cross-lane ---------------------------------------------------------------------------------
+// value of `x` in lane `src` (any lane of the wave), through the LDS crossbar (ds_bpermute_b32)
+__device__ __forceinline__ int lane_get(int x, int src) { return __builtin_amdgcn_ds_bpermute(src << 2, x); }
+__device__ __forceinline__ float lane_get(float x, int src)
+{
+    return __int_as_float(__builtin_amdgcn_ds_bpermute(src << 2, __float_as_int(x)));
+}
+// wave-uniform source lane: v_readlane_b32 into an SGPR
+__device__ __forceinline__ int lane_bcast(int x, int src) { return __builtin_amdgcn_readlane(x, src); }
+__device__ __forceinline__ float lane_bcast(float x, int src)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), src));
+}
+
+// DPP move inside a 16-lane row; CTRL is the dpp_ctrl immediate
+template <int CTRL> __device__ __forceinline__ float dpp_move(float x)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true));
+}
+constexpr int kDppQuadSwap1 = 0xB1;      // quad_perm [1,0,3,2]: lane ^ 1
+constexpr int kDppQuadSwap2 = 0x4E;      // quad_perm [2,3,0,1]: lane ^ 2
+constexpr int kDppRowHalfMirror = 0x141; // lane i <-> 7 - i inside each group of 8
+constexpr int kDppRowMirror = 0x140;     // lane i <-> 15 - i inside each row of 16
+
+// Sum of x over aligned groups of G lanes, result in every lane of the group. G in {1,2,4,8,16,32,64}.
+// Steps up to 16 lanes are DPP (full VALU rate); 32 and 64 go through ds_bpermute.
+template <int G> __device__ __forceinline__ float group_sum(float x)
+{
+    if constexpr (G >= 2) x += dpp_move<kDppQuadSwap1>(x);
+    if constexpr (G >= 4) x += dpp_move<kDppQuadSwap2>(x);
+    if constexpr (G >= 8) x += dpp_move<kDppRowHalfMirror>(x);  // quads already uniform: mirror pairs quad 0 with quad 1
+    if constexpr (G >= 16) x += dpp_move<kDppRowMirror>(x);     // halves already uniform: mirror pairs the two halves
+    if constexpr (G >= 32) x += lane_get(x, (int)(threadIdx.x & 63) ^ 16);
+    if constexpr (G >= 64) x += lane_get(x, (int)(threadIdx.x & 63) ^ 32);
+    return x;
+}
+
+// ---- work split -----------------------------------------------------------------------------------
+// A workgroup of W waves owns a block of consecutive rows holding T nonzeros in all; wave w takes the
+// contiguous nonzero range [w*per, (w+1)*per) of them (clipped to T) regardless of row boundaries.
+__host__ __device__ __forceinline__ int split_per_wave(int T, int W)
+{
+    int per = (T + W - 1) / W;
+    return per < 1 ? 1 : per;
+}
+
+// ---- dense-row accumulation (SpMM kernel and stage 2 of the fused kernel) -----------------------------
+// The wave holds `cnt` <= 64 nonzeros of one row segment, one per lane: column index `c` and value `av`
+// (lanes >= cnt hold c = 0, av = 0). Adds sum_j av_j * dense[c_j, colv[v] .. colv[v]+VEC) into acc[v].
+// G lanes cover one dense row; the S = 64/G lane groups ("slots") take different nonzeros j = t*S + slot.
+// Loads are issued U dense rows at a time before the first FMA so that U*V requests per lane are in
+// flight. `colv` must be a valid column for every lane (lanes outside the matrix pass a safe column and
+// simply never store their accumulator), so the loop body has no predicates.
+template <int VEC, int G, int V>
+__device__ __forceinline__ void dense_rows_fma(Vec<VEC>* acc, int c, float av, int cnt, const float* __restrict__ dense,
+                                               int ld, const int* colv, int lane)
+{
+    using VecT = Vec<VEC>;
+    constexpr int S = kWave / G;
+    constexpr int U = V >= 4 ? 2 : 8 / V;
+    const int slot = lane / G;
+    const int full = cnt / S;  // steps in which every slot has a nonzero
+    int t = 0;
+    for (; t + U <= full; t += U) {
+        VecT bv[U][V];
+        float aj[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int cj;
+            if constexpr (S == 1) {
+                cj = lane_bcast(c, t + u);
+                aj[u] = lane_bcast(av, t + u);
+            } else {
+                cj = lane_get(c, (t + u) * S + slot);
+                aj[u] = lane_get(av, (t + u) * S + slot);
+            }
+            const float* row = dense + (size_t)cj * ld;
+#pragma unroll
+            for (int v = 0; v < V; ++v) bv[u][v] = VecT::load(row + colv[v]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int v = 0; v < V; ++v) acc[v].fma(aj[u], bv[u][v]);
+    }
+    if (t < full) {  // fewer than U steps left: same batching, each step guarded by a wave-uniform test
+        const int rem = full - t;
+        VecT bv[U - 1][V];
+        float aj[U - 1];
+#pragma unroll
+        for (int u = 0; u < U - 1; ++u) {
+            if (u < rem) {
+                int cj;
+                if constexpr (S == 1) {
+                    cj = lane_bcast(c, t + u);
+                    aj[u] = lane_bcast(av, t + u);
+                } else {
+                    cj = lane_get(c, (t + u) * S + slot);
+                    aj[u] = lane_get(av, (t + u) * S + slot);
+                }
+                const float* row = dense + (size_t)cj * ld;
+#pragma unroll
+                for (int v = 0; v < V; ++v) bv[u][v] = VecT::load(row + colv[v]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U - 1; ++u) {
+            if (u < rem) {
+#pragma unroll
+                for (int v = 0; v < V; ++v) acc[v].fma(aj[u], bv[u][v]);
+            }
+        }
+    }
+    if constexpr (S > 1) {
+        if (full * S < cnt) {  // last step: only the first cnt - full*S slots have a nonzero
+            const int jj = full * S + slot;
+            const int cj = lane_get(c, jj & 63);  // lanes >= cnt hold column 0: a valid row, result unused
+            const float aj = lane_get(av, jj & 63);
+            const float* row = dense + (size_t)cj * ld;
+            VecT bv[V];
+#pragma unroll
+            for (int v = 0; v < V; ++v) bv[v] = VecT::load(row + colv[v]);
+            if (jj < cnt) {
+#pragma unroll
+                for (int v = 0; v < V; ++v) acc[v].fma(aj, bv[v]);
+            }
+        }
+    }
+}
+
+// Adds the slots' partial sums so that every lane (in particular slot 0) ends with the total.
+template <int VEC, int G, int V> __device__ __forceinline__ void slots_sum(Vec<VEC>* acc, int lane)
+{
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+#pragma unroll
+        for (int step = G; step < kWave; step <<= 1) {
+            Vec<VEC> o;
+            if constexpr (VEC == 4) {
+                o.v.x = lane_get(acc[v].v.x, lane ^ step);
+                o.v.y = lane_get(acc[v].v.y, lane ^ step);
+                o.v.z = lane_get(acc[v].v.z, lane ^ step);
+                o.v.w = lane_get(acc[v].v.w, lane ^ step);
+            } else {
+                o.v = lane_get(acc[v].v, lane ^ step);
+            }
+            acc[v].add(o);
+        }
+    }
+}
+
+// ---- sampled dot products (SDDMM kernel and stage 1 of the fused kernel) -------------------------------
+// One round: the lane group handling nonzero `n` of the chunk (column index fetched from lane n) reads
+// that rhs row against the lhs row and returns the group's dot product in all of its lanes.
+// MASKED: D is not a multiple of G1*VEC*DS, lanes past D read a safe in-row address and contribute 0.
+template <int VEC, int G1, int DS, bool MASKED>
+__device__ __forceinline__ void sddmm_rounds_load(int D, int g, const float* __restrict__ rhs, int cn, Vec<VEC>* x)
+{
+    const float* rrow = rhs + (size_t)cn * D;
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+        const int d = (s * G1 + g) * VEC;
+        if constexpr (MASKED) {
+            x[s] = Vec<VEC>::load(rrow + (d < D ? d : 0));
+            if (d >= D) x[s] = Vec<VEC>::zero();  // not 0 * (whatever sits at column 0): that could be 0 * inf
+        } else {
+            x[s] = Vec<VEC>::load(rrow + d);
+        }
+    }
+}
+
+// One chunk of up to 64 nonzeros [base, q) of one row: returns in lane l the dot product of nonzero
+// base + l (lanes past the chunk return an unspecified value that the caller must not store).
+// `c` receives the lane's column index (0 past the chunk). `lq` holds the lhs row as laid out by the
+// caller: lq[s] = lhs_row[(s*G1 + g)*VEC ..], zero past D. With DS = 0 the row is re-read from lhs_row.
+template <int VEC, int G1, int DS, bool MASKED>
+__device__ __forceinline__ float sddmm_chunk(int D, int lane, int base, int q, const int* __restrict__ col_indices,
+                                             const float* __restrict__ lhs_row, const Vec<VEC>* lq,
+                                             const float* __restrict__ rhs, int& c)
+{
+    using VecT = Vec<VEC>;
+    constexpr int P = kWave / G1;  // nonzeros in flight per access
+    const int g = lane % G1;
+    const int grp = lane / G1;
+    const int idx = base + lane;
+    c = idx < q ? col_indices[idx] : 0;
+    const int cnt = min(kWave, q - base);
+    const int rounds = (cnt + P - 1) / P;  // <= G1
+    float res = 0.f;
+    if constexpr (DS > 0) {
+        constexpr int U = DS >= 8 ? 1 : 8 / DS;  // rounds whose loads are issued together
+        int t = 0;
+        for (; t + U <= rounds; t += U) {
+            VecT x[U][DS];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int cn = lane_get(c, ((t + u) * P + grp) & 63);
+                sddmm_rounds_load<VEC, G1, DS, MASKED>(D, g, rhs, cn, x[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float dot = 0.f;
+#pragma unroll
+                for (int s = 0; s < DS; ++s) dot = lq[s].dot(x[u][s], dot);
+                dot = group_sum<G1>(dot);
+                if (g == t + u) res = dot;  // lane grp*G1 + t keeps the result of nonzero t*P + grp
+            }
+        }
+        if constexpr (U > 1) {
+            if (t < rounds) {  // fewer than U rounds left: same batching under wave-uniform guards
+                const int rem = rounds - t;
+                VecT x[U - 1][DS];
+#pragma unroll
+                for (int u = 0; u < U - 1; ++u) {
+                    if (u < rem) {
+                        const int cn = lane_get(c, ((t + u) * P + grp) & 63);
+                        sddmm_rounds_load<VEC, G1, DS, MASKED>(D, g, rhs, cn, x[u]);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < U - 1; ++u) {
+                    if (u < rem) {
+                        float dot = 0.f;
+#pragma unroll
+                        for (int s = 0; s < DS; ++s) dot = lq[s].dot(x[u][s], dot);
+                        dot = group_sum<G1>(dot);
+                        if (g == t + u) res = dot;
+                    }
+                }
+            }
+        }
+    } else {
+        for (int t = 0; t < rounds; ++t) {
+            const int cn = lane_get(c, (t * P + grp) & 63);
+            const float* rrow = rhs + (size_t)cn * D;
+            float dot = 0.f;
+            for (int d = g * VEC; d < D; d += G1 * VEC) dot = VecT::load(lhs_row + d).dot(VecT::load(rrow + d), dot);
+            dot = group_sum<G1>(dot);
+            if (g == t) res = dot;
+        }
+    }
+    // transpose: lane l wants nonzero l, which sits in lane (l % P) * G1 + l / P
+    return lane_get(res, (lane % P) * G1 + lane / P);
+}
+
+}  // namespace dlspm

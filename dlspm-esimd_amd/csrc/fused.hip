@@ -1,0 +1,218 @@
+// Fused SDDMM -> SpMM, O[M x D] = (S .* (Q * Kmat^T) * scale) * V with S given as a CSR pattern, fp32, gfx950.
+//
+// Computes what Sddmm followed by Spmm compute in the reference's FUSED/fused.cpp:47-89 (with scale = 1)
+// and takes the place of its ESIMD kernel FusedEsimd (FUSED/fused-esimd_cb.cpp:100-189), which handles
+// one row per hardware thread and keeps 32 scores in a register vector between its two inner loops.
+// Here, per chunk of up to 64 nonzeros of a row segment:
+//   stage 1  the wave computes the 64 sampled scores exactly as the SDDMM kernel does (G1 lanes per dot
+//            product, DPP reduction, one transpose) and multiplies them by `scale`: lane l then holds the
+//            score and the column index of nonzero l in registers;
+//   stage 2  the same wave consumes them as the A-values of an SpMM step against V: G lanes cover one row
+//            of V with VEC*V2 floats each and the 64/G lane groups take different nonzeros, fetching score
+//            and column index from the owning lane by ds_bpermute.
+// The scores never leave the register file, so nothing of size nnz is written to or read from memory.
+// Work split, partial-sum handling for rows shared by several waves, and zero rows are as in the SpMM
+// kernel (per-wave partial sums in LDS, added in wave order after one barrier).
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace dlspm {
+
+template <int VEC, int G1, int DS, int G, int V2, int W, int R>
+__global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_tiles, float scale,
+                                                       const int* __restrict__ row_offsets,
+                                                       const int* __restrict__ col_indices,
+                                                       const float* __restrict__ Q, const float* __restrict__ Kmat,
+                                                       const float* __restrict__ Vmat, float* __restrict__ O)
+{
+    constexpr int S = kWave / G;
+    constexpr int TW = G * VEC * V2;
+    constexpr int NP = R == 1 ? 1 : 2;
+    using VecT = Vec<VEC>;
+
+    __shared__ int s_off[R + 1];
+    __shared__ float s_part[W][NP][TW];
+
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g1 = lane % G1;
+    const int g = lane % G;
+    const int slot = lane / G;
+    const int rb = blockIdx.x / col_tiles;
+    const int ct = blockIdx.x - rb * col_tiles;
+    const int r0 = rb * R;
+    const int nr = min(R, M - r0);
+
+    if ((int)threadIdx.x <= nr) s_off[threadIdx.x] = row_offsets[r0 + threadIdx.x];
+    __syncthreads();
+
+    int colv[V2];
+    bool act[V2];
+#pragma unroll
+    for (int v = 0; v < V2; ++v) {
+        const int col = ct * TW + (v * G + g) * VEC;
+        act[v] = col < D;
+        colv[v] = act[v] ? col : 0;
+    }
+    const bool exact = DS > 0 && D == G1 * VEC * DS;
+
+    const int T0 = s_off[0];
+    const int T = s_off[nr] - T0;
+    const int per = split_per_wave(T, W);
+    const int a = __builtin_amdgcn_readfirstlane(T0 + min(T, w * per));
+    const int b = __builtin_amdgcn_readfirstlane(T0 + min(T, (w + 1) * per));
+
+    if (a < b) {
+        int r = 0;
+        while (s_off[r + 1] <= a) ++r;
+        int pos = a;
+        while (pos < b) {
+            const int rs = s_off[r];
+            const int re = s_off[r + 1];
+            const int q = __builtin_amdgcn_readfirstlane(min(re, b));
+            const int p = __builtin_amdgcn_readfirstlane(pos);
+            const float* q_row = Q + (size_t)(r0 + r) * D;
+
+            VecT lq[DS > 0 ? DS : 1];
+            if constexpr (DS > 0) {
+#pragma unroll
+                for (int s = 0; s < DS; ++s) {
+                    const int d = (s * G1 + g1) * VEC;
+                    lq[s] = d < D ? VecT::load(q_row + d) : VecT::zero();
+                }
+            }
+            VecT acc[V2];
+#pragma unroll
+            for (int v = 0; v < V2; ++v) acc[v] = VecT::zero();
+
+            for (int base = p; base < q; base += kWave) {
+                int c;
+                // stage 1: lane l <- score of nonzero base + l (fp32, as between the reference's two loops)
+                float score =
+                    exact ? sddmm_chunk<VEC, G1, DS, false>(D, lane, base, q, col_indices, q_row, lq, Kmat, c)
+                          : sddmm_chunk<VEC, G1, DS, true>(D, lane, base, q, col_indices, q_row, lq, Kmat, c);
+                score = base + lane < q ? score * scale : 0.f;
+                // stage 2: acc += score_j * V[col_j, :]
+                dense_rows_fma<VEC, G, V2>(acc, c, score, min(kWave, q - base), Vmat, D, colv, lane);
+            }
+            if constexpr (S > 1) slots_sum<VEC, G, V2>(acc, lane);
+
+            const bool whole_row = (p == rs) && (q == re);
+            if (slot == 0) {
+                if (whole_row) {
+                    float* orow = O + (size_t)(r0 + r) * D;
+#pragma unroll
+                    for (int v = 0; v < V2; ++v)
+                        if (act[v]) acc[v].store(orow + colv[v]);
+                } else {
+                    float* part = s_part[w][(NP == 1 || p == a) ? 0 : 1];
+#pragma unroll
+                    for (int v = 0; v < V2; ++v) acc[v].store(part + (v * G + g) * VEC);
+                }
+            }
+            pos = q;
+            ++r;
+            while (r < nr && s_off[r + 1] <= pos) ++r;
+        }
+    }
+    __syncthreads();
+
+    if (slot == 0) {
+        for (int r = w; r < nr; r += W) {
+            const int rs = s_off[r];
+            const int re = s_off[r + 1];
+            float* orow = O + (size_t)(r0 + r) * D;
+            if (rs == re) {
+#pragma unroll
+                for (int v = 0; v < V2; ++v)
+                    if (act[v]) VecT::zero().store(orow + colv[v]);
+                continue;
+            }
+            const int wl = (rs - T0) / per;
+            const int wh = (re - 1 - T0) / per;
+            if (wl == wh) continue;
+#pragma unroll
+            for (int v = 0; v < V2; ++v) {
+                VecT sum = VecT::zero();
+                for (int x = wl; x <= wh; ++x) {
+                    const int k = (NP == 2 && x == wl && T0 + x * per != rs) ? 1 : 0;
+                    sum.add(VecT::load(&s_part[x][k][(v * G + g) * VEC]));
+                }
+                if (act[v]) sum.store(orow + colv[v]);
+            }
+        }
+    }
+}
+
+// ---- host side --------------------------------------------------------------------------------------
+
+template <int VEC, int G1, int DS, int G, int V2, int W, int R>
+static hipError_t launch_one(const FusedArgs& x, hipStream_t stream)
+{
+    constexpr int TW = G * VEC * V2;
+    const int col_tiles = (x.D + TW - 1) / TW;
+    const long long blocks = (long long)((x.M + R - 1) / R) * col_tiles;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream,
+                       x.M, x.D, col_tiles, x.scale, x.row_offsets, x.col_indices, x.Q, x.Kmat, x.V, x.O);
+    return hipGetLastError();
+}
+
+template <int VEC, int G1, int DS, int G, int V2>
+static hipError_t launch_wr(const FusedArgs& x, int W, int R, hipStream_t stream)
+{
+#define DLSPM_WR(w_, r_) \
+    if (W == w_ && R == r_) return launch_one<VEC, G1, DS, G, V2, w_, r_>(x, stream);
+    DLSPM_WR(4, 16)
+    DLSPM_WR(4, 8)
+    DLSPM_WR(4, 4)
+    DLSPM_WR(4, 2)
+    DLSPM_WR(4, 1)
+    if constexpr (G * VEC * V2 < 1024) {  // wider tiles: the per-wave partial sums of 8 or 16 waves do not fit in LDS
+        DLSPM_WR(8, 4)
+        DLSPM_WR(8, 2)
+        DLSPM_WR(8, 1)
+        DLSPM_WR(16, 1)
+    }
+#undef DLSPM_WR
+    return hipErrorInvalidValue;
+}
+
+FusedShape fused_choose(int M, int D, int nnz, bool vec4)
+{
+    FusedShape s{};
+    s.vec = vec4 ? 4 : 1;
+    if (vec4) {
+        if (D <= 16) { s.G1 = 4; s.DS = 1; s.G = 8; s.V = 1; }
+        else if (D <= 32) { s.G1 = 8; s.DS = 1; s.G = 8; s.V = 1; }
+        else if (D <= 64) { s.G1 = 8; s.DS = 2; s.G = 16; s.V = 1; }
+        else if (D <= 128) { s.G1 = 8; s.DS = 4; s.G = 32; s.V = 1; }
+        else if (D <= 256) { s.G1 = 8; s.DS = 8; s.G = 64; s.V = 1; }
+        else if (D <= 512) { s.G1 = 8; s.DS = 16; s.G = 64; s.V = 2; }
+        else { s.G1 = 8; s.DS = 0; s.G = 64; s.V = 4; }  // wider D: column tiles of 1024, scores recomputed per tile
+    } else {
+        s.G1 = 16; s.DS = 0; s.G = 64; s.V = 4;
+    }
+    const int tw = s.G * s.vec * s.V;
+    choose_split(M, (D + tw - 1) / tw, nnz, 64, tw >= 1024 ? 4 : 16, s.W, s.R);
+    return s;
+}
+
+hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream)
+{
+    if (s.vec == 4) {
+        if (s.G1 == 4 && s.DS == 1 && s.G == 8 && s.V == 1) return launch_wr<4, 4, 1, 8, 1>(x, s.W, s.R, stream);
+        if (s.G1 == 8 && s.DS == 1 && s.G == 8 && s.V == 1) return launch_wr<4, 8, 1, 8, 1>(x, s.W, s.R, stream);
+        if (s.G1 == 8 && s.DS == 2 && s.G == 16 && s.V == 1) return launch_wr<4, 8, 2, 16, 1>(x, s.W, s.R, stream);
+        if (s.G1 == 8 && s.DS == 4 && s.G == 32 && s.V == 1) return launch_wr<4, 8, 4, 32, 1>(x, s.W, s.R, stream);
+        if (s.G1 == 8 && s.DS == 8 && s.G == 64 && s.V == 1) return launch_wr<4, 8, 8, 64, 1>(x, s.W, s.R, stream);
+        if (s.G1 == 8 && s.DS == 16 && s.G == 64 && s.V == 2) return launch_wr<4, 8, 16, 64, 2>(x, s.W, s.R, stream);
+        if (s.G1 == 8 && s.DS == 0 && s.G == 64 && s.V == 4) return launch_wr<4, 8, 0, 64, 4>(x, s.W, s.R, stream);
+    } else if (s.G1 == 16 && s.DS == 0 && s.G == 64 && s.V == 4) {
+        return launch_wr<1, 16, 0, 64, 4>(x, s.W, s.R, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace dlspm

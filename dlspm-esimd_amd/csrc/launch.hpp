@@ -1,0 +1,58 @@
+// Argument bundles and launch-shape records shared by the kernel files and the C ABI layer.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace dlspm {
+
+// Lane layout and work split of one launch.
+//   vec : floats per lane per access (4 = dwordx4, 1 = dword)
+//   G   : lanes covering one dense row (SpMM / fused stage 2)          V  : accesses per lane per dense row
+//   G1  : lanes covering one dot product (SDDMM / fused stage 1)        DS : accesses per lane per dot
+//         product (0 = run-time loop, lhs row re-read instead of kept in registers)
+//   W   : waves per workgroup                                           R  : consecutive rows per workgroup
+struct SpmmShape { int vec, G, V, W, R; };
+struct SddmmShape { int vec, G1, DS, W, R; };
+struct FusedShape { int vec, G1, DS, G, V, W, R; };
+
+struct SpmmArgs {
+    int M, K, N, nnz;
+    const int* row_offsets;
+    const int* col_indices;
+    const float* values;
+    const float* B;
+    float* C;
+};
+struct SddmmArgs {
+    int M, K, D, nnz;
+    const int* row_offsets;
+    const int* col_indices;
+    const float* lhs;
+    const float* rhs;
+    float* out;
+};
+struct FusedArgs {
+    int M, K, D, nnz;
+    const int* row_offsets;
+    const int* col_indices;
+    const float* Q;
+    const float* Kmat;
+    const float* V;
+    float scale;
+    float* O;
+};
+
+SpmmShape spmm_choose(int M, int N, int nnz, bool vec4);
+hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
+
+SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4);
+hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t stream);
+
+FusedShape fused_choose(int M, int D, int nnz, bool vec4);
+hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream);
+
+// Picks (W, R), W <= max_w, so that a wave gets about `target` nonzeros and the grid stays wide enough for
+// 256 CUs. Only the pairs the kernels are instantiated for are returned.
+void choose_split(int M, long long col_tiles, int nnz, int target, int max_w, int& W, int& R);
+
+}  // namespace dlspm

@@ -1,0 +1,143 @@
+// CSR-sampled SDDMM, out[j] = <lhs[i, :], rhs[col[j], :]> for every slot j of CSR row i, fp32, gfx950.
+//
+// Computes what the reference's CPU loop Sddmm (SDDMM/sddmm-esimd-fromfile.cpp:18-36) computes and
+// takes the place of its ESIMD kernels (SDDMM/sddmm-esimd-fromfile.hpp:59-131 and the small-K variant
+// SDDMM/sddmm-esimd-fromfile_v4.hpp:102-177, which adds partial dot products with float atomics).
+// Here:
+//   * a workgroup of W waves owns R consecutive rows and splits their nonzeros evenly over its waves;
+//   * a wave keeps the lhs row of its current segment in registers (DS accesses of VEC floats per
+//     lane), reads 64 column indices with one coalesced load, and works on 64/G1 nonzeros at a time:
+//     G1 lanes read one rhs row (a full 128-byte line per group and access when G1 = 8, VEC = 4),
+//     multiply, and reduce with DPP inside their 16-lane row;
+//   * after up to G1 such rounds every lane holds one finished dot product; one ds_bpermute puts them
+//     in CSR order and one coalesced store writes 64 results straight into the sampled slots.
+// Every slot is written exactly once and no atomics are used, so the output needs no zeroing and is
+// deterministic. The CSR index arrays are only read.
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace dlspm {
+
+template <int VEC, int G1, int DS, int W, int R>
+__global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* __restrict__ row_offsets,
+                                                       const int* __restrict__ col_indices,
+                                                       const float* __restrict__ lhs, const float* __restrict__ rhs,
+                                                       float* __restrict__ out)
+{
+    using VecT = Vec<VEC>;
+    __shared__ int s_off[R + 1];
+
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = lane % G1;
+    const int r0 = blockIdx.x * R;
+    const int nr = min(R, M - r0);
+
+    if ((int)threadIdx.x <= nr) s_off[threadIdx.x] = row_offsets[r0 + threadIdx.x];
+    __syncthreads();
+
+    const int T0 = s_off[0];
+    const int T = s_off[nr] - T0;
+    const int per = split_per_wave(T, W);
+    const int a = __builtin_amdgcn_readfirstlane(T0 + min(T, w * per));
+    const int b = __builtin_amdgcn_readfirstlane(T0 + min(T, (w + 1) * per));
+    if (a >= b) return;
+    const bool exact = DS > 0 && D == G1 * VEC * DS;  // every lane's accesses fall inside the row
+
+    int r = 0;
+    while (s_off[r + 1] <= a) ++r;
+    int pos = a;
+    while (pos < b) {
+        const int q = __builtin_amdgcn_readfirstlane(min(s_off[r + 1], b));
+        const int p = __builtin_amdgcn_readfirstlane(pos);
+        const float* lhs_row = lhs + (size_t)(r0 + r) * D;
+
+        VecT lq[DS > 0 ? DS : 1];
+        if constexpr (DS > 0) {
+#pragma unroll
+            for (int s = 0; s < DS; ++s) {
+                const int d = (s * G1 + g) * VEC;
+                lq[s] = d < D ? VecT::load(lhs_row + d) : VecT::zero();
+            }
+        }
+        for (int base = p; base < q; base += kWave) {
+            int c;
+            const float o = exact ? sddmm_chunk<VEC, G1, DS, false>(D, lane, base, q, col_indices, lhs_row, lq, rhs, c)
+                                  : sddmm_chunk<VEC, G1, DS, true>(D, lane, base, q, col_indices, lhs_row, lq, rhs, c);
+            if (base + lane < q) out[base + lane] = o;
+        }
+        pos = q;
+        ++r;
+        while (r < nr && s_off[r + 1] <= pos) ++r;
+    }
+}
+
+// ---- host side --------------------------------------------------------------------------------------
+
+template <int VEC, int G1, int DS, int W, int R>
+static hipError_t launch_one(const SddmmArgs& x, hipStream_t stream)
+{
+    const int blocks = (x.M + R - 1) / R;
+    if (blocks <= 0) return hipSuccess;
+    hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M, x.D,
+                       x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
+    return hipGetLastError();
+}
+
+template <int VEC, int G1, int DS>
+static hipError_t launch_wr(const SddmmArgs& x, int W, int R, hipStream_t stream)
+{
+#define DLSPM_WR(w_, r_) \
+    if (W == w_ && R == r_) return launch_one<VEC, G1, DS, w_, r_>(x, stream);
+    DLSPM_WR(4, 16)
+    DLSPM_WR(4, 8)
+    DLSPM_WR(4, 4)
+    DLSPM_WR(4, 2)
+    DLSPM_WR(4, 1)
+    DLSPM_WR(8, 4)
+    DLSPM_WR(8, 2)
+    DLSPM_WR(8, 1)
+    DLSPM_WR(16, 1)
+#undef DLSPM_WR
+    return hipErrorInvalidValue;
+}
+
+SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4)
+{
+    SddmmShape s{};
+    s.vec = vec4 ? 4 : 1;
+    if (vec4) {
+        if (D <= 16) { s.G1 = 4; s.DS = 1; }
+        else {
+            s.G1 = 8;
+            s.DS = D <= 32 ? 1 : D <= 64 ? 2 : D <= 128 ? 4 : D <= 256 ? 8 : D <= 512 ? 16 : 0;
+        }
+    } else {
+        s.G1 = 16;
+        s.DS = 0;
+    }
+    choose_split(M, 1, nnz, 64, 16, s.W, s.R);
+    return s;
+}
+
+hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t stream)
+{
+    if (s.vec == 4) {
+        if (s.G1 == 4 && s.DS == 1) return launch_wr<4, 4, 1>(x, s.W, s.R, stream);
+        if (s.G1 == 8) {
+            switch (s.DS) {
+                case 1: return launch_wr<4, 8, 1>(x, s.W, s.R, stream);
+                case 2: return launch_wr<4, 8, 2>(x, s.W, s.R, stream);
+                case 4: return launch_wr<4, 8, 4>(x, s.W, s.R, stream);
+                case 8: return launch_wr<4, 8, 8>(x, s.W, s.R, stream);
+                case 16: return launch_wr<4, 8, 16>(x, s.W, s.R, stream);
+                case 0: return launch_wr<4, 8, 0>(x, s.W, s.R, stream);
+            }
+        }
+    } else if (s.G1 == 16 && s.DS == 0) {
+        return launch_wr<1, 16, 0>(x, s.W, s.R, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace dlspm

@@ -1,0 +1,206 @@
+// CSR SpMM, C[M x N] = A_csr[M x K] * B[K x N], fp32, for gfx950.
+//
+// Computes what the reference's CPU loop Spmm (SPMM/spmm-esimd-fromfile2.cpp:63-83) computes and takes
+// the place of its ESIMD kernel SpmmEsimd<CH> (SPMM/spmmesimd2.hpp:63-147). The decomposition is not
+// the reference's (one hardware thread per (row, CH-wide column slice), sized by an occupancy
+// heuristic): here
+//   * a workgroup of W waves owns R consecutive rows and splits the nonzeros of those rows evenly
+//     over its waves regardless of row boundaries (a merge-path split inside the row block), so a long
+//     row is shared by several waves and several short rows share one wave;
+//   * inside a wave, G lanes cover one row of B with VEC*V floats each (dwordx4 loads when VEC = 4),
+//     and the 64/G lane groups ("slots") work on different nonzeros of the same row segment at once;
+//   * a wave reads 64 (column, value) pairs with one coalesced load each and hands them out by
+//     v_readlane (G = 64) or ds_bpermute (G < 64), so the CSR arrays are read exactly once per column tile;
+//   * rows finished inside one wave are stored straight to C; rows shared by several waves leave
+//     per-wave partial sums in LDS which are added in wave order after one barrier, so the result does
+//     not depend on timing (no atomics, no pre-zeroed output); rows without nonzeros are written as 0.
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace dlspm {
+
+template <int VEC, int G, int V, int W, int R>
+__global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tiles,
+                                                      const int* __restrict__ row_offsets,
+                                                      const int* __restrict__ col_indices,
+                                                      const float* __restrict__ values,
+                                                      const float* __restrict__ B, float* __restrict__ C)
+{
+    constexpr int S = kWave / G;     // rows of B in flight per load instruction
+    constexpr int TW = G * VEC * V;  // columns of C covered by one wave
+    using VecT = Vec<VEC>;
+
+    __shared__ int s_off[R + 1];
+    constexpr int NP = R == 1 ? 1 : 2;  // with one row per workgroup a wave never ends a second segment
+    __shared__ float s_part[W][NP][TW];
+
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = lane % G;
+    const int slot = lane / G;
+    const int rb = blockIdx.x / col_tiles;
+    const int ct = blockIdx.x - rb * col_tiles;
+    const int r0 = rb * R;
+    const int nr = min(R, M - r0);
+
+    if ((int)threadIdx.x <= nr) s_off[threadIdx.x] = row_offsets[r0 + threadIdx.x];
+    __syncthreads();
+
+    int colv[V];  // first of this lane's VEC columns for access v; clamped to a valid column when outside
+    bool act[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        const int col = ct * TW + (v * G + g) * VEC;
+        act[v] = col < N;  // N % VEC == 0, so a lane's VEC columns are inside or outside together
+        colv[v] = act[v] ? col : 0;
+    }
+
+    const int T0 = s_off[0];
+    const int T = s_off[nr] - T0;
+    const int per = split_per_wave(T, W);
+    const int a = __builtin_amdgcn_readfirstlane(T0 + min(T, w * per));
+    const int b = __builtin_amdgcn_readfirstlane(T0 + min(T, (w + 1) * per));
+
+    if (a < b) {
+        int r = 0;
+        while (s_off[r + 1] <= a) ++r;  // first row owning nonzero `a`; exists because a < s_off[nr]
+        int pos = a;
+        while (pos < b) {
+            const int rs = s_off[r];
+            const int re = s_off[r + 1];
+            const int q = __builtin_amdgcn_readfirstlane(min(re, b));
+            const int p = __builtin_amdgcn_readfirstlane(pos);
+
+            VecT acc[V];
+#pragma unroll
+            for (int v = 0; v < V; ++v) acc[v] = VecT::zero();
+
+            for (int base = p; base < q; base += kWave) {
+                const int idx = base + lane;
+                int c = 0;
+                float av = 0.f;
+                if (idx < q) {
+                    c = col_indices[idx];
+                    av = values[idx];
+                }
+                dense_rows_fma<VEC, G, V>(acc, c, av, min(kWave, q - base), B, N, colv, lane);
+            }
+            if constexpr (S > 1) slots_sum<VEC, G, V>(acc, lane);
+
+            const bool whole_row = (p == rs) && (q == re);
+            if (slot == 0) {
+                if (whole_row) {
+                    float* crow = C + (size_t)(r0 + r) * N;
+#pragma unroll
+                    for (int v = 0; v < V; ++v)
+                        if (act[v]) acc[v].store(crow + colv[v]);
+                } else {
+                    float* part = s_part[w][(NP == 1 || p == a) ? 0 : 1];
+#pragma unroll
+                    for (int v = 0; v < V; ++v) acc[v].store(part + (v * G + g) * VEC);
+                }
+            }
+            pos = q;
+            ++r;
+            while (r < nr && s_off[r + 1] <= pos) ++r;  // skip rows without nonzeros
+        }
+    }
+    __syncthreads();
+
+    // rows shared by several waves: add the partial sums in wave order; empty rows: write zeros
+    if (slot == 0) {
+        for (int r = w; r < nr; r += W) {
+            const int rs = s_off[r];
+            const int re = s_off[r + 1];
+            float* crow = C + (size_t)(r0 + r) * N;
+            if (rs == re) {
+#pragma unroll
+                for (int v = 0; v < V; ++v)
+                    if (act[v]) VecT::zero().store(crow + colv[v]);
+                continue;
+            }
+            const int wl = (rs - T0) / per;
+            const int wh = (re - 1 - T0) / per;
+            if (wl == wh) continue;  // finished inside one wave, already stored
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                VecT sum = VecT::zero();
+                for (int x = wl; x <= wh; ++x) {
+                    const int k = (NP == 2 && x == wl && T0 + x * per != rs) ? 1 : 0;
+                    sum.add(VecT::load(&s_part[x][k][(v * G + g) * VEC]));
+                }
+                if (act[v]) sum.store(crow + colv[v]);
+            }
+        }
+    }
+}
+
+// ---- host side --------------------------------------------------------------------------------------
+
+template <int VEC, int G, int V, int W, int R>
+static hipError_t launch_one(const SpmmArgs& x, hipStream_t stream)
+{
+    constexpr int TW = G * VEC * V;
+    const int col_tiles = (x.N + TW - 1) / TW;
+    const long long blocks = (long long)((x.M + R - 1) / R) * col_tiles;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((spmm_kernel<VEC, G, V, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream, x.M, x.N,
+                       col_tiles, x.row_offsets, x.col_indices, x.values, x.B, x.C);
+    return hipGetLastError();
+}
+
+template <int VEC, int G, int V>
+static hipError_t launch_wr(const SpmmArgs& x, int W, int R, hipStream_t stream)
+{
+#define DLSPM_WR(w_, r_) \
+    if (W == w_ && R == r_) return launch_one<VEC, G, V, w_, r_>(x, stream);
+    DLSPM_WR(4, 16)
+    DLSPM_WR(4, 8)
+    DLSPM_WR(4, 4)
+    DLSPM_WR(8, 4)
+    DLSPM_WR(8, 2)
+    DLSPM_WR(8, 1)
+    DLSPM_WR(16, 1)
+    DLSPM_WR(4, 2)
+    DLSPM_WR(4, 1)
+#undef DLSPM_WR
+    return hipErrorInvalidValue;
+}
+
+// Chooses the lane layout from N and the (W, R) split from the mean row length.
+SpmmShape spmm_choose(int M, int N, int nnz, bool vec4)
+{
+    SpmmShape s{};
+    s.vec = vec4 ? 4 : 1;
+    if (vec4) {
+        if (N > 256) { s.G = 64; s.V = 2; }
+        else if (N > 128) { s.G = 64; s.V = 1; }
+        else if (N > 64) { s.G = 32; s.V = 1; }
+        else if (N > 32) { s.G = 16; s.V = 1; }
+        else { s.G = 8; s.V = 1; }
+    } else {
+        s.G = 64;
+        s.V = N > 64 ? 4 : 1;
+    }
+    const int tw = s.G * s.vec * s.V;
+    choose_split(M, (N + tw - 1) / tw, nnz, 32, 16, s.W, s.R);
+    return s;
+}
+
+hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream)
+{
+    if (s.vec == 4) {
+        if (s.G == 64 && s.V == 1) return launch_wr<4, 64, 1>(x, s.W, s.R, stream);
+        if (s.G == 64 && s.V == 2) return launch_wr<4, 64, 2>(x, s.W, s.R, stream);
+        if (s.G == 32 && s.V == 1) return launch_wr<4, 32, 1>(x, s.W, s.R, stream);
+        if (s.G == 16 && s.V == 1) return launch_wr<4, 16, 1>(x, s.W, s.R, stream);
+        if (s.G == 8 && s.V == 1) return launch_wr<4, 8, 1>(x, s.W, s.R, stream);
+    } else {
+        if (s.G == 64 && s.V == 1) return launch_wr<1, 64, 1>(x, s.W, s.R, stream);
+        if (s.G == 64 && s.V == 4) return launch_wr<1, 64, 4>(x, s.W, s.R, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace dlspm

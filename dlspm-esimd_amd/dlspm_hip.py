@@ -1,0 +1,283 @@
+"""ctypes binding of libdlspm_hip.so (the C ABI declared in include/dlspm_hip.h) for the Python tests and the
+benchmark. PyTorch is used for device memory and the stream only; every computation happens inside the
+library's HIP kernels. There is no fallback: if the shared library is missing or a call fails, an exception
+is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdlspm_hip.so")
+GEN_LIB_PATH = os.path.join(_HERE, "libdlspm_gen.so")
+
+OK = 0
+E_INVALID_ARG = -1
+E_WORKSPACE = -2
+E_LAUNCH = -3
+E_INVALID_CSR = -4
+E_NO_DEVICE = -5
+
+OP_SPMM, OP_SDDMM, OP_FUSED = 0, 1, 2
+
+EXPORTS = (
+    "spmm_csr_f32",
+    "sddmm_csr_f32",
+    "fused_sddmm_spmm_f32",
+    "dlspm_workspace_bytes",
+    "dlspm_csr_check",
+    "dlspm_status_string",
+    "dlspm_last_hip_error",
+    "dlspm_version",
+)
+
+
+class DlspmError(RuntimeError):
+    def __init__(self, status: int, where: str):
+        self.status = status
+        super().__init__(f"{where}: status {status} ({status_string(status)}), hip error {lib().dlspm_last_hip_error()}")
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded libdlspm_hip.so. Raises if it has not been built (run `make -C dlspm-esimd_amd lib`)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(f"{LIB_PATH} is missing: build it with `make -C {_HERE} lib` (hipcc, gfx950)")
+        L = ctypes.CDLL(LIB_PATH)
+        vp, ci, cf, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+        L.spmm_csr_f32.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.spmm_csr_f32.restype = ci
+        L.sddmm_csr_f32.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.sddmm_csr_f32.restype = ci
+        L.fused_sddmm_spmm_f32.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, cf, vp, vp, sz, vp]
+        L.fused_sddmm_spmm_f32.restype = ci
+        L.dlspm_workspace_bytes.argtypes = [ci, ci, ci, ci, ci]
+        L.dlspm_workspace_bytes.restype = sz
+        L.dlspm_csr_check.argtypes = [ci, ci, ci, vp, vp, vp]
+        L.dlspm_csr_check.restype = ci
+        L.dlspm_status_string.argtypes = [ci]
+        L.dlspm_status_string.restype = ctypes.c_char_p
+        L.dlspm_last_hip_error.restype = ci
+        L.dlspm_version.restype = ctypes.c_char_p
+        _lib = L
+    return _lib
+
+
+def status_string(status: int) -> str:
+    return lib().dlspm_status_string(status).decode()
+
+
+def version() -> str:
+    return lib().dlspm_version().decode()
+
+
+def _ptr(t, dtype, name):
+    import torch
+
+    if t is None:
+        return None
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError(f"{name} must be a device tensor")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous (row-major)")
+    return ctypes.c_void_p(t.data_ptr()) if t.numel() > 0 else None
+
+
+def _stream():
+    import torch
+
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def spmm(row_offsets, col_indices, values, B, K=None, out=None):
+    """C = A_csr @ B on the current stream. row_offsets/col_indices int32, values/B float32, all on the GPU."""
+    import torch
+
+    M = row_offsets.numel() - 1
+    nnz = col_indices.numel()
+    Kd, N = B.shape
+    K = Kd if K is None else K
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=B.device)
+    st = lib().spmm_csr_f32(M, K, N, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
+                            _ptr(col_indices, torch.int32, "col_indices"), _ptr(values, torch.float32, "values"),
+                            _ptr(B, torch.float32, "B"), _ptr(out, torch.float32, "C"), None, 0, _stream())
+    if st != OK:
+        raise DlspmError(st, "spmm_csr_f32")
+    return out
+
+
+def sddmm(row_offsets, col_indices, lhs, rhs, out=None):
+    """out[j] = <lhs[i], rhs[col[j]]> for each CSR slot j of row i, on the current stream."""
+    import torch
+
+    M = row_offsets.numel() - 1
+    nnz = col_indices.numel()
+    K, D = rhs.shape
+    if out is None:
+        out = torch.empty((nnz,), dtype=torch.float32, device=lhs.device)
+    st = lib().sddmm_csr_f32(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
+                             _ptr(col_indices, torch.int32, "col_indices"), _ptr(lhs, torch.float32, "lhs"),
+                             _ptr(rhs, torch.float32, "rhs"), _ptr(out, torch.float32, "out"), None, 0, _stream())
+    if st != OK:
+        raise DlspmError(st, "sddmm_csr_f32")
+    return out
+
+
+def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None):
+    """O = (S .* (Q Kmat^T) * scale) V on the current stream; the scores are never stored."""
+    import torch
+
+    M = row_offsets.numel() - 1
+    nnz = col_indices.numel()
+    K, D = Kmat.shape
+    if out is None:
+        out = torch.empty((M, D), dtype=torch.float32, device=Q.device)
+    st = lib().fused_sddmm_spmm_f32(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
+                                    _ptr(col_indices, torch.int32, "col_indices"), _ptr(Q, torch.float32, "Q"),
+                                    _ptr(Kmat, torch.float32, "Kmat"), _ptr(V, torch.float32, "V"),
+                                    ctypes.c_float(scale), _ptr(out, torch.float32, "O"), None, 0, _stream())
+    if st != OK:
+        raise DlspmError(st, "fused_sddmm_spmm_f32")
+    return out
+
+
+def csr_check(M, K, row_offsets, col_indices) -> int:
+    """Status of the device-side CSR check (OK or E_INVALID_CSR); synchronises the current stream."""
+    import torch
+
+    nnz = col_indices.numel()
+    return int(lib().dlspm_csr_check(M, K, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
+                                     _ptr(col_indices, torch.int32, "col_indices"), _stream()))
+
+
+# ------------------------------------------------------------------------------------------------------
+# seeded inputs (libdlspm_gen.so): the same generators the C++ drivers use
+# ------------------------------------------------------------------------------------------------------
+_gen = None
+
+
+def gen_lib() -> ctypes.CDLL:
+    global _gen
+    if _gen is None:
+        if not os.path.exists(GEN_LIB_PATH):
+            raise FileNotFoundError(f"{GEN_LIB_PATH} is missing: build it with `make -C {_HERE} gen`")
+        G = ctypes.CDLL(GEN_LIB_PATH)
+        vp, ci = ctypes.c_void_p, ctypes.c_int
+        G.dlspm_gen_config_create.argtypes = [ci]
+        G.dlspm_gen_config_create.restype = vp
+        G.dlspm_gen_config_destroy.argtypes = [vp]
+        G.dlspm_gen_config_dims.argtypes = [vp, ctypes.POINTER(ci), ctypes.POINTER(ctypes.c_float)]
+        G.dlspm_gen_config_name.argtypes = [ci]
+        G.dlspm_gen_config_name.restype = ctypes.c_char_p
+        for f in ("row_offsets", "col_indices", "values"):
+            getattr(G, "dlspm_gen_config_" + f).argtypes = [vp]
+            getattr(G, "dlspm_gen_config_" + f).restype = vp
+        G.dlspm_gen_config_dense.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_size_t)]
+        G.dlspm_gen_config_dense.restype = vp
+        G.dlspm_gen_pattern_create.argtypes = [ci, ctypes.c_uint64, ci, ci, ctypes.c_double, ctypes.c_double]
+        G.dlspm_gen_pattern_create.restype = vp
+        G.dlspm_gen_pattern_destroy.argtypes = [vp]
+        G.dlspm_gen_pattern_nnz.argtypes = [vp]
+        G.dlspm_gen_pattern_nnz.restype = ci
+        G.dlspm_gen_pattern_copy.argtypes = [vp, vp, vp]
+        G.dlspm_gen_fill_uniform.argtypes = [ctypes.c_uint64, ctypes.c_size_t, ctypes.c_float, ctypes.c_float, vp]
+        G.dlspm_gen_fill_normal.argtypes = [ctypes.c_uint64, ctypes.c_size_t, ctypes.c_float, ctypes.c_float, vp]
+        G.dlspm_gen_fill_relu_like.argtypes = [ctypes.c_uint64, ctypes.c_size_t, ctypes.c_double, vp]
+        G.dlspm_account.argtypes = [ci] + [ctypes.c_double] * 4 + [ctypes.POINTER(ctypes.c_double)]
+        _gen = G
+    return _gen
+
+
+PATTERN_UNIFORM_ROWS, PATTERN_LOGNORMAL_ROWS, PATTERN_BERNOULLI, PATTERN_BAND_RANDOM = 0, 1, 2, 3
+
+
+def make_pattern(kind: int, seed: int, M: int, K: int, p0: float, p1: float = 0.0):
+    """(row_offsets, col_indices) as numpy int32 arrays from one of the seeded pattern generators."""
+    import numpy as np
+
+    G = gen_lib()
+    h = G.dlspm_gen_pattern_create(kind, seed, M, K, p0, p1)
+    if not h:
+        raise ValueError(f"unknown pattern kind {kind}")
+    try:
+        nnz = G.dlspm_gen_pattern_nnz(h)
+        ro = np.empty(M + 1, dtype=np.int32)
+        ci = np.empty(max(nnz, 1), dtype=np.int32)
+        G.dlspm_gen_pattern_copy(h, ro.ctypes.data, ci.ctypes.data)
+        return ro, ci[:nnz]
+    finally:
+        G.dlspm_gen_pattern_destroy(h)
+
+
+def fill(kind: str, seed: int, shape, a: float = 0.0, b: float = 1.0):
+    """Seeded float32 numpy array: kind 'uniform' (a = lo, b = hi), 'normal' (a = mean, b = std), 'relu' (a = p_zero)."""
+    import numpy as np
+
+    G = gen_lib()
+    out = np.empty(shape, dtype=np.float32)
+    if kind == "uniform":
+        G.dlspm_gen_fill_uniform(seed, out.size, a, b, out.ctypes.data)
+    elif kind == "normal":
+        G.dlspm_gen_fill_normal(seed, out.size, a, b, out.ctypes.data)
+    elif kind == "relu":
+        G.dlspm_gen_fill_relu_like(seed, out.size, a, out.ctypes.data)
+    else:
+        raise ValueError(kind)
+    return out
+
+
+def make_config(cfg: int) -> dict:
+    """Benchmark configuration cfg (1..5) as numpy arrays:
+    {'cfg','name','op','M','K','N','nnz','scale','row_offsets','col_indices','values','d0','d1','d2'}."""
+    import numpy as np
+
+    G = gen_lib()
+    h = G.dlspm_gen_config_create(cfg)
+    if not h:
+        raise ValueError(f"unknown configuration {cfg}")
+    try:
+        dims = (ctypes.c_int * 5)()
+        scale = ctypes.c_float()
+        G.dlspm_gen_config_dims(h, dims, ctypes.byref(scale))
+        op, M, K, N, nnz = (int(x) for x in dims)
+
+        def arr(ptr, n, dtype):
+            if n == 0 or not ptr:
+                return np.empty(0, dtype=dtype)
+            ctype = ctypes.c_int if dtype == np.int32 else ctypes.c_float
+            return np.ctypeslib.as_array(ctypes.cast(ptr, ctypes.POINTER(ctype)), shape=(n,)).copy()
+
+        out = {
+            "cfg": cfg, "name": G.dlspm_gen_config_name(cfg).decode(), "op": op, "M": M, "K": K, "N": N, "nnz": nnz,
+            "scale": float(scale.value),
+            "row_offsets": arr(G.dlspm_gen_config_row_offsets(h), M + 1, np.int32),
+            "col_indices": arr(G.dlspm_gen_config_col_indices(h), nnz, np.int32),
+            "values": arr(G.dlspm_gen_config_values(h), nnz if op == OP_SPMM else 0, np.float32),
+        }
+        for which in range(3):
+            cnt = ctypes.c_size_t()
+            p = G.dlspm_gen_config_dense(h, which, ctypes.byref(cnt))
+            out[f"d{which}"] = arr(p, int(cnt.value), np.float32)
+        rows = {OP_SPMM: (K, None, None), OP_SDDMM: (M, K, None), OP_FUSED: (M, K, K)}[op]
+        for which, r in enumerate(rows):
+            if r is not None:
+                out[f"d{which}"] = out[f"d{which}"].reshape(r, N)
+        return out
+    finally:
+        G.dlspm_gen_config_destroy(h)
+
+
+def account(op: int, M: int, K: int, N: int, nnz: int) -> dict:
+    """{'flops', 'algorithmic_bytes', 'effective_bytes'} for one launch (the reference's flop formulas; bytes as
+    every operand once / every gathered dense row counted)."""
+    out = (ctypes.c_double * 3)()
+    gen_lib().dlspm_account(op, float(M), float(K), float(N), float(nnz), out)
+    return {"flops": out[0], "algorithmic_bytes": out[1], "effective_bytes": out[2]}

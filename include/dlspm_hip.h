@@ -1,0 +1,122 @@
+/*
+ * libdlspm_hip -- fp32 CSR sparse kernels for AMD MI355X (gfx950): SpMM, CSR-sampled SDDMM and the
+ * fused SDDMM->SpMM, behind a plain C ABI.
+ *
+ * Conventions shared by every entry point (they restate what the reference's drivers do around
+ * their kernel launches, /root/reference paths relative to the reference tree):
+ *   - every pointer is a DEVICE pointer owned by the caller (the reference allocates with
+ *     sycl::malloc_device in main(), e.g. SPMM/spmm-esimd-fromfile2.cpp:172-180);
+ *   - indices and sizes are 32-bit ints, CSR is zero-based, dense operands are row-major and
+ *     contiguous (leading dimension = N or D);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); calls only enqueue
+ *     work on it and return, they never synchronise;
+ *   - the CSR structure (row_offsets, col_indices) is read-only: the library never writes it;
+ *   - outputs are fully overwritten, including rows with no nonzero, so no pre-zeroing is needed
+ *     (the reference kernels return early on empty rows and rely on the driver's memset,
+ *     SPMM/spmmesimd2.hpp:90-91, SPMM/spmm-esimd-fromfile2.cpp:196);
+ *   - no input needs padding (the reference over-allocates col/val by 2*VLC for its unmasked tail
+ *     loads, SPMM/spmm-esimd-fromfile2.cpp:174-176);
+ *   - any N / D >= 1 is accepted (the reference rejects N % 16 != 0,
+ *     SPMM/spmm-esimd-fromfile2.cpp:230-231); multiples of 4 with 16-byte aligned dense operands
+ *     take the dwordx4 path, everything else a scalar-load path of the same kernels;
+ *   - results are deterministic: no floating-point atomics (the reference's SDDMM v4 uses them,
+ *     SDDMM/sddmm-esimd-fromfile_v4.hpp:161,175);
+ *   - errors are returned as a negative status, nothing is thrown across the ABI (the reference
+ *     throws std::invalid_argument / std::logic_error on the host before launching).
+ * Calls on different streams may run concurrently from different host threads; the library keeps
+ * no mutable global state.
+ */
+#ifndef DLSPM_HIP_H
+#define DLSPM_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* status codes */
+#define DLSPM_OK              0
+#define DLSPM_E_INVALID_ARG  (-1) /* negative size, NULL pointer for a non-empty operand, nnz/M/K inconsistent */
+#define DLSPM_E_WORKSPACE    (-2) /* workspace smaller than dlspm_workspace_bytes() or misaligned          */
+#define DLSPM_E_LAUNCH       (-3) /* the HIP runtime refused the launch (see dlspm_last_hip_error)         */
+#define DLSPM_E_INVALID_CSR  (-4) /* dlspm_csr_check found a malformed CSR structure                        */
+#define DLSPM_E_NO_DEVICE    (-5) /* no gfx950 device is current                                            */
+
+/* operation selectors for dlspm_workspace_bytes */
+#define DLSPM_OP_SPMM   0
+#define DLSPM_OP_SDDMM  1
+#define DLSPM_OP_FUSED  2
+
+/*
+ * C[M x N] = A_csr[M x K] * B[K x N].
+ * Replaces the kernel launch `SpmmEsimd<CH>(values_dev, row_offsets_dev, column_indices_dev,
+ * rhs_matrix_dev, output_dev, item, MSZ, KSZ, NSZ)` of SPMM/spmm-esimd-fromfile2.cpp:199-228
+ * (kernel: SPMM/spmmesimd2.hpp:63-147, launch sizing ComputeNT: SPMM/spmmesimd2.hpp:30-60) and
+ * computes what the CPU loop Spmm of SPMM/spmm-esimd-fromfile2.cpp:63-83 computes.
+ *   row_offsets[M+1], col_indices[nnz], values[nnz]; B is K x N, C is M x N, both row-major.
+ */
+int spmm_csr_f32(int M, int K, int N, int nnz,
+                 const int* row_offsets, const int* col_indices, const float* values,
+                 const float* B, float* C,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * out_values[j] = dot(lhs[i, :], rhs[col_indices[j], :]) for every CSR slot j of row i
+ * (S .* (lhs * rhs^T) written in S's own CSR order; indices are neither copied nor permuted).
+ * Replaces `Launcher(row_offsets, column_indices, lhs, rhs, out, NSZ, NT, nh_threads, queue)` of
+ * SDDMM/sddmm-esimd-fromfile.hpp:180-212 (kernel :59-131; the small-K variant
+ * SDDMM/sddmm-esimd-fromfile_v4.hpp:102-177) and computes what the CPU loop Sddmm of
+ * SDDMM/sddmm-esimd-fromfile.cpp:18-36 computes. D is the inner (feature) dimension, called NSZ in
+ * the reference's SDDMM files.
+ *   lhs is M x D, rhs is K x D (the un-transposed storage of rhs^T), out_values[nnz].
+ */
+int sddmm_csr_f32(int M, int K, int D, int nnz,
+                  const int* row_offsets, const int* col_indices,
+                  const float* lhs, const float* rhs, float* out_values,
+                  void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * O[M x D] = (S .* (Q * Kmat^T) * scale) * V, with the sampled scores kept on chip.
+ * Replaces `FusedEsimd(a_row_offsets, a_column_indices, c, b, d, e, item)` of
+ * FUSED/fused-esimd_cb.cpp:100-189 (launch :318-331; c->Q, b->Kmat, d->V, e->O) and computes what
+ * Sddmm followed by Spmm compute in FUSED/fused.cpp:47-89. scale = 1.0f gives exactly the
+ * reference's semantics (it has no scale); the scores are fp32 between the two stages as there.
+ *   Q is M x D, Kmat and V are K x D, O is M x D.
+ */
+int fused_sddmm_spmm_f32(int M, int K, int D, int nnz,
+                         const int* row_offsets, const int* col_indices,
+                         const float* Q, const float* Kmat, const float* V, float scale,
+                         float* O,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Bytes of device workspace the op wants for these sizes (0 = none; `workspace` may then be NULL).
+ * Takes the place of the host-side launch sizing the reference does before each launch
+ * (SPMM/spmm-esimd-fromfile2.cpp:188-192, SDDMM/sddmm-esimd-fromfile_v4.cpp:146-160).
+ */
+size_t dlspm_workspace_bytes(int op, int M, int K, int N_or_D, int nnz);
+
+/*
+ * Device-side restatement of the reference's SanityCheck (SPMM/spmm-esimd-fromfile2.cpp:36-61):
+ * row_offsets[0] == 0, row_offsets[M] == nnz, offsets non-decreasing, no row longer than K, every
+ * column index in [0, K). Synchronises `stream`. Returns DLSPM_OK or DLSPM_E_INVALID_CSR.
+ * The compute entry points do not call it; a malformed CSR handed to them is undefined behaviour,
+ * as it is for the reference's kernels.
+ */
+int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* col_indices,
+                    void* stream);
+
+/* Human-readable text for a status code (never NULL). */
+const char* dlspm_status_string(int status);
+
+/* hipError_t (as int) of the last failed HIP call made by this thread inside the library, 0 if none. */
+int dlspm_last_hip_error(void);
+
+/* "dlspm_hip <major>.<minor> gfx950" */
+const char* dlspm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DLSPM_HIP_H */

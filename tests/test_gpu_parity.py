@@ -1,0 +1,253 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle on the same seeded inputs.
+
+Bars (BASELINE.json): the CSR structure must come back bit-identical (the library may not touch it), values
+within 1e-4 relative Frobenius error of the reference's CPU loops. Sizes here are ones the oracle finishes
+in seconds; the five benchmark configurations are checked at full size.
+"""
+import numpy as np
+import pytest
+
+from conftest import random_csr
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-4  # relative Frobenius error, from BASELINE.json's north_star
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return torch
+
+
+def dev(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def check_csr_untouched(ro_d, ci_d, ro, ci):
+    assert np.array_equal(ro_d.cpu().numpy(), ro), "row_offsets changed"
+    assert np.array_equal(ci_d.cpu().numpy(), ci), "col_indices changed"
+
+
+# (M, K, N, kind, density): N picks the lane layout (G = 8/16/32/64, V = 1/2, scalar path for N % 4 != 0),
+# density and kind pick the (W, R) split and exercise shared rows, empty rows and ragged tails.
+SPMM_CASES = [
+    (1, 1, 1, "full", 1.0),
+    (3, 5, 4, "uniform", 0.5),
+    (64, 64, 8, "uniform", 0.2),
+    (100, 300, 32, "uniform", 0.05),
+    (257, 129, 64, "skewed", 0.1),
+    (128, 512, 128, "uniform", 0.3),
+    (333, 512, 256, "skewed", 0.1),
+    (200, 512, 392, "uniform", 0.2),
+    (64, 256, 512, "uniform", 0.1),
+    (50, 200, 1000, "skewed", 0.05),
+    (77, 130, 33, "uniform", 0.1),
+    (40, 100, 7, "empty_rows", 0.3),
+    (90, 64, 130, "skewed", 0.3),
+    (256, 256, 128, "empty_rows", 0.1),
+    (64, 128, 256, "empty", 0.0),
+    (16, 700, 256, "full", 1.0),
+    (5, 2048, 64, "full", 1.0),
+    (1000, 64, 16, "uniform", 0.02),
+]
+
+
+@pytest.mark.parametrize("M,K,N,kind,density", SPMM_CASES)
+def test_spmm_matches_oracle(torch_cuda, dl, oracle, M, K, N, kind, density):
+    torch = torch_cuda
+    rng = np.random.default_rng(1234 + M * 7 + N)
+    ro, ci = random_csr(rng, M, K, kind, density)
+    va = rng.uniform(-1, 1, ci.size).astype(np.float32)
+    B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    ref = oracle.spmm(ro, ci, va, B)
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")  # poisoned: every element must be written
+    dl.spmm(ro_d, ci_d, dev(torch, va), dev(torch, B), K=K, out=C)
+    torch.cuda.synchronize()
+    got = C.cpu().numpy()
+    assert np.isfinite(got).all(), "an output element was not written"
+    assert oracle.rel_frobenius(got, ref) <= TOL
+    # the reference drivers' own metric: max |diff| (SPMM/spmm-esimd-fromfile2.cpp:266-276)
+    assert np.abs(got - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max())
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+    empty = np.diff(ro) == 0
+    assert (got[empty] == 0).all(), "rows without nonzeros must be written as exact zeros"
+
+
+SDDMM_CASES = [
+    (1, 1, 1, "full", 1.0),
+    (7, 9, 4, "uniform", 0.5),
+    (64, 64, 16, "uniform", 0.3),
+    (100, 300, 32, "uniform", 0.1),
+    (130, 257, 64, "skewed", 0.1),
+    (256, 512, 128, "uniform", 0.05),
+    (99, 200, 256, "skewed", 0.1),
+    (40, 128, 512, "uniform", 0.2),
+    (30, 64, 1024, "uniform", 0.3),
+    (50, 100, 48, "uniform", 0.2),
+    (50, 100, 100, "skewed", 0.2),
+    (33, 77, 13, "uniform", 0.3),
+    (64, 128, 1, "uniform", 0.3),
+    (200, 300, 128, "empty_rows", 0.1),
+    (8, 1500, 128, "full", 1.0),
+    (20, 40, 0, "uniform", 0.3),
+]
+
+
+@pytest.mark.parametrize("M,K,D,kind,density", SDDMM_CASES)
+def test_sddmm_matches_oracle(torch_cuda, dl, oracle, M, K, D, kind, density):
+    torch = torch_cuda
+    rng = np.random.default_rng(4321 + M * 5 + D)
+    ro, ci = random_csr(rng, M, K, kind, density)
+    lhs = rng.normal(0, 1, (M, D)).astype(np.float32)
+    rhs = rng.normal(0, 1, (K, D)).astype(np.float32)
+    ref = oracle.sddmm(ro, ci, lhs, rhs)
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    out = torch.full((ci.size,), float("nan"), dtype=torch.float32, device="cuda")
+    dl.sddmm(ro_d, ci_d, dev(torch, lhs), dev(torch, rhs), out=out)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.isfinite(got).all(), "a CSR slot was not written"
+    assert oracle.rel_frobenius(got, ref) <= TOL
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
+FUSED_CASES = [
+    (1, 1, 4, "full", 1.0, 1.0),
+    (9, 11, 8, "uniform", 0.5, 1.0),
+    (64, 64, 16, "uniform", 0.3, 0.25),
+    (100, 300, 32, "uniform", 0.1, 1.0),
+    (130, 257, 64, "skewed", 0.1, 0.125),
+    (256, 512, 128, "uniform", 0.05, 1.0),
+    (99, 200, 256, "skewed", 0.1, 0.0625),
+    (40, 128, 512, "uniform", 0.2, 1.0),
+    (20, 64, 1024, "uniform", 0.3, 1.0),
+    (12, 64, 2048 + 64, "uniform", 0.3, 1.0),
+    (50, 100, 48, "uniform", 0.2, 1.0),
+    (33, 77, 13, "uniform", 0.3, 0.5),
+    (200, 300, 64, "empty_rows", 0.1, 0.125),
+    (8, 1500, 64, "full", 1.0, 0.125),
+    (64, 128, 64, "empty", 0.0, 1.0),
+]
+
+
+@pytest.mark.parametrize("M,K,D,kind,density,scale", FUSED_CASES)
+def test_fused_matches_oracle(torch_cuda, dl, oracle, M, K, D, kind, density, scale):
+    torch = torch_cuda
+    rng = np.random.default_rng(999 + M * 3 + D)
+    ro, ci = random_csr(rng, M, K, kind, density)
+    Q = rng.normal(0, 1, (M, D)).astype(np.float32)
+    Km = rng.normal(0, 1, (K, D)).astype(np.float32)
+    V = rng.normal(0, 1, (K, D)).astype(np.float32)
+    ref = oracle.fused(ro, ci, Q, Km, V, scale)
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    O = torch.full((M, D), float("nan"), dtype=torch.float32, device="cuda")
+    dl.fused(ro_d, ci_d, dev(torch, Q), dev(torch, Km), dev(torch, V), scale, out=O)
+    torch.cuda.synchronize()
+    got = O.cpu().numpy()
+    assert np.isfinite(got).all(), "an output element was not written"
+    assert oracle.rel_frobenius(got, ref) <= TOL
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+    empty = np.diff(ro) == 0
+    assert (got[empty] == 0).all()
+
+
+def test_fused_equals_unfused_on_gpu(torch_cuda, dl, oracle):
+    """fused(Q, K, V, scale) == spmm(sddmm(Q, K) * scale, V), both on the GPU (the reference checks its fused
+    emulation against Sddmm -> Spmm the same way, FUSED/fused.cpp:400-413)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(5)
+    M, K, D, scale = 300, 400, 64, 0.125
+    ro, ci = random_csr(rng, M, K, "skewed", 0.1)
+    Q, Km, V = (dev(torch, rng.normal(0, 1, s).astype(np.float32)) for s in ((M, D), (K, D), (K, D)))
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    scores = dl.sddmm(ro_d, ci_d, Q, Km) * scale
+    unfused = dl.spmm(ro_d, ci_d, scores, V, K=K)
+    fusedO = dl.fused(ro_d, ci_d, Q, Km, V, scale)
+    torch.cuda.synchronize()
+    assert oracle.rel_frobenius(fusedO.cpu().numpy(), unfused.cpu().numpy()) <= 1e-5
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
+def test_benchmark_configs_full_size(torch_cuda, dl, oracle, cfg):
+    """The five BASELINE.json configurations at full size against the oracle."""
+    torch = torch_cuda
+    c = dl.make_config(cfg)
+    ro_d, ci_d = dev(torch, c["row_offsets"]), dev(torch, c["col_indices"])
+    if c["op"] == dl.OP_SPMM:
+        ref = oracle.spmm(c["row_offsets"], c["col_indices"], c["values"], c["d0"], omp=True)
+        got = dl.spmm(ro_d, ci_d, dev(torch, c["values"]), dev(torch, c["d0"]), K=c["K"])
+    elif c["op"] == dl.OP_SDDMM:
+        ref = oracle.sddmm(c["row_offsets"], c["col_indices"], c["d0"], c["d1"], omp=True)
+        got = dl.sddmm(ro_d, ci_d, dev(torch, c["d0"]), dev(torch, c["d1"]))
+    else:
+        ref = oracle.fused(c["row_offsets"], c["col_indices"], c["d0"], c["d1"], c["d2"], c["scale"], omp=True)
+        got = dl.fused(ro_d, ci_d, dev(torch, c["d0"]), dev(torch, c["d1"]), dev(torch, c["d2"]), c["scale"])
+    torch.cuda.synchronize()
+    err = oracle.rel_frobenius(got.cpu().numpy(), ref)
+    print(f"cfg{cfg} {c['name']}: nnz={c['nnz']} rel_frobenius={err:.3e}")
+    assert err <= TOL
+    check_csr_untouched(ro_d, ci_d, c["row_offsets"], c["col_indices"])
+    assert dl.csr_check(c["M"], c["K"], ro_d, ci_d) == dl.OK
+
+
+def test_misaligned_operands_take_scalar_path(torch_cuda, dl, oracle):
+    """Dense operands that start 4 bytes off a 16-byte boundary must still give the right answer."""
+    torch = torch_cuda
+    rng = np.random.default_rng(77)
+    M, K, N = 60, 90, 64
+    ro, ci = random_csr(rng, M, K, "uniform", 0.2)
+    va = rng.uniform(-1, 1, ci.size).astype(np.float32)
+    B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    buf = torch.empty(K * N + 1, dtype=torch.float32, device="cuda")
+    Bd = buf[1:].view(K, N)
+    Bd.copy_(torch.from_numpy(B))
+    assert Bd.data_ptr() % 16 != 0
+    got = dl.spmm(dev(torch, ro), dev(torch, ci), dev(torch, va), Bd, K=K)
+    torch.cuda.synchronize()
+    assert oracle.rel_frobenius(got.cpu().numpy(), oracle.spmm(ro, ci, va, B)) <= TOL
+
+
+def test_deterministic(torch_cuda, dl):
+    """Two launches on the same inputs give bit-identical outputs (no atomics anywhere)."""
+    torch = torch_cuda
+    c = dl.make_config(2)
+    args = [dev(torch, c[k]) for k in ("row_offsets", "col_indices", "values", "d0")]
+    a = dl.spmm(*args, K=c["K"]).clone()
+    b = dl.spmm(*args, K=c["K"]).clone()
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+def test_linearity_at_full_size(torch_cuda, dl, oracle):
+    """Size-independent property at cfg4's shape: spmm(A, B1 + B2) == spmm(A, B1) + spmm(A, B2) up to rounding."""
+    torch = torch_cuda
+    c = dl.make_config(4)
+    ro, ci, va = (dev(torch, c[k]) for k in ("row_offsets", "col_indices", "values"))
+    B1 = dev(torch, c["d0"])
+    B2 = torch.flip(B1, dims=[0]).contiguous()
+    lhs = dl.spmm(ro, ci, va, (B1 + B2).contiguous(), K=c["K"])
+    rhs = dl.spmm(ro, ci, va, B1, K=c["K"]) + dl.spmm(ro, ci, va, B2, K=c["K"])
+    torch.cuda.synchronize()
+    assert oracle.rel_frobenius(lhs.cpu().numpy(), rhs.cpu().numpy()) <= 1e-5
+
+
+def test_error_statuses(torch_cuda, dl):
+    torch = torch_cuda
+    z = torch.zeros(4, dtype=torch.int32, device="cuda")
+    f = torch.zeros(16, dtype=torch.float32, device="cuda")
+    L = dl.lib()
+    assert L.spmm_csr_f32(-1, 1, 1, 0, z.data_ptr(), None, None, None, f.data_ptr(), None, 0, None) == dl.E_INVALID_ARG
+    assert L.spmm_csr_f32(2, 2, 2, 5, z.data_ptr(), z.data_ptr(), f.data_ptr(), f.data_ptr(), f.data_ptr(), None, 0, None) == dl.E_INVALID_ARG
+    assert L.spmm_csr_f32(2, 2, 2, 1, None, z.data_ptr(), f.data_ptr(), f.data_ptr(), f.data_ptr(), None, 0, None) == dl.E_INVALID_ARG
+    assert L.spmm_csr_f32(0, 2, 2, 0, None, None, None, None, None, None, 0, None) == dl.OK
+    # malformed CSR structures are caught by the device-side check
+    bad_ro = torch.tensor([0, 3, 2, 4], dtype=torch.int32, device="cuda")
+    ci = torch.tensor([0, 1, 2, 3], dtype=torch.int32, device="cuda")
+    assert dl.csr_check(3, 4, bad_ro, ci) == dl.E_INVALID_CSR
+    good_ro = torch.tensor([0, 2, 2, 4], dtype=torch.int32, device="cuda")
+    assert dl.csr_check(3, 4, good_ro, ci) == dl.OK
+    assert dl.csr_check(3, 3, good_ro, ci) == dl.E_INVALID_CSR  # column 3 >= K
