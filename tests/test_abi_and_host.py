@@ -1,0 +1,100 @@
+"""CPU-side checks: the C ABI library loads and exports every function include/dlspm_hip.h declares (no
+compute call is made without a GPU), and the host-side generators and accounting behave as documented."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "dlspm_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"^\s*(?:const\s+)?(?:int|size_t|char\s*\*|void)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
+
+
+def test_header_declares_the_three_named_entry_points():
+    names = declared_functions()
+    for required in ("spmm_csr_f32", "sddmm_csr_f32", "fused_sddmm_spmm_f32"):
+        assert required in names
+    assert len(names) >= 8
+
+
+def test_library_exports_every_declared_symbol(dl):
+    lib = ctypes.CDLL(dl.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} is declared in include/dlspm_hip.h but not exported"
+    assert set(declared_functions()) == set(dl.EXPORTS)
+
+
+def test_host_only_entry_points_answer_without_a_gpu(dl):
+    L = dl.lib()
+    assert dl.version().startswith("dlspm_hip") and "gfx950" in dl.version()
+    assert dl.status_string(dl.OK) == "ok"
+    for code in (dl.E_INVALID_ARG, dl.E_WORKSPACE, dl.E_LAUNCH, dl.E_INVALID_CSR, dl.E_NO_DEVICE, -99):
+        assert isinstance(dl.status_string(code), str) and dl.status_string(code)
+    assert L.dlspm_workspace_bytes(dl.OP_SPMM, 2048, 512, 256, 100000) == 0
+    # argument validation happens before any HIP call, so it can be checked here
+    assert L.spmm_csr_f32(-1, 1, 1, 0, None, None, None, None, None, None, 0, None) == dl.E_INVALID_ARG
+    assert L.spmm_csr_f32(2, 2, 2, 5, None, None, None, None, None, None, 0, None) == dl.E_INVALID_ARG  # nnz > M*K
+    assert L.spmm_csr_f32(2, 2, 2, 1, None, None, None, None, None, None, 0, None) == dl.E_INVALID_ARG  # NULL CSR
+    assert L.sddmm_csr_f32(2, 2, -4, 1, None, None, None, None, None, None, 0, None) == dl.E_INVALID_ARG
+    assert L.fused_sddmm_spmm_f32(2, 2, 4, 1, None, None, None, None, None, 1.0, None, None, 0, None) == dl.E_INVALID_ARG
+    assert L.spmm_csr_f32(0, 5, 5, 0, None, None, None, None, None, None, 0, None) == dl.OK  # empty problem
+    assert L.sddmm_csr_f32(5, 5, 4, 0, None, None, None, None, None, None, 0, None) == dl.OK
+
+
+def test_binding_refuses_host_tensors(dl):
+    import torch
+
+    ro = torch.zeros(3, dtype=torch.int32)
+    with pytest.raises(TypeError):
+        dl.spmm(ro, ro, torch.zeros(3), torch.zeros(2, 2))
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
+def test_benchmark_configs_are_as_specified(dl, oracle, cfg):
+    c = dl.make_config(cfg)
+    again = dl.make_config(cfg)
+    for k in ("row_offsets", "col_indices", "values", "d0", "d1", "d2"):
+        assert np.array_equal(c[k], again[k]), "generators must be deterministic"
+    ro, ci = c["row_offsets"], c["col_indices"]
+    assert oracle.csr_check(c["M"], c["K"], c["nnz"], ro, ci) == 0
+    lens = np.diff(ro)
+    rows = np.repeat(np.arange(c["M"]), lens)
+    inside = np.ones(ci.size, dtype=bool)
+    inside[ro[:-1][lens > 0]] = False
+    assert (np.diff(ci.astype(np.int64), prepend=-1)[inside] > 0).all(), "columns ascend strictly inside each row"
+    sparsity = 1.0 - c["nnz"] / (c["M"] * c["K"])
+    expect = {1: (0, 512, 512, 128, 0.70), 2: (0, 2048, 512, 256, 0.90), 3: (1, 2048, 2048, 128, 0.95),
+              4: (0, 2048, 512, 392, 0.80), 5: (2, 4096, 4096, 64, 0.98)}[cfg]
+    assert (c["op"], c["M"], c["K"], c["N"]) == expect[:4]
+    assert abs(sparsity - expect[4]) < 0.005
+    if cfg == 2:
+        assert lens.max() > 4 * lens.mean(), "row lengths must be skewed"
+        assert abs(c["values"].std() - 0.02) < 0.001
+    if cfg == 4:
+        assert (lens == 102).all()
+        assert abs((c["d0"] == 0).mean() - 0.5) < 0.01 and c["d0"].min() >= 0
+    if cfg == 5:
+        assert c["scale"] == 0.125 and lens.max() <= 80
+        i = 1000
+        band = np.arange(i - 16, i + 16)
+        assert np.isin(band, ci[ro[i]:ro[i + 1]]).all(), "the local band of width 32 is present"
+
+
+def test_accounting_formulas(dl):
+    a = dl.account(dl.OP_SPMM, 2048, 512, 256, 104858)
+    assert a["flops"] == (2 * 104858 - 2048) * 256                       # SPMM/spmm-esimd-fromfile2.cpp:253
+    assert a["algorithmic_bytes"] == 4 * 2049 + 8 * 104858 + 4 * 512 * 256 + 4 * 2048 * 256
+    assert a["effective_bytes"] == 4 * 2049 + 8 * 104858 + 4 * 104858 * 256 + 4 * 2048 * 256
+    s = dl.account(dl.OP_SDDMM, 2048, 2048, 128, 209715)
+    assert s["flops"] == 209715 * (2 * 128 - 1)                          # SDDMM/sddmm-esimd-fromfile.cpp:160
+    assert s["algorithmic_bytes"] == 4 * 2049 + 4 * 209715 + 4 * 2048 * 128 * 2 + 4 * 209715
+    f = dl.account(dl.OP_FUSED, 4096, 4096, 64, 327680)
+    assert f["flops"] == (2 * 327680 - 4096) * 64 + 327680 * (2 * 64 - 1) + 327680
+    assert f["algorithmic_bytes"] == 4 * 4097 + 4 * 327680 + 4 * 4096 * 64 + 8 * 4096 * 64 + 4 * 4096 * 64
