@@ -1,0 +1,139 @@
+"""The C++ drivers (dlspm-esimd_amd/bin/{spmm,sddmm,fused}_run): command-line and file error handling on the CPU,
+and on the GPU their single-matrix, from-file, batch and sweep runs, whose dumped outputs are checked here against
+the CPU oracle (the drivers themselves only cross-check on the device)."""
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from conftest import random_csr
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "dlspm-esimd_amd", "bin")
+
+
+def run(app, *args):
+    exe = os.path.join(BIN, app)
+    assert os.path.exists(exe), f"{exe} is missing: run `make -C dlspm-esimd_amd drivers`"
+    p = subprocess.run([exe, *map(str, args)], capture_output=True, text=True, timeout=300)
+    return p.returncode, p.stdout + p.stderr
+
+
+def write_smtx(path, M, K, ro, ci):
+    with open(path, "w") as f:
+        f.write(f"{M}, {K}, {len(ci)}\n")
+        f.write(" ".join(map(str, ro)) + "\n")
+        f.write(" ".join(map(str, ci)) + "\n")
+
+
+# ---- CPU: the failure paths the reference's drivers have (SURVEY: wrong argc, unopenable file, short file, bad CSR)
+@pytest.mark.parametrize("app", ["spmm_run", "sddmm_run", "fused_run"])
+def test_usage_and_file_errors(app, tmp_path):
+    rc, out = run(app)
+    assert rc == 1 and "Usage:" in out and ".smtx" in out
+    rc, out = run(app, "only_one_positional.smtx")
+    assert rc == 1 and "Usage:" in out
+    rc, out = run(app, tmp_path / "missing.smtx", 64)
+    assert rc == 1 and "Error opening file!" in out
+    (tmp_path / "short.smtx").write_text("4, 4, 5\n0 1 2\n")
+    rc, out = run(app, tmp_path / "short.smtx", 64)
+    assert rc == 1 and "Something went wrong reading row_offsets" in out
+    (tmp_path / "garbled.smtx").write_text("four by four\n")
+    rc, out = run(app, tmp_path / "garbled.smtx", 64)
+    assert rc == 1 and "Something went wrong readin M, K, nnz" in out
+    (tmp_path / "nocols.smtx").write_text("2, 4, 3\n0 2 3\n0 1\n")
+    rc, out = run(app, tmp_path / "nocols.smtx", 64)
+    assert rc == 1 and "Something went wrong reading column_indices" in out
+
+
+@pytest.mark.parametrize("text,message", [
+    ("2, 2, 3\n0 2 3\n0 1 5\n", "a_column_indices[i] >= KSZ"),
+    ("2, 2, 3\n0 2 4\n0 1 1\n", "a_row_offsets[MSZ] != nnz."),
+    ("3, 4, 3\n0 2 1 3\n0 1 1\n", "a_row_offsets[i+1] < a_row_offsets[i]"),
+    ("1, 2, 3\n0 3\n0 1 1\n", "nnz is larger than matrix."),
+    ("2, 2, 3\n0 3 3\n0 1 1\n", "a_row_offsets[i + 1] - a_row_offsets[i] > KSZ"),
+])
+def test_sanity_check_messages(tmp_path, text, message):
+    """Same tests and messages as the reference's SanityCheck (SPMM/spmm-esimd-fromfile2.cpp:36-61)."""
+    (tmp_path / "bad.smtx").write_text(text)
+    rc, out = run("spmm_run", tmp_path / "bad.smtx", 16)
+    assert rc == 1 and message in out
+
+
+def test_cfg_of_wrong_kind_is_refused():
+    rc, out = run("spmm_run", "--cfg", 3)
+    assert rc == 1 and "not an SpMM configuration" in out
+
+
+# ---- GPU -------------------------------------------------------------------------------------------------------------
+def load_dump(d):
+    meta = json.load(open(os.path.join(d, "meta.json")))
+    arr = lambda name, dt: np.fromfile(os.path.join(d, name), dtype=dt)
+    return meta, arr
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cfg,app", [(1, "spmm_run"), (2, "spmm_run"), (4, "spmm_run"), (3, "sddmm_run"), (5, "fused_run")])
+def test_driver_runs_benchmark_configuration(oracle, dl, tmp_path, cfg, app):
+    rc, out = run(app, "--cfg", cfg, "--dump", tmp_path, "--csv", tmp_path / "r.csv", "--cold")
+    print(out)
+    assert rc == 0 and "PASS" in out and "bit-identical" in out and "GFLOPS:" in out and "Total kernel time was" in out
+    meta, arr = load_dump(str(tmp_path))
+    c = dl.make_config(cfg)  # the Python binding and the driver share one generator: same data
+    ro, ci = arr("row_offsets.i32", np.int32), arr("col_indices.i32", np.int32)
+    assert np.array_equal(ro, c["row_offsets"]) and np.array_equal(ci, c["col_indices"])
+    M, K, N = meta["M"], meta["K"], meta["N"]
+    if meta["op"] == "spmm":
+        ref = oracle.spmm(ro, ci, arr("values.f32", np.float32), arr("B.f32", np.float32).reshape(K, N), omp=True)
+        got = arr("C.f32", np.float32).reshape(M, N)
+    elif meta["op"] == "sddmm":
+        ref = oracle.sddmm(ro, ci, arr("lhs.f32", np.float32).reshape(M, N), arr("rhs.f32", np.float32).reshape(K, N), omp=True)
+        got = arr("out.f32", np.float32)
+    else:
+        ref = oracle.fused(ro, ci, arr("Q.f32", np.float32).reshape(M, N), arr("K.f32", np.float32).reshape(K, N),
+                           arr("V.f32", np.float32).reshape(K, N), meta["scale"], omp=True)
+        got = arr("O.f32", np.float32).reshape(M, N)
+    assert oracle.rel_frobenius(got, ref) <= 1e-4
+    assert len(open(tmp_path / "r.csv").read().strip().split(",")) >= 6
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("app,width", [("spmm_run", 49), ("sddmm_run", 64), ("fused_run", 32)])
+def test_driver_from_file_and_batch(oracle, tmp_path, app, width):
+    """`./app <file>.smtx <N>` as in the reference, N = 49 being one of the un-padded rn50 batch sizes."""
+    rng = np.random.default_rng(3)
+    M, K = 128, 300
+    ro, ci = random_csr(rng, M, K, "empty_rows", 0.1)
+    write_smtx(tmp_path / "a.smtx", M, K, ro, ci)
+    dump = tmp_path / "dump"
+    dump.mkdir()
+    rc, out = run(app, tmp_path / "a.smtx", width, "--dump", dump, "--csv", tmp_path / "f.csv")
+    print(out)
+    assert rc == 0 and "PASS" in out and f"nnz: {len(ci)}" in out
+    meta, arr = load_dump(str(dump))
+    assert np.array_equal(arr("row_offsets.i32", np.int32), ro) and np.array_equal(arr("col_indices.i32", np.int32), ci)
+    if meta["op"] == "spmm":
+        ref = oracle.spmm(ro, ci, arr("values.f32", np.float32), arr("B.f32", np.float32).reshape(K, width))
+        got = arr("C.f32", np.float32).reshape(M, width)
+        assert len(open(tmp_path / "f.csv").read().strip().split(",")) == 7  # M,N,K,SP,gflops,max_diff,opcount
+    elif meta["op"] == "sddmm":
+        ref = oracle.sddmm(ro, ci, arr("lhs.f32", np.float32).reshape(M, width), arr("rhs.f32", np.float32).reshape(K, width))
+        got = arr("out.f32", np.float32)
+    else:
+        ref = oracle.fused(ro, ci, arr("Q.f32", np.float32).reshape(M, width), arr("K.f32", np.float32).reshape(K, width),
+                           arr("V.f32", np.float32).reshape(K, width), 1.0)
+        got = arr("O.f32", np.float32).reshape(M, width)
+    assert oracle.rel_frobenius(got, ref) <= 1e-4
+    (tmp_path / "list.txt").write_text(f"# two runs of the same pattern\n{tmp_path / 'a.smtx'} 16\n{tmp_path / 'a.smtx'} 128\n")
+    rc, out = run(app, "--batch", tmp_path / "list.txt")
+    assert rc == 0 and out.count("PASS") == 2
+
+
+@pytest.mark.gpu
+def test_driver_shape_and_small_sweep():
+    rc, out = run("spmm_run", "--shape", 512, 256, 64, 0.2, "--seed", 9)
+    assert rc == 0 and "PASS" in out and "MSZ = 512 KSZ = 256 NSZ = 64" in out
+    rc, out = run("sddmm_run", "--sweep", "--max-m", 1024, "--iters", 5)
+    assert rc == 0 and out.count("PASS") == 6  # (1024,1024) x N in {32,128} x density in {0.3,0.2,0.1}
