@@ -23,23 +23,17 @@ static int fail_hip(hipError_t e)
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Optional launch-shape override for tuning sweeps: DLSPM_SPLIT="W,R" read once per process.
+// Optional launch-shape override for tuning sweeps: DLSPM_SPLIT="W,R", read at every call.
 static bool split_override(int& W, int& R)
 {
-    static const struct Ov {
-        bool on = false;
-        int W = 0, R = 0;
-        Ov()
-        {
-            const char* e = std::getenv("DLSPM_SPLIT");
-            if (e && std::sscanf(e, "%d,%d", &W, &R) == 2) on = true;
-        }
-    } ov;
-    if (ov.on) {
-        W = ov.W;
-        R = ov.R;
+    const char* e = std::getenv("DLSPM_SPLIT");
+    int w = 0, r = 0;
+    if (e && std::sscanf(e, "%d,%d", &w, &r) == 2) {
+        W = w;
+        R = r;
+        return true;
     }
-    return ov.on;
+    return false;
 }
 
 void choose_split(int M, long long col_tiles, int nnz, int target, int max_w, int& W, int& R)
@@ -115,8 +109,8 @@ int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int
     if (!row_offsets || !C) return DLSPM_E_INVALID_ARG;
     if (nnz > 0 && (!col_indices || !values || !B)) return DLSPM_E_INVALID_ARG;
     const bool vec4 = (N % 4 == 0) && aligned16(B) && aligned16(C);
-    const SpmmShape shape = spmm_choose(M, N, nnz, vec4);
     const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C};
+    const SpmmShape shape = spmm_choose(M, N, nnz, vec4);
     const hipError_t e = spmm_launch(args, shape, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }

@@ -61,16 +61,39 @@ constexpr int kDppQuadSwap2 = 0x4E;      // quad_perm [2,3,0,1]: lane ^ 2
 constexpr int kDppRowHalfMirror = 0x141; // lane i <-> 7 - i inside each group of 8
 constexpr int kDppRowMirror = 0x140;     // lane i <-> 15 - i inside each row of 16
 
+// x[lane] + x[lane ^ 8 | 16 | 32] in every lane, without touching LDS: a DPP row rotate for 8, and the gfx950
+// v_permlane16_swap / v_permlane32_swap (which exchange the odd 16- or 32-lane blocks of one register with the
+// even blocks of another; applied to two copies of x they leave (even, even) and (odd, odd) copies to add).
+constexpr int kDppRowRor8 = 0x128;
+__device__ __forceinline__ float add_xor8(float x) { return x + dpp_move<kDppRowRor8>(x); }
+__device__ __forceinline__ float add_xor16(float x)
+{
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float add_xor32(float x)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+template <int STEP> __device__ __forceinline__ float add_xor(float x)
+{
+    static_assert(STEP == 8 || STEP == 16 || STEP == 32, "cross-group sums start at 8 lanes");
+    if constexpr (STEP == 8) return add_xor8(x);
+    else if constexpr (STEP == 16) return add_xor16(x);
+    else return add_xor32(x);
+}
+
 // Sum of x over aligned groups of G lanes, result in every lane of the group. G in {1,2,4,8,16,32,64}.
-// Steps up to 16 lanes are DPP (full VALU rate); 32 and 64 go through ds_bpermute.
+// Must be called with all lanes of the wave active.
 template <int G> __device__ __forceinline__ float group_sum(float x)
 {
     if constexpr (G >= 2) x += dpp_move<kDppQuadSwap1>(x);
     if constexpr (G >= 4) x += dpp_move<kDppQuadSwap2>(x);
     if constexpr (G >= 8) x += dpp_move<kDppRowHalfMirror>(x);  // quads already uniform: mirror pairs quad 0 with quad 1
     if constexpr (G >= 16) x += dpp_move<kDppRowMirror>(x);     // halves already uniform: mirror pairs the two halves
-    if constexpr (G >= 32) x += lane_get(x, (int)(threadIdx.x & 63) ^ 16);
-    if constexpr (G >= 64) x += lane_get(x, (int)(threadIdx.x & 63) ^ 32);
+    if constexpr (G >= 32) x = add_xor16(x);
+    if constexpr (G >= 64) x = add_xor32(x);
     return x;
 }
 
@@ -167,23 +190,20 @@ __device__ __forceinline__ void dense_rows_fma(Vec<VEC>* acc, int c, float av, i
     }
 }
 
-// Adds the slots' partial sums so that every lane (in particular slot 0) ends with the total.
+// Adds the slots' partial sums so that every lane (in particular slot 0) ends with the total. G >= 8.
 template <int VEC, int G, int V> __device__ __forceinline__ void slots_sum(Vec<VEC>* acc, int lane)
 {
+    (void)lane;
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-#pragma unroll
-        for (int step = G; step < kWave; step <<= 1) {
-            Vec<VEC> o;
-            if constexpr (VEC == 4) {
-                o.v.x = lane_get(acc[v].v.x, lane ^ step);
-                o.v.y = lane_get(acc[v].v.y, lane ^ step);
-                o.v.z = lane_get(acc[v].v.z, lane ^ step);
-                o.v.w = lane_get(acc[v].v.w, lane ^ step);
-            } else {
-                o.v = lane_get(acc[v].v, lane ^ step);
-            }
-            acc[v].add(o);
+        if constexpr (VEC == 4) {
+            if constexpr (G <= 8) { acc[v].v.x = add_xor8(acc[v].v.x); acc[v].v.y = add_xor8(acc[v].v.y); acc[v].v.z = add_xor8(acc[v].v.z); acc[v].v.w = add_xor8(acc[v].v.w); }
+            if constexpr (G <= 16) { acc[v].v.x = add_xor16(acc[v].v.x); acc[v].v.y = add_xor16(acc[v].v.y); acc[v].v.z = add_xor16(acc[v].v.z); acc[v].v.w = add_xor16(acc[v].v.w); }
+            if constexpr (G <= 32) { acc[v].v.x = add_xor32(acc[v].v.x); acc[v].v.y = add_xor32(acc[v].v.y); acc[v].v.z = add_xor32(acc[v].v.z); acc[v].v.w = add_xor32(acc[v].v.w); }
+        } else {
+            if constexpr (G <= 8) acc[v].v = add_xor8(acc[v].v);
+            if constexpr (G <= 16) acc[v].v = add_xor16(acc[v].v);
+            if constexpr (G <= 32) acc[v].v = add_xor32(acc[v].v);
         }
     }
 }

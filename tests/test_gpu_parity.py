@@ -52,6 +52,10 @@ SPMM_CASES = [
     (16, 700, 256, "full", 1.0),
     (5, 2048, 64, "full", 1.0),
     (1000, 64, 16, "uniform", 0.02),
+    (700, 512, 256, "skewed", 0.12),
+    (1500, 1024, 96, "uniform", 0.1),
+    (2000, 300, 40, "empty_rows", 0.4),
+    (300, 512, 64, "full", 1.0),
 ]
 
 
