@@ -36,29 +36,26 @@ static bool split_override(int& W, int& R)
     return false;
 }
 
-void choose_split(int M, long long col_tiles, int nnz, int target, int max_w, int& W, int& R)
+void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w, int& W, int& R)
 {
     static const int kPairs[][2] = {{4, 16}, {4, 8}, {4, 4}, {4, 2}, {4, 1}, {8, 4}, {8, 2}, {8, 1}, {16, 1}};
     if (split_override(W, R)) {
         for (const auto& pr : kPairs)
             if (pr[0] == W && pr[1] == R && W <= max_w) return;
     }
+    // Measured on MI355X over the benchmark configurations and the 12 x {32,128} x {0.3,0.2,0.1} sweep grid:
+    // four-wave workgroups win whenever the matrix has enough rows to fill the device (16-wave workgroups were up
+    // to 2x slower on long rows: their barrier makes every wave wait for the slowest of sixteen), and rows are
+    // grouped only as far as the grid keeps `min_blocks` workgroups and a workgroup stays below ~512 nonzeros.
     const double avg = M > 0 ? (double)nnz / M : 0.0;
-    double best = 1e300;
-    W = 4;
-    R = 4;
-    for (const auto& pr : kPairs) {
-        const int w = pr[0], r = pr[1];
-        if (w > max_w) continue;
-        const double per = avg * r / w;  // nonzeros per wave
-        double cost = per > target ? std::log2(per / target) : std::log2((target + 1.0) / (per + 1.0)) * 0.75;
-        const double blocks = (double)((M + r - 1) / r) * (double)col_tiles;
-        const double want = 1024.0;  // 4 workgroups per CU keeps every SIMD busy while others drain
-        if (blocks < want && (M + r - 1) / r < M) cost += 0.5 * std::log2(want / (blocks < 1 ? 1 : blocks));
-        cost += 0.05 * (w / 4);  // prefer fewer waves per workgroup when otherwise equal (cheaper barrier)
-        if (cost < best) {
-            best = cost;
-            W = w;
+    const long long work_rows = (long long)M * col_tiles;
+    W = work_rows >= 512 ? 4 : work_rows >= 256 ? 8 : 16;
+    if (W > max_w) W = max_w;
+    R = 1;
+    if (W == 4) {
+        for (int r = 2; r <= 16; r *= 2) {
+            const long long blocks = (long long)((M + r - 1) / r) * col_tiles;
+            if (blocks < min_blocks || avg * r > 512.0) break;
             R = r;
         }
     }

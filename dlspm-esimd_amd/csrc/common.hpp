@@ -228,22 +228,18 @@ __device__ __forceinline__ void sddmm_rounds_load(int D, int g, const float* __r
     }
 }
 
-// One chunk of up to 64 nonzeros [base, q) of one row: returns in lane l the dot product of nonzero
-// base + l (lanes past the chunk return an unspecified value that the caller must not store).
-// `c` receives the lane's column index (0 past the chunk). `lq` holds the lhs row as laid out by the
-// caller: lq[s] = lhs_row[(s*G1 + g)*VEC ..], zero past D. With DS = 0 the row is re-read from lhs_row.
+// One chunk of `cnt` <= 64 nonzeros of one row: returns in lane l the dot product of the chunk's nonzero l
+// (lanes past the chunk return an unspecified value that the caller must not store). `c` is the lane's
+// column index (0 past the chunk). `lq` holds the lhs row as laid out by the caller:
+// lq[s] = lhs_row[(s*G1 + g)*VEC ..], zero past D. With DS = 0 the row is re-read from lhs_row.
 template <int VEC, int G1, int DS, bool MASKED>
-__device__ __forceinline__ float sddmm_chunk(int D, int lane, int base, int q, const int* __restrict__ col_indices,
-                                             const float* __restrict__ lhs_row, const Vec<VEC>* lq,
-                                             const float* __restrict__ rhs, int& c)
+__device__ __forceinline__ float sddmm_chunk(int D, int lane, int cnt, int c, const float* __restrict__ lhs_row,
+                                             const Vec<VEC>* lq, const float* __restrict__ rhs)
 {
     using VecT = Vec<VEC>;
     constexpr int P = kWave / G1;  // nonzeros in flight per access
     const int g = lane % G1;
     const int grp = lane / G1;
-    const int idx = base + lane;
-    c = idx < q ? col_indices[idx] : 0;
-    const int cnt = min(kWave, q - base);
     const int rounds = (cnt + P - 1) / P;  // <= G1
     float res = 0.f;
     if constexpr (DS > 0) {

@@ -85,15 +85,17 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
 #pragma unroll
             for (int v = 0; v < V2; ++v) acc[v] = VecT::zero();
 
+            int c_nxt = col_indices[min(p + lane, q - 1)];  // next pass's columns are requested one pass ahead
             for (int base = p; base < q; base += kWave) {
-                int c;
+                const int c = base + lane < q ? c_nxt : 0;
+                c_nxt = col_indices[min(base + kWave + lane, q - 1)];
+                const int cnt = min(kWave, q - base);
                 // stage 1: lane l <- score of nonzero base + l (fp32, as between the reference's two loops)
-                float score =
-                    exact ? sddmm_chunk<VEC, G1, DS, false>(D, lane, base, q, col_indices, q_row, lq, Kmat, c)
-                          : sddmm_chunk<VEC, G1, DS, true>(D, lane, base, q, col_indices, q_row, lq, Kmat, c);
+                float score = exact ? sddmm_chunk<VEC, G1, DS, false>(D, lane, cnt, c, q_row, lq, Kmat)
+                                    : sddmm_chunk<VEC, G1, DS, true>(D, lane, cnt, c, q_row, lq, Kmat);
                 score = base + lane < q ? score * scale : 0.f;
                 // stage 2: acc += score_j * V[col_j, :]
-                dense_rows_fma<VEC, G, V2>(acc, c, score, min(kWave, q - base), Vmat, D, colv, lane);
+                dense_rows_fma<VEC, G, V2>(acc, c, score, cnt, Vmat, D, colv, lane);
             }
             if constexpr (S > 1) slots_sum<VEC, G, V2>(acc, lane);
 
@@ -195,7 +197,7 @@ FusedShape fused_choose(int M, int D, int nnz, bool vec4)
         s.G1 = 16; s.DS = 0; s.G = 64; s.V = 4;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(M, (D + tw - 1) / tw, nnz, 64, tw >= 1024 ? 4 : 16, s.W, s.R);
+    choose_split(M, (D + tw - 1) / tw, nnz, 512, tw >= 1024 ? 4 : 16, s.W, s.R);
     return s;
 }
 

@@ -51,8 +51,8 @@ hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t str
 FusedShape fused_choose(int M, int D, int nnz, bool vec4);
 hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream);
 
-// Picks (W, R), W <= max_w, so that a wave gets about `target` nonzeros and the grid stays wide enough for
-// 256 CUs. Only the pairs the kernels are instantiated for are returned.
-void choose_split(int M, long long col_tiles, int nnz, int target, int max_w, int& W, int& R);
+// Picks (W, R), W <= max_w: waves per workgroup from the number of rows, rows per workgroup as large as keeps
+// `min_blocks` workgroups in the grid. Only the pairs the kernels are instantiated for are returned.
+void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w, int& W, int& R);
 
 }  // namespace dlspm

@@ -60,10 +60,15 @@ __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* 
                 lq[s] = d < D ? VecT::load(lhs_row + d) : VecT::zero();
             }
         }
+        // 64 column indices per pass, one per lane; the next 64 are requested (index clamped, no condition) before
+        // the rhs rows of the current ones
+        int c_nxt = col_indices[min(p + lane, q - 1)];
         for (int base = p; base < q; base += kWave) {
-            int c;
-            const float o = exact ? sddmm_chunk<VEC, G1, DS, false>(D, lane, base, q, col_indices, lhs_row, lq, rhs, c)
-                                  : sddmm_chunk<VEC, G1, DS, true>(D, lane, base, q, col_indices, lhs_row, lq, rhs, c);
+            const int c = base + lane < q ? c_nxt : 0;
+            c_nxt = col_indices[min(base + kWave + lane, q - 1)];
+            const int cnt = min(kWave, q - base);
+            const float o = exact ? sddmm_chunk<VEC, G1, DS, false>(D, lane, cnt, c, lhs_row, lq, rhs)
+                                  : sddmm_chunk<VEC, G1, DS, true>(D, lane, cnt, c, lhs_row, lq, rhs);
             if (base + lane < q) out[base + lane] = o;
         }
         pos = q;
@@ -116,7 +121,7 @@ SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4)
         s.G1 = 16;
         s.DS = 0;
     }
-    choose_split(M, 1, nnz, 64, 16, s.W, s.R);
+    choose_split(M, 1, nnz, 512, 16, s.W, s.R);
     return s;
 }
 

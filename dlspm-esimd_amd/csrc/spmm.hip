@@ -75,14 +75,18 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
 #pragma unroll
             for (int v = 0; v < V; ++v) acc[v] = VecT::zero();
 
+            // 64 (column, value) pairs per pass, one per lane; the next 64 are requested (index clamped, so the
+            // loads carry no condition) before the rows of B for the current ones, and arrive behind them
+            const int first = min(p + lane, q - 1);
+            int c_nxt = col_indices[first];
+            float a_nxt = values[first];
             for (int base = p; base < q; base += kWave) {
-                const int idx = base + lane;
-                int c = 0;
-                float av = 0.f;
-                if (idx < q) {
-                    c = col_indices[idx];
-                    av = values[idx];
-                }
+                const bool mine = base + lane < q;
+                const int c = mine ? c_nxt : 0;
+                const float av = mine ? a_nxt : 0.f;
+                const int ahead = min(base + kWave + lane, q - 1);
+                c_nxt = col_indices[ahead];
+                a_nxt = values[ahead];
                 dense_rows_fma<VEC, G, V>(acc, c, av, min(kWave, q - base), B, N, colv, lane);
             }
             if constexpr (S > 1) slots_sum<VEC, G, V>(acc, lane);
@@ -184,7 +188,7 @@ SpmmShape spmm_choose(int M, int N, int nnz, bool vec4)
         s.V = N > 64 ? 4 : 1;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(M, (N + tw - 1) / tw, nnz, 32, 16, s.W, s.R);
+    choose_split(M, (N + tw - 1) / tw, nnz, 2048, 16, s.W, s.R);
     return s;
 }
 
