@@ -50,6 +50,7 @@ void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w
     const double avg = M > 0 ? (double)nnz / M : 0.0;
     const long long work_rows = (long long)M * col_tiles;
     W = work_rows >= 512 ? 4 : work_rows >= 256 ? 8 : 16;
+    if (avg >= 1536.0) W = 16;  // very long rows: more waves per row beat the barrier cost (measured, ~8 %)
     if (W > max_w) W = max_w;
     R = 1;
     if (W == 4) {
