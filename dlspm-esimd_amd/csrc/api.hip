@@ -182,6 +182,31 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
     return h_flags == 0 ? DLSPM_OK : DLSPM_E_INVALID_CSR;
 }
 
+int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int aligned16, int* shape)
+{
+    (void)K;
+    if (!shape || M < 0 || N_or_D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
+    const int n = N_or_D;
+    const bool vec4 = aligned16 != 0 && n > 0 && n % 4 == 0;
+    for (int i = 0; i < 8; ++i) shape[i] = 0;
+    if (op == DLSPM_OP_SPMM) {
+        const SpmmShape s = spmm_choose(M, n, nnz, vec4);
+        const int tw = s.G * s.vec * s.V;
+        shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[5] = s.W; shape[6] = s.R; shape[7] = (n + tw - 1) / tw;
+    } else if (op == DLSPM_OP_SDDMM) {
+        const SddmmShape s = sddmm_choose(M, n, nnz, vec4);
+        shape[0] = s.vec; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R; shape[7] = 1;
+    } else if (op == DLSPM_OP_FUSED) {
+        const FusedShape s = fused_choose(M, n, nnz, vec4);
+        const int tw = s.G * s.vec * s.V;
+        shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R;
+        shape[7] = (n + tw - 1) / tw;
+    } else {
+        return DLSPM_E_INVALID_ARG;
+    }
+    return DLSPM_OK;
+}
+
 const char* dlspm_status_string(int status)
 {
     switch (status) {

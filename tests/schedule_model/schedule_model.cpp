@@ -1,0 +1,160 @@
+// Host model of the GPU schedule: the same work split (workgroups of W waves owning R rows, nonzeros divided
+// evenly over the waves, lane groups taking every S-th nonzero, partial sums added in wave order) and the same
+// fp32 operation sequence per output element as the HIP kernels in dlspm-esimd_amd/csrc, in scalar C++.
+// TEST INFRASTRUCTURE: it lets the work decomposition be checked without a GPU (every output written exactly
+// once, nothing read out of range) and lets the GPU results be compared BIT FOR BIT instead of within a
+// tolerance. It plays the role the reference's SpmmEsimdCPU / FusedEsimdCPU (SPMM/spmm-esimd-v1.cpp:83-169,
+// FUSED/fused.cpp:93-216) play for its kernels. The library never uses it.
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <vector>
+
+namespace {
+
+int split_per_wave(int T, int W)
+{
+    int per = (T + W - 1) / W;
+    return per < 1 ? 1 : per;
+}
+
+// sum of the S lane groups' accumulators in the order the kernel's cross-lane steps add them:
+// neighbours first (xor G), then pairs of pairs (xor 2G), ... : a balanced tree over the slots
+float slots_tree(const float* s, int S)
+{
+    if (S == 1) return s[0];
+    std::vector<float> v(s, s + S);
+    for (int step = 1; step < S; step <<= 1)
+        for (int i = 0; i + step < S; i += 2 * step) v[i] = v[i] + v[i + step];
+    return v[0];
+}
+
+// C[M x N] (+= semantics: every element written exactly once; `writes` counts them) for "values" per nonzero.
+// Mirrors spmm_kernel / stage 2 of fused_kernel: shape = lanes G per dense row (S = 64/G slots), W waves, R rows.
+int model_rows(int M, int N, const int* ro, const int* ci, const float* va, const float* B, int G, int W, int R,
+               float* C, int* writes)
+{
+    const int S = 64 / G;
+    std::vector<float> acc((size_t)S * N), part;
+    for (int r0 = 0; r0 < M; r0 += R) {
+        const int nr = std::min(R, M - r0);
+        const int* off = ro + r0;
+        const int T0 = off[0], T = off[nr] - T0;
+        const int per = split_per_wave(T, W);
+        part.assign((size_t)W * 2 * N, NAN);
+        for (int w = 0; w < W; ++w) {
+            const int a = T0 + std::min(T, w * per), b = T0 + std::min(T, (w + 1) * per);
+            if (a >= b) continue;
+            int r = 0;
+            while (off[r + 1] <= a) ++r;
+            int pos = a;
+            while (pos < b) {
+                const int rs = off[r], re = off[r + 1];
+                const int p = pos, q = std::min(re, b);
+                std::fill(acc.begin(), acc.end(), 0.0f);
+                for (int idx = p; idx < q; ++idx) {
+                    const int slot = (idx - p) % S;  // 64 % S == 0, so the chunking does not change the slot
+                    const float* brow = B + (size_t)ci[idx] * N;
+                    float* as = acc.data() + (size_t)slot * N;
+                    for (int j = 0; j < N; ++j) as[j] = std::fmaf(va[idx], brow[j], as[j]);
+                }
+                std::vector<float> sl(S);
+                const bool whole = (p == rs) && (q == re);
+                for (int j = 0; j < N; ++j) {
+                    for (int s = 0; s < S; ++s) sl[s] = acc[(size_t)s * N + j];
+                    const float tot = slots_tree(sl.data(), S);
+                    if (whole) {
+                        C[(size_t)(r0 + r) * N + j] = tot;
+                        writes[(size_t)(r0 + r) * N + j]++;
+                    } else {
+                        part[((size_t)w * 2 + (p == a || R == 1 ? 0 : 1)) * N + j] = tot;
+                    }
+                }
+                pos = q;
+                ++r;
+                while (r < nr && off[r + 1] <= pos) ++r;
+            }
+        }
+        for (int r = 0; r < nr; ++r) {
+            const int rs = off[r], re = off[r + 1];
+            float* crow = C + (size_t)(r0 + r) * N;
+            int* wrow = writes + (size_t)(r0 + r) * N;
+            if (rs == re) {
+                for (int j = 0; j < N; ++j) { crow[j] = 0.0f; wrow[j]++; }
+                continue;
+            }
+            const int wl = (rs - T0) / per, wh = (re - 1 - T0) / per;
+            if (wl == wh) continue;
+            for (int j = 0; j < N; ++j) {
+                float sum = 0.0f;
+                for (int x = wl; x <= wh; ++x) {
+                    const int k = (R != 1 && x == wl && T0 + x * per != rs) ? 1 : 0;
+                    const float pv = part[((size_t)x * 2 + k) * N + j];
+                    if (std::isnan(pv) && !std::isnan(B[0])) return 1;  // a partial sum the schedule never produced
+                    sum = sum + pv;
+                }
+                crow[j] = sum;
+                wrow[j]++;
+            }
+        }
+    }
+    return 0;
+}
+
+// dot product of one nonzero as the SDDMM lane group computes it: lane g accumulates its elements in order with
+// fused multiply-adds, then the G1 lanes are added pairwise (lane^1, lane^2, then the mirrored halves)
+float model_dot(const float* l, const float* r, int D, int vec, int G1, int DS)
+{
+    std::vector<float> lane(G1, 0.0f);
+    for (int g = 0; g < G1; ++g) {
+        float acc = 0.0f;
+        if (DS > 0) {
+            for (int s = 0; s < DS; ++s) {
+                const int d = (s * G1 + g) * vec;
+                for (int e = 0; e < vec; ++e)
+                    if (d + e < D) acc = std::fmaf(l[d + e], r[d + e], acc);
+                    else acc = std::fmaf(0.0f, 0.0f, acc);
+            }
+        } else {
+            for (int d = g * vec; d < D; d += G1 * vec)
+                for (int e = 0; e < vec; ++e) acc = std::fmaf(l[d + e], r[d + e], acc);
+        }
+        lane[g] = acc;
+    }
+    for (int step = 1; step < G1; step <<= 1)
+        for (int i = 0; i + step < G1; i += 2 * step) lane[i] = lane[i] + lane[i + step];
+    return lane[0];
+}
+
+}  // namespace
+
+extern "C" {
+
+// returns 0, or 1 if the schedule is inconsistent (a partial sum consumed that no wave produced)
+int model_spmm(int M, int N, const int* ro, const int* ci, const float* va, const float* B, int G, int W, int R, float* C,
+               int* writes)
+{
+    std::memset(writes, 0, (size_t)M * N * sizeof(int));
+    return model_rows(M, N, ro, ci, va, B, G, W, R, C, writes);
+}
+
+void model_sddmm(int M, int D, const int* ro, const int* ci, const float* lhs, const float* rhs, int vec, int G1, int DS,
+                 float* out)
+{
+    for (int i = 0; i < M; ++i)
+        for (int j = ro[i]; j < ro[i + 1]; ++j)
+            out[j] = model_dot(lhs + (size_t)i * D, rhs + (size_t)ci[j] * D, D, vec, G1, DS);
+}
+
+int model_fused(int M, int D, const int* ro, const int* ci, const float* Q, const float* Km, const float* V, float scale,
+                int vec, int G1, int DS, int G, int W, int R, float* scores, float* O, int* writes)
+{
+    model_sddmm(M, D, ro, ci, Q, Km, vec, G1, DS, scores);
+    const int nnz = ro[M];
+    for (int j = 0; j < nnz; ++j) scores[j] = scores[j] * scale;
+    std::memset(writes, 0, (size_t)M * D * sizeof(int));
+    return model_rows(M, D, ro, ci, scores, V, G, W, R, O, writes);
+}
+
+}  // extern "C"

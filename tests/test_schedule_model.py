@@ -1,0 +1,179 @@
+"""Host model of the GPU schedule (tests/schedule_model/schedule_model.cpp).
+
+CPU part: for every workgroup shape the kernels are instantiated for, the modelled work split writes every output
+element exactly once, never consumes a partial sum that no wave produced, and agrees with the oracle.
+GPU part: with the launch shape the library reports for a problem (dlspm_describe_launch), the model reproduces the
+kernels' fp32 operation order, so the GPU output must equal the model's BIT FOR BIT -- a much sharper check than
+the 1e-4 tolerance, and one that would expose a dropped, duplicated or reordered nonzero of any size.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from conftest import random_csr
+
+HERE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "schedule_model")
+_i = ctypes.POINTER(ctypes.c_int)
+_f = ctypes.POINTER(ctypes.c_float)
+
+
+@pytest.fixture(scope="module")
+def model():
+    so = os.path.join(HERE, "libschedule_model.so")
+    if not os.path.exists(so):
+        subprocess.run(["make", "-s", "-C", HERE], check=True)
+    L = ctypes.CDLL(so)
+    ci = ctypes.c_int
+    L.model_spmm.argtypes = [ci, ci, _i, _i, _f, _f, ci, ci, ci, _f, _i]
+    L.model_spmm.restype = ci
+    L.model_sddmm.argtypes = [ci, ci, _i, _i, _f, _f, ci, ci, ci, _f]
+    L.model_sddmm.restype = None
+    L.model_fused.argtypes = [ci, ci, _i, _i, _f, _f, _f, ctypes.c_float, ci, ci, ci, ci, ci, ci, _f, _f, _i]
+    L.model_fused.restype = ci
+    return L
+
+
+def pi(a):
+    return a.ctypes.data_as(_i)
+
+
+def pf(a):
+    return a.ctypes.data_as(_f)
+
+
+def run_spmm(L, ro, ci, va, B, G, W, R):
+    M, N = ro.size - 1, B.shape[1]
+    C = np.full((M, N), np.nan, dtype=np.float32)
+    writes = np.zeros((M, N), dtype=np.int32)
+    ci2 = ci if ci.size else np.zeros(1, np.int32)
+    va2 = va if va.size else np.zeros(1, np.float32)
+    rc = L.model_spmm(M, N, pi(ro), pi(ci2), pf(va2), pf(B), G, W, R, pf(C), pi(writes))
+    return rc, C, writes
+
+
+SPLITS = [(4, 16), (4, 8), (4, 4), (4, 2), (4, 1), (8, 4), (8, 2), (8, 1), (16, 1)]
+
+
+@pytest.mark.parametrize("kind,density", [("uniform", 0.2), ("skewed", 0.1), ("empty_rows", 0.3), ("full", 1.0), ("empty", 0.0)])
+def test_every_split_writes_each_output_once_and_matches_the_oracle(model, oracle, kind, density):
+    rng = np.random.default_rng(11)
+    M, K, N = 53, 97, 12
+    ro, ci = random_csr(rng, M, K, kind, density)
+    va = rng.normal(0, 1, ci.size).astype(np.float32)
+    B = rng.normal(0, 1, (K, N)).astype(np.float32)
+    ref = oracle.spmm(ro, ci, va, B)
+    for (W, R) in SPLITS:
+        for G in (64, 32, 16, 8):
+            rc, C, writes = run_spmm(model, ro, ci, va, B, G, W, R)
+            assert rc == 0, f"inconsistent partial sums for W={W} R={R} G={G}"
+            assert (writes == 1).all(), f"W={W} R={R} G={G}: an element was written {writes.min()}..{writes.max()} times"
+            assert oracle.rel_frobenius(C, ref) < 1e-6
+
+
+def test_model_sddmm_and_fused_match_the_oracle(model, oracle):
+    rng = np.random.default_rng(12)
+    M, K = 40, 70
+    ro, ci = random_csr(rng, M, K, "skewed", 0.2)
+    for (D, vec, G1, DS) in [(128, 4, 8, 4), (64, 4, 8, 2), (16, 4, 4, 1), (48, 4, 8, 2), (1024, 4, 8, 0), (13, 1, 16, 0)]:
+        Q = rng.normal(0, 1, (M, D)).astype(np.float32)
+        Km = rng.normal(0, 1, (K, D)).astype(np.float32)
+        V = rng.normal(0, 1, (K, D)).astype(np.float32)
+        out = np.empty(ci.size, dtype=np.float32)
+        model.model_sddmm(M, D, pi(ro), pi(ci), pf(Q), pf(Km), vec, G1, DS, pf(out))
+        assert oracle.rel_frobenius(out, oracle.sddmm(ro, ci, Q, Km)) < 1e-6
+        scores = np.empty(ci.size, dtype=np.float32)
+        O = np.full((M, D), np.nan, dtype=np.float32)
+        writes = np.zeros((M, D), dtype=np.int32)
+        rc = model.model_fused(M, D, pi(ro), pi(ci), pf(Q), pf(Km), pf(V), 0.125, vec, G1, DS, 16, 4, 4, pf(scores), pf(O), pi(writes))
+        assert rc == 0 and (writes == 1).all()
+        assert oracle.rel_frobenius(O, oracle.fused(ro, ci, Q, Km, V, 0.125)) < 1e-6
+
+
+# ---- GPU: bit-for-bit ---------------------------------------------------------------------------------------------------
+def dev(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+GPU_SPMM = [(300, 200, 256, "skewed", 0.15), (128, 512, 128, "uniform", 0.3), (257, 129, 64, "skewed", 0.1),
+            (100, 300, 32, "uniform", 0.05), (200, 512, 392, "uniform", 0.2), (90, 64, 130, "skewed", 0.3),
+            (1000, 64, 16, "empty_rows", 0.05), (16, 700, 256, "full", 1.0), (4100, 300, 64, "skewed", 0.05)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,N,kind,density", GPU_SPMM)
+def test_gpu_spmm_equals_model_bit_for_bit(model, dl, M, K, N, kind, density):
+    import torch
+
+    rng = np.random.default_rng(21 + M + N)
+    ro, ci = random_csr(rng, M, K, kind, density)
+    va = rng.normal(0, 1, ci.size).astype(np.float32)
+    B = rng.normal(0, 1, (K, N)).astype(np.float32)
+    sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size)
+    rc, C, writes = run_spmm(model, ro, ci, va, B, sh["G"], sh["W"], sh["R"])
+    assert rc == 0 and (writes == 1).all()
+    got = dl.spmm(dev(torch, ro), dev(torch, ci), dev(torch, va), dev(torch, B), K=K).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), C.view(np.uint32)), \
+        f"shape {sh}: {np.count_nonzero(got.view(np.uint32) != C.view(np.uint32))} of {got.size} elements differ in their bits"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,D,kind,density", [(130, 257, 64, "skewed", 0.1), (256, 512, 128, "uniform", 0.05),
+                                                (50, 100, 48, "uniform", 0.2), (64, 64, 16, "uniform", 0.3),
+                                                (30, 64, 1024, "uniform", 0.3), (33, 77, 13, "uniform", 0.3)])
+def test_gpu_sddmm_and_fused_equal_model_bit_for_bit(model, dl, M, K, D, kind, density):
+    import torch
+
+    rng = np.random.default_rng(31 + M + D)
+    ro, ci = random_csr(rng, M, K, kind, density)
+    Q = rng.normal(0, 1, (M, D)).astype(np.float32)
+    Km = rng.normal(0, 1, (K, D)).astype(np.float32)
+    V = rng.normal(0, 1, (K, D)).astype(np.float32)
+    sh = dl.describe_launch(dl.OP_SDDMM, M, K, D, ci.size)
+    out = np.empty(ci.size, dtype=np.float32)
+    model.model_sddmm(M, D, pi(ro), pi(ci), pf(Q), pf(Km), sh["vec"], sh["G1"], sh["DS"], pf(out))
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    got = dl.sddmm(ro_d, ci_d, dev(torch, Q), dev(torch, Km)).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), out.view(np.uint32)), f"sddmm shape {sh}"
+
+    fs = dl.describe_launch(dl.OP_FUSED, M, K, D, ci.size)
+    scores = np.empty(ci.size, dtype=np.float32)
+    O = np.full((M, D), np.nan, dtype=np.float32)
+    writes = np.zeros((M, D), dtype=np.int32)
+    rc = model.model_fused(M, D, pi(ro), pi(ci), pf(Q), pf(Km), pf(V), 0.125, fs["vec"], fs["G1"], fs["DS"], fs["G"],
+                           fs["W"], fs["R"], pf(scores), pf(O), pi(writes))
+    assert rc == 0 and (writes == 1).all()
+    gotO = dl.fused(ro_d, ci_d, dev(torch, Q), dev(torch, Km), dev(torch, V), 0.125).cpu().numpy()
+    assert np.array_equal(gotO.view(np.uint32), O.view(np.uint32)), f"fused shape {fs}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cfg", [1, 2, 3, 5])
+def test_gpu_benchmark_configs_equal_model_bit_for_bit(model, dl, cfg):
+    import torch
+
+    c = dl.make_config(cfg)
+    ro, ci = c["row_offsets"], c["col_indices"]
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    sh = dl.describe_launch(c["op"], c["M"], c["K"], c["N"], c["nnz"])
+    if c["op"] == dl.OP_SPMM:
+        rc, C, writes = run_spmm(model, ro, ci, c["values"], c["d0"], sh["G"], sh["W"], sh["R"])
+        got = dl.spmm(ro_d, ci_d, dev(torch, c["values"]), dev(torch, c["d0"]), K=c["K"]).cpu().numpy()
+        assert rc == 0 and (writes == 1).all()
+        assert np.array_equal(got.view(np.uint32), C.view(np.uint32))
+    elif c["op"] == dl.OP_SDDMM:
+        out = np.empty(c["nnz"], dtype=np.float32)
+        model.model_sddmm(c["M"], c["N"], pi(ro), pi(ci), pf(c["d0"]), pf(c["d1"]), sh["vec"], sh["G1"], sh["DS"], pf(out))
+        got = dl.sddmm(ro_d, ci_d, dev(torch, c["d0"]), dev(torch, c["d1"])).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), out.view(np.uint32))
+    else:
+        scores = np.empty(c["nnz"], dtype=np.float32)
+        O = np.full((c["M"], c["N"]), np.nan, dtype=np.float32)
+        writes = np.zeros((c["M"], c["N"]), dtype=np.int32)
+        rc = model.model_fused(c["M"], c["N"], pi(ro), pi(ci), pf(c["d0"]), pf(c["d1"]), pf(c["d2"]), c["scale"], sh["vec"],
+                               sh["G1"], sh["DS"], sh["G"], sh["W"], sh["R"], pf(scores), pf(O), pi(writes))
+        got = dl.fused(ro_d, ci_d, dev(torch, c["d0"]), dev(torch, c["d1"]), dev(torch, c["d2"]), c["scale"]).cpu().numpy()
+        assert rc == 0 and (writes == 1).all()
+        assert np.array_equal(got.view(np.uint32), O.view(np.uint32))
