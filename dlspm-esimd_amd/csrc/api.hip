@@ -51,6 +51,10 @@ void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w
     const long long work_rows = (long long)M * col_tiles;
     W = work_rows >= 512 ? 4 : work_rows >= 256 ? 8 : 16;
     if (avg >= 1536.0) W = 16;  // very long rows: more waves per row beat the barrier cost (measured, ~8 %)
+    // few rows, each long (pruned ResNet-50 layers at small batch): four waves per row leave the device with a
+    // couple of waves per SIMD, each walking hundreds of nonzeros in sequence (measured 15-25 % slower)
+    if (work_rows < 1024 && avg >= 768.0) W = 16;
+    else if (work_rows < 1024 && avg >= 384.0 && W < 8) W = 8;
     if (W > max_w) W = max_w;
     R = 1;
     if (W == 4) {

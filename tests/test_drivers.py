@@ -137,3 +137,64 @@ def test_driver_shape_and_small_sweep():
     assert rc == 0 and "PASS" in out and "MSZ = 512 KSZ = 256 NSZ = 64" in out
     rc, out = run("sddmm_run", "--sweep", "--max-m", 1024, "--iters", 5)
     assert rc == 0 and out.count("PASS") == 6  # (1024,1024) x N in {32,128} x density in {0.3,0.2,0.1}
+
+
+DLMC = os.path.join(ROOT, "tests", "golden", "dlmc")
+DLMC_CASES = [  # file, un-padded batch size of that layer (dlmc/rn50_batchsizes.txt)
+    ("rn50_emp0.96_bottleneck_3_block_group_projection_block_group1.smtx", 3136),
+    ("rn50_emp0.98_bottleneck_2_block_group2_3_1.smtx", 784),
+    ("rn50_emp0.98_bottleneck_3_block_group3_5_1.smtx", 196),
+]
+
+
+def read_smtx(path):
+    with open(path) as f:
+        M, K, nnz = (int(x) for x in f.readline().replace(",", " ").split())
+        ro = np.array(f.readline().split(), dtype=np.int32)
+        ci = np.array(f.readline().split(), dtype=np.int32)
+    assert ro.size == M + 1 and ci.size == nnz
+    return M, K, ro, ci
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,width", DLMC_CASES)
+def test_real_dlmc_patterns_through_the_drivers_and_the_abi(oracle, dl, tmp_path, name, width):
+    """Real pruned-ResNet-50 patterns (skewed rows, empty rows) with the layer's own un-padded batch size, which the
+    reference would have to pad to a multiple of 16 (dlmc/rn50_batchsizes_noconv.txt)."""
+    import torch
+
+    path = os.path.join(DLMC, name)
+    M, K, ro, ci = read_smtx(path)
+    # the from-file driver, result dumped and checked against the oracle
+    rc, out = run("spmm_run", path, width, "--dump", tmp_path)
+    print(out)
+    assert rc == 0 and "PASS" in out and f"nnz: {ci.size}" in out
+    arr = lambda n, dt: np.fromfile(os.path.join(tmp_path, n), dtype=dt)
+    assert np.array_equal(arr("row_offsets.i32", np.int32), ro) and np.array_equal(arr("col_indices.i32", np.int32), ci)
+    ref = oracle.spmm(ro, ci, arr("values.f32", np.float32), arr("B.f32", np.float32).reshape(K, width), omp=True)
+    assert oracle.rel_frobenius(arr("C.f32", np.float32).reshape(M, width), ref) <= 1e-4
+    # the same pattern through the C ABI for SDDMM and the fused op (inner dimension 64)
+    rng = np.random.default_rng(5)
+    D = 64
+    Q = rng.normal(0, 1, (M, D)).astype(np.float32)
+    Km = rng.normal(0, 1, (K, D)).astype(np.float32)
+    V = rng.normal(0, 1, (K, D)).astype(np.float32)
+    d = lambda a: torch.from_numpy(a).cuda()
+    ro_d, ci_d = d(ro), d(ci)
+    assert dl.csr_check(M, K, ro_d, ci_d) == dl.OK
+    got = dl.sddmm(ro_d, ci_d, d(Q), d(Km)).cpu().numpy()
+    assert oracle.rel_frobenius(got, oracle.sddmm(ro, ci, Q, Km)) <= 1e-4
+    gotO = dl.fused(ro_d, ci_d, d(Q), d(Km), d(V), 0.125).cpu().numpy()
+    assert oracle.rel_frobenius(gotO, oracle.fused(ro, ci, Q, Km, V, 0.125)) <= 1e-4
+    assert (gotO[np.diff(ro) == 0] == 0).all()
+
+
+@pytest.mark.gpu
+def test_dlmc_batch_list(tmp_path):
+    """The reference's shell loop over DLMC files (SPMM/batch-run-spmm_fromfile:34-46) as one --batch run."""
+    lines = "".join(f"{os.path.join(DLMC, n)} {w}\n" for n, w in DLMC_CASES)
+    (tmp_path / "rn50.txt").write_text("# file batchsize\n" + lines)
+    for app in ("spmm_run", "sddmm_run", "fused_run"):
+        rc, out = run(app, "--batch", tmp_path / "rn50.txt", "--csv", tmp_path / f"{app}.csv", "--iters", 5)
+        assert rc == 0 and out.count("PASS") == 3, out
+        assert len(open(tmp_path / f"{app}.csv").read().strip().splitlines()) == 3

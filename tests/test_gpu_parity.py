@@ -239,6 +239,48 @@ def test_linearity_at_full_size(torch_cuda, dl, oracle):
     assert oracle.rel_frobenius(lhs.cpu().numpy(), rhs.cpu().numpy()) <= 1e-5
 
 
+def test_large_shape_against_oracle(torch_cuda, dl, oracle):
+    """The largest shape of the reference's synthetic sweep (SPMM/batch-run-spmm:9-12: M = 32768, K = 8192, N = 128,
+    here at its 10 % density) against the multi-threaded oracle: 26.8 M nonzeros."""
+    torch = torch_cuda
+    M, K, N = 32768, 8192, 128
+    ro, ci = dl.make_pattern(dl.PATTERN_UNIFORM_ROWS, 21, M, K, 0.1 * K, 0.0)
+    va = dl.fill("uniform", 22, (ci.size,), -1.0, 1.0)
+    B = dl.fill("uniform", 23, (K, N), -1.0, 1.0)
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    got = dl.spmm(ro_d, ci_d, dev(torch, va), dev(torch, B), K=K)
+    torch.cuda.synchronize()
+    assert oracle.rel_frobenius(got.cpu().numpy(), oracle.spmm(ro, ci, va, B, omp=True)) <= TOL
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
+def test_exact_integer_properties_at_large_size(torch_cuda, dl):
+    """Size-independent, bit-exact checks on 65536 skewed rows (several million nonzeros), no oracle needed: with small-integer
+    operands every fp32 product and sum is exact whatever the summation order, so
+      SpMM  with A = 1, B = 1            gives C[i, :] = length of row i,
+      SDDMM with lhs = 1, rhs[k, :] = k/D gives out[j] = col_indices[j]   (D a power of two),
+      fused with those and V = 1          gives O[i, :] = sum of row i's column indices."""
+    torch = torch_cuda
+    M, K, D = 65536, 4096, 128
+    ro, ci = dl.make_pattern(dl.PATTERN_LOGNORMAL_ROWS, 31, M, K, 64.0, 1.0)
+    lens = np.diff(ro).astype(np.int64)
+    colsum = np.add.reduceat(np.append(ci.astype(np.int64), 0), ro[:-1])[:M] * (lens > 0)
+    assert colsum.max() < 2**24
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    ones_nnz = torch.ones(ci.size, dtype=torch.float32, device="cuda")
+    ones_KD = torch.ones(K, D, dtype=torch.float32, device="cuda")
+    ones_MD = torch.ones(M, D, dtype=torch.float32, device="cuda")
+    ramp = (torch.arange(K, dtype=torch.float32, device="cuda") / D)[:, None].expand(K, D).contiguous()
+
+    C = dl.spmm(ro_d, ci_d, ones_nnz, ones_KD, K=K)
+    assert torch.equal(C, torch.from_numpy(lens.astype(np.float32)).cuda()[:, None].expand(M, D))
+    out = dl.sddmm(ro_d, ci_d, ones_MD, ramp)
+    assert torch.equal(out, ci_d.to(torch.float32))
+    O = dl.fused(ro_d, ci_d, ones_MD, ramp, ones_KD, 1.0)
+    assert torch.equal(O, torch.from_numpy(colsum.astype(np.float32)).cuda()[:, None].expand(M, D))
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
 def test_error_statuses(torch_cuda, dl):
     torch = torch_cuda
     z = torch.zeros(4, dtype=torch.int32, device="cuda")
