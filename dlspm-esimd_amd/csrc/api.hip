@@ -21,7 +21,6 @@ static int fail_hip(hipError_t e)
     return DLSPM_E_LAUNCH;
 }
 
-static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Optional launch-shape override for tuning sweeps: DLSPM_SPLIT="W,R", read at every call.
 static bool split_override(int& W, int& R)
@@ -36,7 +35,7 @@ static bool split_override(int& W, int& R)
     return false;
 }
 
-void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w, int& W, int& R)
+void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w, int slots, int& W, int& R)
 {
     static const int kPairs[][2] = {{4, 16}, {4, 8}, {4, 4}, {4, 2}, {4, 1}, {8, 4}, {8, 2}, {8, 1}, {16, 1}};
     if (split_override(W, R)) {
@@ -52,9 +51,11 @@ void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w
     W = work_rows >= 512 ? 4 : work_rows >= 256 ? 8 : 16;
     if (avg >= 1536.0) W = 16;  // very long rows: more waves per row beat the barrier cost (measured, ~8 %)
     // few rows, each long (pruned ResNet-50 layers at small batch): four waves per row leave the device with a
-    // couple of waves per SIMD, each walking hundreds of nonzeros in sequence (measured 15-25 % slower)
-    if (work_rows < 1024 && avg >= 768.0) W = 16;
-    else if (work_rows < 1024 && avg >= 384.0 && W < 8) W = 8;
+    // couple of waves per SIMD, each walking hundreds of steps in sequence (measured 15-25 % slower); a step
+    // takes `slots` nonzeros of the row at once
+    const double steps = avg / (slots > 0 ? slots : 1);
+    if (work_rows < 1024 && steps >= 768.0) W = 16;
+    else if (work_rows < 1024 && steps >= 384.0 && W < 8) W = 8;
     if (W > max_w) W = max_w;
     R = 1;
     if (W == 4) {
@@ -64,6 +65,13 @@ void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w
             R = r;
         }
     }
+}
+
+// D == 0 in SDDMM: every dot product is the empty sum (a kernel, not a memset, so that callers may capture the call)
+__global__ void fill_zero_kernel(float* __restrict__ out, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = 0.f;
 }
 
 // ---- device-side CSR check ------------------------------------------------------------------------
@@ -110,7 +118,7 @@ int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int
     if (M == 0 || N == 0) return DLSPM_OK;
     if (!row_offsets || !C) return DLSPM_E_INVALID_ARG;
     if (nnz > 0 && (!col_indices || !values || !B)) return DLSPM_E_INVALID_ARG;
-    const bool vec4 = (N % 4 == 0) && aligned16(B) && aligned16(C);
+    const bool vec4 = N >= 4;  // dwordx4 accesses need only dword alignment
     const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C};
     const SpmmShape shape = spmm_choose(M, N, nnz, vec4);
     const hipError_t e = spmm_launch(args, shape, static_cast<hipStream_t>(stream));
@@ -126,8 +134,14 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
     if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
     if (M == 0 || nnz == 0) return DLSPM_OK;
     if (!row_offsets || !col_indices || !out_values) return DLSPM_E_INVALID_ARG;
-    if (D > 0 && (!lhs || !rhs)) return DLSPM_E_INVALID_ARG;  // D == 0: every dot product is the empty sum, 0
-    const bool vec4 = (D % 4 == 0) && D > 0 && aligned16(lhs) && aligned16(rhs);
+    if (D > 0 && (!lhs || !rhs)) return DLSPM_E_INVALID_ARG;
+    if (D == 0) {
+        const unsigned blocks = (unsigned)((nnz + 255) / 256);
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), out_values, nnz);
+        const hipError_t e0 = hipGetLastError();
+        return e0 == hipSuccess ? DLSPM_OK : fail_hip(e0);
+    }
+    const bool vec4 = D >= 4;  // dwordx4 accesses need only dword alignment
     const SddmmShape shape = sddmm_choose(M, D, nnz, vec4);
     const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values};
     const hipError_t e = sddmm_launch(args, shape, static_cast<hipStream_t>(stream));
@@ -145,7 +159,7 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz, const int* row_offsets, c
     if (M == 0 || D == 0) return DLSPM_OK;
     if (!row_offsets || !O) return DLSPM_E_INVALID_ARG;
     if (nnz > 0 && (!col_indices || !Q || !Kmat || !V)) return DLSPM_E_INVALID_ARG;
-    const bool vec4 = (D % 4 == 0) && aligned16(Q) && aligned16(Kmat) && aligned16(V) && aligned16(O);
+    const bool vec4 = D >= 4;
     const FusedShape shape = fused_choose(M, D, nnz, vec4);
     const FusedArgs args{M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O};
     const hipError_t e = fused_launch(args, shape, static_cast<hipStream_t>(stream));
@@ -186,12 +200,12 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
     return h_flags == 0 ? DLSPM_OK : DLSPM_E_INVALID_CSR;
 }
 
-int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int aligned16, int* shape)
+int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape)
 {
     (void)K;
     if (!shape || M < 0 || N_or_D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     const int n = N_or_D;
-    const bool vec4 = aligned16 != 0 && n > 0 && n % 4 == 0;
+    const bool vec4 = n >= 4;
     for (int i = 0; i < 8; ++i) shape[i] = 0;
     if (op == DLSPM_OP_SPMM) {
         const SpmmShape s = spmm_choose(M, n, nnz, vec4);

@@ -11,11 +11,37 @@ constexpr int kWave = 64;
 
 // ---- VEC floats per lane: dwordx4 (VEC = 4) or dword (VEC = 1) global accesses --------------------
 template <int VEC> struct Vec;
+// four floats that need only 4-byte alignment: global_load/store_dwordx4 accept any dword address
+typedef float float4_dword_aligned __attribute__((ext_vector_type(4), aligned(4)));
 template <> struct Vec<4> {
     float4 v;
     __device__ __forceinline__ static Vec zero() { return Vec{make_float4(0.f, 0.f, 0.f, 0.f)}; }
+    // 16-byte aligned address (LDS)
     __device__ __forceinline__ static Vec load(const float* p) { return Vec{*reinterpret_cast<const float4*>(p)}; }
     __device__ __forceinline__ void store(float* p) const { *reinterpret_cast<float4*>(p) = v; }
+    // any float address (global memory): rows of a dense operand whose width is not a multiple of 4 floats
+    __device__ __forceinline__ static Vec gload(const float* p)
+    {
+        const float4_dword_aligned t = *reinterpret_cast<const float4_dword_aligned*>(p);
+        return Vec{make_float4(t.x, t.y, t.z, t.w)};
+    }
+    __device__ __forceinline__ void gstore(float* p) const
+    {
+        float4_dword_aligned t = {v.x, v.y, v.z, v.w};
+        *reinterpret_cast<float4_dword_aligned*>(p) = t;
+    }
+    // elements [d, d+4) of a row of D >= 4 floats, d < D, for sums over the row: a lane whose four elements
+    // would run past D reads the last four instead and zeroes the ones its left neighbour already covers
+    __device__ __forceinline__ static Vec gload_clip(const float* row, int d, int D)
+    {
+        const int dl = min(d, D - 4);
+        Vec t = gload(row + dl);
+        const int ov = d - dl;
+        t.v.x = ov > 0 ? 0.f : t.v.x;
+        t.v.y = ov > 1 ? 0.f : t.v.y;
+        t.v.z = ov > 2 ? 0.f : t.v.z;
+        return t;
+    }
     __device__ __forceinline__ void fma(float a, const Vec& b)
     {
         v.x = fmaf(a, b.v.x, v.x); v.y = fmaf(a, b.v.y, v.y); v.z = fmaf(a, b.v.z, v.z); v.w = fmaf(a, b.v.w, v.w);
@@ -32,6 +58,9 @@ template <> struct Vec<1> {
     __device__ __forceinline__ static Vec zero() { return Vec{0.f}; }
     __device__ __forceinline__ static Vec load(const float* p) { return Vec{*p}; }
     __device__ __forceinline__ void store(float* p) const { *p = v; }
+    __device__ __forceinline__ static Vec gload(const float* p) { return Vec{*p}; }
+    __device__ __forceinline__ void gstore(float* p) const { *p = v; }
+    __device__ __forceinline__ static Vec gload_clip(const float* row, int d, int) { return Vec{row[d]}; }
     __device__ __forceinline__ void fma(float a, const Vec& b) { v = fmaf(a, b.v, v); }
     __device__ __forceinline__ void add(const Vec& b) { v += b.v; }
     __device__ __forceinline__ float dot(const Vec& b, float acc) const { return fmaf(v, b.v, acc); }
@@ -138,7 +167,7 @@ __device__ __forceinline__ void dense_rows_fma(Vec<VEC>* acc, int c, float av, i
             }
             const float* row = dense + (size_t)cj * ld;
 #pragma unroll
-            for (int v = 0; v < V; ++v) bv[u][v] = VecT::load(row + colv[v]);
+            for (int v = 0; v < V; ++v) bv[u][v] = VecT::gload(row + colv[v]);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
@@ -162,7 +191,7 @@ __device__ __forceinline__ void dense_rows_fma(Vec<VEC>* acc, int c, float av, i
                 }
                 const float* row = dense + (size_t)cj * ld;
 #pragma unroll
-                for (int v = 0; v < V; ++v) bv[u][v] = VecT::load(row + colv[v]);
+                for (int v = 0; v < V; ++v) bv[u][v] = VecT::gload(row + colv[v]);
             }
         }
 #pragma unroll
@@ -181,7 +210,7 @@ __device__ __forceinline__ void dense_rows_fma(Vec<VEC>* acc, int c, float av, i
             const float* row = dense + (size_t)cj * ld;
             VecT bv[V];
 #pragma unroll
-            for (int v = 0; v < V; ++v) bv[v] = VecT::load(row + colv[v]);
+            for (int v = 0; v < V; ++v) bv[v] = VecT::gload(row + colv[v]);
             if (jj < cnt) {
 #pragma unroll
                 for (int v = 0; v < V; ++v) acc[v].fma(aj, bv[v]);
@@ -211,7 +240,8 @@ template <int VEC, int G, int V> __device__ __forceinline__ void slots_sum(Vec<V
 // ---- sampled dot products (SDDMM kernel and stage 1 of the fused kernel) -------------------------------
 // One round: the lane group handling nonzero `n` of the chunk (column index fetched from lane n) reads
 // that rhs row against the lhs row and returns the group's dot product in all of its lanes.
-// MASKED: D is not a multiple of G1*VEC*DS, lanes past D read a safe in-row address and contribute 0.
+// MASKED: D is not G1*VEC*DS; lanes past D read a safe in-row address and contribute 0, the lane that straddles D
+// reads the row's last VEC floats with the overlap zeroed.
 template <int VEC, int G1, int DS, bool MASKED>
 __device__ __forceinline__ void sddmm_rounds_load(int D, int g, const float* __restrict__ rhs, int cn, Vec<VEC>* x)
 {
@@ -220,10 +250,10 @@ __device__ __forceinline__ void sddmm_rounds_load(int D, int g, const float* __r
     for (int s = 0; s < DS; ++s) {
         const int d = (s * G1 + g) * VEC;
         if constexpr (MASKED) {
-            x[s] = Vec<VEC>::load(rrow + (d < D ? d : 0));
+            x[s] = Vec<VEC>::gload_clip(rrow, d < D ? d : 0, D);
             if (d >= D) x[s] = Vec<VEC>::zero();  // not 0 * (whatever sits at column 0): that could be 0 * inf
         } else {
-            x[s] = Vec<VEC>::load(rrow + d);
+            x[s] = Vec<VEC>::gload(rrow + d);
         }
     }
 }
@@ -231,7 +261,7 @@ __device__ __forceinline__ void sddmm_rounds_load(int D, int g, const float* __r
 // One chunk of `cnt` <= 64 nonzeros of one row: returns in lane l the dot product of the chunk's nonzero l
 // (lanes past the chunk return an unspecified value that the caller must not store). `c` is the lane's
 // column index (0 past the chunk). `lq` holds the lhs row as laid out by the caller:
-// lq[s] = lhs_row[(s*G1 + g)*VEC ..], zero past D. With DS = 0 the row is re-read from lhs_row.
+// lq[s] = lhs_row[(s*G1 + g)*VEC ..] (Vec::gload_clip), zero past D. With DS = 0 the row is re-read from lhs_row.
 template <int VEC, int G1, int DS, bool MASKED>
 __device__ __forceinline__ float sddmm_chunk(int D, int lane, int cnt, int c, const float* __restrict__ lhs_row,
                                              const Vec<VEC>* lq, const float* __restrict__ rhs)
@@ -289,7 +319,8 @@ __device__ __forceinline__ float sddmm_chunk(int D, int lane, int cnt, int c, co
             const int cn = lane_get(c, (t * P + grp) & 63);
             const float* rrow = rhs + (size_t)cn * D;
             float dot = 0.f;
-            for (int d = g * VEC; d < D; d += G1 * VEC) dot = VecT::load(lhs_row + d).dot(VecT::load(rrow + d), dot);
+            for (int d = g * VEC; d < D; d += G1 * VEC)
+                dot = VecT::gload_clip(lhs_row, d, D).dot(VecT::gload_clip(rrow, d, D), dot);
             dot = group_sum<G1>(dot);
             if (g == t) res = dot;
         }

@@ -18,7 +18,8 @@
 
 namespace dlspm {
 
-template <int VEC, int G1, int DS, int G, int V2, int W, int R>
+// MASKED = false: D == G1 * VEC * DS exactly, every stage-1 access of every lane falls inside the row.
+template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R>
 __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_tiles, float scale,
                                                        const int* __restrict__ row_offsets,
                                                        const int* __restrict__ col_indices,
@@ -52,9 +53,8 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
     for (int v = 0; v < V2; ++v) {
         const int col = ct * TW + (v * G + g) * VEC;
         act[v] = col < D;
-        colv[v] = act[v] ? col : 0;
+        colv[v] = act[v] ? min(col, D - VEC) : 0;  // a lane that would run past D repeats its neighbour's columns
     }
-    const bool exact = DS > 0 && D == G1 * VEC * DS;
 
     const int T0 = s_off[0];
     const int T = s_off[nr] - T0;
@@ -78,7 +78,8 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
 #pragma unroll
                 for (int s = 0; s < DS; ++s) {
                     const int d = (s * G1 + g1) * VEC;
-                    lq[s] = d < D ? VecT::load(q_row + d) : VecT::zero();
+                    if constexpr (MASKED) lq[s] = d < D ? VecT::gload_clip(q_row, d, D) : VecT::zero();
+                    else lq[s] = VecT::gload(q_row + d);
                 }
             }
             VecT acc[V2];
@@ -91,8 +92,7 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
                 c_nxt = col_indices[min(base + kWave + lane, q - 1)];
                 const int cnt = min(kWave, q - base);
                 // stage 1: lane l <- score of nonzero base + l (fp32, as between the reference's two loops)
-                float score = exact ? sddmm_chunk<VEC, G1, DS, false>(D, lane, cnt, c, q_row, lq, Kmat)
-                                    : sddmm_chunk<VEC, G1, DS, true>(D, lane, cnt, c, q_row, lq, Kmat);
+                float score = sddmm_chunk<VEC, G1, DS, MASKED>(D, lane, cnt, c, q_row, lq, Kmat);
                 score = base + lane < q ? score * scale : 0.f;
                 // stage 2: acc += score_j * V[col_j, :]
                 dense_rows_fma<VEC, G, V2>(acc, c, score, cnt, Vmat, D, colv, lane);
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
                     float* orow = O + (size_t)(r0 + r) * D;
 #pragma unroll
                     for (int v = 0; v < V2; ++v)
-                        if (act[v]) acc[v].store(orow + colv[v]);
+                        if (act[v]) acc[v].gstore(orow + colv[v]);
                 } else {
                     float* part = s_part[w][(NP == 1 || p == a) ? 0 : 1];
 #pragma unroll
@@ -127,7 +127,7 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
             if (rs == re) {
 #pragma unroll
                 for (int v = 0; v < V2; ++v)
-                    if (act[v]) VecT::zero().store(orow + colv[v]);
+                    if (act[v]) VecT::zero().gstore(orow + colv[v]);
                 continue;
             }
             const int wl = (rs - T0) / per;
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
                     const int k = (NP == 2 && x == wl && T0 + x * per != rs) ? 1 : 0;
                     sum.add(VecT::load(&s_part[x][k][(v * G + g) * VEC]));
                 }
-                if (act[v]) sum.store(orow + colv[v]);
+                if (act[v]) sum.gstore(orow + colv[v]);
             }
         }
     }
@@ -156,7 +156,15 @@ static hipError_t launch_one(const FusedArgs& x, hipStream_t stream)
     const long long blocks = (long long)((x.M + R - 1) / R) * col_tiles;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream,
+    if constexpr (DS > 0) {
+        if (x.D == G1 * VEC * DS) {
+            hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, false, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64),
+                               0, stream, x.M, x.D, col_tiles, x.scale, x.row_offsets, x.col_indices, x.Q, x.Kmat, x.V,
+                               x.O);
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, true, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream,
                        x.M, x.D, col_tiles, x.scale, x.row_offsets, x.col_indices, x.Q, x.Kmat, x.V, x.O);
     return hipGetLastError();
 }
@@ -193,11 +201,11 @@ FusedShape fused_choose(int M, int D, int nnz, bool vec4)
         else if (D <= 256) { s.G1 = 8; s.DS = 8; s.G = 64; s.V = 1; }
         else if (D <= 512) { s.G1 = 8; s.DS = 16; s.G = 64; s.V = 2; }
         else { s.G1 = 8; s.DS = 0; s.G = 64; s.V = 4; }  // wider D: column tiles of 1024, scores recomputed per tile
-    } else {
-        s.G1 = 16; s.DS = 0; s.G = 64; s.V = 4;
+    } else {  // D < 4: one float per lane
+        s.G1 = 4; s.DS = 1; s.G = 8; s.V = 1;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(M, (D + tw - 1) / tw, nnz, 512, tw >= 1024 ? 4 : 16, s.W, s.R);
+    choose_split(M, (D + tw - 1) / tw, nnz, 512, tw >= 1024 ? 4 : 16, kWave / s.G, s.W, s.R);
     return s;
 }
 
@@ -211,8 +219,8 @@ hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t str
         if (s.G1 == 8 && s.DS == 8 && s.G == 64 && s.V == 1) return launch_wr<4, 8, 8, 64, 1>(x, s.W, s.R, stream);
         if (s.G1 == 8 && s.DS == 16 && s.G == 64 && s.V == 2) return launch_wr<4, 8, 16, 64, 2>(x, s.W, s.R, stream);
         if (s.G1 == 8 && s.DS == 0 && s.G == 64 && s.V == 4) return launch_wr<4, 8, 0, 64, 4>(x, s.W, s.R, stream);
-    } else if (s.G1 == 16 && s.DS == 0 && s.G == 64 && s.V == 4) {
-        return launch_wr<1, 16, 0, 64, 4>(x, s.W, s.R, stream);
+    } else if (s.G1 == 4 && s.DS == 1 && s.G == 8 && s.V == 1) {
+        return launch_wr<1, 4, 1, 8, 1>(x, s.W, s.R, stream);
     }
     return hipErrorInvalidValue;
 }

@@ -6,7 +6,7 @@
 namespace dlspm {
 
 // Lane layout and work split of one launch.
-//   vec : floats per lane per access (4 = dwordx4, 1 = dword)
+//   vec : floats per lane per access (4 = dwordx4 when the dense width is at least 4, else 1 = dword)
 //   G   : lanes covering one dense row (SpMM / fused stage 2)          V  : accesses per lane per dense row
 //   G1  : lanes covering one dot product (SDDMM / fused stage 1)        DS : accesses per lane per dot
 //         product (0 = run-time loop, lhs row re-read instead of kept in registers)
@@ -52,7 +52,8 @@ FusedShape fused_choose(int M, int D, int nnz, bool vec4);
 hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream);
 
 // Picks (W, R), W <= max_w: waves per workgroup from the number of rows, rows per workgroup as large as keeps
-// `min_blocks` workgroups in the grid. Only the pairs the kernels are instantiated for are returned.
-void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w, int& W, int& R);
+// `min_blocks` workgroups in the grid. `slots` = nonzeros of a row a wave works on at once (64 / G).
+// Only the pairs the kernels are instantiated for are returned.
+void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w, int slots, int& W, int& R);
 
 }  // namespace dlspm

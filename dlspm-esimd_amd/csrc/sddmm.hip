@@ -18,7 +18,8 @@
 
 namespace dlspm {
 
-template <int VEC, int G1, int DS, int W, int R>
+// MASKED = false: D == G1 * VEC * DS exactly, every access of every lane falls inside the row.
+template <int VEC, int G1, int DS, bool MASKED, int W, int R>
 __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* __restrict__ row_offsets,
                                                        const int* __restrict__ col_indices,
                                                        const float* __restrict__ lhs, const float* __restrict__ rhs,
@@ -42,7 +43,6 @@ __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* 
     const int a = __builtin_amdgcn_readfirstlane(T0 + min(T, w * per));
     const int b = __builtin_amdgcn_readfirstlane(T0 + min(T, (w + 1) * per));
     if (a >= b) return;
-    const bool exact = DS > 0 && D == G1 * VEC * DS;  // every lane's accesses fall inside the row
 
     int r = 0;
     while (s_off[r + 1] <= a) ++r;
@@ -57,7 +57,8 @@ __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* 
 #pragma unroll
             for (int s = 0; s < DS; ++s) {
                 const int d = (s * G1 + g) * VEC;
-                lq[s] = d < D ? VecT::load(lhs_row + d) : VecT::zero();
+                if constexpr (MASKED) lq[s] = d < D ? VecT::gload_clip(lhs_row, d, D) : VecT::zero();
+                else lq[s] = VecT::gload(lhs_row + d);
             }
         }
         // 64 column indices per pass, one per lane; the next 64 are requested (index clamped, no condition) before
@@ -67,8 +68,7 @@ __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* 
             const int c = base + lane < q ? c_nxt : 0;
             c_nxt = col_indices[min(base + kWave + lane, q - 1)];
             const int cnt = min(kWave, q - base);
-            const float o = exact ? sddmm_chunk<VEC, G1, DS, false>(D, lane, cnt, c, lhs_row, lq, rhs)
-                                  : sddmm_chunk<VEC, G1, DS, true>(D, lane, cnt, c, lhs_row, lq, rhs);
+            const float o = sddmm_chunk<VEC, G1, DS, MASKED>(D, lane, cnt, c, lhs_row, lq, rhs);
             if (base + lane < q) out[base + lane] = o;
         }
         pos = q;
@@ -84,7 +84,14 @@ static hipError_t launch_one(const SddmmArgs& x, hipStream_t stream)
 {
     const int blocks = (x.M + R - 1) / R;
     if (blocks <= 0) return hipSuccess;
-    hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M, x.D,
+    if constexpr (DS > 0) {
+        if (x.D == G1 * VEC * DS) {
+            hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, false, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M,
+                               x.D, x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, true, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M, x.D,
                        x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
     return hipGetLastError();
 }
@@ -117,11 +124,11 @@ SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4)
             s.G1 = 8;
             s.DS = D <= 32 ? 1 : D <= 64 ? 2 : D <= 128 ? 4 : D <= 256 ? 8 : D <= 512 ? 16 : 0;
         }
-    } else {
-        s.G1 = 16;
-        s.DS = 0;
+    } else {  // D < 4: one float per lane
+        s.G1 = 4;
+        s.DS = 1;
     }
-    choose_split(M, 1, nnz, 512, 16, s.W, s.R);
+    choose_split(M, 1, nnz, 512, 16, kWave / s.G1, s.W, s.R);
     return s;
 }
 
@@ -139,8 +146,8 @@ hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t str
                 case 0: return launch_wr<4, 8, 0>(x, s.W, s.R, stream);
             }
         }
-    } else if (s.G1 == 16 && s.DS == 0) {
-        return launch_wr<1, 16, 0>(x, s.W, s.R, stream);
+    } else if (s.G1 == 4 && s.DS == 1) {
+        return launch_wr<1, 4, 1>(x, s.W, s.R, stream);
     }
     return hipErrorInvalidValue;
 }

@@ -51,8 +51,10 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
 #pragma unroll
     for (int v = 0; v < V; ++v) {
         const int col = ct * TW + (v * G + g) * VEC;
-        act[v] = col < N;  // N % VEC == 0, so a lane's VEC columns are inside or outside together
-        colv[v] = act[v] ? col : 0;
+        act[v] = col < N;
+        // a lane whose VEC columns would run past N moves back to end at N: it then repeats columns of its
+        // left neighbour, with the same operations, and stores the same values there (N >= VEC)
+        colv[v] = act[v] ? min(col, N - VEC) : 0;
     }
 
     const int T0 = s_off[0];
@@ -97,7 +99,7 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
                     float* crow = C + (size_t)(r0 + r) * N;
 #pragma unroll
                     for (int v = 0; v < V; ++v)
-                        if (act[v]) acc[v].store(crow + colv[v]);
+                        if (act[v]) acc[v].gstore(crow + colv[v]);
                 } else {
                     float* part = s_part[w][(NP == 1 || p == a) ? 0 : 1];
 #pragma unroll
@@ -120,7 +122,7 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
             if (rs == re) {
 #pragma unroll
                 for (int v = 0; v < V; ++v)
-                    if (act[v]) VecT::zero().store(crow + colv[v]);
+                    if (act[v]) VecT::zero().gstore(crow + colv[v]);
                 continue;
             }
             const int wl = (rs - T0) / per;
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
                     const int k = (NP == 2 && x == wl && T0 + x * per != rs) ? 1 : 0;
                     sum.add(VecT::load(&s_part[x][k][(v * G + g) * VEC]));
                 }
-                if (act[v]) sum.store(crow + colv[v]);
+                if (act[v]) sum.gstore(crow + colv[v]);
             }
         }
     }
@@ -183,12 +185,12 @@ SpmmShape spmm_choose(int M, int N, int nnz, bool vec4)
         else if (N > 64) { s.G = 32; s.V = 1; }
         else if (N > 32) { s.G = 16; s.V = 1; }
         else { s.G = 8; s.V = 1; }
-    } else {
-        s.G = 64;
-        s.V = N > 64 ? 4 : 1;
+    } else {  // N < 4: one float per lane, eight nonzeros per access
+        s.G = 8;
+        s.V = 1;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(M, (N + tw - 1) / tw, nnz, 2048, 16, s.W, s.R);
+    choose_split(M, (N + tw - 1) / tw, nnz, 2048, 16, kWave / s.G, s.W, s.R);
     return s;
 }
 
@@ -201,8 +203,7 @@ hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream
         if (s.G == 16 && s.V == 1) return launch_wr<4, 16, 1>(x, s.W, s.R, stream);
         if (s.G == 8 && s.V == 1) return launch_wr<4, 8, 1>(x, s.W, s.R, stream);
     } else {
-        if (s.G == 64 && s.V == 1) return launch_wr<1, 64, 1>(x, s.W, s.R, stream);
-        if (s.G == 64 && s.V == 4) return launch_wr<1, 64, 4>(x, s.W, s.R, stream);
+        if (s.G == 8 && s.V == 1) return launch_wr<1, 8, 1>(x, s.W, s.R, stream);
     }
     return hipErrorInvalidValue;
 }

@@ -61,7 +61,7 @@ def lib() -> ctypes.CDLL:
         L.dlspm_workspace_bytes.restype = sz
         L.dlspm_csr_check.argtypes = [ci, ci, ci, vp, vp, vp]
         L.dlspm_csr_check.restype = ci
-        L.dlspm_describe_launch.argtypes = [ci, ci, ci, ci, ci, ci, ctypes.POINTER(ci)]
+        L.dlspm_describe_launch.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci)]
         L.dlspm_describe_launch.restype = ci
         L.dlspm_status_string.argtypes = [ci]
         L.dlspm_status_string.restype = ctypes.c_char_p
@@ -152,10 +152,10 @@ def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None):
     return out
 
 
-def describe_launch(op: int, M: int, K: int, N: int, nnz: int, aligned16: bool = True) -> dict:
+def describe_launch(op: int, M: int, K: int, N: int, nnz: int) -> dict:
     """Launch shape the library uses for these sizes: {'vec','G','V','G1','DS','W','R','col_tiles'} (host only)."""
     out = (ctypes.c_int * 8)()
-    st = lib().dlspm_describe_launch(op, M, K, N, nnz, 1 if aligned16 else 0, out)
+    st = lib().dlspm_describe_launch(op, M, K, N, nnz, out)
     if st != OK:
         raise DlspmError(st, "dlspm_describe_launch")
     return dict(zip(("vec", "G", "V", "G1", "DS", "W", "R", "col_tiles"), (int(x) for x in out)))

@@ -16,9 +16,10 @@
  *     SPMM/spmmesimd2.hpp:90-91, SPMM/spmm-esimd-fromfile2.cpp:196);
  *   - no input needs padding (the reference over-allocates col/val by 2*VLC for its unmasked tail
  *     loads, SPMM/spmm-esimd-fromfile2.cpp:174-176);
- *   - any N / D >= 1 is accepted (the reference rejects N % 16 != 0,
- *     SPMM/spmm-esimd-fromfile2.cpp:230-231); multiples of 4 with 16-byte aligned dense operands
- *     take the dwordx4 path, everything else a scalar-load path of the same kernels;
+ *   - any N / D >= 1 and any float-aligned dense operand is accepted (the reference rejects
+ *     N % 16 != 0, SPMM/spmm-esimd-fromfile2.cpp:230-231): every width of at least 4 takes the
+ *     dwordx4 path (those accesses need only dword alignment; a row's last lane reads and writes the
+ *     row's last four floats), widths 1 to 3 a dword path of the same kernels;
  *   - results are deterministic: no floating-point atomics (the reference's SDDMM v4 uses them,
  *     SDDMM/sddmm-esimd-fromfile_v4.hpp:161,175);
  *   - errors are returned as a negative status, nothing is thrown across the ABI (the reference
@@ -111,13 +112,12 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
  * Launch shape the library would use for these sizes, for tuning reports and for host-side models of the
  * schedule (the reference's SpmmEsimdCPU / FusedEsimdCPU, SPMM/spmm-esimd-v1.cpp:83-169 and
  * FUSED/fused.cpp:93-216, play that role for its kernels). Host-only, never touches the device.
- * `aligned16` says whether the dense operands are 16-byte aligned (the dwordx4 path needs that and N_or_D % 4 == 0).
  * shape[8] receives: [0] floats per lane per access (4 or 1), [1] G lanes per dense row (SpMM, fused stage 2; 0 for
  * SDDMM), [2] accesses per lane per dense row, [3] G1 lanes per dot product (SDDMM, fused stage 1; 0 for SpMM),
  * [4] accesses per lane per dot product (0 = run-time loop), [5] waves per workgroup, [6] rows per workgroup,
  * [7] column tiles. Returns DLSPM_OK or DLSPM_E_INVALID_ARG.
  */
-int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int aligned16, int* shape);
+int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape);
 
 /* Human-readable text for a status code (never NULL). */
 const char* dlspm_status_string(int status);

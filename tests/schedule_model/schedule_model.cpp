@@ -103,7 +103,8 @@ int model_rows(int M, int N, const int* ro, const int* ci, const float* va, cons
 }
 
 // dot product of one nonzero as the SDDMM lane group computes it: lane g accumulates its elements in order with
-// fused multiply-adds, then the G1 lanes are added pairwise (lane^1, lane^2, then the mirrored halves)
+// fused multiply-adds, then the G1 lanes are added pairwise (lane^1, lane^2, then the mirrored halves). Positions
+// past D contribute fma(0, 0, acc) = acc, wherever the kernel places them in a lane's sequence.
 float model_dot(const float* l, const float* r, int D, int vec, int G1, int DS)
 {
     std::vector<float> lane(G1, 0.0f);
@@ -118,7 +119,8 @@ float model_dot(const float* l, const float* r, int D, int vec, int G1, int DS)
             }
         } else {
             for (int d = g * vec; d < D; d += G1 * vec)
-                for (int e = 0; e < vec; ++e) acc = std::fmaf(l[d + e], r[d + e], acc);
+                for (int e = 0; e < vec; ++e)
+                    if (d + e < D) acc = std::fmaf(l[d + e], r[d + e], acc);
         }
         lane[g] = acc;
     }

@@ -56,6 +56,18 @@ SPMM_CASES = [
     (1500, 1024, 96, "uniform", 0.1),
     (2000, 300, 40, "empty_rows", 0.4),
     (300, 512, 64, "full", 1.0),
+    # widths that are not a multiple of 4: the row's last lane works on the last four floats; 1 to 3: dword path
+    (70, 90, 5, "uniform", 0.3),
+    (70, 90, 6, "skewed", 0.3),
+    (64, 128, 49, "skewed", 0.2),
+    (64, 128, 50, "uniform", 0.2),
+    (33, 64, 129, "uniform", 0.3),
+    (20, 64, 258, "uniform", 0.3),
+    (10, 64, 1026, "uniform", 0.3),
+    (12, 64, 1030, "skewed", 0.3),
+    (50, 80, 2, "uniform", 0.3),
+    (50, 80, 3, "empty_rows", 0.3),
+    (300, 80, 1, "skewed", 0.3),
 ]
 
 
@@ -98,6 +110,21 @@ SDDMM_CASES = [
     (200, 300, 128, "empty_rows", 0.1),
     (8, 1500, 128, "full", 1.0),
     (20, 40, 0, "uniform", 0.3),
+    # inner dimensions that are not a multiple of 4 (the straddling lane reads the last four floats, overlap zeroed)
+    (40, 60, 2, "uniform", 0.3),
+    (40, 60, 3, "skewed", 0.3),
+    (40, 60, 5, "uniform", 0.3),
+    (40, 60, 6, "uniform", 0.3),
+    (40, 60, 7, "empty_rows", 0.3),
+    (40, 60, 17, "uniform", 0.3),
+    (40, 60, 33, "skewed", 0.3),
+    (40, 60, 49, "uniform", 0.3),
+    (40, 60, 63, "uniform", 0.3),
+    (40, 60, 65, "uniform", 0.3),
+    (40, 60, 130, "skewed", 0.3),
+    (40, 60, 257, "uniform", 0.3),
+    (30, 60, 513, "uniform", 0.3),
+    (20, 60, 1027, "uniform", 0.3),
 ]
 
 
@@ -135,6 +162,18 @@ FUSED_CASES = [
     (200, 300, 64, "empty_rows", 0.1, 0.125),
     (8, 1500, 64, "full", 1.0, 0.125),
     (64, 128, 64, "empty", 0.0, 1.0),
+    (40, 60, 1, "uniform", 0.3, 1.0),
+    (40, 60, 2, "uniform", 0.3, 0.5),
+    (40, 60, 3, "skewed", 0.3, 1.0),
+    (40, 60, 5, "uniform", 0.3, 1.0),
+    (40, 60, 7, "empty_rows", 0.3, 0.5),
+    (40, 60, 17, "uniform", 0.3, 1.0),
+    (40, 60, 49, "skewed", 0.3, 0.125),
+    (40, 60, 65, "uniform", 0.3, 1.0),
+    (40, 60, 130, "uniform", 0.3, 1.0),
+    (40, 60, 257, "skewed", 0.3, 1.0),
+    (30, 60, 513, "uniform", 0.3, 1.0),
+    (20, 60, 1027, "uniform", 0.3, 1.0),
 ]
 
 
@@ -198,21 +237,37 @@ def test_benchmark_configs_full_size(torch_cuda, dl, oracle, cfg):
     assert dl.csr_check(c["M"], c["K"], ro_d, ci_d) == dl.OK
 
 
-def test_misaligned_operands_take_scalar_path(torch_cuda, dl, oracle):
-    """Dense operands that start 4 bytes off a 16-byte boundary must still give the right answer."""
+@pytest.mark.parametrize("off", [1, 2, 3])
+def test_misaligned_operands(torch_cuda, dl, oracle, off):
+    """Dense operands and outputs that start 4, 8 or 12 bytes off a 16-byte boundary (dwordx4 accesses need only
+    dword alignment), all three entry points, widths that are and are not multiples of 4."""
     torch = torch_cuda
-    rng = np.random.default_rng(77)
-    M, K, N = 60, 90, 64
-    ro, ci = random_csr(rng, M, K, "uniform", 0.2)
-    va = rng.uniform(-1, 1, ci.size).astype(np.float32)
-    B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
-    buf = torch.empty(K * N + 1, dtype=torch.float32, device="cuda")
-    Bd = buf[1:].view(K, N)
-    Bd.copy_(torch.from_numpy(B))
-    assert Bd.data_ptr() % 16 != 0
-    got = dl.spmm(dev(torch, ro), dev(torch, ci), dev(torch, va), Bd, K=K)
-    torch.cuda.synchronize()
-    assert oracle.rel_frobenius(got.cpu().numpy(), oracle.spmm(ro, ci, va, B)) <= TOL
+    rng = np.random.default_rng(77 + off)
+
+    def shifted(a):
+        buf = torch.empty(a.size + off, dtype=torch.float32, device="cuda")
+        view = buf[off:].view(*a.shape)
+        view.copy_(torch.from_numpy(a))
+        assert view.data_ptr() % 16 == 4 * off
+        return view
+
+    for N in (64, 50):
+        M, K = 60, 90
+        ro, ci = random_csr(rng, M, K, "skewed", 0.2)
+        va = rng.uniform(-1, 1, ci.size).astype(np.float32)
+        B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+        Q = rng.normal(0, 1, (M, N)).astype(np.float32)
+        V = rng.normal(0, 1, (K, N)).astype(np.float32)
+        ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+        C = shifted(np.full((M, N), np.nan, dtype=np.float32))
+        dl.spmm(ro_d, ci_d, shifted(va), shifted(B), K=K, out=C)
+        assert oracle.rel_frobenius(C.cpu().numpy(), oracle.spmm(ro, ci, va, B)) <= TOL
+        out = shifted(np.full(ci.size, np.nan, dtype=np.float32))
+        dl.sddmm(ro_d, ci_d, shifted(Q), shifted(B), out=out)
+        assert oracle.rel_frobenius(out.cpu().numpy(), oracle.sddmm(ro, ci, Q, B)) <= TOL
+        O = shifted(np.full((M, N), np.nan, dtype=np.float32))
+        dl.fused(ro_d, ci_d, shifted(Q), shifted(B), shifted(V), 0.5, out=O)
+        assert oracle.rel_frobenius(O.cpu().numpy(), oracle.fused(ro, ci, Q, B, V, 0.5)) <= TOL
 
 
 def test_deterministic(torch_cuda, dl):

@@ -99,7 +99,9 @@ def dev(torch, a):
 
 GPU_SPMM = [(300, 200, 256, "skewed", 0.15), (128, 512, 128, "uniform", 0.3), (257, 129, 64, "skewed", 0.1),
             (100, 300, 32, "uniform", 0.05), (200, 512, 392, "uniform", 0.2), (90, 64, 130, "skewed", 0.3),
-            (1000, 64, 16, "empty_rows", 0.05), (16, 700, 256, "full", 1.0), (4100, 300, 64, "skewed", 0.05)]
+            (1000, 64, 16, "empty_rows", 0.05), (16, 700, 256, "full", 1.0), (4100, 300, 64, "skewed", 0.05),
+            (64, 128, 49, "skewed", 0.2), (70, 90, 5, "uniform", 0.3), (10, 64, 1026, "uniform", 0.3),
+            (300, 80, 1, "skewed", 0.3), (50, 80, 3, "uniform", 0.3)]
 
 
 @pytest.mark.gpu
@@ -122,7 +124,10 @@ def test_gpu_spmm_equals_model_bit_for_bit(model, dl, M, K, N, kind, density):
 @pytest.mark.gpu
 @pytest.mark.parametrize("M,K,D,kind,density", [(130, 257, 64, "skewed", 0.1), (256, 512, 128, "uniform", 0.05),
                                                 (50, 100, 48, "uniform", 0.2), (64, 64, 16, "uniform", 0.3),
-                                                (30, 64, 1024, "uniform", 0.3), (33, 77, 13, "uniform", 0.3)])
+                                                (30, 64, 1024, "uniform", 0.3), (33, 77, 13, "uniform", 0.3),
+                                                (40, 60, 49, "skewed", 0.3), (40, 60, 130, "uniform", 0.3),
+                                                (30, 60, 513, "uniform", 0.3), (20, 60, 1027, "uniform", 0.3),
+                                                (40, 60, 3, "uniform", 0.3), (40, 60, 7, "uniform", 0.3)])
 def test_gpu_sddmm_and_fused_equal_model_bit_for_bit(model, dl, M, K, D, kind, density):
     import torch
 
