@@ -135,6 +135,53 @@ __host__ __device__ __forceinline__ int split_per_wave(int T, int W)
     return per < 1 ? 1 : per;
 }
 
+// ---- flat schedule: every wave owns `chunk` consecutive nonzeros of the whole matrix ------------------------
+// Largest row r with row_offsets[r] <= pos, for 0 <= pos < row_offsets[M] (so the row is not empty and holds
+// nonzero `pos`). A 64-ary search by the whole wave: each round reads 64 evenly spaced offsets with one load and
+// narrows the interval to one of 65 parts; ceil(log64(M)) dependent loads. Everything is wave-uniform.
+__device__ __forceinline__ int find_row(const int* __restrict__ row_offsets, int M, int pos, int lane)
+{
+    int lo = 0, hi = M;  // row_offsets[lo] <= pos < row_offsets[hi]
+    while (hi - lo > 1) {
+        const long long span = hi - lo;
+        const int idx = lo + (int)((span * (lane + 1)) >> 6);  // non-decreasing in lane, lane 63 reads `hi`
+        const unsigned long long le = __ballot(row_offsets[idx] <= pos);  // a prefix of the lanes
+        const int n = __popcll(le);                                        // < 64 because row_offsets[hi] > pos
+        const int new_lo = lo + (int)((span * n) >> 6);        // n == 0: lo itself
+        const int new_hi = lo + (int)((span * (n + 1)) >> 6);  // first sample above pos
+        lo = __builtin_amdgcn_readfirstlane(new_lo);
+        hi = __builtin_amdgcn_readfirstlane(new_hi);
+    }
+    return lo;
+}
+
+// 64 consecutive row offsets in the lanes of one register (offsets past M repeat row_offsets[M]); entry j is read
+// with v_readlane. Rows rbase .. rbase+62 have both their ends inside the window.
+constexpr int kWinRows = 63;
+__device__ __forceinline__ int window_load(const int* __restrict__ row_offsets, int M, int rbase, int lane)
+{
+    return row_offsets[min(rbase + lane, M)];
+}
+__device__ __forceinline__ int window_get(int win, int j)
+{
+    return __builtin_amdgcn_readlane(win, __builtin_amdgcn_readfirstlane(j));
+}
+// First row after the one that ended at `pos` that holds nonzero `pos` (rows without nonzeros are skipped), for
+// pos < row_offsets[M]. Reloads the window (by search) when that row is not inside it.
+__device__ __forceinline__ int window_next_row(const int* __restrict__ row_offsets, int M, int pos, int lane, int& win,
+                                               int& rbase)
+{
+    const unsigned long long gt = __ballot(win > pos);  // a suffix of the lanes: entries are non-decreasing
+    if (gt != 0) {
+        const int t = __builtin_ctzll(gt);  // smallest entry above pos: the row ends there, so it is row t - 1
+        return rbase + t - 1;               // t >= 1: entry 0 is the start of a row at or before pos
+    }
+    const int r = find_row(row_offsets, M, pos, lane);
+    rbase = r;
+    win = window_load(row_offsets, M, rbase, lane);
+    return r;
+}
+
 // ---- dense-row accumulation (SpMM kernel and stage 2 of the fused kernel) -----------------------------
 // The wave holds `cnt` <= 64 nonzeros of one row segment, one per lane: column index `c` and value `av`
 // (lanes >= cnt hold c = 0, av = 0). Adds sum_j av_j * dense[c_j, colv[v] .. colv[v]+VEC) into acc[v].

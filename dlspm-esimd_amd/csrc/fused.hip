@@ -18,6 +18,42 @@
 
 namespace dlspm {
 
+// acc[v] = sum over the nonzeros [p, q) of one mask row (p < q, wave-uniform) of scale * <q_row, Kmat[column]> *
+// Vmat[column, colv[v] ..], summed over the wave's slots so that every lane ends with the total.
+template <int VEC, int G1, int DS, bool MASKED, int G, int V2>
+__device__ __forceinline__ void fused_segment(Vec<VEC>* acc, int p, int q, int D, float scale,
+                                              const int* __restrict__ col_indices, const float* __restrict__ q_row,
+                                              const float* __restrict__ Kmat, const float* __restrict__ Vmat,
+                                              const int* colv, int lane)
+{
+    using VecT = Vec<VEC>;
+    const int g1 = lane % G1;
+    VecT lq[DS > 0 ? DS : 1];
+    if constexpr (DS > 0) {
+#pragma unroll
+        for (int s = 0; s < DS; ++s) {
+            const int d = (s * G1 + g1) * VEC;
+            if constexpr (MASKED) lq[s] = d < D ? VecT::gload_clip(q_row, d, D) : VecT::zero();
+            else lq[s] = VecT::gload(q_row + d);
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < V2; ++v) acc[v] = VecT::zero();
+
+    int c_nxt = col_indices[min(p + lane, q - 1)];  // next pass's columns are requested one pass ahead
+    for (int base = p; base < q; base += kWave) {
+        const int c = base + lane < q ? c_nxt : 0;
+        c_nxt = col_indices[min(base + kWave + lane, q - 1)];
+        const int cnt = min(kWave, q - base);
+        // stage 1: lane l <- score of nonzero base + l (fp32, as between the reference's two loops)
+        float score = sddmm_chunk<VEC, G1, DS, MASKED>(D, lane, cnt, c, q_row, lq, Kmat);
+        score = base + lane < q ? score * scale : 0.f;
+        // stage 2: acc += score_j * V[col_j, :]
+        dense_rows_fma<VEC, G, V2>(acc, c, score, cnt, Vmat, D, colv, lane);
+    }
+    if constexpr (kWave / G > 1) slots_sum<VEC, G, V2>(acc, lane);
+}
+
 // MASKED = false: D == G1 * VEC * DS exactly, every stage-1 access of every lane falls inside the row.
 template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R>
 __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_tiles, float scale,
@@ -26,7 +62,6 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
                                                        const float* __restrict__ Q, const float* __restrict__ Kmat,
                                                        const float* __restrict__ Vmat, float* __restrict__ O)
 {
-    constexpr int S = kWave / G;
     constexpr int TW = G * VEC * V2;
     constexpr int NP = R == 1 ? 1 : 2;
     using VecT = Vec<VEC>;
@@ -36,7 +71,6 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int g1 = lane % G1;
     const int g = lane % G;
     const int slot = lane / G;
     const int rb = blockIdx.x / col_tiles;
@@ -73,31 +107,8 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
             const int p = __builtin_amdgcn_readfirstlane(pos);
             const float* q_row = Q + (size_t)(r0 + r) * D;
 
-            VecT lq[DS > 0 ? DS : 1];
-            if constexpr (DS > 0) {
-#pragma unroll
-                for (int s = 0; s < DS; ++s) {
-                    const int d = (s * G1 + g1) * VEC;
-                    if constexpr (MASKED) lq[s] = d < D ? VecT::gload_clip(q_row, d, D) : VecT::zero();
-                    else lq[s] = VecT::gload(q_row + d);
-                }
-            }
             VecT acc[V2];
-#pragma unroll
-            for (int v = 0; v < V2; ++v) acc[v] = VecT::zero();
-
-            int c_nxt = col_indices[min(p + lane, q - 1)];  // next pass's columns are requested one pass ahead
-            for (int base = p; base < q; base += kWave) {
-                const int c = base + lane < q ? c_nxt : 0;
-                c_nxt = col_indices[min(base + kWave + lane, q - 1)];
-                const int cnt = min(kWave, q - base);
-                // stage 1: lane l <- score of nonzero base + l (fp32, as between the reference's two loops)
-                float score = sddmm_chunk<VEC, G1, DS, MASKED>(D, lane, cnt, c, q_row, lq, Kmat);
-                score = base + lane < q ? score * scale : 0.f;
-                // stage 2: acc += score_j * V[col_j, :]
-                dense_rows_fma<VEC, G, V2>(acc, c, score, cnt, Vmat, D, colv, lane);
-            }
-            if constexpr (S > 1) slots_sum<VEC, G, V2>(acc, lane);
+            fused_segment<VEC, G1, DS, MASKED, G, V2>(acc, p, q, D, scale, col_indices, q_row, Kmat, Vmat, colv, lane);
 
             const bool whole_row = (p == rs) && (q == re);
             if (slot == 0) {
@@ -221,6 +232,110 @@ hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t str
         if (s.G1 == 8 && s.DS == 0 && s.G == 64 && s.V == 4) return launch_wr<4, 8, 0, 64, 4>(x, s.W, s.R, stream);
     } else if (s.G1 == 4 && s.DS == 1 && s.G == 8 && s.V == 1) {
         return launch_wr<1, 4, 1, 8, 1>(x, s.W, s.R, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+// ---- flat schedule (see spmm.hip): every wave owns `chunk` consecutive nonzeros of the mask ------------------------
+template <int VEC, int G1, int DS, bool MASKED, int G, int V2>
+__global__ __launch_bounds__(kFlatWaves * 64) void fused_flat_kernel(int M, int D, int nnz, int chunk, int col_tiles,
+                                                                      float scale, const int* __restrict__ row_offsets,
+                                                                      const int* __restrict__ col_indices,
+                                                                      const float* __restrict__ Q,
+                                                                      const float* __restrict__ Kmat,
+                                                                      const float* __restrict__ Vmat, float* __restrict__ O,
+                                                                      float* __restrict__ partial)
+{
+    constexpr int TW = G * VEC * V2;
+    using VecT = Vec<VEC>;
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = lane % G;
+    const int slot = lane / G;
+    const long long id = (long long)blockIdx.x * kFlatWaves + w;
+    const int unit = (int)(id / col_tiles);
+    const int ct = (int)(id - (long long)unit * col_tiles);
+    const long long a64 = (long long)unit * chunk;
+    if (a64 >= nnz) return;  // wave-uniform
+    const int a = (int)a64;
+    const int b = (int)min((long long)nnz, a64 + chunk);
+
+    int colv[V2];
+    bool act[V2];
+#pragma unroll
+    for (int v = 0; v < V2; ++v) {
+        const int col = ct * TW + (v * G + g) * VEC;
+        act[v] = col < D;
+        colv[v] = act[v] ? min(col, D - VEC) : 0;
+    }
+
+    int r = find_row(row_offsets, M, a, lane);
+    int rbase = r;
+    int win = window_load(row_offsets, M, rbase, lane);
+    int pos = a;
+    while (true) {
+        if (r - rbase >= kWinRows) {
+            rbase = r;
+            win = window_load(row_offsets, M, rbase, lane);
+        }
+        const int rs = window_get(win, r - rbase);
+        const int re = window_get(win, r - rbase + 1);
+        const int p = pos;
+        const int q = min(re, b);
+
+        VecT acc[V2];
+        fused_segment<VEC, G1, DS, MASKED, G, V2>(acc, p, q, D, scale, col_indices, Q + (size_t)r * D, Kmat, Vmat, colv,
+                                                  lane);
+        if (slot == 0) {
+            float* dst = (p == rs && q == re) ? O + (size_t)r * D : partial + ((size_t)unit * 2 + (p == a ? 0 : 1)) * D;
+#pragma unroll
+            for (int v = 0; v < V2; ++v)
+                if (act[v]) acc[v].gstore(dst + colv[v]);
+        }
+        pos = q;
+        if (pos >= b) break;
+        r = window_next_row(row_offsets, M, pos, lane, win, rbase);
+    }
+}
+
+template <int VEC, int G1, int DS, int G, int V2>
+static hipError_t launch_flat(const FusedArgs& x, const FlatPlan& plan, float* partial, hipStream_t stream)
+{
+    constexpr int TW = G * VEC * V2;
+    const int col_tiles = (x.D + TW - 1) / TW;
+    const long long waves = (long long)plan.units * col_tiles;
+    const long long blocks = (waves + kFlatWaves - 1) / kFlatWaves;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    bool exact = false;
+    if constexpr (DS > 0) exact = x.D == G1 * VEC * DS;
+    if constexpr (DS > 0) {
+        if (exact)
+            hipLaunchKernelGGL((fused_flat_kernel<VEC, G1, DS, false, G, V2>), dim3((unsigned)blocks), dim3(kFlatWaves * 64),
+                               0, stream, x.M, x.D, x.nnz, plan.chunk, col_tiles, x.scale, x.row_offsets, x.col_indices, x.Q,
+                               x.Kmat, x.V, x.O, partial);
+    }
+    if (!exact)
+        hipLaunchKernelGGL((fused_flat_kernel<VEC, G1, DS, true, G, V2>), dim3((unsigned)blocks), dim3(kFlatWaves * 64), 0,
+                           stream, x.M, x.D, x.nnz, plan.chunk, col_tiles, x.scale, x.row_offsets, x.col_indices, x.Q,
+                           x.Kmat, x.V, x.O, partial);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return row_fixup_launch(x.M, x.D, plan.chunk, x.row_offsets, partial, x.O, stream);
+}
+
+hipError_t fused_flat_launch(const FusedArgs& x, const FusedShape& s, const FlatPlan& plan, float* partial,
+                             hipStream_t stream)
+{
+    if (s.vec == 4) {
+        if (s.G1 == 4 && s.DS == 1 && s.G == 8 && s.V == 1) return launch_flat<4, 4, 1, 8, 1>(x, plan, partial, stream);
+        if (s.G1 == 8 && s.DS == 1 && s.G == 8 && s.V == 1) return launch_flat<4, 8, 1, 8, 1>(x, plan, partial, stream);
+        if (s.G1 == 8 && s.DS == 2 && s.G == 16 && s.V == 1) return launch_flat<4, 8, 2, 16, 1>(x, plan, partial, stream);
+        if (s.G1 == 8 && s.DS == 4 && s.G == 32 && s.V == 1) return launch_flat<4, 8, 4, 32, 1>(x, plan, partial, stream);
+        if (s.G1 == 8 && s.DS == 8 && s.G == 64 && s.V == 1) return launch_flat<4, 8, 8, 64, 1>(x, plan, partial, stream);
+        if (s.G1 == 8 && s.DS == 16 && s.G == 64 && s.V == 2) return launch_flat<4, 8, 16, 64, 2>(x, plan, partial, stream);
+        if (s.G1 == 8 && s.DS == 0 && s.G == 64 && s.V == 4) return launch_flat<4, 8, 0, 64, 4>(x, plan, partial, stream);
+    } else if (s.G1 == 4 && s.DS == 1 && s.G == 8 && s.V == 1) {
+        return launch_flat<1, 4, 1, 8, 1>(x, plan, partial, stream);
     }
     return hipErrorInvalidValue;
 }

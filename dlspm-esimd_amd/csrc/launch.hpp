@@ -42,14 +42,30 @@ struct FusedArgs {
     float* O;
 };
 
+// Flat schedule: `units` waves of `chunk` consecutive nonzeros each; `bytes` of device workspace for the partial
+// rows (units x 2 x width floats). chunk == 0: not used for this problem.
+constexpr int kFlatWaves = 4;  // waves per workgroup of the flat kernels (the waves are independent)
+struct FlatPlan {
+    int chunk;
+    int units;
+    size_t bytes;
+};
+FlatPlan flat_plan(int M, int nnz, int width, int G);
+hipError_t row_fixup_launch(int M, int N, int chunk, const int* row_offsets, const float* partial, float* out,
+                            hipStream_t stream);
+
 SpmmShape spmm_choose(int M, int N, int nnz, bool vec4);
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
+hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPlan& plan, float* partial,
+                            hipStream_t stream);
 
 SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4);
 hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t stream);
 
 FusedShape fused_choose(int M, int D, int nnz, bool vec4);
 hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream);
+hipError_t fused_flat_launch(const FusedArgs& x, const FusedShape& s, const FlatPlan& plan, float* partial,
+                             hipStream_t stream);
 
 // Picks (W, R), W <= max_w: waves per workgroup from the number of rows, rows per workgroup as large as keeps
 // `min_blocks` workgroups in the grid. `slots` = nonzeros of a row a wave works on at once (64 / G).

@@ -19,6 +19,33 @@
 
 namespace dlspm {
 
+// acc[v] = sum over the nonzeros [p, q) of one row (p < q, wave-uniform) of value * B[column, colv[v] ..], summed over
+// the wave's S = 64/G slots, so that every lane (slot 0 in particular) ends with the total.
+template <int VEC, int G, int V>
+__device__ __forceinline__ void spmm_segment(Vec<VEC>* acc, int p, int q, const int* __restrict__ col_indices,
+                                             const float* __restrict__ values, const float* __restrict__ B, int N,
+                                             const int* colv, int lane)
+{
+    using VecT = Vec<VEC>;
+#pragma unroll
+    for (int v = 0; v < V; ++v) acc[v] = VecT::zero();
+    // 64 (column, value) pairs per pass, one per lane; the next 64 are requested (index clamped, so the
+    // loads carry no condition) before the rows of B for the current ones, and arrive behind them
+    const int first = min(p + lane, q - 1);
+    int c_nxt = col_indices[first];
+    float a_nxt = values[first];
+    for (int base = p; base < q; base += kWave) {
+        const bool mine = base + lane < q;
+        const int c = mine ? c_nxt : 0;
+        const float av = mine ? a_nxt : 0.f;
+        const int ahead = min(base + kWave + lane, q - 1);
+        c_nxt = col_indices[ahead];
+        a_nxt = values[ahead];
+        dense_rows_fma<VEC, G, V>(acc, c, av, min(kWave, q - base), B, N, colv, lane);
+    }
+    if constexpr (kWave / G > 1) slots_sum<VEC, G, V>(acc, lane);
+}
+
 template <int VEC, int G, int V, int W, int R>
 __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tiles,
                                                       const int* __restrict__ row_offsets,
@@ -26,7 +53,6 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
                                                       const float* __restrict__ values,
                                                       const float* __restrict__ B, float* __restrict__ C)
 {
-    constexpr int S = kWave / G;     // rows of B in flight per load instruction
     constexpr int TW = G * VEC * V;  // columns of C covered by one wave
     using VecT = Vec<VEC>;
 
@@ -74,24 +100,7 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
             const int p = __builtin_amdgcn_readfirstlane(pos);
 
             VecT acc[V];
-#pragma unroll
-            for (int v = 0; v < V; ++v) acc[v] = VecT::zero();
-
-            // 64 (column, value) pairs per pass, one per lane; the next 64 are requested (index clamped, so the
-            // loads carry no condition) before the rows of B for the current ones, and arrive behind them
-            const int first = min(p + lane, q - 1);
-            int c_nxt = col_indices[first];
-            float a_nxt = values[first];
-            for (int base = p; base < q; base += kWave) {
-                const bool mine = base + lane < q;
-                const int c = mine ? c_nxt : 0;
-                const float av = mine ? a_nxt : 0.f;
-                const int ahead = min(base + kWave + lane, q - 1);
-                c_nxt = col_indices[ahead];
-                a_nxt = values[ahead];
-                dense_rows_fma<VEC, G, V>(acc, c, av, min(kWave, q - base), B, N, colv, lane);
-            }
-            if constexpr (S > 1) slots_sum<VEC, G, V>(acc, lane);
+            spmm_segment<VEC, G, V>(acc, p, q, col_indices, values, B, N, colv, lane);
 
             const bool whole_row = (p == rs) && (q == re);
             if (slot == 0) {
@@ -204,6 +213,104 @@ hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream
         if (s.G == 8 && s.V == 1) return launch_wr<4, 8, 1>(x, s.W, s.R, stream);
     } else {
         if (s.G == 8 && s.V == 1) return launch_wr<1, 8, 1>(x, s.W, s.R, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+// ---- flat schedule ----------------------------------------------------------------------------------
+// Every wave owns `chunk` consecutive nonzeros of the whole matrix (and one column tile), whatever rows they
+// belong to, so the time of a wave does not depend on how the nonzeros are spread over the rows: one row of a
+// million nonzeros is shared by thousands of waves. A wave finds its first row by search, walks the rows of its
+// range with a register window of row offsets, stores rows that lie wholly inside its range straight to C, and
+// leaves at most two partial rows (the one that began before its range, the one that continues after it) in
+// `partial[unit][0 or 1][N]`. row_fixup_kernel then adds the partial rows in unit order and writes rows without
+// nonzeros as zeros, so the result is deterministic. No LDS, no barrier, no atomics.
+template <int VEC, int G, int V>
+__global__ __launch_bounds__(kFlatWaves * 64) void spmm_flat_kernel(int M, int N, int nnz, int chunk, int col_tiles,
+                                                                     const int* __restrict__ row_offsets,
+                                                                     const int* __restrict__ col_indices,
+                                                                     const float* __restrict__ values,
+                                                                     const float* __restrict__ B, float* __restrict__ C,
+                                                                     float* __restrict__ partial)
+{
+    constexpr int TW = G * VEC * V;
+    using VecT = Vec<VEC>;
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = lane % G;
+    const int slot = lane / G;
+    const long long id = (long long)blockIdx.x * kFlatWaves + w;
+    const int unit = (int)(id / col_tiles);
+    const int ct = (int)(id - (long long)unit * col_tiles);
+    const long long a64 = (long long)unit * chunk;
+    if (a64 >= nnz) return;  // wave-uniform
+    const int a = (int)a64;
+    const int b = (int)min((long long)nnz, a64 + chunk);
+
+    int colv[V];
+    bool act[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        const int col = ct * TW + (v * G + g) * VEC;
+        act[v] = col < N;
+        colv[v] = act[v] ? min(col, N - VEC) : 0;
+    }
+
+    int r = find_row(row_offsets, M, a, lane);
+    int rbase = r;
+    int win = window_load(row_offsets, M, rbase, lane);
+    int pos = a;
+    while (true) {
+        if (r - rbase >= kWinRows) {
+            rbase = r;
+            win = window_load(row_offsets, M, rbase, lane);
+        }
+        const int rs = window_get(win, r - rbase);
+        const int re = window_get(win, r - rbase + 1);
+        const int p = pos;
+        const int q = min(re, b);
+
+        VecT acc[V];
+        spmm_segment<VEC, G, V>(acc, p, q, col_indices, values, B, N, colv, lane);
+
+        if (slot == 0) {
+            float* dst = (p == rs && q == re) ? C + (size_t)r * N : partial + ((size_t)unit * 2 + (p == a ? 0 : 1)) * N;
+#pragma unroll
+            for (int v = 0; v < V; ++v)
+                if (act[v]) acc[v].gstore(dst + colv[v]);
+        }
+        pos = q;
+        if (pos >= b) break;
+        r = window_next_row(row_offsets, M, pos, lane, win, rbase);
+    }
+}
+
+template <int VEC, int G, int V>
+static hipError_t launch_flat(const SpmmArgs& x, const FlatPlan& plan, float* partial, hipStream_t stream)
+{
+    constexpr int TW = G * VEC * V;
+    const int col_tiles = (x.N + TW - 1) / TW;
+    const long long waves = (long long)plan.units * col_tiles;
+    const long long blocks = (waves + kFlatWaves - 1) / kFlatWaves;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((spmm_flat_kernel<VEC, G, V>), dim3((unsigned)blocks), dim3(kFlatWaves * 64), 0, stream, x.M, x.N,
+                       x.nnz, plan.chunk, col_tiles, x.row_offsets, x.col_indices, x.values, x.B, x.C, partial);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return row_fixup_launch(x.M, x.N, plan.chunk, x.row_offsets, partial, x.C, stream);
+}
+
+hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPlan& plan, float* partial,
+                            hipStream_t stream)
+{
+    if (s.vec == 4) {
+        if (s.G == 64 && s.V == 1) return launch_flat<4, 64, 1>(x, plan, partial, stream);
+        if (s.G == 64 && s.V == 2) return launch_flat<4, 64, 2>(x, plan, partial, stream);
+        if (s.G == 32 && s.V == 1) return launch_flat<4, 32, 1>(x, plan, partial, stream);
+        if (s.G == 16 && s.V == 1) return launch_flat<4, 16, 1>(x, plan, partial, stream);
+        if (s.G == 8 && s.V == 1) return launch_flat<4, 8, 1>(x, plan, partial, stream);
+    } else if (s.G == 8 && s.V == 1) {
+        return launch_flat<1, 8, 1>(x, plan, partial, stream);
     }
     return hipErrorInvalidValue;
 }

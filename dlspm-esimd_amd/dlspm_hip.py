@@ -99,8 +99,9 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def spmm(row_offsets, col_indices, values, B, K=None, out=None):
-    """C = A_csr @ B on the current stream. row_offsets/col_indices int32, values/B float32, all on the GPU."""
+def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None):
+    """C = A_csr @ B on the current stream. row_offsets/col_indices int32, values/B float32, all on the GPU.
+    `workspace`: optional GPU tensor of at least workspace_bytes(OP_SPMM, ...) bytes."""
     import torch
 
     M = row_offsets.numel() - 1
@@ -109,9 +110,10 @@ def spmm(row_offsets, col_indices, values, B, K=None, out=None):
     K = Kd if K is None else K
     if out is None:
         out = torch.empty((M, N), dtype=torch.float32, device=B.device)
+    wp, wb = _workspace(workspace)
     st = lib().spmm_csr_f32(M, K, N, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
                             _ptr(col_indices, torch.int32, "col_indices"), _ptr(values, torch.float32, "values"),
-                            _ptr(B, torch.float32, "B"), _ptr(out, torch.float32, "C"), None, 0, _stream())
+                            _ptr(B, torch.float32, "B"), _ptr(out, torch.float32, "C"), wp, wb, _stream())
     if st != OK:
         raise DlspmError(st, "spmm_csr_f32")
     return out
@@ -134,8 +136,9 @@ def sddmm(row_offsets, col_indices, lhs, rhs, out=None):
     return out
 
 
-def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None):
-    """O = (S .* (Q Kmat^T) * scale) V on the current stream; the scores are never stored."""
+def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None, workspace=None):
+    """O = (S .* (Q Kmat^T) * scale) V on the current stream; the scores are never stored.
+    `workspace`: optional GPU tensor of at least workspace_bytes(OP_FUSED, ...) bytes."""
     import torch
 
     M = row_offsets.numel() - 1
@@ -146,19 +149,36 @@ def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None):
     st = lib().fused_sddmm_spmm_f32(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
                                     _ptr(col_indices, torch.int32, "col_indices"), _ptr(Q, torch.float32, "Q"),
                                     _ptr(Kmat, torch.float32, "Kmat"), _ptr(V, torch.float32, "V"),
-                                    ctypes.c_float(scale), _ptr(out, torch.float32, "O"), None, 0, _stream())
+                                    ctypes.c_float(scale), _ptr(out, torch.float32, "O"), *_workspace(workspace),
+                                    _stream())
     if st != OK:
         raise DlspmError(st, "fused_sddmm_spmm_f32")
     return out
 
 
 def describe_launch(op: int, M: int, K: int, N: int, nnz: int) -> dict:
-    """Launch shape the library uses for these sizes: {'vec','G','V','G1','DS','W','R','col_tiles'} (host only)."""
-    out = (ctypes.c_int * 8)()
+    """Launch shape the library uses for these sizes: {'vec','G','V','G1','DS','W','R','col_tiles','flat_chunk',
+    'flat_units'} (host only)."""
+    out = (ctypes.c_int * 10)()
     st = lib().dlspm_describe_launch(op, M, K, N, nnz, out)
     if st != OK:
         raise DlspmError(st, "dlspm_describe_launch")
-    return dict(zip(("vec", "G", "V", "G1", "DS", "W", "R", "col_tiles"), (int(x) for x in out)))
+    return dict(zip(("vec", "G", "V", "G1", "DS", "W", "R", "col_tiles", "flat_chunk", "flat_units"),
+                    (int(x) for x in out)))
+
+
+def workspace_bytes(op: int, M: int, K: int, N: int, nnz: int) -> int:
+    """Bytes of device workspace the op can use for these sizes (0 = none)."""
+    return int(lib().dlspm_workspace_bytes(op, M, K, N, nnz))
+
+
+def _workspace(ws):
+    """(pointer, bytes) of an optional workspace tensor (any dtype, contiguous, on the GPU)."""
+    if ws is None:
+        return None, 0
+    if not ws.is_cuda or not ws.is_contiguous():
+        raise ValueError("workspace must be a contiguous GPU tensor")
+    return ctypes.c_void_p(ws.data_ptr()), ws.numel() * ws.element_size()
 
 
 def csr_check(M, K, row_offsets, col_indices) -> int:

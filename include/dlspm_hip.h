@@ -112,10 +112,11 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
  * Launch shape the library would use for these sizes, for tuning reports and for host-side models of the
  * schedule (the reference's SpmmEsimdCPU / FusedEsimdCPU, SPMM/spmm-esimd-v1.cpp:83-169 and
  * FUSED/fused.cpp:93-216, play that role for its kernels). Host-only, never touches the device.
- * shape[8] receives: [0] floats per lane per access (4 or 1), [1] G lanes per dense row (SpMM, fused stage 2; 0 for
+ * shape[10] receives: [0] floats per lane per access (4 or 1), [1] G lanes per dense row (SpMM, fused stage 2; 0 for
  * SDDMM), [2] accesses per lane per dense row, [3] G1 lanes per dot product (SDDMM, fused stage 1; 0 for SpMM),
  * [4] accesses per lane per dot product (0 = run-time loop), [5] waves per workgroup, [6] rows per workgroup,
- * [7] column tiles. Returns DLSPM_OK or DLSPM_E_INVALID_ARG.
+ * [7] column tiles, [8] nonzeros per wave of the flat schedule that a call WITH workspace would use (0 = such a call
+ * uses the workgroup-per-row-block schedule too), [9] number of such waves. Returns DLSPM_OK or DLSPM_E_INVALID_ARG.
  */
 int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape);
 

@@ -129,6 +129,122 @@ float model_dot(const float* l, const float* r, int D, int vec, int G1, int DS)
     return lane[0];
 }
 
+
+// ---- flat schedule (spmm_flat_kernel / fused_flat_kernel + row_fixup_kernel) ------------------------------------
+// The row search and the 64-entry offset window are modelled lane by lane, with every index checked, so that an
+// indexing mistake in them shows on the CPU: any out-of-range access makes the model return 2.
+struct Checked {
+    const int* ro;
+    int M;
+    bool bad = false;
+    int at(long long i)
+    {
+        if (i < 0 || i > M) { bad = true; return 0; }
+        return ro[i];
+    }
+};
+
+int model_find_row(Checked& c, int pos)
+{
+    int lo = 0, hi = c.M;
+    while (hi - lo > 1) {
+        const long long span = hi - lo;
+        int n = 0;
+        bool prefix = true;
+        for (int lane = 0; lane < 64; ++lane) {
+            const int idx = lo + (int)((span * (lane + 1)) >> 6);
+            const bool le = c.at(idx) <= pos;
+            if (le && !prefix) c.bad = true;  // the kernel counts on a prefix of lanes
+            if (le) ++n; else prefix = false;
+        }
+        if (n >= 64) { c.bad = true; return lo; }
+        const int new_lo = lo + (int)((span * n) >> 6);
+        const int new_hi = lo + (int)((span * (n + 1)) >> 6);
+        if (new_hi - new_lo >= hi - lo) { c.bad = true; return lo; }  // no progress
+        lo = new_lo;
+        hi = new_hi;
+    }
+    return lo;
+}
+
+void model_window_load(Checked& c, int rbase, int* win)
+{
+    for (int lane = 0; lane < 64; ++lane) win[lane] = c.at(std::min(rbase + lane, c.M));
+}
+
+int model_rows_flat(int M, int N, int nnz, const int* ro, const int* ci, const float* va, const float* B, int G, int chunk,
+                    float* C, int* writes)
+{
+    const int S = 64 / G;
+    const int units = (int)(((long long)nnz + chunk - 1) / chunk);
+    std::vector<float> part((size_t)units * 2 * N, NAN), acc((size_t)S * N), sl(S);
+    Checked c{ro, M};
+    for (int unit = 0; unit < units; ++unit) {
+        const int a = unit * chunk, b = std::min(nnz, a + chunk);
+        int r = model_find_row(c, a);
+        int rbase = r, win[64];
+        model_window_load(c, rbase, win);
+        int pos = a;
+        while (true) {
+            if (r - rbase >= 63) { rbase = r; model_window_load(c, rbase, win); }
+            if (r - rbase < 0 || r - rbase + 1 > 63) return 2;
+            const int rs = win[r - rbase], re = win[r - rbase + 1];
+            if (r < 0 || r >= M || rs != ro[r] || re != ro[r + 1] || !(rs <= pos && pos < re)) return 2;
+            const int p = pos, q = std::min(re, b);
+            std::fill(acc.begin(), acc.end(), 0.0f);
+            for (int idx = p; idx < q; ++idx) {
+                const float* brow = B + (size_t)ci[idx] * N;
+                float* as = acc.data() + (size_t)((idx - p) % S) * N;
+                for (int j = 0; j < N; ++j) as[j] = std::fmaf(va[idx], brow[j], as[j]);
+            }
+            const bool whole = p == rs && q == re;
+            for (int j = 0; j < N; ++j) {
+                for (int s = 0; s < S; ++s) sl[s] = acc[(size_t)s * N + j];
+                const float tot = slots_tree(sl.data(), S);
+                if (whole) { C[(size_t)r * N + j] = tot; writes[(size_t)r * N + j]++; }
+                else part[((size_t)unit * 2 + (p == a ? 0 : 1)) * N + j] = tot;
+            }
+            pos = q;
+            if (pos >= b) break;
+            int t = -1;
+            for (int lane = 0; lane < 64; ++lane)
+                if (win[lane] > pos) { t = lane; break; }
+            if (t >= 0) {
+                if (t < 1) return 2;
+                r = rbase + t - 1;
+            } else {
+                r = model_find_row(c, pos);
+                rbase = r;
+                model_window_load(c, rbase, win);
+            }
+        }
+    }
+    if (c.bad) return 2;
+    for (int r = 0; r < M; ++r) {
+        const int rs = ro[r], re = ro[r + 1];
+        float* crow = C + (size_t)r * N;
+        int* wrow = writes + (size_t)r * N;
+        if (rs == re) {
+            for (int j = 0; j < N; ++j) { crow[j] = 0.0f; wrow[j]++; }
+            continue;
+        }
+        const int ul = rs / chunk, uh = (re - 1) / chunk;
+        if (ul == uh) continue;
+        for (int j = 0; j < N; ++j) {
+            float sum = 0.0f;
+            for (int u = ul; u <= uh; ++u) {
+                const int k = (u == ul && (long long)u * chunk != rs) ? 1 : 0;
+                const float pv = part[((size_t)u * 2 + k) * N + j];
+                if (std::isnan(pv) && !std::isnan(B[0])) return 1;
+                sum = sum + pv;
+            }
+            crow[j] = sum;
+            wrow[j]++;
+        }
+    }
+    return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -140,6 +256,18 @@ int model_spmm(int M, int N, const int* ro, const int* ci, const float* va, cons
     std::memset(writes, 0, (size_t)M * N * sizeof(int));
     return model_rows(M, N, ro, ci, va, B, G, W, R, C, writes);
 }
+
+// flat schedule: 0 ok, 1 a partial row consumed that no wave produced, 2 an index out of range in the row search or
+// the offset window
+int model_spmm_flat(int M, int N, const int* ro, const int* ci, const float* va, const float* B, int G, int chunk,
+                    float* C, int* writes)
+{
+    std::memset(writes, 0, (size_t)M * N * sizeof(int));
+    return model_rows_flat(M, N, ro[M], ro, ci, va, B, G, chunk, C, writes);
+}
+
+int model_fused_flat(int M, int D, const int* ro, const int* ci, const float* Q, const float* Km, const float* V,
+                     float scale, int vec, int G1, int DS, int G, int chunk, float* scores, float* O, int* writes);
 
 void model_sddmm(int M, int D, const int* ro, const int* ci, const float* lhs, const float* rhs, int vec, int G1, int DS,
                  float* out)
@@ -157,6 +285,16 @@ int model_fused(int M, int D, const int* ro, const int* ci, const float* Q, cons
     for (int j = 0; j < nnz; ++j) scores[j] = scores[j] * scale;
     std::memset(writes, 0, (size_t)M * D * sizeof(int));
     return model_rows(M, D, ro, ci, scores, V, G, W, R, O, writes);
+}
+
+int model_fused_flat(int M, int D, const int* ro, const int* ci, const float* Q, const float* Km, const float* V,
+                     float scale, int vec, int G1, int DS, int G, int chunk, float* scores, float* O, int* writes)
+{
+    model_sddmm(M, D, ro, ci, Q, Km, vec, G1, DS, scores);
+    const int nnz = ro[M];
+    for (int j = 0; j < nnz; ++j) scores[j] = scores[j] * scale;
+    std::memset(writes, 0, (size_t)M * D * sizeof(int));
+    return model_rows_flat(M, D, nnz, ro, ci, scores, V, G, chunk, O, writes);
 }
 
 }  // extern "C"

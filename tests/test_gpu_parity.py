@@ -309,6 +309,42 @@ def test_large_shape_against_oracle(torch_cuda, dl, oracle):
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
+@pytest.mark.parametrize("sigma", [0.0, 1.5])
+def test_flat_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
+    """A matrix large enough (3.4 M nonzeros, 410 per row on average, N = 128) that a call WITH workspace takes the flat
+    schedule by the library's own rule: uniform rows and heavily skewed rows (lognormal, sigma 1.5: rows from 0 to 4096
+    nonzeros), SpMM and the fused op against the multi-threaded oracle; the same call without workspace must agree."""
+    torch = torch_cuda
+    M, K, N = 8192, 4096, 128
+    if sigma == 0.0:
+        ro, ci = dl.make_pattern(dl.PATTERN_UNIFORM_ROWS, 61, M, K, 0.1)
+    else:
+        ro, ci = dl.make_pattern(dl.PATTERN_LOGNORMAL_ROWS, 62, M, K, 0.1 * K, sigma)
+    nnz = ci.size
+    va = dl.fill("uniform", 63, (nnz,), -1.0, 1.0)
+    B = dl.fill("uniform", 64, (K, N), -1.0, 1.0)
+    Q = dl.fill("normal", 65, (M, N), 0.0, 1.0)
+    sh = dl.describe_launch(dl.OP_SPMM, M, K, N, nnz)
+    need = dl.workspace_bytes(dl.OP_SPMM, M, K, N, nnz)
+    assert sh["flat_chunk"] > 0 and need == sh["flat_units"] * 2 * N * 4
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    ro_d, ci_d, va_d, B_d, Q_d = (dev(torch, x) for x in (ro, ci, va, B, Q))
+    got = dl.spmm(ro_d, ci_d, va_d, B_d, K=K, workspace=ws)
+    ref = oracle.spmm(ro, ci, va, B, omp=True)
+    assert oracle.rel_frobenius(got.cpu().numpy(), ref) <= TOL
+    assert oracle.rel_frobenius(dl.spmm(ro_d, ci_d, va_d, B_d, K=K).cpu().numpy(), ref) <= TOL
+    assert (got.cpu().numpy()[np.diff(ro) == 0] == 0).all()
+
+    needf = dl.workspace_bytes(dl.OP_FUSED, M, K, N, nnz)
+    assert needf > 0
+    wsf = torch.empty(needf, dtype=torch.uint8, device="cuda")
+    gotO = dl.fused(ro_d, ci_d, Q_d, B_d, B_d, 0.01, workspace=wsf)
+    refO = oracle.fused(ro, ci, Q, B, B, 0.01, omp=True)
+    assert oracle.rel_frobenius(gotO.cpu().numpy(), refO) <= TOL
+    assert oracle.rel_frobenius(dl.fused(ro_d, ci_d, Q_d, B_d, B_d, 0.01).cpu().numpy(), refO) <= TOL
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
 def test_exact_integer_properties_at_large_size(torch_cuda, dl):
     """Size-independent, bit-exact checks on 65536 skewed rows (several million nonzeros), no oracle needed: with small-integer
     operands every fp32 product and sum is exact whatever the summation order, so

@@ -33,6 +33,10 @@ def model():
     L.model_sddmm.restype = None
     L.model_fused.argtypes = [ci, ci, _i, _i, _f, _f, _f, ctypes.c_float, ci, ci, ci, ci, ci, ci, _f, _f, _i]
     L.model_fused.restype = ci
+    L.model_spmm_flat.argtypes = [ci, ci, _i, _i, _f, _f, ci, ci, _f, _i]
+    L.model_spmm_flat.restype = ci
+    L.model_fused_flat.argtypes = [ci, ci, _i, _i, _f, _f, _f, ctypes.c_float, ci, ci, ci, ci, ci, _f, _f, _i]
+    L.model_fused_flat.restype = ci
     return L
 
 
@@ -90,6 +94,57 @@ def test_model_sddmm_and_fused_match_the_oracle(model, oracle):
         rc = model.model_fused(M, D, pi(ro), pi(ci), pf(Q), pf(Km), pf(V), 0.125, vec, G1, DS, 16, 4, 4, pf(scores), pf(O), pi(writes))
         assert rc == 0 and (writes == 1).all()
         assert oracle.rel_frobenius(O, oracle.fused(ro, ci, Q, Km, V, 0.125)) < 1e-6
+
+
+def run_spmm_flat(L, ro, ci, va, B, G, chunk):
+    M, N = ro.size - 1, B.shape[1]
+    C = np.full((M, N), np.nan, dtype=np.float32)
+    writes = np.zeros((M, N), dtype=np.int32)
+    rc = L.model_spmm_flat(M, N, pi(ro), pi(ci), pf(va), pf(B), G, chunk, pf(C), pi(writes))
+    return rc, C, writes
+
+
+def long_and_empty_rows(rng, M, K, n_long, long_len, short_avg):
+    """A few very long rows, runs of hundreds of empty rows, short rows in between."""
+    lens = rng.poisson(short_avg, M)
+    lens[rng.random(M) < 0.5] = 0
+    start = M // 3
+    lens[start:start + min(400, M // 2)] = 0  # a run of empty rows longer than the 64-entry offset window
+    for i in rng.choice(M, n_long, replace=False):
+        lens[i] = long_len
+    lens = np.minimum(lens, K)
+    ro = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ci = np.concatenate([np.sort(rng.choice(K, n, replace=False)) for n in lens] + [np.zeros(0, np.int64)]).astype(np.int32)
+    return ro, ci
+
+
+@pytest.mark.parametrize("case", ["uniform", "skewed", "empty_rows", "full", "long_and_empty", "one_row", "many_rows"])
+def test_flat_schedule_writes_each_output_once_and_matches_the_oracle(model, oracle, case):
+    """The flat schedule's row search, offset window and partial-row bookkeeping, index-checked on the CPU, for chunk
+    sizes below, at and above the row lengths."""
+    rng = np.random.default_rng(13)
+    N = 8
+    if case == "long_and_empty":
+        M, K = 1500, 700
+        ro, ci = long_and_empty_rows(rng, M, K, 3, 650, 3)
+    elif case == "one_row":
+        M, K = 1, 900
+        ro, ci = random_csr(rng, M, K, "full", 1.0)
+    elif case == "many_rows":
+        M, K = 9000, 40  # more rows than two rounds of the 64-ary search cover
+        ro, ci = random_csr(rng, M, K, "empty_rows", 0.05)
+    else:
+        M, K = 150, 300
+        ro, ci = random_csr(rng, M, K, case, 0.2 if case != "full" else 1.0)
+    va = rng.normal(0, 1, ci.size).astype(np.float32)
+    B = rng.normal(0, 1, (K, N)).astype(np.float32)
+    ref = oracle.spmm(ro, ci, va, B)
+    for chunk in (64, 128, 192, 512, 4096):
+        for G in (64, 8):
+            rc, C, writes = run_spmm_flat(model, ro, ci, va, B, G, chunk)
+            assert rc == 0, f"chunk {chunk} G {G}: model returned {rc}"
+            assert (writes == 1).all(), f"chunk {chunk} G {G}: an element was written {writes.min()}..{writes.max()} times"
+            assert oracle.rel_frobenius(C, ref) < 1e-6
 
 
 # ---- GPU: bit-for-bit ---------------------------------------------------------------------------------------------------
@@ -182,3 +237,80 @@ def test_gpu_benchmark_configs_equal_model_bit_for_bit(model, dl, cfg):
         got = dl.fused(ro_d, ci_d, dev(torch, c["d0"]), dev(torch, c["d1"]), dev(torch, c["d2"]), c["scale"]).cpu().numpy()
         assert rc == 0 and (writes == 1).all()
         assert np.array_equal(got.view(np.uint32), O.view(np.uint32))
+
+
+FLAT_GPU = [("uniform", 300, 200, 256, 0, 128), ("skewed", 257, 129, 64, 0, 64), ("long_and_empty", 1500, 700, 128, 3, 256),
+            ("long_and_empty", 1500, 700, 49, 3, 512), ("long_and_empty", 5000, 600, 32, 5, 64), ("uniform", 200, 512, 392, 0, 192),
+            ("full", 16, 700, 1030, 0, 320), ("empty_rows", 2000, 300, 5, 0, 64), ("skewed", 300, 80, 1, 0, 128)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,M,K,N,n_long,chunk", FLAT_GPU)
+def test_gpu_flat_spmm_equals_model_bit_for_bit(model, dl, monkeypatch, kind, M, K, N, n_long, chunk):
+    """The flat schedule (every wave owns `chunk` consecutive nonzeros; partial rows in the workspace, added by a second
+    kernel), forced on small matrices and with small chunks so that rows are shared by many waves."""
+    import torch
+
+    rng = np.random.default_rng(41 + M + N)
+    if kind == "long_and_empty":
+        ro, ci = long_and_empty_rows(rng, M, K, n_long, K - 50, 3)
+    else:
+        ro, ci = random_csr(rng, M, K, kind, 1.0 if kind == "full" else 0.2)
+    va = rng.normal(0, 1, ci.size).astype(np.float32)
+    B = rng.normal(0, 1, (K, N)).astype(np.float32)
+    monkeypatch.setenv("DLSPM_FLAT", "1")
+    monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
+    sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size)
+    assert sh["flat_chunk"] == chunk and sh["flat_units"] == -(-ci.size // chunk)
+    need = dl.workspace_bytes(dl.OP_SPMM, M, K, N, ci.size)
+    assert need == sh["flat_units"] * 2 * N * 4
+    rc, C, writes = run_spmm_flat(model, ro, ci, va, B, sh["G"], chunk)
+    assert rc == 0 and (writes == 1).all()
+    ws = torch.full((need // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    out = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    args = (dev(torch, ro), dev(torch, ci), dev(torch, va), dev(torch, B))
+    dl.spmm(*args, K=K, out=out, workspace=ws)
+    got = out.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), C.view(np.uint32)), \
+        f"shape {sh}: {np.count_nonzero(got.view(np.uint32) != C.view(np.uint32))} of {got.size} elements differ in their bits"
+    # a workspace that is too small is refused, none at all selects the workgroup-per-row-block schedule
+    with pytest.raises(dl.DlspmError) as e:
+        dl.spmm(*args, K=K, out=out, workspace=ws[: need // 4 - 1])
+    assert e.value.status == dl.E_WORKSPACE
+    out2 = dl.spmm(*args, K=K).cpu().numpy()
+    assert np.linalg.norm(out2 - C) <= 1e-5 * np.linalg.norm(C)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,M,K,D,n_long,chunk", [("uniform", 300, 200, 64, 0, 128), ("long_and_empty", 1500, 700, 128, 3, 256),
+                                                      ("skewed", 130, 257, 49, 0, 64), ("long_and_empty", 900, 600, 256, 2, 192),
+                                                      ("uniform", 40, 300, 1027, 0, 320), ("empty_rows", 500, 100, 3, 0, 64)])
+def test_gpu_flat_fused_equals_model_bit_for_bit(model, dl, monkeypatch, kind, M, K, D, n_long, chunk):
+    import torch
+
+    rng = np.random.default_rng(51 + M + D)
+    if kind == "long_and_empty":
+        ro, ci = long_and_empty_rows(rng, M, K, n_long, K - 50, 3)
+    else:
+        ro, ci = random_csr(rng, M, K, kind, 0.2)
+    Q = rng.normal(0, 1, (M, D)).astype(np.float32)
+    Km = rng.normal(0, 1, (K, D)).astype(np.float32)
+    V = rng.normal(0, 1, (K, D)).astype(np.float32)
+    monkeypatch.setenv("DLSPM_FLAT", "1")
+    monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
+    fs = dl.describe_launch(dl.OP_FUSED, M, K, D, ci.size)
+    assert fs["flat_chunk"] == chunk
+    need = dl.workspace_bytes(dl.OP_FUSED, M, K, D, ci.size)
+    assert need == fs["flat_units"] * 2 * D * 4
+    scores = np.empty(ci.size, dtype=np.float32)
+    O = np.full((M, D), np.nan, dtype=np.float32)
+    writes = np.zeros((M, D), dtype=np.int32)
+    rc = model.model_fused_flat(M, D, pi(ro), pi(ci), pf(Q), pf(Km), pf(V), 0.125, fs["vec"], fs["G1"], fs["DS"], fs["G"],
+                                chunk, pf(scores), pf(O), pi(writes))
+    assert rc == 0 and (writes == 1).all()
+    ws = torch.full((need // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    out = torch.full((M, D), float("nan"), dtype=torch.float32, device="cuda")
+    dl.fused(dev(torch, ro), dev(torch, ci), dev(torch, Q), dev(torch, Km), dev(torch, V), 0.125, out=out, workspace=ws)
+    got = out.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), O.view(np.uint32)), \
+        f"shape {fs}: {np.count_nonzero(got.view(np.uint32) != O.view(np.uint32))} of {got.size} elements differ in their bits"
