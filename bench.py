@@ -48,17 +48,20 @@ def make_step(dl, torch, c):
     """Uploads configuration c and returns (step_fn, output tensor)."""
     d = lambda a: torch.from_numpy(a).cuda()
     ro, ci = d(c["row_offsets"]), d(c["col_indices"])
+    # the caller owns the workspace; the library asks for none at the sizes of the five configurations
+    need = dl.workspace_bytes(c["op"], c["M"], c["K"], c["N"], c["nnz"])
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda") if need else None
     if c["op"] == dl.OP_SPMM:
         va, B = d(c["values"]), d(c["d0"])
         out = torch.empty((c["M"], c["N"]), dtype=torch.float32, device="cuda")
-        return (lambda: dl.spmm(ro, ci, va, B, K=c["K"], out=out)), out
+        return (lambda: dl.spmm(ro, ci, va, B, K=c["K"], out=out, workspace=ws)), out
     if c["op"] == dl.OP_SDDMM:
         lhs, rhs = d(c["d0"]), d(c["d1"])
         out = torch.empty((c["nnz"],), dtype=torch.float32, device="cuda")
         return (lambda: dl.sddmm(ro, ci, lhs, rhs, out=out)), out
     Q, Km, V = d(c["d0"]), d(c["d1"]), d(c["d2"])
     out = torch.empty((c["M"], c["N"]), dtype=torch.float32, device="cuda")
-    return (lambda: dl.fused(ro, ci, Q, Km, V, c["scale"], out=out)), out
+    return (lambda: dl.fused(ro, ci, Q, Km, V, c["scale"], out=out, workspace=ws)), out
 
 
 def time_steps(torch, step, steps, warmup, use_graph):

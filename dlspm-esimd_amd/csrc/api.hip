@@ -293,7 +293,7 @@ const char* dlspm_status_string(int status)
     switch (status) {
         case DLSPM_OK: return "ok";
         case DLSPM_E_INVALID_ARG: return "invalid argument (negative size, NULL operand, or nnz larger than M*K)";
-        case DLSPM_E_WORKSPACE: return "workspace too small or misaligned";
+        case DLSPM_E_WORKSPACE: return "workspace smaller than dlspm_workspace_bytes()";
         case DLSPM_E_LAUNCH: return "HIP runtime error at launch (see dlspm_last_hip_error)";
         case DLSPM_E_INVALID_CSR: return "malformed CSR structure";
         case DLSPM_E_NO_DEVICE: return "no gfx950 device is current";

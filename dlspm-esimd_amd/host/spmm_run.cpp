@@ -40,8 +40,12 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     if (dlspm_csr_check(M, K, nnz, ro_d.p, ci_d.p, nullptr) != DLSPM_OK) throw std::invalid_argument("malformed CSR structure");
     DLSPM_HIP_CHECK(hipMemset(C_d.p, 0xFF, (size_t)M * N * sizeof(float)));  // NaN pattern: every element must be written
 
+    // the caller owns the workspace, as it owns every other buffer: 0 bytes for small problems
+    const size_t ws_bytes = dlspm_workspace_bytes(DLSPM_OP_SPMM, M, K, N, nnz);
+    DevBuf<char> ws(ws_bytes);
+    if (ws_bytes) std::printf("workspace: %zu bytes (flat schedule)\n", ws_bytes);
     const Timing t = time_launches(opt, [&]() {
-        return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, nullptr, 0, nullptr);
+        return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, ws_bytes ? ws.p : nullptr, ws_bytes, nullptr);
     });
     hipLaunchKernelGGL(check_spmm_kernel, dim3(blocks_for((long long)M * N)), dim3(256), 0, nullptr, M, N, ro_d.p, ci_d.p,
                        va_d.p, B_d.p, Cref_d.p);

@@ -24,8 +24,16 @@
  *     SDDMM/sddmm-esimd-fromfile_v4.hpp:161,175);
  *   - errors are returned as a negative status, nothing is thrown across the ABI (the reference
  *     throws std::invalid_argument / std::logic_error on the host before launching).
- * Calls on different streams may run concurrently from different host threads; the library keeps
- * no mutable global state.
+ *   - `workspace` is optional device memory owned by the caller. NULL (or 0 bytes) is always valid and
+ *     selects the schedule that needs none. A caller that passes at least dlspm_workspace_bytes()
+ *     bytes lets SpMM and the fused op use the flat schedule where the library's size rule selects it
+ *     (large matrices with long rows: every wave then owns a fixed run of nonzeros, however they are
+ *     spread over the rows, and a second kernel adds the partial rows kept in the workspace, in a
+ *     fixed order). A non-NULL workspace smaller than that is refused with DLSPM_E_WORKSPACE. The
+ *     contents need no initialisation and mean nothing afterwards; two calls that share a workspace
+ *     must not overlap in time.
+ * Calls on different streams may run concurrently from different host threads (each with its own
+ * workspace); the library keeps no mutable global state.
  */
 #ifndef DLSPM_HIP_H
 #define DLSPM_HIP_H
@@ -39,7 +47,7 @@ extern "C" {
 /* status codes */
 #define DLSPM_OK              0
 #define DLSPM_E_INVALID_ARG  (-1) /* negative size, NULL pointer for a non-empty operand, nnz/M/K inconsistent */
-#define DLSPM_E_WORKSPACE    (-2) /* workspace smaller than dlspm_workspace_bytes() or misaligned          */
+#define DLSPM_E_WORKSPACE    (-2) /* a workspace was passed, but smaller than dlspm_workspace_bytes()        */
 #define DLSPM_E_LAUNCH       (-3) /* the HIP runtime refused the launch (see dlspm_last_hip_error)         */
 #define DLSPM_E_INVALID_CSR  (-4) /* dlspm_csr_check found a malformed CSR structure                        */
 #define DLSPM_E_NO_DEVICE    (-5) /* no gfx950 device is current                                            */
@@ -92,9 +100,10 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz,
                          void* workspace, size_t workspace_bytes, void* stream);
 
 /*
- * Bytes of device workspace the op wants for these sizes (0 = none; `workspace` may then be NULL).
- * Takes the place of the host-side launch sizing the reference does before each launch
- * (SPMM/spmm-esimd-fromfile2.cpp:188-192, SDDMM/sddmm-esimd-fromfile_v4.cpp:146-160).
+ * Bytes of device workspace the op can use for these sizes (0 = none, as for every SDDMM and for small
+ * or short-row problems; `workspace` may always be NULL). Host-only. Takes the place of the host-side
+ * launch sizing the reference does before each launch (SPMM/spmm-esimd-fromfile2.cpp:188-192,
+ * SDDMM/sddmm-esimd-fromfile_v4.cpp:146-160).
  */
 size_t dlspm_workspace_bytes(int op, int M, int K, int N_or_D, int nnz);
 
