@@ -185,7 +185,11 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
     const bool vec4 = D >= 4;  // dwordx4 accesses need only dword alignment
     const SddmmShape shape = sddmm_choose(M, D, nnz, vec4);
     const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values};
-    const hipError_t e = sddmm_launch(args, shape, static_cast<hipStream_t>(stream));
+    // the flat schedule needs no workspace here (nothing to combine), so the size rule alone decides; it has no
+    // width condition for SDDMM (measured for D = 32 ... 256: equal on uniform rows, 15-33 % faster on skewed ones)
+    const FlatPlan plan = flat_plan(M, nnz, D, kWave);
+    const hipError_t e = plan.chunk > 0 ? sddmm_flat_launch(args, shape, plan.chunk, static_cast<hipStream_t>(stream))
+                                        : sddmm_launch(args, shape, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }
 
@@ -275,6 +279,8 @@ int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape)
     } else if (op == DLSPM_OP_SDDMM) {
         const SddmmShape s = sddmm_choose(M, n, nnz, vec4);
         shape[0] = s.vec; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R; shape[7] = 1;
+        const FlatPlan fp = flat_plan(M, nnz, n, kWave);
+        shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_FUSED) {
         const FusedShape s = fused_choose(M, n, nnz, vec4);
         const int tw = s.G * s.vec * s.V;

@@ -61,6 +61,7 @@ hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPla
 
 SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4);
 hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t stream);
+hipError_t sddmm_flat_launch(const SddmmArgs& x, const SddmmShape& s, int chunk, hipStream_t stream);
 
 FusedShape fused_choose(int M, int D, int nnz, bool vec4);
 hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream);

@@ -18,6 +18,35 @@
 
 namespace dlspm {
 
+// out[j] = <lhs_row, rhs[col_indices[j]]> for the nonzeros j in [p, q) of one row (p < q, wave-uniform).
+template <int VEC, int G1, int DS, bool MASKED>
+__device__ __forceinline__ void sddmm_segment(int p, int q, int D, const int* __restrict__ col_indices,
+                                              const float* __restrict__ lhs_row, const float* __restrict__ rhs,
+                                              float* __restrict__ out, int lane)
+{
+    using VecT = Vec<VEC>;
+    const int g = lane % G1;
+    VecT lq[DS > 0 ? DS : 1];
+    if constexpr (DS > 0) {
+#pragma unroll
+        for (int s = 0; s < DS; ++s) {
+            const int d = (s * G1 + g) * VEC;
+            if constexpr (MASKED) lq[s] = d < D ? VecT::gload_clip(lhs_row, d, D) : VecT::zero();
+            else lq[s] = VecT::gload(lhs_row + d);
+        }
+    }
+    // 64 column indices per pass, one per lane; the next 64 are requested (index clamped, no condition) before
+    // the rhs rows of the current ones
+    int c_nxt = col_indices[min(p + lane, q - 1)];
+    for (int base = p; base < q; base += kWave) {
+        const int c = base + lane < q ? c_nxt : 0;
+        c_nxt = col_indices[min(base + kWave + lane, q - 1)];
+        const int cnt = min(kWave, q - base);
+        const float o = sddmm_chunk<VEC, G1, DS, MASKED>(D, lane, cnt, c, lhs_row, lq, rhs);
+        if (base + lane < q) out[base + lane] = o;
+    }
+}
+
 // MASKED = false: D == G1 * VEC * DS exactly, every access of every lane falls inside the row.
 template <int VEC, int G1, int DS, bool MASKED, int W, int R>
 __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* __restrict__ row_offsets,
@@ -25,12 +54,10 @@ __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* 
                                                        const float* __restrict__ lhs, const float* __restrict__ rhs,
                                                        float* __restrict__ out)
 {
-    using VecT = Vec<VEC>;
     __shared__ int s_off[R + 1];
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int g = lane % G1;
     const int r0 = blockIdx.x * R;
     const int nr = min(R, M - r0);
 
@@ -52,25 +79,7 @@ __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* 
         const int p = __builtin_amdgcn_readfirstlane(pos);
         const float* lhs_row = lhs + (size_t)(r0 + r) * D;
 
-        VecT lq[DS > 0 ? DS : 1];
-        if constexpr (DS > 0) {
-#pragma unroll
-            for (int s = 0; s < DS; ++s) {
-                const int d = (s * G1 + g) * VEC;
-                if constexpr (MASKED) lq[s] = d < D ? VecT::gload_clip(lhs_row, d, D) : VecT::zero();
-                else lq[s] = VecT::gload(lhs_row + d);
-            }
-        }
-        // 64 column indices per pass, one per lane; the next 64 are requested (index clamped, no condition) before
-        // the rhs rows of the current ones
-        int c_nxt = col_indices[min(p + lane, q - 1)];
-        for (int base = p; base < q; base += kWave) {
-            const int c = base + lane < q ? c_nxt : 0;
-            c_nxt = col_indices[min(base + kWave + lane, q - 1)];
-            const int cnt = min(kWave, q - base);
-            const float o = sddmm_chunk<VEC, G1, DS, MASKED>(D, lane, cnt, c, lhs_row, lq, rhs);
-            if (base + lane < q) out[base + lane] = o;
-        }
+        sddmm_segment<VEC, G1, DS, MASKED>(p, q, D, col_indices, lhs_row, rhs, out, lane);
         pos = q;
         ++r;
         while (r < nr && s_off[r + 1] <= pos) ++r;
@@ -148,6 +157,76 @@ hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t str
         }
     } else if (s.G1 == 4 && s.DS == 1) {
         return launch_wr<1, 4, 1>(x, s.W, s.R, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+// ---- flat schedule: every wave owns `chunk` consecutive nonzeros of the mask, whatever rows they belong to ---------
+// (see spmm.hip; here every result goes to its own CSR slot, so there is nothing to combine and no workspace)
+template <int VEC, int G1, int DS, bool MASKED>
+__global__ __launch_bounds__(kFlatWaves * 64) void sddmm_flat_kernel(int M, int D, int nnz, int chunk,
+                                                                      const int* __restrict__ row_offsets,
+                                                                      const int* __restrict__ col_indices,
+                                                                      const float* __restrict__ lhs,
+                                                                      const float* __restrict__ rhs, float* __restrict__ out)
+{
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const long long a64 = ((long long)blockIdx.x * kFlatWaves + w) * chunk;
+    if (a64 >= nnz) return;  // wave-uniform
+    const int a = (int)a64;
+    const int b = (int)min((long long)nnz, a64 + chunk);
+    int r = find_row(row_offsets, M, a, lane);
+    int rbase = r;
+    int win = window_load(row_offsets, M, rbase, lane);
+    int pos = a;
+    while (true) {
+        if (r - rbase >= kWinRows) {
+            rbase = r;
+            win = window_load(row_offsets, M, rbase, lane);
+        }
+        const int re = window_get(win, r - rbase + 1);
+        const int q = min(re, b);
+        sddmm_segment<VEC, G1, DS, MASKED>(pos, q, D, col_indices, lhs + (size_t)r * D, rhs, out, lane);
+        pos = q;
+        if (pos >= b) break;
+        r = window_next_row(row_offsets, M, pos, lane, win, rbase);
+    }
+}
+
+template <int VEC, int G1, int DS>
+static hipError_t launch_flat(const SddmmArgs& x, int chunk, hipStream_t stream)
+{
+    const long long units = ((long long)x.nnz + chunk - 1) / chunk;
+    const unsigned blocks = (unsigned)((units + kFlatWaves - 1) / kFlatWaves);
+    if constexpr (DS > 0) {
+        if (x.D == G1 * VEC * DS) {
+            hipLaunchKernelGGL((sddmm_flat_kernel<VEC, G1, DS, false>), dim3(blocks), dim3(kFlatWaves * 64), 0, stream, x.M,
+                               x.D, x.nnz, chunk, x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((sddmm_flat_kernel<VEC, G1, DS, true>), dim3(blocks), dim3(kFlatWaves * 64), 0, stream, x.M, x.D,
+                       x.nnz, chunk, x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
+    return hipGetLastError();
+}
+
+hipError_t sddmm_flat_launch(const SddmmArgs& x, const SddmmShape& s, int chunk, hipStream_t stream)
+{
+    if (s.vec == 4) {
+        if (s.G1 == 4 && s.DS == 1) return launch_flat<4, 4, 1>(x, chunk, stream);
+        if (s.G1 == 8) {
+            switch (s.DS) {
+                case 1: return launch_flat<4, 8, 1>(x, chunk, stream);
+                case 2: return launch_flat<4, 8, 2>(x, chunk, stream);
+                case 4: return launch_flat<4, 8, 4>(x, chunk, stream);
+                case 8: return launch_flat<4, 8, 8>(x, chunk, stream);
+                case 16: return launch_flat<4, 8, 16>(x, chunk, stream);
+                case 0: return launch_flat<4, 8, 0>(x, chunk, stream);
+            }
+        }
+    } else if (s.G1 == 4 && s.DS == 1) {
+        return launch_flat<1, 4, 1>(x, chunk, stream);
     }
     return hipErrorInvalidValue;
 }

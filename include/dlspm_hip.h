@@ -125,7 +125,8 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
  * SDDMM), [2] accesses per lane per dense row, [3] G1 lanes per dot product (SDDMM, fused stage 1; 0 for SpMM),
  * [4] accesses per lane per dot product (0 = run-time loop), [5] waves per workgroup, [6] rows per workgroup,
  * [7] column tiles, [8] nonzeros per wave of the flat schedule that a call WITH workspace would use (0 = such a call
- * uses the workgroup-per-row-block schedule too), [9] number of such waves. Returns DLSPM_OK or DLSPM_E_INVALID_ARG.
+ * uses the workgroup-per-row-block schedule too; SDDMM needs no workspace for it), [9] number of such waves.
+ * Returns DLSPM_OK or DLSPM_E_INVALID_ARG.
  */
 int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape);
 

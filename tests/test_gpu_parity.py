@@ -335,6 +335,10 @@ def test_flat_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
     assert oracle.rel_frobenius(dl.spmm(ro_d, ci_d, va_d, B_d, K=K).cpu().numpy(), ref) <= TOL
     assert (got.cpu().numpy()[np.diff(ro) == 0] == 0).all()
 
+    assert dl.describe_launch(dl.OP_SDDMM, M, K, N, nnz)["flat_chunk"] > 0  # SDDMM: by the size rule alone
+    gotS = dl.sddmm(ro_d, ci_d, Q_d, B_d)
+    assert oracle.rel_frobenius(gotS.cpu().numpy(), oracle.sddmm(ro, ci, Q, B, omp=True)) <= TOL
+
     needf = dl.workspace_bytes(dl.OP_FUSED, M, K, N, nnz)
     assert needf > 0
     wsf = torch.empty(needf, dtype=torch.uint8, device="cuda")

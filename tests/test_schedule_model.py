@@ -314,3 +314,35 @@ def test_gpu_flat_fused_equals_model_bit_for_bit(model, dl, monkeypatch, kind, M
     got = out.cpu().numpy()
     assert np.array_equal(got.view(np.uint32), O.view(np.uint32)), \
         f"shape {fs}: {np.count_nonzero(got.view(np.uint32) != O.view(np.uint32))} of {got.size} elements differ in their bits"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,M,K,D,n_long,chunk", [("uniform", 300, 200, 64, 0, 128), ("long_and_empty", 1500, 700, 128, 3, 256),
+                                                      ("skewed", 130, 257, 49, 0, 64), ("long_and_empty", 5000, 600, 32, 5, 64),
+                                                      ("uniform", 40, 300, 1027, 0, 320), ("empty_rows", 500, 100, 3, 0, 64)])
+def test_gpu_flat_sddmm_equals_model_and_the_row_block_schedule_bit_for_bit(model, dl, monkeypatch, kind, M, K, D, n_long, chunk):
+    """SDDMM's flat schedule changes which wave computes a dot product, not how: both schedules must give the model's bits."""
+    import torch
+
+    rng = np.random.default_rng(61 + M + D)
+    if kind == "long_and_empty":
+        ro, ci = long_and_empty_rows(rng, M, K, n_long, K - 50, 3)
+    else:
+        ro, ci = random_csr(rng, M, K, kind, 0.2)
+    Q = rng.normal(0, 1, (M, D)).astype(np.float32)
+    Km = rng.normal(0, 1, (K, D)).astype(np.float32)
+    sh = dl.describe_launch(dl.OP_SDDMM, M, K, D, ci.size)
+    assert sh["flat_chunk"] == 0
+    ref = np.empty(ci.size, dtype=np.float32)
+    model.model_sddmm(M, D, pi(ro), pi(ci), pf(Q), pf(Km), sh["vec"], sh["G1"], sh["DS"], pf(ref))
+    args = (dev(torch, ro), dev(torch, ci), dev(torch, Q), dev(torch, Km))
+    block = dl.sddmm(*args).cpu().numpy()
+    monkeypatch.setenv("DLSPM_FLAT", "1")
+    monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
+    assert dl.describe_launch(dl.OP_SDDMM, M, K, D, ci.size)["flat_chunk"] == chunk
+    assert dl.workspace_bytes(dl.OP_SDDMM, M, K, D, ci.size) == 0
+    out = torch.full((ci.size,), float("nan"), dtype=torch.float32, device="cuda")
+    dl.sddmm(*args, out=out)
+    flat = out.cpu().numpy()
+    assert np.array_equal(flat.view(np.uint32), ref.view(np.uint32))
+    assert np.array_equal(block.view(np.uint32), ref.view(np.uint32))
