@@ -153,8 +153,8 @@ def cpu_baseline(dl, c, acct):
 def main():
     args = parse()
     if args.gpus != 1:
-        print("bench.py measures one GPU: this path has no multi-GPU part (rows are independent; see DESIGN.md). "
-              "Run with --gpus 1.", file=sys.stderr)
+        print("bench.py measures one GPU: this path has no multi-GPU part (output rows are independent, so sharding "
+              "would split the rows and replicate the dense operand, with no exchange). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
     import numpy as np
     import torch

@@ -28,7 +28,7 @@ def write_smtx(path, M, K, ro, ci):
         f.write(" ".join(map(str, ci)) + "\n")
 
 
-# ---- CPU: the failure paths the reference's drivers have (SURVEY: wrong argc, unopenable file, short file, bad CSR)
+# ---- CPU: the failure paths the reference's drivers have (wrong argc, unopenable file, short file, bad CSR)
 @pytest.mark.parametrize("app", ["spmm_run", "sddmm_run", "fused_run"])
 def test_usage_and_file_errors(app, tmp_path):
     rc, out = run(app)
