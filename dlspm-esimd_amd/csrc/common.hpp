@@ -146,7 +146,8 @@ __device__ __forceinline__ int find_row(const int* __restrict__ row_offsets, int
         const long long span = hi - lo;
         const int idx = lo + (int)((span * (lane + 1)) >> 6);  // non-decreasing in lane, lane 63 reads `hi`
         const unsigned long long le = __ballot(row_offsets[idx] <= pos);  // a prefix of the lanes
-        const int n = __popcll(le);                                        // < 64 because row_offsets[hi] > pos
+        const int n = min(__popcll(le), 63);  // < 64 because row_offsets[hi] > pos (clamped: offsets that are not
+                                              // sorted must not take the search outside [0, M])
         const int new_lo = lo + (int)((span * n) >> 6);        // n == 0: lo itself
         const int new_hi = lo + (int)((span * (n + 1)) >> 6);  // first sample above pos
         lo = __builtin_amdgcn_readfirstlane(new_lo);
@@ -174,7 +175,8 @@ __device__ __forceinline__ int window_next_row(const int* __restrict__ row_offse
     const unsigned long long gt = __ballot(win > pos);  // a suffix of the lanes: entries are non-decreasing
     if (gt != 0) {
         const int t = __builtin_ctzll(gt);  // smallest entry above pos: the row ends there, so it is row t - 1
-        return rbase + t - 1;               // t >= 1: entry 0 is the start of a row at or before pos
+        return min(rbase + max(t, 1) - 1, M - 1);  // t >= 1 (entry 0 starts a row at or before pos) and the row is
+                                                   // below M for sorted offsets; clamped for unsorted ones
     }
     const int r = find_row(row_offsets, M, pos, lane);
     rbase = r;

@@ -204,6 +204,7 @@ struct Options {
     int warmup = 5;
     int iters = 20;  // the reference keeps the minimum of 20 launches (SPMM/spmm-esimd-fromfile2.cpp:194-243)
     bool cold = false;
+    bool workspace = true;  // allocate and pass what dlspm_workspace_bytes asks for (--no-workspace: pass none)
     std::string csv, dump;
     double tol = 1e-4;  // relative Frobenius error allowed between the kernel and the check kernel
 };
@@ -286,9 +287,17 @@ struct CaseSpec {
     int cfg = 0;
     int M = 0, K = 0, N = 0;
     double density = 0;
+    double sigma = 0;  // > 0: row lengths lognormal around density*K with this sigma (skewed rows) instead of Bernoulli
     uint64_t seed = 1;
     std::string file;
 };
+
+// pattern of a --shape case
+inline Csr synthetic_pattern(const CaseSpec& s)
+{
+    return s.sigma > 0 ? pattern_lognormal_rows(s.seed, s.M, s.K, s.density * s.K, s.sigma)
+                       : pattern_bernoulli(s.seed, s.M, s.K, s.density);
+}
 
 // the grid of SPMM/spmm-esimd-allbenchs2.cpp:252-255 (same in SDDMM/sddmm-esimd-allbench_v4.cpp:241-244)
 inline std::vector<CaseSpec> sputnik_grid(int max_m)
@@ -321,10 +330,11 @@ inline std::string usage(const char* app, const char* width)
     std::ostringstream u;
     u << "Usage: " << app << " <filename>.smtx <" << width << ">            one matrix from a DLMC .smtx file\n"
       << "       " << app << " --batch <list>                      lines '<filename>.smtx <" << width << ">', '#' comments\n"
-      << "       " << app << " --shape M K " << width << " density [--seed S]   one synthetic matrix (Bernoulli pattern)\n"
+      << "       " << app << " --shape M K " << width << " density [--seed S] [--sigma s]   one synthetic matrix (Bernoulli pattern;\n"
+      << "                                                     --sigma: lognormal row lengths, skewed)\n"
       << "       " << app << " --sweep [--max-m M]                  the 12 x {32,128} x {0.3,0.2,0.1} benchmark grid\n"
       << "       " << app << " --cfg <id>                           a seeded benchmark configuration (1..5)\n"
-      << "options: --iters n (20)  --warmup n (5)  --cold  --csv <file>  --dump <dir>  --tol x (1e-4)";
+      << "options: --iters n (20)  --warmup n (5)  --cold  --csv <file>  --dump <dir>  --tol x (1e-4)  --no-workspace";
     return u.str();
 }
 
@@ -348,6 +358,8 @@ inline Cli parse_cli(int argc, char** argv, const char* app, const char* width)
             cli.cases.push_back(s);
         }
         else if (a == "--seed") { need(i, 1); const uint64_t sd = std::stoull(argv[++i]); if (!cli.cases.empty()) cli.cases.back().seed = sd; }
+        else if (a == "--sigma") { need(i, 1); const double sg = std::stod(argv[++i]); if (!cli.cases.empty()) cli.cases.back().sigma = sg; }
+        else if (a == "--no-workspace") cli.opt.workspace = false;
         else if (a == "--sweep") sweep = true;
         else if (a == "--max-m") { need(i, 1); max_m = std::stoi(argv[++i]); }
         else if (a == "--batch") {

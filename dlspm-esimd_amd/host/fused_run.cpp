@@ -26,7 +26,7 @@ static bool run_case(const CaseSpec& s, const Options& opt)
             std::cout << "Filename = " << s.file << ", batchsize (=NSZ) = " << D << std::endl;
             a = load_smtx(s.file);
         } else {
-            a = pattern_bernoulli(s.seed, s.M, s.K, s.density);
+            a = synthetic_pattern(s);
         }
         if (D < 1) throw std::invalid_argument("NSZ must be at least 1");
         Q.resize((size_t)a.M * D);
@@ -44,7 +44,7 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     if (dlspm_csr_check(M, K, nnz, ro_d.p, ci_d.p, nullptr) != DLSPM_OK) throw std::invalid_argument("malformed CSR structure");
     DLSPM_HIP_CHECK(hipMemset(O_d.p, 0xFF, (size_t)M * D * sizeof(float)));
 
-    const size_t ws_bytes = dlspm_workspace_bytes(DLSPM_OP_FUSED, M, K, D, nnz);  // 0 for small problems
+    const size_t ws_bytes = opt.workspace ? dlspm_workspace_bytes(DLSPM_OP_FUSED, M, K, D, nnz) : 0;  // 0 for small problems
     DevBuf<char> ws(ws_bytes);
     if (ws_bytes) std::printf("workspace: %zu bytes (flat schedule)\n", ws_bytes);
     const Timing t = time_launches(opt, [&]() {

@@ -23,7 +23,7 @@ static bool run_case(const CaseSpec& s, const Options& opt)
             std::cout << "Filename = " << s.file << ", batchsize (=NSZ) = " << D << std::endl;
             a = load_smtx(s.file);
         } else {
-            a = pattern_bernoulli(s.seed, s.M, s.K, s.density);
+            a = synthetic_pattern(s);
         }
         if (D < 1) throw std::invalid_argument("NSZ must be at least 1");
         lhs.resize((size_t)a.M * D);

@@ -22,7 +22,7 @@ static bool run_case(const CaseSpec& s, const Options& opt)
             std::cout << "Filename = " << s.file << ", batchsize (=NSZ) = " << N << std::endl;
             a = load_smtx(s.file);
         } else {
-            a = pattern_bernoulli(s.seed, s.M, s.K, s.density);
+            a = synthetic_pattern(s);
         }
         if (N < 1) throw std::invalid_argument("NSZ must be at least 1");
         values.resize(a.nnz());
@@ -41,7 +41,7 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     DLSPM_HIP_CHECK(hipMemset(C_d.p, 0xFF, (size_t)M * N * sizeof(float)));  // NaN pattern: every element must be written
 
     // the caller owns the workspace, as it owns every other buffer: 0 bytes for small problems
-    const size_t ws_bytes = dlspm_workspace_bytes(DLSPM_OP_SPMM, M, K, N, nnz);
+    const size_t ws_bytes = opt.workspace ? dlspm_workspace_bytes(DLSPM_OP_SPMM, M, K, N, nnz) : 0;
     DevBuf<char> ws(ws_bytes);
     if (ws_bytes) std::printf("workspace: %zu bytes (flat schedule)\n", ws_bytes);
     const Timing t = time_launches(opt, [&]() {
