@@ -100,6 +100,19 @@ void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w
     }
 }
 
+// longest row and number of rows without nonzeros (dlspm_csr_row_stats); stats[0] = max, stats[1] = empty rows
+__global__ void row_stats_kernel(int M, const int* __restrict__ row_offsets, int* __restrict__ stats)
+{
+    int longest = 0, empty = 0;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < M; i += gridDim.x * blockDim.x) {
+        const int len = row_offsets[i + 1] - row_offsets[i];
+        longest = max(longest, len);
+        empty += len == 0 ? 1 : 0;
+    }
+    if (longest > 0) atomicMax(&stats[0], longest);
+    if (empty > 0) atomicAdd(&stats[1], empty);
+}
+
 // D == 0 in SDDMM: every dot product is the empty sum (a kernel, not a memset, so that callers may capture the call)
 __global__ void fill_zero_kernel(float* __restrict__ out, int n)
 {
@@ -261,6 +274,32 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
     (void)hipFree(d_flags);
     if (e != hipSuccess) return fail_hip(e);
     return h_flags == 0 ? DLSPM_OK : DLSPM_E_INVALID_CSR;
+}
+
+int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_row_len, int* empty_rows)
+{
+    if (M < 0 || (M > 0 && !row_offsets)) return DLSPM_E_INVALID_ARG;
+    int h[2] = {0, 0};
+    if (M > 0) {
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        int* d = nullptr;
+        hipError_t e = hipMalloc(&d, 2 * sizeof(int));
+        if (e != hipSuccess) return fail_hip(e);
+        e = hipMemsetAsync(d, 0, 2 * sizeof(int), s);
+        if (e == hipSuccess) {
+            int blocks = (M + 255) / 256;
+            blocks = blocks > 1024 ? 1024 : blocks;
+            hipLaunchKernelGGL(row_stats_kernel, dim3(blocks), dim3(256), 0, s, M, row_offsets, d);
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess) e = hipMemcpyAsync(h, d, 2 * sizeof(int), hipMemcpyDeviceToHost, s);
+        if (e == hipSuccess) e = hipStreamSynchronize(s);
+        (void)hipFree(d);
+        if (e != hipSuccess) return fail_hip(e);
+    }
+    if (max_row_len) *max_row_len = h[0];
+    if (empty_rows) *empty_rows = h[1];
+    return DLSPM_OK;
 }
 
 int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape)

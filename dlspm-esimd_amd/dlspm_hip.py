@@ -28,6 +28,7 @@ EXPORTS = (
     "dlspm_workspace_bytes",
     "dlspm_csr_check",
     "dlspm_describe_launch",
+    "dlspm_csr_row_stats",
     "dlspm_status_string",
     "dlspm_last_hip_error",
     "dlspm_version",
@@ -63,6 +64,8 @@ def lib() -> ctypes.CDLL:
         L.dlspm_csr_check.restype = ci
         L.dlspm_describe_launch.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci)]
         L.dlspm_describe_launch.restype = ci
+        L.dlspm_csr_row_stats.argtypes = [ci, vp, vp, ctypes.POINTER(ci), ctypes.POINTER(ci)]
+        L.dlspm_csr_row_stats.restype = ci
         L.dlspm_status_string.argtypes = [ci]
         L.dlspm_status_string.restype = ctypes.c_char_p
         L.dlspm_last_hip_error.restype = ci
@@ -179,6 +182,18 @@ def _workspace(ws):
     if not ws.is_cuda or not ws.is_contiguous():
         raise ValueError("workspace must be a contiguous GPU tensor")
     return ctypes.c_void_p(ws.data_ptr()), ws.numel() * ws.element_size()
+
+
+def csr_row_stats(row_offsets):
+    """(longest row, rows without nonzeros) of a CSR structure on the GPU; synchronises the current stream."""
+    import torch
+
+    mx, em = ctypes.c_int(0), ctypes.c_int(0)
+    st = lib().dlspm_csr_row_stats(row_offsets.numel() - 1, _ptr(row_offsets, torch.int32, "row_offsets"), _stream(),
+                                   ctypes.byref(mx), ctypes.byref(em))
+    if st != OK:
+        raise DlspmError(st, "dlspm_csr_row_stats")
+    return mx.value, em.value
 
 
 def csr_check(M, K, row_offsets, col_indices) -> int:

@@ -204,10 +204,29 @@ struct Options {
     int warmup = 5;
     int iters = 20;  // the reference keeps the minimum of 20 launches (SPMM/spmm-esimd-fromfile2.cpp:194-243)
     bool cold = false;
-    bool workspace = true;  // allocate and pass what dlspm_workspace_bytes asks for (--no-workspace: pass none)
+    // whether to allocate and pass what dlspm_workspace_bytes asks for: by default only for matrices whose longest row
+    // is at least four times the mean row (dlspm_csr_row_stats); --workspace: always, --no-workspace: never
+    enum Workspace { kAuto, kAlways, kNever } workspace = kAuto;
     std::string csv, dump;
     double tol = 1e-4;  // relative Frobenius error allowed between the kernel and the check kernel
 };
+
+// Bytes of workspace this run passes to the library: what it asks for when the rows are uneven enough for the flat
+// schedule to pay (measured: from lognormal sigma ~1 on, i.e. a longest row several times the mean), none for even rows.
+inline size_t workspace_to_pass(const Options& opt, int op, int M, int K, int width, int nnz, const int* row_offsets_dev)
+{
+    const size_t want = dlspm_workspace_bytes(op, M, K, width, nnz);
+    if (want == 0 || opt.workspace == Options::kNever) return 0;
+    int longest = 0, empty = 0;
+    if (dlspm_csr_row_stats(M, row_offsets_dev, nullptr, &longest, &empty) != DLSPM_OK) throw std::runtime_error("dlspm_csr_row_stats failed");
+    const double mean = M > 0 ? (double)nnz / M : 0.0;
+    const bool uneven = longest >= 4.0 * mean;
+    std::printf("rows: longest %d, mean %.1f, empty %d -> %s\n", longest, mean, empty,
+                opt.workspace == Options::kAlways ? "workspace passed (--workspace)"
+                : uneven                          ? "uneven, workspace passed (flat schedule)"
+                                                  : "even, no workspace (row-block schedule)");
+    return (opt.workspace == Options::kAlways || uneven) ? want : 0;
+}
 
 template <typename Launch> Timing time_launches(const Options& opt, Launch&& launch)
 {
@@ -334,7 +353,7 @@ inline std::string usage(const char* app, const char* width)
       << "                                                     --sigma: lognormal row lengths, skewed)\n"
       << "       " << app << " --sweep [--max-m M]                  the 12 x {32,128} x {0.3,0.2,0.1} benchmark grid\n"
       << "       " << app << " --cfg <id>                           a seeded benchmark configuration (1..5)\n"
-      << "options: --iters n (20)  --warmup n (5)  --cold  --csv <file>  --dump <dir>  --tol x (1e-4)  --no-workspace";
+      << "options: --iters n (20)  --warmup n (5)  --cold  --csv <file>  --dump <dir>  --tol x (1e-4)  --workspace | --no-workspace";
     return u.str();
 }
 
@@ -359,7 +378,8 @@ inline Cli parse_cli(int argc, char** argv, const char* app, const char* width)
         }
         else if (a == "--seed") { need(i, 1); const uint64_t sd = std::stoull(argv[++i]); if (!cli.cases.empty()) cli.cases.back().seed = sd; }
         else if (a == "--sigma") { need(i, 1); const double sg = std::stod(argv[++i]); if (!cli.cases.empty()) cli.cases.back().sigma = sg; }
-        else if (a == "--no-workspace") cli.opt.workspace = false;
+        else if (a == "--no-workspace") cli.opt.workspace = Options::kNever;
+        else if (a == "--workspace") cli.opt.workspace = Options::kAlways;
         else if (a == "--sweep") sweep = true;
         else if (a == "--max-m") { need(i, 1); max_m = std::stoi(argv[++i]); }
         else if (a == "--batch") {

@@ -118,6 +118,16 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
                     void* stream);
 
 /*
+ * Longest row and number of rows without nonzeros of a CSR structure that lives on the device (either result
+ * pointer may be NULL). Synchronises `stream`; meant to be called once per matrix, like dlspm_csr_check. It
+ * has no counterpart in the reference, whose launch sizing looks at M and N only
+ * (SPMM/spmmesimd2.hpp:30-60).
+ * Use: the compute calls cannot see how evenly the nonzeros are spread over the rows; a caller who finds
+ * max_row_len several times nnz / M should pass a workspace (see above), a caller with even rows need not.
+ */
+int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_row_len, int* empty_rows);
+
+/*
  * Launch shape the library would use for these sizes, for tuning reports and for host-side models of the
  * schedule (the reference's SpmmEsimdCPU / FusedEsimdCPU, SPMM/spmm-esimd-v1.cpp:83-169 and
  * FUSED/fused.cpp:93-216, play that role for its kernels). Host-only, never touches the device.

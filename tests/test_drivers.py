@@ -198,3 +198,17 @@ def test_dlmc_batch_list(tmp_path):
         rc, out = run(app, "--batch", tmp_path / "rn50.txt", "--csv", tmp_path / f"{app}.csv", "--iters", 5)
         assert rc == 0 and out.count("PASS") == 3, out
         assert len(open(tmp_path / f"{app}.csv").read().strip().splitlines()) == 3
+
+
+@pytest.mark.gpu
+def test_drivers_pass_the_workspace_only_for_uneven_rows():
+    """3.3 M nonzeros: large enough for the flat schedule. Even rows: the driver passes no workspace; lognormal rows
+    (sigma 1.5): it does; both self-check against the on-device gold loop."""
+    rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--iters", 3)
+    assert rc == 0 and "PASS" in out and "even, no workspace" in out and "workspace:" not in out, out
+    rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 1.5, "--iters", 3)
+    assert rc == 0 and "PASS" in out and "uneven, workspace passed" in out and "workspace:" in out, out
+    rc, out = run("fused_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 1.5, "--iters", 3)
+    assert rc == 0 and "PASS" in out and "uneven, workspace passed" in out, out
+    rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--workspace", "--iters", 3)
+    assert rc == 0 and "PASS" in out and "workspace passed (--workspace)" in out, out

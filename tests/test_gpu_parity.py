@@ -376,6 +376,15 @@ def test_exact_integer_properties_at_large_size(torch_cuda, dl):
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
+def test_csr_row_stats(torch_cuda, dl):
+    torch = torch_cuda
+    rng = np.random.default_rng(3)
+    for (M, K, kind) in [(1, 1, "empty"), (1000, 300, "skewed"), (5000, 64, "empty_rows"), (70000, 40, "uniform")]:
+        ro, ci = random_csr(rng, M, K, kind, 0.1)
+        lens = np.diff(ro)
+        assert dl.csr_row_stats(dev(torch, ro)) == (int(lens.max()), int((lens == 0).sum()))
+
+
 def test_error_statuses(torch_cuda, dl):
     torch = torch_cuda
     z = torch.zeros(4, dtype=torch.int32, device="cuda")
