@@ -48,6 +48,31 @@ def test_host_only_entry_points_answer_without_a_gpu(dl):
     assert L.sddmm_csr_f32(5, 5, 4, 0, None, None, None, None, None, None, 0, None) == dl.OK
 
 
+def test_flat_schedule_rule_and_workspace_size(dl, monkeypatch):
+    """Host-only: the size rule of the flat schedule and the workspace it asks for (units x 2 x width floats)."""
+    monkeypatch.delenv("DLSPM_FLAT", raising=False)
+    monkeypatch.delenv("DLSPM_FLAT_CHUNK", raising=False)
+    M, K, nnz = 8192, 4096, 3355443
+    sh = dl.describe_launch(dl.OP_SPMM, M, K, 128, nnz)
+    assert sh["flat_chunk"] == 512 and sh["flat_units"] == -(-nnz // 512)
+    assert dl.workspace_bytes(dl.OP_SPMM, M, K, 128, nnz) == sh["flat_units"] * 2 * 128 * 4
+    assert dl.workspace_bytes(dl.OP_FUSED, M, K, 128, nnz) == sh["flat_units"] * 2 * 128 * 4
+    assert dl.workspace_bytes(dl.OP_SDDMM, M, K, 128, nnz) == 0               # nothing to combine
+    assert dl.describe_launch(dl.OP_SDDMM, M, K, 32, nnz)["flat_chunk"] == 512  # but the schedule is used, any width
+    assert dl.workspace_bytes(dl.OP_SPMM, M, K, 64, nnz) == 0                 # narrow dense rows: row-block schedule
+    assert dl.workspace_bytes(dl.OP_SPMM, M, K, 128, (1 << 21) - 1) == 0      # too few nonzeros
+    assert dl.workspace_bytes(dl.OP_SPMM, 65536, K, 128, nnz) == 0            # rows too short (51 on average)
+    big = 26843545                                                            # the chunk grows to keep ~32768 units
+    shb = dl.describe_launch(dl.OP_SPMM, 32768, 8192, 128, big)
+    assert shb["flat_chunk"] == 832 and shb["flat_units"] == -(-big // 832)
+    for cfg_sizes in [(512, 512, 128, 78643), (2048, 512, 256, 105687), (2048, 512, 392, 208896), (4096, 4096, 64, 324737)]:
+        for op in (dl.OP_SPMM, dl.OP_SDDMM, dl.OP_FUSED):
+            assert dl.workspace_bytes(op, *cfg_sizes) == 0 and dl.describe_launch(op, *cfg_sizes)["flat_chunk"] == 0
+    monkeypatch.setenv("DLSPM_FLAT", "1")
+    monkeypatch.setenv("DLSPM_FLAT_CHUNK", "192")
+    assert dl.workspace_bytes(dl.OP_SPMM, 100, 50, 7, 1000) == -(-1000 // 192) * 2 * 7 * 4
+
+
 def test_binding_refuses_host_tensors(dl):
     import torch
 
