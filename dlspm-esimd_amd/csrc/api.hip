@@ -38,10 +38,10 @@ static bool split_override(int& W, int& R)
 // Flat schedule (every wave owns a fixed number of consecutive nonzeros; partial rows in the caller's workspace):
 // chosen when the matrix is large enough that the second launch does not matter, its rows are long enough that a wave
 // walks few of them in sequence, and a dense row is wide enough to keep a whole wave or half of one busy. Measured on
-// MI355X against the workgroup-per-row-block schedule: equal within a few per cent on uniform row lengths from these
-// sizes on, 1.2-1.9x faster on lognormal row lengths (sigma 1-2); slower below them (short rows cost a wave one
-// dependent memory round trip each). DLSPM_FLAT=0/1 overrides the rule and DLSPM_FLAT_CHUNK the nonzeros per wave, for
-// tuning sweeps and tests.
+// MI355X against the workgroup-per-row-block schedule (SpMM and fused, 2-27 M nonzeros, widths 128 and 256): 5-15 %
+// slower on even row lengths, 10-30 % faster on lognormal row lengths (sigma 1-2); below these sizes it loses (short
+// rows cost a wave one dependent memory round trip each). DLSPM_FLAT=0/1 overrides the rule and DLSPM_FLAT_CHUNK the
+// nonzeros per wave, for tuning sweeps and tests.
 constexpr int kFlatMinNnz = 1 << 21;
 constexpr int kFlatMinRow = 256;         // mean nonzeros per row
 constexpr int kFlatMinLanes = 32;        // lanes per dense row (widths above 64 floats)

@@ -31,7 +31,7 @@ def check_csr_untouched(ro_d, ci_d, ro, ci):
     assert np.array_equal(ci_d.cpu().numpy(), ci), "col_indices changed"
 
 
-# (M, K, N, kind, density): N picks the lane layout (G = 8/16/32/64, V = 1/2, scalar path for N % 4 != 0),
+# (M, K, N, kind, density): N picks the lane layout (G = 8/16/32/64, V = 1/2, dword path for N < 4),
 # density and kind pick the (W, R) split and exercise shared rows, empty rows and ragged tails.
 SPMM_CASES = [
     (1, 1, 1, "full", 1.0),
