@@ -376,6 +376,85 @@ def test_exact_integer_properties_at_large_size(torch_cuda, dl):
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
+def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
+    """Both schedules only enqueue kernels (no memset, no allocation, no synchronisation), so a call may be captured.
+    The graph is replayed several times with eager work and synchronisations in between, on changed inputs, and every
+    replay must equal the eager result bit for bit."""
+    torch = torch_cuda
+    rng = np.random.default_rng(91)
+    M, K, N = 700, 400, 128
+    ro, ci = random_csr(rng, M, K, "skewed", 0.2)
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    va = torch.randn(ci.size, device="cuda")
+    B = torch.randn(K, N, device="cuda")
+    Q = torch.randn(M, N, device="cuda")
+    for flat in (False, True):
+        if flat:
+            monkeypatch.setenv("DLSPM_FLAT", "1")
+            monkeypatch.setenv("DLSPM_FLAT_CHUNK", "128")
+        need = max(dl.workspace_bytes(dl.OP_SPMM, M, K, N, ci.size), dl.workspace_bytes(dl.OP_FUSED, M, K, N, ci.size))
+        assert (need > 0) == flat
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda") if flat else None
+        C = torch.empty(M, N, device="cuda")
+        S = torch.empty(ci.size, device="cuda")
+        O = torch.empty(M, N, device="cuda")
+        stream = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            dl.spmm(ro_d, ci_d, va, B, K=K, out=C, workspace=ws)  # warm-up outside the capture
+            stream.synchronize()
+            with torch.cuda.graph(graph, stream=stream):
+                dl.spmm(ro_d, ci_d, va, B, K=K, out=C, workspace=ws)
+                dl.sddmm(ro_d, ci_d, Q, B, out=S)
+                dl.fused(ro_d, ci_d, Q, B, B, 0.5, out=O, workspace=ws)
+        for rep in range(4):
+            va.copy_(torch.randn(ci.size, device="cuda"))  # eager work between the replays: new inputs
+            B.copy_(torch.randn(K, N, device="cuda"))
+            torch.cuda.synchronize()
+            C.fill_(float("nan")); S.fill_(float("nan")); O.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            got = (C.clone(), S.clone(), O.clone())
+            want = (dl.spmm(ro_d, ci_d, va, B, K=K, workspace=ws).clone(), dl.sddmm(ro_d, ci_d, Q, B).clone(),
+                    dl.fused(ro_d, ci_d, Q, B, B, 0.5, workspace=ws).clone())
+            torch.cuda.synchronize()
+            for g, w in zip(got, want):
+                assert torch.equal(g, w), f"replay {rep}, flat={flat}"
+
+
+def test_concurrent_calls_from_two_threads_on_two_streams(torch_cuda, dl, oracle):
+    """The library keeps no mutable global state: two host threads, each with its own stream, outputs and workspace."""
+    import threading
+
+    torch = torch_cuda
+    c = dl.make_config(2)
+    ro_d, ci_d, va, B = (dev(torch, c[k]) for k in ("row_offsets", "col_indices", "values", "d0"))
+    ref = dl.spmm(ro_d, ci_d, va, B, K=c["K"]).clone()
+    torch.cuda.synchronize()
+    results, errors = {}, []
+
+    def worker(tid):
+        try:
+            stream = torch.cuda.Stream()
+            out = torch.empty_like(ref)
+            with torch.cuda.stream(stream):
+                for _ in range(200):
+                    dl.spmm(ro_d, ci_d, va, B, K=c["K"], out=out)
+                stream.synchronize()
+            results[tid] = out
+        except Exception as e:  # surfaced in the main thread below
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for out in results.values():
+        assert torch.equal(out, ref)
+
+
 def test_csr_row_stats(torch_cuda, dl):
     torch = torch_cuda
     rng = np.random.default_rng(3)
