@@ -3,6 +3,7 @@ compute call is made without a GPU), and the host-side generators and accounting
 import ctypes
 import os
 import re
+import subprocess
 
 import numpy as np
 import pytest
@@ -22,6 +23,18 @@ def test_header_declares_the_three_named_entry_points():
     for required in ("spmm_csr_f32", "sddmm_csr_f32", "fused_sddmm_spmm_f32"):
         assert required in names
     assert len(names) >= 8
+
+
+def test_header_is_plain_c(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 (no C++ types, no torch types, no HIP headers)."""
+    src = tmp_path / "abi.c"
+    src.write_text('#include "dlspm_hip.h"\n'
+                   "int use(void) { int shape[10]; return dlspm_describe_launch(DLSPM_OP_SPMM, 1, 1, 1, 1, shape)"
+                   " + (int)dlspm_workspace_bytes(DLSPM_OP_FUSED, 1, 1, 1, 1); }\n")
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    r = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-fsyntax-only", "-I", inc, str(src)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
 
 
 def test_library_exports_every_declared_symbol(dl):
