@@ -346,3 +346,72 @@ def test_gpu_flat_sddmm_equals_model_and_the_row_block_schedule_bit_for_bit(mode
     flat = out.cpu().numpy()
     assert np.array_equal(flat.view(np.uint32), ref.view(np.uint32))
     assert np.array_equal(block.view(np.uint32), ref.view(np.uint32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_gpu_random_shapes_equal_model_bit_for_bit(model, dl, monkeypatch, seed):
+    """Forty random (shape, pattern, width, schedule, chunk) draws per seed, all three entry points, bit for bit."""
+    import torch
+
+    rng = np.random.default_rng(seed)
+    for it in range(40):
+        M = int(rng.choice([1, 2, 7, 63, 64, 65, 200, 700, 2500])) + int(rng.integers(0, 5))
+        K = int(rng.choice([1, 3, 64, 130, 500, 1500])) + int(rng.integers(0, 5))
+        N = int(rng.choice([1, 2, 3, 4, 5, 8, 31, 32, 33, 64, 100, 128, 196, 256, 257, 392, 512, 700, 1030]))
+        kind = str(rng.choice(["uniform", "skewed", "empty_rows", "full", "empty"]))
+        if kind == "full" and M * K > 300000:
+            kind = "uniform"
+        density = float(rng.choice([0.02, 0.1, 0.3, 0.7]))
+        ro, ci = random_csr(rng, M, K, kind, 1.0 if kind == "full" else density)
+        nnz = ci.size
+        flat = bool(rng.integers(0, 2)) and nnz > 0
+        chunk = int(rng.choice([64, 128, 192, 320, 512, 1024]))
+        monkeypatch.setenv("DLSPM_FLAT", "1" if flat else "0")
+        monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
+        tag = f"seed {seed} draw {it}: M {M} K {K} N {N} {kind} {density} nnz {nnz} flat {flat} chunk {chunk}"
+        print(tag, flush=True)
+        va = rng.normal(0, 1, max(nnz, 1)).astype(np.float32)
+        B = rng.normal(0, 1, (K, N)).astype(np.float32)
+        Q = rng.normal(0, 1, (M, N)).astype(np.float32)
+        V = rng.normal(0, 1, (K, N)).astype(np.float32)
+        ci2 = ci if nnz else np.zeros(1, np.int32)
+        ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+        bits = lambda a: np.ascontiguousarray(a).view(np.uint32)
+
+        sh = dl.describe_launch(dl.OP_SPMM, M, K, N, nnz)
+        if flat:
+            rc, C, writes = run_spmm_flat(model, ro, ci2, va, B, sh["G"], chunk)
+        else:
+            rc, C, writes = run_spmm(model, ro, ci2, va, B, sh["G"], sh["W"], sh["R"])
+        assert rc == 0 and (writes == 1).all(), tag
+        need = dl.workspace_bytes(dl.OP_SPMM, M, K, N, nnz)
+        ws = torch.full((max(need // 4, 1),), float("nan"), device="cuda") if flat else None
+        out = torch.full((M, N), float("nan"), device="cuda")
+        dl.spmm(ro_d, ci_d, dev(torch, va)[:nnz], dev(torch, B), K=K, out=out, workspace=ws)
+        assert np.array_equal(bits(out.cpu().numpy()), bits(C)), "spmm " + tag
+
+        if nnz:
+            sh = dl.describe_launch(dl.OP_SDDMM, M, K, N, nnz)
+            ref = np.empty(nnz, np.float32)
+            model.model_sddmm(M, N, pi(ro), pi(ci), pf(Q), pf(B), sh["vec"], sh["G1"], sh["DS"], pf(ref))
+            o = torch.full((nnz,), float("nan"), device="cuda")
+            dl.sddmm(ro_d, ci_d, dev(torch, Q), dev(torch, B), out=o)
+            assert np.array_equal(bits(o.cpu().numpy()), bits(ref)), "sddmm " + tag
+
+        fs = dl.describe_launch(dl.OP_FUSED, M, K, N, nnz)
+        scores = np.empty(max(nnz, 1), np.float32)
+        O = np.full((M, N), np.nan, np.float32)
+        writes = np.zeros((M, N), np.int32)
+        if flat:
+            rc = model.model_fused_flat(M, N, pi(ro), pi(ci2), pf(Q), pf(B), pf(V), 0.25, fs["vec"], fs["G1"], fs["DS"], fs["G"],
+                                        chunk, pf(scores), pf(O), pi(writes))
+        else:
+            rc = model.model_fused(M, N, pi(ro), pi(ci2), pf(Q), pf(B), pf(V), 0.25, fs["vec"], fs["G1"], fs["DS"], fs["G"],
+                                   fs["W"], fs["R"], pf(scores), pf(O), pi(writes))
+        assert rc == 0 and (writes == 1).all(), tag
+        need = dl.workspace_bytes(dl.OP_FUSED, M, K, N, nnz)
+        ws = torch.full((max(need // 4, 1),), float("nan"), device="cuda") if flat else None
+        out = torch.full((M, N), float("nan"), device="cuda")
+        dl.fused(ro_d, ci_d, dev(torch, Q), dev(torch, B), dev(torch, V), 0.25, out=out, workspace=ws)
+        assert np.array_equal(bits(out.cpu().numpy()), bits(O)), "fused " + tag
