@@ -38,14 +38,19 @@ static bool split_override(int& W, int& R)
 // Flat schedule (every wave owns a fixed number of consecutive nonzeros; partial rows in the caller's workspace):
 // chosen when the matrix is large enough that the second launch does not matter, its rows are long enough that a wave
 // walks few of them in sequence, and a dense row is wide enough to keep a whole wave or half of one busy. Measured on
-// MI355X against the workgroup-per-row-block schedule (SpMM and fused, 2-27 M nonzeros, widths 128 and 256): 5-15 %
-// slower on even row lengths, 10-30 % faster on lognormal row lengths (sigma 1-2); below these sizes it loses (short
-// rows cost a wave one dependent memory round trip each). DLSPM_FLAT=0/1 overrides the rule and DLSPM_FLAT_CHUNK the
-// nonzeros per wave, for tuning sweeps and tests.
-constexpr int kFlatMinNnz = 1 << 21;
-constexpr int kFlatMinRow = 256;         // mean nonzeros per row
+// MI355X against the workgroup-per-row-block schedule (SpMM and fused, 0.5-27 M nonzeros, widths 128 and 256): 5-40 %
+// slower on even row lengths (most below 2 M nonzeros), 10-60 % faster on lognormal row lengths (sigma 1-2); below
+// these sizes it loses even there (short rows cost a wave one dependent memory round trip each). Passing the
+// workspace is therefore the caller's way of saying that the rows are uneven (dlspm_csr_row_stats tells).
+// DLSPM_FLAT=0/1 overrides the rule and DLSPM_FLAT_CHUNK the nonzeros per wave, for tuning sweeps and tests.
+constexpr int kFlatMinNnz = 1 << 19;
+constexpr int kFlatMinRow = 64;          // mean nonzeros per row
 constexpr int kFlatMinLanes = 32;        // lanes per dense row (widths above 64 floats)
 constexpr int kFlatTargetUnits = 32768;  // waves wanted at least: four rounds of 8 waves on each of 1024 SIMDs
+// SDDMM takes the flat schedule by this rule alone (it needs no workspace, so the caller has no say): only where it
+// was measured to be equal on even rows
+constexpr int kFlatMinNnzSddmm = 1 << 21;
+constexpr int kFlatMinRowSddmm = 256;
 
 FlatPlan flat_plan(int M, int nnz, int width, int G)
 {
@@ -55,7 +60,7 @@ FlatPlan flat_plan(int M, int nnz, int width, int G)
     if (const char* e = std::getenv("DLSPM_FLAT")) force = std::atoi(e);
     const bool by_rule = nnz >= kFlatMinNnz && (long long)nnz >= (long long)kFlatMinRow * M && G >= kFlatMinLanes;
     if (force == 0 || (force < 0 && !by_rule)) return p;
-    long long chunk = 512;  // eight passes of 64 nonzeros per wave at least
+    long long chunk = nnz >= (1 << 21) ? 512 : 256;  // at least eight (four) passes of 64 nonzeros per wave
     const long long even = ((long long)nnz + kFlatTargetUnits - 1) / kFlatTargetUnits;
     if (even > chunk) chunk = (even + 63) / 64 * 64;
     if (const char* e = std::getenv("DLSPM_FLAT_CHUNK")) {
@@ -66,6 +71,14 @@ FlatPlan flat_plan(int M, int nnz, int width, int G)
     p.units = (int)(((long long)nnz + chunk - 1) / chunk);
     p.bytes = (size_t)p.units * 2 * (size_t)width * sizeof(float);
     return p;
+}
+
+static FlatPlan sddmm_flat_plan(int M, int nnz, int D)
+{
+    int force = -1;
+    if (const char* e = std::getenv("DLSPM_FLAT")) force = std::atoi(e);
+    if (force < 0 && (nnz < kFlatMinNnzSddmm || (long long)nnz < (long long)kFlatMinRowSddmm * M)) return FlatPlan{0, 0, 0};
+    return flat_plan(M, nnz, D, kWave);
 }
 
 void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w, int slots, int& W, int& R)
@@ -200,7 +213,7 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
     const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values};
     // the flat schedule needs no workspace here (nothing to combine), so the size rule alone decides; it has no
     // width condition for SDDMM (measured for D = 32 ... 256: equal on uniform rows, 15-33 % faster on skewed ones)
-    const FlatPlan plan = flat_plan(M, nnz, D, kWave);
+    const FlatPlan plan = sddmm_flat_plan(M, nnz, D);
     const hipError_t e = plan.chunk > 0 ? sddmm_flat_launch(args, shape, plan.chunk, static_cast<hipStream_t>(stream))
                                         : sddmm_launch(args, shape, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
@@ -318,7 +331,7 @@ int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape)
     } else if (op == DLSPM_OP_SDDMM) {
         const SddmmShape s = sddmm_choose(M, n, nnz, vec4);
         shape[0] = s.vec; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R; shape[7] = 1;
-        const FlatPlan fp = flat_plan(M, nnz, n, kWave);
+        const FlatPlan fp = sddmm_flat_plan(M, nnz, n);
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_FUSED) {
         const FusedShape s = fused_choose(M, n, nnz, vec4);

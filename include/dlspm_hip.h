@@ -26,10 +26,12 @@
  *     throws std::invalid_argument / std::logic_error on the host before launching).
  *   - `workspace` is optional device memory owned by the caller. NULL (or 0 bytes) is always valid and
  *     selects the schedule that needs none. A caller that passes at least dlspm_workspace_bytes()
- *     bytes lets SpMM and the fused op use the flat schedule where the library's size rule selects it
- *     (large matrices with long rows: every wave then owns a fixed run of nonzeros, however they are
- *     spread over the rows, and a second kernel adds the partial rows kept in the workspace, in a
- *     fixed order). A non-NULL workspace smaller than that is refused with DLSPM_E_WORKSPACE. The
+ *     bytes lets SpMM and the fused op use the flat schedule where the library's size rule allows it
+ *     (from about half a million nonzeros, 64 per row on average, dense width above 64: every wave then
+ *     owns a fixed run of nonzeros, however they are spread over the rows, and a second kernel adds the
+ *     partial rows kept in the workspace, in a fixed order). That schedule is the faster one when row
+ *     lengths are uneven and the slower one when they are even, so pass the workspace for matrices
+ *     whose longest row is several times the mean (dlspm_csr_row_stats) and NULL otherwise. A non-NULL workspace smaller than that is refused with DLSPM_E_WORKSPACE. The
  *     contents need no initialisation and mean nothing afterwards; two calls that share a workspace
  *     must not overlap in time.
  * Calls on different streams may run concurrently from different host threads (each with its own

@@ -73,7 +73,11 @@ def test_flat_schedule_rule_and_workspace_size(dl, monkeypatch):
     assert dl.workspace_bytes(dl.OP_SDDMM, M, K, 128, nnz) == 0               # nothing to combine
     assert dl.describe_launch(dl.OP_SDDMM, M, K, 32, nnz)["flat_chunk"] == 512  # but the schedule is used, any width
     assert dl.workspace_bytes(dl.OP_SPMM, M, K, 64, nnz) == 0                 # narrow dense rows: row-block schedule
-    assert dl.workspace_bytes(dl.OP_SPMM, M, K, 128, (1 << 21) - 1) == 0      # too few nonzeros
+    mid = 838860                                                              # below 2 M nonzeros: 256 per wave
+    shm = dl.describe_launch(dl.OP_SPMM, 4096, 4096, 256, mid)
+    assert shm["flat_chunk"] == 256 and dl.workspace_bytes(dl.OP_SPMM, 4096, 4096, 256, mid) == -(-mid // 256) * 2 * 256 * 4
+    assert dl.describe_launch(dl.OP_SDDMM, 4096, 4096, 128, mid)["flat_chunk"] == 0  # SDDMM: only from 2 M nonzeros on
+    assert dl.workspace_bytes(dl.OP_SPMM, M, K, 128, (1 << 19) - 1) == 0      # too few nonzeros
     assert dl.workspace_bytes(dl.OP_SPMM, 65536, K, 128, nnz) == 0            # rows too short (51 on average)
     big = 26843545                                                            # the chunk grows to keep ~32768 units
     shb = dl.describe_launch(dl.OP_SPMM, 32768, 8192, 128, big)
