@@ -66,7 +66,6 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
     constexpr int NP = R == 1 ? 1 : 2;
     using VecT = Vec<VEC>;
 
-    __shared__ int s_off[R + 1];
     __shared__ float s_part[W][NP][TW];
 
     const int lane = threadIdx.x & 63;
@@ -78,8 +77,19 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
     const int r0 = rb * R;
     const int nr = min(R, M - r0);
 
-    if ((int)threadIdx.x <= nr) s_off[threadIdx.x] = row_offsets[r0 + threadIdx.x];
-    __syncthreads();
+    // the block's R + 1 row offsets without LDS or a barrier (see spmm_kernel)
+    int off_lo = 0, off_hi = 0, off_win = 0;
+    if constexpr (R == 1) {
+        off_lo = row_offsets[r0];
+        off_hi = row_offsets[r0 + 1];
+    } else {
+        static_assert(R + 1 <= kWave, "one offset per lane");
+        off_win = row_offsets[r0 + min(lane, nr)];
+    }
+    auto s_off = [&](int i) -> int {
+        if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
+        else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
+    };
 
     int colv[V2];
     bool act[V2];
@@ -90,19 +100,19 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
         colv[v] = act[v] ? min(col, D - VEC) : 0;  // a lane that would run past D repeats its neighbour's columns
     }
 
-    const int T0 = s_off[0];
-    const int T = s_off[nr] - T0;
+    const int T0 = s_off(0);
+    const int T = s_off(nr) - T0;
     const int per = split_per_wave(T, W);
     const int a = __builtin_amdgcn_readfirstlane(T0 + min(T, w * per));
     const int b = __builtin_amdgcn_readfirstlane(T0 + min(T, (w + 1) * per));
 
     if (a < b) {
         int r = 0;
-        while (s_off[r + 1] <= a) ++r;
+        while (s_off(r + 1) <= a) ++r;
         int pos = a;
         while (pos < b) {
-            const int rs = s_off[r];
-            const int re = s_off[r + 1];
+            const int rs = s_off(r);
+            const int re = s_off(r + 1);
             const int q = __builtin_amdgcn_readfirstlane(min(re, b));
             const int p = __builtin_amdgcn_readfirstlane(pos);
             const float* q_row = Q + (size_t)(r0 + r) * D;
@@ -125,15 +135,15 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
             }
             pos = q;
             ++r;
-            while (r < nr && s_off[r + 1] <= pos) ++r;
+            while (r < nr && s_off(r + 1) <= pos) ++r;
         }
     }
     __syncthreads();
 
     if (slot == 0) {
         for (int r = w; r < nr; r += W) {
-            const int rs = s_off[r];
-            const int re = s_off[r + 1];
+            const int rs = s_off(r);
+            const int re = s_off(r + 1);
             float* orow = O + (size_t)(r0 + r) * D;
             if (rs == re) {
 #pragma unroll

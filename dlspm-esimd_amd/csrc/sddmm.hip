@@ -54,35 +54,44 @@ __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* 
                                                        const float* __restrict__ lhs, const float* __restrict__ rhs,
                                                        float* __restrict__ out)
 {
-    __shared__ int s_off[R + 1];
-
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r0 = blockIdx.x * R;
     const int nr = min(R, M - r0);
 
-    if ((int)threadIdx.x <= nr) s_off[threadIdx.x] = row_offsets[r0 + threadIdx.x];
-    __syncthreads();
+    // the block's R + 1 row offsets without LDS or a barrier (see spmm_kernel): this kernel then has neither
+    int off_lo = 0, off_hi = 0, off_win = 0;
+    if constexpr (R == 1) {
+        off_lo = row_offsets[r0];
+        off_hi = row_offsets[r0 + 1];
+    } else {
+        static_assert(R + 1 <= kWave, "one offset per lane");
+        off_win = row_offsets[r0 + min(lane, nr)];
+    }
+    auto s_off = [&](int i) -> int {
+        if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
+        else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
+    };
 
-    const int T0 = s_off[0];
-    const int T = s_off[nr] - T0;
+    const int T0 = s_off(0);
+    const int T = s_off(nr) - T0;
     const int per = split_per_wave(T, W);
     const int a = __builtin_amdgcn_readfirstlane(T0 + min(T, w * per));
     const int b = __builtin_amdgcn_readfirstlane(T0 + min(T, (w + 1) * per));
     if (a >= b) return;
 
     int r = 0;
-    while (s_off[r + 1] <= a) ++r;
+    while (s_off(r + 1) <= a) ++r;
     int pos = a;
     while (pos < b) {
-        const int q = __builtin_amdgcn_readfirstlane(min(s_off[r + 1], b));
+        const int q = __builtin_amdgcn_readfirstlane(min(s_off(r + 1), b));
         const int p = __builtin_amdgcn_readfirstlane(pos);
         const float* lhs_row = lhs + (size_t)(r0 + r) * D;
 
         sddmm_segment<VEC, G1, DS, MASKED>(p, q, D, col_indices, lhs_row, rhs, out, lane);
         pos = q;
         ++r;
-        while (r < nr && s_off[r + 1] <= pos) ++r;
+        while (r < nr && s_off(r + 1) <= pos) ++r;
     }
 }
 

@@ -56,7 +56,6 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
     constexpr int TW = G * VEC * V;  // columns of C covered by one wave
     using VecT = Vec<VEC>;
 
-    __shared__ int s_off[R + 1];
     constexpr int NP = R == 1 ? 1 : 2;  // with one row per workgroup a wave never ends a second segment
     __shared__ float s_part[W][NP][TW];
 
@@ -69,8 +68,20 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
     const int r0 = rb * R;
     const int nr = min(R, M - r0);
 
-    if ((int)threadIdx.x <= nr) s_off[threadIdx.x] = row_offsets[r0 + threadIdx.x];
-    __syncthreads();
+    // The block's R + 1 row offsets, without LDS or a barrier: with R == 1 they are the same two words for every
+    // lane (scalar loads); otherwise lane i of every wave holds offset i and v_readlane picks one.
+    int off_lo = 0, off_hi = 0, off_win = 0;
+    if constexpr (R == 1) {
+        off_lo = row_offsets[r0];
+        off_hi = row_offsets[r0 + 1];
+    } else {
+        static_assert(R + 1 <= kWave, "one offset per lane");
+        off_win = row_offsets[r0 + min(lane, nr)];
+    }
+    auto s_off = [&](int i) -> int {
+        if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
+        else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
+    };
 
     int colv[V];  // first of this lane's VEC columns for access v; clamped to a valid column when outside
     bool act[V];
@@ -83,19 +94,19 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
         colv[v] = act[v] ? min(col, N - VEC) : 0;
     }
 
-    const int T0 = s_off[0];
-    const int T = s_off[nr] - T0;
+    const int T0 = s_off(0);
+    const int T = s_off(nr) - T0;
     const int per = split_per_wave(T, W);
     const int a = __builtin_amdgcn_readfirstlane(T0 + min(T, w * per));
     const int b = __builtin_amdgcn_readfirstlane(T0 + min(T, (w + 1) * per));
 
     if (a < b) {
         int r = 0;
-        while (s_off[r + 1] <= a) ++r;  // first row owning nonzero `a`; exists because a < s_off[nr]
+        while (s_off(r + 1) <= a) ++r;  // first row owning nonzero `a`; exists because a < s_off(nr)
         int pos = a;
         while (pos < b) {
-            const int rs = s_off[r];
-            const int re = s_off[r + 1];
+            const int rs = s_off(r);
+            const int re = s_off(r + 1);
             const int q = __builtin_amdgcn_readfirstlane(min(re, b));
             const int p = __builtin_amdgcn_readfirstlane(pos);
 
@@ -117,7 +128,7 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
             }
             pos = q;
             ++r;
-            while (r < nr && s_off[r + 1] <= pos) ++r;  // skip rows without nonzeros
+            while (r < nr && s_off(r + 1) <= pos) ++r;  // skip rows without nonzeros
         }
     }
     __syncthreads();
@@ -125,8 +136,8 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
     // rows shared by several waves: add the partial sums in wave order; empty rows: write zeros
     if (slot == 0) {
         for (int r = w; r < nr; r += W) {
-            const int rs = s_off[r];
-            const int re = s_off[r + 1];
+            const int rs = s_off(r);
+            const int re = s_off(r + 1);
             float* crow = C + (size_t)(r0 + r) * N;
             if (rs == re) {
 #pragma unroll
