@@ -63,7 +63,7 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane % G;
     const int slot = lane / G;
-    const int rb = blockIdx.x / col_tiles;
+    const int rb = col_tiles == 1 ? (int)blockIdx.x : (int)(blockIdx.x / col_tiles);  // no division in the usual case
     const int ct = blockIdx.x - rb * col_tiles;
     const int r0 = rb * R;
     const int nr = min(R, M - r0);
