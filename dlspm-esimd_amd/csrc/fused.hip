@@ -140,6 +140,28 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
     }
     __syncthreads();
 
+    if constexpr (R == 1) {
+        // one row per workgroup: wave x had nonzeros iff x * per < T, and wave 0 adds them up (no division, the
+        // partial sums of all waves are requested from LDS together)
+        if (w == 0 && slot == 0) {
+            float* orow = O + (size_t)r0 * D;
+            if (T == 0) {
+#pragma unroll
+                for (int v = 0; v < V2; ++v)
+                    if (act[v]) VecT::zero().gstore(orow + colv[v]);
+            } else if (T > per) {  // T <= per: wave 0 held the whole row and has stored it
+#pragma unroll
+                for (int v = 0; v < V2; ++v) {
+                    VecT sum = VecT::zero();
+#pragma unroll
+                    for (int x = 0; x < W; ++x)
+                        if (x * per < T) sum.add(VecT::load(&s_part[x][0][(v * G + g) * VEC]));
+                    if (act[v]) sum.gstore(orow + colv[v]);
+                }
+            }
+        }
+        return;
+    }
     if (slot == 0) {
         for (int r = w; r < nr; r += W) {
             const int rs = s_off(r);
