@@ -126,6 +126,12 @@ template <int G> __device__ __forceinline__ float group_sum(float x)
     return x;
 }
 
+// Asks for kernel arguments now: the compiler otherwise fetches a pointer from the argument segment only where it
+// is first used, and that scalar load then sits in the middle of the kernel's chain of dependent memory accesses
+// (row offsets -> column indices -> dense rows). Fetched together at entry, they cost one round trip in all.
+template <typename P> __device__ __forceinline__ void fetch_arg_now(P p) { asm volatile("" : : "s"(p)); }
+template <typename... P> __device__ __forceinline__ void fetch_args_now(P... p) { (fetch_arg_now(p), ...); }
+
 // ---- work split -----------------------------------------------------------------------------------
 // A workgroup of W waves owns a block of consecutive rows holding T nonzeros in all; wave w takes the
 // contiguous nonzero range [w*per, (w+1)*per) of them (clipped to T) regardless of row boundaries.

@@ -86,6 +86,7 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
         static_assert(R + 1 <= kWave, "one offset per lane");
         off_win = row_offsets[r0 + min(lane, nr)];
     }
+    fetch_args_now(col_indices, Q, Kmat, Vmat, O);  // with the offsets' request: one round trip for both
     auto s_off = [&](int i) -> int {
         if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
         else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
@@ -278,6 +279,7 @@ __global__ __launch_bounds__(kFlatWaves * 64) void fused_flat_kernel(int M, int 
                                                                       const float* __restrict__ Vmat, float* __restrict__ O,
                                                                       float* __restrict__ partial)
 {
+    fetch_args_now(row_offsets, col_indices, Q, Kmat, Vmat, O, partial);
     constexpr int TW = G * VEC * V2;
     using VecT = Vec<VEC>;
     const int lane = threadIdx.x & 63;

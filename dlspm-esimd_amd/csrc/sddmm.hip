@@ -68,6 +68,7 @@ __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* 
         static_assert(R + 1 <= kWave, "one offset per lane");
         off_win = row_offsets[r0 + min(lane, nr)];
     }
+    fetch_args_now(col_indices, lhs, rhs, out);  // with the offsets' request: one round trip for both
     auto s_off = [&](int i) -> int {
         if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
         else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
@@ -179,6 +180,7 @@ __global__ __launch_bounds__(kFlatWaves * 64) void sddmm_flat_kernel(int M, int 
                                                                       const float* __restrict__ lhs,
                                                                       const float* __restrict__ rhs, float* __restrict__ out)
 {
+    fetch_args_now(row_offsets, col_indices, lhs, rhs, out);
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const long long a64 = ((long long)blockIdx.x * kFlatWaves + w) * chunk;

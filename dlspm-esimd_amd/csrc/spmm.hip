@@ -78,6 +78,7 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
         static_assert(R + 1 <= kWave, "one offset per lane");
         off_win = row_offsets[r0 + min(lane, nr)];
     }
+    fetch_args_now(col_indices, values, B, C);  // after the offsets were requested: both arrive in one round trip
     auto s_off = [&](int i) -> int {
         if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
         else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
@@ -266,6 +267,7 @@ __global__ __launch_bounds__(kFlatWaves * 64) void spmm_flat_kernel(int M, int N
                                                                      const float* __restrict__ B, float* __restrict__ C,
                                                                      float* __restrict__ partial)
 {
+    fetch_args_now(row_offsets, col_indices, values, B, C, partial);
     constexpr int TW = G * VEC * V;
     using VecT = Vec<VEC>;
     const int lane = threadIdx.x & 63;
