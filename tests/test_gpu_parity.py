@@ -4,6 +4,9 @@ Bars (BASELINE.json): the CSR structure must come back bit-identical (the librar
 within 1e-4 relative Frobenius error of the reference's CPU loops. Sizes here are ones the oracle finishes
 in seconds; the five benchmark configurations are checked at full size.
 """
+import glob
+import os
+
 import numpy as np
 import pytest
 
@@ -196,6 +199,31 @@ def test_fused_matches_oracle(torch_cuda, dl, oracle, M, K, D, kind, density, sc
     check_csr_untouched(ro_d, ci_d, ro, ci)
     empty = np.diff(ro) == 0
     assert (got[empty] == 0).all()
+
+
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "fused_ref_M*_K*_N*.npz")))
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p) for p in GOLDEN])
+def test_kernels_against_the_references_own_outputs(torch_cuda, dl, oracle, path):
+    """Directly against what the REFERENCE's functions (compiled from its FUSED/fused.cpp) returned for the fixture's
+    inputs: Sddmm, Spmm applied to those scores (= the fused gold, no scale), the fp32 SpMM emulation and the fp32
+    fused emulation. No oracle in between."""
+    torch = torch_cuda
+    z = np.load(path)
+    ro, ci = z["row_offsets"], z["col_indices"]
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    K = z["b"].shape[0]
+    got = dl.sddmm(ro_d, ci_d, dev(torch, z["c"]), dev(torch, z["b"])).cpu().numpy()
+    assert oracle.rel_frobenius(got, z["sddmm"]) <= TOL
+    got = dl.spmm(ro_d, ci_d, dev(torch, z["values"]), dev(torch, z["d"]), K=K).cpu().numpy()
+    assert oracle.rel_frobenius(got, z["spmm_f32"]) <= TOL
+    got = dl.spmm(ro_d, ci_d, dev(torch, z["sddmm"]), dev(torch, z["d"]), K=K).cpu().numpy()
+    assert oracle.rel_frobenius(got, z["spmm_f64acc"]) <= TOL
+    got = dl.fused(ro_d, ci_d, dev(torch, z["c"]), dev(torch, z["b"]), dev(torch, z["d"]), 1.0).cpu().numpy()
+    assert oracle.rel_frobenius(got, z["spmm_f64acc"]) <= TOL   # the reference's gold: Sddmm then Spmm
+    assert oracle.rel_frobenius(got, z["fused_emul"]) <= TOL    # and its own fp32 emulation of the fused kernel
+    check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
 def test_fused_equals_unfused_on_gpu(torch_cuda, dl, oracle):
