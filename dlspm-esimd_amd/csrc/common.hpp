@@ -141,6 +141,64 @@ __host__ __device__ __forceinline__ int split_per_wave(int T, int W)
     return per < 1 ? 1 : per;
 }
 
+// Row-aligned variant of that split, used when it is nearly as even: with R = k*W rows per workgroup wave w takes the
+// k rows w*k .. w*k+k-1 whole; with W = m*R waves per row the m waves of a row take equal parts of it. A wave then
+// never works on the tail of one row and the head of the next (two dependent chains of memory accesses in sequence),
+// whole rows are stored without a partial sum, and a matrix of even rows loses nothing in balance (measured on
+// 2048x2048, 102-103 nonzeros per row, D = 128: 6.2 -> 5.7 us). It is taken when no wave would get more than 5/4 of
+// the even share `per`; every wave of the workgroup evaluates the same test on the same offsets. `off(i)` returns
+// row offset i of the block (i <= nr); the offsets of rows past nr count as off(nr).
+template <int W, int R, typename Off> __host__ __device__ __forceinline__ bool split_is_row_aligned(Off&& off, int nr, int per)
+{
+    if constexpr (R == 1) {
+        return false;  // one row per workgroup: the even split is the aligned one
+    } else {
+        const int cap = per + (per >> 2);
+        int worst = 0;
+        if constexpr (R % W == 0) {
+            constexpr int k = R / W;
+            for (int x = 0; x < W; ++x) {
+                const int lo = x * k < nr ? x * k : nr, hi = (x + 1) * k < nr ? (x + 1) * k : nr;
+                const int load = off(hi) - off(lo);
+                worst = load > worst ? load : worst;
+            }
+        } else {
+            static_assert(W % R == 0, "rows per workgroup and waves per workgroup divide one another");
+            constexpr int m = W / R;
+            for (int r = 0; r < nr; ++r) {
+                const int load = (off(r + 1) - off(r) + m - 1) / m;
+                worst = load > worst ? load : worst;
+            }
+        }
+        return worst <= cap;
+    }
+}
+// nonzero range [a, b) of wave w (absolute positions), for either split
+template <int W, int R, typename Off>
+__host__ __device__ __forceinline__ void wave_range(bool aligned, Off&& off, int nr, int w, int T0, int T, int per, int& a,
+                                                    int& b)
+{
+    if (!aligned) {
+        a = T0 + (T < w * per ? T : w * per);
+        b = T0 + (T < (w + 1) * per ? T : (w + 1) * per);
+    } else if constexpr (R % W == 0) {
+        constexpr int k = R / W;
+        a = off(w * k < nr ? w * k : nr);
+        b = off((w + 1) * k < nr ? (w + 1) * k : nr);
+    } else {
+        constexpr int m = W / R;
+        const int r = w / m, j = w % m;
+        if (r >= nr) {
+            a = b = T0 + T;
+        } else {
+            const int rs = off(r), len = off(r + 1) - rs;
+            const int part = (len + m - 1) / m;
+            a = rs + (len < j * part ? len : j * part);
+            b = rs + (len < (j + 1) * part ? len : (j + 1) * part);
+        }
+    }
+}
+
 // ---- flat schedule: every wave owns `chunk` consecutive nonzeros of the whole matrix ------------------------
 // Largest row r with row_offsets[r] <= pos, for 0 <= pos < row_offsets[M] (so the row is not empty and holds
 // nonzero `pos`). A 64-ary search by the whole wave: each round reads 64 evenly spaced offsets with one load and

@@ -104,8 +104,11 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
     const int T0 = s_off(0);
     const int T = s_off(nr) - T0;
     const int per = split_per_wave(T, W);
-    const int a = __builtin_amdgcn_readfirstlane(T0 + min(T, w * per));
-    const int b = __builtin_amdgcn_readfirstlane(T0 + min(T, (w + 1) * per));
+    const bool aligned = split_is_row_aligned<W, R>(s_off, nr, per);
+    int a_, b_;
+    wave_range<W, R>(aligned, s_off, nr, w, T0, T, per, a_, b_);
+    const int a = __builtin_amdgcn_readfirstlane(a_);
+    const int b = __builtin_amdgcn_readfirstlane(b_);
 
     if (a < b) {
         int r = 0;
@@ -138,6 +141,41 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
             ++r;
             while (r < nr && s_off(r + 1) <= pos) ++r;
         }
+    }
+    if (aligned) {  // R > 1 only, and the same for every wave of the workgroup
+        if constexpr (R % W == 0) {
+            // every wave stored its rows whole: nothing to combine, no barrier; rows without nonzeros are left
+            if (slot == 0) {
+                for (int r = w; r < nr; r += W) {
+                    if (s_off(r) != s_off(r + 1)) continue;
+                    float* orow = O + (size_t)(r0 + r) * D;
+#pragma unroll
+                    for (int v = 0; v < V2; ++v)
+                        if (act[v]) VecT::zero().gstore(orow + colv[v]);
+                }
+            }
+        } else {
+            // the m = W/R waves of a row hold its parts in order, each in its first partial slot
+            constexpr int m = W / R;
+            __syncthreads();
+            if (slot == 0) {
+                for (int r = w; r < nr; r += W) {
+                    const int len = s_off(r + 1) - s_off(r);
+                    const int part = (len + m - 1) / m;
+                    float* orow = O + (size_t)(r0 + r) * D;
+                    if (len > 0 && len <= part) continue;  // one wave held the whole row and stored it
+#pragma unroll
+                    for (int v = 0; v < V2; ++v) {
+                        VecT sum = VecT::zero();
+#pragma unroll
+                        for (int j = 0; j < m; ++j)
+                            if (j * part < len) sum.add(VecT::load(&s_part[r * m + j][0][(v * G + g) * VEC]));
+                        if (act[v]) sum.gstore(orow + colv[v]);
+                    }
+                }
+            }
+        }
+        return;
     }
     __syncthreads();
 

@@ -77,8 +77,11 @@ __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* 
     const int T0 = s_off(0);
     const int T = s_off(nr) - T0;
     const int per = split_per_wave(T, W);
-    const int a = __builtin_amdgcn_readfirstlane(T0 + min(T, w * per));
-    const int b = __builtin_amdgcn_readfirstlane(T0 + min(T, (w + 1) * per));
+    const bool aligned = split_is_row_aligned<W, R>(s_off, nr, per);
+    int a_, b_;
+    wave_range<W, R>(aligned, s_off, nr, w, T0, T, per, a_, b_);
+    const int a = __builtin_amdgcn_readfirstlane(a_);
+    const int b = __builtin_amdgcn_readfirstlane(b_);
     if (a >= b) return;
 
     int r = 0;

@@ -19,6 +19,40 @@ int split_per_wave(int T, int W)
     return per < 1 ? 1 : per;
 }
 
+// the row-aligned split of the kernels (common.hpp: split_is_row_aligned, wave_range), with W and R at run time
+bool split_is_row_aligned(const int* off, int nr, int per, int W, int R)
+{
+    if (R == 1) return false;
+    const int cap = per + (per >> 2);
+    int worst = 0;
+    if (R % W == 0) {
+        const int k = R / W;
+        for (int x = 0; x < W; ++x) worst = std::max(worst, off[std::min((x + 1) * k, nr)] - off[std::min(x * k, nr)]);
+    } else {
+        const int m = W / R;
+        for (int r = 0; r < nr; ++r) worst = std::max(worst, (off[r + 1] - off[r] + m - 1) / m);
+    }
+    return worst <= cap;
+}
+
+void wave_range(bool aligned, const int* off, int nr, int w, int T0, int T, int per, int W, int R, int& a, int& b)
+{
+    if (!aligned) {
+        a = T0 + std::min(T, w * per);
+        b = T0 + std::min(T, (w + 1) * per);
+    } else if (R % W == 0) {
+        const int k = R / W;
+        a = off[std::min(w * k, nr)];
+        b = off[std::min((w + 1) * k, nr)];
+    } else {
+        const int m = W / R, r = w / m, j = w % m;
+        if (r >= nr) { a = b = T0 + T; return; }
+        const int rs = off[r], len = off[r + 1] - rs, piece = (len + m - 1) / m;
+        a = rs + std::min(len, j * piece);
+        b = rs + std::min(len, (j + 1) * piece);
+    }
+}
+
 // sum of the S lane groups' accumulators in the order the kernel's cross-lane steps add them:
 // neighbours first (xor G), then pairs of pairs (xor 2G), ... : a balanced tree over the slots
 float slots_tree(const float* s, int S)
@@ -42,9 +76,11 @@ int model_rows(int M, int N, const int* ro, const int* ci, const float* va, cons
         const int* off = ro + r0;
         const int T0 = off[0], T = off[nr] - T0;
         const int per = split_per_wave(T, W);
+        const bool aligned = split_is_row_aligned(off, nr, per, W, R);
         part.assign((size_t)W * 2 * N, NAN);
         for (int w = 0; w < W; ++w) {
-            const int a = T0 + std::min(T, w * per), b = T0 + std::min(T, (w + 1) * per);
+            int a, b;
+            wave_range(aligned, off, nr, w, T0, T, per, W, R, a, b);
             if (a >= b) continue;
             int r = 0;
             while (off[r + 1] <= a) ++r;
@@ -82,6 +118,23 @@ int model_rows(int M, int N, const int* ro, const int* ci, const float* va, cons
             int* wrow = writes + (size_t)(r0 + r) * N;
             if (rs == re) {
                 for (int j = 0; j < N; ++j) { crow[j] = 0.0f; wrow[j]++; }
+                continue;
+            }
+            if (aligned && R % W == 0) continue;  // every wave stored its rows whole
+            if (aligned) {                        // the m = W/R waves of the row hold its parts in order
+                const int m = W / R, len = re - rs, piece = (len + m - 1) / m;
+                if (len <= piece) continue;
+                for (int j = 0; j < N; ++j) {
+                    float sum = 0.0f;
+                    for (int x = 0; x < m; ++x) {
+                        if (x * piece >= len) continue;
+                        const float pv = part[((size_t)(r * m + x) * 2) * N + j];
+                        if (std::isnan(pv) && !std::isnan(B[0])) return 1;
+                        sum = sum + pv;
+                    }
+                    crow[j] = sum;
+                    wrow[j]++;
+                }
                 continue;
             }
             const int wl = (rs - T0) / per, wh = (re - 1 - T0) / per;
