@@ -483,6 +483,37 @@ def test_concurrent_calls_from_two_threads_on_two_streams(torch_cuda, dl, oracle
         assert torch.equal(out, ref)
 
 
+def test_operands_beyond_2_31_elements(torch_cuda, dl):
+    """Dense operands of 2.3e9 floats (9.2 GB each): every element offset inside the kernels must be 64-bit. One
+    nonzero per row with value 1 makes SpMM a row gather, SDDMM a row-by-row dot product and the fused op a scaled row
+    gather, all checked on the device against torch."""
+    torch = torch_cuda
+    M, K, N = 70001, 64, 32768
+    assert M * N > 2**31
+    g = torch.Generator(device="cuda")
+    g.manual_seed(7)
+    ci_d = torch.randint(0, K, (M,), dtype=torch.int32, device="cuda", generator=g)
+    ro_d = torch.arange(M + 1, dtype=torch.int32, device="cuda")
+    ones = torch.ones(M, dtype=torch.float32, device="cuda")
+    B = torch.randn(K, N, device="cuda", generator=g)
+    C = torch.empty(M, N, device="cuda")
+    dl.spmm(ro_d, ci_d, ones, B, K=K, out=C)
+    for lo in range(0, M, 10000):  # compare in slices: the gathered reference would be another 9.2 GB
+        hi = min(M, lo + 10000)
+        assert torch.equal(C[lo:hi], B[ci_d[lo:hi].long()]), f"rows {lo}..{hi}"
+    # SDDMM: lhs = C (M x N, 9.2 GB): out[i] = <C[i], B[col_i]> = |B[col_i]|^2
+    out = dl.sddmm(ro_d, ci_d, C, B)
+    want = (B.double() ** 2).sum(1)[ci_d.long()]
+    assert torch.allclose(out.double(), want, rtol=1e-4)
+    # fused: O[i] = (<Q[i], B[col_i]> * scale) * V[col_i], Q = C so the score is |B[col_i]|^2 again; O reuses no input
+    O = torch.empty(M, N, device="cuda")
+    dl.fused(ro_d, ci_d, C, B, B, 1.0 / N, out=O)
+    for lo in range(0, M, 10000):
+        hi = min(M, lo + 10000)
+        ref = (want[lo:hi] / N).float()[:, None] * B[ci_d[lo:hi].long()]
+        assert torch.allclose(O[lo:hi], ref, rtol=1e-3, atol=1e-5), f"rows {lo}..{hi}"
+
+
 def test_csr_row_stats(torch_cuda, dl):
     torch = torch_cuda
     rng = np.random.default_rng(3)
