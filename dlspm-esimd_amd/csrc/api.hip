@@ -81,12 +81,12 @@ static FlatPlan sddmm_flat_plan(int M, int nnz, int D)
     return flat_plan(M, nnz, D, kWave);
 }
 
-void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w, int slots, int& W, int& R)
+void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bool rows_even, int& W, int& R)
 {
     static const int kPairs[][2] = {{4, 16}, {4, 8}, {4, 4}, {4, 2}, {4, 1}, {8, 4}, {8, 2}, {8, 1}, {16, 1}};
     if (split_override(W, R)) {
         for (const auto& pr : kPairs)
-            if (pr[0] == W && pr[1] == R && W <= max_w) return;
+            if (pr[0] == W && pr[1] == R && W <= rule.max_w) return;
     }
     // Measured on MI355X over the benchmark configurations and the 12 x {32,128} x {0.3,0.2,0.1} sweep grid:
     // four-wave workgroups win whenever the matrix has enough rows to fill the device (16-wave workgroups were up
@@ -95,21 +95,31 @@ void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w
     const double avg = M > 0 ? (double)nnz / M : 0.0;
     const long long work_rows = (long long)M * col_tiles;
     W = work_rows >= 512 ? 4 : work_rows >= 256 ? 8 : 16;
-    if (avg >= 1536.0) W = 16;  // very long rows: more waves per row beat the barrier cost (measured, ~8 %)
+    // very long rows in a tall matrix: sixteen waves per row gain 5-8 % in SpMM (24576 and 32768 rows of ~2000
+    // nonzeros); with 8192 rows they lose as much, and the fused kernel loses 25-50 % with them at any height
+    if (rule.w16_long_rows && avg >= 1536.0 && work_rows >= 16384) W = 16;
     // few rows, each long (pruned ResNet-50 layers at small batch): four waves per row leave the device with a
     // couple of waves per SIMD, each walking hundreds of steps in sequence (measured 15-25 % slower); a step
     // takes `slots` nonzeros of the row at once
-    const double steps = avg / (slots > 0 ? slots : 1);
+    const double steps = avg / (rule.slots > 0 ? rule.slots : 1);
     if (work_rows < 1024 && steps >= 768.0) W = 16;
     else if (work_rows < 1024 && steps >= 384.0 && W < 8) W = 8;
-    if (W > max_w) W = max_w;
+    if (W > rule.max_w) W = rule.max_w;
     R = 1;
     if (W == 4) {
         for (int r = 2; r <= 16; r *= 2) {
             const long long blocks = (long long)((M + r - 1) / r) * col_tiles;
-            if (blocks < min_blocks || avg * r > 512.0) break;
+            if (blocks < rule.min_blocks || avg * r > 512.0) break;
             R = r;
         }
+        // Rows known to be even: four rows per four-wave workgroup, which the kernels then run as one whole row per
+        // wave (no partial sums, no barrier, one chain of accesses per row instead of four): 3-17 % faster than one
+        // row per workgroup from 4096 rows on, and 1.3-1.7x where the gathered operands exceed one L2 (8192 x 128
+        // floats twice in the fused op), because waves that start together then sweep the columns together. With
+        // uneven rows the same grouping is 5-20 % slower (four rows of work per workgroup make the tail of the
+        // launch coarser), hence only on the caller's word. Rows below 128 nonzeros keep the grouping of the size rule
+        // (4096 rows of ~100: four per workgroup measured 6 % slower than two).
+        if (rows_even && R < 4 && avg >= 128.0 && (long long)((M + 3) / 4) * col_tiles >= 1024) R = 4;
     }
 }
 
@@ -177,9 +187,10 @@ int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int
     if (nnz > 0 && (!col_indices || !values || !B)) return DLSPM_E_INVALID_ARG;
     const bool vec4 = N >= 4;  // dwordx4 accesses need only dword alignment
     const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C};
-    const SpmmShape shape = spmm_choose(M, N, nnz, vec4);
+    const bool even = workspace == DLSPM_ROWS_EVEN;  // a constant that says something about the rows, not memory
+    const SpmmShape shape = spmm_choose(M, N, nnz, vec4, even);
     hipError_t e;
-    if (workspace != nullptr && workspace_bytes > 0) {
+    if (!even && workspace != nullptr && workspace_bytes > 0) {
         const FlatPlan plan = flat_plan(M, nnz, N, shape.G);
         if (workspace_bytes < plan.bytes) return DLSPM_E_WORKSPACE;
         if (plan.chunk > 0)
@@ -195,7 +206,6 @@ int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int
 int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* lhs,
                   const float* rhs, float* out_values, void* workspace, size_t workspace_bytes, void* stream)
 {
-    (void)workspace;
     (void)workspace_bytes;
     if (M < 0 || K < 0 || D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
@@ -209,7 +219,7 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
         return e0 == hipSuccess ? DLSPM_OK : fail_hip(e0);
     }
     const bool vec4 = D >= 4;  // dwordx4 accesses need only dword alignment
-    const SddmmShape shape = sddmm_choose(M, D, nnz, vec4);
+    const SddmmShape shape = sddmm_choose(M, D, nnz, vec4, workspace == DLSPM_ROWS_EVEN);
     const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values};
     // the flat schedule needs no workspace here (nothing to combine), so the size rule alone decides; it has no
     // width condition for SDDMM (measured for D = 32 ... 256: equal on uniform rows, 15-33 % faster on skewed ones)
@@ -229,10 +239,11 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz, const int* row_offsets, c
     if (!row_offsets || !O) return DLSPM_E_INVALID_ARG;
     if (nnz > 0 && (!col_indices || !Q || !Kmat || !V)) return DLSPM_E_INVALID_ARG;
     const bool vec4 = D >= 4;
-    const FusedShape shape = fused_choose(M, D, nnz, vec4);
+    const bool even = workspace == DLSPM_ROWS_EVEN;
+    const FusedShape shape = fused_choose(M, D, nnz, vec4, even);
     const FusedArgs args{M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O};
     hipError_t e;
-    if (workspace != nullptr && workspace_bytes > 0) {
+    if (!even && workspace != nullptr && workspace_bytes > 0) {
         const FlatPlan plan = flat_plan(M, nnz, D, shape.G);
         if (workspace_bytes < plan.bytes) return DLSPM_E_WORKSPACE;
         if (plan.chunk > 0)
@@ -315,26 +326,27 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
     return DLSPM_OK;
 }
 
-int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape)
+int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int rows_even, int* shape)
 {
     (void)K;
+    const bool even = rows_even != 0;
     if (!shape || M < 0 || N_or_D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     const int n = N_or_D;
     const bool vec4 = n >= 4;
     for (int i = 0; i < 10; ++i) shape[i] = 0;
     if (op == DLSPM_OP_SPMM) {
-        const SpmmShape s = spmm_choose(M, n, nnz, vec4);
+        const SpmmShape s = spmm_choose(M, n, nnz, vec4, even);
         const int tw = s.G * s.vec * s.V;
         shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[5] = s.W; shape[6] = s.R; shape[7] = (n + tw - 1) / tw;
         const FlatPlan fp = flat_plan(M, nnz, n, s.G);
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_SDDMM) {
-        const SddmmShape s = sddmm_choose(M, n, nnz, vec4);
+        const SddmmShape s = sddmm_choose(M, n, nnz, vec4, even);
         shape[0] = s.vec; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R; shape[7] = 1;
         const FlatPlan fp = sddmm_flat_plan(M, nnz, n);
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_FUSED) {
-        const FusedShape s = fused_choose(M, n, nnz, vec4);
+        const FusedShape s = fused_choose(M, n, nnz, vec4, even);
         const int tw = s.G * s.vec * s.V;
         shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R;
         shape[7] = (n + tw - 1) / tw;
@@ -344,6 +356,11 @@ int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape)
         return DLSPM_E_INVALID_ARG;
     }
     return DLSPM_OK;
+}
+
+int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape)
+{
+    return dlspm_describe_launch_rows(op, M, K, N_or_D, nnz, 0, shape);
 }
 
 const char* dlspm_status_string(int status)

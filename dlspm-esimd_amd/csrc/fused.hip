@@ -271,7 +271,7 @@ static hipError_t launch_wr(const FusedArgs& x, int W, int R, hipStream_t stream
     return hipErrorInvalidValue;
 }
 
-FusedShape fused_choose(int M, int D, int nnz, bool vec4)
+FusedShape fused_choose(int M, int D, int nnz, bool vec4, bool rows_even)
 {
     FusedShape s{};
     s.vec = vec4 ? 4 : 1;
@@ -287,7 +287,7 @@ FusedShape fused_choose(int M, int D, int nnz, bool vec4)
         s.G1 = 4; s.DS = 1; s.G = 8; s.V = 1;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(M, (D + tw - 1) / tw, nnz, 512, tw >= 1024 ? 4 : 16, kWave / s.G, s.W, s.R);
+    choose_split(M, (D + tw - 1) / tw, nnz, SplitRule{512, tw >= 1024 ? 4 : 16, kWave / s.G, false}, rows_even, s.W, s.R);
     return s;
 }
 

@@ -54,23 +54,30 @@ FlatPlan flat_plan(int M, int nnz, int width, int G);
 hipError_t row_fixup_launch(int M, int N, int chunk, const int* row_offsets, const float* partial, float* out,
                             hipStream_t stream);
 
-SpmmShape spmm_choose(int M, int N, int nnz, bool vec4);
+SpmmShape spmm_choose(int M, int N, int nnz, bool vec4, bool rows_even = false);
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
 hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPlan& plan, float* partial,
                             hipStream_t stream);
 
-SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4);
+SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4, bool rows_even = false);
 hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t stream);
 hipError_t sddmm_flat_launch(const SddmmArgs& x, const SddmmShape& s, int chunk, hipStream_t stream);
 
-FusedShape fused_choose(int M, int D, int nnz, bool vec4);
+FusedShape fused_choose(int M, int D, int nnz, bool vec4, bool rows_even = false);
 hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream);
 hipError_t fused_flat_launch(const FusedArgs& x, const FusedShape& s, const FlatPlan& plan, float* partial,
                              hipStream_t stream);
 
 // Picks (W, R), W <= max_w: waves per workgroup from the number of rows, rows per workgroup as large as keeps
-// `min_blocks` workgroups in the grid. `slots` = nonzeros of a row a wave works on at once (64 / G).
-// Only the pairs the kernels are instantiated for are returned.
-void choose_split(int M, long long col_tiles, int nnz, int min_blocks, int max_w, int slots, int& W, int& R);
+// `min_blocks` workgroups in the grid. `slots` = nonzeros of a row a wave works on at once (64 / G); `w16_long_rows`:
+// the op gains from sixteen waves per row on tall matrices of very long rows. `rows_even`: the caller knows that no
+// row is much longer than the mean. Only the pairs the kernels are instantiated for are returned.
+struct SplitRule {
+    int min_blocks;
+    int max_w;
+    int slots;
+    bool w16_long_rows;
+};
+void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bool rows_even, int& W, int& R);
 
 }  // namespace dlspm

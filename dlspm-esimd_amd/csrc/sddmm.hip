@@ -136,7 +136,7 @@ static hipError_t launch_wr(const SddmmArgs& x, int W, int R, hipStream_t stream
     return hipErrorInvalidValue;
 }
 
-SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4)
+SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4, bool rows_even)
 {
     SddmmShape s{};
     s.vec = vec4 ? 4 : 1;
@@ -150,7 +150,7 @@ SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4)
         s.G1 = 4;
         s.DS = 1;
     }
-    choose_split(M, 1, nnz, 512, 16, kWave / s.G1, s.W, s.R);
+    choose_split(M, 1, nnz, SplitRule{512, 16, kWave / s.G1, true}, rows_even, s.W, s.R);
     return s;
 }
 

@@ -256,7 +256,7 @@ static hipError_t launch_wr(const SpmmArgs& x, int W, int R, hipStream_t stream)
 }
 
 // Chooses the lane layout from N and the (W, R) split from the mean row length.
-SpmmShape spmm_choose(int M, int N, int nnz, bool vec4)
+SpmmShape spmm_choose(int M, int N, int nnz, bool vec4, bool rows_even)
 {
     SpmmShape s{};
     s.vec = vec4 ? 4 : 1;
@@ -271,7 +271,7 @@ SpmmShape spmm_choose(int M, int N, int nnz, bool vec4)
         s.V = 1;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(M, (N + tw - 1) / tw, nnz, 2048, 16, kWave / s.G, s.W, s.R);
+    choose_split(M, (N + tw - 1) / tw, nnz, SplitRule{2048, 16, kWave / s.G, true}, rows_even, s.W, s.R);
     return s;
 }
 

@@ -21,6 +21,17 @@ E_NO_DEVICE = -5
 
 OP_SPMM, OP_SDDMM, OP_FUSED = 0, 1, 2
 
+
+class _RowsEven:
+    """The header's DLSPM_ROWS_EVEN: passed as `workspace`, it tells the library that no row is much longer than the
+    mean (at most 1.5 x nnz / M); it stands for no memory."""
+
+    def __repr__(self):
+        return "ROWS_EVEN"
+
+
+ROWS_EVEN = _RowsEven()
+
 EXPORTS = (
     "spmm_csr_f32",
     "sddmm_csr_f32",
@@ -28,6 +39,7 @@ EXPORTS = (
     "dlspm_workspace_bytes",
     "dlspm_csr_check",
     "dlspm_describe_launch",
+    "dlspm_describe_launch_rows",
     "dlspm_csr_row_stats",
     "dlspm_status_string",
     "dlspm_last_hip_error",
@@ -63,6 +75,8 @@ def lib() -> ctypes.CDLL:
         L.dlspm_csr_check.argtypes = [ci, ci, ci, vp, vp, vp]
         L.dlspm_csr_check.restype = ci
         L.dlspm_describe_launch.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci)]
+        L.dlspm_describe_launch_rows.argtypes = [ci, ci, ci, ci, ci, ci, ctypes.POINTER(ci)]
+        L.dlspm_describe_launch_rows.restype = ci
         L.dlspm_describe_launch.restype = ci
         L.dlspm_csr_row_stats.argtypes = [ci, vp, vp, ctypes.POINTER(ci), ctypes.POINTER(ci)]
         L.dlspm_csr_row_stats.restype = ci
@@ -104,7 +118,7 @@ def _stream():
 
 def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None):
     """C = A_csr @ B on the current stream. row_offsets/col_indices int32, values/B float32, all on the GPU.
-    `workspace`: optional GPU tensor of at least workspace_bytes(OP_SPMM, ...) bytes."""
+    `workspace`: optional GPU tensor of at least workspace_bytes(OP_SPMM, ...) bytes, or ROWS_EVEN."""
     import torch
 
     M = row_offsets.numel() - 1
@@ -122,8 +136,9 @@ def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None):
     return out
 
 
-def sddmm(row_offsets, col_indices, lhs, rhs, out=None):
-    """out[j] = <lhs[i], rhs[col[j]]> for each CSR slot j of row i, on the current stream."""
+def sddmm(row_offsets, col_indices, lhs, rhs, out=None, workspace=None):
+    """out[j] = <lhs[i], rhs[col[j]]> for each CSR slot j of row i, on the current stream.
+    `workspace`: None or ROWS_EVEN (SDDMM needs no memory)."""
     import torch
 
     M = row_offsets.numel() - 1
@@ -133,7 +148,8 @@ def sddmm(row_offsets, col_indices, lhs, rhs, out=None):
         out = torch.empty((nnz,), dtype=torch.float32, device=lhs.device)
     st = lib().sddmm_csr_f32(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
                              _ptr(col_indices, torch.int32, "col_indices"), _ptr(lhs, torch.float32, "lhs"),
-                             _ptr(rhs, torch.float32, "rhs"), _ptr(out, torch.float32, "out"), None, 0, _stream())
+                             _ptr(rhs, torch.float32, "rhs"), _ptr(out, torch.float32, "out"), *_workspace(workspace),
+                             _stream())
     if st != OK:
         raise DlspmError(st, "sddmm_csr_f32")
     return out
@@ -141,7 +157,7 @@ def sddmm(row_offsets, col_indices, lhs, rhs, out=None):
 
 def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None, workspace=None):
     """O = (S .* (Q Kmat^T) * scale) V on the current stream; the scores are never stored.
-    `workspace`: optional GPU tensor of at least workspace_bytes(OP_FUSED, ...) bytes."""
+    `workspace`: optional GPU tensor of at least workspace_bytes(OP_FUSED, ...) bytes, or ROWS_EVEN."""
     import torch
 
     M = row_offsets.numel() - 1
@@ -159,11 +175,11 @@ def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None, workspace=N
     return out
 
 
-def describe_launch(op: int, M: int, K: int, N: int, nnz: int) -> dict:
+def describe_launch(op: int, M: int, K: int, N: int, nnz: int, rows_even: bool = False) -> dict:
     """Launch shape the library uses for these sizes: {'vec','G','V','G1','DS','W','R','col_tiles','flat_chunk',
-    'flat_units'} (host only)."""
+    'flat_units'} (host only). rows_even: for a call that passes ROWS_EVEN."""
     out = (ctypes.c_int * 10)()
-    st = lib().dlspm_describe_launch(op, M, K, N, nnz, out)
+    st = lib().dlspm_describe_launch_rows(op, M, K, N, nnz, 1 if rows_even else 0, out)
     if st != OK:
         raise DlspmError(st, "dlspm_describe_launch")
     return dict(zip(("vec", "G", "V", "G1", "DS", "W", "R", "col_tiles", "flat_chunk", "flat_units"),
@@ -179,6 +195,8 @@ def _workspace(ws):
     """(pointer, bytes) of an optional workspace tensor (any dtype, contiguous, on the GPU)."""
     if ws is None:
         return None, 0
+    if ws is ROWS_EVEN:
+        return ctypes.c_void_p(1), 0
     if not ws.is_cuda or not ws.is_contiguous():
         raise ValueError("workspace must be a contiguous GPU tensor")
     return ctypes.c_void_p(ws.data_ptr()), ws.numel() * ws.element_size()

@@ -44,12 +44,12 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     if (dlspm_csr_check(M, K, nnz, ro_d.p, ci_d.p, nullptr) != DLSPM_OK) throw std::invalid_argument("malformed CSR structure");
     DLSPM_HIP_CHECK(hipMemset(O_d.p, 0xFF, (size_t)M * D * sizeof(float)));
 
-    const size_t ws_bytes = workspace_to_pass(opt, DLSPM_OP_FUSED, M, K, D, nnz, ro_d.p);  // 0 for small problems
-    DevBuf<char> ws(ws_bytes);
-    if (ws_bytes) std::printf("workspace: %zu bytes\n", ws_bytes);
+    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_FUSED, M, K, D, nnz, ro_d.p);  // 0 bytes for small problems
+    DevBuf<char> ws(wc.bytes);
+    if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
     const Timing t = time_launches(opt, [&]() {
-        return fused_sddmm_spmm_f32(M, K, D, nnz, ro_d.p, ci_d.p, Q_d.p, K_d.p, V_d.p, scale, O_d.p, ws_bytes ? ws.p : nullptr,
-                                    ws_bytes, nullptr);
+        return fused_sddmm_spmm_f32(M, K, D, nnz, ro_d.p, ci_d.p, Q_d.p, K_d.p, V_d.p, scale, O_d.p, wc.arg(ws.p),
+                                    wc.bytes, nullptr);
     });
     hipLaunchKernelGGL(check_row_of_slot_kernel, dim3(blocks_for(M)), dim3(256), 0, nullptr, M, ro_d.p, rowof_d.p);
     hipLaunchKernelGGL(check_sddmm_kernel, dim3(blocks_for(nnz)), dim3(256), 0, nullptr, nnz, D, rowof_d.p, ci_d.p, Q_d.p, K_d.p,

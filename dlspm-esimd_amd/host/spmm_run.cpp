@@ -41,11 +41,11 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     DLSPM_HIP_CHECK(hipMemset(C_d.p, 0xFF, (size_t)M * N * sizeof(float)));  // NaN pattern: every element must be written
 
     // the caller owns the workspace, as it owns every other buffer: 0 bytes for small problems
-    const size_t ws_bytes = workspace_to_pass(opt, DLSPM_OP_SPMM, M, K, N, nnz, ro_d.p);
-    DevBuf<char> ws(ws_bytes);
-    if (ws_bytes) std::printf("workspace: %zu bytes\n", ws_bytes);
+    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_SPMM, M, K, N, nnz, ro_d.p);
+    DevBuf<char> ws(wc.bytes);
+    if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
     const Timing t = time_launches(opt, [&]() {
-        return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, ws_bytes ? ws.p : nullptr, ws_bytes, nullptr);
+        return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, wc.arg(ws.p), wc.bytes, nullptr);
     });
     hipLaunchKernelGGL(check_spmm_kernel, dim3(blocks_for((long long)M * N)), dim3(256), 0, nullptr, M, N, ro_d.p, ci_d.p,
                        va_d.p, B_d.p, Cref_d.p);

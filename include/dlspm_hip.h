@@ -31,9 +31,17 @@
  *     owns a fixed run of nonzeros, however they are spread over the rows, and a second kernel adds the
  *     partial rows kept in the workspace, in a fixed order). That schedule is the faster one when row
  *     lengths are uneven and the slower one when they are even, so pass the workspace for matrices
- *     whose longest row is several times the mean (dlspm_csr_row_stats) and NULL otherwise. A non-NULL workspace smaller than that is refused with DLSPM_E_WORKSPACE. The
- *     contents need no initialisation and mean nothing afterwards; two calls that share a workspace
- *     must not overlap in time.
+ *     whose longest row is several times the mean (dlspm_csr_row_stats) and NULL otherwise. A non-NULL
+ *     workspace smaller than that is refused with DLSPM_E_WORKSPACE. The contents need no
+ *     initialisation and mean nothing afterwards; two calls that share a workspace must not overlap
+ *     in time.
+ *   - A caller who knows the opposite, that no row is much longer than the mean (longest row at most
+ *     one and a half times nnz / M), may say so by passing the constant DLSPM_ROWS_EVEN as `workspace`
+ *     (with workspace_bytes 0; it stands for no memory and is never dereferenced). Tall matrices of
+ *     long rows then run one whole row per wave, which is the faster split for even rows and the
+ *     slower one for uneven rows. It is a hint about speed only: a wrong one costs time, never
+ *     correctness (a row's products are added in a different, equally fixed order), and other sizes
+ *     ignore it.
  * Calls on different streams may run concurrently from different host threads (each with its own
  * workspace); the library keeps no mutable global state.
  */
@@ -53,6 +61,9 @@ extern "C" {
 #define DLSPM_E_LAUNCH       (-3) /* the HIP runtime refused the launch (see dlspm_last_hip_error)         */
 #define DLSPM_E_INVALID_CSR  (-4) /* dlspm_csr_check found a malformed CSR structure                        */
 #define DLSPM_E_NO_DEVICE    (-5) /* no gfx950 device is current                                            */
+
+/* `workspace` value that carries the caller's knowledge "row lengths are even" instead of memory (see above) */
+#define DLSPM_ROWS_EVEN ((void*)1)
 
 /* operation selectors for dlspm_workspace_bytes */
 #define DLSPM_OP_SPMM   0
@@ -125,7 +136,8 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
  * has no counterpart in the reference, whose launch sizing looks at M and N only
  * (SPMM/spmmesimd2.hpp:30-60).
  * Use: the compute calls cannot see how evenly the nonzeros are spread over the rows; a caller who finds
- * max_row_len several times nnz / M should pass a workspace (see above), a caller with even rows need not.
+ * max_row_len at least four times nnz / M should pass a workspace, one who finds it at most one and a half times
+ * nnz / M may pass DLSPM_ROWS_EVEN (see above), anyone else NULL.
  */
 int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_row_len, int* empty_rows);
 
@@ -141,6 +153,9 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
  * Returns DLSPM_OK or DLSPM_E_INVALID_ARG.
  */
 int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape);
+
+/* The same for a call that passes DLSPM_ROWS_EVEN (rows_even != 0) or does not (rows_even == 0). */
+int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int rows_even, int* shape);
 
 /* Human-readable text for a status code (never NULL). */
 const char* dlspm_status_string(int status);

@@ -30,11 +30,41 @@ def test_header_is_plain_c(tmp_path):
     src = tmp_path / "abi.c"
     src.write_text('#include "dlspm_hip.h"\n'
                    "int use(void) { int shape[10]; return dlspm_describe_launch(DLSPM_OP_SPMM, 1, 1, 1, 1, shape)"
-                   " + (int)dlspm_workspace_bytes(DLSPM_OP_FUSED, 1, 1, 1, 1); }\n")
+                   " + (int)dlspm_workspace_bytes(DLSPM_OP_FUSED, 1, 1, 1, 1)"
+                   " + spmm_csr_f32(0, 0, 0, 0, 0, 0, 0, 0, 0, DLSPM_ROWS_EVEN, 0, 0); }\n")
     inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
     r = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-fsyntax-only", "-I", inc, str(src)],
                        capture_output=True, text=True)
     assert r.returncode == 0, r.stderr
+
+
+def test_split_rule_and_the_even_rows_hint(dl):
+    """Rows per workgroup: one for long rows of unknown evenness, four (a whole row per wave) once the caller says the
+    rows are even and the matrix has at least 4096 rows; the hint changes nothing for the benchmark configurations'
+    sizes or for short rows. Sixteen waves per row: never in the fused op on tall matrices, in SpMM only from
+    16384 rows on."""
+    for op in (dl.OP_SPMM, dl.OP_SDDMM, dl.OP_FUSED):
+        for width in (32, 128, 256):
+            nnz = 8192 * 600
+            a = dl.describe_launch(op, 8192, 4096, width, nnz)
+            b = dl.describe_launch(op, 8192, 4096, width, nnz, rows_even=True)
+            assert (a["W"], a["R"]) == (4, 1) and (b["W"], b["R"]) == (4, 4)
+            assert {k: v for k, v in a.items() if k != "R"} == {k: v for k, v in b.items() if k != "R"}
+            # too few rows for 1024 workgroups of four rows: unchanged
+            assert dl.describe_launch(op, 2048, 4096, width, 2048 * 600, rows_even=True)["R"] == 1
+        # short rows are grouped by the size rule already; the hint never makes the groups smaller
+        a = dl.describe_launch(op, 65536, 1024, 64, 65536 * 20)
+        b = dl.describe_launch(op, 65536, 1024, 64, 65536 * 20, rows_even=True)
+        assert a == b and a["R"] == 16
+    for cfg in ((dl.OP_SPMM, 512, 512, 128, 78848), (dl.OP_SPMM, 2048, 512, 256, 105687),
+                (dl.OP_SDDMM, 2048, 2048, 128, 209715), (dl.OP_SPMM, 2048, 512, 392, 208896),
+                (dl.OP_FUSED, 4096, 4096, 64, 323000)):
+        assert dl.describe_launch(*cfg) == dl.describe_launch(*cfg, rows_even=True)
+    long_rows = 2000
+    assert dl.describe_launch(dl.OP_SPMM, 8192, 8192, 128, 8192 * long_rows)["W"] == 4
+    assert dl.describe_launch(dl.OP_SPMM, 24576, 8192, 128, 24576 * long_rows)["W"] == 16
+    assert dl.describe_launch(dl.OP_FUSED, 24576, 8192, 128, 24576 * long_rows)["W"] == 4
+    assert dl.describe_launch(dl.OP_FUSED, 300, 8192, 32, 300 * 7000)["W"] == 16  # few rows, very long: still sixteen
 
 
 def test_library_exports_every_declared_symbol(dl):

@@ -202,10 +202,18 @@ def test_dlmc_batch_list(tmp_path):
 
 @pytest.mark.gpu
 def test_drivers_pass_the_workspace_only_for_uneven_rows():
-    """3.3 M nonzeros: large enough for the flat schedule. Even rows: the driver passes no workspace; lognormal rows
-    (sigma 1.5): it does; both self-check against the on-device gold loop."""
+    """3.3 M nonzeros: large enough for the flat schedule. Even rows: the driver passes DLSPM_ROWS_EVEN and no memory;
+    lognormal rows (sigma 1.5): the workspace; in between (sigma 0.2) nothing; all self-check against the on-device
+    gold loop."""
     rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--iters", 3)
-    assert rc == 0 and "PASS" in out and "even, no workspace" in out and "workspace:" not in out, out
+    assert rc == 0 and "PASS" in out and "even, DLSPM_ROWS_EVEN passed" in out and "workspace:" not in out, out
+    for app in ("sddmm_run", "fused_run"):
+        rc, out = run(app, "--shape", 8192, 4096, 128, 0.1, "--iters", 3)
+        assert rc == 0 and "PASS" in out and "even, DLSPM_ROWS_EVEN passed" in out, out
+    rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 0.2, "--iters", 3)
+    assert rc == 0 and "PASS" in out and "nothing passed" in out and "workspace:" not in out, out
+    rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--no-workspace", "--iters", 3)
+    assert rc == 0 and "PASS" in out and "rows:" not in out, out
     rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 1.5, "--iters", 3)
     assert rc == 0 and "PASS" in out and "uneven, workspace passed" in out and "workspace:" in out, out
     rc, out = run("fused_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 1.5, "--iters", 3)

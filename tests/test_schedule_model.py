@@ -210,6 +210,49 @@ def test_gpu_sddmm_and_fused_equal_model_bit_for_bit(model, dl, M, K, D, kind, d
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kind,N,density", [("uniform", 128, 0.4), ("uniform", 32, 0.4), ("skewed", 128, 0.4),
+                                            ("empty_rows", 64, 0.7)])
+def test_gpu_rows_even_hint_equals_model_bit_for_bit(model, dl, kind, N, density):
+    """A call that passes ROWS_EVEN on a tall matrix of long rows runs four rows per workgroup (one whole row per wave
+    where the rows of a block are even, the nonzero-even split where they are not): the model reproduces both, also
+    when the hint is wrong, and the results stay within the parity tolerance of the default call's."""
+    import torch
+
+    M, K = 4200, 600
+    rng = np.random.default_rng(61 + N)
+    ro, ci = random_csr(rng, M, K, kind, density)
+    va = rng.normal(0, 1, ci.size).astype(np.float32)
+    B = rng.normal(0, 1, (K, N)).astype(np.float32)
+    Q = rng.normal(0, 1, (M, N)).astype(np.float32)
+    ro_d, ci_d, va_d, B_d, Q_d = (dev(torch, x) for x in (ro, ci, va, B, Q))
+
+    sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size, rows_even=True)
+    assert (sh["W"], sh["R"]) == (4, 4) and dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size)["R"] < 4
+    rc, C, writes = run_spmm(model, ro, ci, va, B, sh["G"], sh["W"], sh["R"])
+    assert rc == 0 and (writes == 1).all()
+    got = dl.spmm(ro_d, ci_d, va_d, B_d, K=K, workspace=dl.ROWS_EVEN).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), C.view(np.uint32)), f"spmm shape {sh}"
+    plain = dl.spmm(ro_d, ci_d, va_d, B_d, K=K).cpu().numpy()
+    assert np.linalg.norm(got - plain) <= 1e-5 * np.linalg.norm(plain)
+
+    fs = dl.describe_launch(dl.OP_FUSED, M, K, N, ci.size, rows_even=True)
+    assert (fs["W"], fs["R"]) == (4, 4)
+    scores = np.empty(ci.size, dtype=np.float32)
+    O = np.full((M, N), np.nan, dtype=np.float32)
+    writes = np.zeros((M, N), dtype=np.int32)
+    rc = model.model_fused(M, N, pi(ro), pi(ci), pf(Q), pf(B), pf(B), 0.125, fs["vec"], fs["G1"], fs["DS"], fs["G"],
+                           fs["W"], fs["R"], pf(scores), pf(O), pi(writes))
+    assert rc == 0 and (writes == 1).all()
+    gotO = dl.fused(ro_d, ci_d, Q_d, B_d, B_d, 0.125, workspace=dl.ROWS_EVEN).cpu().numpy()
+    assert np.array_equal(gotO.view(np.uint32), O.view(np.uint32)), f"fused shape {fs}"
+
+    # SDDMM: every slot is one wave-independent dot product, so the hint cannot change a bit
+    a = dl.sddmm(ro_d, ci_d, Q_d, B_d, workspace=dl.ROWS_EVEN)
+    b = dl.sddmm(ro_d, ci_d, Q_d, B_d)
+    assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("cfg", [1, 2, 3, 5])
 def test_gpu_benchmark_configs_equal_model_bit_for_bit(model, dl, cfg):
     import torch
