@@ -114,12 +114,12 @@ void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bo
         }
         // Rows known to be even: four rows per four-wave workgroup, which the kernels then run as one whole row per
         // wave (no partial sums, no barrier, one chain of accesses per row instead of four): 3-17 % faster than one
-        // row per workgroup from 4096 rows on, and 1.3-1.7x where the gathered operands exceed one L2 (8192 x 128
+        // row per workgroup from 2048 rows on, and 1.3-1.7x where the gathered operands exceed one L2 (8192 x 128
         // floats twice in the fused op), because waves that start together then sweep the columns together. With
         // uneven rows the same grouping is 5-20 % slower (four rows of work per workgroup make the tail of the
         // launch coarser), hence only on the caller's word. Rows below 128 nonzeros keep the grouping of the size rule
         // (4096 rows of ~100: four per workgroup measured 6 % slower than two).
-        if (rows_even && R < 4 && avg >= 128.0 && (long long)((M + 3) / 4) * col_tiles >= 1024) R = 4;
+        if (rows_even && R < 4 && avg >= 128.0 && (long long)((M + 3) / 4) * col_tiles >= 512) R = 4;
     }
 }
 

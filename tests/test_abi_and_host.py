@@ -40,7 +40,7 @@ def test_header_is_plain_c(tmp_path):
 
 def test_split_rule_and_the_even_rows_hint(dl):
     """Rows per workgroup: one for long rows of unknown evenness, four (a whole row per wave) once the caller says the
-    rows are even and the matrix has at least 4096 rows; the hint changes nothing for the benchmark configurations'
+    rows are even and the matrix has at least 2048 rows; the hint changes nothing for the benchmark configurations'
     sizes or for short rows. Sixteen waves per row: never in the fused op on tall matrices, in SpMM only from
     16384 rows on."""
     for op in (dl.OP_SPMM, dl.OP_SDDMM, dl.OP_FUSED):
@@ -50,8 +50,9 @@ def test_split_rule_and_the_even_rows_hint(dl):
             b = dl.describe_launch(op, 8192, 4096, width, nnz, rows_even=True)
             assert (a["W"], a["R"]) == (4, 1) and (b["W"], b["R"]) == (4, 4)
             assert {k: v for k, v in a.items() if k != "R"} == {k: v for k, v in b.items() if k != "R"}
-            # too few rows for 1024 workgroups of four rows: unchanged
-            assert dl.describe_launch(op, 2048, 4096, width, 2048 * 600, rows_even=True)["R"] == 1
+            # too few rows for 512 workgroups of four rows: unchanged
+            assert dl.describe_launch(op, 2048, 4096, width, 2048 * 600, rows_even=True)["R"] == 4
+            assert dl.describe_launch(op, 1536, 4096, width, 1536 * 600, rows_even=True)["R"] == 1
         # short rows are grouped by the size rule already; the hint never makes the groups smaller
         a = dl.describe_launch(op, 65536, 1024, 64, 65536 * 20)
         b = dl.describe_launch(op, 65536, 1024, 64, 65536 * 20, rows_even=True)
