@@ -141,6 +141,18 @@ __host__ __device__ __forceinline__ int split_per_wave(int T, int W)
     return per < 1 ? 1 : per;
 }
 
+// Lane i <- sum of x over the lanes below i, for i < 32 (five rounds through the LDS crossbar; the whole wave calls it).
+__device__ __forceinline__ int lanes_exclusive_sum32(int x, int lane)
+{
+    int inc = x;
+#pragma unroll
+    for (int d = 1; d < 32; d *= 2) {
+        const int y = lane_get(inc, lane >= d ? lane - d : lane);
+        inc += lane >= d ? y : 0;
+    }
+    return inc - x;
+}
+
 // Row-aligned variant of that split, used when it is nearly as even: with R = k*W rows per workgroup wave w takes the
 // k rows w*k .. w*k+k-1 whole; with W = m*R waves per row the m waves of a row take equal parts of it. A wave then
 // never works on the tail of one row and the head of the next (two dependent chains of memory accesses in sequence),

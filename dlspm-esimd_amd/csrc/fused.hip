@@ -54,13 +54,14 @@ __device__ __forceinline__ void fused_segment(Vec<VEC>* acc, int p, int q, int D
     if constexpr (kWave / G > 1) slots_sum<VEC, G, V2>(acc, lane);
 }
 
-// MASKED = false: D == G1 * VEC * DS exactly, every stage-1 access of every lane falls inside the row.
-template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R>
-__global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_tiles, float scale,
-                                                       const int* __restrict__ row_offsets,
-                                                       const int* __restrict__ col_indices,
-                                                       const float* __restrict__ Q, const float* __restrict__ Kmat,
-                                                       const float* __restrict__ Vmat, float* __restrict__ O)
+// The work of workgroup `bid`; SLICED as in spmm_block: row i owns [row_offsets[i], row_ends[i]), the part of the CSR
+// row inside one range of columns, and the split works on the running sum of the lengths.
+template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R, bool SLICED>
+__device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles, float scale,
+                                            const int* __restrict__ row_offsets, const int* __restrict__ row_ends,
+                                            const int* __restrict__ col_indices, const float* __restrict__ Q,
+                                            const float* __restrict__ Kmat, const float* __restrict__ Vmat,
+                                            float* __restrict__ O)
 {
     constexpr int TW = G * VEC * V2;
     constexpr int NP = R == 1 ? 1 : 2;
@@ -72,24 +73,41 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane % G;
     const int slot = lane / G;
-    const int rb = col_tiles == 1 ? (int)blockIdx.x : (int)(blockIdx.x / col_tiles);  // no division in the usual case
-    const int ct = blockIdx.x - rb * col_tiles;
+    const int rb = col_tiles == 1 ? bid : bid / col_tiles;  // no division in the usual case
+    const int ct = bid - rb * col_tiles;
     const int r0 = rb * R;
     const int nr = min(R, M - r0);
 
-    // the block's R + 1 row offsets without LDS or a barrier (see spmm_kernel)
-    int off_lo = 0, off_hi = 0, off_win = 0;
-    if constexpr (R == 1) {
-        off_lo = row_offsets[r0];
-        off_hi = row_offsets[r0 + 1];
+    // the block's R + 1 row offsets without LDS or a barrier (see spmm_block)
+    int off_lo = 0, off_hi = 0, off_win = 0, start_lo = 0, start_win = 0;
+    if constexpr (!SLICED) {
+        if constexpr (R == 1) {
+            off_lo = row_offsets[r0];
+            off_hi = row_offsets[r0 + 1];
+        } else {
+            static_assert(R + 1 <= kWave, "one offset per lane");
+            off_win = row_offsets[r0 + min(lane, nr)];
+        }
     } else {
-        static_assert(R + 1 <= kWave, "one offset per lane");
-        off_win = row_offsets[r0 + min(lane, nr)];
+        if constexpr (R == 1) {
+            start_lo = row_offsets[r0];
+            off_hi = row_ends[r0] - start_lo;
+        } else {
+            static_assert(R + 1 <= 32, "the running sum covers 32 lanes");
+            const int i = r0 + min(lane, nr - 1);
+            start_win = row_offsets[i];
+            off_win = lanes_exclusive_sum32(lane < nr ? row_ends[i] - start_win : 0, lane);
+        }
     }
     fetch_args_now(col_indices, Q, Kmat, Vmat, O);  // with the offsets' request: one round trip for both
     auto s_off = [&](int i) -> int {
         if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
         else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
+    };
+    auto s_shift = [&](int i) -> int {
+        if constexpr (!SLICED) return 0;
+        else if constexpr (R == 1) return start_lo;
+        else return __builtin_amdgcn_readlane(start_win, __builtin_amdgcn_readfirstlane(i)) - s_off(i);
     };
 
     int colv[V2];
@@ -122,7 +140,9 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
             const float* q_row = Q + (size_t)(r0 + r) * D;
 
             VecT acc[V2];
-            fused_segment<VEC, G1, DS, MASKED, G, V2>(acc, p, q, D, scale, col_indices, q_row, Kmat, Vmat, colv, lane);
+            const int shift = s_shift(r);
+            fused_segment<VEC, G1, DS, MASKED, G, V2>(acc, p + shift, q + shift, D, scale, col_indices, q_row, Kmat, Vmat,
+                                                      colv, lane);
 
             const bool whole_row = (p == rs) && (q == re);
             if (slot == 0) {
@@ -226,6 +246,36 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
             }
         }
     }
+}
+
+// MASKED = false: D == G1 * VEC * DS exactly, every stage-1 access of every lane falls inside the row.
+template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R>
+__global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_tiles, float scale,
+                                                       const int* __restrict__ row_offsets,
+                                                       const int* __restrict__ col_indices,
+                                                       const float* __restrict__ Q, const float* __restrict__ Kmat,
+                                                       const float* __restrict__ Vmat, float* __restrict__ O)
+{
+    fused_block<VEC, G1, DS, MASKED, G, V2, W, R, false>((int)blockIdx.x, M, D, col_tiles, scale, row_offsets, nullptr,
+                                                         col_indices, Q, Kmat, Vmat, O);
+}
+
+// Column-sliced schedule (see spmm_sliced_kernel): the row blocks once per slice of columns, slice after slice, so
+// that the rows of Kmat and V gathered at any time come from one slice; partial[s][i][:] is row i's share of slice s.
+template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int R>
+__global__ __launch_bounds__(4 * 64) void fused_sliced_kernel(int M, int D, int col_tiles, int slice_blocks, float scale,
+                                                              const int* __restrict__ bounds,
+                                                              const int* __restrict__ col_indices,
+                                                              const float* __restrict__ Q,
+                                                              const float* __restrict__ Kmat,
+                                                              const float* __restrict__ Vmat,
+                                                              float* __restrict__ partial)
+{
+    const int sl = (int)(blockIdx.x / (unsigned)slice_blocks);
+    const int bid = (int)blockIdx.x - sl * slice_blocks;
+    fused_block<VEC, G1, DS, MASKED, G, V2, 4, R, true>(bid, M, D, col_tiles, scale, bounds + (size_t)sl * M,
+                                                        bounds + (size_t)(sl + 1) * M, col_indices, Q, Kmat, Vmat,
+                                                        partial + (size_t)sl * M * D);
 }
 
 // ---- host side --------------------------------------------------------------------------------------
@@ -410,6 +460,60 @@ hipError_t fused_flat_launch(const FusedArgs& x, const FusedShape& s, const Flat
         return launch_flat<1, 4, 1, 8, 1>(x, plan, partial, stream);
     }
     return hipErrorInvalidValue;
+}
+
+// ---- column-sliced schedule ------------------------------------------------------------------------
+
+template <int VEC, int G1, int DS, int G, int V2, int R>
+static hipError_t launch_sliced_r(const FusedArgs& x, const SlicePlan& plan, const int* bounds, float* partial,
+                                  hipStream_t stream)
+{
+    constexpr int TW = G * VEC * V2;
+    const int col_tiles = (x.D + TW - 1) / TW;
+    const long long slice_blocks = (long long)((x.M + R - 1) / R) * col_tiles;
+    const long long blocks = slice_blocks * plan.slices;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    if constexpr (DS > 0) {
+        if (x.D == G1 * VEC * DS) {
+            hipLaunchKernelGGL((fused_sliced_kernel<VEC, G1, DS, false, G, V2, R>), dim3((unsigned)blocks), dim3(4 * 64), 0,
+                               stream, x.M, x.D, col_tiles, (int)slice_blocks, x.scale, bounds, x.col_indices, x.Q, x.Kmat,
+                               x.V, partial);
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((fused_sliced_kernel<VEC, G1, DS, true, G, V2, R>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream,
+                       x.M, x.D, col_tiles, (int)slice_blocks, x.scale, bounds, x.col_indices, x.Q, x.Kmat, x.V, partial);
+    return hipGetLastError();
+}
+
+template <int VEC, int G1, int DS, int G, int V2>
+static hipError_t launch_sliced(const FusedArgs& x, const SlicePlan& plan, const int* bounds, float* partial,
+                                hipStream_t stream)
+{
+    switch (plan.R) {
+        case 1: return launch_sliced_r<VEC, G1, DS, G, V2, 1>(x, plan, bounds, partial, stream);
+        case 2: return launch_sliced_r<VEC, G1, DS, G, V2, 2>(x, plan, bounds, partial, stream);
+        case 4: return launch_sliced_r<VEC, G1, DS, G, V2, 4>(x, plan, bounds, partial, stream);
+        case 8: return launch_sliced_r<VEC, G1, DS, G, V2, 8>(x, plan, bounds, partial, stream);
+        case 16: return launch_sliced_r<VEC, G1, DS, G, V2, 16>(x, plan, bounds, partial, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+hipError_t fused_sliced_launch(const FusedArgs& x, const FusedShape& s, const SlicePlan& plan, void* workspace,
+                               hipStream_t stream)
+{
+    int* bounds = static_cast<int*>(workspace);
+    float* partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + plan.bounds_bytes);
+    hipError_t e = slice_bounds_launch(x.M, x.K, plan.slices, x.row_offsets, x.col_indices, bounds, stream);
+    if (e != hipSuccess) return e;
+    e = hipErrorInvalidValue;
+    if (s.vec == 4 && s.G1 == 8 && s.DS == 4 && s.G == 32 && s.V == 1) e = launch_sliced<4, 8, 4, 32, 1>(x, plan, bounds, partial, stream);
+    else if (s.vec == 4 && s.G1 == 8 && s.DS == 8 && s.G == 64 && s.V == 1) e = launch_sliced<4, 8, 8, 64, 1>(x, plan, bounds, partial, stream);
+    else if (s.vec == 4 && s.G1 == 8 && s.DS == 16 && s.G == 64 && s.V == 2) e = launch_sliced<4, 8, 16, 64, 2>(x, plan, bounds, partial, stream);
+    if (e != hipSuccess) return e;
+    return slice_sum_launch((long long)x.M * x.D, plan.slices, partial, x.O, stream);
 }
 
 }  // namespace dlspm

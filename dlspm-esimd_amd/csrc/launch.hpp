@@ -54,10 +54,29 @@ FlatPlan flat_plan(int M, int nnz, int width, int G);
 hipError_t row_fixup_launch(int M, int N, int chunk, const int* row_offsets, const float* partial, float* out,
                             hipStream_t stream);
 
+// Column-sliced schedule: the columns of the sparse matrix (the rows of the gathered dense operands) are cut into
+// `slices` equal ranges which the device works through one after the other, `R` rows per four-wave workgroup; the
+// workspace holds the (slices + 1) x M slice boundaries of the rows, then slices x M x width partial rows.
+// slices == 0: not used for this problem.
+struct SlicePlan {
+    int slices;
+    int R;
+    size_t bounds_bytes;
+    size_t bytes;
+};
+// `operands`: dense operands gathered per nonzero (1 SpMM, 2 fused); G, col_tiles, slots: the op's lane layout
+SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int G, long long col_tiles, int slots,
+                     int min_blocks);
+hipError_t slice_bounds_launch(int M, int K, int slices, const int* row_offsets, const int* col_indices, int* bounds,
+                               hipStream_t stream);
+hipError_t slice_sum_launch(long long count, int slices, const float* partial, float* out, hipStream_t stream);
+
 SpmmShape spmm_choose(int M, int N, int nnz, bool vec4, bool rows_even = false);
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
 hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPlan& plan, float* partial,
                             hipStream_t stream);
+hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const SlicePlan& plan, void* workspace,
+                              hipStream_t stream);
 
 SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4, bool rows_even = false);
 hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t stream);
@@ -67,6 +86,8 @@ FusedShape fused_choose(int M, int D, int nnz, bool vec4, bool rows_even = false
 hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream);
 hipError_t fused_flat_launch(const FusedArgs& x, const FusedShape& s, const FlatPlan& plan, float* partial,
                              hipStream_t stream);
+hipError_t fused_sliced_launch(const FusedArgs& x, const FusedShape& s, const SlicePlan& plan, void* workspace,
+                               hipStream_t stream);
 
 // Picks (W, R), W <= max_w: waves per workgroup from the number of rows, rows per workgroup as large as keeps
 // `min_blocks` workgroups in the grid. `slots` = nonzeros of a row a wave works on at once (64 / G); `w16_long_rows`:

@@ -46,12 +46,15 @@ __device__ __forceinline__ void spmm_segment(Vec<VEC>* acc, int p, int q, const 
     if constexpr (kWave / G > 1) slots_sum<VEC, G, V>(acc, lane);
 }
 
-template <int VEC, int G, int V, int W, int R>
-__global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tiles,
-                                                      const int* __restrict__ row_offsets,
-                                                      const int* __restrict__ col_indices,
-                                                      const float* __restrict__ values,
-                                                      const float* __restrict__ B, float* __restrict__ C)
+// The work of workgroup `bid`. SLICED = false: row i owns the nonzeros [row_offsets[i], row_offsets[i + 1]).
+// SLICED = true: row i owns [row_offsets[i], row_ends[i]), a part of the CSR row (its columns inside one range of
+// columns), so the rows of a block are not contiguous in memory: the split then works on the running sum of their
+// lengths ("virtual" offsets, 0 at the block's first row) and every segment is shifted back to where it lies.
+template <int VEC, int G, int V, int W, int R, bool SLICED>
+__device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles, const int* __restrict__ row_offsets,
+                                           const int* __restrict__ row_ends, const int* __restrict__ col_indices,
+                                           const float* __restrict__ values, const float* __restrict__ B,
+                                           float* __restrict__ C)
 {
     constexpr int TW = G * VEC * V;  // columns of C covered by one wave
     using VecT = Vec<VEC>;
@@ -63,25 +66,43 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane % G;
     const int slot = lane / G;
-    const int rb = col_tiles == 1 ? (int)blockIdx.x : (int)(blockIdx.x / col_tiles);  // no division in the usual case
-    const int ct = blockIdx.x - rb * col_tiles;
+    const int rb = col_tiles == 1 ? bid : bid / col_tiles;  // no division in the usual case
+    const int ct = bid - rb * col_tiles;
     const int r0 = rb * R;
     const int nr = min(R, M - r0);
 
     // The block's R + 1 row offsets, without LDS or a barrier: with R == 1 they are the same two words for every
     // lane (scalar loads); otherwise lane i of every wave holds offset i and v_readlane picks one.
-    int off_lo = 0, off_hi = 0, off_win = 0;
-    if constexpr (R == 1) {
-        off_lo = row_offsets[r0];
-        off_hi = row_offsets[r0 + 1];
+    int off_lo = 0, off_hi = 0, off_win = 0, start_lo = 0, start_win = 0;
+    if constexpr (!SLICED) {
+        if constexpr (R == 1) {
+            off_lo = row_offsets[r0];
+            off_hi = row_offsets[r0 + 1];
+        } else {
+            static_assert(R + 1 <= kWave, "one offset per lane");
+            off_win = row_offsets[r0 + min(lane, nr)];
+        }
     } else {
-        static_assert(R + 1 <= kWave, "one offset per lane");
-        off_win = row_offsets[r0 + min(lane, nr)];
+        if constexpr (R == 1) {
+            start_lo = row_offsets[r0];
+            off_hi = row_ends[r0] - start_lo;
+        } else {
+            static_assert(R + 1 <= 32, "the running sum covers 32 lanes");
+            const int i = r0 + min(lane, nr - 1);
+            start_win = row_offsets[i];
+            off_win = lanes_exclusive_sum32(lane < nr ? row_ends[i] - start_win : 0, lane);
+        }
     }
     fetch_args_now(col_indices, values, B, C);  // after the offsets were requested: both arrive in one round trip
     auto s_off = [&](int i) -> int {
         if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
         else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
+    };
+    // where row i's first nonzero lies in memory, minus its offset in the split
+    auto s_shift = [&](int i) -> int {
+        if constexpr (!SLICED) return 0;
+        else if constexpr (R == 1) return start_lo;
+        else return __builtin_amdgcn_readlane(start_win, __builtin_amdgcn_readfirstlane(i)) - s_off(i);
     };
 
     int colv[V];  // first of this lane's VEC columns for access v; clamped to a valid column when outside
@@ -115,7 +136,8 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
             const int p = __builtin_amdgcn_readfirstlane(pos);
 
             VecT acc[V];
-            spmm_segment<VEC, G, V>(acc, p, q, col_indices, values, B, N, colv, lane);
+            const int shift = s_shift(r);
+            spmm_segment<VEC, G, V>(acc, p + shift, q + shift, col_indices, values, B, N, colv, lane);
 
             const bool whole_row = (p == rs) && (q == re);
             if (slot == 0) {
@@ -220,6 +242,32 @@ __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tile
             }
         }
     }
+}
+
+template <int VEC, int G, int V, int W, int R>
+__global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tiles,
+                                                      const int* __restrict__ row_offsets,
+                                                      const int* __restrict__ col_indices,
+                                                      const float* __restrict__ values,
+                                                      const float* __restrict__ B, float* __restrict__ C)
+{
+    spmm_block<VEC, G, V, W, R, false>((int)blockIdx.x, M, N, col_tiles, row_offsets, nullptr, col_indices, values, B, C);
+}
+
+// Column-sliced schedule: the grid holds the row blocks once per slice of columns, slice after slice, so that at
+// any time the device gathers rows of B from one slice only (a dense operand larger than one L2 is then read at L2
+// speed). Slice s of row i is [bounds[s][i], bounds[s + 1][i]); its partial row goes to partial[s][i][:].
+template <int VEC, int G, int V, int R>
+__global__ __launch_bounds__(4 * 64) void spmm_sliced_kernel(int M, int N, int col_tiles, int slice_blocks,
+                                                             const int* __restrict__ bounds,
+                                                             const int* __restrict__ col_indices,
+                                                             const float* __restrict__ values,
+                                                             const float* __restrict__ B, float* __restrict__ partial)
+{
+    const int sl = (int)(blockIdx.x / (unsigned)slice_blocks);
+    const int bid = (int)blockIdx.x - sl * slice_blocks;
+    spmm_block<VEC, G, V, 4, R, true>(bid, M, N, col_tiles, bounds + (size_t)sl * M, bounds + (size_t)(sl + 1) * M,
+                                      col_indices, values, B, partial + (size_t)sl * M * N);
 }
 
 // ---- host side --------------------------------------------------------------------------------------
@@ -386,6 +434,52 @@ hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPla
         return launch_flat<1, 8, 1>(x, plan, partial, stream);
     }
     return hipErrorInvalidValue;
+}
+
+// ---- column-sliced schedule ------------------------------------------------------------------------
+
+template <int VEC, int G, int V, int R>
+static hipError_t launch_sliced_r(const SpmmArgs& x, const SlicePlan& plan, const int* bounds, float* partial,
+                                  hipStream_t stream)
+{
+    constexpr int TW = G * VEC * V;
+    const int col_tiles = (x.N + TW - 1) / TW;
+    const long long slice_blocks = (long long)((x.M + R - 1) / R) * col_tiles;
+    const long long blocks = slice_blocks * plan.slices;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((spmm_sliced_kernel<VEC, G, V, R>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M, x.N,
+                       col_tiles, (int)slice_blocks, bounds, x.col_indices, x.values, x.B, partial);
+    return hipGetLastError();
+}
+
+template <int VEC, int G, int V>
+static hipError_t launch_sliced(const SpmmArgs& x, const SlicePlan& plan, const int* bounds, float* partial,
+                                hipStream_t stream)
+{
+    switch (plan.R) {
+        case 1: return launch_sliced_r<VEC, G, V, 1>(x, plan, bounds, partial, stream);
+        case 2: return launch_sliced_r<VEC, G, V, 2>(x, plan, bounds, partial, stream);
+        case 4: return launch_sliced_r<VEC, G, V, 4>(x, plan, bounds, partial, stream);
+        case 8: return launch_sliced_r<VEC, G, V, 8>(x, plan, bounds, partial, stream);
+        case 16: return launch_sliced_r<VEC, G, V, 16>(x, plan, bounds, partial, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const SlicePlan& plan, void* workspace,
+                              hipStream_t stream)
+{
+    int* bounds = static_cast<int*>(workspace);
+    float* partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + plan.bounds_bytes);
+    hipError_t e = slice_bounds_launch(x.M, x.K, plan.slices, x.row_offsets, x.col_indices, bounds, stream);
+    if (e != hipSuccess) return e;
+    e = hipErrorInvalidValue;
+    if (s.vec == 4 && s.G == 64 && s.V == 1) e = launch_sliced<4, 64, 1>(x, plan, bounds, partial, stream);
+    else if (s.vec == 4 && s.G == 64 && s.V == 2) e = launch_sliced<4, 64, 2>(x, plan, bounds, partial, stream);
+    else if (s.vec == 4 && s.G == 32 && s.V == 1) e = launch_sliced<4, 32, 1>(x, plan, bounds, partial, stream);
+    if (e != hipSuccess) return e;
+    return slice_sum_launch((long long)x.M * x.N, plan.slices, partial, x.C, stream);
 }
 
 }  // namespace dlspm

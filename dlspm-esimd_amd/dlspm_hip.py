@@ -40,6 +40,7 @@ EXPORTS = (
     "dlspm_csr_check",
     "dlspm_describe_launch",
     "dlspm_describe_launch_rows",
+    "dlspm_describe_slices",
     "dlspm_csr_row_stats",
     "dlspm_status_string",
     "dlspm_last_hip_error",
@@ -77,6 +78,8 @@ def lib() -> ctypes.CDLL:
         L.dlspm_describe_launch.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci)]
         L.dlspm_describe_launch_rows.argtypes = [ci, ci, ci, ci, ci, ci, ctypes.POINTER(ci)]
         L.dlspm_describe_launch_rows.restype = ci
+        L.dlspm_describe_slices.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci), ctypes.POINTER(ci)]
+        L.dlspm_describe_slices.restype = ci
         L.dlspm_describe_launch.restype = ci
         L.dlspm_csr_row_stats.argtypes = [ci, vp, vp, ctypes.POINTER(ci), ctypes.POINTER(ci)]
         L.dlspm_csr_row_stats.restype = ci
@@ -184,6 +187,15 @@ def describe_launch(op: int, M: int, K: int, N: int, nnz: int, rows_even: bool =
         raise DlspmError(st, "dlspm_describe_launch")
     return dict(zip(("vec", "G", "V", "G1", "DS", "W", "R", "col_tiles", "flat_chunk", "flat_units"),
                     (int(x) for x in out)))
+
+
+def describe_slices(op: int, M: int, K: int, N: int, nnz: int) -> tuple:
+    """(slices, rows per workgroup) of the column-sliced schedule a call with workspace would use; slices == 0: none."""
+    a, b = ctypes.c_int(0), ctypes.c_int(0)
+    st = lib().dlspm_describe_slices(op, M, K, N, nnz, ctypes.byref(a), ctypes.byref(b))
+    if st != OK:
+        raise DlspmError(st, "dlspm_describe_slices")
+    return a.value, b.value
 
 
 def workspace_bytes(op: int, M: int, K: int, N: int, nnz: int) -> int:

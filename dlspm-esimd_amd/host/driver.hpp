@@ -204,18 +204,21 @@ struct Options {
     int warmup = 5;
     int iters = 20;  // the reference keeps the minimum of 20 launches (SPMM/spmm-esimd-fromfile2.cpp:194-243)
     bool cold = false;
-    // what to pass as `workspace`: by default the memory dlspm_workspace_bytes asks for when the longest row is at least
-    // four times the mean row (dlspm_csr_row_stats), DLSPM_ROWS_EVEN when it is at most one and a half times the mean;
+    // what to pass as `workspace`: by default the memory dlspm_workspace_bytes asks for when the column-sliced schedule
+    // applies or the longest row is at least four times the mean row (dlspm_csr_row_stats), DLSPM_ROWS_EVEN when it is
+    // at most one and a half times the mean;
     // --workspace: always the memory, --no-workspace: always NULL
     enum Workspace { kAuto, kAlways, kNever } workspace = kAuto;
     std::string csv, dump;
     double tol = 1e-4;  // relative Frobenius error allowed between the kernel and the check kernel
 };
 
-// What this run tells the library about the rows through the `workspace` argument, from one look at the row lengths
-// (dlspm_csr_row_stats): the memory it asks for when the rows are uneven enough for the flat schedule to pay (measured:
-// from lognormal sigma ~1 on, i.e. a longest row of at least four times the mean), the constant DLSPM_ROWS_EVEN when no
-// row is longer than one and a half times the mean, nothing otherwise.
+// What this run passes as `workspace`, from the sizes and one look at the row lengths (dlspm_csr_row_stats):
+//   * the memory the library asks for when the column-sliced schedule applies (dense operands beyond 4 MiB: faster for
+//     every row-length distribution measured), or when the rows are uneven enough for the flat schedule to pay
+//     (measured: from lognormal sigma ~1 on, i.e. a longest row of at least four times the mean);
+//   * the constant DLSPM_ROWS_EVEN when no row is longer than one and a half times the mean;
+//   * nothing otherwise.
 struct WorkspaceChoice {
     size_t bytes = 0;        // device memory to allocate and pass
     bool rows_even = false;  // pass DLSPM_ROWS_EVEN instead
@@ -227,14 +230,17 @@ inline WorkspaceChoice workspace_to_pass(const Options& opt, int op, int M, int 
     WorkspaceChoice c;
     if (opt.workspace == Options::kNever || M <= 0 || nnz <= 0) return c;
     const size_t want = dlspm_workspace_bytes(op, M, K, width, nnz);
+    int slices = 0;
+    if (dlspm_describe_slices(op, M, K, width, nnz, &slices, nullptr) != DLSPM_OK) throw std::runtime_error("dlspm_describe_slices failed");
     int longest = 0, empty = 0;
     if (dlspm_csr_row_stats(M, row_offsets_dev, nullptr, &longest, &empty) != DLSPM_OK) throw std::runtime_error("dlspm_csr_row_stats failed");
     const double mean = (double)nnz / M;
     const bool uneven = longest >= 4.0 * mean, even = longest <= 1.5 * mean;
-    if (opt.workspace == Options::kAlways || (uneven && want > 0)) c.bytes = want;
+    if (opt.workspace == Options::kAlways || slices > 0 || (uneven && want > 0)) c.bytes = want;
     else c.rows_even = even;
     std::printf("rows: longest %d, mean %.1f, empty %d -> %s\n", longest, mean, empty,
                 opt.workspace == Options::kAlways ? "workspace passed (--workspace)"
+                : slices > 0                      ? "dense operands beyond 4 MiB, workspace passed (column-sliced schedule)"
                 : c.bytes                         ? "uneven, workspace passed (flat schedule)"
                 : c.rows_even                     ? "even, DLSPM_ROWS_EVEN passed"
                                                   : "nothing passed");

@@ -29,7 +29,11 @@
  *     bytes lets SpMM and the fused op use the flat schedule where the library's size rule allows it
  *     (from about half a million nonzeros, 64 per row on average, dense width above 64: every wave then
  *     owns a fixed run of nonzeros, however they are spread over the rows, and a second kernel adds the
- *     partial rows kept in the workspace, in a fixed order). That schedule is the faster one when row
+ *     partial rows kept in the workspace, in a fixed order), or, when the dense operands gathered per
+ *     nonzero exceed 4 MiB together (K x N floats in SpMM, twice K x D in the fused op), the
+ *     column-sliced schedule (the column ranges of the sparse matrix one after the other, so that the
+ *     part of the dense operands in use fits the cache; partial rows per range in the workspace, added
+ *     in range order). The flat schedule is the faster one when row
  *     lengths are uneven and the slower one when they are even, so pass the workspace for matrices
  *     whose longest row is several times the mean (dlspm_csr_row_stats) and NULL otherwise. A non-NULL
  *     workspace smaller than that is refused with DLSPM_E_WORKSPACE. The contents need no
@@ -156,6 +160,14 @@ int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape)
 
 /* The same for a call that passes DLSPM_ROWS_EVEN (rows_even != 0) or does not (rows_even == 0). */
 int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int rows_even, int* shape);
+
+/*
+ * Column-sliced schedule that a call WITH workspace would use for these sizes: *slices = number of column ranges
+ * the device works through one after the other (0 = that schedule is not used: dense operands of at most 4 MiB,
+ * narrow dense rows, short rows, every SDDMM), *rows_per_workgroup = rows of one slice handled by a four-wave
+ * workgroup. Either pointer may be NULL. Host-only. No counterpart in the reference.
+ */
+int dlspm_describe_slices(int op, int M, int K, int N_or_D, int nnz, int* slices, int* rows_per_workgroup);
 
 /* Human-readable text for a status code (never NULL). */
 const char* dlspm_status_string(int status);

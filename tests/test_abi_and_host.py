@@ -68,6 +68,34 @@ def test_split_rule_and_the_even_rows_hint(dl):
     assert dl.describe_launch(dl.OP_FUSED, 300, 8192, 32, 300 * 7000)["W"] == 16  # few rows, very long: still sixteen
 
 
+def test_column_sliced_schedule_rule(dl):
+    """Slices of at most 2 MiB of gathered dense operand, only when the operand exceeds 4 MiB, the dense rows are wide
+    and a row keeps at least 16 nonzeros per slice on average; the workspace then holds the boundaries and the
+    partial rows of every slice."""
+    M = K = 8192
+    nnz = M * 800
+    assert dl.describe_slices(dl.OP_FUSED, M, K, 128, nnz)[0] == 4      # Kmat + V: 8 MiB
+    assert dl.describe_slices(dl.OP_FUSED, M, K, 256, nnz)[0] == 8      # 16 MiB
+    assert dl.describe_slices(dl.OP_FUSED, M, K, 64, nnz)[0] == 0       # 4 MiB: fits
+    assert dl.describe_slices(dl.OP_SPMM, M, K, 256, nnz)[0] == 4       # B: 8 MiB
+    assert dl.describe_slices(dl.OP_SPMM, M, K, 200, nnz)[0] == 4       # 6.25 MiB
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, nnz)[0] == 16      # 128 MiB: the most slices there are
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, M * 100)[0] == 6   # ... but a row keeps 16 nonzeros per slice
+    assert dl.describe_slices(dl.OP_SPMM, M, K, 128, nnz)[0] == 0       # 4 MiB: fits
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 20, 32, nnz)[0] == 0  # narrow dense rows: not built for them
+    assert dl.describe_slices(dl.OP_SPMM, M, K, 256, M * 70)[0] == 4    # 70 nonzeros per row: four slices of 17
+    assert dl.describe_slices(dl.OP_SPMM, M, K, 256, M * 40)[0] == 0    # 40 per row, 0.33 M nonzeros: too small
+    assert dl.describe_slices(dl.OP_SPMM, 4 * M, K, 256, 4 * M * 40)[0] == 2  # 1.3 M nonzeros: two slices of 20
+    assert dl.describe_slices(dl.OP_SPMM, 4 * M, K, 256, 4 * M * 30)[0] == 0  # 30 per row: not even two
+    assert dl.describe_slices(dl.OP_SDDMM, M, K, 256, nnz)[0] == 0
+    slices, R = dl.describe_slices(dl.OP_FUSED, M, K, 256, nnz)
+    assert R == 4                                                       # 100 nonzeros per row and slice
+    bounds = -(-(slices + 1) * M * 4 // 256) * 256
+    assert dl.workspace_bytes(dl.OP_FUSED, M, K, 256, nnz) == bounds + slices * M * 256 * 4
+    # below the sliced rule the flat schedule's size is reported as before
+    assert dl.workspace_bytes(dl.OP_SPMM, M, K, 128, nnz) == dl.describe_launch(dl.OP_SPMM, M, K, 128, nnz)["flat_units"] * 2 * 128 * 4
+
+
 def test_library_exports_every_declared_symbol(dl):
     lib = ctypes.CDLL(dl.LIB_PATH)
     for name in declared_functions():
@@ -117,6 +145,7 @@ def test_flat_schedule_rule_and_workspace_size(dl, monkeypatch):
         for op in (dl.OP_SPMM, dl.OP_SDDMM, dl.OP_FUSED):
             assert dl.workspace_bytes(op, *cfg_sizes) == 0 and dl.describe_launch(op, *cfg_sizes)["flat_chunk"] == 0
     monkeypatch.setenv("DLSPM_FLAT", "1")
+    monkeypatch.setenv("DLSPM_SLICES", "0")
     monkeypatch.setenv("DLSPM_FLAT_CHUNK", "192")
     assert dl.workspace_bytes(dl.OP_SPMM, 100, 50, 7, 1000) == -(-1000 // 192) * 2 * 7 * 4
 

@@ -419,6 +419,7 @@ def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
     for flat in (False, True):
         if flat:
             monkeypatch.setenv("DLSPM_FLAT", "1")
+            monkeypatch.setenv("DLSPM_SLICES", "0")
             monkeypatch.setenv("DLSPM_FLAT_CHUNK", "128")
         need = max(dl.workspace_bytes(dl.OP_SPMM, M, K, N, ci.size), dl.workspace_bytes(dl.OP_FUSED, M, K, N, ci.size))
         assert (need > 0) == flat

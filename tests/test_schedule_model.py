@@ -302,6 +302,7 @@ def test_gpu_flat_spmm_equals_model_bit_for_bit(model, dl, monkeypatch, kind, M,
     va = rng.normal(0, 1, ci.size).astype(np.float32)
     B = rng.normal(0, 1, (K, N)).astype(np.float32)
     monkeypatch.setenv("DLSPM_FLAT", "1")
+    monkeypatch.setenv("DLSPM_SLICES", "0")
     monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
     sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size)
     assert sh["flat_chunk"] == chunk and sh["flat_units"] == -(-ci.size // chunk)
@@ -340,6 +341,7 @@ def test_gpu_flat_fused_equals_model_bit_for_bit(model, dl, monkeypatch, kind, M
     Km = rng.normal(0, 1, (K, D)).astype(np.float32)
     V = rng.normal(0, 1, (K, D)).astype(np.float32)
     monkeypatch.setenv("DLSPM_FLAT", "1")
+    monkeypatch.setenv("DLSPM_SLICES", "0")
     monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
     fs = dl.describe_launch(dl.OP_FUSED, M, K, D, ci.size)
     assert fs["flat_chunk"] == chunk
@@ -381,6 +383,7 @@ def test_gpu_flat_sddmm_equals_model_and_the_row_block_schedule_bit_for_bit(mode
     args = (dev(torch, ro), dev(torch, ci), dev(torch, Q), dev(torch, Km))
     block = dl.sddmm(*args).cpu().numpy()
     monkeypatch.setenv("DLSPM_FLAT", "1")
+    monkeypatch.setenv("DLSPM_SLICES", "0")
     monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
     assert dl.describe_launch(dl.OP_SDDMM, M, K, D, ci.size)["flat_chunk"] == chunk
     assert dl.workspace_bytes(dl.OP_SDDMM, M, K, D, ci.size) == 0
@@ -411,6 +414,7 @@ def test_gpu_random_shapes_equal_model_bit_for_bit(model, dl, monkeypatch, seed)
         flat = bool(rng.integers(0, 2)) and nnz > 0
         chunk = int(rng.choice([64, 128, 192, 320, 512, 1024]))
         monkeypatch.setenv("DLSPM_FLAT", "1" if flat else "0")
+        monkeypatch.setenv("DLSPM_SLICES", "0")
         monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
         tag = f"seed {seed} draw {it}: M {M} K {K} N {N} {kind} {density} nnz {nnz} flat {flat} chunk {chunk}"
         print(tag, flush=True)
@@ -458,3 +462,135 @@ def test_gpu_random_shapes_equal_model_bit_for_bit(model, dl, monkeypatch, seed)
         out = torch.full((M, N), float("nan"), device="cuda")
         dl.fused(ro_d, ci_d, dev(torch, Q), dev(torch, B), dev(torch, V), 0.25, out=out, workspace=ws)
         assert np.array_equal(bits(out.cpu().numpy()), bits(O)), "fused " + tag
+
+
+# ---- column-sliced schedule ------------------------------------------------------------------------------------------
+def column_slices(ro, ci, K, slices):
+    """The sparse matrix cut into `slices` equal column ranges: per range its own CSR row offsets and the mask of the
+    nonzeros it keeps (columns ascend inside a row, so each row's share is one run of the row)."""
+    M = ro.size - 1
+    rows = np.repeat(np.arange(M), np.diff(ro))
+    out = []
+    for p in range(slices):
+        lo, hi = p * K // slices, (p + 1) * K // slices
+        keep = (ci >= lo) & (ci < hi)
+        rop = np.zeros(M + 1, dtype=np.int32)
+        rop[1:] = np.cumsum(np.bincount(rows[keep], minlength=M))
+        out.append((rop, keep))
+    assert sum(k.sum() for _, k in out) == ci.size
+    return out
+
+
+SLICED_CASES = [("uniform", 300, 512, 128, 3), ("skewed", 1100, 700, 256, 2), ("empty_rows", 500, 300, 392, 4),
+                ("long_and_empty", 1500, 700, 128, 5), ("full", 40, 256, 96, 16), ("uniform", 70, 900, 513, 7)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,M,K,N,slices", SLICED_CASES)
+def test_gpu_sliced_spmm_equals_model_bit_for_bit(model, dl, oracle, monkeypatch, kind, M, K, N, slices):
+    """Column-sliced SpMM = the row-block kernel's arithmetic on each column range of the matrix (the model, run on
+    that range's own CSR arrays with the split the library reports), the ranges' partial rows added in range order."""
+    import torch
+
+    rng = np.random.default_rng(71 + M + N)
+    if kind == "long_and_empty":
+        ro, ci = long_and_empty_rows(rng, M, K, 3, K - 50, 3)
+    else:
+        ro, ci = random_csr(rng, M, K, kind, 1.0 if kind == "full" else 0.2)
+    va = rng.normal(0, 1, ci.size).astype(np.float32)
+    B = rng.normal(0, 1, (K, N)).astype(np.float32)
+    assert dl.describe_slices(dl.OP_SPMM, M, K, N, ci.size)[0] == 0       # far too small for the rule
+    monkeypatch.setenv("DLSPM_SLICES", str(slices))
+    got_slices, R = dl.describe_slices(dl.OP_SPMM, M, K, N, ci.size)
+    assert got_slices == slices and R in (1, 2, 4, 8, 16)
+    sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size)
+    need = dl.workspace_bytes(dl.OP_SPMM, M, K, N, ci.size)
+    assert need >= (slices + 1) * M * 4 + slices * M * N * 4
+
+    expect = None
+    for rop, keep in column_slices(ro, ci, K, slices):
+        rc, part, writes = run_spmm(model, rop, ci[keep], va[keep], B, sh["G"], 4, R)
+        assert rc == 0 and (writes == 1).all()
+        expect = part if expect is None else expect + part
+    ws = torch.full((need // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    out = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    args = (dev(torch, ro), dev(torch, ci), dev(torch, va), dev(torch, B))
+    dl.spmm(*args, K=K, out=out, workspace=ws)
+    got = out.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), expect.view(np.uint32)), \
+        f"{np.count_nonzero(got.view(np.uint32) != expect.view(np.uint32))} of {got.size} elements differ in their bits"
+    ref = oracle.spmm(ro, ci, va, B)
+    assert np.linalg.norm(got - ref) <= 1e-5 * max(np.linalg.norm(ref), 1e-30)
+    with pytest.raises(dl.DlspmError) as e:
+        dl.spmm(*args, K=K, out=out, workspace=ws[: need // 4 - 1])
+    assert e.value.status == dl.E_WORKSPACE
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,M,K,D,slices", [("uniform", 300, 512, 128, 3), ("skewed", 700, 600, 256, 2),
+                                               ("long_and_empty", 900, 600, 100, 4), ("empty_rows", 200, 300, 512, 5),
+                                               ("uniform", 150, 400, 200, 16)])
+def test_gpu_sliced_fused_equals_model_bit_for_bit(model, dl, oracle, monkeypatch, kind, M, K, D, slices):
+    import torch
+
+    rng = np.random.default_rng(81 + M + D)
+    if kind == "long_and_empty":
+        ro, ci = long_and_empty_rows(rng, M, K, 2, K - 50, 3)
+    else:
+        ro, ci = random_csr(rng, M, K, kind, 0.2)
+    Q = rng.normal(0, 1, (M, D)).astype(np.float32)
+    Km = rng.normal(0, 1, (K, D)).astype(np.float32)
+    V = rng.normal(0, 1, (K, D)).astype(np.float32)
+    monkeypatch.setenv("DLSPM_SLICES", str(slices))
+    got_slices, R = dl.describe_slices(dl.OP_FUSED, M, K, D, ci.size)
+    assert got_slices == slices
+    fs = dl.describe_launch(dl.OP_FUSED, M, K, D, ci.size)
+    need = dl.workspace_bytes(dl.OP_FUSED, M, K, D, ci.size)
+
+    expect = None
+    for rop, keep in column_slices(ro, ci, K, slices):
+        cip = ci[keep] if keep.any() else np.zeros(1, np.int32)
+        scores = np.empty(max(int(keep.sum()), 1), dtype=np.float32)
+        part = np.full((M, D), np.nan, dtype=np.float32)
+        writes = np.zeros((M, D), dtype=np.int32)
+        rc = model.model_fused(M, D, pi(rop), pi(cip), pf(Q), pf(Km), pf(V), 0.125, fs["vec"], fs["G1"], fs["DS"], fs["G"],
+                               4, R, pf(scores), pf(part), pi(writes))
+        assert rc == 0 and (writes == 1).all()
+        expect = part if expect is None else expect + part
+    ws = torch.full((need // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    out = torch.full((M, D), float("nan"), dtype=torch.float32, device="cuda")
+    dl.fused(dev(torch, ro), dev(torch, ci), dev(torch, Q), dev(torch, Km), dev(torch, V), 0.125, out=out, workspace=ws)
+    got = out.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), expect.view(np.uint32)), \
+        f"{np.count_nonzero(got.view(np.uint32) != expect.view(np.uint32))} of {got.size} elements differ in their bits"
+    ref = oracle.fused(ro, ci, Q, Km, V, 0.125)
+    assert np.linalg.norm(got - ref) <= 1e-5 * max(np.linalg.norm(ref), 1e-30)
+
+
+@pytest.mark.gpu
+def test_gpu_sliced_schedule_does_not_need_ascending_columns(dl, oracle, monkeypatch):
+    """The slice boundaries are found by a search that assumes ascending columns; with any other order they are still
+    a partition of every row (a running maximum), so the result stays right."""
+    import torch
+
+    rng = np.random.default_rng(91)
+    M, K, N = 400, 500, 128
+    ro, ci = random_csr(rng, M, K, "skewed", 0.2)
+    ci = ci.copy()
+    for i in range(M):
+        rng.shuffle(ci[ro[i]:ro[i + 1]])
+    va = rng.normal(0, 1, ci.size).astype(np.float32)
+    B = rng.normal(0, 1, (K, N)).astype(np.float32)
+    monkeypatch.setenv("DLSPM_SLICES", "4")
+    need = dl.workspace_bytes(dl.OP_SPMM, M, K, N, ci.size)
+    ws = torch.empty(need // 4, dtype=torch.float32, device="cuda")
+    got = dl.spmm(dev(torch, ro), dev(torch, ci), dev(torch, va), dev(torch, B), K=K, workspace=ws).cpu().numpy()
+    ref = oracle.spmm(ro, ci, va, B)
+    assert np.linalg.norm(got - ref) <= 1e-5 * np.linalg.norm(ref)
+    Q = rng.normal(0, 1, (M, N)).astype(np.float32)
+    need = dl.workspace_bytes(dl.OP_FUSED, M, K, N, ci.size)
+    ws = torch.empty(need // 4, dtype=torch.float32, device="cuda")
+    gotO = dl.fused(dev(torch, ro), dev(torch, ci), dev(torch, Q), dev(torch, B), dev(torch, B), 0.125, workspace=ws).cpu().numpy()
+    refO = oracle.fused(ro, ci, Q, B, B, 0.125)
+    assert np.linalg.norm(gotO - refO) <= 1e-5 * np.linalg.norm(refO)
+
