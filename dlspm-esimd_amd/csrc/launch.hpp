@@ -56,7 +56,7 @@ hipError_t row_fixup_launch(int M, int N, int chunk, const int* row_offsets, con
 
 // Column-sliced schedule: the columns of the sparse matrix (the rows of the gathered dense operands) are cut into
 // `slices` equal ranges which the device works through one after the other, `R` rows per four-wave workgroup; the
-// workspace holds the (slices + 1) x M slice boundaries of the rows, then slices x M x width partial rows.
+// workspace holds the (slices + 1) x M slice boundaries of the rows, then slices x M x width partial rows (SpMM, fused).
 // slices == 0: not used for this problem.
 struct SlicePlan {
     int slices;
@@ -64,9 +64,10 @@ struct SlicePlan {
     size_t bounds_bytes;
     size_t bytes;
 };
-// `operands`: dense operands gathered per nonzero (1 SpMM, 2 fused); G, col_tiles, slots: the op's lane layout
-SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int G, long long col_tiles, int slots,
-                     int min_blocks);
+// `operands`: dense operands gathered per nonzero (1 SpMM and SDDMM, 2 fused); `partial_width`: floats of a partial
+// row (0 for SDDMM, whose results need no adding up); G, col_tiles, slots: the op's lane layout
+SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial_width, int G, long long col_tiles,
+                     int slots, int min_blocks);
 hipError_t slice_bounds_launch(int M, int K, int slices, const int* row_offsets, const int* col_indices, int* bounds,
                                hipStream_t stream);
 hipError_t slice_sum_launch(long long count, int slices, const float* partial, float* out, hipStream_t stream);
@@ -81,6 +82,8 @@ hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const Slice
 SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4, bool rows_even = false);
 hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t stream);
 hipError_t sddmm_flat_launch(const SddmmArgs& x, const SddmmShape& s, int chunk, hipStream_t stream);
+hipError_t sddmm_sliced_launch(const SddmmArgs& x, const SddmmShape& s, const SlicePlan& plan, void* workspace,
+                               hipStream_t stream);
 
 FusedShape fused_choose(int M, int D, int nnz, bool vec4, bool rows_even = false);
 hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream);

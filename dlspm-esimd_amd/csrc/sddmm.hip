@@ -47,31 +47,51 @@ __device__ __forceinline__ void sddmm_segment(int p, int q, int D, const int* __
     }
 }
 
-// MASKED = false: D == G1 * VEC * DS exactly, every access of every lane falls inside the row.
-template <int VEC, int G1, int DS, bool MASKED, int W, int R>
-__global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* __restrict__ row_offsets,
-                                                       const int* __restrict__ col_indices,
-                                                       const float* __restrict__ lhs, const float* __restrict__ rhs,
-                                                       float* __restrict__ out)
+// The work of workgroup `bid`. SLICED = false: row i owns the nonzeros [row_offsets[i], row_offsets[i + 1]); SLICED =
+// true: [row_offsets[i], row_ends[i]), the part of the CSR row inside one range of columns (see spmm_block): the split
+// works on the running sum of the lengths and every segment is shifted back to where it lies, which is also where its
+// results go.
+template <int VEC, int G1, int DS, bool MASKED, int W, int R, bool SLICED>
+__device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __restrict__ row_offsets,
+                                            const int* __restrict__ row_ends, const int* __restrict__ col_indices,
+                                            const float* __restrict__ lhs, const float* __restrict__ rhs,
+                                            float* __restrict__ out)
 {
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int r0 = blockIdx.x * R;
+    const int r0 = bid * R;
     const int nr = min(R, M - r0);
 
-    // the block's R + 1 row offsets without LDS or a barrier (see spmm_kernel): this kernel then has neither
-    int off_lo = 0, off_hi = 0, off_win = 0;
-    if constexpr (R == 1) {
-        off_lo = row_offsets[r0];
-        off_hi = row_offsets[r0 + 1];
+    // the block's R + 1 row offsets without LDS or a barrier (see spmm_block): this kernel then has neither
+    int off_lo = 0, off_hi = 0, off_win = 0, start_lo = 0, start_win = 0;
+    if constexpr (!SLICED) {
+        if constexpr (R == 1) {
+            off_lo = row_offsets[r0];
+            off_hi = row_offsets[r0 + 1];
+        } else {
+            static_assert(R + 1 <= kWave, "one offset per lane");
+            off_win = row_offsets[r0 + min(lane, nr)];
+        }
     } else {
-        static_assert(R + 1 <= kWave, "one offset per lane");
-        off_win = row_offsets[r0 + min(lane, nr)];
+        if constexpr (R == 1) {
+            start_lo = row_offsets[r0];
+            off_hi = row_ends[r0] - start_lo;
+        } else {
+            static_assert(R + 1 <= 32, "the running sum covers 32 lanes");
+            const int i = r0 + min(lane, nr - 1);
+            start_win = row_offsets[i];
+            off_win = lanes_exclusive_sum32(lane < nr ? row_ends[i] - start_win : 0, lane);
+        }
     }
     fetch_args_now(col_indices, lhs, rhs, out);  // with the offsets' request: one round trip for both
     auto s_off = [&](int i) -> int {
         if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
         else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
+    };
+    auto s_shift = [&](int i) -> int {
+        if constexpr (!SLICED) return 0;
+        else if constexpr (R == 1) return start_lo;
+        else return __builtin_amdgcn_readlane(start_win, __builtin_amdgcn_readfirstlane(i)) - s_off(i);
     };
 
     const int T0 = s_off(0);
@@ -92,11 +112,38 @@ __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* 
         const int p = __builtin_amdgcn_readfirstlane(pos);
         const float* lhs_row = lhs + (size_t)(r0 + r) * D;
 
-        sddmm_segment<VEC, G1, DS, MASKED>(p, q, D, col_indices, lhs_row, rhs, out, lane);
+        const int shift = s_shift(r);
+        sddmm_segment<VEC, G1, DS, MASKED>(p + shift, q + shift, D, col_indices, lhs_row, rhs, out, lane);
         pos = q;
         ++r;
         while (r < nr && s_off(r + 1) <= pos) ++r;
     }
+}
+
+// MASKED = false: D == G1 * VEC * DS exactly, every access of every lane falls inside the row.
+template <int VEC, int G1, int DS, bool MASKED, int W, int R>
+__global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* __restrict__ row_offsets,
+                                                       const int* __restrict__ col_indices,
+                                                       const float* __restrict__ lhs, const float* __restrict__ rhs,
+                                                       float* __restrict__ out)
+{
+    sddmm_block<VEC, G1, DS, MASKED, W, R, false>((int)blockIdx.x, M, D, row_offsets, nullptr, col_indices, lhs, rhs, out);
+}
+
+// Column-sliced schedule (see spmm_sliced_kernel): the row blocks once per slice of columns, slice after slice, so that
+// the rows of rhs gathered at any time come from one slice. Every result still goes to its own CSR slot: no partial
+// rows, no second pass, and the same bits as under any other schedule.
+template <int VEC, int G1, int DS, bool MASKED, int R>
+__global__ __launch_bounds__(4 * 64) void sddmm_sliced_kernel(int M, int D, int slice_blocks,
+                                                              const int* __restrict__ bounds,
+                                                              const int* __restrict__ col_indices,
+                                                              const float* __restrict__ lhs,
+                                                              const float* __restrict__ rhs, float* __restrict__ out)
+{
+    const int sl = (int)(blockIdx.x / (unsigned)slice_blocks);
+    const int bid = (int)blockIdx.x - sl * slice_blocks;
+    sddmm_block<VEC, G1, DS, MASKED, 4, R, true>(bid, M, D, bounds + (size_t)sl * M, bounds + (size_t)(sl + 1) * M,
+                                                 col_indices, lhs, rhs, out);
 }
 
 // ---- host side --------------------------------------------------------------------------------------
@@ -242,6 +289,50 @@ hipError_t sddmm_flat_launch(const SddmmArgs& x, const SddmmShape& s, int chunk,
     } else if (s.G1 == 4 && s.DS == 1) {
         return launch_flat<1, 4, 1>(x, chunk, stream);
     }
+    return hipErrorInvalidValue;
+}
+
+// ---- column-sliced schedule ------------------------------------------------------------------------
+
+template <int VEC, int G1, int DS, int R>
+static hipError_t launch_sliced_r(const SddmmArgs& x, const SlicePlan& plan, const int* bounds, hipStream_t stream)
+{
+    const long long slice_blocks = (x.M + R - 1) / R;
+    const long long blocks = slice_blocks * plan.slices;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    if (x.D == G1 * VEC * DS)
+        hipLaunchKernelGGL((sddmm_sliced_kernel<VEC, G1, DS, false, R>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream,
+                           x.M, x.D, (int)slice_blocks, bounds, x.col_indices, x.lhs, x.rhs, x.out);
+    else
+        hipLaunchKernelGGL((sddmm_sliced_kernel<VEC, G1, DS, true, R>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream,
+                           x.M, x.D, (int)slice_blocks, bounds, x.col_indices, x.lhs, x.rhs, x.out);
+    return hipGetLastError();
+}
+
+template <int VEC, int G1, int DS>
+static hipError_t launch_sliced(const SddmmArgs& x, const SlicePlan& plan, const int* bounds, hipStream_t stream)
+{
+    switch (plan.R) {
+        case 1: return launch_sliced_r<VEC, G1, DS, 1>(x, plan, bounds, stream);
+        case 2: return launch_sliced_r<VEC, G1, DS, 2>(x, plan, bounds, stream);
+        case 4: return launch_sliced_r<VEC, G1, DS, 4>(x, plan, bounds, stream);
+        case 8: return launch_sliced_r<VEC, G1, DS, 8>(x, plan, bounds, stream);
+        case 16: return launch_sliced_r<VEC, G1, DS, 16>(x, plan, bounds, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+// built for 64 < D <= 512 (G1 = 8 with 4, 8 or 16 accesses per lane)
+hipError_t sddmm_sliced_launch(const SddmmArgs& x, const SddmmShape& s, const SlicePlan& plan, void* workspace,
+                               hipStream_t stream)
+{
+    int* bounds = static_cast<int*>(workspace);
+    const hipError_t e = slice_bounds_launch(x.M, x.K, plan.slices, x.row_offsets, x.col_indices, bounds, stream);
+    if (e != hipSuccess) return e;
+    if (s.vec == 4 && s.G1 == 8 && s.DS == 4) return launch_sliced<4, 8, 4>(x, plan, bounds, stream);
+    if (s.vec == 4 && s.G1 == 8 && s.DS == 8) return launch_sliced<4, 8, 8>(x, plan, bounds, stream);
+    if (s.vec == 4 && s.G1 == 8 && s.DS == 16) return launch_sliced<4, 8, 16>(x, plan, bounds, stream);
     return hipErrorInvalidValue;
 }
 

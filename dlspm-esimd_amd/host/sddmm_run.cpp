@@ -39,10 +39,13 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     if (dlspm_csr_check(M, K, nnz, ro_d.p, ci_d.p, nullptr) != DLSPM_OK) throw std::invalid_argument("malformed CSR structure");
     DLSPM_HIP_CHECK(hipMemset(out_d.p, 0xFF, std::max(nnz, 1) * sizeof(float)));
 
-    // SDDMM needs no memory; the argument only carries what is known about the rows
+    // SDDMM needs memory only for the slice boundaries of the column-sliced schedule; otherwise the argument only
+    // carries what is known about the rows
     const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_SDDMM, M, K, D, nnz, ro_d.p);
+    DevBuf<char> ws(wc.bytes);
+    if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
     const Timing t = time_launches(opt, [&]() {
-        return sddmm_csr_f32(M, K, D, nnz, ro_d.p, ci_d.p, lhs_d.p, rhs_d.p, out_d.p, wc.arg(nullptr), 0, nullptr);
+        return sddmm_csr_f32(M, K, D, nnz, ro_d.p, ci_d.p, lhs_d.p, rhs_d.p, out_d.p, wc.arg(ws.p), wc.bytes, nullptr);
     });
     hipLaunchKernelGGL(check_row_of_slot_kernel, dim3(blocks_for(M)), dim3(256), 0, nullptr, M, ro_d.p, rowof_d.p);
     hipLaunchKernelGGL(check_sddmm_kernel, dim3(blocks_for(nnz)), dim3(256), 0, nullptr, nnz, D, rowof_d.p, ci_d.p, lhs_d.p,

@@ -30,10 +30,10 @@
  *     (from about half a million nonzeros, 64 per row on average, dense width above 64: every wave then
  *     owns a fixed run of nonzeros, however they are spread over the rows, and a second kernel adds the
  *     partial rows kept in the workspace, in a fixed order), or, when the dense operands gathered per
- *     nonzero exceed 4 MiB together (K x N floats in SpMM, twice K x D in the fused op), the
+ *     nonzero exceed 4 MiB together (K x N floats in SpMM, K x D in SDDMM, twice K x D in the fused op), the
  *     column-sliced schedule (the column ranges of the sparse matrix one after the other, so that the
  *     part of the dense operands in use fits the cache; partial rows per range in the workspace, added
- *     in range order). The flat schedule is the faster one when row
+ *     in range order; SDDMM keeps only the range boundaries there). The flat schedule is the faster one when row
  *     lengths are uneven and the slower one when they are even, so pass the workspace for matrices
  *     whose longest row is several times the mean (dlspm_csr_row_stats) and NULL otherwise. A non-NULL
  *     workspace smaller than that is refused with DLSPM_E_WORKSPACE. The contents need no
@@ -117,8 +117,9 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz,
                          void* workspace, size_t workspace_bytes, void* stream);
 
 /*
- * Bytes of device workspace the op can use for these sizes (0 = none, as for every SDDMM and for small
- * or short-row problems; `workspace` may always be NULL). Host-only. Takes the place of the host-side
+ * Bytes of device workspace the op can use for these sizes (0 = none, as for small or short-row problems;
+ * SDDMM uses one only for the slice boundaries of the column-sliced schedule; `workspace` may always be NULL).
+ * Host-only. Takes the place of the host-side
  * launch sizing the reference does before each launch (SPMM/spmm-esimd-fromfile2.cpp:188-192,
  * SDDMM/sddmm-esimd-fromfile_v4.cpp:146-160).
  */
@@ -164,7 +165,7 @@ int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int ro
 /*
  * Column-sliced schedule that a call WITH workspace would use for these sizes: *slices = number of column ranges
  * the device works through one after the other (0 = that schedule is not used: dense operands of at most 4 MiB,
- * narrow dense rows, short rows, every SDDMM), *rows_per_workgroup = rows of one slice handled by a four-wave
+ * narrow dense rows, short rows), *rows_per_workgroup = rows of one slice handled by a four-wave
  * workgroup. Either pointer may be NULL. Host-only. No counterpart in the reference.
  */
 int dlspm_describe_slices(int op, int M, int K, int N_or_D, int nnz, int* slices, int* rows_per_workgroup);

@@ -87,7 +87,9 @@ def test_column_sliced_schedule_rule(dl):
     assert dl.describe_slices(dl.OP_SPMM, M, K, 256, M * 40)[0] == 0    # 40 per row, 0.33 M nonzeros: too small
     assert dl.describe_slices(dl.OP_SPMM, 4 * M, K, 256, 4 * M * 40)[0] == 2  # 1.3 M nonzeros: two slices of 20
     assert dl.describe_slices(dl.OP_SPMM, 4 * M, K, 256, 4 * M * 30)[0] == 0  # 30 per row: not even two
-    assert dl.describe_slices(dl.OP_SDDMM, M, K, 256, nnz)[0] == 0
+    assert dl.describe_slices(dl.OP_SDDMM, M, K, 256, nnz)[0] == 4      # rhs: 8 MiB; only the boundaries need memory
+    assert dl.workspace_bytes(dl.OP_SDDMM, M, K, 256, nnz) == -(-5 * M * 4 // 256) * 256
+    assert dl.describe_slices(dl.OP_SDDMM, M, K, 128, nnz)[0] == 0 and dl.workspace_bytes(dl.OP_SDDMM, M, K, 128, nnz) == 0
     slices, R = dl.describe_slices(dl.OP_FUSED, M, K, 256, nnz)
     assert R == 4                                                       # 100 nonzeros per row and slice
     bounds = -(-(slices + 1) * M * 4 // 256) * 256

@@ -594,3 +594,37 @@ def test_gpu_sliced_schedule_does_not_need_ascending_columns(dl, oracle, monkeyp
     refO = oracle.fused(ro, ci, Q, B, B, 0.125)
     assert np.linalg.norm(gotO - refO) <= 1e-5 * np.linalg.norm(refO)
 
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,M,K,D,slices", [("uniform", 300, 512, 128, 3), ("skewed", 700, 600, 256, 2),
+                                               ("long_and_empty", 900, 600, 100, 4), ("empty_rows", 200, 300, 512, 5),
+                                               ("full", 60, 256, 65, 16)])
+def test_gpu_sliced_sddmm_gives_the_same_bits(dl, oracle, monkeypatch, kind, M, K, D, slices):
+    """Every SDDMM result is one dot product computed by one lane group in a fixed order, whatever the schedule: the
+    column-sliced call must reproduce the plain call bit for bit, and leave no slot unwritten."""
+    import torch
+
+    rng = np.random.default_rng(95 + M + D)
+    if kind == "long_and_empty":
+        ro, ci = long_and_empty_rows(rng, M, K, 2, K - 50, 3)
+    else:
+        ro, ci = random_csr(rng, M, K, kind, 1.0 if kind == "full" else 0.2)
+    Q = rng.normal(0, 1, (M, D)).astype(np.float32)
+    Km = rng.normal(0, 1, (K, D)).astype(np.float32)
+    args = (dev(torch, ro), dev(torch, ci), dev(torch, Q), dev(torch, Km))
+    plain = dl.sddmm(*args)
+    assert dl.workspace_bytes(dl.OP_SDDMM, M, K, D, ci.size) == 0
+    monkeypatch.setenv("DLSPM_SLICES", str(slices))
+    assert dl.describe_slices(dl.OP_SDDMM, M, K, D, ci.size)[0] == slices
+    need = dl.workspace_bytes(dl.OP_SDDMM, M, K, D, ci.size)
+    assert need >= (slices + 1) * M * 4
+    ws = torch.empty(need // 4, dtype=torch.int32, device="cuda")
+    out = torch.full((ci.size,), float("nan"), dtype=torch.float32, device="cuda")
+    dl.sddmm(*args, out=out, workspace=ws)
+    assert torch.equal(out, plain)
+    ref = oracle.sddmm(ro, ci, Q, Km)
+    assert np.linalg.norm(out.cpu().numpy() - ref) <= 1e-5 * np.linalg.norm(ref)
+    with pytest.raises(dl.DlspmError) as e:
+        dl.sddmm(*args, out=out, workspace=ws[: need // 4 - 1])
+    assert e.value.status == dl.E_WORKSPACE
+
