@@ -405,7 +405,7 @@ def test_exact_integer_properties_at_large_size(torch_cuda, dl):
 
 
 def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
-    """Both schedules only enqueue kernels (no memset, no allocation, no synchronisation), so a call may be captured.
+    """All three schedules only enqueue kernels (no memset, no allocation, no synchronisation), so a call may be captured.
     The graph is replayed several times with eager work and synchronisations in between, on changed inputs, and every
     replay must equal the eager result bit for bit."""
     torch = torch_cuda
@@ -416,14 +416,17 @@ def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
     va = torch.randn(ci.size, device="cuda")
     B = torch.randn(K, N, device="cuda")
     Q = torch.randn(M, N, device="cuda")
-    for flat in (False, True):
-        if flat:
+    for schedule in ("row-block", "flat", "sliced"):
+        if schedule == "flat":
             monkeypatch.setenv("DLSPM_FLAT", "1")
             monkeypatch.setenv("DLSPM_SLICES", "0")
             monkeypatch.setenv("DLSPM_FLAT_CHUNK", "128")
-        need = max(dl.workspace_bytes(dl.OP_SPMM, M, K, N, ci.size), dl.workspace_bytes(dl.OP_FUSED, M, K, N, ci.size))
-        assert (need > 0) == flat
-        ws = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda") if flat else None
+        elif schedule == "sliced":
+            monkeypatch.setenv("DLSPM_SLICES", "3")
+        need = max(dl.workspace_bytes(op, M, K, N, ci.size) for op in (dl.OP_SPMM, dl.OP_SDDMM, dl.OP_FUSED))
+        assert (need > 0) == (schedule != "row-block")
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda") if need else None
+        ws_s = ws if schedule == "sliced" else None  # SDDMM uses a workspace under the sliced schedule only
         C = torch.empty(M, N, device="cuda")
         S = torch.empty(ci.size, device="cuda")
         O = torch.empty(M, N, device="cuda")
@@ -434,7 +437,7 @@ def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
             stream.synchronize()
             with torch.cuda.graph(graph, stream=stream):
                 dl.spmm(ro_d, ci_d, va, B, K=K, out=C, workspace=ws)
-                dl.sddmm(ro_d, ci_d, Q, B, out=S)
+                dl.sddmm(ro_d, ci_d, Q, B, out=S, workspace=ws_s)
                 dl.fused(ro_d, ci_d, Q, B, B, 0.5, out=O, workspace=ws)
         for rep in range(4):
             va.copy_(torch.randn(ci.size, device="cuda"))  # eager work between the replays: new inputs
@@ -444,11 +447,11 @@ def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
             graph.replay()
             torch.cuda.synchronize()
             got = (C.clone(), S.clone(), O.clone())
-            want = (dl.spmm(ro_d, ci_d, va, B, K=K, workspace=ws).clone(), dl.sddmm(ro_d, ci_d, Q, B).clone(),
+            want = (dl.spmm(ro_d, ci_d, va, B, K=K, workspace=ws).clone(), dl.sddmm(ro_d, ci_d, Q, B, workspace=ws_s).clone(),
                     dl.fused(ro_d, ci_d, Q, B, B, 0.5, workspace=ws).clone())
             torch.cuda.synchronize()
             for g, w in zip(got, want):
-                assert torch.equal(g, w), f"replay {rep}, flat={flat}"
+                assert torch.equal(g, w), f"replay {rep}, schedule {schedule}"
 
 
 def test_concurrent_calls_from_two_threads_on_two_streams(torch_cuda, dl, oracle):
