@@ -86,12 +86,13 @@ static FlatPlan sddmm_flat_plan(int M, int nnz, int D)
 // XCD's 4 MiB L2; the slices are cut to 2 MiB of them. Measured on MI355X (8192 x 8192, 30 % dense, lognormal rows,
 // sigma 0.6; row-block / flat / sliced): fused, D = 128 (8 MiB of Kmat and V): 1429 / 1374 / 676 us, D = 256 (16 MiB):
 // 4024 / 3946 / 1328 us; SpMM, N = 256: 1472 / 1390 / 685 us; slices of 4 MiB instead: 769, 1441, 803 us. Operands of
-// exactly 4 MiB gain 10 % at 30 % density and lose 5 % at 3 %: left alone. Like the flat schedule only from half a
+// exactly 4 MiB (8192 x 128 floats) gain 13-16 % at 10-30 % density and lose 5 % at 3 %: sliced in two for long rows only. Like the flat schedule only from half a
 // million nonzeros on (two more launches). DLSPM_SLICES=0 switches it off, DLSPM_SLICES=n forces n slices (tuning, tests).
 constexpr long long kSliceMinOperand = 4ll << 20;  // bytes gathered from; above this the operand is sliced
 constexpr long long kSliceBytes = 2ll << 20;       // bytes of it per slice
 constexpr int kSliceMaxSlices = 16;
 constexpr int kSliceMinRow = 16;  // mean nonzeros of a row inside one slice; fewer slices rather than shorter shares
+constexpr int kSliceMinRowAtL2 = 256;  // the same for an operand of exactly kSliceMinOperand bytes
 
 SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial_width, int G, long long col_tiles,
                      int slots, int min_blocks)
@@ -103,9 +104,11 @@ SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial
     const long long bytes = (long long)K * width * (long long)sizeof(float) * operands;
     long long slices = (bytes + kSliceBytes - 1) / kSliceBytes;
     if (slices > kSliceMaxSlices) slices = kSliceMaxSlices;
-    const long long fit = (long long)nnz / ((long long)kSliceMinRow * M);  // slices that leave a row kSliceMinRow nonzeros
+    // slices that leave a row its minimum share; an operand that just fills the L2 is worth slicing for long rows only
+    const int min_row = bytes > kSliceMinOperand ? kSliceMinRow : kSliceMinRowAtL2;
+    const long long fit = (long long)nnz / ((long long)min_row * M);
     if (slices > fit) slices = fit;
-    const bool by_rule = bytes > kSliceMinOperand && nnz >= kFlatMinNnz && slices >= 2;
+    const bool by_rule = bytes >= kSliceMinOperand && nnz >= kFlatMinNnz && slices >= 2;
     if (force == 0 || force == 1 || (force < 0 && !by_rule)) return p;
     if (force >= 2) slices = force < kSliceMaxSlices ? force : kSliceMaxSlices;
     if (slices > K) slices = K;

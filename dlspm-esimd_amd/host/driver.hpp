@@ -214,8 +214,8 @@ struct Options {
 };
 
 // What this run passes as `workspace`, from the sizes and one look at the row lengths (dlspm_csr_row_stats):
-//   * the memory the library asks for when the column-sliced schedule applies (dense operands beyond 4 MiB: faster for
-//     every row-length distribution measured), or when the rows are uneven enough for the flat schedule to pay
+//   * the memory the library asks for when the column-sliced schedule applies (dense operands of 4 MiB or more: faster
+//     for every row-length distribution measured, except even rows at two slices), or when the rows are uneven enough for the flat schedule to pay
 //     (measured: from lognormal sigma ~1 on, i.e. a longest row of at least four times the mean);
 //   * the constant DLSPM_ROWS_EVEN when no row is longer than one and a half times the mean;
 //   * nothing otherwise.
@@ -236,11 +236,14 @@ inline WorkspaceChoice workspace_to_pass(const Options& opt, int op, int M, int 
     if (dlspm_csr_row_stats(M, row_offsets_dev, nullptr, &longest, &empty) != DLSPM_OK) throw std::runtime_error("dlspm_csr_row_stats failed");
     const double mean = (double)nnz / M;
     const bool uneven = longest >= 4.0 * mean, even = longest <= 1.5 * mean;
-    if (opt.workspace == Options::kAlways || slices > 0 || (uneven && want > 0)) c.bytes = want;
+    // even rows and an operand that only just exceeds the L2 (two slices): one whole row per wave does as well or better
+    // (measured: SpMM and fused 5-9 % faster at exactly 4 MiB, equal at 8 MiB; SDDMM 2-12 % slower)
+    const bool sliced = slices > 0 && !(even && slices <= 2 && op != DLSPM_OP_SDDMM);
+    if (opt.workspace == Options::kAlways || sliced || (uneven && want > 0 && slices == 0)) c.bytes = want;
     else c.rows_even = even;
     std::printf("rows: longest %d, mean %.1f, empty %d -> %s\n", longest, mean, empty,
                 opt.workspace == Options::kAlways ? "workspace passed (--workspace)"
-                : slices > 0                      ? "dense operands beyond 4 MiB, workspace passed (column-sliced schedule)"
+                : sliced                          ? "dense operands beyond one L2, workspace passed (column-sliced schedule)"
                 : c.bytes                         ? "uneven, workspace passed (flat schedule)"
                 : c.rows_even                     ? "even, DLSPM_ROWS_EVEN passed"
                                                   : "nothing passed");

@@ -76,12 +76,16 @@ def test_column_sliced_schedule_rule(dl):
     nnz = M * 800
     assert dl.describe_slices(dl.OP_FUSED, M, K, 128, nnz)[0] == 4      # Kmat + V: 8 MiB
     assert dl.describe_slices(dl.OP_FUSED, M, K, 256, nnz)[0] == 8      # 16 MiB
-    assert dl.describe_slices(dl.OP_FUSED, M, K, 64, nnz)[0] == 0       # 4 MiB: fits
+    assert dl.describe_slices(dl.OP_FUSED, M, K, 64, nnz)[0] == 0       # 4 MiB, but narrow dense rows
+    assert dl.describe_slices(dl.OP_FUSED, M, K // 2, 128, nnz)[0] == 2 # 4 MiB just fills the L2: in two for long rows
+    assert dl.describe_slices(dl.OP_FUSED, M, K // 2, 128, M * 400)[0] == 0  # ... not for 200 nonzeros per slice
     assert dl.describe_slices(dl.OP_SPMM, M, K, 256, nnz)[0] == 4       # B: 8 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, K, 200, nnz)[0] == 4       # 6.25 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, nnz)[0] == 16      # 128 MiB: the most slices there are
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, M * 100)[0] == 6   # ... but a row keeps 16 nonzeros per slice
-    assert dl.describe_slices(dl.OP_SPMM, M, K, 128, nnz)[0] == 0       # 4 MiB: fits
+    assert dl.describe_slices(dl.OP_SPMM, M, K, 128, nnz)[0] == 2       # 4 MiB, 400 nonzeros per slice
+    assert dl.describe_slices(dl.OP_SPMM, M, K, 128, M * 400)[0] == 0   # 4 MiB, 200 nonzeros per slice
+    assert dl.describe_slices(dl.OP_SPMM, M, K, 100, nnz)[0] == 0       # 3.1 MiB: fits
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 20, 32, nnz)[0] == 0  # narrow dense rows: not built for them
     assert dl.describe_slices(dl.OP_SPMM, M, K, 256, M * 70)[0] == 4    # 70 nonzeros per row: four slices of 17
     assert dl.describe_slices(dl.OP_SPMM, M, K, 256, M * 40)[0] == 0    # 40 per row, 0.33 M nonzeros: too small
@@ -89,13 +93,13 @@ def test_column_sliced_schedule_rule(dl):
     assert dl.describe_slices(dl.OP_SPMM, 4 * M, K, 256, 4 * M * 30)[0] == 0  # 30 per row: not even two
     assert dl.describe_slices(dl.OP_SDDMM, M, K, 256, nnz)[0] == 4      # rhs: 8 MiB; only the boundaries need memory
     assert dl.workspace_bytes(dl.OP_SDDMM, M, K, 256, nnz) == -(-5 * M * 4 // 256) * 256
-    assert dl.describe_slices(dl.OP_SDDMM, M, K, 128, nnz)[0] == 0 and dl.workspace_bytes(dl.OP_SDDMM, M, K, 128, nnz) == 0
+    assert dl.describe_slices(dl.OP_SDDMM, M, K, 100, nnz)[0] == 0 and dl.workspace_bytes(dl.OP_SDDMM, M, K, 100, nnz) == 0
     slices, R = dl.describe_slices(dl.OP_FUSED, M, K, 256, nnz)
     assert R == 4                                                       # 100 nonzeros per row and slice
     bounds = -(-(slices + 1) * M * 4 // 256) * 256
     assert dl.workspace_bytes(dl.OP_FUSED, M, K, 256, nnz) == bounds + slices * M * 256 * 4
     # below the sliced rule the flat schedule's size is reported as before
-    assert dl.workspace_bytes(dl.OP_SPMM, M, K, 128, nnz) == dl.describe_launch(dl.OP_SPMM, M, K, 128, nnz)["flat_units"] * 2 * 128 * 4
+    assert dl.workspace_bytes(dl.OP_SPMM, M, K, 100, nnz) == dl.describe_launch(dl.OP_SPMM, M, K, 100, nnz)["flat_units"] * 2 * 100 * 4
 
 
 def test_library_exports_every_declared_symbol(dl):

@@ -377,6 +377,46 @@ def test_flat_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
+@pytest.mark.parametrize("sigma", [0.0, 1.5])
+def test_column_sliced_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
+    """Dense operands of 8 MiB (SpMM, SDDMM) and 16 MiB (fused) at K = 8192, N = D = 256: a call WITH workspace takes the
+    column-sliced schedule by the library's own rule (4 and 8 slices); all three ops against the multi-threaded oracle,
+    on near-uniform and on heavily skewed rows, and the same calls without workspace must agree."""
+    torch = torch_cuda
+    M, K, N = 4096, 8192, 256
+    if sigma == 0.0:
+        ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 71, M, K, 0.05)
+    else:
+        ro, ci = dl.make_pattern(dl.PATTERN_LOGNORMAL_ROWS, 72, M, K, 0.05 * K, sigma)
+    nnz = ci.size
+    va = dl.fill("uniform", 73, (nnz,), -1.0, 1.0)
+    B = dl.fill("uniform", 74, (K, N), -1.0, 1.0)
+    Q = dl.fill("normal", 75, (M, N), 0.0, 1.0)
+    ro_d, ci_d, va_d, B_d, Q_d = (dev(torch, x) for x in (ro, ci, va, B, Q))
+    assert dl.describe_slices(dl.OP_SPMM, M, K, N, nnz)[0] == 4
+    assert dl.describe_slices(dl.OP_SDDMM, M, K, N, nnz)[0] == 4
+    assert dl.describe_slices(dl.OP_FUSED, M, K, N, nnz)[0] == 8
+
+    ws = torch.empty(dl.workspace_bytes(dl.OP_SPMM, M, K, N, nnz), dtype=torch.uint8, device="cuda")
+    got = dl.spmm(ro_d, ci_d, va_d, B_d, K=K, workspace=ws)
+    ref = oracle.spmm(ro, ci, va, B, omp=True)
+    assert oracle.rel_frobenius(got.cpu().numpy(), ref) <= TOL
+    assert oracle.rel_frobenius(dl.spmm(ro_d, ci_d, va_d, B_d, K=K).cpu().numpy(), ref) <= TOL
+    assert (got.cpu().numpy()[np.diff(ro) == 0] == 0).all()
+
+    wss = torch.empty(dl.workspace_bytes(dl.OP_SDDMM, M, K, N, nnz), dtype=torch.uint8, device="cuda")
+    gotS = dl.sddmm(ro_d, ci_d, Q_d, B_d, workspace=wss)
+    assert torch.equal(gotS, dl.sddmm(ro_d, ci_d, Q_d, B_d))
+    assert oracle.rel_frobenius(gotS.cpu().numpy(), oracle.sddmm(ro, ci, Q, B, omp=True)) <= TOL
+
+    wsf = torch.empty(dl.workspace_bytes(dl.OP_FUSED, M, K, N, nnz), dtype=torch.uint8, device="cuda")
+    gotO = dl.fused(ro_d, ci_d, Q_d, B_d, B_d, 0.01, workspace=wsf)
+    refO = oracle.fused(ro, ci, Q, B, B, 0.01, omp=True)
+    assert oracle.rel_frobenius(gotO.cpu().numpy(), refO) <= TOL
+    assert oracle.rel_frobenius(dl.fused(ro_d, ci_d, Q_d, B_d, B_d, 0.01).cpu().numpy(), refO) <= TOL
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
 def test_exact_integer_properties_at_large_size(torch_cuda, dl):
     """Size-independent, bit-exact checks on 65536 skewed rows (several million nonzeros), no oracle needed: with small-integer
     operands every fp32 product and sum is exact whatever the summation order, so
