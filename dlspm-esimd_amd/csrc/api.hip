@@ -216,7 +216,10 @@ __global__ void csr_check_kernel(int M, int K, int nnz, const int* __restrict__ 
 static SlicePlan spmm_slice_plan(int M, int K, int N, int nnz, const SpmmShape& s)
 {
     const int tw = s.G * s.vec * s.V;
-    return slice_plan(M, K, N, nnz, 1, N, s.vec == 4 ? s.G : 0, (N + tw - 1) / tw, kWave / s.G, 2048);
+    // the column tiles are worked through one after the other: one tile's slab of B is what is gathered from at a time
+    SlicePlan p = slice_plan(M, K, N < tw ? N : tw, nnz, 1, 0, s.vec == 4 ? s.G : 0, (N + tw - 1) / tw, kWave / s.G, 2048);
+    p.bytes = p.slices > 0 ? p.bounds_bytes + (size_t)p.slices * M * (size_t)N * sizeof(float) : 0;
+    return p;
 }
 static SlicePlan fused_slice_plan(int M, int K, int D, int nnz, const FusedShape& s)
 {
@@ -247,7 +250,7 @@ int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int
     const bool vec4 = N >= 4;  // dwordx4 accesses need only dword alignment
     const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C};
     const bool even = workspace == DLSPM_ROWS_EVEN;  // a constant that says something about the rows, not memory
-    const SpmmShape shape = spmm_choose(M, N, nnz, vec4, even);
+    const SpmmShape shape = spmm_choose(M, K, N, nnz, vec4, even);
     hipError_t e;
     if (!even && workspace != nullptr && workspace_bytes > 0) {
         const SlicePlan sliced = spmm_slice_plan(M, K, N, nnz, shape);
@@ -336,7 +339,7 @@ size_t dlspm_workspace_bytes(int op, int M, int K, int N_or_D, int nnz)
     // workspace; a call without workspace runs the row-block schedule instead.
     if (M <= 0 || N_or_D <= 0 || nnz <= 0) return 0;
     if (op == DLSPM_OP_SPMM) {
-        const SpmmShape s = spmm_choose(M, N_or_D, nnz, N_or_D >= 4);
+        const SpmmShape s = spmm_choose(M, K, N_or_D, nnz, N_or_D >= 4);
         const SlicePlan sliced = spmm_slice_plan(M, K, N_or_D, nnz, s);
         return sliced.slices > 0 ? sliced.bytes : flat_plan(M, nnz, N_or_D, s.G).bytes;
     }
@@ -413,7 +416,7 @@ int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int ro
     const bool vec4 = n >= 4;
     for (int i = 0; i < 10; ++i) shape[i] = 0;
     if (op == DLSPM_OP_SPMM) {
-        const SpmmShape s = spmm_choose(M, n, nnz, vec4, even);
+        const SpmmShape s = spmm_choose(M, K, n, nnz, vec4, even);
         const int tw = s.G * s.vec * s.V;
         shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[5] = s.W; shape[6] = s.R; shape[7] = (n + tw - 1) / tw;
         const FlatPlan fp = flat_plan(M, nnz, n, s.G);
@@ -445,7 +448,7 @@ int dlspm_describe_slices(int op, int M, int K, int N_or_D, int nnz, int* slices
 {
     if (M < 0 || K < 0 || N_or_D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     SlicePlan p{0, 1, 0, 0};
-    if (op == DLSPM_OP_SPMM) p = spmm_slice_plan(M, K, N_or_D, nnz, spmm_choose(M, N_or_D, nnz, N_or_D >= 4));
+    if (op == DLSPM_OP_SPMM) p = spmm_slice_plan(M, K, N_or_D, nnz, spmm_choose(M, K, N_or_D, nnz, N_or_D >= 4));
     else if (op == DLSPM_OP_FUSED) p = fused_slice_plan(M, K, N_or_D, nnz, fused_choose(M, N_or_D, nnz, N_or_D >= 4));
     else if (op == DLSPM_OP_SDDMM) p = sddmm_slice_plan(M, K, N_or_D, nnz, sddmm_choose(M, N_or_D, nnz, N_or_D >= 4));
     else return DLSPM_E_INVALID_ARG;

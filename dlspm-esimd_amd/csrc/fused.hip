@@ -73,8 +73,10 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane % G;
     const int slot = lane / G;
-    const int rb = col_tiles == 1 ? bid : bid / col_tiles;  // no division in the usual case
-    const int ct = bid - rb * col_tiles;
+    // column tiles (D > 1024) tile-major, as in spmm_block; no division in the usual case of one tile
+    const int row_blocks = (M + R - 1) / R;
+    const int ct = col_tiles == 1 ? 0 : bid / row_blocks;
+    const int rb = bid - ct * row_blocks;
     const int r0 = rb * R;
     const int nr = min(R, M - r0);
 
@@ -375,10 +377,12 @@ __global__ __launch_bounds__(kFlatWaves * 64) void fused_flat_kernel(int M, int 
     const int g = lane % G;
     const int slot = lane / G;
     const long long id = (long long)blockIdx.x * kFlatWaves + w;
-    const int unit = (int)(id / col_tiles);
-    const int ct = (int)(id - (long long)unit * col_tiles);
+    // column tiles tile-major, as in the row-block kernel: all units of tile 0, then of tile 1, ...
+    const int units = (int)(((long long)nnz + chunk - 1) / chunk);
+    const int ct = col_tiles == 1 ? 0 : (int)(id / units);
+    const int unit = (int)(id - (long long)ct * units);
     const long long a64 = (long long)unit * chunk;
-    if (a64 >= nnz) return;  // wave-uniform
+    if (ct >= col_tiles || a64 >= nnz) return;  // wave-uniform
     const int a = (int)a64;
     const int b = (int)min((long long)nnz, a64 + chunk);
 

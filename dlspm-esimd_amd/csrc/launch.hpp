@@ -11,7 +11,7 @@ namespace dlspm {
 //   G1  : lanes covering one dot product (SDDMM / fused stage 1)        DS : accesses per lane per dot
 //         product (0 = run-time loop, lhs row re-read instead of kept in registers)
 //   W   : waves per workgroup                                           R  : consecutive rows per workgroup
-struct SpmmShape { int vec, G, V, W, R; };
+struct SpmmShape { int vec, G, V, W, R, tile_major; };  // tile_major: column tiles one after the other (else row blocks)
 struct SddmmShape { int vec, G1, DS, W, R; };
 struct FusedShape { int vec, G1, DS, G, V, W, R; };
 
@@ -72,7 +72,7 @@ hipError_t slice_bounds_launch(int M, int K, int slices, const int* row_offsets,
                                hipStream_t stream);
 hipError_t slice_sum_launch(long long count, int slices, const float* partial, float* out, hipStream_t stream);
 
-SpmmShape spmm_choose(int M, int N, int nnz, bool vec4, bool rows_even = false);
+SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even = false);
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
 hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPlan& plan, float* partial,
                             hipStream_t stream);

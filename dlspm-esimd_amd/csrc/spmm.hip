@@ -14,6 +14,8 @@
 //   * rows finished inside one wave are stored straight to C; rows shared by several waves leave
 //     per-wave partial sums in LDS which are added in wave order after one barrier, so the result does
 //     not depend on timing (no atomics, no pre-zeroed output); rows without nonzeros are written as 0.
+#include <cstdlib>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -51,7 +53,8 @@ __device__ __forceinline__ void spmm_segment(Vec<VEC>* acc, int p, int q, const 
 // columns), so the rows of a block are not contiguous in memory: the split then works on the running sum of their
 // lengths ("virtual" offsets, 0 at the block's first row) and every segment is shifted back to where it lies.
 template <int VEC, int G, int V, int W, int R, bool SLICED>
-__device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles, const int* __restrict__ row_offsets,
+__device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles, int tile_major,
+                                           const int* __restrict__ row_offsets,
                                            const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                            const float* __restrict__ values, const float* __restrict__ B,
                                            float* __restrict__ C)
@@ -66,8 +69,22 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane % G;
     const int slot = lane / G;
-    const int rb = col_tiles == 1 ? bid : bid / col_tiles;  // no division in the usual case
-    const int ct = bid - rb * col_tiles;
+    // Column tiles (dense rows wider than one wave covers): row-major order (the tiles of a row block next to each
+    // other, so the CSR arrays are read from memory once) while all of B fits one L2; tile-major order (all row blocks
+    // of tile 0, then of tile 1, ...) when it does not, so that the device gathers from one K x TW slab of B at a time.
+    // Measured on 512 x 4608, N = 3136 (B: 55 MiB): 708 -> 239 us tile-major; on 2048 x 1024, N = 784 (3 MiB), lognormal
+    // rows: 81 us row-major, 93 us tile-major. No division in the usual case of one tile.
+    int ct = 0, rb = bid;
+    if (col_tiles != 1) {
+        if (tile_major) {
+            const int row_blocks = (M + R - 1) / R;
+            ct = bid / row_blocks;
+            rb = bid - ct * row_blocks;
+        } else {
+            rb = bid / col_tiles;
+            ct = bid - rb * col_tiles;
+        }
+    }
     const int r0 = rb * R;
     const int nr = min(R, M - r0);
 
@@ -245,35 +262,36 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
 }
 
 template <int VEC, int G, int V, int W, int R>
-__global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tiles,
+__global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tiles, int tile_major,
                                                       const int* __restrict__ row_offsets,
                                                       const int* __restrict__ col_indices,
                                                       const float* __restrict__ values,
                                                       const float* __restrict__ B, float* __restrict__ C)
 {
-    spmm_block<VEC, G, V, W, R, false>((int)blockIdx.x, M, N, col_tiles, row_offsets, nullptr, col_indices, values, B, C);
+    spmm_block<VEC, G, V, W, R, false>((int)blockIdx.x, M, N, col_tiles, tile_major, row_offsets, nullptr, col_indices,
+                                       values, B, C);
 }
 
 // Column-sliced schedule: the grid holds the row blocks once per slice of columns, slice after slice, so that at
 // any time the device gathers rows of B from one slice only (a dense operand larger than one L2 is then read at L2
 // speed). Slice s of row i is [bounds[s][i], bounds[s + 1][i]); its partial row goes to partial[s][i][:].
 template <int VEC, int G, int V, int R>
-__global__ __launch_bounds__(4 * 64) void spmm_sliced_kernel(int M, int N, int col_tiles, int slice_blocks,
-                                                             const int* __restrict__ bounds,
+__global__ __launch_bounds__(4 * 64) void spmm_sliced_kernel(int M, int N, int col_tiles, int tile_major,
+                                                             int slice_blocks, const int* __restrict__ bounds,
                                                              const int* __restrict__ col_indices,
                                                              const float* __restrict__ values,
                                                              const float* __restrict__ B, float* __restrict__ partial)
 {
     const int sl = (int)(blockIdx.x / (unsigned)slice_blocks);
     const int bid = (int)blockIdx.x - sl * slice_blocks;
-    spmm_block<VEC, G, V, 4, R, true>(bid, M, N, col_tiles, bounds + (size_t)sl * M, bounds + (size_t)(sl + 1) * M,
-                                      col_indices, values, B, partial + (size_t)sl * M * N);
+    spmm_block<VEC, G, V, 4, R, true>(bid, M, N, col_tiles, tile_major, bounds + (size_t)sl * M,
+                                      bounds + (size_t)(sl + 1) * M, col_indices, values, B, partial + (size_t)sl * M * N);
 }
 
 // ---- host side --------------------------------------------------------------------------------------
 
 template <int VEC, int G, int V, int W, int R>
-static hipError_t launch_one(const SpmmArgs& x, hipStream_t stream)
+static hipError_t launch_one(const SpmmArgs& x, int tile_major, hipStream_t stream)
 {
     constexpr int TW = G * VEC * V;
     const int col_tiles = (x.N + TW - 1) / TW;
@@ -281,15 +299,15 @@ static hipError_t launch_one(const SpmmArgs& x, hipStream_t stream)
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     hipLaunchKernelGGL((spmm_kernel<VEC, G, V, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream, x.M, x.N,
-                       col_tiles, x.row_offsets, x.col_indices, x.values, x.B, x.C);
+                       col_tiles, tile_major, x.row_offsets, x.col_indices, x.values, x.B, x.C);
     return hipGetLastError();
 }
 
 template <int VEC, int G, int V>
-static hipError_t launch_wr(const SpmmArgs& x, int W, int R, hipStream_t stream)
+static hipError_t launch_wr(const SpmmArgs& x, int W, int R, int tile_major, hipStream_t stream)
 {
 #define DLSPM_WR(w_, r_) \
-    if (W == w_ && R == r_) return launch_one<VEC, G, V, w_, r_>(x, stream);
+    if (W == w_ && R == r_) return launch_one<VEC, G, V, w_, r_>(x, tile_major, stream);
     DLSPM_WR(4, 16)
     DLSPM_WR(4, 8)
     DLSPM_WR(4, 4)
@@ -304,12 +322,33 @@ static hipError_t launch_wr(const SpmmArgs& x, int W, int R, hipStream_t stream)
 }
 
 // Chooses the lane layout from N and the (W, R) split from the mean row length.
-SpmmShape spmm_choose(int M, int N, int nnz, bool vec4, bool rows_even)
+SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even)
 {
     SpmmShape s{};
     s.vec = vec4 ? 4 : 1;
+    // Several column tiles and a B that does not fit one XCD's 4 MiB L2: the tiles are worked through one after the
+    // other, each the widest whose K x TW slab of B still fits (measured on 8192 x 4096, N = 1024: 1460 us with tiles of
+    // 512, 930 us with 256; on 512 x 4608, N = 3136: 309 us against 273 us). DLSPM_TILE_MAJOR=0|1 and
+    // DLSPM_TILE_WIDTH=512|256|128 override both for tuning sweeps.
+    // (not for grids the device holds all at once: there the order cannot help, and 64 x 147 at N = 12544 lost 4 us)
+    s.tile_major = N > 512 && (long long)K * N * (long long)sizeof(float) > (4ll << 20) &&
+                           (long long)M * ((N + 511) / 512) >= 2048
+                       ? 1
+                       : 0;
+    if (const char* e = std::getenv("DLSPM_TILE_MAJOR")) s.tile_major = std::atoi(e) != 0 && N > 512 ? 1 : 0;
     if (vec4) {
-        if (N > 256) { s.G = 64; s.V = 2; }
+        if (N > 512 && s.tile_major) {
+            const long long slab512 = (long long)K * 512 * (long long)sizeof(float);
+            int tile = slab512 <= (4ll << 20) ? 512 : slab512 <= (8ll << 20) ? 256 : 128;
+            if (const char* e = std::getenv("DLSPM_TILE_WIDTH")) {
+                const int t = std::atoi(e);
+                if (t == 512 || t == 256 || t == 128) tile = t;
+            }
+            if (tile == 512) { s.G = 64; s.V = 2; }
+            else if (tile == 256) { s.G = 64; s.V = 1; }
+            else { s.G = 32; s.V = 1; }
+        }
+        else if (N > 256) { s.G = 64; s.V = 2; }
         else if (N > 128) { s.G = 64; s.V = 1; }
         else if (N > 64) { s.G = 32; s.V = 1; }
         else if (N > 32) { s.G = 16; s.V = 1; }
@@ -326,13 +365,13 @@ SpmmShape spmm_choose(int M, int N, int nnz, bool vec4, bool rows_even)
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream)
 {
     if (s.vec == 4) {
-        if (s.G == 64 && s.V == 1) return launch_wr<4, 64, 1>(x, s.W, s.R, stream);
-        if (s.G == 64 && s.V == 2) return launch_wr<4, 64, 2>(x, s.W, s.R, stream);
-        if (s.G == 32 && s.V == 1) return launch_wr<4, 32, 1>(x, s.W, s.R, stream);
-        if (s.G == 16 && s.V == 1) return launch_wr<4, 16, 1>(x, s.W, s.R, stream);
-        if (s.G == 8 && s.V == 1) return launch_wr<4, 8, 1>(x, s.W, s.R, stream);
+        if (s.G == 64 && s.V == 1) return launch_wr<4, 64, 1>(x, s.W, s.R, s.tile_major, stream);
+        if (s.G == 64 && s.V == 2) return launch_wr<4, 64, 2>(x, s.W, s.R, s.tile_major, stream);
+        if (s.G == 32 && s.V == 1) return launch_wr<4, 32, 1>(x, s.W, s.R, s.tile_major, stream);
+        if (s.G == 16 && s.V == 1) return launch_wr<4, 16, 1>(x, s.W, s.R, s.tile_major, stream);
+        if (s.G == 8 && s.V == 1) return launch_wr<4, 8, 1>(x, s.W, s.R, s.tile_major, stream);
     } else {
-        if (s.G == 8 && s.V == 1) return launch_wr<1, 8, 1>(x, s.W, s.R, stream);
+        if (s.G == 8 && s.V == 1) return launch_wr<1, 8, 1>(x, s.W, s.R, s.tile_major, stream);
     }
     return hipErrorInvalidValue;
 }
@@ -347,6 +386,7 @@ hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream
 // nonzeros as zeros, so the result is deterministic. No LDS, no barrier, no atomics.
 template <int VEC, int G, int V>
 __global__ __launch_bounds__(kFlatWaves * 64) void spmm_flat_kernel(int M, int N, int nnz, int chunk, int col_tiles,
+                                                                     int tile_major,
                                                                      const int* __restrict__ row_offsets,
                                                                      const int* __restrict__ col_indices,
                                                                      const float* __restrict__ values,
@@ -361,10 +401,20 @@ __global__ __launch_bounds__(kFlatWaves * 64) void spmm_flat_kernel(int M, int N
     const int g = lane % G;
     const int slot = lane / G;
     const long long id = (long long)blockIdx.x * kFlatWaves + w;
-    const int unit = (int)(id / col_tiles);
-    const int ct = (int)(id - (long long)unit * col_tiles);
+    // column tiles in the order the row-block kernel uses (tile-major: all units of tile 0, then of tile 1, ...)
+    int ct = 0, unit = (int)id;
+    if (col_tiles != 1) {
+        if (tile_major) {
+            const int units = (int)(((long long)nnz + chunk - 1) / chunk);
+            ct = (int)(id / units);
+            unit = (int)(id - (long long)ct * units);
+        } else {
+            unit = (int)(id / col_tiles);
+            ct = (int)(id - (long long)unit * col_tiles);
+        }
+    }
     const long long a64 = (long long)unit * chunk;
-    if (a64 >= nnz) return;  // wave-uniform
+    if (ct >= col_tiles || a64 >= nnz) return;  // wave-uniform
     const int a = (int)a64;
     const int b = (int)min((long long)nnz, a64 + chunk);
 
@@ -407,7 +457,7 @@ __global__ __launch_bounds__(kFlatWaves * 64) void spmm_flat_kernel(int M, int N
 }
 
 template <int VEC, int G, int V>
-static hipError_t launch_flat(const SpmmArgs& x, const FlatPlan& plan, float* partial, hipStream_t stream)
+static hipError_t launch_flat(const SpmmArgs& x, const FlatPlan& plan, int tile_major, float* partial, hipStream_t stream)
 {
     constexpr int TW = G * VEC * V;
     const int col_tiles = (x.N + TW - 1) / TW;
@@ -415,7 +465,7 @@ static hipError_t launch_flat(const SpmmArgs& x, const FlatPlan& plan, float* pa
     const long long blocks = (waves + kFlatWaves - 1) / kFlatWaves;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     hipLaunchKernelGGL((spmm_flat_kernel<VEC, G, V>), dim3((unsigned)blocks), dim3(kFlatWaves * 64), 0, stream, x.M, x.N,
-                       x.nnz, plan.chunk, col_tiles, x.row_offsets, x.col_indices, x.values, x.B, x.C, partial);
+                       x.nnz, plan.chunk, col_tiles, tile_major, x.row_offsets, x.col_indices, x.values, x.B, x.C, partial);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     return row_fixup_launch(x.M, x.N, plan.chunk, x.row_offsets, partial, x.C, stream);
@@ -425,13 +475,13 @@ hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPla
                             hipStream_t stream)
 {
     if (s.vec == 4) {
-        if (s.G == 64 && s.V == 1) return launch_flat<4, 64, 1>(x, plan, partial, stream);
-        if (s.G == 64 && s.V == 2) return launch_flat<4, 64, 2>(x, plan, partial, stream);
-        if (s.G == 32 && s.V == 1) return launch_flat<4, 32, 1>(x, plan, partial, stream);
-        if (s.G == 16 && s.V == 1) return launch_flat<4, 16, 1>(x, plan, partial, stream);
-        if (s.G == 8 && s.V == 1) return launch_flat<4, 8, 1>(x, plan, partial, stream);
+        if (s.G == 64 && s.V == 1) return launch_flat<4, 64, 1>(x, plan, s.tile_major, partial, stream);
+        if (s.G == 64 && s.V == 2) return launch_flat<4, 64, 2>(x, plan, s.tile_major, partial, stream);
+        if (s.G == 32 && s.V == 1) return launch_flat<4, 32, 1>(x, plan, s.tile_major, partial, stream);
+        if (s.G == 16 && s.V == 1) return launch_flat<4, 16, 1>(x, plan, s.tile_major, partial, stream);
+        if (s.G == 8 && s.V == 1) return launch_flat<4, 8, 1>(x, plan, s.tile_major, partial, stream);
     } else if (s.G == 8 && s.V == 1) {
-        return launch_flat<1, 8, 1>(x, plan, partial, stream);
+        return launch_flat<1, 8, 1>(x, plan, s.tile_major, partial, stream);
     }
     return hipErrorInvalidValue;
 }
@@ -439,8 +489,8 @@ hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPla
 // ---- column-sliced schedule ------------------------------------------------------------------------
 
 template <int VEC, int G, int V, int R>
-static hipError_t launch_sliced_r(const SpmmArgs& x, const SlicePlan& plan, const int* bounds, float* partial,
-                                  hipStream_t stream)
+static hipError_t launch_sliced_r(const SpmmArgs& x, const SlicePlan& plan, int tile_major, const int* bounds,
+                                  float* partial, hipStream_t stream)
 {
     constexpr int TW = G * VEC * V;
     const int col_tiles = (x.N + TW - 1) / TW;
@@ -449,20 +499,20 @@ static hipError_t launch_sliced_r(const SpmmArgs& x, const SlicePlan& plan, cons
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     hipLaunchKernelGGL((spmm_sliced_kernel<VEC, G, V, R>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M, x.N,
-                       col_tiles, (int)slice_blocks, bounds, x.col_indices, x.values, x.B, partial);
+                       col_tiles, tile_major, (int)slice_blocks, bounds, x.col_indices, x.values, x.B, partial);
     return hipGetLastError();
 }
 
 template <int VEC, int G, int V>
-static hipError_t launch_sliced(const SpmmArgs& x, const SlicePlan& plan, const int* bounds, float* partial,
-                                hipStream_t stream)
+static hipError_t launch_sliced(const SpmmArgs& x, const SlicePlan& plan, int tile_major, const int* bounds,
+                                float* partial, hipStream_t stream)
 {
     switch (plan.R) {
-        case 1: return launch_sliced_r<VEC, G, V, 1>(x, plan, bounds, partial, stream);
-        case 2: return launch_sliced_r<VEC, G, V, 2>(x, plan, bounds, partial, stream);
-        case 4: return launch_sliced_r<VEC, G, V, 4>(x, plan, bounds, partial, stream);
-        case 8: return launch_sliced_r<VEC, G, V, 8>(x, plan, bounds, partial, stream);
-        case 16: return launch_sliced_r<VEC, G, V, 16>(x, plan, bounds, partial, stream);
+        case 1: return launch_sliced_r<VEC, G, V, 1>(x, plan, tile_major, bounds, partial, stream);
+        case 2: return launch_sliced_r<VEC, G, V, 2>(x, plan, tile_major, bounds, partial, stream);
+        case 4: return launch_sliced_r<VEC, G, V, 4>(x, plan, tile_major, bounds, partial, stream);
+        case 8: return launch_sliced_r<VEC, G, V, 8>(x, plan, tile_major, bounds, partial, stream);
+        case 16: return launch_sliced_r<VEC, G, V, 16>(x, plan, tile_major, bounds, partial, stream);
     }
     return hipErrorInvalidValue;
 }
@@ -475,9 +525,9 @@ hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const Slice
     hipError_t e = slice_bounds_launch(x.M, x.K, plan.slices, x.row_offsets, x.col_indices, bounds, stream);
     if (e != hipSuccess) return e;
     e = hipErrorInvalidValue;
-    if (s.vec == 4 && s.G == 64 && s.V == 1) e = launch_sliced<4, 64, 1>(x, plan, bounds, partial, stream);
-    else if (s.vec == 4 && s.G == 64 && s.V == 2) e = launch_sliced<4, 64, 2>(x, plan, bounds, partial, stream);
-    else if (s.vec == 4 && s.G == 32 && s.V == 1) e = launch_sliced<4, 32, 1>(x, plan, bounds, partial, stream);
+    if (s.vec == 4 && s.G == 64 && s.V == 1) e = launch_sliced<4, 64, 1>(x, plan, s.tile_major, bounds, partial, stream);
+    else if (s.vec == 4 && s.G == 64 && s.V == 2) e = launch_sliced<4, 64, 2>(x, plan, s.tile_major, bounds, partial, stream);
+    else if (s.vec == 4 && s.G == 32 && s.V == 1) e = launch_sliced<4, 32, 1>(x, plan, s.tile_major, bounds, partial, stream);
     if (e != hipSuccess) return e;
     return slice_sum_launch((long long)x.M * x.N, plan.slices, partial, x.C, stream);
 }

@@ -68,6 +68,16 @@ def test_split_rule_and_the_even_rows_hint(dl):
     assert dl.describe_launch(dl.OP_FUSED, 300, 8192, 32, 300 * 7000)["W"] == 16  # few rows, very long: still sixteen
 
 
+def test_column_tiles_narrow_with_the_height_of_the_dense_operand(dl):
+    """Dense rows wider than 512 floats are covered by several column tiles, worked through one after the other: the
+    widest tile whose K x tile slab of B fits 4 MiB."""
+    nnz = 4096 * 100
+    for K, tile in ((512, 512), (2048, 512), (2049, 256), (4096, 256), (4097, 128), (1 << 16, 128)):
+        sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz)
+        assert sh["G"] * sh["vec"] * sh["V"] == tile and sh["col_tiles"] == -(-3136 // tile), (K, sh)
+    assert dl.describe_launch(dl.OP_SPMM, 4096, 1 << 16, 512, nnz)["col_tiles"] == 1  # one tile: nothing to order
+
+
 def test_column_sliced_schedule_rule(dl):
     """Slices of at most 2 MiB of gathered dense operand, only when the operand exceeds 4 MiB, the dense rows are wide
     and a row keeps at least 16 nonzeros per slice on average; the workspace then holds the boundaries and the

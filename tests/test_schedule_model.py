@@ -156,7 +156,9 @@ GPU_SPMM = [(300, 200, 256, "skewed", 0.15), (128, 512, 128, "uniform", 0.3), (2
             (100, 300, 32, "uniform", 0.05), (200, 512, 392, "uniform", 0.2), (90, 64, 130, "skewed", 0.3),
             (1000, 64, 16, "empty_rows", 0.05), (16, 700, 256, "full", 1.0), (4100, 300, 64, "skewed", 0.05),
             (64, 128, 49, "skewed", 0.2), (70, 90, 5, "uniform", 0.3), (10, 64, 1026, "uniform", 0.3),
-            (300, 80, 1, "skewed", 0.3), (50, 80, 3, "uniform", 0.3)]
+            (300, 80, 1, "skewed", 0.3), (50, 80, 3, "uniform", 0.3),
+            # several column tiles, narrower the taller B is: 256 columns from K > 2048, 128 from K > 4096
+            (40, 2100, 600, "skewed", 0.05), (30, 4200, 530, "uniform", 0.02), (700, 4100, 1030, "empty_rows", 0.01)]
 
 
 @pytest.mark.gpu
@@ -482,7 +484,8 @@ def column_slices(ro, ci, K, slices):
 
 
 SLICED_CASES = [("uniform", 300, 512, 128, 3), ("skewed", 1100, 700, 256, 2), ("empty_rows", 500, 300, 392, 4),
-                ("long_and_empty", 1500, 700, 128, 5), ("full", 40, 256, 96, 16), ("uniform", 70, 900, 513, 7)]
+                ("long_and_empty", 1500, 700, 128, 5), ("full", 40, 256, 96, 16), ("uniform", 70, 900, 513, 7),
+                ("skewed", 90, 4200, 530, 3)]
 
 
 @pytest.mark.gpu
