@@ -326,28 +326,31 @@ SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even)
 {
     SpmmShape s{};
     s.vec = vec4 ? 4 : 1;
-    // Several column tiles and a B that does not fit one XCD's 4 MiB L2: the tiles are worked through one after the
-    // other, each the widest whose K x TW slab of B still fits (measured on 8192 x 4096, N = 1024: 1460 us with tiles of
-    // 512, 930 us with 256; on 512 x 4608, N = 3136: 309 us against 273 us). DLSPM_TILE_MAJOR=0|1 and
-    // DLSPM_TILE_WIDTH=512|256|128 override both for tuning sweeps.
-    // (not for grids the device holds all at once: there the order cannot help, and 64 x 147 at N = 12544 lost 4 us)
-    s.tile_major = N > 512 && (long long)K * N * (long long)sizeof(float) > (4ll << 20) &&
-                           (long long)M * ((N + 511) / 512) >= 2048
-                       ? 1
-                       : 0;
-    if (const char* e = std::getenv("DLSPM_TILE_MAJOR")) s.tile_major = std::atoi(e) != 0 && N > 512 ? 1 : 0;
-    if (vec4) {
-        if (N > 512 && s.tile_major) {
+    // A B that does not fit one XCD's 4 MiB L2 is cut into column tiles that are worked through one after the other
+    // (tile-major grid order), each the widest of 512 / 256 / 128 columns whose K x tile slab still fits (measured on
+    // 8192 x 4096, N = 1024: 1460 us with tiles of 512, 930 us with 256; on 512 x 4608, N = 3136: 309 us against 273 us);
+    // also where one wave could cover the whole width (N <= 512). Not for grids the device holds all at once: there the
+    // order cannot help, and 64 x 147 at N = 12544 lost 4 us. DLSPM_TILE_MAJOR=0|1 and DLSPM_TILE_WIDTH=512|256|128
+    // override both for tuning sweeps.
+    int tile = 0;  // 0: one tile if a wave can cover N, else tiles of 512 in row-major order
+    if (vec4 && N > 128) {
+        bool on = (long long)K * N * (long long)sizeof(float) > (4ll << 20) && (long long)M * ((N + 511) / 512) >= 2048;
+        if (const char* e = std::getenv("DLSPM_TILE_MAJOR")) on = std::atoi(e) != 0;
+        if (on) {
             const long long slab512 = (long long)K * 512 * (long long)sizeof(float);
-            int tile = slab512 <= (4ll << 20) ? 512 : slab512 <= (8ll << 20) ? 256 : 128;
+            tile = slab512 <= (4ll << 20) ? 512 : slab512 <= (8ll << 20) ? 256 : 128;
             if (const char* e = std::getenv("DLSPM_TILE_WIDTH")) {
                 const int t = std::atoi(e);
                 if (t == 512 || t == 256 || t == 128) tile = t;
             }
-            if (tile == 512) { s.G = 64; s.V = 2; }
-            else if (tile == 256) { s.G = 64; s.V = 1; }
-            else { s.G = 32; s.V = 1; }
+            if (tile >= N) tile = 0;  // a single tile: nothing to order
         }
+    }
+    s.tile_major = tile > 0 ? 1 : 0;
+    if (vec4) {
+        if (tile == 512) { s.G = 64; s.V = 2; }
+        else if (tile == 256) { s.G = 64; s.V = 1; }
+        else if (tile == 128) { s.G = 32; s.V = 1; }
         else if (N > 256) { s.G = 64; s.V = 2; }
         else if (N > 128) { s.G = 64; s.V = 1; }
         else if (N > 64) { s.G = 32; s.V = 1; }

@@ -75,7 +75,13 @@ def test_column_tiles_narrow_with_the_height_of_the_dense_operand(dl):
     for K, tile in ((512, 512), (2048, 512), (2049, 256), (4096, 256), (4097, 128), (1 << 16, 128)):
         sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz)
         assert sh["G"] * sh["vec"] * sh["V"] == tile and sh["col_tiles"] == -(-3136 // tile), (K, sh)
-    assert dl.describe_launch(dl.OP_SPMM, 4096, 1 << 16, 512, nnz)["col_tiles"] == 1  # one tile: nothing to order
+    # the same where one wave could cover the whole width, once B exceeds the L2
+    sh = dl.describe_launch(dl.OP_SPMM, 4096, 8192, 256, nnz)
+    assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (128, 2)
+    sh = dl.describe_launch(dl.OP_SPMM, 4096, 4096, 512, nnz)
+    assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (256, 2)
+    assert dl.describe_launch(dl.OP_SPMM, 4096, 4096, 256, nnz)["col_tiles"] == 1   # 4 MiB: fits
+    assert dl.describe_launch(dl.OP_SPMM, 1024, 8192, 256, nnz)["col_tiles"] == 1   # a grid the device holds at once
 
 
 def test_column_sliced_schedule_rule(dl):
@@ -89,18 +95,19 @@ def test_column_sliced_schedule_rule(dl):
     assert dl.describe_slices(dl.OP_FUSED, M, K, 64, nnz)[0] == 0       # 4 MiB, but narrow dense rows
     assert dl.describe_slices(dl.OP_FUSED, M, K // 2, 128, nnz)[0] == 2 # 4 MiB just fills the L2: in two for long rows
     assert dl.describe_slices(dl.OP_FUSED, M, K // 2, 128, M * 400)[0] == 0  # ... not for 200 nonzeros per slice
-    assert dl.describe_slices(dl.OP_SPMM, M, K, 256, nnz)[0] == 4       # B: 8 MiB
-    assert dl.describe_slices(dl.OP_SPMM, M, K, 200, nnz)[0] == 4       # 6.25 MiB
-    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, nnz)[0] == 16      # 128 MiB: the most slices there are
-    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, M * 100)[0] == 6   # ... but a row keeps 16 nonzeros per slice
-    assert dl.describe_slices(dl.OP_SPMM, M, K, 128, nnz)[0] == 2       # 4 MiB, 400 nonzeros per slice
-    assert dl.describe_slices(dl.OP_SPMM, M, K, 128, M * 400)[0] == 0   # 4 MiB, 200 nonzeros per slice
+    # SpMM cuts a B beyond 4 MiB into column tiles first (8192 x 128 floats here: 4 MiB per tile), and slices the tile
+    assert dl.describe_slices(dl.OP_SPMM, M, K, 256, nnz)[0] == 2       # 4 MiB per tile, 400 nonzeros per slice
+    assert dl.describe_slices(dl.OP_SPMM, M, K, 256, M * 400)[0] == 0   # ... 200 nonzeros per slice: not at exactly 4 MiB
+    assert dl.describe_slices(dl.OP_SPMM, M, K, 128, nnz)[0] == 2       # one tile of 4 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, K, 100, nnz)[0] == 0       # 3.1 MiB: fits
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, nnz)[0] == 8   # 32768 x 128 floats per tile: 16 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 20, 32, nnz)[0] == 0  # narrow dense rows: not built for them
-    assert dl.describe_slices(dl.OP_SPMM, M, K, 256, M * 70)[0] == 4    # 70 nonzeros per row: four slices of 17
-    assert dl.describe_slices(dl.OP_SPMM, M, K, 256, M * 40)[0] == 0    # 40 per row, 0.33 M nonzeros: too small
-    assert dl.describe_slices(dl.OP_SPMM, 4 * M, K, 256, 4 * M * 40)[0] == 2  # 1.3 M nonzeros: two slices of 20
-    assert dl.describe_slices(dl.OP_SPMM, 4 * M, K, 256, 4 * M * 30)[0] == 0  # 30 per row: not even two
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 70)[0] == 4    # 70 nonzeros per row: four slices of 17
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 40)[0] == 0    # 40 per row, 0.33 M nonzeros: too small
+    assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 40)[0] == 2  # 1.3 M nonzeros: two slices of 20
+    assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 30)[0] == 0  # 30 per row: not even two
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, nnz)[0] == 16      # 64 MiB per tile: the most slices there are
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, M * 100)[0] == 6   # ... but a row keeps 16 nonzeros per slice
     assert dl.describe_slices(dl.OP_SDDMM, M, K, 256, nnz)[0] == 4      # rhs: 8 MiB; only the boundaries need memory
     assert dl.workspace_bytes(dl.OP_SDDMM, M, K, 256, nnz) == -(-5 * M * 4 // 256) * 256
     assert dl.describe_slices(dl.OP_SDDMM, M, K, 100, nnz)[0] == 0 and dl.workspace_bytes(dl.OP_SDDMM, M, K, 100, nnz) == 0
