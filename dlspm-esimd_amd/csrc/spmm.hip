@@ -14,6 +14,10 @@
 //   * rows finished inside one wave are stored straight to C; rows shared by several waves leave
 //     per-wave partial sums in LDS which are added in wave order after one barrier, so the result does
 //     not depend on timing (no atomics, no pre-zeroed output); rows without nonzeros are written as 0.
+// Two more schedules reuse these pieces when the caller passes a workspace: the flat schedule (every wave
+// owns a fixed run of nonzeros of the whole matrix; for very uneven rows) and the column-sliced schedule
+// (the same workgroups on one range of columns of A after the other; for a B larger than one L2), and a
+// B larger than one L2 is always cut into column tiles that the grid works through one after the other.
 #include <cstdlib>
 
 #include "common.hpp"
