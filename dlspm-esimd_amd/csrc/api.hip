@@ -91,21 +91,27 @@ static FlatPlan sddmm_flat_plan(int M, int nnz, int D)
 constexpr long long kSliceMinOperand = 4ll << 20;  // bytes gathered from; above this the operand is sliced
 constexpr long long kSliceBytes = 2ll << 20;       // bytes of it per slice
 constexpr int kSliceMaxSlices = 16;
-constexpr int kSliceMinRow = 16;  // mean nonzeros of a row inside one slice; fewer slices rather than shorter shares
+constexpr int kSliceMinRow = 16;  // least mean nonzeros of a row inside one slice; fewer slices rather than shorter shares
 constexpr int kSliceMinRowAtL2 = 256;  // the same for an operand of exactly kSliceMinOperand bytes
 
 SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial_width, int G, long long col_tiles,
                      int slots, int min_blocks)
 {
     SlicePlan p{0, 1, 0, 0};
-    if (M <= 0 || K <= 0 || nnz <= 0 || width <= 0 || G < kFlatMinLanes) return p;
+    if (M <= 0 || K <= 0 || nnz <= 0 || width <= 0 || G <= 0) return p;  // G == 0: no sliced kernel for this layout
     int force = -1;
     if (const char* e = std::getenv("DLSPM_SLICES")) force = std::atoi(e);
     const long long bytes = (long long)K * width * (long long)sizeof(float) * operands;
     long long slices = (bytes + kSliceBytes - 1) / kSliceBytes;
     if (slices > kSliceMaxSlices) slices = kSliceMaxSlices;
-    // slices that leave a row its minimum share; an operand that just fills the L2 is worth slicing for long rows only
-    const int min_row = bytes > kSliceMinOperand ? kSliceMinRow : kSliceMinRowAtL2;
+    // Slices that leave a row its minimum share: 16 nonzeros per slice for dense rows of 256 floats and more, in
+    // inverse proportion more for narrower ones (measured with D = 64: 28 per slice lost 20 %, 48 and more gained; with
+    // D = 32: 48 lost, 164 gained). An operand that just fills the L2 is worth slicing for long rows only, and only
+    // for dense rows of at least 128 floats (narrower: 327 nonzeros per slice still lost 10 %).
+    const bool just_fills = bytes <= kSliceMinOperand;
+    const int per_width = 4096 / width;
+    const int min_row = just_fills ? kSliceMinRowAtL2 : per_width > kSliceMinRow ? per_width : kSliceMinRow;
+    if (just_fills && width < 128) slices = 0;
     const long long fit = (long long)nnz / ((long long)min_row * M);
     if (slices > fit) slices = fit;
     const bool by_rule = bytes >= kSliceMinOperand && nnz >= kFlatMinNnz && slices >= 2;
@@ -224,12 +230,12 @@ static SlicePlan spmm_slice_plan(int M, int K, int N, int nnz, const SpmmShape& 
 static SlicePlan fused_slice_plan(int M, int K, int D, int nnz, const FusedShape& s)
 {
     const int tw = s.G * s.vec * s.V;
-    const bool built = s.vec == 4 && s.DS > 0 && tw >= D;  // the widths the sliced kernels are built for (65 .. 512)
+    const bool built = s.vec == 4 && s.G1 == 8 && s.DS > 0 && tw >= D;  // the widths the sliced kernels are built for (17 .. 512)
     return slice_plan(M, K, D, nnz, 2, D, built ? s.G : 0, 1, kWave / s.G, 512);
 }
 static SlicePlan sddmm_slice_plan(int M, int K, int D, int nnz, const SddmmShape& s)
 {
-    const bool built = s.vec == 4 && s.G1 == 8 && s.DS >= 4;  // 64 < D <= 512
+    const bool built = s.vec == 4 && s.G1 == 8 && s.DS >= 1;  // 16 < D <= 512
     return slice_plan(M, K, D, nnz, 1, 0, built ? kWave : 0, 1, kWave / s.G1, 512);
 }
 

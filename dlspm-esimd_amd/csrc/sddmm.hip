@@ -323,7 +323,7 @@ static hipError_t launch_sliced(const SddmmArgs& x, const SlicePlan& plan, const
     return hipErrorInvalidValue;
 }
 
-// built for 64 < D <= 512 (G1 = 8 with 4, 8 or 16 accesses per lane)
+// built for 16 < D <= 512 (G1 = 8 with 1 to 16 accesses per lane)
 hipError_t sddmm_sliced_launch(const SddmmArgs& x, const SddmmShape& s, const SlicePlan& plan, void* workspace,
                                hipStream_t stream)
 {
@@ -333,6 +333,8 @@ hipError_t sddmm_sliced_launch(const SddmmArgs& x, const SddmmShape& s, const Sl
     if (s.vec == 4 && s.G1 == 8 && s.DS == 4) return launch_sliced<4, 8, 4>(x, plan, bounds, stream);
     if (s.vec == 4 && s.G1 == 8 && s.DS == 8) return launch_sliced<4, 8, 8>(x, plan, bounds, stream);
     if (s.vec == 4 && s.G1 == 8 && s.DS == 16) return launch_sliced<4, 8, 16>(x, plan, bounds, stream);
+    if (s.vec == 4 && s.G1 == 8 && s.DS == 2) return launch_sliced<4, 8, 2>(x, plan, bounds, stream);
+    if (s.vec == 4 && s.G1 == 8 && s.DS == 1) return launch_sliced<4, 8, 1>(x, plan, bounds, stream);
     return hipErrorInvalidValue;
 }
 

@@ -535,6 +535,8 @@ hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const Slice
     if (s.vec == 4 && s.G == 64 && s.V == 1) e = launch_sliced<4, 64, 1>(x, plan, s.tile_major, bounds, partial, stream);
     else if (s.vec == 4 && s.G == 64 && s.V == 2) e = launch_sliced<4, 64, 2>(x, plan, s.tile_major, bounds, partial, stream);
     else if (s.vec == 4 && s.G == 32 && s.V == 1) e = launch_sliced<4, 32, 1>(x, plan, s.tile_major, bounds, partial, stream);
+    else if (s.vec == 4 && s.G == 16 && s.V == 1) e = launch_sliced<4, 16, 1>(x, plan, s.tile_major, bounds, partial, stream);
+    else if (s.vec == 4 && s.G == 8 && s.V == 1) e = launch_sliced<4, 8, 1>(x, plan, s.tile_major, bounds, partial, stream);
     if (e != hipSuccess) return e;
     return slice_sum_launch((long long)x.M * x.N, plan.slices, partial, x.C, stream);
 }

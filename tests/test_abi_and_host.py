@@ -92,7 +92,10 @@ def test_column_sliced_schedule_rule(dl):
     nnz = M * 800
     assert dl.describe_slices(dl.OP_FUSED, M, K, 128, nnz)[0] == 4      # Kmat + V: 8 MiB
     assert dl.describe_slices(dl.OP_FUSED, M, K, 256, nnz)[0] == 8      # 16 MiB
-    assert dl.describe_slices(dl.OP_FUSED, M, K, 64, nnz)[0] == 0       # 4 MiB, but narrow dense rows
+    assert dl.describe_slices(dl.OP_FUSED, M, K, 64, nnz)[0] == 0       # 4 MiB of narrow dense rows: left alone
+    assert dl.describe_slices(dl.OP_FUSED, M, 4 * K, 64, nnz)[0] == 8   # sparse attention over 32768 keys, D = 64: 16 MiB
+    assert dl.describe_slices(dl.OP_FUSED, M, 4 * K, 64, M * 200)[0] == 3   # ... a row keeps 64 nonzeros per slice at D = 64
+    assert dl.describe_slices(dl.OP_FUSED, M, 4 * K, 16, nnz)[0] == 0   # D <= 16: not built for it
     assert dl.describe_slices(dl.OP_FUSED, M, K // 2, 128, nnz)[0] == 2 # 4 MiB just fills the L2: in two for long rows
     assert dl.describe_slices(dl.OP_FUSED, M, K // 2, 128, M * 400)[0] == 0  # ... not for 200 nonzeros per slice
     # SpMM cuts a B beyond 4 MiB into column tiles first (8192 x 128 floats here: 4 MiB per tile), and slices the tile
@@ -101,13 +104,17 @@ def test_column_sliced_schedule_rule(dl):
     assert dl.describe_slices(dl.OP_SPMM, M, K, 128, nnz)[0] == 2       # one tile of 4 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, K, 100, nnz)[0] == 0       # 3.1 MiB: fits
     assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, nnz)[0] == 8   # 32768 x 128 floats per tile: 16 MiB
-    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 20, 32, nnz)[0] == 0  # narrow dense rows: not built for them
-    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 70)[0] == 4    # 70 nonzeros per row: four slices of 17
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 16, 32, nnz)[0] == 4  # narrow dense rows, very tall B: 8 MiB
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 16, 32, M * 300)[0] == 2  # ... 128 nonzeros per slice at N = 32
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 20, 3, nnz)[0] == 0   # fewer than four columns: not built for them
+    # ... in tiles of 128 columns a row keeps at least 32 nonzeros per slice
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 140)[0] == 4   # 140 nonzeros per row: four slices of 35
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 70)[0] == 2    # 70 per row: two
     assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 40)[0] == 0    # 40 per row, 0.33 M nonzeros: too small
-    assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 40)[0] == 2  # 1.3 M nonzeros: two slices of 20
-    assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 30)[0] == 0  # 30 per row: not even two
+    assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 64)[0] == 2  # 2.1 M nonzeros, 64 per row: two slices
+    assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 60)[0] == 0  # 60 per row: not even two
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, nnz)[0] == 16      # 64 MiB per tile: the most slices there are
-    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, M * 100)[0] == 6   # ... but a row keeps 16 nonzeros per slice
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, M * 100)[0] == 3   # ... but a row keeps 32 nonzeros per slice
     assert dl.describe_slices(dl.OP_SDDMM, M, K, 256, nnz)[0] == 4      # rhs: 8 MiB; only the boundaries need memory
     assert dl.workspace_bytes(dl.OP_SDDMM, M, K, 256, nnz) == -(-5 * M * 4 // 256) * 256
     assert dl.describe_slices(dl.OP_SDDMM, M, K, 100, nnz)[0] == 0 and dl.workspace_bytes(dl.OP_SDDMM, M, K, 100, nnz) == 0

@@ -485,7 +485,8 @@ def column_slices(ro, ci, K, slices):
 
 SLICED_CASES = [("uniform", 300, 512, 128, 3), ("skewed", 1100, 700, 256, 2), ("empty_rows", 500, 300, 392, 4),
                 ("long_and_empty", 1500, 700, 128, 5), ("full", 40, 256, 96, 16), ("uniform", 70, 900, 513, 7),
-                ("skewed", 90, 4200, 530, 3)]
+                ("skewed", 90, 4200, 530, 3), ("skewed", 300, 400, 48, 3), ("uniform", 200, 300, 20, 4),
+                ("empty_rows", 400, 200, 7, 2)]
 
 
 @pytest.mark.gpu
@@ -532,7 +533,8 @@ def test_gpu_sliced_spmm_equals_model_bit_for_bit(model, dl, oracle, monkeypatch
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind,M,K,D,slices", [("uniform", 300, 512, 128, 3), ("skewed", 700, 600, 256, 2),
                                                ("long_and_empty", 900, 600, 100, 4), ("empty_rows", 200, 300, 512, 5),
-                                               ("uniform", 150, 400, 200, 16)])
+                                               ("uniform", 150, 400, 200, 16), ("skewed", 500, 700, 64, 3),
+                                               ("uniform", 300, 200, 24, 4)])
 def test_gpu_sliced_fused_equals_model_bit_for_bit(model, dl, oracle, monkeypatch, kind, M, K, D, slices):
     import torch
 
@@ -601,7 +603,8 @@ def test_gpu_sliced_schedule_does_not_need_ascending_columns(dl, oracle, monkeyp
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind,M,K,D,slices", [("uniform", 300, 512, 128, 3), ("skewed", 700, 600, 256, 2),
                                                ("long_and_empty", 900, 600, 100, 4), ("empty_rows", 200, 300, 512, 5),
-                                               ("full", 60, 256, 65, 16)])
+                                               ("full", 60, 256, 65, 16), ("skewed", 500, 700, 64, 3),
+                                               ("uniform", 300, 200, 20, 4)])
 def test_gpu_sliced_sddmm_gives_the_same_bits(dl, oracle, monkeypatch, kind, M, K, D, slices):
     """Every SDDMM result is one dot product computed by one lane group in a fixed order, whatever the schedule: the
     column-sliced call must reproduce the plain call bit for bit, and leave no slot unwritten."""
