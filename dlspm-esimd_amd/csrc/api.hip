@@ -86,8 +86,9 @@ static FlatPlan sddmm_flat_plan(int M, int nnz, int D)
 // XCD's 4 MiB L2; the slices are cut to 2 MiB of them. Measured on MI355X (8192 x 8192, 30 % dense, lognormal rows,
 // sigma 0.6; row-block / flat / sliced): fused, D = 128 (8 MiB of Kmat and V): 1429 / 1374 / 676 us, D = 256 (16 MiB):
 // 4024 / 3946 / 1328 us; SpMM, N = 256: 1472 / 1390 / 685 us; slices of 4 MiB instead: 769, 1441, 803 us. Operands of
-// exactly 4 MiB (8192 x 128 floats) gain 13-16 % at 10-30 % density and lose 5 % at 3 %: sliced in two for long rows only. Like the flat schedule only from half a
-// million nonzeros on (two more launches). DLSPM_SLICES=0 switches it off, DLSPM_SLICES=n forces n slices (tuning, tests).
+// exactly 4 MiB (8192 x 128 floats) gain 13-16 % at 10-30 % density and lose 5 % at 3 %: sliced in two for long rows
+// only. Like the flat schedule only from half a million nonzeros on (two more launches). DLSPM_SLICES=0 switches it
+// off, DLSPM_SLICES=n forces n slices (tuning, tests).
 constexpr long long kSliceMinOperand = 4ll << 20;  // bytes gathered from; above this the operand is sliced
 constexpr long long kSliceBytes = 2ll << 20;       // bytes of it per slice
 constexpr int kSliceMaxSlices = 16;

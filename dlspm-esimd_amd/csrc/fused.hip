@@ -513,11 +513,16 @@ hipError_t fused_sliced_launch(const FusedArgs& x, const FusedShape& s, const Sl
     hipError_t e = slice_bounds_launch(x.M, x.K, plan.slices, x.row_offsets, x.col_indices, bounds, stream);
     if (e != hipSuccess) return e;
     e = hipErrorInvalidValue;
-    if (s.vec == 4 && s.G1 == 8 && s.DS == 4 && s.G == 32 && s.V == 1) e = launch_sliced<4, 8, 4, 32, 1>(x, plan, bounds, partial, stream);
-    else if (s.vec == 4 && s.G1 == 8 && s.DS == 8 && s.G == 64 && s.V == 1) e = launch_sliced<4, 8, 8, 64, 1>(x, plan, bounds, partial, stream);
-    else if (s.vec == 4 && s.G1 == 8 && s.DS == 16 && s.G == 64 && s.V == 2) e = launch_sliced<4, 8, 16, 64, 2>(x, plan, bounds, partial, stream);
-    else if (s.vec == 4 && s.G1 == 8 && s.DS == 2 && s.G == 16 && s.V == 1) e = launch_sliced<4, 8, 2, 16, 1>(x, plan, bounds, partial, stream);
-    else if (s.vec == 4 && s.G1 == 8 && s.DS == 1 && s.G == 8 && s.V == 1) e = launch_sliced<4, 8, 1, 8, 1>(x, plan, bounds, partial, stream);
+    // built for 16 < D <= 512: the layouts fused_choose gives those widths
+#define DLSPM_SLICED(g1_, ds_, g_, v_)                                                \
+    if (s.vec == 4 && s.G1 == g1_ && s.DS == ds_ && s.G == g_ && s.V == v_)           \
+        e = launch_sliced<4, g1_, ds_, g_, v_>(x, plan, bounds, partial, stream);
+    DLSPM_SLICED(8, 1, 8, 1)
+    DLSPM_SLICED(8, 2, 16, 1)
+    DLSPM_SLICED(8, 4, 32, 1)
+    DLSPM_SLICED(8, 8, 64, 1)
+    DLSPM_SLICED(8, 16, 64, 2)
+#undef DLSPM_SLICED
     if (e != hipSuccess) return e;
     return slice_sum_launch((long long)x.M * x.D, plan.slices, partial, x.O, stream);
 }

@@ -532,11 +532,15 @@ hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const Slice
     hipError_t e = slice_bounds_launch(x.M, x.K, plan.slices, x.row_offsets, x.col_indices, bounds, stream);
     if (e != hipSuccess) return e;
     e = hipErrorInvalidValue;
-    if (s.vec == 4 && s.G == 64 && s.V == 1) e = launch_sliced<4, 64, 1>(x, plan, s.tile_major, bounds, partial, stream);
-    else if (s.vec == 4 && s.G == 64 && s.V == 2) e = launch_sliced<4, 64, 2>(x, plan, s.tile_major, bounds, partial, stream);
-    else if (s.vec == 4 && s.G == 32 && s.V == 1) e = launch_sliced<4, 32, 1>(x, plan, s.tile_major, bounds, partial, stream);
-    else if (s.vec == 4 && s.G == 16 && s.V == 1) e = launch_sliced<4, 16, 1>(x, plan, s.tile_major, bounds, partial, stream);
-    else if (s.vec == 4 && s.G == 8 && s.V == 1) e = launch_sliced<4, 8, 1>(x, plan, s.tile_major, bounds, partial, stream);
+    // built for every dwordx4 layout spmm_choose gives (N >= 4)
+#define DLSPM_SLICED(g_, v_) \
+    if (s.vec == 4 && s.G == g_ && s.V == v_) e = launch_sliced<4, g_, v_>(x, plan, s.tile_major, bounds, partial, stream);
+    DLSPM_SLICED(64, 2)
+    DLSPM_SLICED(64, 1)
+    DLSPM_SLICED(32, 1)
+    DLSPM_SLICED(16, 1)
+    DLSPM_SLICED(8, 1)
+#undef DLSPM_SLICED
     if (e != hipSuccess) return e;
     return slice_sum_launch((long long)x.M * x.N, plan.slices, partial, x.C, stream);
 }
