@@ -141,7 +141,8 @@ def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None):
 
 def sddmm(row_offsets, col_indices, lhs, rhs, out=None, workspace=None):
     """out[j] = <lhs[i], rhs[col[j]]> for each CSR slot j of row i, on the current stream.
-    `workspace`: None or ROWS_EVEN (SDDMM needs no memory)."""
+    `workspace`: None, ROWS_EVEN, or a GPU tensor of workspace_bytes(OP_SDDMM, ...) bytes (the slice boundaries of the
+    column-sliced schedule; 0 bytes where that schedule does not apply)."""
     import torch
 
     M = row_offsets.numel() - 1
