@@ -41,6 +41,7 @@ EXPORTS = (
     "dlspm_describe_launch",
     "dlspm_describe_launch_rows",
     "dlspm_describe_slices",
+    "dlspm_workspace_advice",
     "dlspm_csr_row_stats",
     "dlspm_status_string",
     "dlspm_last_hip_error",
@@ -80,6 +81,8 @@ def lib() -> ctypes.CDLL:
         L.dlspm_describe_launch_rows.restype = ci
         L.dlspm_describe_slices.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci), ctypes.POINTER(ci)]
         L.dlspm_describe_slices.restype = ci
+        L.dlspm_workspace_advice.argtypes = [ci, ci, ci, ci, ci, ci]
+        L.dlspm_workspace_advice.restype = ci
         L.dlspm_describe_launch.restype = ci
         L.dlspm_csr_row_stats.argtypes = [ci, vp, vp, ctypes.POINTER(ci), ctypes.POINTER(ci)]
         L.dlspm_csr_row_stats.restype = ci
@@ -197,6 +200,14 @@ def describe_slices(op: int, M: int, K: int, N: int, nnz: int) -> tuple:
     if st != OK:
         raise DlspmError(st, "dlspm_describe_slices")
     return a.value, b.value
+
+
+PASS_NULL, PASS_ROWS_EVEN, PASS_WORKSPACE = 0, 1, 2
+
+
+def workspace_advice(op: int, M: int, K: int, N: int, nnz: int, max_row_len: int = -1) -> int:
+    """What to pass as `workspace` (PASS_NULL / PASS_ROWS_EVEN / PASS_WORKSPACE) given the longest row (-1: unknown)."""
+    return int(lib().dlspm_workspace_advice(op, M, K, N, nnz, max_row_len))
 
 
 def workspace_bytes(op: int, M: int, K: int, N: int, nnz: int) -> int:

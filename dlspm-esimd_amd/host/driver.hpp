@@ -213,12 +213,8 @@ struct Options {
     double tol = 1e-4;  // relative Frobenius error allowed between the kernel and the check kernel
 };
 
-// What this run passes as `workspace`, from the sizes and one look at the row lengths (dlspm_csr_row_stats):
-//   * the memory the library asks for when the column-sliced schedule applies (dense operands of 4 MiB or more: faster
-//     for every row-length distribution measured, except even rows at two slices), or when the rows are uneven enough for the flat schedule to pay
-//     (measured: from lognormal sigma ~1 on, i.e. a longest row of at least four times the mean);
-//   * the constant DLSPM_ROWS_EVEN when no row is longer than one and a half times the mean;
-//   * nothing otherwise.
+// What this run passes as `workspace`: what dlspm_workspace_advice says for the sizes and the longest row
+// (dlspm_csr_row_stats, one look per matrix) -- device memory, the constant DLSPM_ROWS_EVEN, or nothing.
 struct WorkspaceChoice {
     size_t bytes = 0;        // device memory to allocate and pass
     bool rows_even = false;  // pass DLSPM_ROWS_EVEN instead
@@ -230,20 +226,16 @@ inline WorkspaceChoice workspace_to_pass(const Options& opt, int op, int M, int 
     WorkspaceChoice c;
     if (opt.workspace == Options::kNever || M <= 0 || nnz <= 0) return c;
     const size_t want = dlspm_workspace_bytes(op, M, K, width, nnz);
-    int slices = 0;
-    if (dlspm_describe_slices(op, M, K, width, nnz, &slices, nullptr) != DLSPM_OK) throw std::runtime_error("dlspm_describe_slices failed");
     int longest = 0, empty = 0;
     if (dlspm_csr_row_stats(M, row_offsets_dev, nullptr, &longest, &empty) != DLSPM_OK) throw std::runtime_error("dlspm_csr_row_stats failed");
-    const double mean = (double)nnz / M;
-    const bool uneven = longest >= 4.0 * mean, even = longest <= 1.5 * mean;
-    // even rows and an operand that only just exceeds the L2 (two slices): one whole row per wave does as well or better
-    // (measured: SpMM and fused 5-9 % faster at exactly 4 MiB, equal at 8 MiB; SDDMM 2-12 % slower)
-    const bool sliced = slices > 0 && !(even && slices <= 2 && op != DLSPM_OP_SDDMM);
-    if (opt.workspace == Options::kAlways || sliced || (uneven && want > 0 && slices == 0)) c.bytes = want;
-    else c.rows_even = even;
-    std::printf("rows: longest %d, mean %.1f, empty %d -> %s\n", longest, mean, empty,
+    const int advice = dlspm_workspace_advice(op, M, K, width, nnz, longest);
+    int slices = 0;
+    (void)dlspm_describe_slices(op, M, K, width, nnz, &slices, nullptr);
+    if (opt.workspace == Options::kAlways || advice == DLSPM_PASS_WORKSPACE) c.bytes = want;
+    else c.rows_even = advice == DLSPM_PASS_ROWS_EVEN;
+    std::printf("rows: longest %d, mean %.1f, empty %d -> %s\n", longest, (double)nnz / M, empty,
                 opt.workspace == Options::kAlways ? "workspace passed (--workspace)"
-                : sliced                          ? "dense operands beyond one L2, workspace passed (column-sliced schedule)"
+                : c.bytes && slices > 0           ? "dense operands beyond one L2, workspace passed (column-sliced schedule)"
                 : c.bytes                         ? "uneven, workspace passed (flat schedule)"
                 : c.rows_even                     ? "even, DLSPM_ROWS_EVEN passed"
                                                   : "nothing passed");

@@ -147,6 +147,20 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
 int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_row_len, int* empty_rows);
 
 /*
+ * What to pass as `workspace` for a matrix of these sizes whose longest row has max_row_len nonzeros (from
+ * dlspm_csr_row_stats, or known to the caller): DLSPM_PASS_NULL, DLSPM_PASS_ROWS_EVEN (the constant DLSPM_ROWS_EVEN)
+ * or DLSPM_PASS_WORKSPACE (dlspm_workspace_bytes() bytes of device memory). It holds the measured rules in one place:
+ * the memory where the column-sliced schedule applies (except even rows at two slices in SpMM and the fused op) or
+ * where the longest row is at least four times the mean and the flat schedule applies; the constant where the
+ * longest row is at most one and a half times the mean; NULL otherwise. Host-only; a negative max_row_len means
+ * "unknown" and gives the memory only for the column-sliced schedule. No counterpart in the reference.
+ */
+#define DLSPM_PASS_NULL       0
+#define DLSPM_PASS_ROWS_EVEN  1
+#define DLSPM_PASS_WORKSPACE  2
+int dlspm_workspace_advice(int op, int M, int K, int N_or_D, int nnz, int max_row_len);
+
+/*
  * Launch shape the library would use for these sizes, for tuning reports and for host-side models of the
  * schedule (the reference's SpmmEsimdCPU / FusedEsimdCPU, SPMM/spmm-esimd-v1.cpp:83-169 and
  * FUSED/fused.cpp:93-216, play that role for its kernels). Host-only, never touches the device.

@@ -126,6 +126,30 @@ def test_column_sliced_schedule_rule(dl):
     assert dl.workspace_bytes(dl.OP_SPMM, M, K, 100, nnz) == dl.describe_launch(dl.OP_SPMM, M, K, 100, nnz)["flat_units"] * 2 * 100 * 4
 
 
+def test_workspace_advice(dl):
+    """One host call holds the measured rules for what to pass as `workspace`."""
+    M = K = 8192
+    nnz = M * 800
+    mean = nnz // M
+    A = dl.workspace_advice
+    # column-sliced schedule (fused, 8 MiB of Kmat and V: four slices): the memory, whatever the rows
+    for longest in (-1, mean, 3 * mean, 10 * mean):
+        assert A(dl.OP_FUSED, M, K, 128, nnz, longest) == dl.PASS_WORKSPACE
+    # two slices (4 MiB, long rows): even rows rather take the hint in SpMM and the fused op, never in SDDMM
+    assert dl.describe_slices(dl.OP_SPMM, M, K, 128, nnz)[0] == 2
+    assert A(dl.OP_SPMM, M, K, 128, nnz, mean + 10) == dl.PASS_ROWS_EVEN
+    assert A(dl.OP_SPMM, M, K, 128, nnz, 3 * mean) == dl.PASS_WORKSPACE
+    assert A(dl.OP_SDDMM, M, K, 128, nnz, mean + 10) == dl.PASS_WORKSPACE
+    # no slices: the memory for rows at least four times the mean where the flat schedule applies, the hint for even rows
+    assert A(dl.OP_SPMM, M, 2048, 128, nnz, 4 * mean) == dl.PASS_WORKSPACE
+    assert A(dl.OP_SPMM, M, 2048, 128, nnz, 3 * mean) == dl.PASS_NULL
+    assert A(dl.OP_SPMM, M, 2048, 128, nnz, -1) == dl.PASS_NULL
+    assert A(dl.OP_SPMM, M, 2048, 128, nnz, int(1.5 * mean)) == dl.PASS_ROWS_EVEN
+    assert A(dl.OP_SPMM, 2048, 512, 256, 105687, 300) == dl.PASS_NULL      # small and uneven: nothing helps
+    assert A(dl.OP_SDDMM, M, 2048, 128, nnz, 10 * mean) == dl.PASS_NULL    # SDDMM's flat schedule needs no memory
+    assert A(dl.OP_SPMM, 0, 0, 0, 0, 0) == dl.PASS_NULL and A(7, M, K, 128, nnz, mean) == dl.PASS_NULL
+
+
 def test_library_exports_every_declared_symbol(dl):
     lib = ctypes.CDLL(dl.LIB_PATH)
     for name in declared_functions():
