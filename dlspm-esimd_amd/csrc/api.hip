@@ -257,9 +257,10 @@ int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int
     const bool vec4 = N >= 4;  // dwordx4 accesses need only dword alignment
     const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C};
     const bool even = workspace == DLSPM_ROWS_EVEN;  // a constant that says something about the rows, not memory
-    const SpmmShape shape = spmm_choose(M, K, N, nnz, vec4, even);
+    const bool memory = !even && workspace != nullptr && workspace_bytes > 0;
+    const SpmmShape shape = spmm_choose(M, K, N, nnz, vec4, even, !memory);
     hipError_t e;
-    if (!even && workspace != nullptr && workspace_bytes > 0) {
+    if (memory) {
         const SlicePlan sliced = spmm_slice_plan(M, K, N, nnz, shape);
         const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(M, nnz, N, shape.G);
         if (workspace_bytes < (sliced.slices > 0 ? sliced.bytes : plan.bytes)) return DLSPM_E_WORKSPACE;
@@ -346,7 +347,7 @@ size_t dlspm_workspace_bytes(int op, int M, int K, int N_or_D, int nnz)
     // workspace; a call without workspace runs the row-block schedule instead.
     if (M <= 0 || N_or_D <= 0 || nnz <= 0) return 0;
     if (op == DLSPM_OP_SPMM) {
-        const SpmmShape s = spmm_choose(M, K, N_or_D, nnz, N_or_D >= 4);
+        const SpmmShape s = spmm_choose(M, K, N_or_D, nnz, N_or_D >= 4, false, false);  // a call with memory
         const SlicePlan sliced = spmm_slice_plan(M, K, N_or_D, nnz, s);
         return sliced.slices > 0 ? sliced.bytes : flat_plan(M, nnz, N_or_D, s.G).bytes;
     }
@@ -414,16 +415,18 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
     return DLSPM_OK;
 }
 
-int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int rows_even, int* shape)
+int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int passing, int* shape)
 {
-    (void)K;
-    const bool even = rows_even != 0;
+    if (passing != DLSPM_PASS_NULL && passing != DLSPM_PASS_ROWS_EVEN && passing != DLSPM_PASS_WORKSPACE)
+        return DLSPM_E_INVALID_ARG;
+    const bool even = passing == DLSPM_PASS_ROWS_EVEN;
+    const bool memory = passing == DLSPM_PASS_WORKSPACE;
     if (!shape || M < 0 || N_or_D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     const int n = N_or_D;
     const bool vec4 = n >= 4;
     for (int i = 0; i < 10; ++i) shape[i] = 0;
     if (op == DLSPM_OP_SPMM) {
-        const SpmmShape s = spmm_choose(M, K, n, nnz, vec4, even);
+        const SpmmShape s = spmm_choose(M, K, n, nnz, vec4, even, !memory);
         const int tw = s.G * s.vec * s.V;
         shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[5] = s.W; shape[6] = s.R; shape[7] = (n + tw - 1) / tw;
         const FlatPlan fp = flat_plan(M, nnz, n, s.G);
@@ -448,7 +451,7 @@ int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int ro
 
 int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape)
 {
-    return dlspm_describe_launch_rows(op, M, K, N_or_D, nnz, 0, shape);
+    return dlspm_describe_launch_rows(op, M, K, N_or_D, nnz, DLSPM_PASS_NULL, shape);
 }
 
 int dlspm_workspace_advice(int op, int M, int K, int N_or_D, int nnz, int max_row_len)
@@ -472,7 +475,7 @@ int dlspm_describe_slices(int op, int M, int K, int N_or_D, int nnz, int* slices
 {
     if (M < 0 || K < 0 || N_or_D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     SlicePlan p{0, 1, 0, 0};
-    if (op == DLSPM_OP_SPMM) p = spmm_slice_plan(M, K, N_or_D, nnz, spmm_choose(M, K, N_or_D, nnz, N_or_D >= 4));
+    if (op == DLSPM_OP_SPMM) p = spmm_slice_plan(M, K, N_or_D, nnz, spmm_choose(M, K, N_or_D, nnz, N_or_D >= 4, false, false));
     else if (op == DLSPM_OP_FUSED) p = fused_slice_plan(M, K, N_or_D, nnz, fused_choose(M, N_or_D, nnz, N_or_D >= 4));
     else if (op == DLSPM_OP_SDDMM) p = sddmm_slice_plan(M, K, N_or_D, nnz, sddmm_choose(M, N_or_D, nnz, N_or_D >= 4));
     else return DLSPM_E_INVALID_ARG;

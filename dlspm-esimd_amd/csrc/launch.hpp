@@ -72,7 +72,8 @@ hipError_t slice_bounds_launch(int M, int K, int slices, const int* row_offsets,
                                hipStream_t stream);
 hipError_t slice_sum_launch(long long count, int slices, const float* partial, float* out, hipStream_t stream);
 
-SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even = false);
+// narrow_tiles: the call passes no workspace memory (column tiles below 128 columns are then allowed)
+SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles);
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
 hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPlan& plan, float* partial,
                             hipStream_t stream);

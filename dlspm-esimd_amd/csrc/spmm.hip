@@ -326,26 +326,34 @@ static hipError_t launch_wr(const SpmmArgs& x, int W, int R, int tile_major, hip
 }
 
 // Chooses the lane layout from N and the (W, R) split from the mean row length.
-SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even)
+SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles)
 {
     SpmmShape s{};
     s.vec = vec4 ? 4 : 1;
     // A B that does not fit one XCD's 4 MiB L2 is cut into column tiles that are worked through one after the other
-    // (tile-major grid order), each the widest of 512 / 256 / 128 columns whose K x tile slab still fits (measured on
+    // (tile-major grid order), each the widest of 512 ... 32 columns whose K x tile slab still fits (measured on
     // 8192 x 4096, N = 1024: 1460 us with tiles of 512, 930 us with 256; on 512 x 4608, N = 3136: 309 us against 273 us);
     // also where one wave could cover the whole width (N <= 512). Not for grids the device holds all at once: there the
-    // order cannot help, and 64 x 147 at N = 12544 lost 4 us. DLSPM_TILE_MAJOR=0|1 and DLSPM_TILE_WIDTH=512|256|128
+    // order cannot help, and 64 x 147 at N = 12544 lost 4 us. DLSPM_TILE_MAJOR=0|1 and DLSPM_TILE_WIDTH=512|...|32
     // override both for tuning sweeps.
+    // Tiles narrower than 128 columns (lane groups of 16 or 8 per dense row) only for a call without workspace: with
+    // one, slicing the columns of A keeps wider, more efficient dense rows (8192 x 65536, N = 128: 330 us untiled,
+    // 236 us in tiles of 32, 137 us in 16 slices of the full width).
+    const int min_tile = narrow_tiles ? 32 : 128;
     int tile = 0;  // 0: one tile if a wave can cover N, else tiles of 512 in row-major order
-    if (vec4 && N > 128) {
+    if (vec4 && N > min_tile) {
         bool on = (long long)K * N * (long long)sizeof(float) > (4ll << 20) && (long long)M * ((N + 511) / 512) >= 2048;
         if (const char* e = std::getenv("DLSPM_TILE_MAJOR")) on = std::atoi(e) != 0;
         if (on) {
-            const long long slab512 = (long long)K * 512 * (long long)sizeof(float);
-            tile = slab512 <= (4ll << 20) ? 512 : slab512 <= (8ll << 20) ? 256 : 128;
+            tile = min_tile;
+            for (int t = 512; t > min_tile; t /= 2)
+                if ((long long)K * t * (long long)sizeof(float) <= (4ll << 20)) {
+                    tile = t;
+                    break;
+                }
             if (const char* e = std::getenv("DLSPM_TILE_WIDTH")) {
                 const int t = std::atoi(e);
-                if (t == 512 || t == 256 || t == 128) tile = t;
+                if ((t == 512 || t == 256 || t == 128 || t == 64 || t == 32) && t >= min_tile) tile = t;
             }
             if (tile >= N) tile = 0;  // a single tile: nothing to order
         }
@@ -355,6 +363,8 @@ SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even)
         if (tile == 512) { s.G = 64; s.V = 2; }
         else if (tile == 256) { s.G = 64; s.V = 1; }
         else if (tile == 128) { s.G = 32; s.V = 1; }
+        else if (tile == 64) { s.G = 16; s.V = 1; }
+        else if (tile == 32) { s.G = 8; s.V = 1; }
         else if (N > 256) { s.G = 64; s.V = 2; }
         else if (N > 128) { s.G = 64; s.V = 1; }
         else if (N > 64) { s.G = 32; s.V = 1; }

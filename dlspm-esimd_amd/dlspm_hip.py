@@ -182,11 +182,14 @@ def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None, workspace=N
     return out
 
 
-def describe_launch(op: int, M: int, K: int, N: int, nnz: int, rows_even: bool = False) -> dict:
+def describe_launch(op: int, M: int, K: int, N: int, nnz: int, rows_even: bool = False,
+                    with_workspace: bool = False) -> dict:
     """Launch shape the library uses for these sizes: {'vec','G','V','G1','DS','W','R','col_tiles','flat_chunk',
-    'flat_units'} (host only). rows_even: for a call that passes ROWS_EVEN."""
+    'flat_units'} (host only). rows_even: for a call that passes ROWS_EVEN; with_workspace: for one that passes
+    workspace memory; neither: for one that passes None."""
     out = (ctypes.c_int * 10)()
-    st = lib().dlspm_describe_launch_rows(op, M, K, N, nnz, 1 if rows_even else 0, out)
+    passing = PASS_WORKSPACE if with_workspace else PASS_ROWS_EVEN if rows_even else PASS_NULL
+    st = lib().dlspm_describe_launch_rows(op, M, K, N, nnz, passing, out)
     if st != OK:
         raise DlspmError(st, "dlspm_describe_launch")
     return dict(zip(("vec", "G", "V", "G1", "DS", "W", "R", "col_tiles", "flat_chunk", "flat_units"),

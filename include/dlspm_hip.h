@@ -173,8 +173,13 @@ int dlspm_workspace_advice(int op, int M, int K, int N_or_D, int nnz, int max_ro
  */
 int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape);
 
-/* The same for a call that passes DLSPM_ROWS_EVEN (rows_even != 0) or does not (rows_even == 0). */
-int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int rows_even, int* shape);
+/*
+ * The same for a call that passes NULL, DLSPM_ROWS_EVEN or workspace memory (`passing` = DLSPM_PASS_NULL,
+ * DLSPM_PASS_ROWS_EVEN, DLSPM_PASS_WORKSPACE, defined with dlspm_workspace_advice): the lane layout of SpMM
+ * (column tiles narrower than 128 only without memory) and the rows per workgroup (more for rows known to be even)
+ * depend on it. dlspm_describe_launch is the DLSPM_PASS_NULL case.
+ */
+int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int passing, int* shape);
 
 /*
  * Column-sliced schedule that a call WITH workspace would use for these sizes: *slices = number of column ranges

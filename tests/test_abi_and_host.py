@@ -72,12 +72,22 @@ def test_column_tiles_narrow_with_the_height_of_the_dense_operand(dl):
     """Dense rows wider than 512 floats are covered by several column tiles, worked through one after the other: the
     widest tile whose K x tile slab of B fits 4 MiB."""
     nnz = 4096 * 100
-    for K, tile in ((512, 512), (2048, 512), (2049, 256), (4096, 256), (4097, 128), (1 << 16, 128)):
+    for K, tile in ((512, 512), (2048, 512), (2049, 256), (4096, 256), (4097, 128), (8193, 64), (1 << 16, 32)):
         sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz)
         assert sh["G"] * sh["vec"] * sh["V"] == tile and sh["col_tiles"] == -(-3136 // tile), (K, sh)
-    # the same where one wave could cover the whole width, once B exceeds the L2
+        sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz, with_workspace=True)
+        assert sh["G"] * sh["vec"] * sh["V"] == max(tile, 128)
+    # the same where one wave could cover the whole width, once B exceeds the L2; tiles below 128 columns only for a
+    # call without workspace memory (with it the columns of A are sliced instead)
     sh = dl.describe_launch(dl.OP_SPMM, 4096, 8192, 256, nnz)
     assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (128, 2)
+    for K, tile in ((16384, 64), (32768, 32), (1 << 17, 32)):
+        sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 128, nnz)
+        assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (tile, 128 // tile)
+        assert dl.describe_launch(dl.OP_SPMM, 4096, K, 128, nnz, with_workspace=True)["col_tiles"] == 1
+        assert dl.describe_launch(dl.OP_SPMM, 4096, K, 128, nnz, rows_even=True)["col_tiles"] == 128 // tile
+    assert dl.describe_launch(dl.OP_SPMM, 4096, 32768, 64, nnz)["col_tiles"] == 2
+    assert dl.describe_launch(dl.OP_SPMM, 4096, 32768, 32, nnz)["col_tiles"] == 1   # 32 columns: the narrowest tile
     sh = dl.describe_launch(dl.OP_SPMM, 4096, 4096, 512, nnz)
     assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (256, 2)
     assert dl.describe_launch(dl.OP_SPMM, 4096, 4096, 256, nnz)["col_tiles"] == 1   # 4 MiB: fits

@@ -394,7 +394,7 @@ def test_column_sliced_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
     B = dl.fill("uniform", 74, (K, N), -1.0, 1.0)
     Q = dl.fill("normal", 75, (M, N), 0.0, 1.0)
     ro_d, ci_d, va_d, B_d, Q_d = (dev(torch, x) for x in (ro, ci, va, B, Q))
-    assert dl.describe_slices(dl.OP_SPMM, M, K, N, nnz)[0] == 4 and dl.describe_launch(dl.OP_SPMM, M, K, N, nnz)["col_tiles"] == 2
+    assert dl.describe_slices(dl.OP_SPMM, M, K, N, nnz)[0] == 4 and dl.describe_launch(dl.OP_SPMM, M, K, N, nnz, with_workspace=True)["col_tiles"] == 2
     assert dl.describe_slices(dl.OP_SDDMM, M, K, N, nnz)[0] == 8
     assert dl.describe_slices(dl.OP_FUSED, M, K, N, nnz)[0] == 16
 

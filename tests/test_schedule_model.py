@@ -158,7 +158,9 @@ GPU_SPMM = [(300, 200, 256, "skewed", 0.15), (128, 512, 128, "uniform", 0.3), (2
             (64, 128, 49, "skewed", 0.2), (70, 90, 5, "uniform", 0.3), (10, 64, 1026, "uniform", 0.3),
             (300, 80, 1, "skewed", 0.3), (50, 80, 3, "uniform", 0.3),
             # several column tiles, narrower the taller B is: 256 columns from K > 2048, 128 from K > 4096
-            (40, 2100, 600, "skewed", 0.05), (30, 4200, 530, "uniform", 0.02), (700, 4100, 1030, "empty_rows", 0.01)]
+            (40, 2100, 600, "skewed", 0.05), (30, 4200, 530, "uniform", 0.02), (700, 4100, 1030, "empty_rows", 0.01),
+            # ... down to 64 and 32 columns for a very tall B (no workspace in these calls)
+            (2100, 16500, 100, "uniform", 0.005), (2060, 9000, 120, "skewed", 0.01)]
 
 
 @pytest.mark.gpu
@@ -306,7 +308,7 @@ def test_gpu_flat_spmm_equals_model_bit_for_bit(model, dl, monkeypatch, kind, M,
     monkeypatch.setenv("DLSPM_FLAT", "1")
     monkeypatch.setenv("DLSPM_SLICES", "0")
     monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
-    sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size)
+    sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size, with_workspace=True)
     assert sh["flat_chunk"] == chunk and sh["flat_units"] == -(-ci.size // chunk)
     need = dl.workspace_bytes(dl.OP_SPMM, M, K, N, ci.size)
     assert need == sh["flat_units"] * 2 * N * 4
@@ -428,7 +430,7 @@ def test_gpu_random_shapes_equal_model_bit_for_bit(model, dl, monkeypatch, seed)
         ro_d, ci_d = dev(torch, ro), dev(torch, ci)
         bits = lambda a: np.ascontiguousarray(a).view(np.uint32)
 
-        sh = dl.describe_launch(dl.OP_SPMM, M, K, N, nnz)
+        sh = dl.describe_launch(dl.OP_SPMM, M, K, N, nnz, with_workspace=flat)
         if flat:
             rc, C, writes = run_spmm_flat(model, ro, ci2, va, B, sh["G"], chunk)
         else:
@@ -507,7 +509,7 @@ def test_gpu_sliced_spmm_equals_model_bit_for_bit(model, dl, oracle, monkeypatch
     monkeypatch.setenv("DLSPM_SLICES", str(slices))
     got_slices, R = dl.describe_slices(dl.OP_SPMM, M, K, N, ci.size)
     assert got_slices == slices and R in (1, 2, 4, 8, 16)
-    sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size)
+    sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size, with_workspace=True)
     need = dl.workspace_bytes(dl.OP_SPMM, M, K, N, ci.size)
     assert need >= (slices + 1) * M * 4 + slices * M * N * 4
 
