@@ -351,6 +351,12 @@ SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, b
                     tile = t;
                     break;
                 }
+            // More tiles than a wave needs to cover N cost every row its start-up once more per tile: only for rows
+            // of at least 32 nonzeros on average, and only while the slab is at most twice the L2 (measured on graph-
+            // like shapes, K = 262144 ... 1048576, 8 nonzeros per row: tiles of 32 up to 2x slower than one tile;
+            // 32 per row: equal; K = 65536, slab 8 MiB, 655 per row: 330 -> 236 us).
+            const bool narrow_ok = (long long)nnz >= 32ll * M && (long long)K * tile * (long long)sizeof(float) <= (8ll << 20);
+            if (!narrow_ok) tile = 512;
             if (const char* e = std::getenv("DLSPM_TILE_WIDTH")) {
                 const int t = std::atoi(e);
                 if ((t == 512 || t == 256 || t == 128 || t == 64 || t == 32) && t >= min_tile) tile = t;

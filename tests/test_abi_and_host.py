@@ -76,16 +76,21 @@ def test_column_tiles_narrow_with_the_height_of_the_dense_operand(dl):
         sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz)
         assert sh["G"] * sh["vec"] * sh["V"] == tile and sh["col_tiles"] == -(-3136 // tile), (K, sh)
         sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz, with_workspace=True)
-        assert sh["G"] * sh["vec"] * sh["V"] == max(tile, 128)
+        assert sh["G"] * sh["vec"] * sh["V"] == (max(tile, 128) if K * 128 * 4 <= (8 << 20) else 512)
     # the same where one wave could cover the whole width, once B exceeds the L2; tiles below 128 columns only for a
     # call without workspace memory (with it the columns of A are sliced instead)
     sh = dl.describe_launch(dl.OP_SPMM, 4096, 8192, 256, nnz)
     assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (128, 2)
-    for K, tile in ((16384, 64), (32768, 32), (1 << 17, 32)):
+    for K, tile in ((16384, 64), (32768, 32), (1 << 16, 32)):
         sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 128, nnz)
         assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (tile, 128 // tile)
         assert dl.describe_launch(dl.OP_SPMM, 4096, K, 128, nnz, with_workspace=True)["col_tiles"] == 1
         assert dl.describe_launch(dl.OP_SPMM, 4096, K, 128, nnz, rows_even=True)["col_tiles"] == 128 // tile
+    # not when even the narrowest slab is beyond twice the L2, nor for rows below 32 nonzeros (graph-like shapes):
+    # more tiles than needed cost every row its start-up once more
+    assert dl.describe_launch(dl.OP_SPMM, 4096, 1 << 17, 128, nnz)["col_tiles"] == 1
+    assert dl.describe_launch(dl.OP_SPMM, 4096, 1 << 17, 3136, nnz)["col_tiles"] == 7      # the usual tiles of 512
+    assert dl.describe_launch(dl.OP_SPMM, 1 << 18, 32768, 128, (1 << 18) * 8)["col_tiles"] == 1
     assert dl.describe_launch(dl.OP_SPMM, 4096, 32768, 64, nnz)["col_tiles"] == 2
     assert dl.describe_launch(dl.OP_SPMM, 4096, 32768, 32, nnz)["col_tiles"] == 1   # 32 columns: the narrowest tile
     sh = dl.describe_launch(dl.OP_SPMM, 4096, 4096, 512, nnz)
@@ -113,18 +118,21 @@ def test_column_sliced_schedule_rule(dl):
     assert dl.describe_slices(dl.OP_SPMM, M, K, 256, M * 400)[0] == 0   # ... 200 nonzeros per slice: not at exactly 4 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, K, 128, nnz)[0] == 2       # one tile of 4 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, K, 100, nnz)[0] == 0       # 3.1 MiB: fits
-    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, nnz)[0] == 8   # 32768 x 128 floats per tile: 16 MiB
+    assert dl.describe_slices(dl.OP_SPMM, M, 2 * K, 256, nnz)[0] == 4   # 16384 x 128 floats per tile: 8 MiB
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, nnz)[0] == 16  # taller: no tile would fit, 32 MiB in one piece
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 16, 32, nnz)[0] == 4  # narrow dense rows, very tall B: 8 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 16, 32, M * 300)[0] == 2  # ... 128 nonzeros per slice at N = 32
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 20, 3, nnz)[0] == 0   # fewer than four columns: not built for them
-    # ... in tiles of 128 columns a row keeps at least 32 nonzeros per slice
-    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 140)[0] == 4   # 140 nonzeros per row: four slices of 35
-    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 70)[0] == 2    # 70 per row: two
+    # a row keeps at least max(16, 4096 / width) nonzeros per slice: 16 at 256 columns, 32 in tiles of 128
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 140)[0] == 8   # 140 nonzeros per row: eight slices of 17
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 70)[0] == 4    # 70 per row: four
+    assert dl.describe_slices(dl.OP_SPMM, M, 2 * K, 256, M * 140)[0] == 4   # tiles of 128: four slices of 35
+    assert dl.describe_slices(dl.OP_SPMM, M, 2 * K, 256, M * 70)[0] == 2    # 70 per row: two
     assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 40)[0] == 0    # 40 per row, 0.33 M nonzeros: too small
-    assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 64)[0] == 2  # 2.1 M nonzeros, 64 per row: two slices
-    assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 60)[0] == 0  # 60 per row: not even two
-    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, nnz)[0] == 16      # 64 MiB per tile: the most slices there are
-    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, M * 100)[0] == 3   # ... but a row keeps 32 nonzeros per slice
+    assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 64)[0] == 4  # 2.1 M nonzeros, 64 per row
+    assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 30)[0] == 0  # 30 per row: not even two of 16
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, nnz)[0] == 16      # 128 MiB: the most slices there are
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, M * 100)[0] == 6   # ... but a row keeps 16 nonzeros per slice
     assert dl.describe_slices(dl.OP_SDDMM, M, K, 256, nnz)[0] == 4      # rhs: 8 MiB; only the boundaries need memory
     assert dl.workspace_bytes(dl.OP_SDDMM, M, K, 256, nnz) == -(-5 * M * 4 // 256) * 256
     assert dl.describe_slices(dl.OP_SDDMM, M, K, 100, nnz)[0] == 0 and dl.workspace_bytes(dl.OP_SDDMM, M, K, 100, nnz) == 0
