@@ -325,45 +325,49 @@ static hipError_t launch_wr(const SpmmArgs& x, int W, int R, int tile_major, hip
     return hipErrorInvalidValue;
 }
 
-// Chooses the lane layout from N and the (W, R) split from the mean row length.
+// Width of the column tiles of B that the grid works through one after the other (tile-major order), or 0: one tile
+// if a wave can cover N, else tiles of 512 in row-major order.
+// A B that does not fit one XCD's 4 MiB L2 is cut into tiles, each the widest of 512 ... 32 columns whose K x tile
+// slab still fits (measured on 8192 x 4096, N = 1024: 1460 us with tiles of 512, 930 us with 256; on 512 x 4608,
+// N = 3136: 309 us against 273 us); also where one wave could cover the whole width (N <= 512). Not for grids the
+// device holds all at once: there the order cannot help, and 64 x 147 at N = 12544 lost 4 us.
+// Tiles narrower than 128 columns (lane groups of 16 or 8 per dense row) only for a call without workspace memory
+// (`narrow_tiles`): with it, slicing the columns of A keeps wider, more efficient dense rows (8192 x 65536, N = 128:
+// 330 us untiled, 236 us in tiles of 32, 137 us in 16 slices of the full width).
+// More tiles than a wave needs to cover N cost every row its start-up once more per tile: the tile is narrowed only
+// for rows of at least 32 nonzeros on average, and only while the slab is at most twice the L2 (measured on graph-
+// like shapes, K = 262144 ... 1048576, 8 nonzeros per row: tiles of 32 up to 2x slower than one tile; 32 per row:
+// equal; K = 65536, slab 8 MiB, 655 per row: 330 -> 236 us).
+// DLSPM_TILE_MAJOR=0|1 and DLSPM_TILE_WIDTH=512|...|32 override the rule for tuning sweeps.
+static int spmm_tile_width(int M, int K, int N, int nnz, bool narrow_tiles)
+{
+    const long long l2 = 4ll << 20;
+    const int min_tile = narrow_tiles ? 32 : 128;
+    if (N <= min_tile) return 0;
+    bool on = (long long)K * N * (long long)sizeof(float) > l2 && (long long)M * ((N + 511) / 512) >= 2048;
+    if (const char* e = std::getenv("DLSPM_TILE_MAJOR")) on = std::atoi(e) != 0;
+    if (!on) return 0;
+    int tile = min_tile;
+    for (int t = 512; t > min_tile; t /= 2)
+        if ((long long)K * t * (long long)sizeof(float) <= l2) {
+            tile = t;
+            break;
+        }
+    const bool narrow_ok = (long long)nnz >= 32ll * M && (long long)K * tile * (long long)sizeof(float) <= 2 * l2;
+    if (!narrow_ok) tile = 512;
+    if (const char* e = std::getenv("DLSPM_TILE_WIDTH")) {
+        const int t = std::atoi(e);
+        if ((t == 512 || t == 256 || t == 128 || t == 64 || t == 32) && t >= min_tile) tile = t;
+    }
+    return tile < N ? tile : 0;  // a single tile: nothing to order
+}
+
+// Chooses the lane layout from N (and the height of B) and the (W, R) split from the mean row length.
 SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles)
 {
     SpmmShape s{};
     s.vec = vec4 ? 4 : 1;
-    // A B that does not fit one XCD's 4 MiB L2 is cut into column tiles that are worked through one after the other
-    // (tile-major grid order), each the widest of 512 ... 32 columns whose K x tile slab still fits (measured on
-    // 8192 x 4096, N = 1024: 1460 us with tiles of 512, 930 us with 256; on 512 x 4608, N = 3136: 309 us against 273 us);
-    // also where one wave could cover the whole width (N <= 512). Not for grids the device holds all at once: there the
-    // order cannot help, and 64 x 147 at N = 12544 lost 4 us. DLSPM_TILE_MAJOR=0|1 and DLSPM_TILE_WIDTH=512|...|32
-    // override both for tuning sweeps.
-    // Tiles narrower than 128 columns (lane groups of 16 or 8 per dense row) only for a call without workspace: with
-    // one, slicing the columns of A keeps wider, more efficient dense rows (8192 x 65536, N = 128: 330 us untiled,
-    // 236 us in tiles of 32, 137 us in 16 slices of the full width).
-    const int min_tile = narrow_tiles ? 32 : 128;
-    int tile = 0;  // 0: one tile if a wave can cover N, else tiles of 512 in row-major order
-    if (vec4 && N > min_tile) {
-        bool on = (long long)K * N * (long long)sizeof(float) > (4ll << 20) && (long long)M * ((N + 511) / 512) >= 2048;
-        if (const char* e = std::getenv("DLSPM_TILE_MAJOR")) on = std::atoi(e) != 0;
-        if (on) {
-            tile = min_tile;
-            for (int t = 512; t > min_tile; t /= 2)
-                if ((long long)K * t * (long long)sizeof(float) <= (4ll << 20)) {
-                    tile = t;
-                    break;
-                }
-            // More tiles than a wave needs to cover N cost every row its start-up once more per tile: only for rows
-            // of at least 32 nonzeros on average, and only while the slab is at most twice the L2 (measured on graph-
-            // like shapes, K = 262144 ... 1048576, 8 nonzeros per row: tiles of 32 up to 2x slower than one tile;
-            // 32 per row: equal; K = 65536, slab 8 MiB, 655 per row: 330 -> 236 us).
-            const bool narrow_ok = (long long)nnz >= 32ll * M && (long long)K * tile * (long long)sizeof(float) <= (8ll << 20);
-            if (!narrow_ok) tile = 512;
-            if (const char* e = std::getenv("DLSPM_TILE_WIDTH")) {
-                const int t = std::atoi(e);
-                if ((t == 512 || t == 256 || t == 128 || t == 64 || t == 32) && t >= min_tile) tile = t;
-            }
-            if (tile >= N) tile = 0;  // a single tile: nothing to order
-        }
-    }
+    const int tile = vec4 ? spmm_tile_width(M, K, N, nnz, narrow_tiles) : 0;
     s.tile_major = tile > 0 ? 1 : 0;
     if (vec4) {
         if (tile == 512) { s.G = 64; s.V = 2; }
