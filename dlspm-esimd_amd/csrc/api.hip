@@ -115,7 +115,7 @@ SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial
     if (just_fills && width < 128) slices = 0;
     const long long fit = (long long)nnz / ((long long)min_row * M);
     if (slices > fit) slices = fit;
-    const bool by_rule = bytes >= kSliceMinOperand && nnz >= kFlatMinNnz && slices >= 2;
+    const bool by_rule = bytes >= kSliceMinOperand && nnz >= kSlicedMinNnz && slices >= 2;
     if (force == 0 || force == 1 || (force < 0 && !by_rule)) return p;
     if (force >= 2) slices = force < kSliceMaxSlices ? force : kSliceMaxSlices;
     if (slices > K) slices = K;
@@ -224,7 +224,10 @@ static SlicePlan spmm_slice_plan(int M, int K, int N, int nnz, const SpmmShape& 
 {
     const int tw = s.G * s.vec * s.V;
     // the column tiles are worked through one after the other: one tile's slab of B is what is gathered from at a time
-    SlicePlan p = slice_plan(M, K, N < tw ? N : tw, nnz, 1, 0, s.vec == 4 ? s.G : 0, (N + tw - 1) / tw, kWave / s.G, 2048);
+    // and the workgroups of one (slice, tile) pair should fill the device by themselves, or it gathers from several
+    // slabs at once: rows per workgroup as if there were one tile (4096 x 65536, N = 3136, 25 tiles of 128, 131 or
+    // 656 nonzeros per row: 856 -> 716 us and 2320 -> 2133 us)
+    SlicePlan p = slice_plan(M, K, N < tw ? N : tw, nnz, 1, 0, s.vec == 4 ? s.G : 0, 1, kWave / s.G, 2048);
     p.bytes = p.slices > 0 ? p.bounds_bytes + (size_t)p.slices * M * (size_t)N * sizeof(float) : 0;
     return p;
 }
@@ -466,7 +469,16 @@ int dlspm_workspace_advice(int op, int M, int K, int N_or_D, int nnz, int max_ro
     const bool even = known && max_row_len <= 1.5 * mean, uneven = known && max_row_len >= 4.0 * mean;
     // even rows and an operand that only just exceeds the L2 (two slices): one whole row per wave does as well or better
     // (measured: SpMM and fused 5-9 % faster at exactly 4 MiB, equal at 8 MiB; SDDMM 2-12 % slower)
-    const bool sliced = slices > 0 && !(even && slices <= 2 && op != DLSPM_OP_SDDMM);
+    bool sliced = slices > 0 && !(even && slices <= 2 && op != DLSPM_OP_SDDMM);
+    // SpMM on rows below ~128 nonzeros: a call without memory that works in narrower column tiles is faster than the
+    // slices (8192 x 32768, N = 256: 51 against 66 us at 70 per row, equal at 140, 157 against 139 us at 328;
+    // 32768 x 32768, N = 256: 228 against 282 us at 128; 16384 x 32768, N = 1024: 418 against 459 us at 70,
+    // 788 against 590 us at 140)
+    if (sliced && op == DLSPM_OP_SPMM && mean < 128.0) {
+        const SpmmShape without = spmm_choose(M, K, N_or_D, nnz, N_or_D >= 4, false, true);
+        const SpmmShape with = spmm_choose(M, K, N_or_D, nnz, N_or_D >= 4, false, false);
+        if (without.tile_major && without.G * without.V < with.G * with.V) sliced = false;
+    }
     if (sliced || (uneven && want > 0 && slices == 0)) return DLSPM_PASS_WORKSPACE;
     return even ? DLSPM_PASS_ROWS_EVEN : DLSPM_PASS_NULL;
 }

@@ -176,7 +176,8 @@ int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape)
 /*
  * The same for a call that passes NULL, DLSPM_ROWS_EVEN or workspace memory (`passing` = DLSPM_PASS_NULL,
  * DLSPM_PASS_ROWS_EVEN, DLSPM_PASS_WORKSPACE, defined with dlspm_workspace_advice): the lane layout of SpMM
- * (column tiles narrower than 128 only without memory) and the rows per workgroup (more for rows known to be even)
+ * (column tiles narrower than 128 only without memory; tiles of 128 on a B of any height only with it, where the
+ * column-sliced schedule cuts the tile's slab of B) and the rows per workgroup (more for rows known to be even)
  * depend on it. dlspm_describe_launch is the DLSPM_PASS_NULL case.
  */
 int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int passing, int* shape);

@@ -77,6 +77,16 @@ def test_column_tiles_narrow_with_the_height_of_the_dense_operand(dl):
         assert sh["G"] * sh["vec"] * sh["V"] == tile and sh["col_tiles"] == -(-3136 // tile), (K, sh)
         sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz, with_workspace=True)
         assert sh["G"] * sh["vec"] * sh["V"] == (max(tile, 128) if K * 128 * 4 <= (8 << 20) else 512)
+    # ... with memory and rows long enough for the column-sliced schedule (64 nonzeros per row, half a million in
+    # all), tiles of 128 at any height: the slices cut the slab along K
+    for n, tiles in ((3136, 25), (1024, 8), (256, 2)):
+        sh = dl.describe_launch(dl.OP_SPMM, 8192, 1 << 15, n, 8192 * 300, with_workspace=True)
+        assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (128, tiles)
+    assert dl.describe_launch(dl.OP_SPMM, 8192, 1 << 15, 1024, 8192 * 63, with_workspace=True)["col_tiles"] == 2
+    # the workgroups of one (slice, tile) pair fill the device by themselves: rows per workgroup from M alone
+    assert dl.describe_slices(dl.OP_SPMM, 8192, 1 << 15, 1024, 8192 * 300) == (8, 4)
+    assert dl.describe_slices(dl.OP_SPMM, 4096, 1 << 16, 3136, 4096 * 131) == (4, 2)
+    assert dl.describe_slices(dl.OP_SPMM, 2048, 1 << 17, 512, 2048 * 655) == (16, 1)
     # the same where one wave could cover the whole width, once B exceeds the L2; tiles below 128 columns only for a
     # call without workspace memory (with it the columns of A are sliced instead)
     sh = dl.describe_launch(dl.OP_SPMM, 4096, 8192, 256, nnz)
@@ -119,20 +129,21 @@ def test_column_sliced_schedule_rule(dl):
     assert dl.describe_slices(dl.OP_SPMM, M, K, 128, nnz)[0] == 2       # one tile of 4 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, K, 100, nnz)[0] == 0       # 3.1 MiB: fits
     assert dl.describe_slices(dl.OP_SPMM, M, 2 * K, 256, nnz)[0] == 4   # 16384 x 128 floats per tile: 8 MiB
-    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, nnz)[0] == 16  # taller: no tile would fit, 32 MiB in one piece
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, nnz)[0] == 8   # taller: tiles of 128 all the same, 16 MiB each
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 16, 32, nnz)[0] == 4  # narrow dense rows, very tall B: 8 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 16, 32, M * 300)[0] == 2  # ... 128 nonzeros per slice at N = 32
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 20, 3, nnz)[0] == 0   # fewer than four columns: not built for them
     # a row keeps at least max(16, 4096 / width) nonzeros per slice: 16 at 256 columns, 32 in tiles of 128
-    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 140)[0] == 8   # 140 nonzeros per row: eight slices of 17
-    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 70)[0] == 4    # 70 per row: four
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 140)[0] == 4   # 140 nonzeros per row: four slices of 35
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 70)[0] == 2    # 70 per row: two
+    assert dl.describe_slices(dl.OP_SPMM, 2 * M, 4 * K, 256, 2 * M * 60)[0] == 3  # below 64 per row: one tile of 256, three slices of 20
     assert dl.describe_slices(dl.OP_SPMM, M, 2 * K, 256, M * 140)[0] == 4   # tiles of 128: four slices of 35
     assert dl.describe_slices(dl.OP_SPMM, M, 2 * K, 256, M * 70)[0] == 2    # 70 per row: two
     assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 40)[0] == 0    # 40 per row, 0.33 M nonzeros: too small
-    assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 64)[0] == 4  # 2.1 M nonzeros, 64 per row
+    assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 64)[0] == 2  # 2.1 M nonzeros, 64 per row
     assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 30)[0] == 0  # 30 per row: not even two of 16
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, nnz)[0] == 16      # 128 MiB: the most slices there are
-    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, M * 100)[0] == 6   # ... but a row keeps 16 nonzeros per slice
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, M * 100)[0] == 3   # ... but a row keeps 32 nonzeros per slice
     assert dl.describe_slices(dl.OP_SDDMM, M, K, 256, nnz)[0] == 4      # rhs: 8 MiB; only the boundaries need memory
     assert dl.workspace_bytes(dl.OP_SDDMM, M, K, 256, nnz) == -(-5 * M * 4 // 256) * 256
     assert dl.describe_slices(dl.OP_SDDMM, M, K, 100, nnz)[0] == 0 and dl.workspace_bytes(dl.OP_SDDMM, M, K, 100, nnz) == 0
@@ -158,6 +169,13 @@ def test_workspace_advice(dl):
     assert A(dl.OP_SPMM, M, K, 128, nnz, mean + 10) == dl.PASS_ROWS_EVEN
     assert A(dl.OP_SPMM, M, K, 128, nnz, 3 * mean) == dl.PASS_WORKSPACE
     assert A(dl.OP_SDDMM, M, K, 128, nnz, mean + 10) == dl.PASS_WORKSPACE
+    # SpMM on rows below 128 nonzeros: narrower column tiles without memory beat the slices
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 120)[0] == 3
+    assert A(dl.OP_SPMM, M, 4 * K, 256, M * 120, 3 * 120) == dl.PASS_NULL
+    assert A(dl.OP_SPMM, M, 4 * K, 256, M * 120, 130) == dl.PASS_ROWS_EVEN
+    assert A(dl.OP_SPMM, M, 4 * K, 256, M * 130, 3 * 130) == dl.PASS_WORKSPACE
+    assert A(dl.OP_SPMM, M, 1 << 18, 256, M * 120, 3 * 120) == dl.PASS_WORKSPACE   # no tile would fit: the slices
+    assert A(dl.OP_FUSED, M, 4 * K, 256, M * 120, 3 * 120) == dl.PASS_WORKSPACE    # the other two ops have no tiles
     # no slices: the memory for rows at least four times the mean where the flat schedule applies, the hint for even rows
     assert A(dl.OP_SPMM, M, 2048, 128, nnz, 4 * mean) == dl.PASS_WORKSPACE
     assert A(dl.OP_SPMM, M, 2048, 128, nnz, 3 * mean) == dl.PASS_NULL
