@@ -418,6 +418,40 @@ def test_column_sliced_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
+@pytest.mark.parametrize("sigma", [0.0, 1.0])
+def test_sliced_column_tiles_on_a_tall_wide_dense_operand(torch_cuda, dl, oracle, sigma):
+    """B of 24576 x 392 floats (37 MiB; not even a tile of 128 columns fits twice the L2) under rows of ~130 nonzeros:
+    a call WITH workspace works in four column tiles of 128 (the last one 8 columns wide) and cuts each into slices,
+    a call without in tiles of 32; both against the multi-threaded oracle, and the integer-exact row lengths."""
+    torch = torch_cuda
+    M, K, N = 4100, 24576, 392
+    if sigma == 0.0:
+        ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 81, M, K, 130.0 / K)
+    else:
+        ro, ci = dl.make_pattern(dl.PATTERN_LOGNORMAL_ROWS, 82, M, K, 130.0, sigma)
+    nnz = ci.size
+    assert nnz >= 1 << 19
+    va = dl.fill("uniform", 83, (nnz,), -1.0, 1.0)
+    B = dl.fill("uniform", 84, (K, N), -1.0, 1.0)
+    ro_d, ci_d, va_d, B_d = (dev(torch, x) for x in (ro, ci, va, B))
+    sh = dl.describe_launch(dl.OP_SPMM, M, K, N, nnz, with_workspace=True)
+    assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (128, 4)
+    slices, R = dl.describe_slices(dl.OP_SPMM, M, K, N, nnz)
+    assert slices == 4 and R == 2                       # 32 nonzeros per row and slice; 2050 workgroups per (slice, tile)
+    assert dl.describe_launch(dl.OP_SPMM, M, K, N, nnz)["col_tiles"] == 13   # without memory: tiles of 32
+
+    ws = torch.empty(dl.workspace_bytes(dl.OP_SPMM, M, K, N, nnz), dtype=torch.uint8, device="cuda")
+    got = dl.spmm(ro_d, ci_d, va_d, B_d, K=K, workspace=ws)
+    ref = oracle.spmm(ro, ci, va, B, omp=True)
+    assert oracle.rel_frobenius(got.cpu().numpy(), ref) <= TOL
+    assert oracle.rel_frobenius(dl.spmm(ro_d, ci_d, va_d, B_d, K=K).cpu().numpy(), ref) <= TOL
+    assert (got.cpu().numpy()[np.diff(ro) == 0] == 0).all()
+    ones_v, ones_B = torch.ones(nnz, device="cuda"), torch.ones(K, N, device="cuda")
+    lengths = torch.from_numpy(np.diff(ro).astype(np.float32)).cuda()[:, None].expand(M, N)
+    assert torch.equal(dl.spmm(ro_d, ci_d, ones_v, ones_B, K=K, workspace=ws), lengths)
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
 def test_exact_integer_properties_at_large_size(torch_cuda, dl):
     """Size-independent, bit-exact checks on 65536 skewed rows (several million nonzeros), no oracle needed: with small-integer
     operands every fp32 product and sum is exact whatever the summation order, so
