@@ -83,19 +83,23 @@ static FlatPlan sddmm_flat_plan(int M, int nnz, int D)
 
 // Column-sliced schedule (the device works through the column ranges of the sparse matrix one after the other, partial
 // rows in the caller's workspace): chosen when the dense operands gathered per nonzero are together larger than one
-// XCD's 4 MiB L2; the slices are cut to 2 MiB of them. Measured on MI355X (8192 x 8192, 30 % dense, lognormal rows,
+// XCD's 4 MiB L2; the slices are cut to 2 MiB of them (8/3 MiB with partial rows). Measured on MI355X (8192 x 8192, 30 % dense, lognormal rows,
 // sigma 0.6; row-block / flat / sliced): fused, D = 128 (8 MiB of Kmat and V): 1429 / 1374 / 676 us, D = 256 (16 MiB):
-// 4024 / 3946 / 1328 us; SpMM, N = 256: 1472 / 1390 / 685 us; slices of 4 MiB instead: 769, 1441, 803 us. Operands of
+// 4024 / 3946 / 1328 us; SpMM, N = 256: 1472 / 1390 / 685 us; slices of 4 MiB instead: 769, 1441, 803 us. SpMM and
+// the fused op write a partial row per row and slice, and slices of 8/3 MiB instead of 2 MiB are 3 % faster for them in
+// the geometric mean of 24 cases (0.88 ... 1.09; most on a tall B under wide dense rows); SDDMM has no partial rows and
+// gains nothing from larger slices (0.92 ... 1.04, mean 1.00). Operands of
 // exactly 4 MiB (8192 x 128 floats) gain 13-16 % at 10-30 % density and lose 5 % at 3 %: sliced in two for long rows
 // only. Like the flat schedule only from half a million nonzeros on (two more launches). DLSPM_SLICES=0 switches it
 // off, DLSPM_SLICES=n forces n slices (tuning, tests).
 constexpr long long kSliceMinOperand = 4ll << 20;  // bytes gathered from; above this the operand is sliced
-constexpr long long kSliceBytes = 2ll << 20;       // bytes of it per slice
+constexpr long long kSlicesPer8MiB = 4;            // slices of 2 MiB of it: half the L2 each
+constexpr long long kSlicesPer8MiBPartial = 3;     // ... of 8/3 MiB where every slice costs a partial row per row
 constexpr int kSliceMaxSlices = 16;
 constexpr int kSliceMinRow = 16;  // least mean nonzeros of a row inside one slice; fewer slices rather than shorter shares
 constexpr int kSliceMinRowAtL2 = 256;  // the same for an operand of exactly kSliceMinOperand bytes
 
-SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial_width, int G, long long col_tiles,
+SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial_width, int G, bool partial_rows,
                      int slots, int min_blocks)
 {
     SlicePlan p{0, 1, 0, 0};
@@ -103,7 +107,7 @@ SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial
     int force = -1;
     if (const char* e = std::getenv("DLSPM_SLICES")) force = std::atoi(e);
     const long long bytes = (long long)K * width * (long long)sizeof(float) * operands;
-    long long slices = (bytes + kSliceBytes - 1) / kSliceBytes;
+    long long slices = (bytes * (partial_rows ? kSlicesPer8MiBPartial : kSlicesPer8MiB) + (8ll << 20) - 1) / (8ll << 20);
     if (slices > kSliceMaxSlices) slices = kSliceMaxSlices;
     // Slices that leave a row its minimum share: 16 nonzeros per slice for dense rows of 256 floats and more, in
     // inverse proportion more for narrower ones (measured with D = 64: 28 per slice lost 20 %, 48 and more gained; with
@@ -122,7 +126,7 @@ SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial
     if (slices < 2) return p;
     p.slices = (int)slices;
     int W = 4;
-    choose_split(M, col_tiles, (int)(nnz / slices), SplitRule{min_blocks, 4, slots, false}, false, W, p.R);
+    choose_split(M, 1, (int)(nnz / slices), SplitRule{min_blocks, 4, slots, false}, false, W, p.R);
     if (W != 4) p.R = 1;  // only four-wave workgroups are built for this schedule
     p.bounds_bytes = (((size_t)(slices + 1) * M * sizeof(int)) + 255) / 256 * 256;
     p.bytes = p.bounds_bytes + (size_t)slices * M * (size_t)partial_width * sizeof(float);
@@ -227,7 +231,7 @@ static SlicePlan spmm_slice_plan(int M, int K, int N, int nnz, const SpmmShape& 
     // and the workgroups of one (slice, tile) pair should fill the device by themselves, or it gathers from several
     // slabs at once: rows per workgroup as if there were one tile (4096 x 65536, N = 3136, 25 tiles of 128, 131 or
     // 656 nonzeros per row: 856 -> 716 us and 2320 -> 2133 us)
-    SlicePlan p = slice_plan(M, K, N < tw ? N : tw, nnz, 1, 0, s.vec == 4 ? s.G : 0, 1, kWave / s.G, 2048);
+    SlicePlan p = slice_plan(M, K, N < tw ? N : tw, nnz, 1, 0, s.vec == 4 ? s.G : 0, true, kWave / s.G, 2048);
     p.bytes = p.slices > 0 ? p.bounds_bytes + (size_t)p.slices * M * (size_t)N * sizeof(float) : 0;
     return p;
 }
@@ -235,12 +239,12 @@ static SlicePlan fused_slice_plan(int M, int K, int D, int nnz, const FusedShape
 {
     const int tw = s.G * s.vec * s.V;
     const bool built = s.vec == 4 && s.G1 == 8 && s.DS > 0 && tw >= D;  // the widths the sliced kernels are built for (17 .. 512)
-    return slice_plan(M, K, D, nnz, 2, D, built ? s.G : 0, 1, kWave / s.G, 512);
+    return slice_plan(M, K, D, nnz, 2, D, built ? s.G : 0, true, kWave / s.G, 512);
 }
 static SlicePlan sddmm_slice_plan(int M, int K, int D, int nnz, const SddmmShape& s)
 {
     const bool built = s.vec == 4 && s.G1 == 8 && s.DS >= 1;  // 16 < D <= 512
-    return slice_plan(M, K, D, nnz, 1, 0, built ? kWave : 0, 1, kWave / s.G1, 512);
+    return slice_plan(M, K, D, nnz, 1, 0, built ? kWave : 0, false, kWave / s.G1, 512);
 }
 
 }  // namespace dlspm

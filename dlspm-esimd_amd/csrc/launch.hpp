@@ -66,8 +66,9 @@ struct SlicePlan {
     size_t bytes;
 };
 // `operands`: dense operands gathered per nonzero (1 SpMM and SDDMM, 2 fused); `partial_width`: floats of a partial
-// row (0 for SDDMM, whose results need no adding up); G, col_tiles, slots: the op's lane layout
-SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial_width, int G, long long col_tiles,
+// row that `bytes` accounts for (0: SDDMM has none, SpMM adds its own); `partial_rows`: the op writes partial rows at
+// all (its slices are then a third larger); G, slots: the op's lane layout
+SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial_width, int G, bool partial_rows,
                      int slots, int min_blocks);
 hipError_t slice_bounds_launch(int M, int K, int slices, const int* row_offsets, const int* col_indices, int* bounds,
                                hipStream_t stream);

@@ -84,7 +84,7 @@ def test_column_tiles_narrow_with_the_height_of_the_dense_operand(dl):
         assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (128, tiles)
     assert dl.describe_launch(dl.OP_SPMM, 8192, 1 << 15, 1024, 8192 * 63, with_workspace=True)["col_tiles"] == 2
     # the workgroups of one (slice, tile) pair fill the device by themselves: rows per workgroup from M alone
-    assert dl.describe_slices(dl.OP_SPMM, 8192, 1 << 15, 1024, 8192 * 300) == (8, 4)
+    assert dl.describe_slices(dl.OP_SPMM, 8192, 1 << 15, 1024, 8192 * 300) == (6, 4)
     assert dl.describe_slices(dl.OP_SPMM, 4096, 1 << 16, 3136, 4096 * 131) == (4, 2)
     assert dl.describe_slices(dl.OP_SPMM, 2048, 1 << 17, 512, 2048 * 655) == (16, 1)
     # the same where one wave could cover the whole width, once B exceeds the L2; tiles below 128 columns only for a
@@ -110,15 +110,15 @@ def test_column_tiles_narrow_with_the_height_of_the_dense_operand(dl):
 
 
 def test_column_sliced_schedule_rule(dl):
-    """Slices of at most 2 MiB of gathered dense operand, only when the operand exceeds 4 MiB, the dense rows are wide
+    """Slices of at most 8/3 MiB of gathered dense operand (2 MiB in SDDMM, which writes no partial rows), only when the operand exceeds 4 MiB, the dense rows are wide
     and a row keeps at least 16 nonzeros per slice on average; the workspace then holds the boundaries and the
     partial rows of every slice."""
     M = K = 8192
     nnz = M * 800
-    assert dl.describe_slices(dl.OP_FUSED, M, K, 128, nnz)[0] == 4      # Kmat + V: 8 MiB
-    assert dl.describe_slices(dl.OP_FUSED, M, K, 256, nnz)[0] == 8      # 16 MiB
+    assert dl.describe_slices(dl.OP_FUSED, M, K, 128, nnz)[0] == 3      # Kmat + V: 8 MiB
+    assert dl.describe_slices(dl.OP_FUSED, M, K, 256, nnz)[0] == 6      # 16 MiB
     assert dl.describe_slices(dl.OP_FUSED, M, K, 64, nnz)[0] == 0       # 4 MiB of narrow dense rows: left alone
-    assert dl.describe_slices(dl.OP_FUSED, M, 4 * K, 64, nnz)[0] == 8   # sparse attention over 32768 keys, D = 64: 16 MiB
+    assert dl.describe_slices(dl.OP_FUSED, M, 4 * K, 64, nnz)[0] == 6   # sparse attention over 32768 keys, D = 64: 16 MiB
     assert dl.describe_slices(dl.OP_FUSED, M, 4 * K, 64, M * 200)[0] == 3   # ... a row keeps 64 nonzeros per slice at D = 64
     assert dl.describe_slices(dl.OP_FUSED, M, 4 * K, 16, nnz)[0] == 0   # D <= 16: not built for it
     assert dl.describe_slices(dl.OP_FUSED, M, K // 2, 128, nnz)[0] == 2 # 4 MiB just fills the L2: in two for long rows
@@ -128,27 +128,27 @@ def test_column_sliced_schedule_rule(dl):
     assert dl.describe_slices(dl.OP_SPMM, M, K, 256, M * 400)[0] == 0   # ... 200 nonzeros per slice: not at exactly 4 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, K, 128, nnz)[0] == 2       # one tile of 4 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, K, 100, nnz)[0] == 0       # 3.1 MiB: fits
-    assert dl.describe_slices(dl.OP_SPMM, M, 2 * K, 256, nnz)[0] == 4   # 16384 x 128 floats per tile: 8 MiB
-    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, nnz)[0] == 8   # taller: tiles of 128 all the same, 16 MiB each
-    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 16, 32, nnz)[0] == 4  # narrow dense rows, very tall B: 8 MiB
+    assert dl.describe_slices(dl.OP_SPMM, M, 2 * K, 256, nnz)[0] == 3   # 16384 x 128 floats per tile: 8 MiB
+    assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, nnz)[0] == 6   # taller: tiles of 128 all the same, 16 MiB each
+    assert dl.describe_slices(dl.OP_SPMM, M, 1 << 16, 32, nnz)[0] == 3  # narrow dense rows, very tall B: 8 MiB
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 16, 32, M * 300)[0] == 2  # ... 128 nonzeros per slice at N = 32
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 20, 3, nnz)[0] == 0   # fewer than four columns: not built for them
     # a row keeps at least max(16, 4096 / width) nonzeros per slice: 16 at 256 columns, 32 in tiles of 128
     assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 140)[0] == 4   # 140 nonzeros per row: four slices of 35
     assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 70)[0] == 2    # 70 per row: two
     assert dl.describe_slices(dl.OP_SPMM, 2 * M, 4 * K, 256, 2 * M * 60)[0] == 3  # below 64 per row: one tile of 256, three slices of 20
-    assert dl.describe_slices(dl.OP_SPMM, M, 2 * K, 256, M * 140)[0] == 4   # tiles of 128: four slices of 35
+    assert dl.describe_slices(dl.OP_SPMM, M, 2 * K, 256, M * 140)[0] == 3   # 8 MiB per tile: three, whatever the rows allow
     assert dl.describe_slices(dl.OP_SPMM, M, 2 * K, 256, M * 70)[0] == 2    # 70 per row: two
     assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 40)[0] == 0    # 40 per row, 0.33 M nonzeros: too small
     assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 64)[0] == 2  # 2.1 M nonzeros, 64 per row
     assert dl.describe_slices(dl.OP_SPMM, 4 * M, 4 * K, 256, 4 * M * 30)[0] == 0  # 30 per row: not even two of 16
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, nnz)[0] == 16      # 128 MiB: the most slices there are
     assert dl.describe_slices(dl.OP_SPMM, M, 1 << 17, 256, M * 100)[0] == 3   # ... but a row keeps 32 nonzeros per slice
-    assert dl.describe_slices(dl.OP_SDDMM, M, K, 256, nnz)[0] == 4      # rhs: 8 MiB; only the boundaries need memory
+    assert dl.describe_slices(dl.OP_SDDMM, M, K, 256, nnz)[0] == 4      # rhs: 8 MiB in slices of 2 MiB (no partial rows); only the boundaries need memory
     assert dl.workspace_bytes(dl.OP_SDDMM, M, K, 256, nnz) == -(-5 * M * 4 // 256) * 256
     assert dl.describe_slices(dl.OP_SDDMM, M, K, 100, nnz)[0] == 0 and dl.workspace_bytes(dl.OP_SDDMM, M, K, 100, nnz) == 0
     slices, R = dl.describe_slices(dl.OP_FUSED, M, K, 256, nnz)
-    assert R == 4                                                       # 100 nonzeros per row and slice
+    assert R == 2                                                       # 133 nonzeros per row and slice
     bounds = -(-(slices + 1) * M * 4 // 256) * 256
     assert dl.workspace_bytes(dl.OP_FUSED, M, K, 256, nnz) == bounds + slices * M * 256 * 4
     # below the sliced rule the flat schedule's size is reported as before

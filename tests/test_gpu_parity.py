@@ -380,8 +380,8 @@ def test_flat_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
 @pytest.mark.parametrize("sigma", [0.0, 1.5])
 def test_column_sliced_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
     """Dense operands of 16 MiB (SpMM, SDDMM) and 32 MiB (fused) at K = 16384, N = D = 256: a call WITH workspace takes
-    the column-sliced schedule by the library's own rule (SpMM: 4 slices of each of its two column tiles; SDDMM 8, fused
-    16 slices); all three ops against the multi-threaded oracle, on near-uniform and on heavily skewed rows, and the
+    the column-sliced schedule by the library's own rule (SpMM: 3 slices of each of its two column tiles; SDDMM 8, fused
+    12 slices); all three ops against the multi-threaded oracle, on near-uniform and on heavily skewed rows, and the
     same calls without workspace must agree."""
     torch = torch_cuda
     M, K, N = 4096, 16384, 256
@@ -394,9 +394,9 @@ def test_column_sliced_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
     B = dl.fill("uniform", 74, (K, N), -1.0, 1.0)
     Q = dl.fill("normal", 75, (M, N), 0.0, 1.0)
     ro_d, ci_d, va_d, B_d, Q_d = (dev(torch, x) for x in (ro, ci, va, B, Q))
-    assert dl.describe_slices(dl.OP_SPMM, M, K, N, nnz)[0] == 4 and dl.describe_launch(dl.OP_SPMM, M, K, N, nnz, with_workspace=True)["col_tiles"] == 2
+    assert dl.describe_slices(dl.OP_SPMM, M, K, N, nnz)[0] == 3 and dl.describe_launch(dl.OP_SPMM, M, K, N, nnz, with_workspace=True)["col_tiles"] == 2
     assert dl.describe_slices(dl.OP_SDDMM, M, K, N, nnz)[0] == 8
-    assert dl.describe_slices(dl.OP_FUSED, M, K, N, nnz)[0] == 16
+    assert dl.describe_slices(dl.OP_FUSED, M, K, N, nnz)[0] == 12
 
     ws = torch.empty(dl.workspace_bytes(dl.OP_SPMM, M, K, N, nnz), dtype=torch.uint8, device="cuda")
     got = dl.spmm(ro_d, ci_d, va_d, B_d, K=K, workspace=ws)
