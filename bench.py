@@ -37,6 +37,7 @@ def parse():
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (default 2, the headline)")
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of one HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-plan", action="store_true", help="SpMM: launch in matrix order, without the row plan")
     ap.add_argument("--all-configs", action="store_true", help="also time the other four configurations (short runs)")
     ap.add_argument("--pmc-calib", action="store_true",
                     help="also run a plain 256 MiB device copy a few times: the known-size kernel that rocprofv3 --pmc "
@@ -44,8 +45,10 @@ def parse():
     return ap.parse_args()
 
 
-def make_step(dl, torch, c):
-    """Uploads configuration c and returns (step_fn, output tensor)."""
+def make_step(dl, torch, c, use_plan=True, info=None):
+    """Uploads configuration c and returns (step_fn, output tensor). What a caller does once per matrix happens here,
+    outside the timed steps: one look at the row lengths and, for SpMM on uneven rows, the row plan (its build time
+    goes to info["plan_build_ms"])."""
     d = lambda a: torch.from_numpy(a).cuda()
     ro, ci = d(c["row_offsets"]), d(c["col_indices"])
     # the caller owns the workspace; the library asks for none at the sizes of the five configurations
@@ -54,6 +57,14 @@ def make_step(dl, torch, c):
     if c["op"] == dl.OP_SPMM:
         va, B = d(c["values"]), d(c["d0"])
         out = torch.empty((c["M"], c["N"]), dtype=torch.float32, device="cuda")
+        longest, _ = dl.csr_row_stats(ro)
+        if use_plan and ws is None and dl.row_plan_advice(c["M"], c["K"], c["N"], c["nnz"], longest):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            plan = dl.row_plan(ro)
+            if info is not None:
+                info["plan_build_ms"] = round((time.perf_counter() - t0) * 1e3, 3)
+            return (lambda: dl.spmm(ro, ci, va, B, K=c["K"], out=out, plan=plan)), out
         return (lambda: dl.spmm(ro, ci, va, B, K=c["K"], out=out, workspace=ws)), out
     if c["op"] == dl.OP_SDDMM:
         lhs, rhs = d(c["d0"]), d(c["d1"])
@@ -169,7 +180,8 @@ def main():
 
     c = dl.make_config(args.config)
     acct = dl.account(c["op"], c["M"], c["K"], c["N"], c["nnz"])
-    step, out = make_step(dl, torch, c)
+    info = {}
+    step, out = make_step(dl, torch, c, not args.no_plan, info)
     wall_s, evt_s, mode = time_steps(torch, step, args.steps, args.warmup, not args.no_graph)
     per_launch_s = evt_s / args.steps
     warm_med, warm_min = single_launch_us(torch, step, 30, flush=False)
@@ -190,7 +202,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic (seeded generator, seed 1000+cfg)",
         "config": {"workload": c["name"], "op": ["spmm", "sddmm", "fused"][c["op"]], "M": c["M"], "K": c["K"],
-                   "N_or_D": c["N"], "nnz": c["nnz"], "launch": mode},
+                   "N_or_D": c["N"], "nnz": c["nnz"], "launch": mode, "row_plan": "plan_build_ms" in info},
         "roofline": {"bound": "hbm", "achieved": round(acct["algorithmic_bytes"] / per_launch_s / 1e9, 2),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(acct["algorithmic_bytes"] / per_launch_s / 1e9 / HBM_PEAK_GBPS, 5),
@@ -202,6 +214,13 @@ def main():
         "warm_us": {"median": round(warm_med, 2), "min": round(warm_min, 2)},
         "cold_us": {"median": round(cold_med, 2), "min": round(cold_min, 2)},
     }
+
+    if "plan_build_ms" in info:
+        # the same launches in matrix order (no plan), and what the plan cost once
+        plain, _ = make_step(dl, torch, c, False)
+        _, ev, _ = time_steps(torch, plain, min(args.steps, 500), min(args.warmup, 50), not args.no_graph)
+        result["row_plan"] = {"build_ms_once_per_matrix": info["plan_build_ms"],
+                              "launch_us_without_plan": round(ev / min(args.steps, 500) * 1e6, 3)}
 
     if not args.no_cpu:
         result["cpu_baseline"], ref = cpu_baseline(dl, c, acct)

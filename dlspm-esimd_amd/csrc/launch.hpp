@@ -77,6 +77,10 @@ hipError_t slice_sum_launch(long long count, int slices, const float* partial, f
 // narrow_tiles: the call passes no workspace memory (column tiles below 128 columns are then allowed)
 SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles);
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
+// Row plan (3 x M ints on the device: first nonzero, end and row number of the row that workgroup i works on): only for
+// shapes of one row per four-wave workgroup and one column tile
+bool spmm_plan_applies(const SpmmShape& s, int N);
+hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int* plan, hipStream_t stream);
 hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPlan& plan, float* partial,
                             hipStream_t stream);
 hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const SlicePlan& plan, void* workspace,

@@ -56,13 +56,16 @@ __device__ __forceinline__ void spmm_segment(Vec<VEC>* acc, int p, int q, const 
 // SLICED = true: row i owns [row_offsets[i], row_ends[i]), a part of the CSR row (its columns inside one range of
 // columns), so the rows of a block are not contiguous in memory: the split then works on the running sum of their
 // lengths ("virtual" offsets, 0 at the block's first row) and every segment is shifted back to where it lies.
-template <int VEC, int G, int V, int W, int R, bool SLICED>
+// PLANNED (with SLICED and R == 1): workgroup i works on row row_ids[i], whose nonzeros are [row_offsets[i], row_ends[i]):
+// a row plan hands the rows out in an order of its own.
+template <int VEC, int G, int V, int W, int R, bool SLICED, bool PLANNED = false>
 __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles, int tile_major,
                                            const int* __restrict__ row_offsets,
                                            const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                            const float* __restrict__ values, const float* __restrict__ B,
-                                           float* __restrict__ C)
+                                           float* __restrict__ C, const int* __restrict__ row_ids = nullptr, int nnz = 0)
 {
+    static_assert(!PLANNED || (SLICED && R == 1), "a row plan names one row per workgroup");
     constexpr int TW = G * VEC * V;  // columns of C covered by one wave
     using VecT = Vec<VEC>;
 
@@ -91,6 +94,7 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
     }
     const int r0 = rb * R;
     const int nr = min(R, M - r0);
+    int out_row0 = r0;  // row of C that the block's first row is stored to
 
     // The block's R + 1 row offsets, without LDS or a barrier: with R == 1 they are the same two words for every
     // lane (scalar loads); otherwise lane i of every wave holds offset i and v_readlane picks one.
@@ -107,6 +111,12 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
         if constexpr (R == 1) {
             start_lo = row_offsets[r0];
             off_hi = row_ends[r0] - start_lo;
+            if constexpr (PLANNED) {
+                // a plan that was built for another matrix must not take the kernel outside the arrays
+                out_row0 = min(max(row_ids[r0], 0), M - 1);
+                start_lo = min(max(start_lo, 0), nnz);
+                off_hi = min(max(off_hi, 0), nnz - start_lo);
+            }
         } else {
             static_assert(R + 1 <= 32, "the running sum covers 32 lanes");
             const int i = r0 + min(lane, nr - 1);
@@ -163,7 +173,7 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
             const bool whole_row = (p == rs) && (q == re);
             if (slot == 0) {
                 if (whole_row) {
-                    float* crow = C + (size_t)(r0 + r) * N;
+                    float* crow = C + (size_t)(out_row0 + r) * N;
 #pragma unroll
                     for (int v = 0; v < V; ++v)
                         if (act[v]) acc[v].gstore(crow + colv[v]);
@@ -184,7 +194,7 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
             if (slot == 0) {
                 for (int r = w; r < nr; r += W) {
                     if (s_off(r) != s_off(r + 1)) continue;
-                    float* crow = C + (size_t)(r0 + r) * N;
+                    float* crow = C + (size_t)(out_row0 + r) * N;
 #pragma unroll
                     for (int v = 0; v < V; ++v)
                         if (act[v]) VecT::zero().gstore(crow + colv[v]);
@@ -198,7 +208,7 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
                 for (int r = w; r < nr; r += W) {
                     const int len = s_off(r + 1) - s_off(r);
                     const int part = (len + m - 1) / m;
-                    float* crow = C + (size_t)(r0 + r) * N;
+                    float* crow = C + (size_t)(out_row0 + r) * N;
                     if (len > 0 && len <= part) continue;  // one wave held the whole row and stored it
 #pragma unroll
                     for (int v = 0; v < V; ++v) {
@@ -219,7 +229,7 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
         // one row per workgroup: wave x had nonzeros iff x * per < T, and wave 0 adds them up (no division, the
         // partial sums of all waves are requested from LDS together)
         if (w == 0 && slot == 0) {
-            float* crow = C + (size_t)r0 * N;
+            float* crow = C + (size_t)out_row0 * N;
             if (T == 0) {
 #pragma unroll
                 for (int v = 0; v < V; ++v)
@@ -242,7 +252,7 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
         for (int r = w; r < nr; r += W) {
             const int rs = s_off(r);
             const int re = s_off(r + 1);
-            float* crow = C + (size_t)(r0 + r) * N;
+            float* crow = C + (size_t)(out_row0 + r) * N;
             if (rs == re) {
 #pragma unroll
                 for (int v = 0; v < V; ++v)
@@ -290,6 +300,18 @@ __global__ __launch_bounds__(4 * 64) void spmm_sliced_kernel(int M, int N, int c
     const int bid = (int)blockIdx.x - sl * slice_blocks;
     spmm_block<VEC, G, V, 4, R, true>(bid, M, N, col_tiles, tile_major, bounds + (size_t)sl * M,
                                       bounds + (size_t)(sl + 1) * M, col_indices, values, B, partial + (size_t)sl * M * N);
+}
+
+// Row plan: workgroup i works on the whole row rows[i] = [starts[i], ends[i]) of the CSR matrix (one row per four-wave
+// workgroup, one column tile).
+template <int VEC, int G, int V>
+__global__ __launch_bounds__(4 * 64) void spmm_planned_kernel(int M, int N, int nnz, const int* __restrict__ starts,
+                                                              const int* __restrict__ ends, const int* __restrict__ rows,
+                                                              const int* __restrict__ col_indices,
+                                                              const float* __restrict__ values,
+                                                              const float* __restrict__ B, float* __restrict__ C)
+{
+    spmm_block<VEC, G, V, 4, 1, true, true>((int)blockIdx.x, M, N, 1, 0, starts, ends, col_indices, values, B, C, rows, nnz);
 }
 
 // ---- host side --------------------------------------------------------------------------------------
@@ -568,6 +590,32 @@ hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const Slice
 #undef DLSPM_SLICED
     if (e != hipSuccess) return e;
     return slice_sum_launch((long long)x.M * x.N, plan.slices, partial, x.C, stream);
+}
+
+// ---- row plan ---------------------------------------------------------------------------------------
+
+bool spmm_plan_applies(const SpmmShape& s, int N)
+{
+    return s.vec == 4 && s.W == 4 && s.R == 1 && s.G * s.vec * s.V >= N;  // one row per workgroup, one column tile
+}
+
+hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int* plan, hipStream_t stream)
+{
+    if (x.M <= 0) return hipSuccess;
+    const int *starts = plan, *ends = plan + x.M, *rows = plan + 2 * (size_t)x.M;
+#define DLSPM_PLANNED(g_, v_)                                                                                          \
+    if (s.G == g_ && s.V == v_) {                                                                                      \
+        hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M, x.N,   \
+                           x.nnz, starts, ends, rows, x.col_indices, x.values, x.B, x.C);                                     \
+        return hipGetLastError();                                                                                      \
+    }
+    DLSPM_PLANNED(64, 2)
+    DLSPM_PLANNED(64, 1)
+    DLSPM_PLANNED(32, 1)
+    DLSPM_PLANNED(16, 1)
+    DLSPM_PLANNED(8, 1)
+#undef DLSPM_PLANNED
+    return hipErrorInvalidValue;
 }
 
 }  // namespace dlspm

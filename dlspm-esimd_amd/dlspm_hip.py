@@ -43,6 +43,10 @@ EXPORTS = (
     "dlspm_describe_slices",
     "dlspm_workspace_advice",
     "dlspm_csr_row_stats",
+    "dlspm_row_plan_bytes",
+    "dlspm_row_plan_advice",
+    "dlspm_row_plan_build",
+    "spmm_csr_f32_planned",
     "dlspm_status_string",
     "dlspm_last_hip_error",
     "dlspm_version",
@@ -86,6 +90,14 @@ def lib() -> ctypes.CDLL:
         L.dlspm_describe_launch.restype = ci
         L.dlspm_csr_row_stats.argtypes = [ci, vp, vp, ctypes.POINTER(ci), ctypes.POINTER(ci)]
         L.dlspm_csr_row_stats.restype = ci
+        L.dlspm_row_plan_bytes.argtypes = [ci]
+        L.dlspm_row_plan_bytes.restype = sz
+        L.dlspm_row_plan_advice.argtypes = [ci, ci, ci, ci, ci]
+        L.dlspm_row_plan_advice.restype = ci
+        L.dlspm_row_plan_build.argtypes = [ci, vp, vp, sz, vp]
+        L.dlspm_row_plan_build.restype = ci
+        L.spmm_csr_f32_planned.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.spmm_csr_f32_planned.restype = ci
         L.dlspm_status_string.argtypes = [ci]
         L.dlspm_status_string.restype = ctypes.c_char_p
         L.dlspm_last_hip_error.restype = ci
@@ -122,9 +134,28 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None):
+def row_plan_advice(M, K, N, nnz, max_row_len=-1) -> bool:
+    """Whether a row plan is worth building for an SpMM of these sizes (see dlspm_row_plan_advice)."""
+    return bool(lib().dlspm_row_plan_advice(M, K, N, nnz, max_row_len))
+
+
+def row_plan(row_offsets):
+    """The row plan of one matrix (an int32 GPU tensor of 3 * M entries) for spmm(..., plan=...); synchronises."""
+    import torch
+
+    M = row_offsets.numel() - 1
+    plan = torch.empty((lib().dlspm_row_plan_bytes(M) // 4,), dtype=torch.int32, device=row_offsets.device)
+    st = lib().dlspm_row_plan_build(M, _ptr(row_offsets, torch.int32, "row_offsets"), _ptr(plan, torch.int32, "plan"),
+                                    plan.numel() * 4, _stream())
+    if st != OK:
+        raise DlspmError(st, "dlspm_row_plan_build")
+    return plan
+
+
+def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None, plan=None):
     """C = A_csr @ B on the current stream. row_offsets/col_indices int32, values/B float32, all on the GPU.
-    `workspace`: optional GPU tensor of at least workspace_bytes(OP_SPMM, ...) bytes, or ROWS_EVEN."""
+    `workspace`: optional GPU tensor of at least workspace_bytes(OP_SPMM, ...) bytes, or ROWS_EVEN.
+    `plan`: optional row plan of this matrix (row_plan()), instead of a workspace."""
     import torch
 
     M = row_offsets.numel() - 1
@@ -133,6 +164,17 @@ def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None):
     K = Kd if K is None else K
     if out is None:
         out = torch.empty((M, N), dtype=torch.float32, device=B.device)
+    if plan is not None:
+        if workspace is not None:
+            raise ValueError("pass a row plan or a workspace, not both")
+        st = lib().spmm_csr_f32_planned(M, K, N, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
+                                        _ptr(col_indices, torch.int32, "col_indices"),
+                                        _ptr(values, torch.float32, "values"), _ptr(B, torch.float32, "B"),
+                                        _ptr(out, torch.float32, "C"), _ptr(plan, torch.int32, "plan"),
+                                        plan.numel() * 4, _stream())
+        if st != OK:
+            raise DlspmError(st, "spmm_csr_f32_planned")
+        return out
     wp, wb = _workspace(workspace)
     st = lib().spmm_csr_f32(M, K, N, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
                             _ptr(col_indices, torch.int32, "col_indices"), _ptr(values, torch.float32, "values"),

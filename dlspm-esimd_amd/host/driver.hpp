@@ -209,6 +209,7 @@ struct Options {
     // at most one and a half times the mean;
     // --workspace: always the memory, --no-workspace: always NULL
     enum Workspace { kAuto, kAlways, kNever } workspace = kAuto;
+    bool plan = true;  // SpMM: build a row plan where dlspm_row_plan_advice says so (--no-plan: never)
     std::string csv, dump;
     double tol = 1e-4;  // relative Frobenius error allowed between the kernel and the check kernel
 };
@@ -221,13 +222,15 @@ struct WorkspaceChoice {
     void* arg(void* buffer) const { return rows_even ? DLSPM_ROWS_EVEN : bytes ? buffer : nullptr; }
 };
 inline WorkspaceChoice workspace_to_pass(const Options& opt, int op, int M, int K, int width, int nnz,
-                                         const int* row_offsets_dev)
+                                         const int* row_offsets_dev, int* longest_out = nullptr)
 {
     WorkspaceChoice c;
+    if (longest_out) *longest_out = -1;
     if (opt.workspace == Options::kNever || M <= 0 || nnz <= 0) return c;
     const size_t want = dlspm_workspace_bytes(op, M, K, width, nnz);
     int longest = 0, empty = 0;
     if (dlspm_csr_row_stats(M, row_offsets_dev, nullptr, &longest, &empty) != DLSPM_OK) throw std::runtime_error("dlspm_csr_row_stats failed");
+    if (longest_out) *longest_out = longest;
     const int advice = dlspm_workspace_advice(op, M, K, width, nnz, longest);
     int slices = 0;
     (void)dlspm_describe_slices(op, M, K, width, nnz, &slices, nullptr);
@@ -367,7 +370,7 @@ inline std::string usage(const char* app, const char* width)
       << "                                                     --sigma: lognormal row lengths, skewed)\n"
       << "       " << app << " --sweep [--max-m M]                  the 12 x {32,128} x {0.3,0.2,0.1} benchmark grid\n"
       << "       " << app << " --cfg <id>                           a seeded benchmark configuration (1..5)\n"
-      << "options: --iters n (20)  --warmup n (5)  --cold  --csv <file>  --dump <dir>  --tol x (1e-4)  --workspace | --no-workspace";
+      << "options: --iters n (20)  --warmup n (5)  --cold  --csv <file>  --dump <dir>  --tol x (1e-4)  --workspace | --no-workspace  --no-plan";
     return u.str();
 }
 
@@ -394,6 +397,7 @@ inline Cli parse_cli(int argc, char** argv, const char* app, const char* width)
         else if (a == "--sigma") { need(i, 1); const double sg = std::stod(argv[++i]); if (!cli.cases.empty()) cli.cases.back().sigma = sg; }
         else if (a == "--no-workspace") cli.opt.workspace = Options::kNever;
         else if (a == "--workspace") cli.opt.workspace = Options::kAlways;
+        else if (a == "--no-plan") cli.opt.plan = false;
         else if (a == "--sweep") sweep = true;
         else if (a == "--max-m") { need(i, 1); max_m = std::stoi(argv[++i]); }
         else if (a == "--batch") {

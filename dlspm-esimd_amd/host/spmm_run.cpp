@@ -2,6 +2,8 @@
 // Takes the place of the reference's SpMM drivers: single synthetic matrix (SPMM/spmm-esimd-v1.cpp:281-466),
 // in-process sweep (SPMM/spmm-esimd-allbenchs2.cpp:56-266), from file (SPMM/spmm-esimd-fromfile2.cpp:86-320) and
 // the shell loop over DLMC files (SPMM/batch-run-spmm_fromfile:16-46). See driver.hpp for the shared parts.
+#include <chrono>
+
 #include "driver.hpp"
 
 using namespace dlspm;
@@ -41,10 +43,23 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     DLSPM_HIP_CHECK(hipMemset(C_d.p, 0xFF, (size_t)M * N * sizeof(float)));  // NaN pattern: every element must be written
 
     // the caller owns the workspace, as it owns every other buffer: 0 bytes for small problems
-    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_SPMM, M, K, N, nnz, ro_d.p);
+    int longest = -1;
+    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_SPMM, M, K, N, nnz, ro_d.p, &longest);
     DevBuf<char> ws(wc.bytes);
     if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
+    // uneven rows, one row per workgroup, nothing to pass as workspace: a row plan, built once per matrix like the look
+    // at the row lengths, hands the rows out longest first
+    const bool planned = opt.plan && opt.workspace == Options::kAuto && longest >= 0 && !wc.bytes && !wc.rows_even &&
+                         dlspm_row_plan_advice(M, K, N, nnz, longest) == 1;
+    DevBuf<char> plan(planned ? dlspm_row_plan_bytes(M) : 0);
+    if (planned) {
+        const auto t0 = std::chrono::steady_clock::now();
+        if (dlspm_row_plan_build(M, ro_d.p, plan.p, plan.n, nullptr) != DLSPM_OK) throw std::runtime_error("dlspm_row_plan_build failed");
+        const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        std::printf("row plan: %zu bytes, built in %.3f ms (once per matrix)\n", plan.n, ms);
+    }
     const Timing t = time_launches(opt, [&]() {
+        if (planned) return spmm_csr_f32_planned(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, plan.p, plan.n, nullptr);
         return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, wc.arg(ws.p), wc.bytes, nullptr);
     });
     hipLaunchKernelGGL(check_spmm_kernel, dim3(blocks_for((long long)M * N)), dim3(256), 0, nullptr, M, N, ro_d.p, ci_d.p,

@@ -186,6 +186,30 @@ def test_workspace_advice(dl):
     assert A(dl.OP_SPMM, 0, 0, 0, 0, 0) == dl.PASS_NULL and A(7, M, K, 128, nnz, mean) == dl.PASS_NULL
 
 
+def test_row_plan_host_side(dl):
+    """Size, advice and argument checks of the row plan need no GPU."""
+    L = dl.lib()
+    assert L.dlspm_row_plan_bytes(2048) == 3 * 2048 * 4 and L.dlspm_row_plan_bytes(0) == 0 and L.dlspm_row_plan_bytes(-5) == 0
+    A = dl.row_plan_advice
+    assert A(2048, 512, 256, 105687, 312)            # the headline configuration: uneven rows, one row per workgroup
+    assert A(2048, 512, 256, 105687, -1)             # rows unknown: nothing better to pass
+    assert not A(2048, 512, 256, 105687, 60)         # even rows: another order gains nothing
+    assert not A(4096, 1024, 256, 4096 * 100, 400)   # rows grouped two per workgroup
+    assert not A(600, 512, 784, 600 * 60, 300)       # column tiles
+    assert not A(2048, 512, 3, 105687, 312)          # fewer than four columns
+    assert not A(16384, 4096, 128, 16384 * 400, 4000)  # large and uneven: the flat schedule's workspace instead
+    assert not A(0, 0, 0, 0, 0)
+    bogus = ctypes.c_void_p(256)   # never dereferenced: the checks come first
+    assert L.dlspm_row_plan_build(-1, bogus, bogus, 0, None) == dl.E_INVALID_ARG
+    assert L.dlspm_row_plan_build(8, None, bogus, 96, None) == dl.E_INVALID_ARG
+    assert L.dlspm_row_plan_build(8, bogus, bogus, 95, None) == dl.E_WORKSPACE
+    assert L.dlspm_row_plan_build(0, None, None, 0, None) == dl.OK
+    assert L.spmm_csr_f32_planned(-1, 1, 1, 0, None, None, None, None, None, bogus, 0, None) == dl.E_INVALID_ARG
+    assert L.spmm_csr_f32_planned(2, 2, 2, 5, None, None, None, None, None, bogus, 24, None) == dl.E_INVALID_ARG
+    assert L.spmm_csr_f32_planned(2, 2, 2, 1, bogus, bogus, bogus, bogus, bogus, bogus, 23, None) == dl.E_WORKSPACE
+    assert L.spmm_csr_f32_planned(2, 2, 2, 1, None, None, None, None, None, None, 0, None) == dl.E_INVALID_ARG  # as spmm_csr_f32
+
+
 def test_library_exports_every_declared_symbol(dl):
     lib = ctypes.CDLL(dl.LIB_PATH)
     for name in declared_functions():

@@ -479,6 +479,73 @@ def test_exact_integer_properties_at_large_size(torch_cuda, dl):
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
+def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle):
+    """spmm_csr_f32_planned hands the rows to the workgroups in the plan's order (longest first) and must return the
+    bits of spmm_csr_f32 with a NULL workspace: every row is summed by the same workgroup shape. The plan itself is a
+    permutation of the rows with each row's own offsets. Shapes that do not run one row per workgroup ignore the plan."""
+    torch = torch_cuda
+    rng = np.random.default_rng(97)
+    cases = [("cfg2", None), ("cfg1", None), ("cfg4", None),
+             ("skewed", (2049, 600, 256)), ("empty_rows", (300, 512, 128)), ("skewed", (1, 700, 64)),
+             ("skewed", (5000, 2048, 50)), ("uniform", (4096, 1024, 256)), ("skewed", (2048, 512, 3)),
+             ("skewed", (600, 512, 784))]
+    used = 0
+    for kind, shape in cases:
+        if shape is None:
+            c = dl.make_config(int(kind[3]))
+            ro, ci, va, B, K = c["row_offsets"], c["col_indices"], c["values"], c["d0"], c["K"]
+        else:
+            M, K, N = shape
+            ro, ci = random_csr(rng, M, K, kind, 0.12)
+            va = rng.normal(0, 1, ci.size).astype(np.float32)
+            B = rng.normal(0, 1, (K, N)).astype(np.float32)
+        M, N = ro.size - 1, B.shape[1]
+        print(f"row plan case {kind} {M}x{K} N {N} nnz {ci.size}", flush=True)
+        ro_d, ci_d, va_d, B_d = (dev(torch, x) for x in (ro, ci, va, B))
+        plan = dl.row_plan(ro_d)
+        h = plan.cpu().numpy()
+        starts, ends, rows = h[:M], h[M:2 * M], h[2 * M:]
+        assert np.array_equal(np.sort(rows), np.arange(M))
+        assert np.array_equal(starts, ro[rows]) and np.array_equal(ends, ro[rows + 1])
+        lens = ends - starts
+        assert (lens[:min(M, 256)][:-1] >= lens[:min(M, 256)][1:]).all()        # the first group: longest first
+        if M > 2048:
+            assert (lens[2048:][:-1] >= lens[2048:][1:]).all()                   # after the resident part: descending
+        want = dl.spmm(ro_d, ci_d, va_d, B_d, K=K)
+        got = torch.full((M, N), float("nan"), device="cuda")
+        dl.spmm(ro_d, ci_d, va_d, B_d, K=K, out=got, plan=plan)
+        assert torch.equal(got, want), (kind, shape)
+        assert oracle.rel_frobenius(got.cpu().numpy(), oracle.spmm(ro, ci, va, B)) <= TOL
+        sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size)
+        used += int(sh["vec"] == 4 and sh["W"] == 4 and sh["R"] == 1 and sh["col_tiles"] == 1)
+        check_csr_untouched(ro_d, ci_d, ro, ci)
+    assert 5 <= used < len(cases)   # both the planned kernel and the fall-back were exercised
+
+
+def test_stale_row_plan_stays_inside_the_arrays(torch_cuda, dl):
+    """A plan built from another matrix of the same height gives wrong values, but its offsets are clamped to the arrays
+    of the call: the launch completes and every row of C holds finite numbers or was left alone."""
+    torch = torch_cuda
+    rng = np.random.default_rng(98)
+    M, K, N = 2048, 512, 256
+    ro_big, _ = random_csr(rng, M, K, "skewed", 0.3)
+    ro, ci = random_csr(rng, M, K, "skewed", 0.05)
+    assert ro_big[-1] > ro[-1]
+    va = rng.normal(0, 1, ci.size).astype(np.float32)
+    B = rng.normal(0, 1, (K, N)).astype(np.float32)
+    stale = dl.row_plan(dev(torch, ro_big))
+    ro_d, ci_d, va_d, B_d = (dev(torch, x) for x in (ro, ci, va, B))
+    out = torch.zeros(M, N, device="cuda")
+    dl.spmm(ro_d, ci_d, va_d, B_d, K=K, out=out, plan=stale)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    with pytest.raises(dl.DlspmError):   # a plan for fewer rows is refused before any launch
+        dl.spmm(ro_d, ci_d, va_d, B_d, K=K, out=out, plan=stale[:3 * M - 3])
+    # and the right plan right after gives the right bits
+    good = dl.spmm(ro_d, ci_d, va_d, B_d, K=K, plan=dl.row_plan(ro_d))
+    assert torch.equal(good, dl.spmm(ro_d, ci_d, va_d, B_d, K=K))
+
+
 def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
     """All three schedules only enqueue kernels (no memset, no allocation, no synchronisation), so a call may be captured.
     The graph is replayed several times with eager work and synchronisations in between, on changed inputs, and every
@@ -503,6 +570,8 @@ def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
         ws = torch.empty(need, dtype=torch.uint8, device="cuda") if need else None
         ws_s = ws if schedule == "sliced" else None  # SDDMM uses a workspace under the sliced schedule only
         C = torch.empty(M, N, device="cuda")
+        CP = torch.empty(M, N, device="cuda")
+        plan = dl.row_plan(ro_d)
         S = torch.empty(ci.size, device="cuda")
         O = torch.empty(M, N, device="cuda")
         stream = torch.cuda.Stream()
@@ -514,13 +583,17 @@ def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
                 dl.spmm(ro_d, ci_d, va, B, K=K, out=C, workspace=ws)
                 dl.sddmm(ro_d, ci_d, Q, B, out=S, workspace=ws_s)
                 dl.fused(ro_d, ci_d, Q, B, B, 0.5, out=O, workspace=ws)
+                if schedule == "row-block":
+                    dl.spmm(ro_d, ci_d, va, B, K=K, out=CP, plan=plan)   # a planned launch is one kernel too
         for rep in range(4):
             va.copy_(torch.randn(ci.size, device="cuda"))  # eager work between the replays: new inputs
             B.copy_(torch.randn(K, N, device="cuda"))
             torch.cuda.synchronize()
-            C.fill_(float("nan")); S.fill_(float("nan")); O.fill_(float("nan"))
+            C.fill_(float("nan")); S.fill_(float("nan")); O.fill_(float("nan")); CP.fill_(float("nan"))
             graph.replay()
             torch.cuda.synchronize()
+            if schedule == "row-block":
+                assert torch.equal(CP, C), f"replay {rep}, planned launch"
             got = (C.clone(), S.clone(), O.clone())
             want = (dl.spmm(ro_d, ci_d, va, B, K=K, workspace=ws).clone(), dl.sddmm(ro_d, ci_d, Q, B, workspace=ws_s).clone(),
                     dl.fused(ro_d, ci_d, Q, B, B, 0.5, workspace=ws).clone())
