@@ -300,16 +300,36 @@ int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_
     if (e != hipSuccess) return fail_hip(e);
     // Longest rows first: workgroups are dispatched in index order, so the rows that take longest start first and the
     // short ones fill the gaps as compute units free up. The first kResident workgroups all start at once (eight
-    // four-wave workgroups on each of 256 compute units, dealt round-robin): their groups of 256 alternate between
-    // descending and ascending length, so that a compute unit's eight rows add up to about the same work
-    // (2048 x 512, lognormal rows, N = 256: 7.5 us in matrix order, 7.2 us descending, 6.9 us in this order).
-    constexpr int kGroup = 256, kResident = 2048;
+    // four-wave workgroups on each of 256 compute units) and workgroup i of them runs on compute unit i mod 256, so
+    // those rows are packed into 256 bins of equal size, longest row first into the least loaded bin that has
+    // room, and bin b becomes the workgroups b, b + 256, b + 512, ... A compute unit's rows then add up to about
+    // the same number of nonzeros (2048 x 512, lognormal rows, N = 256: 7.6 us in matrix order, 7.2 us longest first,
+    // 7.0 us with the groups of 256 alternating between descending and ascending length, 6.1 us packed; bins of 8,
+    // one per XCD, do nothing: 7.2 us). DLSPM_PLAN_ORDER=1|2 gives the alternating and the plain descending order.
+    constexpr int kBins = 256, kResident = 2048;
     std::vector<int> order((size_t)M);
     for (int i = 0; i < M; ++i) order[i] = i;
     auto len = [&](int i) { return ro[(size_t)i + 1] - ro[i]; };
     std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return len(a) > len(b); });
     const int head = M < kResident ? M : kResident;
-    for (int g = kGroup; g < head; g += 2 * kGroup) std::reverse(order.begin() + g, order.begin() + (g + kGroup < head ? g + kGroup : head));
+    int variant = 0;
+    if (const char* e = std::getenv("DLSPM_PLAN_ORDER")) variant = std::atoi(e);
+    if (variant == 1) {
+        for (int g = kBins; g < head; g += 2 * kBins) std::reverse(order.begin() + g, order.begin() + (g + kBins < head ? g + kBins : head));
+    } else if (variant != 2) {
+        const int cap = (head + kBins - 1) / kBins;
+        std::vector<long long> load(kBins, 0);
+        std::vector<int> cnt(kBins, 0), placed((size_t)head, -1);
+        for (int i = 0; i < head; ++i) {
+            int best = -1;  // a bin's next workgroup must exist: the last round of bins may be a partial one
+            for (int b = 0; b < kBins; ++b)
+                if (cnt[b] < cap && cnt[b] * kBins + b < head && (best < 0 || load[b] < load[best])) best = b;
+            placed[(size_t)cnt[best] * kBins + best] = order[i];
+            load[best] += len(order[i]);
+            ++cnt[best];
+        }
+        for (int i = 0; i < head; ++i) order[i] = placed[i];
+    }
     std::vector<int> host((size_t)3 * M);
     for (int i = 0; i < M; ++i) {
         host[i] = ro[order[i]];

@@ -150,8 +150,9 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
  * Row plan for SpMM: the order in which a launch hands the rows of one matrix to its workgroups, built once per
  * matrix (like the two calls above) and passed to spmm_csr_f32_planned with every launch. Small matrices with
  * uneven rows, one row per workgroup and every workgroup on the device at once, finish when the compute unit that
- * was handed the most nonzeros does; the plan puts the long rows first and mixes long and short rows on every
- * compute unit (2048 x 512, lognormal row lengths, N = 256: 7.5 -> 6.9 us). The result is bit-identical to
+ * was handed the most nonzeros does; the plan puts the long rows first and packs the rows that start together so
+ * that every compute unit is handed about the same number of nonzeros (2048 x 512, lognormal row lengths, N = 256:
+ * 7.6 -> 6.1 us). The result is bit-identical to
  * spmm_csr_f32 with a NULL workspace: every row is summed by the same workgroup shape in the same order.
  *   dlspm_row_plan_bytes(M)  bytes of DEVICE memory for the plan of a matrix of M rows (3 * M ints).
  *   dlspm_row_plan_build     reads row_offsets (device) back, sorts on the host and writes the plan to `plan`
