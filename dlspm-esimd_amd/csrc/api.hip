@@ -344,10 +344,16 @@ int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_
 int dlspm_row_plan_advice(int M, int K, int N, int nnz, int max_row_len)
 {
     if (M <= 0 || K <= 0 || N <= 0 || nnz <= 0) return 0;
-    if (!spmm_plan_applies(spmm_choose(M, K, N, nnz, N >= 4, false, true), N)) return 0;
-    // rows known to be even gain nothing from another order (and DLSPM_ROWS_EVEN may serve them better); problems for
-    // the flat or the column-sliced schedule are told to pass a workspace instead
-    return dlspm_workspace_advice(DLSPM_OP_SPMM, M, K, N, nnz, max_row_len) == DLSPM_PASS_NULL ? 1 : 0;
+    SpmmShape shape = spmm_choose(M, K, N, nnz, N >= 4, false, true);
+    if (!spmm_plan_applies(shape, M, N, nnz)) return 0;
+    // rows known to be even gain nothing from another order (and DLSPM_ROWS_EVEN may serve them better)
+    if (max_row_len >= 0 && max_row_len <= 1.5 * ((double)nnz / M)) return 0;
+    // a B well beyond one L2 needs the column-sliced schedule's workspace more than it needs balance; the flat
+    // schedule, though, is behind the plan wherever both apply (lognormal rows, sigma 1 ... 2, row-block / flat / plan:
+    // 8192 x 2048, N = 128: 45.4 / 41.2 / 30.8 us; 16384 x 4096: 121 / 105 / 86.6 us; 32768 x 8192: 525 / 466 / 424 us)
+    int slices = 0;
+    (void)dlspm_describe_slices(DLSPM_OP_SPMM, M, K, N, nnz, &slices, nullptr);
+    return slices >= 3 ? 0 : 1;
 }
 
 int spmm_csr_f32_planned(int M, int K, int N, int nnz, const int* row_offsets, const int* col_indices,
@@ -361,8 +367,8 @@ int spmm_csr_f32_planned(int M, int K, int N, int nnz, const int* row_offsets, c
     if (M == 0 || N == 0) return DLSPM_OK;
     if (!row_offsets || !C) return DLSPM_E_INVALID_ARG;
     if (nnz > 0 && (!col_indices || !values || !B)) return DLSPM_E_INVALID_ARG;
-    const SpmmShape shape = spmm_choose(M, K, N, nnz, N >= 4, false, true);
-    if (!spmm_plan_applies(shape, N))  // the order of the rows matters only with one row per workgroup
+    SpmmShape shape = spmm_choose(M, K, N, nnz, N >= 4, false, true);
+    if (!spmm_plan_applies(shape, M, N, nnz))  // short rows grouped per workgroup, or column tiles: the plan has no say
         return spmm_csr_f32(M, K, N, nnz, row_offsets, col_indices, values, B, C, nullptr, 0, stream);
     const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C};
     const hipError_t e = spmm_planned_launch(args, shape, static_cast<const int*>(plan), static_cast<hipStream_t>(stream));

@@ -219,18 +219,23 @@ struct Options {
 struct WorkspaceChoice {
     size_t bytes = 0;        // device memory to allocate and pass
     bool rows_even = false;  // pass DLSPM_ROWS_EVEN instead
+    bool plan = false;       // SpMM: build a row plan and launch spmm_csr_f32_planned instead
     void* arg(void* buffer) const { return rows_even ? DLSPM_ROWS_EVEN : bytes ? buffer : nullptr; }
 };
 inline WorkspaceChoice workspace_to_pass(const Options& opt, int op, int M, int K, int width, int nnz,
-                                         const int* row_offsets_dev, int* longest_out = nullptr)
+                                         const int* row_offsets_dev, bool plan_allowed = false)
 {
     WorkspaceChoice c;
-    if (longest_out) *longest_out = -1;
     if (opt.workspace == Options::kNever || M <= 0 || nnz <= 0) return c;
     const size_t want = dlspm_workspace_bytes(op, M, K, width, nnz);
     int longest = 0, empty = 0;
     if (dlspm_csr_row_stats(M, row_offsets_dev, nullptr, &longest, &empty) != DLSPM_OK) throw std::runtime_error("dlspm_csr_row_stats failed");
-    if (longest_out) *longest_out = longest;
+    if (plan_allowed && opt.workspace == Options::kAuto && dlspm_row_plan_advice(M, K, width, nnz, longest) == 1) {
+        c.plan = true;
+        std::printf("rows: longest %d, mean %.1f, empty %d -> uneven, row plan (one row per workgroup, handed out by length)\n",
+                    longest, (double)nnz / M, empty);
+        return c;
+    }
     const int advice = dlspm_workspace_advice(op, M, K, width, nnz, longest);
     int slices = 0;
     (void)dlspm_describe_slices(op, M, K, width, nnz, &slices, nullptr);

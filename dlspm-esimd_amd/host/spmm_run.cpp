@@ -43,14 +43,12 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     DLSPM_HIP_CHECK(hipMemset(C_d.p, 0xFF, (size_t)M * N * sizeof(float)));  // NaN pattern: every element must be written
 
     // the caller owns the workspace, as it owns every other buffer: 0 bytes for small problems
-    int longest = -1;
-    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_SPMM, M, K, N, nnz, ro_d.p, &longest);
+    // uneven rows that are not short: a row plan, built once per matrix like the look at the row lengths, hands the
+    // rows out by length, one per workgroup (dlspm_row_plan_advice); otherwise what dlspm_workspace_advice says
+    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_SPMM, M, K, N, nnz, ro_d.p, opt.plan);
     DevBuf<char> ws(wc.bytes);
     if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
-    // uneven rows, one row per workgroup, nothing to pass as workspace: a row plan, built once per matrix like the look
-    // at the row lengths, hands the rows out longest first
-    const bool planned = opt.plan && opt.workspace == Options::kAuto && longest >= 0 && !wc.bytes && !wc.rows_even &&
-                         dlspm_row_plan_advice(M, K, N, nnz, longest) == 1;
+    const bool planned = wc.plan;
     DevBuf<char> plan(planned ? dlspm_row_plan_bytes(M) : 0);
     if (planned) {
         const auto t0 = std::chrono::steady_clock::now();

@@ -159,13 +159,18 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
  *                            (device); synchronises `stream`. DLSPM_E_WORKSPACE if plan_bytes is too small.
  *   spmm_csr_f32_planned     spmm_csr_f32 with that plan instead of a workspace. The plan must have been built from
  *                            the same row_offsets (a stale plan gives wrong values but stays inside the arrays).
- *                            Shapes that do not run one row per workgroup (short rows grouped, wide dense rows in
- *                            column tiles) ignore it and run as spmm_csr_f32(..., NULL, 0, stream); plan == NULL too.
+ *                            It runs one row per workgroup also where spmm_csr_f32 would group a few rows, if the
+ *                            rows are long enough (the same sums as spmm_csr_f32 under DLSPM_SPLIT=4,1). Short rows,
+ *                            wide dense rows in column tiles and widths below 4 ignore it and run as
+ *                            spmm_csr_f32(..., NULL, 0, stream); plan == NULL too.
  * No counterpart in the reference, whose kernels take the rows in matrix order (SPMM/spmmesimd2.hpp:63-75).
  */
 size_t dlspm_row_plan_bytes(int M);
 /* 1 if a row plan is worth building for these sizes and this longest row (-1: unknown): spmm_csr_f32_planned would use
- * it and dlspm_workspace_advice has nothing better to pass (uneven rows, no flat or column-sliced schedule); else 0. */
+ * it (one column tile, rows of at least 32 nonzeros on average where the size rule would group rows), the rows are
+ * not known to be even, and B is not so far beyond one L2 that the column-sliced schedule's workspace matters more;
+ * else 0. Ask this before dlspm_workspace_advice: where both a plan and the flat schedule's workspace apply, the plan
+ * is 10-40 % faster. */
 int dlspm_row_plan_advice(int M, int K, int N, int nnz, int max_row_len);
 int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_bytes, void* stream);
 int spmm_csr_f32_planned(int M, int K, int N, int nnz, const int* row_offsets, const int* col_indices,

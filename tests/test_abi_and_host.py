@@ -194,10 +194,18 @@ def test_row_plan_host_side(dl):
     assert A(2048, 512, 256, 105687, 312)            # the headline configuration: uneven rows, one row per workgroup
     assert A(2048, 512, 256, 105687, -1)             # rows unknown: nothing better to pass
     assert not A(2048, 512, 256, 105687, 60)         # even rows: another order gains nothing
-    assert not A(4096, 1024, 256, 4096 * 100, 400)   # rows grouped two per workgroup
+    # where the size rule groups rows per workgroup, a plan ungroups them if they are long enough for that
+    assert dl.describe_launch(dl.OP_SPMM, 4096, 1024, 256, 4096 * 100)["R"] == 2 and A(4096, 1024, 256, 4096 * 100, 400)
+    assert A(8192, 2048, 128, 8192 * 200, 1400) and A(16384, 512, 256, 16384 * 51, 500) and A(65536, 2048, 128, 65536 * 197, 2000)
+    assert not A(32768, 1024, 256, 32768 * 32, 300)  # 32 per row in a tall matrix: grouped rows win
+    assert not A(16384, 2048, 32, 16384 * 101, 1000)  # narrow dense rows in a tall matrix
+    assert not A(8192, 512, 256, 8192 * 24, 200)     # short rows
+    assert A(4096, 512, 32, 4096 * 52, 500)          # ... but any width up to 4096 rows
     assert not A(600, 512, 784, 600 * 60, 300)       # column tiles
     assert not A(2048, 512, 3, 105687, 312)          # fewer than four columns
-    assert not A(16384, 4096, 128, 16384 * 400, 4000)  # large and uneven: the flat schedule's workspace instead
+    assert A(16384, 4096, 128, 16384 * 400, 4000)    # large and uneven: the plan rather than the flat schedule's workspace
+    assert dl.workspace_advice(dl.OP_SPMM, 16384, 4096, 128, 16384 * 400, 4000) == dl.PASS_WORKSPACE   # (what is said without a plan)
+    assert not A(8192, 16384, 128, 8192 * 800, 8000)  # B of 8 MiB: the column-sliced schedule's workspace first
     assert not A(0, 0, 0, 0, 0)
     bogus = ctypes.c_void_p(256)   # never dereferenced: the checks come first
     assert L.dlspm_row_plan_build(-1, bogus, bogus, 0, None) == dl.E_INVALID_ARG

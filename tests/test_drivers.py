@@ -210,12 +210,16 @@ def test_drivers_pass_the_workspace_only_for_uneven_rows():
     for app in ("sddmm_run", "fused_run"):
         rc, out = run(app, "--shape", 8192, 4096, 128, 0.1, "--iters", 3)
         assert rc == 0 and "PASS" in out and "even, DLSPM_ROWS_EVEN passed" in out, out
-    rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 0.2, "--iters", 3)
+    rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 0.2, "--iters", 3, "--no-plan")
     assert rc == 0 and "PASS" in out and "nothing passed" in out and "workspace:" not in out, out
+    rc, out = run("sddmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 0.2, "--iters", 3)
+    assert rc == 0 and "PASS" in out and "nothing passed" in out, out
     rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--no-workspace", "--iters", 3)
     assert rc == 0 and "PASS" in out and "rows:" not in out, out
-    rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 1.5, "--iters", 3)
+    rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 1.5, "--iters", 3, "--no-plan")
     assert rc == 0 and "PASS" in out and "uneven, workspace passed" in out and "workspace:" in out, out
+    rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 1.5, "--iters", 3)   # SpMM prefers a row plan
+    assert rc == 0 and "PASS" in out and "uneven, row plan" in out and "workspace:" not in out, out
     rc, out = run("fused_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 1.5, "--iters", 3)
     assert rc == 0 and "PASS" in out and "uneven, workspace passed" in out, out
     rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--workspace", "--iters", 3)
@@ -227,10 +231,14 @@ def test_spmm_driver_builds_a_row_plan_for_small_uneven_matrices():
     """The headline configuration (2048 x 512, lognormal rows, one row per workgroup): the driver builds the row plan
     once and launches spmm_csr_f32_planned; with --no-plan, or on even rows, it does not; all self-check."""
     rc, out = run("spmm_run", "--cfg", 2, "--iters", 5)
-    assert rc == 0 and "PASS" in out and "row plan:" in out and "nothing passed" in out, out
+    assert rc == 0 and "PASS" in out and "row plan:" in out and "uneven, row plan" in out, out
     rc, out = run("spmm_run", "--cfg", 2, "--iters", 5, "--no-plan")
     assert rc == 0 and "PASS" in out and "row plan:" not in out, out
     rc, out = run("spmm_run", "--cfg", 4, "--iters", 5)          # even rows
     assert rc == 0 and "PASS" in out and "row plan:" not in out, out
     rc, out = run("spmm_run", "--shape", 1024, 1024, 256, 0.1, "--sigma", 0.8, "--iters", 5)
     assert rc == 0 and "PASS" in out and "row plan:" in out, out
+    rc, out = run("spmm_run", "--shape", 4096, 1024, 256, 0.1, "--sigma", 0.8, "--iters", 5)    # rows ungrouped by the plan
+    assert rc == 0 and "PASS" in out and "row plan:" in out, out
+    rc, out = run("spmm_run", "--shape", 8192, 512, 256, 0.04, "--sigma", 0.8, "--iters", 5)    # short rows: no plan
+    assert rc == 0 and "PASS" in out and "row plan:" not in out, out
