@@ -152,8 +152,9 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
  * uneven rows, one row per workgroup and every workgroup on the device at once, finish when the compute unit that
  * was handed the most nonzeros does; the plan puts the long rows first and packs the rows that start together so
  * that every compute unit is handed about the same number of nonzeros (2048 x 512, lognormal row lengths, N = 256:
- * 7.6 -> 6.1 us). The result is bit-identical to
- * spmm_csr_f32 with a NULL workspace: every row is summed by the same workgroup shape in the same order.
+ * 7.6 -> 6.1 us); larger matrices with uneven rows gain as much from the rows being handed out longest first.
+ * Every row is summed by one four-wave workgroup in a fixed order (no atomics): the result is bit-identical to
+ * spmm_csr_f32 with a NULL workspace wherever that call runs one row per workgroup too.
  *   dlspm_row_plan_bytes(M)  bytes of DEVICE memory for the plan of a matrix of M rows (3 * M ints).
  *   dlspm_row_plan_build     reads row_offsets (device) back, sorts on the host and writes the plan to `plan`
  *                            (device); synchronises `stream`. DLSPM_E_WORKSPACE if plan_bytes is too small.
