@@ -58,7 +58,7 @@ def make_step(dl, torch, c, use_plan=True, info=None):
         va, B = d(c["values"]), d(c["d0"])
         out = torch.empty((c["M"], c["N"]), dtype=torch.float32, device="cuda")
         longest, _ = dl.csr_row_stats(ro)
-        if use_plan and dl.row_plan_advice(c["M"], c["K"], c["N"], c["nnz"], longest):
+        if use_plan and dl.row_plan_advice(c["op"], c["M"], c["K"], c["N"], c["nnz"], longest):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             plan = dl.row_plan(ro)

@@ -341,18 +341,30 @@ int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }
 
-int dlspm_row_plan_advice(int M, int K, int N, int nnz, int max_row_len)
+int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row_len)
 {
-    if (M <= 0 || K <= 0 || N <= 0 || nnz <= 0) return 0;
-    SpmmShape shape = spmm_choose(M, K, N, nnz, N >= 4, false, true);
-    if (!spmm_plan_applies(shape, M, N, nnz)) return 0;
+    if (M <= 0 || K <= 0 || N_or_D <= 0 || nnz <= 0) return 0;
+    const bool vec4 = N_or_D >= 4;
+    if (op == DLSPM_OP_SPMM) {
+        SpmmShape shape = spmm_choose(M, K, N_or_D, nnz, vec4, false, true);
+        if (!spmm_plan_applies(shape, M, N_or_D, nnz)) return 0;
+    } else if (op == DLSPM_OP_SDDMM) {
+        SddmmShape shape = sddmm_choose(M, N_or_D, nnz, vec4);
+        if (!sddmm_plan_applies(shape, M, N_or_D, nnz)) return 0;
+    } else if (op == DLSPM_OP_FUSED) {
+        FusedShape shape = fused_choose(M, N_or_D, nnz, vec4);
+        if (!fused_plan_applies(shape, M, N_or_D, nnz)) return 0;
+    } else {
+        return 0;
+    }
     // rows known to be even gain nothing from another order (and DLSPM_ROWS_EVEN may serve them better)
     if (max_row_len >= 0 && max_row_len <= 1.5 * ((double)nnz / M)) return 0;
-    // a B well beyond one L2 needs the column-sliced schedule's workspace more than it needs balance; the flat
-    // schedule, though, is behind the plan wherever both apply (lognormal rows, sigma 1 ... 2, row-block / flat / plan:
-    // 8192 x 2048, N = 128: 45.4 / 41.2 / 30.8 us; 16384 x 4096: 121 / 105 / 86.6 us; 32768 x 8192: 525 / 466 / 424 us)
+    // dense operands well beyond one L2 need the column-sliced schedule's workspace more than they need balance; the
+    // flat schedule, though, is behind the plan wherever both apply (SpMM, lognormal rows, sigma 1 ... 2, row-block /
+    // flat / plan: 8192 x 2048, N = 128: 45.4 / 41.2 / 30.8 us; 16384 x 4096: 121 / 105 / 86.6 us; 32768 x 8192: 525 / 466
+    // / 424 us)
     int slices = 0;
-    (void)dlspm_describe_slices(DLSPM_OP_SPMM, M, K, N, nnz, &slices, nullptr);
+    (void)dlspm_describe_slices(op, M, K, N_or_D, nnz, &slices, nullptr);
     return slices >= 3 ? 0 : 1;
 }
 
@@ -372,6 +384,43 @@ int spmm_csr_f32_planned(int M, int K, int N, int nnz, const int* row_offsets, c
         return spmm_csr_f32(M, K, N, nnz, row_offsets, col_indices, values, B, C, nullptr, 0, stream);
     const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C};
     const hipError_t e = spmm_planned_launch(args, shape, static_cast<const int*>(plan), static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+}
+
+int sddmm_csr_f32_planned(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* lhs,
+                          const float* rhs, float* out_values, const void* plan, size_t plan_bytes, void* stream)
+{
+    if (M < 0 || K < 0 || D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
+    if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
+    if (!plan) return sddmm_csr_f32(M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values, nullptr, 0, stream);
+    if (plan_bytes < dlspm_row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
+    if (M == 0 || nnz == 0) return DLSPM_OK;
+    if (!row_offsets || !col_indices || !out_values) return DLSPM_E_INVALID_ARG;
+    if (D > 0 && (!lhs || !rhs)) return DLSPM_E_INVALID_ARG;
+    SddmmShape shape = sddmm_choose(M, D, nnz, D >= 4);
+    if (D == 0 || !sddmm_plan_applies(shape, M, D, nnz))
+        return sddmm_csr_f32(M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values, nullptr, 0, stream);
+    const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values};
+    const hipError_t e = sddmm_planned_launch(args, shape, static_cast<const int*>(plan), static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+}
+
+int fused_sddmm_spmm_f32_planned(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* Q,
+                                 const float* Kmat, const float* V, float scale, float* O, const void* plan,
+                                 size_t plan_bytes, void* stream)
+{
+    if (M < 0 || K < 0 || D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
+    if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
+    if (!plan) return fused_sddmm_spmm_f32(M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O, nullptr, 0, stream);
+    if (plan_bytes < dlspm_row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
+    if (M == 0 || D == 0) return DLSPM_OK;
+    if (!row_offsets || !O) return DLSPM_E_INVALID_ARG;
+    if (nnz > 0 && (!col_indices || !Q || !Kmat || !V)) return DLSPM_E_INVALID_ARG;
+    FusedShape shape = fused_choose(M, D, nnz, D >= 4);
+    if (!fused_plan_applies(shape, M, D, nnz))
+        return fused_sddmm_spmm_f32(M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O, nullptr, 0, stream);
+    const FusedArgs args{M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O};
+    const hipError_t e = fused_planned_launch(args, shape, static_cast<const int*>(plan), static_cast<hipStream_t>(stream));
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }
 

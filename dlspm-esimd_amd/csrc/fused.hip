@@ -56,13 +56,15 @@ __device__ __forceinline__ void fused_segment(Vec<VEC>* acc, int p, int q, int D
 
 // The work of workgroup `bid`; SLICED as in spmm_block: row i owns [row_offsets[i], row_ends[i]), the part of the CSR
 // row inside one range of columns, and the split works on the running sum of the lengths.
-template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R, bool SLICED>
+// PLANNED (with SLICED and R == 1): workgroup i works on row row_ids[i] of Q, O and the mask, the order of a row plan.
+template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R, bool SLICED, bool PLANNED = false>
 __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles, float scale,
                                             const int* __restrict__ row_offsets, const int* __restrict__ row_ends,
                                             const int* __restrict__ col_indices, const float* __restrict__ Q,
                                             const float* __restrict__ Kmat, const float* __restrict__ Vmat,
-                                            float* __restrict__ O)
+                                            float* __restrict__ O, const int* __restrict__ row_ids = nullptr, int nnz = 0)
 {
+    static_assert(!PLANNED || (SLICED && R == 1), "a row plan names one row per workgroup");
     constexpr int TW = G * VEC * V2;
     constexpr int NP = R == 1 ? 1 : 2;
     using VecT = Vec<VEC>;
@@ -78,7 +80,8 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
     const int ct = col_tiles == 1 ? 0 : bid / row_blocks;
     const int rb = bid - ct * row_blocks;
     const int r0 = rb * R;
-    const int nr = min(R, M - r0);
+    const int nr = PLANNED ? 1 : min(R, M - r0);
+    int out_row0 = r0;  // row of Q and O that belongs to the block's first row
 
     // the block's R + 1 row offsets without LDS or a barrier (see spmm_block)
     int off_lo = 0, off_hi = 0, off_win = 0, start_lo = 0, start_win = 0;
@@ -94,6 +97,11 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
         if constexpr (R == 1) {
             start_lo = row_offsets[r0];
             off_hi = row_ends[r0] - start_lo;
+            if constexpr (PLANNED) {  // a plan built for another matrix must not take the kernel outside the arrays
+                out_row0 = min(max(row_ids[r0], 0), M - 1);
+                start_lo = min(max(start_lo, 0), nnz);
+                off_hi = min(max(off_hi, 0), nnz - start_lo);
+            }
         } else {
             static_assert(R + 1 <= 32, "the running sum covers 32 lanes");
             const int i = r0 + min(lane, nr - 1);
@@ -139,7 +147,7 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
             const int re = s_off(r + 1);
             const int q = __builtin_amdgcn_readfirstlane(min(re, b));
             const int p = __builtin_amdgcn_readfirstlane(pos);
-            const float* q_row = Q + (size_t)(r0 + r) * D;
+            const float* q_row = Q + (size_t)(out_row0 + r) * D;
 
             VecT acc[V2];
             const int shift = s_shift(r);
@@ -149,7 +157,7 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
             const bool whole_row = (p == rs) && (q == re);
             if (slot == 0) {
                 if (whole_row) {
-                    float* orow = O + (size_t)(r0 + r) * D;
+                    float* orow = O + (size_t)(out_row0 + r) * D;
 #pragma unroll
                     for (int v = 0; v < V2; ++v)
                         if (act[v]) acc[v].gstore(orow + colv[v]);
@@ -170,7 +178,7 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
             if (slot == 0) {
                 for (int r = w; r < nr; r += W) {
                     if (s_off(r) != s_off(r + 1)) continue;
-                    float* orow = O + (size_t)(r0 + r) * D;
+                    float* orow = O + (size_t)(out_row0 + r) * D;
 #pragma unroll
                     for (int v = 0; v < V2; ++v)
                         if (act[v]) VecT::zero().gstore(orow + colv[v]);
@@ -184,7 +192,7 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
                 for (int r = w; r < nr; r += W) {
                     const int len = s_off(r + 1) - s_off(r);
                     const int part = (len + m - 1) / m;
-                    float* orow = O + (size_t)(r0 + r) * D;
+                    float* orow = O + (size_t)(out_row0 + r) * D;
                     if (len > 0 && len <= part) continue;  // one wave held the whole row and stored it
 #pragma unroll
                     for (int v = 0; v < V2; ++v) {
@@ -205,7 +213,7 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
         // one row per workgroup: wave x had nonzeros iff x * per < T, and wave 0 adds them up (no division, the
         // partial sums of all waves are requested from LDS together)
         if (w == 0 && slot == 0) {
-            float* orow = O + (size_t)r0 * D;
+            float* orow = O + (size_t)out_row0 * D;
             if (T == 0) {
 #pragma unroll
                 for (int v = 0; v < V2; ++v)
@@ -227,7 +235,7 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
         for (int r = w; r < nr; r += W) {
             const int rs = s_off(r);
             const int re = s_off(r + 1);
-            float* orow = O + (size_t)(r0 + r) * D;
+            float* orow = O + (size_t)(out_row0 + r) * D;
             if (rs == re) {
 #pragma unroll
                 for (int v = 0; v < V2; ++v)
@@ -278,6 +286,20 @@ __global__ __launch_bounds__(4 * 64) void fused_sliced_kernel(int M, int D, int 
     fused_block<VEC, G1, DS, MASKED, G, V2, 4, R, true>(bid, M, D, col_tiles, scale, bounds + (size_t)sl * M,
                                                         bounds + (size_t)(sl + 1) * M, col_indices, Q, Kmat, Vmat,
                                                         partial + (size_t)sl * M * D);
+}
+
+// Row plan: workgroup i works on the whole row rows[i] = [starts[i], ends[i]) (one row per four-wave workgroup, one
+// column tile).
+template <int VEC, int G1, int DS, bool MASKED, int G, int V2>
+__global__ __launch_bounds__(4 * 64) void fused_planned_kernel(int M, int D, int nnz, float scale,
+                                                               const int* __restrict__ starts, const int* __restrict__ ends,
+                                                               const int* __restrict__ rows,
+                                                               const int* __restrict__ col_indices,
+                                                               const float* __restrict__ Q, const float* __restrict__ Kmat,
+                                                               const float* __restrict__ Vmat, float* __restrict__ O)
+{
+    fused_block<VEC, G1, DS, MASKED, G, V2, 4, 1, true, true>((int)blockIdx.x, M, D, 1, scale, starts, ends, col_indices, Q,
+                                                              Kmat, Vmat, O, rows, nnz);
 }
 
 // ---- host side --------------------------------------------------------------------------------------
@@ -525,6 +547,42 @@ hipError_t fused_sliced_launch(const FusedArgs& x, const FusedShape& s, const Sl
 #undef DLSPM_SLICED
     if (e != hipSuccess) return e;
     return slice_sum_launch((long long)x.M * x.D, plan.slices, partial, x.O, stream);
+}
+
+// ---- row plan ---------------------------------------------------------------------------------------
+
+bool fused_plan_applies(FusedShape& s, int M, int D, int nnz)
+{
+    // built for 16 < D <= 512 (the shapes of the column-sliced kernels): one column tile
+    if (s.vec != 4 || s.G1 != 8 || s.DS < 1 || s.W != 4 || s.G * s.vec * s.V < D) return false;
+    if (s.R == 1) return true;
+    if (!plan_ungroups(M, D, nnz)) return false;
+    s.R = 1;
+    return true;
+}
+
+template <int DS, int G, int V2>
+static hipError_t launch_planned(const FusedArgs& x, const int* plan, hipStream_t stream)
+{
+    const int *starts = plan, *ends = plan + x.M, *rows = plan + 2 * (size_t)x.M;
+    if (x.D == 8 * 4 * DS)
+        hipLaunchKernelGGL((fused_planned_kernel<4, 8, DS, false, G, V2>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M,
+                           x.D, x.nnz, x.scale, starts, ends, rows, x.col_indices, x.Q, x.Kmat, x.V, x.O);
+    else
+        hipLaunchKernelGGL((fused_planned_kernel<4, 8, DS, true, G, V2>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M,
+                           x.D, x.nnz, x.scale, starts, ends, rows, x.col_indices, x.Q, x.Kmat, x.V, x.O);
+    return hipGetLastError();
+}
+
+hipError_t fused_planned_launch(const FusedArgs& x, const FusedShape& s, const int* plan, hipStream_t stream)
+{
+    if (x.M <= 0) return hipSuccess;
+    if (s.DS == 1 && s.G == 8 && s.V == 1) return launch_planned<1, 8, 1>(x, plan, stream);
+    if (s.DS == 2 && s.G == 16 && s.V == 1) return launch_planned<2, 16, 1>(x, plan, stream);
+    if (s.DS == 4 && s.G == 32 && s.V == 1) return launch_planned<4, 32, 1>(x, plan, stream);
+    if (s.DS == 8 && s.G == 64 && s.V == 1) return launch_planned<8, 64, 1>(x, plan, stream);
+    if (s.DS == 16 && s.G == 64 && s.V == 2) return launch_planned<16, 64, 2>(x, plan, stream);
+    return hipErrorInvalidValue;
 }
 
 }  // namespace dlspm

@@ -79,6 +79,7 @@ SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, b
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
 // Row plan (3 x M ints on the device: first nonzero, end and row number of the row that workgroup i works on): only for
 // shapes of one row per four-wave workgroup and one column tile
+bool plan_ungroups(int M, int width, int nnz);  // rows long enough that a plan runs them one per workgroup against the size rule
 bool spmm_plan_applies(SpmmShape& s, int M, int N, int nnz);  // true: s is the shape of the planned launch (R = 1)
 hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int* plan, hipStream_t stream);
 hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPlan& plan, float* partial,
@@ -110,5 +111,11 @@ struct SplitRule {
     bool w16_long_rows;
 };
 void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bool rows_even, int& W, int& R);
+
+// the same plan for the other two ops (16 < D <= 512, one row per four-wave workgroup)
+bool sddmm_plan_applies(SddmmShape& s, int M, int D, int nnz);
+hipError_t sddmm_planned_launch(const SddmmArgs& x, const SddmmShape& s, const int* plan, hipStream_t stream);
+bool fused_plan_applies(FusedShape& s, int M, int D, int nnz);
+hipError_t fused_planned_launch(const FusedArgs& x, const FusedShape& s, const int* plan, hipStream_t stream);
 
 }  // namespace dlspm

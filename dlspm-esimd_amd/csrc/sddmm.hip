@@ -51,16 +51,20 @@ __device__ __forceinline__ void sddmm_segment(int p, int q, int D, const int* __
 // true: [row_offsets[i], row_ends[i]), the part of the CSR row inside one range of columns (see spmm_block): the split
 // works on the running sum of the lengths and every segment is shifted back to where it lies, which is also where its
 // results go.
-template <int VEC, int G1, int DS, bool MASKED, int W, int R, bool SLICED>
+// PLANNED (with SLICED and R == 1): workgroup i works on row row_ids[i] = [row_offsets[i], row_ends[i]) of the mask, the
+// order of a row plan (see spmm_block).
+template <int VEC, int G1, int DS, bool MASKED, int W, int R, bool SLICED, bool PLANNED = false>
 __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __restrict__ row_offsets,
                                             const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                             const float* __restrict__ lhs, const float* __restrict__ rhs,
-                                            float* __restrict__ out)
+                                            float* __restrict__ out, const int* __restrict__ row_ids = nullptr, int nnz = 0)
 {
+    static_assert(!PLANNED || (SLICED && R == 1), "a row plan names one row per workgroup");
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r0 = bid * R;
-    const int nr = min(R, M - r0);
+    const int nr = PLANNED ? 1 : min(R, M - r0);
+    int lhs_row0 = r0;  // row of lhs that belongs to the block's first row
 
     // the block's R + 1 row offsets without LDS or a barrier (see spmm_block): this kernel then has neither
     int off_lo = 0, off_hi = 0, off_win = 0, start_lo = 0, start_win = 0;
@@ -76,6 +80,11 @@ __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __
         if constexpr (R == 1) {
             start_lo = row_offsets[r0];
             off_hi = row_ends[r0] - start_lo;
+            if constexpr (PLANNED) {  // a plan built for another matrix must not take the kernel outside the arrays
+                lhs_row0 = min(max(row_ids[r0], 0), M - 1);
+                start_lo = min(max(start_lo, 0), nnz);
+                off_hi = min(max(off_hi, 0), nnz - start_lo);
+            }
         } else {
             static_assert(R + 1 <= 32, "the running sum covers 32 lanes");
             const int i = r0 + min(lane, nr - 1);
@@ -110,7 +119,7 @@ __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __
     while (pos < b) {
         const int q = __builtin_amdgcn_readfirstlane(min(s_off(r + 1), b));
         const int p = __builtin_amdgcn_readfirstlane(pos);
-        const float* lhs_row = lhs + (size_t)(r0 + r) * D;
+        const float* lhs_row = lhs + (size_t)(lhs_row0 + r) * D;
 
         const int shift = s_shift(r);
         sddmm_segment<VEC, G1, DS, MASKED>(p + shift, q + shift, D, col_indices, lhs_row, rhs, out, lane);
@@ -147,6 +156,17 @@ __global__ __launch_bounds__(4 * 64) void sddmm_sliced_kernel(int M, int D, int 
 }
 
 // ---- host side --------------------------------------------------------------------------------------
+
+// Row plan: workgroup i works on the whole row rows[i] = [starts[i], ends[i]) (one row per four-wave workgroup).
+template <int VEC, int G1, int DS, bool MASKED>
+__global__ __launch_bounds__(4 * 64) void sddmm_planned_kernel(int M, int D, int nnz, const int* __restrict__ starts,
+                                                               const int* __restrict__ ends, const int* __restrict__ rows,
+                                                               const int* __restrict__ col_indices,
+                                                               const float* __restrict__ lhs, const float* __restrict__ rhs,
+                                                               float* __restrict__ out)
+{
+    sddmm_block<VEC, G1, DS, MASKED, 4, 1, true, true>((int)blockIdx.x, M, D, starts, ends, col_indices, lhs, rhs, out, rows, nnz);
+}
 
 template <int VEC, int G1, int DS, int W, int R>
 static hipError_t launch_one(const SddmmArgs& x, hipStream_t stream)
@@ -335,6 +355,43 @@ hipError_t sddmm_sliced_launch(const SddmmArgs& x, const SddmmShape& s, const Sl
     if (s.vec == 4 && s.G1 == 8 && s.DS == 16) return launch_sliced<4, 8, 16>(x, plan, bounds, stream);
     if (s.vec == 4 && s.G1 == 8 && s.DS == 2) return launch_sliced<4, 8, 2>(x, plan, bounds, stream);
     if (s.vec == 4 && s.G1 == 8 && s.DS == 1) return launch_sliced<4, 8, 1>(x, plan, bounds, stream);
+    return hipErrorInvalidValue;
+}
+
+// ---- row plan ---------------------------------------------------------------------------------------
+
+bool sddmm_plan_applies(SddmmShape& s, int M, int D, int nnz)
+{
+    if (s.vec != 4 || s.G1 != 8 || s.DS < 1 || s.W != 4) return false;  // built for 16 < D <= 512
+    if (s.R == 1) return true;
+    if (!plan_ungroups(M, D, nnz)) return false;
+    s.R = 1;
+    return true;
+}
+
+template <int DS>
+static hipError_t launch_planned(const SddmmArgs& x, const int* plan, hipStream_t stream)
+{
+    const int *starts = plan, *ends = plan + x.M, *rows = plan + 2 * (size_t)x.M;
+    if (x.D == 8 * 4 * DS)
+        hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, false>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M, x.D,
+                           x.nnz, starts, ends, rows, x.col_indices, x.lhs, x.rhs, x.out);
+    else
+        hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, true>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M, x.D,
+                           x.nnz, starts, ends, rows, x.col_indices, x.lhs, x.rhs, x.out);
+    return hipGetLastError();
+}
+
+hipError_t sddmm_planned_launch(const SddmmArgs& x, const SddmmShape& s, const int* plan, hipStream_t stream)
+{
+    if (x.M <= 0) return hipSuccess;
+    switch (s.DS) {
+        case 1: return launch_planned<1>(x, plan, stream);
+        case 2: return launch_planned<2>(x, plan, stream);
+        case 4: return launch_planned<4>(x, plan, stream);
+        case 8: return launch_planned<8>(x, plan, stream);
+        case 16: return launch_planned<16>(x, plan, stream);
+    }
     return hipErrorInvalidValue;
 }
 

@@ -600,13 +600,17 @@ hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const Slice
 // 18.3 against 24.6 us; 8192 x 2048, 199 per row, N = 128: 29.1 against 37.5 us; 16384 x 512, 51 per row, N = 256: 31.4
 // against 35.3 us; 65536 x 2048, 197 per row, N = 128: 223 against 232 us; but 32768 x 1024, 32 per row, N = 256: 46.6
 // against 43.9 us; 16384 x 2048, 101 per row, N = 32: 17.7 against 14.2 us; rows below 32 nonzeros lose everywhere.
+bool plan_ungroups(int M, int width, int nnz)
+{
+    const long long avg32 = 32ll * M, avg48 = 48ll * M, avg128 = 128ll * M;
+    return nnz >= avg32 && (M <= 4096 || (width >= 128 && (M <= 8192 || (nnz >= avg48 && M <= 16384) || nnz >= avg128)));
+}
+
 bool spmm_plan_applies(SpmmShape& s, int M, int N, int nnz)
 {
     if (s.vec != 4 || s.W != 4 || s.G * s.vec * s.V < N) return false;
     if (s.R == 1) return true;
-    const long long avg32 = 32ll * M, avg48 = 48ll * M, avg128 = 128ll * M;
-    const bool ungroup = nnz >= avg32 && (M <= 4096 || (N >= 128 && (M <= 8192 || (nnz >= avg48 && M <= 16384) || nnz >= avg128)));
-    if (!ungroup) return false;
+    if (!plan_ungroups(M, N, nnz)) return false;
     s.R = 1;
     return true;
 }

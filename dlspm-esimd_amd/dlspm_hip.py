@@ -47,6 +47,8 @@ EXPORTS = (
     "dlspm_row_plan_advice",
     "dlspm_row_plan_build",
     "spmm_csr_f32_planned",
+    "sddmm_csr_f32_planned",
+    "fused_sddmm_spmm_f32_planned",
     "dlspm_status_string",
     "dlspm_last_hip_error",
     "dlspm_version",
@@ -92,12 +94,16 @@ def lib() -> ctypes.CDLL:
         L.dlspm_csr_row_stats.restype = ci
         L.dlspm_row_plan_bytes.argtypes = [ci]
         L.dlspm_row_plan_bytes.restype = sz
-        L.dlspm_row_plan_advice.argtypes = [ci, ci, ci, ci, ci]
+        L.dlspm_row_plan_advice.argtypes = [ci, ci, ci, ci, ci, ci]
         L.dlspm_row_plan_advice.restype = ci
         L.dlspm_row_plan_build.argtypes = [ci, vp, vp, sz, vp]
         L.dlspm_row_plan_build.restype = ci
         L.spmm_csr_f32_planned.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, sz, vp]
         L.spmm_csr_f32_planned.restype = ci
+        L.sddmm_csr_f32_planned.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, sz, vp]
+        L.sddmm_csr_f32_planned.restype = ci
+        L.fused_sddmm_spmm_f32_planned.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, cf, vp, vp, sz, vp]
+        L.fused_sddmm_spmm_f32_planned.restype = ci
         L.dlspm_status_string.argtypes = [ci]
         L.dlspm_status_string.restype = ctypes.c_char_p
         L.dlspm_last_hip_error.restype = ci
@@ -134,9 +140,9 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def row_plan_advice(M, K, N, nnz, max_row_len=-1) -> bool:
-    """Whether a row plan is worth building for an SpMM of these sizes (see dlspm_row_plan_advice)."""
-    return bool(lib().dlspm_row_plan_advice(M, K, N, nnz, max_row_len))
+def row_plan_advice(op, M, K, N_or_D, nnz, max_row_len=-1) -> bool:
+    """Whether a row plan is worth building for op at these sizes (see dlspm_row_plan_advice)."""
+    return bool(lib().dlspm_row_plan_advice(op, M, K, N_or_D, nnz, max_row_len))
 
 
 def row_plan(row_offsets):
@@ -184,7 +190,7 @@ def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None, 
     return out
 
 
-def sddmm(row_offsets, col_indices, lhs, rhs, out=None, workspace=None):
+def sddmm(row_offsets, col_indices, lhs, rhs, out=None, workspace=None, plan=None):
     """out[j] = <lhs[i], rhs[col[j]]> for each CSR slot j of row i, on the current stream.
     `workspace`: None, ROWS_EVEN, or a GPU tensor of workspace_bytes(OP_SDDMM, ...) bytes (the slice boundaries of the
     column-sliced schedule; 0 bytes where that schedule does not apply)."""
@@ -195,6 +201,16 @@ def sddmm(row_offsets, col_indices, lhs, rhs, out=None, workspace=None):
     K, D = rhs.shape
     if out is None:
         out = torch.empty((nnz,), dtype=torch.float32, device=lhs.device)
+    if plan is not None:
+        if workspace is not None:
+            raise ValueError("pass a row plan or a workspace, not both")
+        st = lib().sddmm_csr_f32_planned(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
+                                         _ptr(col_indices, torch.int32, "col_indices"), _ptr(lhs, torch.float32, "lhs"),
+                                         _ptr(rhs, torch.float32, "rhs"), _ptr(out, torch.float32, "out"),
+                                         _ptr(plan, torch.int32, "plan"), plan.numel() * 4, _stream())
+        if st != OK:
+            raise DlspmError(st, "sddmm_csr_f32_planned")
+        return out
     st = lib().sddmm_csr_f32(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
                              _ptr(col_indices, torch.int32, "col_indices"), _ptr(lhs, torch.float32, "lhs"),
                              _ptr(rhs, torch.float32, "rhs"), _ptr(out, torch.float32, "out"), *_workspace(workspace),
@@ -204,9 +220,10 @@ def sddmm(row_offsets, col_indices, lhs, rhs, out=None, workspace=None):
     return out
 
 
-def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None, workspace=None):
+def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None, workspace=None, plan=None):
     """O = (S .* (Q Kmat^T) * scale) V on the current stream; the scores are never stored.
-    `workspace`: optional GPU tensor of at least workspace_bytes(OP_FUSED, ...) bytes, or ROWS_EVEN."""
+    `workspace`: optional GPU tensor of at least workspace_bytes(OP_FUSED, ...) bytes, or ROWS_EVEN.
+    `plan`: optional row plan of the mask (row_plan()), instead of a workspace."""
     import torch
 
     M = row_offsets.numel() - 1
@@ -214,6 +231,17 @@ def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None, workspace=N
     K, D = Kmat.shape
     if out is None:
         out = torch.empty((M, D), dtype=torch.float32, device=Q.device)
+    if plan is not None:
+        if workspace is not None:
+            raise ValueError("pass a row plan or a workspace, not both")
+        st = lib().fused_sddmm_spmm_f32_planned(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
+                                                _ptr(col_indices, torch.int32, "col_indices"), _ptr(Q, torch.float32, "Q"),
+                                                _ptr(Kmat, torch.float32, "Kmat"), _ptr(V, torch.float32, "V"),
+                                                ctypes.c_float(scale), _ptr(out, torch.float32, "O"),
+                                                _ptr(plan, torch.int32, "plan"), plan.numel() * 4, _stream())
+        if st != OK:
+            raise DlspmError(st, "fused_sddmm_spmm_f32_planned")
+        return out
     st = lib().fused_sddmm_spmm_f32(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
                                     _ptr(col_indices, torch.int32, "col_indices"), _ptr(Q, torch.float32, "Q"),
                                     _ptr(Kmat, torch.float32, "Kmat"), _ptr(V, torch.float32, "V"),

@@ -209,7 +209,7 @@ struct Options {
     // at most one and a half times the mean;
     // --workspace: always the memory, --no-workspace: always NULL
     enum Workspace { kAuto, kAlways, kNever } workspace = kAuto;
-    bool plan = true;  // SpMM: build a row plan where dlspm_row_plan_advice says so (--no-plan: never)
+    bool plan = true;  // build a row plan where dlspm_row_plan_advice says so (--no-plan: never)
     std::string csv, dump;
     double tol = 1e-4;  // relative Frobenius error allowed between the kernel and the check kernel
 };
@@ -219,7 +219,7 @@ struct Options {
 struct WorkspaceChoice {
     size_t bytes = 0;        // device memory to allocate and pass
     bool rows_even = false;  // pass DLSPM_ROWS_EVEN instead
-    bool plan = false;       // SpMM: build a row plan and launch spmm_csr_f32_planned instead
+    bool plan = false;       // build a row plan and launch the op's _planned entry point instead
     void* arg(void* buffer) const { return rows_even ? DLSPM_ROWS_EVEN : bytes ? buffer : nullptr; }
 };
 inline WorkspaceChoice workspace_to_pass(const Options& opt, int op, int M, int K, int width, int nnz,
@@ -230,7 +230,7 @@ inline WorkspaceChoice workspace_to_pass(const Options& opt, int op, int M, int 
     const size_t want = dlspm_workspace_bytes(op, M, K, width, nnz);
     int longest = 0, empty = 0;
     if (dlspm_csr_row_stats(M, row_offsets_dev, nullptr, &longest, &empty) != DLSPM_OK) throw std::runtime_error("dlspm_csr_row_stats failed");
-    if (plan_allowed && opt.workspace == Options::kAuto && dlspm_row_plan_advice(M, K, width, nnz, longest) == 1) {
+    if (plan_allowed && opt.workspace == Options::kAuto && dlspm_row_plan_advice(op, M, K, width, nnz, longest) == 1) {
         c.plan = true;
         std::printf("rows: longest %d, mean %.1f, empty %d -> uneven, row plan (one row per workgroup, handed out by length)\n",
                     longest, (double)nnz / M, empty);
@@ -248,6 +248,17 @@ inline WorkspaceChoice workspace_to_pass(const Options& opt, int op, int M, int 
                 : c.rows_even                     ? "even, DLSPM_ROWS_EVEN passed"
                                                   : "nothing passed");
     return c;
+}
+
+// The row plan of one matrix (dlspm_row_plan_build: once per matrix, synchronises), with what it cost.
+inline DevBuf<char> build_row_plan(int M, const int* row_offsets_dev)
+{
+    DevBuf<char> plan(dlspm_row_plan_bytes(M));
+    const auto t0 = std::chrono::steady_clock::now();
+    if (dlspm_row_plan_build(M, row_offsets_dev, plan.p, plan.n, nullptr) != DLSPM_OK) throw std::runtime_error("dlspm_row_plan_build failed");
+    const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+    std::printf("row plan: %zu bytes, built in %.3f ms (once per matrix)\n", plan.n, ms);
+    return plan;
 }
 
 template <typename Launch> Timing time_launches(const Options& opt, Launch&& launch)

@@ -44,10 +44,12 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     if (dlspm_csr_check(M, K, nnz, ro_d.p, ci_d.p, nullptr) != DLSPM_OK) throw std::invalid_argument("malformed CSR structure");
     DLSPM_HIP_CHECK(hipMemset(O_d.p, 0xFF, (size_t)M * D * sizeof(float)));
 
-    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_FUSED, M, K, D, nnz, ro_d.p);  // 0 bytes for small problems
+    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_FUSED, M, K, D, nnz, ro_d.p, opt.plan);  // 0 bytes for small problems
     DevBuf<char> ws(wc.bytes);
     if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
+    DevBuf<char> plan = wc.plan ? build_row_plan(M, ro_d.p) : DevBuf<char>(0);
     const Timing t = time_launches(opt, [&]() {
+        if (wc.plan) return fused_sddmm_spmm_f32_planned(M, K, D, nnz, ro_d.p, ci_d.p, Q_d.p, K_d.p, V_d.p, scale, O_d.p, plan.p, plan.n, nullptr);
         return fused_sddmm_spmm_f32(M, K, D, nnz, ro_d.p, ci_d.p, Q_d.p, K_d.p, V_d.p, scale, O_d.p, wc.arg(ws.p),
                                     wc.bytes, nullptr);
     });

@@ -49,13 +49,7 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     DevBuf<char> ws(wc.bytes);
     if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
     const bool planned = wc.plan;
-    DevBuf<char> plan(planned ? dlspm_row_plan_bytes(M) : 0);
-    if (planned) {
-        const auto t0 = std::chrono::steady_clock::now();
-        if (dlspm_row_plan_build(M, ro_d.p, plan.p, plan.n, nullptr) != DLSPM_OK) throw std::runtime_error("dlspm_row_plan_build failed");
-        const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
-        std::printf("row plan: %zu bytes, built in %.3f ms (once per matrix)\n", plan.n, ms);
-    }
+    DevBuf<char> plan = planned ? build_row_plan(M, ro_d.p) : DevBuf<char>(0);
     const Timing t = time_launches(opt, [&]() {
         if (planned) return spmm_csr_f32_planned(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, plan.p, plan.n, nullptr);
         return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, wc.arg(ws.p), wc.bytes, nullptr);

@@ -190,7 +190,7 @@ def test_row_plan_host_side(dl):
     """Size, advice and argument checks of the row plan need no GPU."""
     L = dl.lib()
     assert L.dlspm_row_plan_bytes(2048) == 3 * 2048 * 4 and L.dlspm_row_plan_bytes(0) == 0 and L.dlspm_row_plan_bytes(-5) == 0
-    A = dl.row_plan_advice
+    A = lambda *a: dl.row_plan_advice(dl.OP_SPMM, *a)
     assert A(2048, 512, 256, 105687, 312)            # the headline configuration: uneven rows, one row per workgroup
     assert A(2048, 512, 256, 105687, -1)             # rows unknown: nothing better to pass
     assert not A(2048, 512, 256, 105687, 60)         # even rows: another order gains nothing

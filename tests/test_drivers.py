@@ -212,7 +212,7 @@ def test_drivers_pass_the_workspace_only_for_uneven_rows():
         assert rc == 0 and "PASS" in out and "even, DLSPM_ROWS_EVEN passed" in out, out
     rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 0.2, "--iters", 3, "--no-plan")
     assert rc == 0 and "PASS" in out and "nothing passed" in out and "workspace:" not in out, out
-    rc, out = run("sddmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 0.2, "--iters", 3)
+    rc, out = run("sddmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 0.2, "--iters", 3, "--no-plan")
     assert rc == 0 and "PASS" in out and "nothing passed" in out, out
     rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--no-workspace", "--iters", 3)
     assert rc == 0 and "PASS" in out and "rows:" not in out, out
@@ -220,8 +220,11 @@ def test_drivers_pass_the_workspace_only_for_uneven_rows():
     assert rc == 0 and "PASS" in out and "uneven, workspace passed" in out and "workspace:" in out, out
     rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 1.5, "--iters", 3)   # SpMM prefers a row plan
     assert rc == 0 and "PASS" in out and "uneven, row plan" in out and "workspace:" not in out, out
-    rc, out = run("fused_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 1.5, "--iters", 3)
+    rc, out = run("fused_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 1.5, "--iters", 3, "--no-plan")
     assert rc == 0 and "PASS" in out and "uneven, workspace passed" in out, out
+    for app in ("fused_run", "sddmm_run"):   # all three ops prefer a row plan on uneven rows
+        rc, out = run(app, "--shape", 8192, 4096, 128, 0.1, "--sigma", 1.5, "--iters", 3)
+        assert rc == 0 and "PASS" in out and "uneven, row plan" in out and "row plan:" in out, out
     rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--workspace", "--iters", 3)
     assert rc == 0 and "PASS" in out and "workspace passed (--workspace)" in out, out
 

@@ -524,7 +524,7 @@ def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle, mon
         if one_tile and sh["R"] == 1:
             assert torch.equal(got, want), (kind, shape)
             used += 1
-        elif one_tile and dl.row_plan_advice(M, K, N, ci.size, -1):
+        elif one_tile and dl.row_plan_advice(dl.OP_SPMM, M, K, N, ci.size, -1):
             assert torch.equal(got, want_one_row), (kind, shape)
             assert not torch.equal(want, want_one_row)   # the two shapes do round differently: the check above means something
             ungrouped += 1
@@ -533,6 +533,45 @@ def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle, mon
         assert oracle.rel_frobenius(got.cpu().numpy(), oracle.spmm(ro, ci, va, B)) <= TOL
         check_csr_untouched(ro_d, ci_d, ro, ci)
     assert used >= 5 and ungrouped >= 1 and used + ungrouped < len(cases)   # planned kernel, ungrouping and the fall-back
+
+
+def test_row_plan_for_sddmm_and_the_fused_op(torch_cuda, dl, oracle, monkeypatch):
+    """The same plan drives sddmm_csr_f32_planned and fused_sddmm_spmm_f32_planned: one row of the mask per four-wave
+    workgroup, in plan order. Their results must have the bits of the plain calls in that same shape (the size rule's
+    own, or DLSPM_SPLIT=4,1 where the rule groups rows), and agree with the oracle; widths outside 16 < D <= 512 and short
+    rows run as without a plan."""
+    torch = torch_cuda
+    rng = np.random.default_rng(99)
+    cases = [("skewed", 2048, 2048, 64, 0.05), ("skewed", 2049, 700, 128, 0.15), ("skewed", 4096, 1024, 40, 0.1),
+             ("empty_rows", 3000, 512, 256, 0.3), ("skewed", 1500, 900, 512, 0.2), ("skewed", 2048, 512, 16, 0.1),
+             ("skewed", 5000, 600, 100, 0.02), ("skewed", 1024, 1024, 33, 0.1)]
+    planned = {dl.OP_SDDMM: 0, dl.OP_FUSED: 0}
+    for kind, M, K, D, den in cases:
+        ro, ci = random_csr(rng, M, K, kind, den)
+        print(f"planned sddmm/fused case {kind} {M}x{K} D {D} nnz {ci.size}", flush=True)
+        Q = rng.normal(0, 1, (M, D)).astype(np.float32)
+        Km = rng.normal(0, 1, (K, D)).astype(np.float32)
+        V = rng.normal(0, 1, (K, D)).astype(np.float32)
+        ro_d, ci_d, Q_d, K_d, V_d = (dev(torch, x) for x in (ro, ci, Q, Km, V))
+        plan = dl.row_plan(ro_d)
+        for op, plain, with_plan in (
+                (dl.OP_SDDMM, lambda: dl.sddmm(ro_d, ci_d, Q_d, K_d).clone(), lambda: dl.sddmm(ro_d, ci_d, Q_d, K_d, plan=plan).clone()),
+                (dl.OP_FUSED, lambda: dl.fused(ro_d, ci_d, Q_d, K_d, V_d, 0.25).clone(), lambda: dl.fused(ro_d, ci_d, Q_d, K_d, V_d, 0.25, plan=plan).clone())):
+            want = plain()
+            monkeypatch.setenv("DLSPM_SPLIT", "4,1")
+            want_one_row = plain()
+            monkeypatch.delenv("DLSPM_SPLIT")
+            got = with_plan()
+            if dl.row_plan_advice(op, M, K, D, ci.size, -1):
+                assert torch.equal(got, want_one_row), (kind, M, K, D, op)
+                planned[op] += 1
+            else:
+                assert torch.equal(got, want), (kind, M, K, D, op)
+        assert oracle.rel_frobenius(dl.sddmm(ro_d, ci_d, Q_d, K_d, plan=plan).cpu().numpy(), oracle.sddmm(ro, ci, Q, Km)) <= TOL
+        assert oracle.rel_frobenius(dl.fused(ro_d, ci_d, Q_d, K_d, V_d, 0.25, plan=plan).cpu().numpy(),
+                                    oracle.fused(ro, ci, Q, Km, V, 0.25)) <= TOL
+        check_csr_untouched(ro_d, ci_d, ro, ci)
+    assert 4 <= planned[dl.OP_SDDMM] < len(cases) and 4 <= planned[dl.OP_FUSED] < len(cases)
 
 
 def test_stale_row_plan_stays_inside_the_arrays(torch_cuda, dl):
