@@ -207,7 +207,23 @@ def test_row_plan_host_side(dl):
     assert dl.workspace_advice(dl.OP_SPMM, 16384, 4096, 128, 16384 * 400, 4000) == dl.PASS_WORKSPACE   # (what is said without a plan)
     assert not A(8192, 16384, 128, 8192 * 800, 8000)  # B of 8 MiB: the column-sliced schedule's workspace first
     assert not A(0, 0, 0, 0, 0)
+    # the other two ops: built for 16 < D <= 512
+    for op in (dl.OP_SDDMM, dl.OP_FUSED):
+        assert dl.row_plan_advice(op, 2048, 2048, 64, 2048 * 100, 500)
+        assert dl.row_plan_advice(op, 8192, 2048, 128, 8192 * 200, 2000)
+        assert not dl.row_plan_advice(op, 2048, 2048, 64, 2048 * 100, 120)     # even rows
+        assert not dl.row_plan_advice(op, 2048, 2048, 16, 2048 * 100, 500)     # D <= 16
+        assert not dl.row_plan_advice(op, 2048, 2048, 1024, 2048 * 100, 500)   # D > 512
+        assert not dl.row_plan_advice(op, 8192, 2048, 64, 8192 * 20, 200)      # short rows
+    assert not dl.row_plan_advice(dl.OP_FUSED, 8192, 8192, 128, 8192 * 800, 8000)   # Kmat and V of 8 MiB: the slices first
+    assert not dl.row_plan_advice(7, 2048, 2048, 64, 2048 * 100, 500)
     bogus = ctypes.c_void_p(256)   # never dereferenced: the checks come first
+    assert L.sddmm_csr_f32_planned(2, 2, -4, 1, None, None, None, None, None, bogus, 24, None) == dl.E_INVALID_ARG
+    assert L.sddmm_csr_f32_planned(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, bogus, 23, None) == dl.E_WORKSPACE
+    assert L.sddmm_csr_f32_planned(2, 2, 32, 1, None, None, None, None, None, None, 0, None) == dl.E_INVALID_ARG
+    assert L.fused_sddmm_spmm_f32_planned(2, 2, 32, 9, None, None, None, None, None, 1.0, None, bogus, 24, None) == dl.E_INVALID_ARG
+    assert L.fused_sddmm_spmm_f32_planned(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, 1.0, bogus, bogus, 23, None) == dl.E_WORKSPACE
+    assert L.fused_sddmm_spmm_f32_planned(2, 2, 32, 1, None, None, None, None, None, 1.0, None, None, 0, None) == dl.E_INVALID_ARG
     assert L.dlspm_row_plan_build(-1, bogus, bogus, 0, None) == dl.E_INVALID_ARG
     assert L.dlspm_row_plan_build(8, None, bogus, 96, None) == dl.E_INVALID_ARG
     assert L.dlspm_row_plan_build(8, bogus, bogus, 95, None) == dl.E_WORKSPACE
