@@ -303,15 +303,17 @@ __global__ __launch_bounds__(4 * 64) void spmm_sliced_kernel(int M, int N, int c
 }
 
 // Row plan: workgroup i works on the whole row rows[i] = [starts[i], ends[i]) of the CSR matrix (one row per four-wave
-// workgroup, one column tile).
+// workgroup); with column tiles the plan is gone through once per tile, tile after tile.
 template <int VEC, int G, int V>
-__global__ __launch_bounds__(4 * 64) void spmm_planned_kernel(int M, int N, int nnz, const int* __restrict__ starts,
+__global__ __launch_bounds__(4 * 64) void spmm_planned_kernel(int M, int N, int nnz, int col_tiles,
+                                                              const int* __restrict__ starts,
                                                               const int* __restrict__ ends, const int* __restrict__ rows,
                                                               const int* __restrict__ col_indices,
                                                               const float* __restrict__ values,
                                                               const float* __restrict__ B, float* __restrict__ C)
 {
-    spmm_block<VEC, G, V, 4, 1, true, true>((int)blockIdx.x, M, N, 1, 0, starts, ends, col_indices, values, B, C, rows, nnz);
+    spmm_block<VEC, G, V, 4, 1, true, true>((int)blockIdx.x, M, N, col_tiles, 1, starts, ends, col_indices, values, B, C, rows,
+                                            nnz);
 }
 
 // ---- host side --------------------------------------------------------------------------------------
@@ -608,7 +610,9 @@ bool plan_ungroups(int M, int width, int nnz)
 
 bool spmm_plan_applies(SpmmShape& s, int M, int N, int nnz)
 {
-    if (s.vec != 4 || s.W != 4 || s.G * s.vec * s.V < N) return false;
+    // one column tile, or tiles in tile-major order (a B beyond one L2): there the workgroups of one tile are consecutive,
+    // as the plan's packing assumes; tiles in row-major order (B within the L2) keep the matrix order
+    if (s.vec != 4 || s.W != 4 || (s.G * s.vec * s.V < N && !s.tile_major)) return false;
     if (s.R == 1) return true;
     if (!plan_ungroups(M, N, nnz)) return false;
     s.R = 1;
@@ -621,8 +625,11 @@ hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int*
     const int *starts = plan, *ends = plan + x.M, *rows = plan + 2 * (size_t)x.M;
 #define DLSPM_PLANNED(g_, v_)                                                                                          \
     if (s.G == g_ && s.V == v_) {                                                                                      \
-        hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M, x.N,   \
-                           x.nnz, starts, ends, rows, x.col_indices, x.values, x.B, x.C);                                     \
+        const int col_tiles = (x.N + g_ * 4 * v_ - 1) / (g_ * 4 * v_);                                                 \
+        const long long blocks = (long long)x.M * col_tiles;                                                           \
+        if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;                                                \
+        hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M, x.N, \
+                           x.nnz, col_tiles, starts, ends, rows, x.col_indices, x.values, x.B, x.C);                   \
         return hipGetLastError();                                                                                      \
     }
     DLSPM_PLANNED(64, 2)

@@ -162,7 +162,7 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
  *                            the same row_offsets (a stale plan gives wrong values but stays inside the arrays).
  *                            It runs one row per workgroup also where spmm_csr_f32 would group a few rows, if the
  *                            rows are long enough (the same sums as spmm_csr_f32 under DLSPM_SPLIT=4,1). Short rows,
- *                            wide dense rows in column tiles and widths below 4 ignore it and run as
+ *                            column tiles of a B that fits one L2 and widths below 4 ignore it and run as
  *                            spmm_csr_f32(..., NULL, 0, stream); plan == NULL too.
  * No counterpart in the reference, whose kernels take the rows in matrix order (SPMM/spmmesimd2.hpp:63-75).
  */

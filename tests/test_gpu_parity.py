@@ -483,15 +483,15 @@ def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle, mon
     """spmm_csr_f32_planned hands the rows to the workgroups in the plan's order (longest first), one row per four-wave
     workgroup, and must return the bits of spmm_csr_f32 (NULL workspace) in that same shape -- which is the size rule's
     own shape for most of these cases, and the shape forced by DLSPM_SPLIT=4,1 where the rule groups rows and the plan
-    ungroups them. The plan itself is a permutation of the rows with each row's own offsets. Short rows, column tiles and
-    widths below 4 ignore the plan and run as without it."""
+    ungroups them. The plan itself is a permutation of the rows with each row's own offsets. Short rows, column tiles of a
+    B that fits the L2 and widths below 4 ignore the plan and run as without it."""
     torch = torch_cuda
     rng = np.random.default_rng(97)
     cases = [("cfg2", None), ("cfg1", None), ("cfg4", None),
              ("skewed", (2049, 600, 256)), ("empty_rows", (300, 512, 128)), ("skewed", (1, 700, 64)),
              ("skewed", (5000, 2048, 50)), ("uniform", (4096, 1024, 256)), ("skewed", (2048, 512, 3)),
-             ("skewed", (600, 512, 784)), ("skewed", (9000, 300, 128))]
-    used = ungrouped = 0
+             ("skewed", (600, 512, 784)), ("skewed", (9000, 300, 128)), ("skewed", (1100, 2200, 1024))]
+    used = ungrouped = tiled = 0
     for kind, shape in cases:
         if shape is None:
             c = dl.make_config(int(kind[3]))
@@ -514,25 +514,25 @@ def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle, mon
         if M > 2048:
             assert (lens[2048:][:-1] >= lens[2048:][1:]).all()                   # after the resident part: descending
         sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size)
-        one_tile = sh["vec"] == 4 and sh["W"] == 4 and sh["col_tiles"] == 1
         want = dl.spmm(ro_d, ci_d, va_d, B_d, K=K).clone()
         monkeypatch.setenv("DLSPM_SPLIT", "4,1")
         want_one_row = dl.spmm(ro_d, ci_d, va_d, B_d, K=K).clone()
         monkeypatch.delenv("DLSPM_SPLIT")
         got = torch.full((M, N), float("nan"), device="cuda")
         dl.spmm(ro_d, ci_d, va_d, B_d, K=K, out=got, plan=plan)
-        if one_tile and sh["R"] == 1:
-            assert torch.equal(got, want), (kind, shape)
-            used += 1
-        elif one_tile and dl.row_plan_advice(dl.OP_SPMM, M, K, N, ci.size, -1):
+        if dl.row_plan_advice(dl.OP_SPMM, M, K, N, ci.size, -1):   # rows unknown: 1 exactly where the planned kernel runs
             assert torch.equal(got, want_one_row), (kind, shape)
-            assert not torch.equal(want, want_one_row)   # the two shapes do round differently: the check above means something
-            ungrouped += 1
+            used += 1
+            tiled += int(sh["col_tiles"] > 1)
+            if sh["R"] != 1:
+                assert not torch.equal(want, want_one_row)   # the two shapes do round differently: the check above means something
+                ungrouped += 1
         else:
             assert torch.equal(got, want), (kind, shape)
         assert oracle.rel_frobenius(got.cpu().numpy(), oracle.spmm(ro, ci, va, B)) <= TOL
         check_csr_untouched(ro_d, ci_d, ro, ci)
-    assert used >= 5 and ungrouped >= 1 and used + ungrouped < len(cases)   # planned kernel, ungrouping and the fall-back
+    # the planned kernel, rows ungrouped by it, column tiles gone through in plan order, and the fall-back
+    assert used >= 6 and ungrouped >= 1 and tiled >= 1 and used < len(cases)
 
 
 def test_row_plan_for_sddmm_and_the_fused_op(torch_cuda, dl, oracle, monkeypatch):
