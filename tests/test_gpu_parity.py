@@ -623,6 +623,8 @@ def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
         ws_s = ws if schedule == "sliced" else None  # SDDMM uses a workspace under the sliced schedule only
         C = torch.empty(M, N, device="cuda")
         CP = torch.empty(M, N, device="cuda")
+        SP = torch.empty(ci.size, device="cuda")
+        OP = torch.empty(M, N, device="cuda")
         plan = dl.row_plan(ro_d)
         S = torch.empty(ci.size, device="cuda")
         O = torch.empty(M, N, device="cuda")
@@ -635,17 +637,23 @@ def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
                 dl.spmm(ro_d, ci_d, va, B, K=K, out=C, workspace=ws)
                 dl.sddmm(ro_d, ci_d, Q, B, out=S, workspace=ws_s)
                 dl.fused(ro_d, ci_d, Q, B, B, 0.5, out=O, workspace=ws)
-                if schedule == "row-block":
-                    dl.spmm(ro_d, ci_d, va, B, K=K, out=CP, plan=plan)   # a planned launch is one kernel too
+                if schedule == "row-block":   # planned launches are one kernel each too
+                    dl.spmm(ro_d, ci_d, va, B, K=K, out=CP, plan=plan)
+                    dl.sddmm(ro_d, ci_d, Q, B, out=SP, plan=plan)
+                    dl.fused(ro_d, ci_d, Q, B, B, 0.5, out=OP, plan=plan)
         for rep in range(4):
             va.copy_(torch.randn(ci.size, device="cuda"))  # eager work between the replays: new inputs
             B.copy_(torch.randn(K, N, device="cuda"))
             torch.cuda.synchronize()
-            C.fill_(float("nan")); S.fill_(float("nan")); O.fill_(float("nan")); CP.fill_(float("nan"))
+            for buf in (C, S, O, CP, SP, OP):
+                buf.fill_(float("nan"))
             graph.replay()
             torch.cuda.synchronize()
             if schedule == "row-block":
-                assert torch.equal(CP, C), f"replay {rep}, planned launch"
+                assert torch.equal(CP, dl.spmm(ro_d, ci_d, va, B, K=K, plan=plan)), f"replay {rep}, planned SpMM"
+                assert torch.equal(SP, dl.sddmm(ro_d, ci_d, Q, B, plan=plan)), f"replay {rep}, planned SDDMM"
+                assert torch.equal(OP, dl.fused(ro_d, ci_d, Q, B, B, 0.5, plan=plan)), f"replay {rep}, planned fused"
+                assert torch.allclose(CP, C, rtol=1e-4, atol=1e-4) and torch.equal(SP, S) and torch.allclose(OP, O, rtol=1e-4, atol=1e-3)
             got = (C.clone(), S.clone(), O.clone())
             want = (dl.spmm(ro_d, ci_d, va, B, K=K, workspace=ws).clone(), dl.sddmm(ro_d, ci_d, Q, B, workspace=ws_s).clone(),
                     dl.fused(ro_d, ci_d, Q, B, B, 0.5, workspace=ws).clone())
