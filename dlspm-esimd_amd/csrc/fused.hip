@@ -556,7 +556,7 @@ bool fused_plan_applies(FusedShape& s, int M, int D, int nnz)
     // built for 16 < D <= 512 (the shapes of the column-sliced kernels): one column tile
     if (s.vec != 4 || s.G1 != 8 || s.DS < 1 || s.W != 4 || s.G * s.vec * s.V < D) return false;
     if (s.R == 1) return true;
-    if (!plan_ungroups(M, D, nnz)) return false;
+    if (!plan_ungroups_dots(M, D, nnz)) return false;
     s.R = 1;
     return true;
 }

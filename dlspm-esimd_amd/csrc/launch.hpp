@@ -79,7 +79,8 @@ SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, b
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
 // Row plan (3 x M ints on the device: first nonzero, end and row number of the row that workgroup i works on): only for
 // shapes of one row per four-wave workgroup and one column tile
-bool plan_ungroups(int M, int width, int nnz);  // rows long enough that a plan runs them one per workgroup against the size rule
+bool plan_ungroups(int M, int width, int nnz);  // SpMM: rows long enough that a plan runs them one per workgroup against the size rule
+bool plan_ungroups_dots(int M, int D, int nnz);  // the same for SDDMM and the fused op
 bool spmm_plan_applies(SpmmShape& s, int M, int N, int nnz);  // true: s is the shape of the planned launch (R = 1)
 hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int* plan, hipStream_t stream);
 hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPlan& plan, float* partial,

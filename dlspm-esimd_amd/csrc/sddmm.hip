@@ -364,7 +364,7 @@ bool sddmm_plan_applies(SddmmShape& s, int M, int D, int nnz)
 {
     if (s.vec != 4 || s.G1 != 8 || s.DS < 1 || s.W != 4) return false;  // built for 16 < D <= 512
     if (s.R == 1) return true;
-    if (!plan_ungroups(M, D, nnz)) return false;
+    if (!plan_ungroups_dots(M, D, nnz)) return false;
     s.R = 1;
     return true;
 }

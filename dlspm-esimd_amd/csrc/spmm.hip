@@ -608,6 +608,15 @@ bool plan_ungroups(int M, int width, int nnz)
     return nnz >= avg32 && (M <= 4096 || (width >= 128 && (M <= 8192 || (nnz >= avg48 && M <= 16384) || nnz >= avg128)));
 }
 
+// The same question for SDDMM and the fused op, which gain less from one row per workgroup: lognormal rows, sigma 0.6, rule's
+// grouping against one row per workgroup in plan order: mask 2048 x 2048, D = 64, 100 per row: fused 12.5 -> 8.6 us;
+// 4096 x 1024: 14.2 -> 11.7 us; 8192 x 2048, D = 128, 197 per row: 76.9 -> 58.1 us; but 16384 x 2048, D = 128, 60 per row: 44.9 ->
+// 55.8 us; 32768 x 4096, D = 64, 100 per row: 68.8 -> 88.1 us; 8192 x 8192, D = 64, 100 per row: equal (SDDMM alike).
+bool plan_ungroups_dots(int M, int D, int nnz)
+{
+    return (long long)nnz >= 32ll * M && (M <= 4096 || (D >= 128 && M <= 8192 && (long long)nnz >= 128ll * M));
+}
+
 bool spmm_plan_applies(SpmmShape& s, int M, int N, int nnz)
 {
     // one column tile, or tiles in tile-major order (a B beyond one L2): there the workgroups of one tile are consecutive,

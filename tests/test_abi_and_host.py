@@ -215,6 +215,9 @@ def test_row_plan_host_side(dl):
         assert not dl.row_plan_advice(op, 2048, 2048, 16, 2048 * 100, 500)     # D <= 16
         assert not dl.row_plan_advice(op, 2048, 2048, 1024, 2048 * 100, 500)   # D > 512
         assert not dl.row_plan_advice(op, 8192, 2048, 64, 8192 * 20, 200)      # short rows
+        assert dl.describe_launch(op, 16384, 2048, 128, 16384 * 60)["R"] == 8
+        assert not dl.row_plan_advice(op, 16384, 2048, 128, 16384 * 60, 600)   # tall mask, grouped rows: the grouping wins
+        assert dl.row_plan_advice(op, 16384, 4096, 128, 16384 * 400, 4000)     # ... rows the rule runs one per workgroup anyway
     assert not dl.row_plan_advice(dl.OP_FUSED, 8192, 8192, 128, 8192 * 800, 8000)   # Kmat and V of 8 MiB: the slices first
     assert not dl.row_plan_advice(7, 2048, 2048, 64, 2048 * 100, 500)
     bogus = ctypes.c_void_p(256)   # never dereferenced: the checks come first
