@@ -163,7 +163,9 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
  *                            It runs one row per workgroup also where spmm_csr_f32 would group a few rows, if the
  *                            rows are long enough (the same sums as spmm_csr_f32 under DLSPM_SPLIT=4,1). Short rows,
  *                            column tiles of a B that fits one L2 and widths below 4 ignore it and run as
- *                            spmm_csr_f32(..., NULL, 0, stream); plan == NULL too.
+ *                            spmm_csr_f32(..., NULL, 0, stream); plan == NULL too. A planned launch is one kernel
+ *                            (no memset, no allocation, no synchronisation): it may be captured in a HIP graph; the
+ *                            plan is only read, so launches may share it.
  * No counterpart in the reference, whose kernels take the rows in matrix order (SPMM/spmmesimd2.hpp:63-75).
  */
 size_t dlspm_row_plan_bytes(int M);
@@ -181,7 +183,8 @@ int spmm_csr_f32_planned(int M, int K, int N, int nnz, const int* row_offsets, c
 /* The same plan (it depends on row_offsets only) for the other two ops, with the arguments of sddmm_csr_f32 and
  * fused_sddmm_spmm_f32 and the plan in place of the workspace. Measured on lognormal rows against the plain calls:
  * 2048 x 2048 mask, D = 64, 100 per row: fused 12.3 -> 8.4 us, SDDMM 6.8 -> 5.0 us; 8192 x 2048, D = 128, 197 per row:
- * 77.6 -> 57.4 us and 41.5 -> 30.8 us. Widths outside 16 < D <= 512, short rows and column tiles ignore the plan. */
+ * 77.6 -> 57.4 us and 41.5 -> 30.8 us. Widths outside 16 < D <= 512, short rows, and rows that the size rule groups in
+ * masks of more than 4096 rows (8192 at D >= 128 and 128 nonzeros per row) ignore the plan. */
 int sddmm_csr_f32_planned(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* lhs,
                           const float* rhs, float* out_values, const void* plan, size_t plan_bytes, void* stream);
 int fused_sddmm_spmm_f32_planned(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices,
