@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-graph] [--no-cpu] [--all-configs]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-graph] [--no-cpu] [--no-plan] [--all-configs]
 
 A "step" is one launch of the configuration's kernel (default: BASELINE.json's configs[1], fp32 CSR SpMM
 2048x512 * 512x256 at 90 % sparsity with lognormal-skewed rows) on inputs that already sit in device memory.
@@ -16,6 +16,9 @@ Prints ONE JSON line:
   cpu_baseline      the CPU oracle (a port of the reference's scalar loop) timed on this host, 1 core, and the
                     same loop over all cores for reference
   cold_us/warm_us   single launches timed with events after flushing the caches with a 1 GiB fill / back to back
+  row_plan          (SpMM on uneven rows) the steps are spmm_csr_f32_planned launches; the plan is built once per matrix
+                    before the timed region, like the look at the row lengths; this object gives what building it cost
+                    and the time of the same launches in matrix order (--no-plan measures those as the headline)
 """
 import argparse
 import json
