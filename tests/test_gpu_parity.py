@@ -478,6 +478,26 @@ def test_exact_integer_properties_at_large_size(torch_cuda, dl):
     assert torch.equal(O, torch.from_numpy(colsum.astype(np.float32)).cuda()[:, None].expand(M, D))
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
+    # the same properties through the planned entry points, on rows long enough (200 on average) that the planned SpMM
+    # launch really runs in plan order (65536 workgroups, one row each); 16384 rows for the other two ops
+    for rows, planned_ops in ((65536, (dl.OP_SPMM,)), (16384, (dl.OP_SPMM, dl.OP_SDDMM, dl.OP_FUSED))):
+        ro, ci = dl.make_pattern(dl.PATTERN_LOGNORMAL_ROWS, 32, rows, K, 200.0 if rows == 65536 else 400.0, 1.0)
+        lens = np.diff(ro).astype(np.int64)
+        colsum = np.add.reduceat(np.append(ci.astype(np.int64), 0), ro[:-1])[:rows] * (lens > 0)
+        assert colsum.max() < 2**24
+        for op in planned_ops:
+            assert dl.row_plan_advice(op, rows, K, D, ci.size, int(lens.max()))
+        ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+        plan = dl.row_plan(ro_d)
+        ones_nnz = torch.ones(ci.size, dtype=torch.float32, device="cuda")
+        C = dl.spmm(ro_d, ci_d, ones_nnz, ones_KD, K=K, plan=plan)
+        assert torch.equal(C, torch.from_numpy(lens.astype(np.float32)).cuda()[:, None].expand(rows, D))
+        out = dl.sddmm(ro_d, ci_d, ones_MD[:rows], ramp, plan=plan)
+        assert torch.equal(out, ci_d.to(torch.float32))
+        O = dl.fused(ro_d, ci_d, ones_MD[:rows], ramp, ones_KD, 1.0, plan=plan)
+        assert torch.equal(O, torch.from_numpy(colsum.astype(np.float32)).cuda()[:, None].expand(rows, D))
+        check_csr_untouched(ro_d, ci_d, ro, ci)
+
 
 def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle, monkeypatch):
     """spmm_csr_f32_planned hands the rows to the workgroups in the plan's order (longest first), one row per four-wave
