@@ -24,6 +24,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <filesystem>
 #include <fstream>
 #include <iostream>
 #include <sstream>
@@ -211,6 +212,7 @@ struct Options {
     enum Workspace { kAuto, kAlways, kNever } workspace = kAuto;
     bool plan = true;  // build a row plan where dlspm_row_plan_advice says so (--no-plan: never)
     std::string csv, dump;
+    std::string dump_each;  // --dump-each DIR: every case dumps into its own sub-directory DIR/case_000, DIR/case_001, ...
     double tol = 1e-4;  // relative Frobenius error allowed between the kernel and the check kernel
 };
 
@@ -386,7 +388,7 @@ inline std::string usage(const char* app, const char* width)
       << "                                                     --sigma: lognormal row lengths, skewed)\n"
       << "       " << app << " --sweep [--max-m M]                  the 12 x {32,128} x {0.3,0.2,0.1} benchmark grid\n"
       << "       " << app << " --cfg <id>                           a seeded benchmark configuration (1..5)\n"
-      << "options: --iters n (20)  --warmup n (5)  --cold  --csv <file>  --dump <dir>  --tol x (1e-4)  --workspace | --no-workspace  --no-plan";
+      << "options: --iters n (20)  --warmup n (5)  --cold  --csv <file>  --dump <dir> | --dump-each <dir>  --tol x (1e-4)  --workspace | --no-workspace  --no-plan";
     return u.str();
 }
 
@@ -434,6 +436,7 @@ inline Cli parse_cli(int argc, char** argv, const char* app, const char* width)
         else if (a == "--cold") cli.opt.cold = true;
         else if (a == "--csv") { need(i, 1); cli.opt.csv = argv[++i]; }
         else if (a == "--dump") { need(i, 1); cli.opt.dump = argv[++i]; }
+        else if (a == "--dump-each") { need(i, 1); cli.opt.dump_each = argv[++i]; }
         else if (a == "--tol") { need(i, 1); cli.opt.tol = std::stod(argv[++i]); }
         else if (a.rfind("--", 0) == 0) throw std::invalid_argument(usage(app, width));
         else pos.push_back(a);
@@ -446,6 +449,19 @@ inline Cli parse_cli(int argc, char** argv, const char* app, const char* width)
     }
     if (cli.cases.empty()) throw std::invalid_argument(usage(app, width));
     return cli;
+}
+
+// Options of case number `index` of a run: with --dump-each every case dumps into a sub-directory of its own (created
+// here), so that a sweep or a batch can be verified case by case from outside.
+inline Options case_options(const Options& opt, size_t index)
+{
+    if (opt.dump_each.empty()) return opt;
+    Options o = opt;
+    char name[32];
+    std::snprintf(name, sizeof name, "case_%03zu", index);
+    o.dump = opt.dump_each + "/" + name;
+    std::filesystem::create_directories(o.dump);
+    return o;
 }
 
 inline void print_device()

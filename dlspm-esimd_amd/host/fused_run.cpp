@@ -98,7 +98,7 @@ int main(int argc, char** argv)
         const Cli cli = parse_cli((int)rest.size(), rest.data(), "fused_run", "NSZ");
         print_device();
         bool ok = true;
-        for (const auto& c : cli.cases) ok = run_case(c, cli.opt) && ok;
+        for (size_t i = 0; i < cli.cases.size(); ++i) ok = run_case(cli.cases[i], case_options(cli.opt, i)) && ok;
         return ok ? 0 : 2;
     } catch (std::exception& e) {
         std::cout << e.what() << std::endl;

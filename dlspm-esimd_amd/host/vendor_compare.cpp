@@ -5,7 +5,9 @@
 // times rocsparse_spmm (every CSR algorithm, preprocess excluded) or rocsparse_sddmm, the fused configuration as
 // rocsparse_sddmm -> scale -> rocsparse_spmm ("unfused vendor path", as MKL's FusedMM = gemm + sparse gemm), and
 // the library's entry point, all as the minimum of `iters` launches bracketed by HIP events, and prints the
-// relative Frobenius difference between the two results.
+// relative Frobenius difference between the two results. Like the reference's comparators it checks itself: the
+// exit status is 2 when the two results differ by more than --tol (1e-4), and `--dump <dir>` writes both results
+// (cfg<id>_dlspm.f32, cfg<id>_rocsparse.f32) so that an external checker can hold each against its own gold.
 #include <rocsparse/rocsparse.h>
 
 #include "driver.hpp"
@@ -154,12 +156,17 @@ int main(int argc, char** argv)
 {
     try {
         int iters = 50, warmup = 10;
+        double tol = 1e-4;
+        std::string dump;
+        bool all_ok = true;
         std::vector<int> cfgs = {1, 2, 3, 4, 5};
         for (int i = 1; i < argc; ++i) {
             const std::string a = argv[i];
             if (a == "--iters" && i + 1 < argc) iters = std::max(1, std::stoi(argv[++i]));
             else if (a == "--cfg" && i + 1 < argc) cfgs = {std::stoi(argv[++i])};
-            else throw std::invalid_argument("Usage: vendor_compare [--cfg <id>] [--iters n]");
+            else if (a == "--tol" && i + 1 < argc) tol = std::stod(argv[++i]);
+            else if (a == "--dump" && i + 1 < argc) dump = argv[++i];
+            else throw std::invalid_argument("Usage: vendor_compare [--cfg <id>] [--iters n] [--tol x] [--dump <dir>]");
         }
         print_device();
         rocsparse_handle h;
@@ -173,11 +180,13 @@ int main(int argc, char** argv)
             DevBuf<int> ro(p.a.row_offsets), ci(p.a.col_indices);
             double t_ours = 0, t_vendor = 0, diff = 0;
             std::string alg = "default";
+            std::vector<float> ours, vendor;
             if (p.op == kSpmm) {
                 DevBuf<float> va(p.values), B(p.d0), C((size_t)M * N), Cv((size_t)M * N);
                 t_ours = min_ms(warmup, iters, [&]() { (void)spmm_csr_f32(M, K, N, nnz, ro.p, ci.p, va.p, B.p, C.p, nullptr, 0, nullptr); });
                 t_vendor = rocsparse_spmm_best(h, M, K, N, nnz, ro.p, ci.p, va.p, B.p, Cv.p, warmup, iters, alg);
-                diff = rel_frob(Cv.to_host(), C.to_host());
+                ours = C.to_host();
+                vendor = Cv.to_host();
             } else if (p.op == kSddmm) {
                 DevBuf<float> lhs(p.d0), rhs(p.d1), out((size_t)nnz), outv((size_t)nnz);
                 DLSPM_HIP_CHECK(hipMemset(outv.p, 0, (size_t)nnz * sizeof(float)));
@@ -185,7 +194,8 @@ int main(int argc, char** argv)
                 RsSddmm rs(h, M, K, N, nnz, ro.p, ci.p, lhs.p, rhs.p, outv.p);
                 t_vendor = min_ms(warmup, iters, [&]() { (void)rs.run(); });
                 std::printf("    rocsparse_sddmm default          %9.2f us\n", t_vendor * 1e3);
-                diff = rel_frob(outv.to_host(), out.to_host());
+                ours = out.to_host();
+                vendor = outv.to_host();
             } else {
                 DevBuf<float> Q(p.d0), Km(p.d1), V(p.d2), O((size_t)M * N), Ov((size_t)M * N), scores((size_t)nnz);
                 DLSPM_HIP_CHECK(hipMemset(scores.p, 0, (size_t)nnz * sizeof(float)));
@@ -203,13 +213,22 @@ int main(int argc, char** argv)
                 std::printf("    unfused vendor path: rocsparse_sddmm %.2f us + scale %.2f us + rocsparse_spmm(%s) %.2f us\n",
                             t_sddmm * 1e3, t_scale * 1e3, alg.c_str(), t_spmm * 1e3);
                 t_vendor = t_sddmm + t_scale + t_spmm;
-                diff = rel_frob(Ov.to_host(), O.to_host());
+                ours = O.to_host();
+                vendor = Ov.to_host();
+            }
+            diff = rel_frob(vendor, ours);
+            if (!(diff <= tol)) all_ok = false;
+            if (!dump.empty()) {
+                const std::string tag = "cfg" + std::to_string(cfg);
+                dump_array(dump, (tag + "_dlspm.f32").c_str(), ours.data(), ours.size() * 4);
+                dump_array(dump, (tag + "_rocsparse.f32").c_str(), vendor.data(), vendor.size() * 4);
             }
             std::printf("%-44s %12.2f %12.2f %7.2fx %12.3e   (best rocSPARSE algorithm: %s)\n\n", p.name, t_ours * 1e3,
                         t_vendor * 1e3, t_vendor / t_ours, diff, alg.c_str());
         }
         (void)rocsparse_destroy_handle(h);
-        return 0;
+        std::printf("vendor_compare %s (tolerance %g)\n", all_ok ? "PASS" : "FAIL", tol);
+        return all_ok ? 0 : 2;
     } catch (std::exception& e) {
         std::cout << e.what() << std::endl;
         return 1;

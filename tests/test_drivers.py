@@ -139,6 +139,84 @@ def test_driver_shape_and_small_sweep():
     assert rc == 0 and out.count("PASS") == 6  # (1024,1024) x N in {32,128} x density in {0.3,0.2,0.1}
 
 
+def verify_dump(oracle, d):
+    """Relative Frobenius error of one driver dump (inputs and the kernel's output) against the CPU oracle."""
+    meta, arr = load_dump(d)
+    M, K, N = meta["M"], meta["K"], meta["N"]
+    ro, ci = arr("row_offsets.i32", np.int32), arr("col_indices.i32", np.int32)
+    assert ro.size == M + 1 and ci.size == meta["nnz"] and ro[-1] == meta["nnz"]
+    if meta["op"] == "spmm":
+        ref = oracle.spmm(ro, ci, arr("values.f32", np.float32), arr("B.f32", np.float32).reshape(K, N), omp=True)
+        got = arr("C.f32", np.float32).reshape(M, N)
+    elif meta["op"] == "sddmm":
+        ref = oracle.sddmm(ro, ci, arr("lhs.f32", np.float32).reshape(M, N), arr("rhs.f32", np.float32).reshape(K, N), omp=True)
+        got = arr("out.f32", np.float32)
+    else:
+        ref = oracle.fused(ro, ci, arr("Q.f32", np.float32).reshape(M, N), arr("K.f32", np.float32).reshape(K, N),
+                           arr("V.f32", np.float32).reshape(K, N), meta["scale"], omp=True)
+        got = arr("O.f32", np.float32).reshape(M, N)
+    return meta, oracle.rel_frobenius(got, ref)
+
+
+SWEEP_GRID_2048 = [(M, K, N, sp) for N in (32, 128) for (M, K) in ((1024, 1024), (2048, 2048)) for sp in (0.3, 0.2, 0.1)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("app", ["spmm_run", "sddmm_run", "fused_run"])
+def test_sweep_against_the_oracle_and_csv_columns(oracle, tmp_path, app):
+    """The in-process sweep of the reference (grid SPMM/spmm-esimd-allbenchs2.cpp:252-266, CSV rows :221-226 and
+    SDDMM/sddmm-esimd-allbench_v4.cpp:204-209) up to 2048 rows: every case's dumped output is verified here against
+    the CPU oracle (the drivers' own PASS only compares with an on-device check kernel), and the CSV has the
+    reference's columns, one row per case, in grid order."""
+    dumps = tmp_path / "dumps"
+    rc, out = run(app, "--sweep", "--max-m", 2048, "--iters", 3, "--warmup", 1, "--dump-each", dumps, "--csv", tmp_path / "s.csv")
+    assert rc == 0 and out.count("PASS") == len(SWEEP_GRID_2048), out[-3000:]
+    rows = [l.split(",") for l in open(tmp_path / "s.csv").read().strip().splitlines()]
+    assert len(rows) == len(SWEEP_GRID_2048)
+    for i, (M, K, N, sp) in enumerate(SWEEP_GRID_2048):
+        meta, err = verify_dump(oracle, str(dumps / f"case_{i:03d}"))
+        assert (meta["M"], meta["K"], meta["N"]) == (M, K, N)
+        assert err <= 1e-4, (app, i, err)
+        row = [float(x) for x in rows[i]]
+        density = meta["nnz"] / (M * K)
+        assert abs(density - sp) < 0.01
+        if app == "spmm_run":    # M,N,K,SP,gflops,max_rel_diff
+            assert len(row) == 6 and row[:3] == [M, N, K] and abs(row[3] - density) < 1e-5 and row[4] > 0 and 0 <= row[5] < 1e-3
+        elif app == "sddmm_run":  # M,K,N,SP,gflops,calc_bw,max_diff
+            assert len(row) == 7 and row[:3] == [M, K, N] and abs(row[3] - density) < 1e-5 and row[4] > 0 and row[5] > 0 and 0 <= row[6] < 1e-3
+        else:                     # M,K,N,SP,gflops,max_diff (FUSED/fused-esimd_cb.cpp prints these; it writes no CSV)
+            assert len(row) == 6 and row[:3] == [M, K, N] and abs(row[3] - density) < 1e-5 and row[4] > 0 and 0 <= row[5] < 1e-3
+
+
+@pytest.mark.gpu
+def test_vendor_comparator_against_the_oracle(oracle, dl, tmp_path):
+    """bin/vendor_compare (rocSPARSE in the role of the reference's cuSPARSE harness, CUSPARSE/spmm_fromfile.cu:175-234,
+    CUSPARSE/sddmm_fromfile.cu:200-224) on all five configurations: exit status 0, every rel.diff <= 1e-4, and BOTH
+    results -- the library's and rocSPARSE's -- within 1e-4 of the CPU oracle on the same seeded inputs."""
+    exe = os.path.join(BIN, "vendor_compare")
+    assert os.path.exists(exe), f"{exe} is missing: run `make -C dlspm-esimd_amd drivers`"
+    p = subprocess.run([exe, "--iters", "5", "--dump", str(tmp_path)], capture_output=True, text=True, timeout=300)
+    out = p.stdout + p.stderr
+    print(out)
+    assert p.returncode == 0 and "vendor_compare PASS" in out
+    diffs = [float(l.split()[4]) for l in out.splitlines() if l.startswith("cfg") and "(best rocSPARSE algorithm" in l]
+    assert len(diffs) == 5 and all(0 <= x <= 1e-4 for x in diffs), diffs
+    for cfg in range(1, 6):
+        c = dl.make_config(cfg)
+        if c["op"] == dl.OP_SPMM:
+            ref = oracle.spmm(c["row_offsets"], c["col_indices"], c["values"], c["d0"], omp=True)
+        elif c["op"] == dl.OP_SDDMM:
+            ref = oracle.sddmm(c["row_offsets"], c["col_indices"], c["d0"], c["d1"], omp=True)
+        else:
+            ref = oracle.fused(c["row_offsets"], c["col_indices"], c["d0"], c["d1"], c["d2"], c["scale"], omp=True)
+        for side in ("dlspm", "rocsparse"):
+            got = np.fromfile(tmp_path / f"cfg{cfg}_{side}.f32", dtype=np.float32).reshape(ref.shape)
+            assert oracle.rel_frobenius(got, ref) <= 1e-4, (cfg, side)
+    # a tolerance nothing can meet: the comparator must fail with status 2, not report success
+    p = subprocess.run([exe, "--cfg", "1", "--iters", "2", "--tol", "0"], capture_output=True, text=True, timeout=300)
+    assert p.returncode == 2 and "vendor_compare FAIL" in p.stdout
+
+
 DLMC = os.path.join(ROOT, "tests", "golden", "dlmc")
 DLMC_CASES = [  # file, un-padded batch size of that layer (dlmc/rn50_batchsizes.txt)
     ("rn50_emp0.96_bottleneck_3_block_group_projection_block_group1.smtx", 3136),
@@ -198,6 +276,83 @@ def test_dlmc_batch_list(tmp_path):
         rc, out = run(app, "--batch", tmp_path / "rn50.txt", "--csv", tmp_path / f"{app}.csv", "--iters", 5)
         assert rc == 0 and out.count("PASS") == 3, out
         assert len(open(tmp_path / f"{app}.csv").read().strip().splitlines()) == 3
+
+
+MORE_DLMC = [  # file, dense width: the layer's un-padded batch size (rn50) or a width of our choosing (transformer)
+    ("rn50_mp0.5_bottleneck_1_block_group_projection_block_group1.smtx", 3136),
+    ("rn50_mp0.8_bottleneck_3_block_group1_1_1.smtx", 3136),
+    ("rn50_rp0.9_bottleneck_3_block_group1_2_1.smtx", 49),
+    ("rn50_vd0.8_initial_conv.smtx", 12544),
+    ("rn50_vd0.95_bottleneck_1_block_group1_1_1.smtx", 196),
+    ("transformer_l0r0.98_body_encoder_layer_4_self_attention_multihead_attention_q.smtx", 64),
+    ("transformer_l0r0.9_body_encoder_layer_1_self_attention_multihead_attention_q.smtx", 128),
+    ("transformer_mp0.98_body_encoder_layer_0_self_attention_multihead_attention_q_fully_connected.smtx", 256),
+    ("transformer_mp0.9_body_decoder_layer_0_ffn_conv1_fully_connected.smtx", 256),
+    ("transformer_rp0.98_body_decoder_layer_4_self_attention_multihead_attention_v_fully_connected.smtx", 100),
+    ("transformer_vd0.95_body_encoder_layer_1_self_attention_multihead_attention_v.smtx", 33),
+    ("transformer_vd0.98_body_encoder_layer_5_self_attention_multihead_attention_k.smtx", 128),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("app", ["spmm_run", "sddmm_run", "fused_run"])
+def test_more_dlmc_patterns_through_batch_runs_against_the_oracle(oracle, tmp_path, app):
+    """Twelve more real patterns (ResNet-50 and transformer; magnitude, random, variational-dropout and l0 pruning;
+    50-98 % sparse; one file without a single nonzero) as one --batch run per driver, every case dumped and verified
+    against the CPU oracle. SDDMM and the fused op take the width as the feature dimension, capped at 256."""
+    cap = (lambda w: w) if app == "spmm_run" else (lambda w: min(w, 256))
+    (tmp_path / "list.txt").write_text("".join(f"{os.path.join(DLMC, n)} {cap(w)}\n" for n, w in MORE_DLMC))
+    dumps = tmp_path / "dumps"
+    rc, out = run(app, "--batch", tmp_path / "list.txt", "--iters", 3, "--warmup", 1, "--dump-each", dumps)
+    assert rc == 0 and out.count("PASS") == len(MORE_DLMC), out[-3000:]
+    for i, (name, w) in enumerate(MORE_DLMC):
+        M, K, ro, ci = read_smtx(os.path.join(DLMC, name))
+        meta, err = verify_dump(oracle, str(dumps / f"case_{i:03d}"))
+        assert (meta["M"], meta["K"], meta["N"], meta["nnz"]) == (M, K, cap(w), ci.size)
+        assert np.array_equal(np.fromfile(dumps / f"case_{i:03d}" / "col_indices.i32", dtype=np.int32), ci)
+        assert err <= 1e-4, (app, name, err)
+
+
+@pytest.mark.gpu
+def test_batch_run_dlmc_script(oracle, tmp_path):
+    """host/batch-run-dlmc, the reference's shell loop over a DLMC directory (SPMM/batch-run-spmm_fromfile:16-46):
+    layer names looked up in a '<layer>,<batch size>' table, files that the table does not name skipped, one CSV row
+    per file; and the fixed-width form. Outputs verified against the oracle through --dump-each."""
+    import shutil
+
+    tree = tmp_path / "dlmc" / "rn50" / "magnitude_pruning" / "0.8"
+    tree.mkdir(parents=True)
+    layers = {  # layer name in the tree -> (fixture, batch size from the table)
+        "bottleneck_3_block_group1_1_1": ("rn50_mp0.8_bottleneck_3_block_group1_1_1.smtx", 3136),
+        "bottleneck_1_block_group_projection_block_group1": ("rn50_mp0.5_bottleneck_1_block_group_projection_block_group1.smtx", 3136),
+        "bottleneck_3_block_group3_5_1": ("rn50_emp0.98_bottleneck_3_block_group3_5_1.smtx", 196),
+    }
+    for layer, (fixture, _) in layers.items():
+        shutil.copy(os.path.join(DLMC, fixture), tree / f"{layer}.smtx")
+    shutil.copy(os.path.join(DLMC, "rn50_vd0.8_initial_conv.smtx"), tree / "not_in_the_table.smtx")
+    table = tmp_path / "batchsizes.txt"
+    table.write_text("".join(f"{layer},{n}\n" for layer, (_, n) in layers.items()))
+    script = os.path.join(ROOT, "dlspm-esimd_amd", "host", "batch-run-dlmc")
+    dumps = tmp_path / "dumps"
+    p = subprocess.run(["bash", script, "spmm_run", str(tmp_path / "dlmc"), str(table), str(tmp_path / "out.csv"),
+                        "--iters", "3", "--dump-each", str(dumps)], capture_output=True, text=True, timeout=300)
+    out = p.stdout + p.stderr
+    assert p.returncode == 0 and "3 files" in out and out.count("PASS") == 3 and "not_in_the_table" not in out, out[-3000:]
+    rows = [l.split(",") for l in open(tmp_path / "out.csv").read().strip().splitlines()]
+    assert len(rows) == 3 and all(len(r) == 7 for r in rows)  # M,N,K,SP,gflops,max_diff,opcount
+    widths = sorted(int(r[1]) for r in rows)
+    assert widths == [196, 3136, 3136]
+    for i in range(3):
+        _, err = verify_dump(oracle, str(dumps / f"case_{i:03d}"))
+        assert err <= 1e-4
+    # fixed width instead of a table: every file below the directory, the fourth one included
+    p = subprocess.run(["bash", script, "sddmm_run", str(tmp_path / "dlmc"), "64", str(tmp_path / "out2.csv"), "--iters", "3"],
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0 and "4 files" in p.stderr and p.stdout.count("PASS") == 4, p.stdout[-3000:]
+    assert len(open(tmp_path / "out2.csv").read().strip().splitlines()) == 4
+    # too few arguments: usage and status 2, nothing run
+    p = subprocess.run(["bash", script, "spmm_run"], capture_output=True, text=True, timeout=60)
+    assert p.returncode == 2 and "batch-run-dlmc <spmm_run|sddmm_run|fused_run>" in p.stdout
 
 
 @pytest.mark.gpu
