@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
 #include <vector>
 #include <cstring>
 
@@ -283,6 +284,56 @@ int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int
         e = spmm_launch(args, shape, static_cast<hipStream_t>(stream));
     }
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+}
+
+// ---- the entry point that allocates nothing --------------------------------------------------------------------
+// Scratch memory of spmm_csr_f32_static: one array per GPU, part of the loaded code object, held until the process ends.
+// `scratch` is the host-side handle of that array, not a device address: the address on the current device comes
+// from hipGetSymbolAddress, once per device, and only that address is ever handed to a kernel.
+constexpr size_t kStaticScratchBytes = (size_t)8 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// address of `scratch` on the current device (looked up at the first call on that device), or nullptr with `e` set
+void* static_scratch(hipError_t& e)
+{
+    int dev = -1;
+    e = hipGetDevice(&dev);
+    if (e != hipSuccess) return nullptr;
+    if (dev < 0 || dev >= kMaxDevices) {
+        e = hipErrorInvalidDevice;
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return nullptr;
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+size_t dlspm_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int spmm_csr_f32_static(int M, int K, int N, int nnz, const int* row_offsets, const int* col_indices, const float* values,
+                        const float* B, float* C, void* stream)
+{
+    if (M < 0 || K < 0 || N < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
+    if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
+    const size_t need = dlspm_workspace_bytes(DLSPM_OP_SPMM, M, K, N, nnz);
+    if (need > kStaticScratchBytes) return DLSPM_E_STATIC_LIMIT;
+    if (need == 0)  // the schedule of these sizes keeps everything in registers and LDS
+        return spmm_csr_f32(M, K, N, nnz, row_offsets, col_indices, values, B, C, nullptr, 0, stream);
+    hipError_t e = hipSuccess;
+    void* ptr = static_scratch(e);
+    if (!ptr) return fail_hip(e);
+    return spmm_csr_f32(M, K, N, nnz, row_offsets, col_indices, values, B, C, ptr, kStaticScratchBytes, stream);
 }
 
 size_t dlspm_row_plan_bytes(int M) { return M > 0 ? (size_t)3 * (size_t)M * sizeof(int) : 0; }
@@ -650,6 +701,7 @@ const char* dlspm_status_string(int status)
         case DLSPM_E_LAUNCH: return "HIP runtime error at launch (see dlspm_last_hip_error)";
         case DLSPM_E_INVALID_CSR: return "malformed CSR structure";
         case DLSPM_E_NO_DEVICE: return "no gfx950 device is current";
+        case DLSPM_E_STATIC_LIMIT: return "the problem needs more scratch memory than spmm_csr_f32_static holds (dlspm_static_scratch_bytes)";
         default: return "unknown status";
     }
 }

@@ -18,6 +18,7 @@ E_WORKSPACE = -2
 E_LAUNCH = -3
 E_INVALID_CSR = -4
 E_NO_DEVICE = -5
+E_STATIC_LIMIT = -6
 
 OP_SPMM, OP_SDDMM, OP_FUSED = 0, 1, 2
 
@@ -49,6 +50,8 @@ EXPORTS = (
     "spmm_csr_f32_planned",
     "sddmm_csr_f32_planned",
     "fused_sddmm_spmm_f32_planned",
+    "spmm_csr_f32_static",
+    "dlspm_static_scratch_bytes",
     "dlspm_status_string",
     "dlspm_last_hip_error",
     "dlspm_version",
@@ -104,6 +107,9 @@ def lib() -> ctypes.CDLL:
         L.sddmm_csr_f32_planned.restype = ci
         L.fused_sddmm_spmm_f32_planned.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, cf, vp, vp, sz, vp]
         L.fused_sddmm_spmm_f32_planned.restype = ci
+        L.spmm_csr_f32_static.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, vp]
+        L.spmm_csr_f32_static.restype = ci
+        L.dlspm_static_scratch_bytes.restype = sz
         L.dlspm_status_string.argtypes = [ci]
         L.dlspm_status_string.restype = ctypes.c_char_p
         L.dlspm_last_hip_error.restype = ci
@@ -187,6 +193,30 @@ def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None, 
                             _ptr(B, torch.float32, "B"), _ptr(out, torch.float32, "C"), wp, wb, _stream())
     if st != OK:
         raise DlspmError(st, "spmm_csr_f32")
+    return out
+
+
+def static_scratch_bytes() -> int:
+    """Size of the library-held scratch array that spmm_static() works in (per GPU)."""
+    return int(lib().dlspm_static_scratch_bytes())
+
+
+def spmm_static(row_offsets, col_indices, values, B, K=None, out=None):
+    """spmm() through spmm_csr_f32_static: the schedule of a call with workspace, in the library's own static scratch
+    array; allocates nothing inside the library. `out` must be given by callers that may not allocate either."""
+    import torch
+
+    M = row_offsets.numel() - 1
+    nnz = col_indices.numel()
+    Kd, N = B.shape
+    K = Kd if K is None else K
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=B.device)
+    st = lib().spmm_csr_f32_static(M, K, N, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
+                                   _ptr(col_indices, torch.int32, "col_indices"), _ptr(values, torch.float32, "values"),
+                                   _ptr(B, torch.float32, "B"), _ptr(out, torch.float32, "C"), _stream())
+    if st != OK:
+        raise DlspmError(st, "spmm_csr_f32_static")
     return out
 
 

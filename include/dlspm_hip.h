@@ -65,6 +65,7 @@ extern "C" {
 #define DLSPM_E_LAUNCH       (-3) /* the HIP runtime refused the launch (see dlspm_last_hip_error)         */
 #define DLSPM_E_INVALID_CSR  (-4) /* dlspm_csr_check found a malformed CSR structure                        */
 #define DLSPM_E_NO_DEVICE    (-5) /* no gfx950 device is current                                            */
+#define DLSPM_E_STATIC_LIMIT (-6) /* spmm_csr_f32_static: the sizes need more scratch than the library holds   */
 
 /* `workspace` value that carries the caller's knowledge "row lengths are even" instead of memory (see above) */
 #define DLSPM_ROWS_EVEN ((void*)1)
@@ -115,6 +116,25 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz,
                          const float* Q, const float* Kmat, const float* V, float scale,
                          float* O,
                          void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * spmm_csr_f32 for callers that cannot allocate device memory and cannot size a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference (whose drivers
+ * allocate everything up front in main()). It runs exactly what spmm_csr_f32 runs when it is handed
+ * dlspm_workspace_bytes() bytes of workspace -- the flat schedule for matrices of half a million nonzeros and more, the
+ * column-sliced schedule for a B beyond one L2, the row-block schedule otherwise -- and returns the same bits, but the
+ * partial rows and slice boundaries live in a buffer that is part of the library itself: a static device array of
+ * dlspm_static_scratch_bytes() = 8 MiB per GPU, held from the moment the library is loaded until the process ends.
+ * The call allocates nothing, frees nothing and never synchronises (its first call on each device looks the array's
+ * address up once). Sizes whose schedule needs more than that are refused with DLSPM_E_STATIC_LIMIT and nothing is
+ * launched (call spmm_csr_f32 with NULL or with a workspace of your own then). Every call on one GPU shares that GPU's
+ * array: calls that overlap in time on one GPU (two streams, two threads) race on it and must be ordered by the caller.
+ * Nothing in the array needs to start at zero: every partial row that is read was written by the same call.
+ */
+int spmm_csr_f32_static(int M, int K, int N, int nnz,
+                        const int* row_offsets, const int* col_indices, const float* values,
+                        const float* B, float* C, void* stream);
+size_t dlspm_static_scratch_bytes(void);
 
 /*
  * Bytes of device workspace the op can use for these sizes (0 = none, as for small or short-row problems;
