@@ -25,17 +25,99 @@ static int fail_hip(hipError_t e)
 }
 
 
-// Optional launch-shape override for tuning sweeps: DLSPM_SPLIT="W,R", read at every call.
-static bool split_override(int& W, int& R)
+// ---- tuning overrides ------------------------------------------------------------------------------------------------
+// One set per host thread (dlspm_set_tuning). A thread that never called it uses the process default, which is read
+// from the environment exactly once: DLSPM_SPLIT="W,R", DLSPM_FLAT=0|1, DLSPM_FLAT_CHUNK=n, DLSPM_SLICES=0|n,
+// DLSPM_TILE_MAJOR=0|1, DLSPM_TILE_WIDTH=512|..|32, DLSPM_PLAN_ORDER=0|1|2 (so that the drivers can be swept from a
+// shell without a rebuild). No launch path reads the environment.
+static Tuning tuning_from_environment()
 {
-    const char* e = std::getenv("DLSPM_SPLIT");
-    int w = 0, r = 0;
-    if (e && std::sscanf(e, "%d,%d", &w, &r) == 2) {
-        W = w;
-        R = r;
-        return true;
+    Tuning t;
+    auto env = [](const char* name) { return std::getenv(name); };
+    if (const char* e = env("DLSPM_SPLIT")) {
+        int w = 0, r = 0;
+        if (std::sscanf(e, "%d,%d", &w, &r) == 2) {
+            t.split_w = w;
+            t.split_r = r;
+        }
     }
-    return false;
+    auto number = [&](const char* name, int& field) {
+        if (const char* e = env(name)) field = std::atoi(e);
+    };
+    number("DLSPM_FLAT", t.flat);
+    number("DLSPM_FLAT_CHUNK", t.flat_chunk);
+    number("DLSPM_SLICES", t.slices);
+    number("DLSPM_TILE_MAJOR", t.tile_major);
+    number("DLSPM_TILE_WIDTH", t.tile_width);
+    number("DLSPM_PLAN_ORDER", t.plan_order);
+    return t;
+}
+static const Tuning& process_tuning()
+{
+    static const Tuning t = tuning_from_environment();
+    return t;
+}
+static thread_local bool t_tuning_set = false;
+static thread_local Tuning t_tuning;
+const Tuning& tuning() { return t_tuning_set ? t_tuning : process_tuning(); }
+
+// ---- the current device ----------------------------------------------------------------------------------------------
+constexpr int kMaxDevices = 64;
+static const DeviceInfo kNoDevice{256, 4ll << 20, false, false};
+const DeviceInfo& device_info()
+{
+    static std::mutex mutex;
+    static DeviceInfo cache[kMaxDevices];
+    static bool known[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();  // a machine without a device is not an error of the caller's next HIP call
+        return kNoDevice;
+    }
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!known[dev]) {
+        DeviceInfo d = kNoDevice;
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) == hipSuccess) {
+            d.present = true;
+            d.gfx950 = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+            if (prop.multiProcessorCount > 0) d.cus = prop.multiProcessorCount;
+            // the size of ONE L2 (each XCD has its own); a figure outside 1 ... 64 MiB is not believed
+            if (prop.l2CacheSize >= (1 << 20) && prop.l2CacheSize <= (64 << 20)) d.l2_bytes = prop.l2CacheSize;
+        } else {
+            (void)hipGetLastError();
+        }
+        cache[dev] = d;
+        known[dev] = true;
+    }
+    return cache[dev];
+}
+// DLSPM_OK if the current device can run the kernels
+static int require_device()
+{
+    const DeviceInfo& d = device_info();
+    return d.present && d.gfx950 ? DLSPM_OK : DLSPM_E_NO_DEVICE;
+}
+
+// What the caller passed as (workspace, workspace_bytes): device memory, and the hints in the upper bits of the size.
+struct WorkspaceArg {
+    void* mem;
+    size_t bytes;
+    bool rows_even;
+    bool row_plan;
+};
+static WorkspaceArg workspace_arg(void* workspace, size_t workspace_bytes)
+{
+    WorkspaceArg a{};
+    a.rows_even = (workspace_bytes & DLSPM_HINT_ROWS_EVEN) != 0 || workspace == DLSPM_ROWS_EVEN;
+    a.row_plan = (workspace_bytes & DLSPM_HINT_ROW_PLAN) != 0;
+    a.bytes = workspace_bytes & ~DLSPM_HINT_MASK;
+    a.mem = workspace == DLSPM_ROWS_EVEN ? nullptr : workspace;
+    if (!a.mem || a.bytes == 0) {
+        a.mem = nullptr;
+        a.bytes = 0;
+    }
+    return a;
 }
 
 // Flat schedule (every wave owns a fixed number of consecutive nonzeros; partial rows in the caller's workspace):
@@ -45,11 +127,11 @@ static bool split_override(int& W, int& R)
 // slower on even row lengths (most below 2 M nonzeros), 10-60 % faster on lognormal row lengths (sigma 1-2); below
 // these sizes it loses even there (short rows cost a wave one dependent memory round trip each). Passing the
 // workspace is therefore the caller's way of saying that the rows are uneven (dlspm_csr_row_stats tells).
-// DLSPM_FLAT=0/1 overrides the rule and DLSPM_FLAT_CHUNK the nonzeros per wave, for tuning sweeps and tests.
+// dlspm_tuning.flat = 0/1 overrides the rule and .flat_chunk the nonzeros per wave, for tuning sweeps and tests.
 constexpr int kFlatMinNnz = 1 << 19;
 constexpr int kFlatMinRow = 64;          // mean nonzeros per row
 constexpr int kFlatMinLanes = 32;        // lanes per dense row (widths above 64 floats)
-constexpr int kFlatTargetUnits = 32768;  // waves wanted at least: four rounds of 8 waves on each of 1024 SIMDs
+constexpr int kFlatUnitsPerCu = 128;     // waves wanted at least: four rounds of 8 waves on each of a compute unit's 4 SIMDs
 // SDDMM takes the flat schedule by this rule alone (it needs no workspace, so the caller has no say): only where it
 // was measured to be equal on even rows
 constexpr int kFlatMinNnzSddmm = 1 << 21;
@@ -59,17 +141,14 @@ FlatPlan flat_plan(int M, int nnz, int width, int G)
 {
     FlatPlan p{0, 0, 0};
     if (M <= 0 || nnz <= 0 || width <= 0) return p;
-    int force = -1;
-    if (const char* e = std::getenv("DLSPM_FLAT")) force = std::atoi(e);
+    const int force = tuning().flat;
     const bool by_rule = nnz >= kFlatMinNnz && (long long)nnz >= (long long)kFlatMinRow * M && G >= kFlatMinLanes;
     if (force == 0 || (force < 0 && !by_rule)) return p;
     long long chunk = nnz >= (1 << 21) ? 512 : 256;  // at least eight (four) passes of 64 nonzeros per wave
-    const long long even = ((long long)nnz + kFlatTargetUnits - 1) / kFlatTargetUnits;
+    const long long target_units = (long long)kFlatUnitsPerCu * device_info().cus;
+    const long long even = ceil_div(nnz, target_units);
     if (even > chunk) chunk = (even + 63) / 64 * 64;
-    if (const char* e = std::getenv("DLSPM_FLAT_CHUNK")) {
-        const int c = std::atoi(e);
-        if (c >= 64) chunk = c;
-    }
+    if (tuning().flat_chunk >= 64) chunk = tuning().flat_chunk;
     p.chunk = (int)chunk;
     p.units = (int)(((long long)nnz + chunk - 1) / chunk);
     p.bytes = (size_t)p.units * 2 * (size_t)width * sizeof(float);
@@ -78,8 +157,7 @@ FlatPlan flat_plan(int M, int nnz, int width, int G)
 
 static FlatPlan sddmm_flat_plan(int M, int nnz, int D)
 {
-    int force = -1;
-    if (const char* e = std::getenv("DLSPM_FLAT")) force = std::atoi(e);
+    const int force = tuning().flat;
     if (force < 0 && (nnz < kFlatMinNnzSddmm || (long long)nnz < (long long)kFlatMinRowSddmm * M)) return FlatPlan{0, 0, 0};
     return flat_plan(M, nnz, D, kWave);
 }
@@ -93,43 +171,43 @@ static FlatPlan sddmm_flat_plan(int M, int nnz, int D)
 // the geometric mean of 24 cases (0.88 ... 1.09; most on a tall B under wide dense rows); SDDMM has no partial rows and
 // gains nothing from larger slices (0.92 ... 1.04, mean 1.00). Operands of
 // exactly 4 MiB (8192 x 128 floats) gain 13-16 % at 10-30 % density and lose 5 % at 3 %: sliced in two for long rows
-// only. Like the flat schedule only from half a million nonzeros on (two more launches). DLSPM_SLICES=0 switches it
-// off, DLSPM_SLICES=n forces n slices (tuning, tests).
-constexpr long long kSliceMinOperand = 4ll << 20;  // bytes gathered from; above this the operand is sliced
-constexpr long long kSlicesPer8MiB = 4;            // slices of 2 MiB of it: half the L2 each
-constexpr long long kSlicesPer8MiBPartial = 3;     // ... of 8/3 MiB where every slice costs a partial row per row
+// only. Like the flat schedule only from half a million nonzeros on (two more launches). dlspm_tuning.slices = 0
+// switches it off, = n forces n slices (tuning, tests). The 4 MiB are the device's own figure for one L2
+// (DeviceInfo::l2_bytes): an operand above it is sliced, in slices of half of it (two thirds with partial rows).
+constexpr long long kSlicesPer2L2 = 4;             // slices of half an L2 of operand each
+constexpr long long kSlicesPer2L2Partial = 3;      // ... of two thirds of an L2 where every slice costs a partial row per row
 constexpr int kSliceMaxSlices = 16;
 constexpr int kSliceMinRow = 16;  // least mean nonzeros of a row inside one slice; fewer slices rather than shorter shares
-constexpr int kSliceMinRowAtL2 = 256;  // the same for an operand of exactly kSliceMinOperand bytes
+constexpr int kSliceMinRowAtL2 = 256;  // the same for an operand that just fills one L2
 
 SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial_width, int G, bool partial_rows,
-                     int slots, int min_blocks)
+                     int slots, int blocks_per_cu)
 {
     SlicePlan p{0, 1, 0, 0};
     if (M <= 0 || K <= 0 || nnz <= 0 || width <= 0 || G <= 0) return p;  // G == 0: no sliced kernel for this layout
-    int force = -1;
-    if (const char* e = std::getenv("DLSPM_SLICES")) force = std::atoi(e);
+    const int force = tuning().slices;
+    const long long l2 = device_info().l2_bytes;
     const long long bytes = (long long)K * width * (long long)sizeof(float) * operands;
-    long long slices = (bytes * (partial_rows ? kSlicesPer8MiBPartial : kSlicesPer8MiB) + (8ll << 20) - 1) / (8ll << 20);
+    long long slices = ceil_div(bytes * (partial_rows ? kSlicesPer2L2Partial : kSlicesPer2L2), 2 * l2);
     if (slices > kSliceMaxSlices) slices = kSliceMaxSlices;
     // Slices that leave a row its minimum share: 16 nonzeros per slice for dense rows of 256 floats and more, in
     // inverse proportion more for narrower ones (measured with D = 64: 28 per slice lost 20 %, 48 and more gained; with
     // D = 32: 48 lost, 164 gained). An operand that just fills the L2 is worth slicing for long rows only, and only
     // for dense rows of at least 128 floats (narrower: 327 nonzeros per slice still lost 10 %).
-    const bool just_fills = bytes <= kSliceMinOperand;
+    const bool just_fills = bytes <= l2;
     const int per_width = 4096 / width;
     const int min_row = just_fills ? kSliceMinRowAtL2 : per_width > kSliceMinRow ? per_width : kSliceMinRow;
     if (just_fills && width < 128) slices = 0;
     const long long fit = (long long)nnz / ((long long)min_row * M);
     if (slices > fit) slices = fit;
-    const bool by_rule = bytes >= kSliceMinOperand && nnz >= kSlicedMinNnz && slices >= 2;
+    const bool by_rule = bytes >= l2 && nnz >= kSlicedMinNnz && slices >= 2;
     if (force == 0 || force == 1 || (force < 0 && !by_rule)) return p;
     if (force >= 2) slices = force < kSliceMaxSlices ? force : kSliceMaxSlices;
     if (slices > K) slices = K;
     if (slices < 2) return p;
     p.slices = (int)slices;
     int W = 4;
-    choose_split(M, 1, (int)(nnz / slices), SplitRule{min_blocks, 4, slots, false}, false, W, p.R);
+    choose_split(M, 1, (int)(nnz / slices), SplitRule{blocks_per_cu, 4, slots, false}, false, W, p.R);
     if (W != 4) p.R = 1;  // only four-wave workgroups are built for this schedule
     p.bounds_bytes = (((size_t)(slices + 1) * M * sizeof(int)) + 255) / 256 * 256;
     p.bytes = p.bounds_bytes + (size_t)slices * M * (size_t)partial_width * sizeof(float);
@@ -139,32 +217,37 @@ SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial
 void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bool rows_even, int& W, int& R)
 {
     static const int kPairs[][2] = {{4, 16}, {4, 8}, {4, 4}, {4, 2}, {4, 1}, {8, 4}, {8, 2}, {8, 1}, {16, 1}};
-    if (split_override(W, R)) {
+    if (tuning().split_w > 0) {
         for (const auto& pr : kPairs)
-            if (pr[0] == W && pr[1] == R && W <= rule.max_w) return;
+            if (pr[0] == tuning().split_w && pr[1] == tuning().split_r && pr[0] <= rule.max_w) {
+                W = pr[0];
+                R = pr[1];
+                return;
+            }
     }
+    const long long cus = device_info().cus;  // the thresholds below were measured on 256 compute units and scale with them
     // Measured on MI355X over the benchmark configurations and the 12 x {32,128} x {0.3,0.2,0.1} sweep grid:
     // four-wave workgroups win whenever the matrix has enough rows to fill the device (16-wave workgroups were up
     // to 2x slower on long rows: their barrier makes every wave wait for the slowest of sixteen), and rows are
-    // grouped only as far as the grid keeps `min_blocks` workgroups and a workgroup stays below ~512 nonzeros.
+    // grouped only as far as the grid keeps `blocks_per_cu` workgroups per compute unit and a workgroup stays below ~512 nonzeros.
     const double avg = M > 0 ? (double)nnz / M : 0.0;
     const long long work_rows = (long long)M * col_tiles;
-    W = work_rows >= 512 ? 4 : work_rows >= 256 ? 8 : 16;
+    W = work_rows >= 2 * cus ? 4 : work_rows >= cus ? 8 : 16;
     // very long rows in a tall matrix: sixteen waves per row gain 5-8 % in SpMM (24576 and 32768 rows of ~2000
     // nonzeros); with 8192 rows they lose as much, and the fused kernel loses 25-50 % with them at any height
-    if (rule.w16_long_rows && avg >= 1536.0 && work_rows >= 16384) W = 16;
+    if (rule.w16_long_rows && avg >= 1536.0 && work_rows >= 64 * cus) W = 16;
     // few rows, each long (pruned ResNet-50 layers at small batch): four waves per row leave the device with a
     // couple of waves per SIMD, each walking hundreds of steps in sequence (measured 15-25 % slower); a step
     // takes `slots` nonzeros of the row at once
     const double steps = avg / (rule.slots > 0 ? rule.slots : 1);
-    if (work_rows < 1024 && steps >= 768.0) W = 16;
-    else if (work_rows < 1024 && steps >= 384.0 && W < 8) W = 8;
+    if (work_rows < 4 * cus && steps >= 768.0) W = 16;
+    else if (work_rows < 4 * cus && steps >= 384.0 && W < 8) W = 8;
     if (W > rule.max_w) W = rule.max_w;
     R = 1;
     if (W == 4) {
         for (int r = 2; r <= 16; r *= 2) {
-            const long long blocks = (long long)((M + r - 1) / r) * col_tiles;
-            if (blocks < rule.min_blocks || avg * r > 512.0) break;
+            const long long blocks = ceil_div(M, r) * col_tiles;
+            if (blocks < rule.blocks_per_cu * cus || avg * r > 512.0) break;
             R = r;
         }
         // Rows known to be even: four rows per four-wave workgroup, which the kernels then run as one whole row per
@@ -174,7 +257,7 @@ void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bo
         // uneven rows the same grouping is 5-20 % slower (four rows of work per workgroup make the tail of the
         // launch coarser), hence only on the caller's word. Rows below 128 nonzeros keep the grouping of the size rule
         // (4096 rows of ~100: four per workgroup measured 6 % slower than two).
-        if (rows_even && R < 4 && avg >= 128.0 && (long long)((M + 3) / 4) * col_tiles >= 512) R = 4;
+        if (rows_even && R < 4 && avg >= 128.0 && ceil_div(M, 4) * col_tiles >= 2 * cus) R = 4;
     }
 }
 
@@ -182,7 +265,8 @@ void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bo
 __global__ void row_stats_kernel(int M, const int* __restrict__ row_offsets, int* __restrict__ stats)
 {
     int longest = 0, empty = 0;
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < M; i += gridDim.x * blockDim.x) {
+    const long long stride = (long long)gridDim.x * blockDim.x;  // 64-bit: i + stride must not wrap for M near INT_MAX
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < M; i += stride) {
         const int len = row_offsets[i + 1] - row_offsets[i];
         longest = max(longest, len);
         empty += len == 0 ? 1 : 0;
@@ -204,20 +288,20 @@ __global__ void fill_zero_kernel(float* __restrict__ out, int n)
 __global__ void csr_check_kernel(int M, int K, int nnz, const int* __restrict__ row_offsets,
                                  const int* __restrict__ col_indices, int* __restrict__ flags)
 {
-    const int tid = blockIdx.x * blockDim.x + threadIdx.x;
-    const int stride = gridDim.x * blockDim.x;
+    const long long tid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long stride = (long long)gridDim.x * blockDim.x;  // 64-bit: i + stride must not wrap near INT_MAX
     int f = 0;
     if (tid == 0) {
         if (row_offsets[M] != nnz) f |= 2;
         if (row_offsets[0] != 0) f |= 32;
     }
-    for (int i = tid; i < M; i += stride) {
+    for (long long i = tid; i < M; i += stride) {
         const int lo = row_offsets[i], hi = row_offsets[i + 1];
         if (hi < lo) f |= 4;
         if (hi - lo > K) f |= 8;
     }
     if (!(f & 2)) {
-        for (int i = tid; i < nnz; i += stride) {
+        for (long long i = tid; i < nnz; i += stride) {
             const int c = col_indices[i];
             if (c >= K) f |= 16;
             if (c < 0) f |= 64;
@@ -234,7 +318,7 @@ static SlicePlan spmm_slice_plan(int M, int K, int N, int nnz, const SpmmShape& 
     // and the workgroups of one (slice, tile) pair should fill the device by themselves, or it gathers from several
     // slabs at once: rows per workgroup as if there were one tile (4096 x 65536, N = 3136, 25 tiles of 128, 131 or
     // 656 nonzeros per row: 856 -> 716 us and 2320 -> 2133 us)
-    SlicePlan p = slice_plan(M, K, N < tw ? N : tw, nnz, 1, 0, s.vec == 4 ? s.G : 0, true, kWave / s.G, 2048);
+    SlicePlan p = slice_plan(M, K, N < tw ? N : tw, nnz, 1, 0, s.vec == 4 ? s.G : 0, true, kWave / s.G, 8);
     p.bytes = p.slices > 0 ? p.bounds_bytes + (size_t)p.slices * M * (size_t)N * sizeof(float) : 0;
     return p;
 }
@@ -242,12 +326,12 @@ static SlicePlan fused_slice_plan(int M, int K, int D, int nnz, const FusedShape
 {
     const int tw = s.G * s.vec * s.V;
     const bool built = s.vec == 4 && s.G1 == 8 && s.DS > 0 && tw >= D;  // the widths the sliced kernels are built for (17 .. 512)
-    return slice_plan(M, K, D, nnz, 2, D, built ? s.G : 0, true, kWave / s.G, 512);
+    return slice_plan(M, K, D, nnz, 2, D, built ? s.G : 0, true, kWave / s.G, 2);
 }
 static SlicePlan sddmm_slice_plan(int M, int K, int D, int nnz, const SddmmShape& s)
 {
     const bool built = s.vec == 4 && s.G1 == 8 && s.DS >= 1;  // 16 < D <= 512
-    return slice_plan(M, K, D, nnz, 1, 0, built ? kWave : 0, false, kWave / s.G1, 512);
+    return slice_plan(M, K, D, nnz, 1, 0, built ? kWave : 0, false, kWave / s.G1, 2);
 }
 
 }  // namespace dlspm
@@ -256,32 +340,87 @@ using namespace dlspm;
 
 extern "C" {
 
+void dlspm_tuning_default(dlspm_tuning* t)
+{
+    if (!t) return;
+    const Tuning d;
+    *t = dlspm_tuning{d.split_w, d.split_r, d.flat, d.flat_chunk, d.slices, d.tile_major, d.tile_width, d.plan_order};
+}
+
+int dlspm_set_tuning(const dlspm_tuning* t)
+{
+    if (!t) {  // back to the process default
+        t_tuning_set = false;
+        return DLSPM_OK;
+    }
+    if (t->split_w < 0 || t->split_r < 0 || t->flat < -1 || t->flat > 1 || t->flat_chunk < 0 || t->slices < -1 ||
+        t->tile_major < -1 || t->tile_major > 1 || t->tile_width < 0 || t->plan_order < 0 || t->plan_order > 2)
+        return DLSPM_E_INVALID_ARG;
+    t_tuning.split_w = t->split_w;
+    t_tuning.split_r = t->split_r;
+    t_tuning.flat = t->flat;
+    t_tuning.flat_chunk = t->flat_chunk;
+    t_tuning.slices = t->slices;
+    t_tuning.tile_major = t->tile_major;
+    t_tuning.tile_width = t->tile_width;
+    t_tuning.plan_order = t->plan_order;
+    t_tuning_set = true;
+    return DLSPM_OK;
+}
+
+int dlspm_get_tuning(dlspm_tuning* t)
+{
+    if (!t) return DLSPM_E_INVALID_ARG;
+    const Tuning& c = tuning();
+    *t = dlspm_tuning{c.split_w, c.split_r, c.flat, c.flat_chunk, c.slices, c.tile_major, c.tile_width, c.plan_order};
+    return DLSPM_OK;
+}
+
+int dlspm_device_info(int* compute_units, long long* l2_bytes, int* is_gfx950)
+{
+    const DeviceInfo& d = device_info();
+    if (compute_units) *compute_units = d.cus;
+    if (l2_bytes) *l2_bytes = d.l2_bytes;
+    if (is_gfx950) *is_gfx950 = d.present && d.gfx950 ? 1 : 0;
+    return d.present ? DLSPM_OK : DLSPM_E_NO_DEVICE;
+}
+
 int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int* col_indices, const float* values,
                  const float* B, float* C, void* workspace, size_t workspace_bytes, void* stream)
 {
     if (M < 0 || K < 0 || N < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
+    const WorkspaceArg ws = workspace_arg(workspace, workspace_bytes);
+    if (ws.row_plan && ws.mem && ws.bytes < row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
     if (M == 0 || N == 0) return DLSPM_OK;
     if (!row_offsets || !C) return DLSPM_E_INVALID_ARG;
     if (nnz > 0 && (!col_indices || !values || !B)) return DLSPM_E_INVALID_ARG;
+    if (const int st = require_device()) return st;
     const bool vec4 = N >= 4;  // dwordx4 accesses need only dword alignment
     const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C};
-    const bool even = workspace == DLSPM_ROWS_EVEN;  // a constant that says something about the rows, not memory
-    const bool memory = !even && workspace != nullptr && workspace_bytes > 0;
-    const SpmmShape shape = spmm_choose(M, K, N, nnz, vec4, even, !memory);
+    hipStream_t st = static_cast<hipStream_t>(stream);
     hipError_t e;
+    if (ws.row_plan && ws.mem) {
+        // the memory holds the row plan of this matrix; sizes a planned launch is not built for run as with NULL
+        SpmmShape shape = spmm_choose(M, K, N, nnz, vec4, false, true);
+        e = spmm_plan_applies(shape, M, N, nnz) ? spmm_planned_launch(args, shape, static_cast<const int*>(ws.mem), st)
+                                                : spmm_launch(args, shape, st);
+        return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+    }
+    const bool memory = !ws.rows_even && ws.mem != nullptr;
+    const SpmmShape shape = spmm_choose(M, K, N, nnz, vec4, ws.rows_even, !memory);
     if (memory) {
         const SlicePlan sliced = spmm_slice_plan(M, K, N, nnz, shape);
         const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(M, nnz, N, shape.G);
-        if (workspace_bytes < (sliced.slices > 0 ? sliced.bytes : plan.bytes)) return DLSPM_E_WORKSPACE;
+        if (ws.bytes < (sliced.slices > 0 ? sliced.bytes : plan.bytes)) return DLSPM_E_WORKSPACE;
         if (sliced.slices > 0)
-            e = spmm_sliced_launch(args, shape, sliced, workspace, static_cast<hipStream_t>(stream));
+            e = spmm_sliced_launch(args, shape, sliced, ws.mem, st);
         else if (plan.chunk > 0)
-            e = spmm_flat_launch(args, shape, plan, static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
+            e = spmm_flat_launch(args, shape, plan, static_cast<float*>(ws.mem), st);
         else
-            e = spmm_launch(args, shape, static_cast<hipStream_t>(stream));
+            e = spmm_launch(args, shape, st);
     } else {
-        e = spmm_launch(args, shape, static_cast<hipStream_t>(stream));
+        e = spmm_launch(args, shape, st);
     }
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }
@@ -294,7 +433,6 @@ constexpr size_t kStaticScratchBytes = (size_t)8 << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace {
-constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 void* g_scratch_ptr[kMaxDevices] = {};
 
@@ -326,7 +464,7 @@ int spmm_csr_f32_static(int M, int K, int N, int nnz, const int* row_offsets, co
 {
     if (M < 0 || K < 0 || N < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
-    const size_t need = dlspm_workspace_bytes(DLSPM_OP_SPMM, M, K, N, nnz);
+    const size_t need = dlspm_workspace_bytes(DLSPM_OP_SPMM, M, K, N, nnz);  // of the flat or column-sliced schedule
     if (need > kStaticScratchBytes) return DLSPM_E_STATIC_LIMIT;
     if (need == 0)  // the schedule of these sizes keeps everything in registers and LDS
         return spmm_csr_f32(M, K, N, nnz, row_offsets, col_indices, values, B, C, nullptr, 0, stream);
@@ -336,59 +474,18 @@ int spmm_csr_f32_static(int M, int K, int N, int nnz, const int* row_offsets, co
     return spmm_csr_f32(M, K, N, nnz, row_offsets, col_indices, values, B, C, ptr, kStaticScratchBytes, stream);
 }
 
-size_t dlspm_row_plan_bytes(int M) { return M > 0 ? (size_t)3 * (size_t)M * sizeof(int) : 0; }
+size_t dlspm_row_plan_bytes(int M) { return row_plan_bytes(M); }
 
 int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_bytes, void* stream)
 {
     if (M < 0) return DLSPM_E_INVALID_ARG;
     if (M == 0) return DLSPM_OK;
     if (!row_offsets || !plan) return DLSPM_E_INVALID_ARG;
-    if (plan_bytes < dlspm_row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    std::vector<int> ro((size_t)M + 1);
-    hipError_t e = hipMemcpyAsync(ro.data(), row_offsets, ro.size() * sizeof(int), hipMemcpyDeviceToHost, st);
-    if (e == hipSuccess) e = hipStreamSynchronize(st);
-    if (e != hipSuccess) return fail_hip(e);
-    // Longest rows first: workgroups are dispatched in index order, so the rows that take longest start first and the
-    // short ones fill the gaps as compute units free up. The first kResident workgroups all start at once (eight
-    // four-wave workgroups on each of 256 compute units) and workgroup i of them runs on compute unit i mod 256, so
-    // those rows are packed into 256 bins of equal size, longest row first into the least loaded bin that has
-    // room, and bin b becomes the workgroups b, b + 256, b + 512, ... A compute unit's rows then add up to about
-    // the same number of nonzeros (2048 x 512, lognormal rows, N = 256: 7.6 us in matrix order, 7.2 us longest first,
-    // 7.0 us with the groups of 256 alternating between descending and ascending length, 6.1 us packed; bins of 8,
-    // one per XCD, do nothing: 7.2 us). DLSPM_PLAN_ORDER=1|2 gives the alternating and the plain descending order.
-    constexpr int kBins = 256, kResident = 2048;
-    std::vector<int> order((size_t)M);
-    for (int i = 0; i < M; ++i) order[i] = i;
-    auto len = [&](int i) { return ro[(size_t)i + 1] - ro[i]; };
-    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return len(a) > len(b); });
-    const int head = M < kResident ? M : kResident;
-    int variant = 0;
-    if (const char* e = std::getenv("DLSPM_PLAN_ORDER")) variant = std::atoi(e);
-    if (variant == 1) {
-        for (int g = kBins; g < head; g += 2 * kBins) std::reverse(order.begin() + g, order.begin() + (g + kBins < head ? g + kBins : head));
-    } else if (variant != 2) {
-        const int cap = (head + kBins - 1) / kBins;
-        std::vector<long long> load(kBins, 0);
-        std::vector<int> cnt(kBins, 0), placed((size_t)head, -1);
-        for (int i = 0; i < head; ++i) {
-            int best = -1;  // a bin's next workgroup must exist: the last round of bins may be a partial one
-            for (int b = 0; b < kBins; ++b)
-                if (cnt[b] < cap && cnt[b] * kBins + b < head && (best < 0 || load[b] < load[best])) best = b;
-            placed[(size_t)cnt[best] * kBins + best] = order[i];
-            load[best] += len(order[i]);
-            ++cnt[best];
-        }
-        for (int i = 0; i < head; ++i) order[i] = placed[i];
-    }
-    std::vector<int> host((size_t)3 * M);
-    for (int i = 0; i < M; ++i) {
-        host[i] = ro[order[i]];
-        host[(size_t)M + i] = ro[(size_t)order[i] + 1];
-        host[2 * (size_t)M + i] = order[i];
-    }
-    e = hipMemcpyAsync(plan, host.data(), host.size() * sizeof(int), hipMemcpyHostToDevice, st);
-    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (plan_bytes < row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
+    if (const int st = require_device()) return st;
+    // one bin per compute unit: the first 8 x bins workgroups of a launch start together, eight on each compute unit
+    const hipError_t e = row_plan_build_launch(M, row_offsets, static_cast<int*>(plan), device_info().cus,
+                                               tuning().plan_order, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }
 
@@ -408,7 +505,7 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
     } else {
         return 0;
     }
-    // rows known to be even gain nothing from another order (and DLSPM_ROWS_EVEN may serve them better)
+    // rows known to be even gain nothing from another order (and the even-rows hint may serve them better)
     if (max_row_len >= 0 && max_row_len <= 1.5 * ((double)nnz / M)) return 0;
     // dense operands well beyond one L2 need the column-sliced schedule's workspace more than they need balance; the
     // flat schedule, though, is behind the plan wherever both apply (SpMM, lognormal rows, sigma 1 ... 2, row-block /
@@ -419,60 +516,34 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
     return slices >= 3 ? 0 : 1;
 }
 
+// the *_planned entry points: the named call with the plan as its workspace and the hint that says so
 int spmm_csr_f32_planned(int M, int K, int N, int nnz, const int* row_offsets, const int* col_indices,
                          const float* values, const float* B, float* C, const void* plan, size_t plan_bytes,
                          void* stream)
 {
-    if (M < 0 || K < 0 || N < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
-    if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
     if (!plan) return spmm_csr_f32(M, K, N, nnz, row_offsets, col_indices, values, B, C, nullptr, 0, stream);
-    if (plan_bytes < dlspm_row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
-    if (M == 0 || N == 0) return DLSPM_OK;
-    if (!row_offsets || !C) return DLSPM_E_INVALID_ARG;
-    if (nnz > 0 && (!col_indices || !values || !B)) return DLSPM_E_INVALID_ARG;
-    SpmmShape shape = spmm_choose(M, K, N, nnz, N >= 4, false, true);
-    if (!spmm_plan_applies(shape, M, N, nnz))  // short rows grouped per workgroup, or column tiles: the plan has no say
-        return spmm_csr_f32(M, K, N, nnz, row_offsets, col_indices, values, B, C, nullptr, 0, stream);
-    const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C};
-    const hipError_t e = spmm_planned_launch(args, shape, static_cast<const int*>(plan), static_cast<hipStream_t>(stream));
-    return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+    if (plan_bytes & DLSPM_HINT_MASK) return DLSPM_E_INVALID_ARG;
+    return spmm_csr_f32(M, K, N, nnz, row_offsets, col_indices, values, B, C, const_cast<void*>(plan),
+                        plan_bytes | DLSPM_HINT_ROW_PLAN, stream);
 }
 
 int sddmm_csr_f32_planned(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* lhs,
                           const float* rhs, float* out_values, const void* plan, size_t plan_bytes, void* stream)
 {
-    if (M < 0 || K < 0 || D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
-    if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
     if (!plan) return sddmm_csr_f32(M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values, nullptr, 0, stream);
-    if (plan_bytes < dlspm_row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
-    if (M == 0 || nnz == 0) return DLSPM_OK;
-    if (!row_offsets || !col_indices || !out_values) return DLSPM_E_INVALID_ARG;
-    if (D > 0 && (!lhs || !rhs)) return DLSPM_E_INVALID_ARG;
-    SddmmShape shape = sddmm_choose(M, D, nnz, D >= 4);
-    if (D == 0 || !sddmm_plan_applies(shape, M, D, nnz))
-        return sddmm_csr_f32(M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values, nullptr, 0, stream);
-    const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values};
-    const hipError_t e = sddmm_planned_launch(args, shape, static_cast<const int*>(plan), static_cast<hipStream_t>(stream));
-    return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+    if (plan_bytes & DLSPM_HINT_MASK) return DLSPM_E_INVALID_ARG;
+    return sddmm_csr_f32(M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values, const_cast<void*>(plan),
+                         plan_bytes | DLSPM_HINT_ROW_PLAN, stream);
 }
 
 int fused_sddmm_spmm_f32_planned(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* Q,
                                  const float* Kmat, const float* V, float scale, float* O, const void* plan,
                                  size_t plan_bytes, void* stream)
 {
-    if (M < 0 || K < 0 || D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
-    if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
     if (!plan) return fused_sddmm_spmm_f32(M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O, nullptr, 0, stream);
-    if (plan_bytes < dlspm_row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
-    if (M == 0 || D == 0) return DLSPM_OK;
-    if (!row_offsets || !O) return DLSPM_E_INVALID_ARG;
-    if (nnz > 0 && (!col_indices || !Q || !Kmat || !V)) return DLSPM_E_INVALID_ARG;
-    FusedShape shape = fused_choose(M, D, nnz, D >= 4);
-    if (!fused_plan_applies(shape, M, D, nnz))
-        return fused_sddmm_spmm_f32(M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O, nullptr, 0, stream);
-    const FusedArgs args{M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O};
-    const hipError_t e = fused_planned_launch(args, shape, static_cast<const int*>(plan), static_cast<hipStream_t>(stream));
-    return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+    if (plan_bytes & DLSPM_HINT_MASK) return DLSPM_E_INVALID_ARG;
+    return fused_sddmm_spmm_f32(M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O, const_cast<void*>(plan),
+                                plan_bytes | DLSPM_HINT_ROW_PLAN, stream);
 }
 
 int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* lhs,
@@ -480,32 +551,43 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
 {
     if (M < 0 || K < 0 || D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
+    const WorkspaceArg ws = workspace_arg(workspace, workspace_bytes);
+    if (ws.row_plan && ws.mem && ws.bytes < row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
     if (M == 0 || nnz == 0) return DLSPM_OK;
     if (!row_offsets || !col_indices || !out_values) return DLSPM_E_INVALID_ARG;
     if (D > 0 && (!lhs || !rhs)) return DLSPM_E_INVALID_ARG;
+    if (const int st = require_device()) return st;
+    hipStream_t st = static_cast<hipStream_t>(stream);
     if (D == 0) {
-        const unsigned blocks = (unsigned)((nnz + 255) / 256);
-        hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), out_values, nnz);
+        const unsigned blocks = (unsigned)ceil_div(nnz, 256);
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, st, out_values, nnz);
         const hipError_t e0 = hipGetLastError();
         return e0 == hipSuccess ? DLSPM_OK : fail_hip(e0);
     }
     const bool vec4 = D >= 4;  // dwordx4 accesses need only dword alignment
-    const SddmmShape shape = sddmm_choose(M, D, nnz, vec4, workspace == DLSPM_ROWS_EVEN);
     const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values};
+    if (ws.row_plan && ws.mem) {
+        SddmmShape shape = sddmm_choose(M, D, nnz, vec4);
+        if (sddmm_plan_applies(shape, M, D, nnz)) {
+            const hipError_t e = sddmm_planned_launch(args, shape, static_cast<const int*>(ws.mem), st);
+            return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+        }
+        // sizes a planned launch is not built for run as with NULL
+    }
+    const SddmmShape shape = sddmm_choose(M, D, nnz, vec4, ws.rows_even);
     // the flat schedule needs no workspace here (nothing to combine), so the size rule alone decides; it has no
     // width condition for SDDMM (measured for D = 32 ... 256: equal on uniform rows, 15-33 % faster on skewed ones)
-    if (workspace != nullptr && workspace != DLSPM_ROWS_EVEN && workspace_bytes > 0) {
+    if (ws.mem && !ws.rows_even && !ws.row_plan) {
         // with a workspace for the slice boundaries: the column-sliced schedule where the rhs operand exceeds one L2
         const SlicePlan sliced = sddmm_slice_plan(M, K, D, nnz, shape);
-        if (workspace_bytes < sliced.bytes) return DLSPM_E_WORKSPACE;
+        if (ws.bytes < sliced.bytes) return DLSPM_E_WORKSPACE;
         if (sliced.slices > 0) {
-            const hipError_t es = sddmm_sliced_launch(args, shape, sliced, workspace, static_cast<hipStream_t>(stream));
+            const hipError_t es = sddmm_sliced_launch(args, shape, sliced, ws.mem, st);
             return es == hipSuccess ? DLSPM_OK : fail_hip(es);
         }
     }
     const FlatPlan plan = sddmm_flat_plan(M, nnz, D);
-    const hipError_t e = plan.chunk > 0 ? sddmm_flat_launch(args, shape, plan.chunk, static_cast<hipStream_t>(stream))
-                                        : sddmm_launch(args, shape, static_cast<hipStream_t>(stream));
+    const hipError_t e = plan.chunk > 0 ? sddmm_flat_launch(args, shape, plan.chunk, st) : sddmm_launch(args, shape, st);
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }
 
@@ -515,26 +597,35 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz, const int* row_offsets, c
 {
     if (M < 0 || K < 0 || D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
+    const WorkspaceArg ws = workspace_arg(workspace, workspace_bytes);
+    if (ws.row_plan && ws.mem && ws.bytes < row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
     if (M == 0 || D == 0) return DLSPM_OK;
     if (!row_offsets || !O) return DLSPM_E_INVALID_ARG;
     if (nnz > 0 && (!col_indices || !Q || !Kmat || !V)) return DLSPM_E_INVALID_ARG;
+    if (const int st = require_device()) return st;
     const bool vec4 = D >= 4;
-    const bool even = workspace == DLSPM_ROWS_EVEN;
-    const FusedShape shape = fused_choose(M, D, nnz, vec4, even);
+    hipStream_t st = static_cast<hipStream_t>(stream);
     const FusedArgs args{M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O};
     hipError_t e;
-    if (!even && workspace != nullptr && workspace_bytes > 0) {
+    if (ws.row_plan && ws.mem) {
+        FusedShape shape = fused_choose(M, D, nnz, vec4);
+        e = fused_plan_applies(shape, M, D, nnz) ? fused_planned_launch(args, shape, static_cast<const int*>(ws.mem), st)
+                                                 : fused_launch(args, shape, st);
+        return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+    }
+    const FusedShape shape = fused_choose(M, D, nnz, vec4, ws.rows_even);
+    if (!ws.rows_even && ws.mem) {
         const SlicePlan sliced = fused_slice_plan(M, K, D, nnz, shape);
         const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(M, nnz, D, shape.G);
-        if (workspace_bytes < (sliced.slices > 0 ? sliced.bytes : plan.bytes)) return DLSPM_E_WORKSPACE;
+        if (ws.bytes < (sliced.slices > 0 ? sliced.bytes : plan.bytes)) return DLSPM_E_WORKSPACE;
         if (sliced.slices > 0)
-            e = fused_sliced_launch(args, shape, sliced, workspace, static_cast<hipStream_t>(stream));
+            e = fused_sliced_launch(args, shape, sliced, ws.mem, st);
         else if (plan.chunk > 0)
-            e = fused_flat_launch(args, shape, plan, static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
+            e = fused_flat_launch(args, shape, plan, static_cast<float*>(ws.mem), st);
         else
-            e = fused_launch(args, shape, static_cast<hipStream_t>(stream));
+            e = fused_launch(args, shape, st);
     } else {
-        e = fused_launch(args, shape, static_cast<hipStream_t>(stream));
+        e = fused_launch(args, shape, st);
     }
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }
@@ -568,6 +659,7 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
     if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_CSR;
     if (!row_offsets) return DLSPM_E_INVALID_ARG;
     if (nnz > 0 && !col_indices) return DLSPM_E_INVALID_ARG;
+    if (const int st = require_device()) return st;
     hipStream_t s = static_cast<hipStream_t>(stream);
     int* d_flags = nullptr;
     hipError_t e = hipMalloc(&d_flags, sizeof(int));
@@ -576,7 +668,7 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
     e = hipMemsetAsync(d_flags, 0, sizeof(int), s);
     if (e == hipSuccess) {
         const long long work = (long long)(M > nnz ? M : nnz);
-        int blocks = (int)((work + 255) / 256);
+        int blocks = (int)ceil_div(work, 256);
         blocks = blocks < 1 ? 1 : blocks > 2048 ? 2048 : blocks;
         hipLaunchKernelGGL(csr_check_kernel, dim3(blocks), dim3(256), 0, s, M, K, nnz, row_offsets, col_indices, d_flags);
         e = hipGetLastError();
@@ -593,14 +685,14 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
     if (M < 0 || (M > 0 && !row_offsets)) return DLSPM_E_INVALID_ARG;
     int h[2] = {0, 0};
     if (M > 0) {
+        if (const int st = require_device()) return st;
         hipStream_t s = static_cast<hipStream_t>(stream);
         int* d = nullptr;
         hipError_t e = hipMalloc(&d, 2 * sizeof(int));
         if (e != hipSuccess) return fail_hip(e);
         e = hipMemsetAsync(d, 0, 2 * sizeof(int), s);
         if (e == hipSuccess) {
-            int blocks = (M + 255) / 256;
-            blocks = blocks > 1024 ? 1024 : blocks;
+            int blocks = (int)std::min<long long>(ceil_div(M, 256), 1024);
             hipLaunchKernelGGL(row_stats_kernel, dim3(blocks), dim3(256), 0, s, M, row_offsets, d);
             e = hipGetLastError();
         }

@@ -211,6 +211,246 @@ __host__ __device__ __forceinline__ void wave_range(bool aligned, Off&& off, int
     }
 }
 
+// ---- the rows of one workgroup (row-block kernels of all three ops) -------------------------------------------
+// A workgroup of W waves owns R consecutive rows ("row block" rb). RowBlock reads their offsets, splits their nonzeros
+// over the waves and walks wave w's share segment by segment (a segment = the part of one row inside the share).
+//   SLICED = false: row i owns the nonzeros [row_offsets[i], row_offsets[i + 1]).
+//   SLICED = true:  row i owns [row_offsets[i], row_ends[i]), a part of the CSR row (its columns inside one range of
+//                   columns), so the rows of a block are not contiguous in memory: the split then works on the running
+//                   sum of their lengths ("virtual" offsets, 0 at the block's first row) and every segment is shifted
+//                   back to where it lies in memory.
+//   PLANNED (with SLICED and R == 1): workgroup i works on row row_ids[i], whose nonzeros are
+//                   [row_offsets[i], row_ends[i]): a row plan hands the rows out in an order of its own.
+// The R + 1 offsets are read without LDS or a barrier: with R == 1 they are the same two words for every lane (scalar
+// loads); otherwise lane i of every wave holds offset i and v_readlane picks one.
+template <int W, int R, bool SLICED, bool PLANNED>
+struct RowBlock {
+    static_assert(!PLANNED || (SLICED && R == 1), "a row plan names one row per workgroup");
+    int lane, w;
+    int nr;    // rows in this block (fewer than R at the end of the matrix)
+    int row0;  // row of the dense operands and of the output that belongs to the block's first row
+    int off_lo, off_hi, off_win, start_lo, start_win;
+    int T0, T, per, a, b;  // first offset, nonzeros of the block, even share of a wave, this wave's range [a, b)
+    bool aligned;          // the row-aligned split is in use (the same for every wave of the workgroup)
+
+    // `prefetch()` is called right after the offsets were requested: what it asks for arrives in the same round trip
+    template <typename Prefetch>
+    __device__ __forceinline__ void load(int rb, int M, int nnz, const int* __restrict__ row_offsets,
+                                         const int* __restrict__ row_ends, const int* __restrict__ row_ids,
+                                         Prefetch&& prefetch)
+    {
+        lane = threadIdx.x & 63;
+        w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const int r0 = rb * R;
+        nr = PLANNED ? 1 : min(R, M - r0);
+        row0 = r0;
+        off_lo = off_hi = off_win = start_lo = start_win = 0;
+        if constexpr (!SLICED) {
+            if constexpr (R == 1) {
+                off_lo = row_offsets[r0];
+                off_hi = row_offsets[r0 + 1];
+            } else {
+                static_assert(R + 1 <= kWave, "one offset per lane");
+                off_win = row_offsets[r0 + min(lane, nr)];
+            }
+        } else {
+            if constexpr (R == 1) {
+                start_lo = row_offsets[r0];
+                off_hi = row_ends[r0] - start_lo;
+                if constexpr (PLANNED) {
+                    // a plan that was built for another matrix must not take the kernel outside the arrays
+                    row0 = min(max(row_ids[r0], 0), M - 1);
+                    start_lo = min(max(start_lo, 0), nnz);
+                    off_hi = min(max(off_hi, 0), nnz - start_lo);
+                }
+            } else {
+                static_assert(R + 1 <= 32, "the running sum covers 32 lanes");
+                const int i = r0 + min(lane, nr - 1);
+                start_win = row_offsets[i];
+                off_win = lanes_exclusive_sum32(lane < nr ? row_ends[i] - start_win : 0, lane);
+            }
+        }
+        prefetch();
+        T0 = off(0);
+        T = off(nr) - T0;
+        per = split_per_wave(T, W);
+        auto o = [&](int i) { return off(i); };
+        aligned = split_is_row_aligned<W, R>(o, nr, per);
+        int a_, b_;
+        wave_range<W, R>(aligned, o, nr, w, T0, T, per, a_, b_);
+        a = __builtin_amdgcn_readfirstlane(a_);
+        b = __builtin_amdgcn_readfirstlane(b_);
+    }
+    // offset i of the block in the split (i <= nr)
+    __device__ __forceinline__ int off(int i) const
+    {
+        if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
+        else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
+    }
+    // where row i's first nonzero lies in memory, minus its offset in the split
+    __device__ __forceinline__ int shift(int i) const
+    {
+        if constexpr (!SLICED) return 0;
+        else if constexpr (R == 1) return start_lo;
+        else return __builtin_amdgcn_readlane(start_win, __builtin_amdgcn_readfirstlane(i)) - off(i);
+    }
+    // f(r, p, q, rs, re) for every segment [p, q) of this wave's range, in order: r = row of the block, [rs, re) that
+    // row's whole range (all in split positions; add shift(r) for memory positions); rows without nonzeros are skipped
+    template <typename F> __device__ __forceinline__ void for_each_segment(F&& f) const
+    {
+        if (a >= b) return;
+        int r = 0;
+        while (off(r + 1) <= a) ++r;  // first row owning nonzero `a`; exists because a < off(nr)
+        int pos = a;
+        while (pos < b) {
+            const int rs = off(r);
+            const int re = off(r + 1);
+            const int q = __builtin_amdgcn_readfirstlane(min(re, b));
+            const int p = __builtin_amdgcn_readfirstlane(pos);
+            f(r, p, q, rs, re);
+            pos = q;
+            ++r;
+            while (r < nr && off(r + 1) <= pos) ++r;
+        }
+    }
+};
+
+// A row block whose result is one dense row per CSR row (SpMM, the fused op): the lanes' columns, the segments of this
+// wave, and the rows' sums. `segment(acc, r, p, q, colv)` leaves in acc[v] the sum over the nonzeros [p, q) (memory
+// positions) of block row r for this lane's columns colv[v] .. colv[v] + VEC of column tile ct. Rows finished inside one
+// wave are stored straight to `out` (row blk.row0 + r, `width` floats per row); rows shared by several waves leave
+// per-wave partial sums in LDS which are added in wave order after one barrier, so the result does not depend on
+// timing (no atomics, no pre-zeroed output); rows without nonzeros are written as zeros.
+template <int VEC, int G, int V, int W, int R, bool SLICED, bool PLANNED, typename Segment>
+__device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PLANNED>& blk, int ct, int width,
+                                                 float* __restrict__ out, Segment&& segment)
+{
+    constexpr int TW = G * VEC * V;  // columns covered by one wave
+    constexpr int NP = R == 1 ? 1 : 2;  // with one row per workgroup a wave never ends a second segment
+    using VecT = Vec<VEC>;
+    __shared__ __attribute__((aligned(16))) float s_part[W][NP][TW];
+
+    const int lane = blk.lane, w = blk.w, nr = blk.nr;
+    const int g = lane % G;
+    const int slot = lane / G;
+    int colv[V];  // first of this lane's VEC columns for access v; clamped to a valid column when outside
+    bool act[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        const int col = ct * TW + (v * G + g) * VEC;
+        act[v] = col < width;
+        // a lane whose VEC columns would run past the width moves back to end there: it then repeats columns of its
+        // left neighbour, with the same operations, and stores the same values there (width >= VEC)
+        colv[v] = act[v] ? min(col, width - VEC) : 0;
+    }
+    auto s_off = [&](int i) { return blk.off(i); };
+    const int T0 = blk.T0, T = blk.T, per = blk.per, a = blk.a;
+
+    blk.for_each_segment([&](int r, int p, int q, int rs, int re) {
+        VecT acc[V];
+        const int shift = blk.shift(r);
+        segment(acc, r, p + shift, q + shift, colv);
+        const bool whole_row = (p == rs) && (q == re);
+        if (slot == 0) {
+            if (whole_row) {
+                float* orow = out + (size_t)(blk.row0 + r) * width;
+#pragma unroll
+                for (int v = 0; v < V; ++v)
+                    if (act[v]) acc[v].gstore(orow + colv[v]);
+            } else {
+                float* part = s_part[w][(NP == 1 || p == a) ? 0 : 1];
+#pragma unroll
+                for (int v = 0; v < V; ++v) acc[v].store(part + (v * G + g) * VEC);
+            }
+        }
+    });
+    if (blk.aligned) {  // R > 1 only, and the same for every wave of the workgroup
+        if constexpr (R % W == 0) {
+            // every wave stored its rows whole: nothing to combine, no barrier; rows without nonzeros are left
+            if (slot == 0) {
+                for (int r = w; r < nr; r += W) {
+                    if (s_off(r) != s_off(r + 1)) continue;
+                    float* orow = out + (size_t)(blk.row0 + r) * width;
+#pragma unroll
+                    for (int v = 0; v < V; ++v)
+                        if (act[v]) VecT::zero().gstore(orow + colv[v]);
+                }
+            }
+        } else {
+            // the m = W/R waves of a row hold its parts in order, each in its first partial slot
+            constexpr int m = W / R;
+            __syncthreads();
+            if (slot == 0) {
+                for (int r = w; r < nr; r += W) {
+                    const int len = s_off(r + 1) - s_off(r);
+                    const int part = (len + m - 1) / m;
+                    float* orow = out + (size_t)(blk.row0 + r) * width;
+                    if (len > 0 && len <= part) continue;  // one wave held the whole row and stored it
+#pragma unroll
+                    for (int v = 0; v < V; ++v) {
+                        VecT sum = VecT::zero();
+#pragma unroll
+                        for (int j = 0; j < m; ++j)
+                            if (j * part < len) sum.add(VecT::load(&s_part[r * m + j][0][(v * G + g) * VEC]));
+                        if (act[v]) sum.gstore(orow + colv[v]);
+                    }
+                }
+            }
+        }
+        return;
+    }
+    __syncthreads();
+
+    if constexpr (R == 1) {
+        // one row per workgroup: wave x had nonzeros iff x * per < T, and wave 0 adds them up (no division, the
+        // partial sums of all waves are requested from LDS together)
+        if (w == 0 && slot == 0) {
+            float* orow = out + (size_t)blk.row0 * width;
+            if (T == 0) {
+#pragma unroll
+                for (int v = 0; v < V; ++v)
+                    if (act[v]) VecT::zero().gstore(orow + colv[v]);
+            } else if (T > per) {  // T <= per: wave 0 held the whole row and has stored it
+#pragma unroll
+                for (int v = 0; v < V; ++v) {
+                    VecT sum = VecT::zero();
+#pragma unroll
+                    for (int x = 0; x < W; ++x)
+                        if (x * per < T) sum.add(VecT::load(&s_part[x][0][(v * G + g) * VEC]));
+                    if (act[v]) sum.gstore(orow + colv[v]);
+                }
+            }
+        }
+        return;
+    }
+    // rows shared by several waves: add the partial sums in wave order; empty rows: write zeros
+    if (slot == 0) {
+        for (int r = w; r < nr; r += W) {
+            const int rs = s_off(r);
+            const int re = s_off(r + 1);
+            float* orow = out + (size_t)(blk.row0 + r) * width;
+            if (rs == re) {
+#pragma unroll
+                for (int v = 0; v < V; ++v)
+                    if (act[v]) VecT::zero().gstore(orow + colv[v]);
+                continue;
+            }
+            const int wl = (rs - T0) / per;
+            const int wh = (re - 1 - T0) / per;
+            if (wl == wh) continue;  // finished inside one wave, already stored
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                VecT sum = VecT::zero();
+                for (int x = wl; x <= wh; ++x) {
+                    const int k = (NP == 2 && x == wl && T0 + x * per != rs) ? 1 : 0;
+                    sum.add(VecT::load(&s_part[x][k][(v * G + g) * VEC]));
+                }
+                if (act[v]) sum.gstore(orow + colv[v]);
+            }
+        }
+    }
+}
+
 // ---- flat schedule: every wave owns `chunk` consecutive nonzeros of the whole matrix ------------------------
 // Largest row r with row_offsets[r] <= pos, for 0 <= pos < row_offsets[M] (so the row is not empty and holds
 // nonzero `pos`). A 64-ary search by the whole wave: each round reads 64 evenly spaced offsets with one load and

@@ -54,9 +54,9 @@ __device__ __forceinline__ void fused_segment(Vec<VEC>* acc, int p, int q, int D
     if constexpr (kWave / G > 1) slots_sum<VEC, G, V2>(acc, lane);
 }
 
-// The work of workgroup `bid`; SLICED as in spmm_block: row i owns [row_offsets[i], row_ends[i]), the part of the CSR
-// row inside one range of columns, and the split works on the running sum of the lengths.
-// PLANNED (with SLICED and R == 1): workgroup i works on row row_ids[i] of Q, O and the mask, the order of a row plan.
+// The work of workgroup `bid` (RowBlock in common.hpp explains SLICED and PLANNED: with PLANNED workgroup i works on row
+// row_ids[i] of Q, O and the mask). Column tiles (D > 1024) tile-major, as in spmm_block; no division in the usual
+// case of one tile.
 template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R, bool SLICED, bool PLANNED = false>
 __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles, float scale,
                                             const int* __restrict__ row_offsets, const int* __restrict__ row_ends,
@@ -64,198 +64,15 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
                                             const float* __restrict__ Kmat, const float* __restrict__ Vmat,
                                             float* __restrict__ O, const int* __restrict__ row_ids = nullptr, int nnz = 0)
 {
-    static_assert(!PLANNED || (SLICED && R == 1), "a row plan names one row per workgroup");
-    constexpr int TW = G * VEC * V2;
-    constexpr int NP = R == 1 ? 1 : 2;
-    using VecT = Vec<VEC>;
-
-    __shared__ float s_part[W][NP][TW];
-
-    const int lane = threadIdx.x & 63;
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int g = lane % G;
-    const int slot = lane / G;
-    // column tiles (D > 1024) tile-major, as in spmm_block; no division in the usual case of one tile
-    const int row_blocks = (M + R - 1) / R;
+    const int row_blocks = (M - 1) / R + 1;
     const int ct = col_tiles == 1 ? 0 : bid / row_blocks;
     const int rb = bid - ct * row_blocks;
-    const int r0 = rb * R;
-    const int nr = PLANNED ? 1 : min(R, M - r0);
-    int out_row0 = r0;  // row of Q and O that belongs to the block's first row
-
-    // the block's R + 1 row offsets without LDS or a barrier (see spmm_block)
-    int off_lo = 0, off_hi = 0, off_win = 0, start_lo = 0, start_win = 0;
-    if constexpr (!SLICED) {
-        if constexpr (R == 1) {
-            off_lo = row_offsets[r0];
-            off_hi = row_offsets[r0 + 1];
-        } else {
-            static_assert(R + 1 <= kWave, "one offset per lane");
-            off_win = row_offsets[r0 + min(lane, nr)];
-        }
-    } else {
-        if constexpr (R == 1) {
-            start_lo = row_offsets[r0];
-            off_hi = row_ends[r0] - start_lo;
-            if constexpr (PLANNED) {  // a plan built for another matrix must not take the kernel outside the arrays
-                out_row0 = min(max(row_ids[r0], 0), M - 1);
-                start_lo = min(max(start_lo, 0), nnz);
-                off_hi = min(max(off_hi, 0), nnz - start_lo);
-            }
-        } else {
-            static_assert(R + 1 <= 32, "the running sum covers 32 lanes");
-            const int i = r0 + min(lane, nr - 1);
-            start_win = row_offsets[i];
-            off_win = lanes_exclusive_sum32(lane < nr ? row_ends[i] - start_win : 0, lane);
-        }
-    }
-    fetch_args_now(col_indices, Q, Kmat, Vmat, O);  // with the offsets' request: one round trip for both
-    auto s_off = [&](int i) -> int {
-        if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
-        else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
-    };
-    auto s_shift = [&](int i) -> int {
-        if constexpr (!SLICED) return 0;
-        else if constexpr (R == 1) return start_lo;
-        else return __builtin_amdgcn_readlane(start_win, __builtin_amdgcn_readfirstlane(i)) - s_off(i);
-    };
-
-    int colv[V2];
-    bool act[V2];
-#pragma unroll
-    for (int v = 0; v < V2; ++v) {
-        const int col = ct * TW + (v * G + g) * VEC;
-        act[v] = col < D;
-        colv[v] = act[v] ? min(col, D - VEC) : 0;  // a lane that would run past D repeats its neighbour's columns
-    }
-
-    const int T0 = s_off(0);
-    const int T = s_off(nr) - T0;
-    const int per = split_per_wave(T, W);
-    const bool aligned = split_is_row_aligned<W, R>(s_off, nr, per);
-    int a_, b_;
-    wave_range<W, R>(aligned, s_off, nr, w, T0, T, per, a_, b_);
-    const int a = __builtin_amdgcn_readfirstlane(a_);
-    const int b = __builtin_amdgcn_readfirstlane(b_);
-
-    if (a < b) {
-        int r = 0;
-        while (s_off(r + 1) <= a) ++r;
-        int pos = a;
-        while (pos < b) {
-            const int rs = s_off(r);
-            const int re = s_off(r + 1);
-            const int q = __builtin_amdgcn_readfirstlane(min(re, b));
-            const int p = __builtin_amdgcn_readfirstlane(pos);
-            const float* q_row = Q + (size_t)(out_row0 + r) * D;
-
-            VecT acc[V2];
-            const int shift = s_shift(r);
-            fused_segment<VEC, G1, DS, MASKED, G, V2>(acc, p + shift, q + shift, D, scale, col_indices, q_row, Kmat, Vmat,
-                                                      colv, lane);
-
-            const bool whole_row = (p == rs) && (q == re);
-            if (slot == 0) {
-                if (whole_row) {
-                    float* orow = O + (size_t)(out_row0 + r) * D;
-#pragma unroll
-                    for (int v = 0; v < V2; ++v)
-                        if (act[v]) acc[v].gstore(orow + colv[v]);
-                } else {
-                    float* part = s_part[w][(NP == 1 || p == a) ? 0 : 1];
-#pragma unroll
-                    for (int v = 0; v < V2; ++v) acc[v].store(part + (v * G + g) * VEC);
-                }
-            }
-            pos = q;
-            ++r;
-            while (r < nr && s_off(r + 1) <= pos) ++r;
-        }
-    }
-    if (aligned) {  // R > 1 only, and the same for every wave of the workgroup
-        if constexpr (R % W == 0) {
-            // every wave stored its rows whole: nothing to combine, no barrier; rows without nonzeros are left
-            if (slot == 0) {
-                for (int r = w; r < nr; r += W) {
-                    if (s_off(r) != s_off(r + 1)) continue;
-                    float* orow = O + (size_t)(out_row0 + r) * D;
-#pragma unroll
-                    for (int v = 0; v < V2; ++v)
-                        if (act[v]) VecT::zero().gstore(orow + colv[v]);
-                }
-            }
-        } else {
-            // the m = W/R waves of a row hold its parts in order, each in its first partial slot
-            constexpr int m = W / R;
-            __syncthreads();
-            if (slot == 0) {
-                for (int r = w; r < nr; r += W) {
-                    const int len = s_off(r + 1) - s_off(r);
-                    const int part = (len + m - 1) / m;
-                    float* orow = O + (size_t)(out_row0 + r) * D;
-                    if (len > 0 && len <= part) continue;  // one wave held the whole row and stored it
-#pragma unroll
-                    for (int v = 0; v < V2; ++v) {
-                        VecT sum = VecT::zero();
-#pragma unroll
-                        for (int j = 0; j < m; ++j)
-                            if (j * part < len) sum.add(VecT::load(&s_part[r * m + j][0][(v * G + g) * VEC]));
-                        if (act[v]) sum.gstore(orow + colv[v]);
-                    }
-                }
-            }
-        }
-        return;
-    }
-    __syncthreads();
-
-    if constexpr (R == 1) {
-        // one row per workgroup: wave x had nonzeros iff x * per < T, and wave 0 adds them up (no division, the
-        // partial sums of all waves are requested from LDS together)
-        if (w == 0 && slot == 0) {
-            float* orow = O + (size_t)out_row0 * D;
-            if (T == 0) {
-#pragma unroll
-                for (int v = 0; v < V2; ++v)
-                    if (act[v]) VecT::zero().gstore(orow + colv[v]);
-            } else if (T > per) {  // T <= per: wave 0 held the whole row and has stored it
-#pragma unroll
-                for (int v = 0; v < V2; ++v) {
-                    VecT sum = VecT::zero();
-#pragma unroll
-                    for (int x = 0; x < W; ++x)
-                        if (x * per < T) sum.add(VecT::load(&s_part[x][0][(v * G + g) * VEC]));
-                    if (act[v]) sum.gstore(orow + colv[v]);
-                }
-            }
-        }
-        return;
-    }
-    if (slot == 0) {
-        for (int r = w; r < nr; r += W) {
-            const int rs = s_off(r);
-            const int re = s_off(r + 1);
-            float* orow = O + (size_t)(out_row0 + r) * D;
-            if (rs == re) {
-#pragma unroll
-                for (int v = 0; v < V2; ++v)
-                    if (act[v]) VecT::zero().gstore(orow + colv[v]);
-                continue;
-            }
-            const int wl = (rs - T0) / per;
-            const int wh = (re - 1 - T0) / per;
-            if (wl == wh) continue;
-#pragma unroll
-            for (int v = 0; v < V2; ++v) {
-                VecT sum = VecT::zero();
-                for (int x = wl; x <= wh; ++x) {
-                    const int k = (NP == 2 && x == wl && T0 + x * per != rs) ? 1 : 0;
-                    sum.add(VecT::load(&s_part[x][k][(v * G + g) * VEC]));
-                }
-                if (act[v]) sum.gstore(orow + colv[v]);
-            }
-        }
-    }
+    RowBlock<W, R, SLICED, PLANNED> blk;
+    blk.load(rb, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, Q, Kmat, Vmat, O); });
+    dense_rows_block<VEC, G, V2>(blk, ct, D, O, [&](Vec<VEC>* acc, int r, int p, int q, const int* colv) {
+        const float* q_row = Q + (size_t)(blk.row0 + r) * D;
+        fused_segment<VEC, G1, DS, MASKED, G, V2>(acc, p, q, D, scale, col_indices, q_row, Kmat, Vmat, colv, blk.lane);
+    });
 }
 
 // MASKED = false: D == G1 * VEC * DS exactly, every stage-1 access of every lane falls inside the row.
@@ -309,7 +126,7 @@ static hipError_t launch_one(const FusedArgs& x, hipStream_t stream)
 {
     constexpr int TW = G * VEC * V2;
     const int col_tiles = (x.D + TW - 1) / TW;
-    const long long blocks = (long long)((x.M + R - 1) / R) * col_tiles;
+    const long long blocks = ceil_div(x.M, R) * col_tiles;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     if constexpr (DS > 0) {
@@ -361,7 +178,7 @@ FusedShape fused_choose(int M, int D, int nnz, bool vec4, bool rows_even)
         s.G1 = 4; s.DS = 1; s.G = 8; s.V = 1;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(M, (D + tw - 1) / tw, nnz, SplitRule{512, tw >= 1024 ? 4 : 16, kWave / s.G, false}, rows_even, s.W, s.R);
+    choose_split(M, (D + tw - 1) / tw, nnz, SplitRule{2, tw >= 1024 ? 4 : 16, kWave / s.G, false}, rows_even, s.W, s.R);
     return s;
 }
 
@@ -496,7 +313,7 @@ static hipError_t launch_sliced_r(const FusedArgs& x, const SlicePlan& plan, con
 {
     constexpr int TW = G * VEC * V2;
     const int col_tiles = (x.D + TW - 1) / TW;
-    const long long slice_blocks = (long long)((x.M + R - 1) / R) * col_tiles;
+    const long long slice_blocks = ceil_div(x.M, R) * col_tiles;
     const long long blocks = slice_blocks * plan.slices;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;

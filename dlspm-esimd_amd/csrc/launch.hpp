@@ -5,6 +5,31 @@
 
 namespace dlspm {
 
+// ceil(a / b) without the overflow of (a + b - 1) for a near INT_MAX
+inline long long ceil_div(long long a, long long b) { return (a + b - 1) / b; }
+
+// The device the calling thread has current, as far as the launch rules need it: compute units and the size of one
+// L2. Read from hipDeviceProp_t once per device and cached; without a device (host-only queries on a machine that has
+// none) the figures of a whole MI355X: 256 compute units, 4 MiB.
+struct DeviceInfo {
+    int cus;
+    long long l2_bytes;
+    bool present;  // a HIP device is current
+    bool gfx950;   // ... and it is the architecture the kernels are built for
+};
+const DeviceInfo& device_info();
+
+// Overrides of the launch rules for tuning sweeps and tests (dlspm_set_tuning; one set per host thread, initialised from
+// the environment once per process). The fields and their "follow the rule" values are those of dlspm_tuning.
+struct Tuning {
+    int split_w = 0, split_r = 0;
+    int flat = -1, flat_chunk = 0;
+    int slices = -1;
+    int tile_major = -1, tile_width = 0;
+    int plan_order = 0;
+};
+const Tuning& tuning();
+
 // Lane layout and work split of one launch.
 //   vec : floats per lane per access (4 = dwordx4 when the dense width is at least 4, else 1 = dword)
 //   G   : lanes covering one dense row (SpMM / fused stage 2)          V  : accesses per lane per dense row
@@ -69,7 +94,7 @@ struct SlicePlan {
 // row that `bytes` accounts for (0: SDDMM has none, SpMM adds its own); `partial_rows`: the op writes partial rows at
 // all (its slices are then a third larger); G, slots: the op's lane layout
 SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial_width, int G, bool partial_rows,
-                     int slots, int min_blocks);
+                     int slots, int blocks_per_cu);
 hipError_t slice_bounds_launch(int M, int K, int slices, const int* row_offsets, const int* col_indices, int* bounds,
                                hipStream_t stream);
 hipError_t slice_sum_launch(long long count, int slices, const float* partial, float* out, hipStream_t stream);
@@ -79,6 +104,8 @@ SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, b
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
 // Row plan (3 x M ints on the device: first nonzero, end and row number of the row that workgroup i works on): only for
 // shapes of one row per four-wave workgroup and one column tile
+hipError_t row_plan_build_launch(int M, const int* row_offsets, int* plan, int bins, int order, hipStream_t stream);
+size_t row_plan_bytes(int M);
 bool plan_ungroups(int M, int width, int nnz);  // SpMM: rows long enough that a plan runs them one per workgroup against the size rule
 bool plan_ungroups_dots(int M, int D, int nnz);  // the same for SDDMM and the fused op
 bool spmm_plan_applies(SpmmShape& s, int M, int N, int nnz);  // true: s is the shape of the planned launch (R = 1)
@@ -102,11 +129,11 @@ hipError_t fused_sliced_launch(const FusedArgs& x, const FusedShape& s, const Sl
                                hipStream_t stream);
 
 // Picks (W, R), W <= max_w: waves per workgroup from the number of rows, rows per workgroup as large as keeps
-// `min_blocks` workgroups in the grid. `slots` = nonzeros of a row a wave works on at once (64 / G); `w16_long_rows`:
+// `blocks_per_cu` workgroups per compute unit in the grid. `slots` = nonzeros of a row a wave works on at once (64 / G); `w16_long_rows`:
 // the op gains from sixteen waves per row on tall matrices of very long rows. `rows_even`: the caller knows that no
 // row is much longer than the mean. Only the pairs the kernels are instantiated for are returned.
 struct SplitRule {
-    int min_blocks;
+    int blocks_per_cu;
     int max_w;
     int slots;
     bool w16_long_rows;

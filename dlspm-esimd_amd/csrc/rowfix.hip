@@ -41,7 +41,7 @@ __global__ __launch_bounds__(kFlatWaves * 64) void row_fixup_kernel(int M, int N
 hipError_t row_fixup_launch(int M, int N, int chunk, const int* row_offsets, const float* partial, float* out,
                             hipStream_t stream)
 {
-    const unsigned blocks = (unsigned)((M + kFlatWaves - 1) / kFlatWaves);
+    const unsigned blocks = (unsigned)ceil_div(M, kFlatWaves);
     if (N >= 4)
         hipLaunchKernelGGL((row_fixup_kernel<4>), dim3(blocks), dim3(kFlatWaves * 64), 0, stream, M, N, chunk, row_offsets,
                            partial, out);

@@ -47,86 +47,22 @@ __device__ __forceinline__ void sddmm_segment(int p, int q, int D, const int* __
     }
 }
 
-// The work of workgroup `bid`. SLICED = false: row i owns the nonzeros [row_offsets[i], row_offsets[i + 1]); SLICED =
-// true: [row_offsets[i], row_ends[i]), the part of the CSR row inside one range of columns (see spmm_block): the split
-// works on the running sum of the lengths and every segment is shifted back to where it lies, which is also where its
-// results go.
-// PLANNED (with SLICED and R == 1): workgroup i works on row row_ids[i] = [row_offsets[i], row_ends[i]) of the mask, the
-// order of a row plan (see spmm_block).
+// The work of workgroup `bid` (RowBlock in common.hpp explains SLICED and PLANNED; a segment's results go where its
+// nonzeros lie, so a sliced or planned launch writes the same slots as any other). This kernel has neither LDS nor a
+// barrier.
 template <int VEC, int G1, int DS, bool MASKED, int W, int R, bool SLICED, bool PLANNED = false>
 __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __restrict__ row_offsets,
                                             const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                             const float* __restrict__ lhs, const float* __restrict__ rhs,
                                             float* __restrict__ out, const int* __restrict__ row_ids = nullptr, int nnz = 0)
 {
-    static_assert(!PLANNED || (SLICED && R == 1), "a row plan names one row per workgroup");
-    const int lane = threadIdx.x & 63;
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int r0 = bid * R;
-    const int nr = PLANNED ? 1 : min(R, M - r0);
-    int lhs_row0 = r0;  // row of lhs that belongs to the block's first row
-
-    // the block's R + 1 row offsets without LDS or a barrier (see spmm_block): this kernel then has neither
-    int off_lo = 0, off_hi = 0, off_win = 0, start_lo = 0, start_win = 0;
-    if constexpr (!SLICED) {
-        if constexpr (R == 1) {
-            off_lo = row_offsets[r0];
-            off_hi = row_offsets[r0 + 1];
-        } else {
-            static_assert(R + 1 <= kWave, "one offset per lane");
-            off_win = row_offsets[r0 + min(lane, nr)];
-        }
-    } else {
-        if constexpr (R == 1) {
-            start_lo = row_offsets[r0];
-            off_hi = row_ends[r0] - start_lo;
-            if constexpr (PLANNED) {  // a plan built for another matrix must not take the kernel outside the arrays
-                lhs_row0 = min(max(row_ids[r0], 0), M - 1);
-                start_lo = min(max(start_lo, 0), nnz);
-                off_hi = min(max(off_hi, 0), nnz - start_lo);
-            }
-        } else {
-            static_assert(R + 1 <= 32, "the running sum covers 32 lanes");
-            const int i = r0 + min(lane, nr - 1);
-            start_win = row_offsets[i];
-            off_win = lanes_exclusive_sum32(lane < nr ? row_ends[i] - start_win : 0, lane);
-        }
-    }
-    fetch_args_now(col_indices, lhs, rhs, out);  // with the offsets' request: one round trip for both
-    auto s_off = [&](int i) -> int {
-        if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
-        else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
-    };
-    auto s_shift = [&](int i) -> int {
-        if constexpr (!SLICED) return 0;
-        else if constexpr (R == 1) return start_lo;
-        else return __builtin_amdgcn_readlane(start_win, __builtin_amdgcn_readfirstlane(i)) - s_off(i);
-    };
-
-    const int T0 = s_off(0);
-    const int T = s_off(nr) - T0;
-    const int per = split_per_wave(T, W);
-    const bool aligned = split_is_row_aligned<W, R>(s_off, nr, per);
-    int a_, b_;
-    wave_range<W, R>(aligned, s_off, nr, w, T0, T, per, a_, b_);
-    const int a = __builtin_amdgcn_readfirstlane(a_);
-    const int b = __builtin_amdgcn_readfirstlane(b_);
-    if (a >= b) return;
-
-    int r = 0;
-    while (s_off(r + 1) <= a) ++r;
-    int pos = a;
-    while (pos < b) {
-        const int q = __builtin_amdgcn_readfirstlane(min(s_off(r + 1), b));
-        const int p = __builtin_amdgcn_readfirstlane(pos);
-        const float* lhs_row = lhs + (size_t)(lhs_row0 + r) * D;
-
-        const int shift = s_shift(r);
-        sddmm_segment<VEC, G1, DS, MASKED>(p + shift, q + shift, D, col_indices, lhs_row, rhs, out, lane);
-        pos = q;
-        ++r;
-        while (r < nr && s_off(r + 1) <= pos) ++r;
-    }
+    RowBlock<W, R, SLICED, PLANNED> blk;
+    blk.load(bid, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, lhs, rhs, out); });
+    blk.for_each_segment([&](int r, int p, int q, int, int) {
+        const float* lhs_row = lhs + (size_t)(blk.row0 + r) * D;
+        const int shift = blk.shift(r);
+        sddmm_segment<VEC, G1, DS, MASKED>(p + shift, q + shift, D, col_indices, lhs_row, rhs, out, blk.lane);
+    });
 }
 
 // MASKED = false: D == G1 * VEC * DS exactly, every access of every lane falls inside the row.
@@ -171,7 +107,7 @@ __global__ __launch_bounds__(4 * 64) void sddmm_planned_kernel(int M, int D, int
 template <int VEC, int G1, int DS, int W, int R>
 static hipError_t launch_one(const SddmmArgs& x, hipStream_t stream)
 {
-    const int blocks = (x.M + R - 1) / R;
+    const int blocks = (int)ceil_div(x.M, R);
     if (blocks <= 0) return hipSuccess;
     if constexpr (DS > 0) {
         if (x.D == G1 * VEC * DS) {
@@ -217,7 +153,7 @@ SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4, bool rows_even)
         s.G1 = 4;
         s.DS = 1;
     }
-    choose_split(M, 1, nnz, SplitRule{512, 16, kWave / s.G1, true}, rows_even, s.W, s.R);
+    choose_split(M, 1, nnz, SplitRule{2, 16, kWave / s.G1, true}, rows_even, s.W, s.R);
     return s;
 }
 
@@ -317,7 +253,7 @@ hipError_t sddmm_flat_launch(const SddmmArgs& x, const SddmmShape& s, int chunk,
 template <int VEC, int G1, int DS, int R>
 static hipError_t launch_sliced_r(const SddmmArgs& x, const SlicePlan& plan, const int* bounds, hipStream_t stream)
 {
-    const long long slice_blocks = (x.M + R - 1) / R;
+    const long long slice_blocks = ceil_div(x.M, R);
     const long long blocks = slice_blocks * plan.slices;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;

@@ -44,7 +44,7 @@ hipError_t slice_bounds_launch(int M, int K, int slices, const int* row_offsets,
                                hipStream_t stream)
 {
     if (slices < 1 || slices > 31) return hipErrorInvalidValue;
-    const unsigned blocks = (unsigned)((M + 7) / 8);
+    const unsigned blocks = (unsigned)ceil_div(M, 8);
     hipLaunchKernelGGL(slice_bounds_kernel, dim3(blocks), dim3(256), 0, stream, M, K, slices, row_offsets, col_indices,
                        bounds);
     return hipGetLastError();

@@ -18,8 +18,6 @@
 // owns a fixed run of nonzeros of the whole matrix; for very uneven rows) and the column-sliced schedule
 // (the same workgroups on one range of columns of A after the other; for a B larger than one L2), and a
 // B larger than one L2 is always cut into column tiles that the grid works through one after the other.
-#include <cstdlib>
-
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -52,12 +50,12 @@ __device__ __forceinline__ void spmm_segment(Vec<VEC>* acc, int p, int q, const 
     if constexpr (kWave / G > 1) slots_sum<VEC, G, V>(acc, lane);
 }
 
-// The work of workgroup `bid`. SLICED = false: row i owns the nonzeros [row_offsets[i], row_offsets[i + 1]).
-// SLICED = true: row i owns [row_offsets[i], row_ends[i]), a part of the CSR row (its columns inside one range of
-// columns), so the rows of a block are not contiguous in memory: the split then works on the running sum of their
-// lengths ("virtual" offsets, 0 at the block's first row) and every segment is shifted back to where it lies.
-// PLANNED (with SLICED and R == 1): workgroup i works on row row_ids[i], whose nonzeros are [row_offsets[i], row_ends[i]):
-// a row plan hands the rows out in an order of its own.
+// The work of workgroup `bid` (RowBlock in common.hpp explains SLICED and PLANNED; `row_ends` and `row_ids` belong to
+// them). Column tiles (dense rows wider than one wave covers): row-major order (the tiles of a row block next to each
+// other, so the CSR arrays are read from memory once) while all of B fits one L2; tile-major order (all row blocks of
+// tile 0, then of tile 1, ...) when it does not, so that the device gathers from one K x TW slab of B at a time.
+// Measured on 512 x 4608, N = 3136 (B: 55 MiB): 708 -> 239 us tile-major; on 2048 x 1024, N = 784 (3 MiB), lognormal
+// rows: 81 us row-major, 93 us tile-major. No division in the usual case of one tile.
 template <int VEC, int G, int V, int W, int R, bool SLICED, bool PLANNED = false>
 __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles, int tile_major,
                                            const int* __restrict__ row_offsets,
@@ -65,26 +63,10 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
                                            const float* __restrict__ values, const float* __restrict__ B,
                                            float* __restrict__ C, const int* __restrict__ row_ids = nullptr, int nnz = 0)
 {
-    static_assert(!PLANNED || (SLICED && R == 1), "a row plan names one row per workgroup");
-    constexpr int TW = G * VEC * V;  // columns of C covered by one wave
-    using VecT = Vec<VEC>;
-
-    constexpr int NP = R == 1 ? 1 : 2;  // with one row per workgroup a wave never ends a second segment
-    __shared__ float s_part[W][NP][TW];
-
-    const int lane = threadIdx.x & 63;
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int g = lane % G;
-    const int slot = lane / G;
-    // Column tiles (dense rows wider than one wave covers): row-major order (the tiles of a row block next to each
-    // other, so the CSR arrays are read from memory once) while all of B fits one L2; tile-major order (all row blocks
-    // of tile 0, then of tile 1, ...) when it does not, so that the device gathers from one K x TW slab of B at a time.
-    // Measured on 512 x 4608, N = 3136 (B: 55 MiB): 708 -> 239 us tile-major; on 2048 x 1024, N = 784 (3 MiB), lognormal
-    // rows: 81 us row-major, 93 us tile-major. No division in the usual case of one tile.
     int ct = 0, rb = bid;
     if (col_tiles != 1) {
         if (tile_major) {
-            const int row_blocks = (M + R - 1) / R;
+            const int row_blocks = (M - 1) / R + 1;
             ct = bid / row_blocks;
             rb = bid - ct * row_blocks;
         } else {
@@ -92,187 +74,11 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
             ct = bid - rb * col_tiles;
         }
     }
-    const int r0 = rb * R;
-    const int nr = min(R, M - r0);
-    int out_row0 = r0;  // row of C that the block's first row is stored to
-
-    // The block's R + 1 row offsets, without LDS or a barrier: with R == 1 they are the same two words for every
-    // lane (scalar loads); otherwise lane i of every wave holds offset i and v_readlane picks one.
-    int off_lo = 0, off_hi = 0, off_win = 0, start_lo = 0, start_win = 0;
-    if constexpr (!SLICED) {
-        if constexpr (R == 1) {
-            off_lo = row_offsets[r0];
-            off_hi = row_offsets[r0 + 1];
-        } else {
-            static_assert(R + 1 <= kWave, "one offset per lane");
-            off_win = row_offsets[r0 + min(lane, nr)];
-        }
-    } else {
-        if constexpr (R == 1) {
-            start_lo = row_offsets[r0];
-            off_hi = row_ends[r0] - start_lo;
-            if constexpr (PLANNED) {
-                // a plan that was built for another matrix must not take the kernel outside the arrays
-                out_row0 = min(max(row_ids[r0], 0), M - 1);
-                start_lo = min(max(start_lo, 0), nnz);
-                off_hi = min(max(off_hi, 0), nnz - start_lo);
-            }
-        } else {
-            static_assert(R + 1 <= 32, "the running sum covers 32 lanes");
-            const int i = r0 + min(lane, nr - 1);
-            start_win = row_offsets[i];
-            off_win = lanes_exclusive_sum32(lane < nr ? row_ends[i] - start_win : 0, lane);
-        }
-    }
-    fetch_args_now(col_indices, values, B, C);  // after the offsets were requested: both arrive in one round trip
-    auto s_off = [&](int i) -> int {
-        if constexpr (R == 1) return i == 0 ? off_lo : off_hi;
-        else return __builtin_amdgcn_readlane(off_win, __builtin_amdgcn_readfirstlane(i));
-    };
-    // where row i's first nonzero lies in memory, minus its offset in the split
-    auto s_shift = [&](int i) -> int {
-        if constexpr (!SLICED) return 0;
-        else if constexpr (R == 1) return start_lo;
-        else return __builtin_amdgcn_readlane(start_win, __builtin_amdgcn_readfirstlane(i)) - s_off(i);
-    };
-
-    int colv[V];  // first of this lane's VEC columns for access v; clamped to a valid column when outside
-    bool act[V];
-#pragma unroll
-    for (int v = 0; v < V; ++v) {
-        const int col = ct * TW + (v * G + g) * VEC;
-        act[v] = col < N;
-        // a lane whose VEC columns would run past N moves back to end at N: it then repeats columns of its
-        // left neighbour, with the same operations, and stores the same values there (N >= VEC)
-        colv[v] = act[v] ? min(col, N - VEC) : 0;
-    }
-
-    const int T0 = s_off(0);
-    const int T = s_off(nr) - T0;
-    const int per = split_per_wave(T, W);
-    const bool aligned = split_is_row_aligned<W, R>(s_off, nr, per);
-    int a_, b_;
-    wave_range<W, R>(aligned, s_off, nr, w, T0, T, per, a_, b_);
-    const int a = __builtin_amdgcn_readfirstlane(a_);
-    const int b = __builtin_amdgcn_readfirstlane(b_);
-
-    if (a < b) {
-        int r = 0;
-        while (s_off(r + 1) <= a) ++r;  // first row owning nonzero `a`; exists because a < s_off(nr)
-        int pos = a;
-        while (pos < b) {
-            const int rs = s_off(r);
-            const int re = s_off(r + 1);
-            const int q = __builtin_amdgcn_readfirstlane(min(re, b));
-            const int p = __builtin_amdgcn_readfirstlane(pos);
-
-            VecT acc[V];
-            const int shift = s_shift(r);
-            spmm_segment<VEC, G, V>(acc, p + shift, q + shift, col_indices, values, B, N, colv, lane);
-
-            const bool whole_row = (p == rs) && (q == re);
-            if (slot == 0) {
-                if (whole_row) {
-                    float* crow = C + (size_t)(out_row0 + r) * N;
-#pragma unroll
-                    for (int v = 0; v < V; ++v)
-                        if (act[v]) acc[v].gstore(crow + colv[v]);
-                } else {
-                    float* part = s_part[w][(NP == 1 || p == a) ? 0 : 1];
-#pragma unroll
-                    for (int v = 0; v < V; ++v) acc[v].store(part + (v * G + g) * VEC);
-                }
-            }
-            pos = q;
-            ++r;
-            while (r < nr && s_off(r + 1) <= pos) ++r;  // skip rows without nonzeros
-        }
-    }
-    if (aligned) {  // R > 1 only, and the same for every wave of the workgroup
-        if constexpr (R % W == 0) {
-            // every wave stored its rows whole: nothing to combine, no barrier; rows without nonzeros are left
-            if (slot == 0) {
-                for (int r = w; r < nr; r += W) {
-                    if (s_off(r) != s_off(r + 1)) continue;
-                    float* crow = C + (size_t)(out_row0 + r) * N;
-#pragma unroll
-                    for (int v = 0; v < V; ++v)
-                        if (act[v]) VecT::zero().gstore(crow + colv[v]);
-                }
-            }
-        } else {
-            // the m = W/R waves of a row hold its parts in order, each in its first partial slot
-            constexpr int m = W / R;
-            __syncthreads();
-            if (slot == 0) {
-                for (int r = w; r < nr; r += W) {
-                    const int len = s_off(r + 1) - s_off(r);
-                    const int part = (len + m - 1) / m;
-                    float* crow = C + (size_t)(out_row0 + r) * N;
-                    if (len > 0 && len <= part) continue;  // one wave held the whole row and stored it
-#pragma unroll
-                    for (int v = 0; v < V; ++v) {
-                        VecT sum = VecT::zero();
-#pragma unroll
-                        for (int j = 0; j < m; ++j)
-                            if (j * part < len) sum.add(VecT::load(&s_part[r * m + j][0][(v * G + g) * VEC]));
-                        if (act[v]) sum.gstore(crow + colv[v]);
-                    }
-                }
-            }
-        }
-        return;
-    }
-    __syncthreads();
-
-    if constexpr (R == 1) {
-        // one row per workgroup: wave x had nonzeros iff x * per < T, and wave 0 adds them up (no division, the
-        // partial sums of all waves are requested from LDS together)
-        if (w == 0 && slot == 0) {
-            float* crow = C + (size_t)out_row0 * N;
-            if (T == 0) {
-#pragma unroll
-                for (int v = 0; v < V; ++v)
-                    if (act[v]) VecT::zero().gstore(crow + colv[v]);
-            } else if (T > per) {  // T <= per: wave 0 held the whole row and has stored it
-#pragma unroll
-                for (int v = 0; v < V; ++v) {
-                    VecT sum = VecT::zero();
-#pragma unroll
-                    for (int x = 0; x < W; ++x)
-                        if (x * per < T) sum.add(VecT::load(&s_part[x][0][(v * G + g) * VEC]));
-                    if (act[v]) sum.gstore(crow + colv[v]);
-                }
-            }
-        }
-        return;
-    }
-    // rows shared by several waves: add the partial sums in wave order; empty rows: write zeros
-    if (slot == 0) {
-        for (int r = w; r < nr; r += W) {
-            const int rs = s_off(r);
-            const int re = s_off(r + 1);
-            float* crow = C + (size_t)(out_row0 + r) * N;
-            if (rs == re) {
-#pragma unroll
-                for (int v = 0; v < V; ++v)
-                    if (act[v]) VecT::zero().gstore(crow + colv[v]);
-                continue;
-            }
-            const int wl = (rs - T0) / per;
-            const int wh = (re - 1 - T0) / per;
-            if (wl == wh) continue;  // finished inside one wave, already stored
-#pragma unroll
-            for (int v = 0; v < V; ++v) {
-                VecT sum = VecT::zero();
-                for (int x = wl; x <= wh; ++x) {
-                    const int k = (NP == 2 && x == wl && T0 + x * per != rs) ? 1 : 0;
-                    sum.add(VecT::load(&s_part[x][k][(v * G + g) * VEC]));
-                }
-                if (act[v]) sum.gstore(crow + colv[v]);
-            }
-        }
-    }
+    RowBlock<W, R, SLICED, PLANNED> blk;
+    blk.load(rb, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, values, B, C); });
+    dense_rows_block<VEC, G, V>(blk, ct, N, C, [&](Vec<VEC>* acc, int, int p, int q, const int* colv) {
+        spmm_segment<VEC, G, V>(acc, p, q, col_indices, values, B, N, colv, blk.lane);
+    });
 }
 
 template <int VEC, int G, int V, int W, int R>
@@ -323,7 +129,7 @@ static hipError_t launch_one(const SpmmArgs& x, int tile_major, hipStream_t stre
 {
     constexpr int TW = G * VEC * V;
     const int col_tiles = (x.N + TW - 1) / TW;
-    const long long blocks = (long long)((x.M + R - 1) / R) * col_tiles;
+    const long long blocks = ceil_div(x.M, R) * col_tiles;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     hipLaunchKernelGGL((spmm_kernel<VEC, G, V, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream, x.M, x.N,
@@ -362,14 +168,15 @@ static hipError_t launch_wr(const SpmmArgs& x, int W, int R, int tile_major, hip
 // for rows of at least 32 nonzeros on average, and only while the slab is at most twice the L2 (measured on graph-
 // like shapes, K = 262144 ... 1048576, 8 nonzeros per row: tiles of 32 up to 2x slower than one tile; 32 per row:
 // equal; K = 65536, slab 8 MiB, 655 per row: 330 -> 236 us).
-// DLSPM_TILE_MAJOR=0|1 and DLSPM_TILE_WIDTH=512|...|32 override the rule for tuning sweeps.
+// dlspm_tuning.tile_major = 0|1 and .tile_width = 512|...|32 override the rule for tuning sweeps. "The L2" is the
+// device's own figure for one of them (4 MiB on MI355X), "all at once" eight workgroups on each compute unit.
 static int spmm_tile_width(int M, int K, int N, int nnz, bool narrow_tiles)
 {
-    const long long l2 = 4ll << 20;
+    const long long l2 = device_info().l2_bytes;
     const int min_tile = narrow_tiles ? 32 : 128;
     if (N <= min_tile) return 0;
-    bool on = (long long)K * N * (long long)sizeof(float) > l2 && (long long)M * ((N + 511) / 512) >= 2048;
-    if (const char* e = std::getenv("DLSPM_TILE_MAJOR")) on = std::atoi(e) != 0;
+    bool on = (long long)K * N * (long long)sizeof(float) > l2 && (long long)M * ((N + 511) / 512) >= 8ll * device_info().cus;
+    if (tuning().tile_major >= 0) on = tuning().tile_major != 0;
     if (!on) return 0;
     int tile = min_tile;
     for (int t = 512; t > min_tile; t /= 2)
@@ -384,8 +191,8 @@ static int spmm_tile_width(int M, int K, int N, int nnz, bool narrow_tiles)
     const bool narrow_ok =
         (long long)nnz >= 32ll * M && ((long long)K * tile * (long long)sizeof(float) <= 2 * l2 || sliced_too);
     if (!narrow_ok) tile = 512;
-    if (const char* e = std::getenv("DLSPM_TILE_WIDTH")) {
-        const int t = std::atoi(e);
+    {
+        const int t = tuning().tile_width;
         if ((t == 512 || t == 256 || t == 128 || t == 64 || t == 32) && t >= min_tile) tile = t;
     }
     return tile < N ? tile : 0;  // a single tile: nothing to order
@@ -414,7 +221,7 @@ SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, b
         s.V = 1;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(M, (N + tw - 1) / tw, nnz, SplitRule{2048, 16, kWave / s.G, true}, rows_even, s.W, s.R);
+    choose_split(M, (N + tw - 1) / tw, nnz, SplitRule{8, 16, kWave / s.G, true}, rows_even, s.W, s.R);
     return s;
 }
 
@@ -550,7 +357,7 @@ static hipError_t launch_sliced_r(const SpmmArgs& x, const SlicePlan& plan, int 
 {
     constexpr int TW = G * VEC * V;
     const int col_tiles = (x.N + TW - 1) / TW;
-    const long long slice_blocks = (long long)((x.M + R - 1) / R) * col_tiles;
+    const long long slice_blocks = ceil_div(x.M, R) * col_tiles;
     const long long blocks = slice_blocks * plan.slices;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
@@ -605,7 +412,8 @@ hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const Slice
 bool plan_ungroups(int M, int width, int nnz)
 {
     const long long avg32 = 32ll * M, avg48 = 48ll * M, avg128 = 128ll * M;
-    return nnz >= avg32 && (M <= 4096 || (width >= 128 && (M <= 8192 || (nnz >= avg48 && M <= 16384) || nnz >= avg128)));
+    const long long cus = device_info().cus;  // measured on 256 compute units: 4096, 8192 and 16384 rows
+    return nnz >= avg32 && (M <= 16 * cus || (width >= 128 && (M <= 32 * cus || (nnz >= avg48 && M <= 64 * cus) || nnz >= avg128)));
 }
 
 // The same question for SDDMM and the fused op, which gain less from one row per workgroup: lognormal rows, sigma 0.6, rule's
@@ -614,7 +422,8 @@ bool plan_ungroups(int M, int width, int nnz)
 // 55.8 us; 32768 x 4096, D = 64, 100 per row: 68.8 -> 88.1 us; 8192 x 8192, D = 64, 100 per row: equal (SDDMM alike).
 bool plan_ungroups_dots(int M, int D, int nnz)
 {
-    return (long long)nnz >= 32ll * M && (M <= 4096 || (D >= 128 && M <= 8192 && (long long)nnz >= 128ll * M));
+    const long long cus = device_info().cus;  // measured on 256 compute units: 4096 and 8192 rows
+    return (long long)nnz >= 32ll * M && (M <= 16 * cus || (D >= 128 && M <= 32 * cus && (long long)nnz >= 128ll * M));
 }
 
 bool spmm_plan_applies(SpmmShape& s, int M, int N, int nnz)

@@ -23,9 +23,13 @@ E_STATIC_LIMIT = -6
 OP_SPMM, OP_SDDMM, OP_FUSED = 0, 1, 2
 
 
+HINT_ROWS_EVEN = 1 << 62
+HINT_ROW_PLAN = 1 << 61
+
+
 class _RowsEven:
-    """The header's DLSPM_ROWS_EVEN: passed as `workspace`, it tells the library that no row is much longer than the
-    mean (at most 1.5 x nnz / M); it stands for no memory."""
+    """The header's DLSPM_HINT_ROWS_EVEN: passed as `workspace`, it tells the library that no row is much longer than
+    the mean (at most 1.5 x nnz / M); it stands for no memory (a NULL workspace with the hint bit in its size)."""
 
     def __repr__(self):
         return "ROWS_EVEN"
@@ -47,6 +51,10 @@ EXPORTS = (
     "dlspm_row_plan_bytes",
     "dlspm_row_plan_advice",
     "dlspm_row_plan_build",
+    "dlspm_tuning_default",
+    "dlspm_set_tuning",
+    "dlspm_get_tuning",
+    "dlspm_device_info",
     "spmm_csr_f32_planned",
     "sddmm_csr_f32_planned",
     "fused_sddmm_spmm_f32_planned",
@@ -56,6 +64,12 @@ EXPORTS = (
     "dlspm_last_hip_error",
     "dlspm_version",
 )
+
+
+class Tuning(ctypes.Structure):
+    """dlspm_tuning of include/dlspm_hip.h."""
+    _fields_ = [(n, ctypes.c_int) for n in ("split_w", "split_r", "flat", "flat_chunk", "slices", "tile_major",
+                                            "tile_width", "plan_order")]
 
 
 class DlspmError(RuntimeError):
@@ -110,6 +124,14 @@ def lib() -> ctypes.CDLL:
         L.spmm_csr_f32_static.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, vp]
         L.spmm_csr_f32_static.restype = ci
         L.dlspm_static_scratch_bytes.restype = sz
+        L.dlspm_tuning_default.argtypes = [ctypes.POINTER(Tuning)]
+        L.dlspm_tuning_default.restype = None
+        L.dlspm_set_tuning.argtypes = [ctypes.POINTER(Tuning)]
+        L.dlspm_set_tuning.restype = ci
+        L.dlspm_get_tuning.argtypes = [ctypes.POINTER(Tuning)]
+        L.dlspm_get_tuning.restype = ci
+        L.dlspm_device_info.argtypes = [ctypes.POINTER(ci), ctypes.POINTER(ctypes.c_longlong), ctypes.POINTER(ci)]
+        L.dlspm_device_info.restype = ci
         L.dlspm_status_string.argtypes = [ci]
         L.dlspm_status_string.restype = ctypes.c_char_p
         L.dlspm_last_hip_error.restype = ci
@@ -126,7 +148,41 @@ def version() -> str:
     return lib().dlspm_version().decode()
 
 
-def _ptr(t, dtype, name):
+def set_tuning(**fields) -> None:
+    """Overrides of the launch rules for the calling thread (dlspm_set_tuning): split=(W, R), flat, flat_chunk, slices,
+    tile_major, tile_width, plan_order; fields not named follow the rules. No argument: back to the process default."""
+    if not fields:
+        st = lib().dlspm_set_tuning(None)
+    else:
+        t = Tuning()
+        lib().dlspm_tuning_default(ctypes.byref(t))
+        if "split" in fields:
+            t.split_w, t.split_r = fields.pop("split")
+        for k, v in fields.items():
+            if not hasattr(t, k):
+                raise TypeError(f"dlspm_tuning has no field {k}")
+            setattr(t, k, int(v))
+        st = lib().dlspm_set_tuning(ctypes.byref(t))
+    if st != OK:
+        raise DlspmError(st, "dlspm_set_tuning")
+
+
+def get_tuning() -> dict:
+    t = Tuning()
+    lib().dlspm_get_tuning(ctypes.byref(t))
+    return {n: getattr(t, n) for n, _ in Tuning._fields_}
+
+
+def device_info() -> dict:
+    """{'status', 'compute_units', 'l2_bytes', 'gfx950'} of the current device as the library sees it."""
+    cu, l2, ok = ctypes.c_int(0), ctypes.c_longlong(0), ctypes.c_int(0)
+    st = lib().dlspm_device_info(ctypes.byref(cu), ctypes.byref(l2), ctypes.byref(ok))
+    return {"status": st, "compute_units": cu.value, "l2_bytes": l2.value, "gfx950": bool(ok.value)}
+
+
+def _ptr(t, dtype, name, numel=None):
+    """Device pointer of tensor t after checking where it lives, its type, its layout and (numel) that it holds at
+    least that many elements: a size mismatch must be a Python exception, not an out-of-bounds access on the device."""
     import torch
 
     if t is None:
@@ -137,6 +193,8 @@ def _ptr(t, dtype, name):
         raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
     if not t.is_contiguous():
         raise ValueError(f"{name} must be contiguous (row-major)")
+    if numel is not None and t.numel() < numel:
+        raise ValueError(f"{name} holds {t.numel()} elements, the call needs {numel}")
     return ctypes.c_void_p(t.data_ptr()) if t.numel() > 0 else None
 
 
@@ -151,46 +209,63 @@ def row_plan_advice(op, M, K, N_or_D, nnz, max_row_len=-1) -> bool:
     return bool(lib().dlspm_row_plan_advice(op, M, K, N_or_D, nnz, max_row_len))
 
 
-def row_plan(row_offsets):
-    """The row plan of one matrix (an int32 GPU tensor of 3 * M entries) for spmm(..., plan=...); synchronises."""
+def row_plan_bytes(M: int) -> int:
+    return int(lib().dlspm_row_plan_bytes(M))
+
+
+def row_plan(row_offsets, out=None):
+    """The row plan of one matrix (an int32 GPU tensor of row_plan_bytes(M) / 4 entries; the launches read the first
+    3 * M) for spmm / sddmm / fused(..., plan=...). Built by kernels on the current stream: no synchronisation.
+    `out`: a tensor to build into (callers under graph capture)."""
     import torch
 
     M = row_offsets.numel() - 1
-    plan = torch.empty((lib().dlspm_row_plan_bytes(M) // 4,), dtype=torch.int32, device=row_offsets.device)
-    st = lib().dlspm_row_plan_build(M, _ptr(row_offsets, torch.int32, "row_offsets"), _ptr(plan, torch.int32, "plan"),
+    need = row_plan_bytes(M) // 4
+    plan = out if out is not None else torch.empty((need,), dtype=torch.int32, device=row_offsets.device)
+    st = lib().dlspm_row_plan_build(M, _ptr(row_offsets, torch.int32, "row_offsets", M + 1), _ptr(plan, torch.int32, "plan", need),
                                     plan.numel() * 4, _stream())
     if st != OK:
         raise DlspmError(st, "dlspm_row_plan_build")
     return plan
 
 
-def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None, plan=None):
-    """C = A_csr @ B on the current stream. row_offsets/col_indices int32, values/B float32, all on the GPU.
-    `workspace`: optional GPU tensor of at least workspace_bytes(OP_SPMM, ...) bytes, or ROWS_EVEN.
-    `plan`: optional row plan of this matrix (row_plan()), instead of a workspace."""
+def _csr_sizes(row_offsets, col_indices):
+    if row_offsets.numel() < 1:
+        raise ValueError("row_offsets must hold M + 1 >= 1 entries")
+    return row_offsets.numel() - 1, col_indices.numel()
+
+
+def _workspace_args(workspace, plan, M):
+    """(pointer, size with hint bits) for the pair (workspace, workspace_bytes) of the three compute entry points."""
     import torch
 
-    M = row_offsets.numel() - 1
-    nnz = col_indices.numel()
-    Kd, N = B.shape
-    K = Kd if K is None else K
-    if out is None:
-        out = torch.empty((M, N), dtype=torch.float32, device=B.device)
     if plan is not None:
         if workspace is not None:
             raise ValueError("pass a row plan or a workspace, not both")
-        st = lib().spmm_csr_f32_planned(M, K, N, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
-                                        _ptr(col_indices, torch.int32, "col_indices"),
-                                        _ptr(values, torch.float32, "values"), _ptr(B, torch.float32, "B"),
-                                        _ptr(out, torch.float32, "C"), _ptr(plan, torch.int32, "plan"),
-                                        plan.numel() * 4, _stream())
-        if st != OK:
-            raise DlspmError(st, "spmm_csr_f32_planned")
-        return out
-    wp, wb = _workspace(workspace)
+        need = row_plan_bytes(M) // 4
+        return _ptr(plan, torch.int32, "plan", need), (plan.numel() * 4) | HINT_ROW_PLAN
+    return _workspace(workspace)
+
+
+def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None, plan=None):
+    """C = A_csr @ B on the current stream (spmm_csr_f32). row_offsets/col_indices int32, values/B float32, all on
+    the GPU. `workspace`: optional GPU tensor of at least workspace_bytes(OP_SPMM, ...) bytes, or ROWS_EVEN.
+    `plan`: optional row plan of this matrix (row_plan()), passed as the workspace with DLSPM_HINT_ROW_PLAN."""
+    import torch
+
+    M, nnz = _csr_sizes(row_offsets, col_indices)
+    if B.dim() != 2:
+        raise ValueError("B must be a K x N matrix")
+    Kd, N = B.shape
+    K = Kd if K is None else K
+    if K > Kd:
+        raise ValueError(f"B has {Kd} rows, the matrix has K = {K} columns")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=B.device)
+    wp, wb = _workspace_args(workspace, plan, M)
     st = lib().spmm_csr_f32(M, K, N, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
-                            _ptr(col_indices, torch.int32, "col_indices"), _ptr(values, torch.float32, "values"),
-                            _ptr(B, torch.float32, "B"), _ptr(out, torch.float32, "C"), wp, wb, _stream())
+                            _ptr(col_indices, torch.int32, "col_indices"), _ptr(values, torch.float32, "values", nnz),
+                            _ptr(B, torch.float32, "B"), _ptr(out, torch.float32, "C", M * N), wp, wb, _stream())
     if st != OK:
         raise DlspmError(st, "spmm_csr_f32")
     return out
@@ -206,77 +281,63 @@ def spmm_static(row_offsets, col_indices, values, B, K=None, out=None):
     array; allocates nothing inside the library. `out` must be given by callers that may not allocate either."""
     import torch
 
-    M = row_offsets.numel() - 1
-    nnz = col_indices.numel()
+    M, nnz = _csr_sizes(row_offsets, col_indices)
     Kd, N = B.shape
     K = Kd if K is None else K
+    if K > Kd:
+        raise ValueError(f"B has {Kd} rows, the matrix has K = {K} columns")
     if out is None:
         out = torch.empty((M, N), dtype=torch.float32, device=B.device)
     st = lib().spmm_csr_f32_static(M, K, N, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
-                                   _ptr(col_indices, torch.int32, "col_indices"), _ptr(values, torch.float32, "values"),
-                                   _ptr(B, torch.float32, "B"), _ptr(out, torch.float32, "C"), _stream())
+                                   _ptr(col_indices, torch.int32, "col_indices"), _ptr(values, torch.float32, "values", nnz),
+                                   _ptr(B, torch.float32, "B"), _ptr(out, torch.float32, "C", M * N), _stream())
     if st != OK:
         raise DlspmError(st, "spmm_csr_f32_static")
     return out
 
 
 def sddmm(row_offsets, col_indices, lhs, rhs, out=None, workspace=None, plan=None):
-    """out[j] = <lhs[i], rhs[col[j]]> for each CSR slot j of row i, on the current stream.
+    """out[j] = <lhs[i], rhs[col[j]]> for each CSR slot j of row i, on the current stream (sddmm_csr_f32).
     `workspace`: None, ROWS_EVEN, or a GPU tensor of workspace_bytes(OP_SDDMM, ...) bytes (the slice boundaries of the
-    column-sliced schedule; 0 bytes where that schedule does not apply)."""
+    column-sliced schedule; 0 bytes where that schedule does not apply). `plan`: a row plan of the mask instead."""
     import torch
 
-    M = row_offsets.numel() - 1
-    nnz = col_indices.numel()
+    M, nnz = _csr_sizes(row_offsets, col_indices)
+    if lhs.dim() != 2 or rhs.dim() != 2 or lhs.shape[1] != rhs.shape[1]:
+        raise ValueError("lhs must be M x D and rhs K x D")
     K, D = rhs.shape
+    if lhs.shape[0] < M:
+        raise ValueError(f"lhs has {lhs.shape[0]} rows, the mask has {M}")
     if out is None:
         out = torch.empty((nnz,), dtype=torch.float32, device=lhs.device)
-    if plan is not None:
-        if workspace is not None:
-            raise ValueError("pass a row plan or a workspace, not both")
-        st = lib().sddmm_csr_f32_planned(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
-                                         _ptr(col_indices, torch.int32, "col_indices"), _ptr(lhs, torch.float32, "lhs"),
-                                         _ptr(rhs, torch.float32, "rhs"), _ptr(out, torch.float32, "out"),
-                                         _ptr(plan, torch.int32, "plan"), plan.numel() * 4, _stream())
-        if st != OK:
-            raise DlspmError(st, "sddmm_csr_f32_planned")
-        return out
+    wp, wb = _workspace_args(workspace, plan, M)
     st = lib().sddmm_csr_f32(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
                              _ptr(col_indices, torch.int32, "col_indices"), _ptr(lhs, torch.float32, "lhs"),
-                             _ptr(rhs, torch.float32, "rhs"), _ptr(out, torch.float32, "out"), *_workspace(workspace),
-                             _stream())
+                             _ptr(rhs, torch.float32, "rhs"), _ptr(out, torch.float32, "out", nnz), wp, wb, _stream())
     if st != OK:
         raise DlspmError(st, "sddmm_csr_f32")
     return out
 
 
 def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None, workspace=None, plan=None):
-    """O = (S .* (Q Kmat^T) * scale) V on the current stream; the scores are never stored.
+    """O = (S .* (Q Kmat^T) * scale) V on the current stream (fused_sddmm_spmm_f32); the scores are never stored.
     `workspace`: optional GPU tensor of at least workspace_bytes(OP_FUSED, ...) bytes, or ROWS_EVEN.
-    `plan`: optional row plan of the mask (row_plan()), instead of a workspace."""
+    `plan`: optional row plan of the mask (row_plan()), passed as the workspace with DLSPM_HINT_ROW_PLAN."""
     import torch
 
-    M = row_offsets.numel() - 1
-    nnz = col_indices.numel()
+    M, nnz = _csr_sizes(row_offsets, col_indices)
+    if Q.dim() != 2 or Kmat.dim() != 2 or V.shape != Kmat.shape or Q.shape[1] != Kmat.shape[1]:
+        raise ValueError("Q must be M x D, Kmat and V K x D")
     K, D = Kmat.shape
+    if Q.shape[0] < M:
+        raise ValueError(f"Q has {Q.shape[0]} rows, the mask has {M}")
     if out is None:
         out = torch.empty((M, D), dtype=torch.float32, device=Q.device)
-    if plan is not None:
-        if workspace is not None:
-            raise ValueError("pass a row plan or a workspace, not both")
-        st = lib().fused_sddmm_spmm_f32_planned(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
-                                                _ptr(col_indices, torch.int32, "col_indices"), _ptr(Q, torch.float32, "Q"),
-                                                _ptr(Kmat, torch.float32, "Kmat"), _ptr(V, torch.float32, "V"),
-                                                ctypes.c_float(scale), _ptr(out, torch.float32, "O"),
-                                                _ptr(plan, torch.int32, "plan"), plan.numel() * 4, _stream())
-        if st != OK:
-            raise DlspmError(st, "fused_sddmm_spmm_f32_planned")
-        return out
+    wp, wb = _workspace_args(workspace, plan, M)
     st = lib().fused_sddmm_spmm_f32(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
                                     _ptr(col_indices, torch.int32, "col_indices"), _ptr(Q, torch.float32, "Q"),
                                     _ptr(Kmat, torch.float32, "Kmat"), _ptr(V, torch.float32, "V"),
-                                    ctypes.c_float(scale), _ptr(out, torch.float32, "O"), *_workspace(workspace),
-                                    _stream())
+                                    ctypes.c_float(scale), _ptr(out, torch.float32, "O", M * D), wp, wb, _stream())
     if st != OK:
         raise DlspmError(st, "fused_sddmm_spmm_f32")
     return out
@@ -323,7 +384,7 @@ def _workspace(ws):
     if ws is None:
         return None, 0
     if ws is ROWS_EVEN:
-        return ctypes.c_void_p(1), 0
+        return None, HINT_ROWS_EVEN
     if not ws.is_cuda or not ws.is_contiguous():
         raise ValueError("workspace must be a contiguous GPU tensor")
     return ctypes.c_void_p(ws.data_ptr()), ws.numel() * ws.element_size()

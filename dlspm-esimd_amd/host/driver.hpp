@@ -206,7 +206,7 @@ struct Options {
     int iters = 20;  // the reference keeps the minimum of 20 launches (SPMM/spmm-esimd-fromfile2.cpp:194-243)
     bool cold = false;
     // what to pass as `workspace`: by default the memory dlspm_workspace_bytes asks for when the column-sliced schedule
-    // applies or the longest row is at least four times the mean row (dlspm_csr_row_stats), DLSPM_ROWS_EVEN when it is
+    // applies or the longest row is at least four times the mean row (dlspm_csr_row_stats), DLSPM_HINT_ROWS_EVEN when it is
     // at most one and a half times the mean;
     // --workspace: always the memory, --no-workspace: always NULL
     enum Workspace { kAuto, kAlways, kNever } workspace = kAuto;
@@ -217,12 +217,13 @@ struct Options {
 };
 
 // What this run passes as `workspace`: what dlspm_workspace_advice says for the sizes and the longest row
-// (dlspm_csr_row_stats, one look per matrix) -- device memory, the constant DLSPM_ROWS_EVEN, or nothing.
+// (dlspm_csr_row_stats, one look per matrix) -- device memory, the hint DLSPM_HINT_ROWS_EVEN, or nothing.
 struct WorkspaceChoice {
     size_t bytes = 0;        // device memory to allocate and pass
-    bool rows_even = false;  // pass DLSPM_ROWS_EVEN instead
-    bool plan = false;       // build a row plan and launch the op's _planned entry point instead
-    void* arg(void* buffer) const { return rows_even ? DLSPM_ROWS_EVEN : bytes ? buffer : nullptr; }
+    bool rows_even = false;  // pass NULL with DLSPM_HINT_ROWS_EVEN instead
+    bool plan = false;       // build a row plan and pass it as the workspace, with DLSPM_HINT_ROW_PLAN
+    void* arg(void* buffer) const { return bytes ? buffer : nullptr; }
+    size_t size() const { return rows_even ? DLSPM_HINT_ROWS_EVEN : bytes; }
 };
 inline WorkspaceChoice workspace_to_pass(const Options& opt, int op, int M, int K, int width, int nnz,
                                          const int* row_offsets_dev, bool plan_allowed = false)
@@ -247,19 +248,30 @@ inline WorkspaceChoice workspace_to_pass(const Options& opt, int op, int M, int 
                 opt.workspace == Options::kAlways ? "workspace passed (--workspace)"
                 : c.bytes && slices > 0           ? "dense operands beyond one L2, workspace passed (column-sliced schedule)"
                 : c.bytes                         ? "uneven, workspace passed (flat schedule)"
-                : c.rows_even                     ? "even, DLSPM_ROWS_EVEN passed"
+                : c.rows_even                     ? "even, DLSPM_HINT_ROWS_EVEN passed"
                                                   : "nothing passed");
     return c;
 }
 
-// The row plan of one matrix (dlspm_row_plan_build: once per matrix, synchronises), with what it cost.
+// The row plan of one matrix (dlspm_row_plan_build: once per matrix, kernels on the stream), with what it cost on the
+// device (HIP events around the second of two builds: the first pays for loading the kernels).
 inline DevBuf<char> build_row_plan(int M, const int* row_offsets_dev)
 {
     DevBuf<char> plan(dlspm_row_plan_bytes(M));
-    const auto t0 = std::chrono::steady_clock::now();
-    if (dlspm_row_plan_build(M, row_offsets_dev, plan.p, plan.n, nullptr) != DLSPM_OK) throw std::runtime_error("dlspm_row_plan_build failed");
-    const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
-    std::printf("row plan: %zu bytes, built in %.3f ms (once per matrix)\n", plan.n, ms);
+    hipEvent_t e0, e1;
+    DLSPM_HIP_CHECK(hipEventCreate(&e0));
+    DLSPM_HIP_CHECK(hipEventCreate(&e1));
+    float ms = 0;
+    for (int rep = 0; rep < 2; ++rep) {
+        DLSPM_HIP_CHECK(hipEventRecord(e0, nullptr));
+        if (dlspm_row_plan_build(M, row_offsets_dev, plan.p, plan.n, nullptr) != DLSPM_OK) throw std::runtime_error("dlspm_row_plan_build failed");
+        DLSPM_HIP_CHECK(hipEventRecord(e1, nullptr));
+        DLSPM_HIP_CHECK(hipEventSynchronize(e1));
+        DLSPM_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    std::printf("row plan: %zu bytes, built on the device in %.1f us (once per matrix)\n", plan.n, ms * 1e3);
     return plan;
 }
 

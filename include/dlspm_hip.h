@@ -39,15 +39,19 @@
  *     workspace smaller than that is refused with DLSPM_E_WORKSPACE. The contents need no
  *     initialisation and mean nothing afterwards; two calls that share a workspace must not overlap
  *     in time.
- *   - A caller who knows the opposite, that no row is much longer than the mean (longest row at most
- *     one and a half times nnz / M), may say so by passing the constant DLSPM_ROWS_EVEN as `workspace`
- *     (with workspace_bytes 0; it stands for no memory and is never dereferenced). Tall matrices of
- *     long rows then run one whole row per wave, which is the faster split for even rows and the
- *     slower one for uneven rows. It is a hint about speed only: a wrong one costs time, never
- *     correctness (a row's products are added in a different, equally fixed order), and other sizes
- *     ignore it.
+ *   - Two more things travel through the same pair of arguments, as hint bits in the upper byte of `workspace_bytes`
+ *     (DLSPM_HINT_*, or-ed into the size; they are no part of the size):
+ *       DLSPM_HINT_ROWS_EVEN, with workspace NULL: the caller knows that no row is much longer than the mean (longest
+ *         row at most one and a half times nnz / M). Tall matrices of long rows then run one whole row per wave, which
+ *         is the faster split for even rows and the slower one for uneven rows. It is a hint about speed only: a wrong
+ *         one costs time, never correctness (a row's products are added in a different, equally fixed order), and
+ *         other sizes ignore it.
+ *       DLSPM_HINT_ROW_PLAN: `workspace` holds the row plan of this matrix (dlspm_row_plan_build, below; at least
+ *         dlspm_row_plan_bytes(M) bytes, else DLSPM_E_WORKSPACE) and the launch hands the rows out in the plan's order.
+ *         The plan is only read.
  * Calls on different streams may run concurrently from different host threads (each with its own
- * workspace); the library keeps no mutable global state.
+ * workspace). The library's only mutable state is per host thread (the tuning overrides of dlspm_set_tuning and the
+ * last HIP error), a cache of the devices' properties, and the static scratch array of spmm_csr_f32_static.
  */
 #ifndef DLSPM_HIP_H
 #define DLSPM_HIP_H
@@ -64,10 +68,16 @@ extern "C" {
 #define DLSPM_E_WORKSPACE    (-2) /* a workspace was passed, but smaller than dlspm_workspace_bytes()        */
 #define DLSPM_E_LAUNCH       (-3) /* the HIP runtime refused the launch (see dlspm_last_hip_error)         */
 #define DLSPM_E_INVALID_CSR  (-4) /* dlspm_csr_check found a malformed CSR structure                        */
-#define DLSPM_E_NO_DEVICE    (-5) /* no gfx950 device is current                                            */
+#define DLSPM_E_NO_DEVICE    (-5) /* the current device is not a gfx950, or there is none                   */
 #define DLSPM_E_STATIC_LIMIT (-6) /* spmm_csr_f32_static: the sizes need more scratch than the library holds   */
 
-/* `workspace` value that carries the caller's knowledge "row lengths are even" instead of memory (see above) */
+/* hints, or-ed into `workspace_bytes` (see above); the size proper is workspace_bytes & ~DLSPM_HINT_MASK */
+#define DLSPM_HINT_ROWS_EVEN ((size_t)1 << 62)
+#define DLSPM_HINT_ROW_PLAN  ((size_t)1 << 61)
+#define DLSPM_HINT_MASK      ((size_t)0xFF << 56)
+
+/* Deprecated spelling of DLSPM_HINT_ROWS_EVEN, still accepted: this constant as `workspace` with workspace_bytes 0.
+ * A pointer value that is no pointer is easy to forward by accident; new code passes the hint bit. */
 #define DLSPM_ROWS_EVEN ((void*)1)
 
 /* operation selectors for dlspm_workspace_bytes */
@@ -162,35 +172,41 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
  * (SPMM/spmmesimd2.hpp:30-60).
  * Use: the compute calls cannot see how evenly the nonzeros are spread over the rows; a caller who finds
  * max_row_len at least four times nnz / M should pass a workspace, one who finds it at most one and a half times
- * nnz / M may pass DLSPM_ROWS_EVEN (see above), anyone else NULL.
+ * nnz / M may pass DLSPM_HINT_ROWS_EVEN (see above), anyone else NULL.
  */
 int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_row_len, int* empty_rows);
 
 /*
- * Row plan for SpMM: the order in which a launch hands the rows of one matrix to its workgroups, built once per
- * matrix (like the two calls above) and passed to spmm_csr_f32_planned with every launch. Small matrices with
- * uneven rows, one row per workgroup and every workgroup on the device at once, finish when the compute unit that
- * was handed the most nonzeros does; the plan puts the long rows first and packs the rows that start together so
- * that every compute unit is handed about the same number of nonzeros (2048 x 512, lognormal row lengths, N = 256:
- * 7.6 -> 6.1 us); larger matrices with uneven rows gain as much from the rows being handed out longest first.
- * Every row is summed by one four-wave workgroup in a fixed order (no atomics): the result is bit-identical to
- * spmm_csr_f32 with a NULL workspace wherever that call runs one row per workgroup too.
- *   dlspm_row_plan_bytes(M)  bytes of DEVICE memory for the plan of a matrix of M rows (3 * M ints).
- *   dlspm_row_plan_build     reads row_offsets (device) back, sorts on the host and writes the plan to `plan`
- *                            (device); synchronises `stream`. DLSPM_E_WORKSPACE if plan_bytes is too small.
- *   spmm_csr_f32_planned     spmm_csr_f32 with that plan instead of a workspace. The plan must have been built from
- *                            the same row_offsets (a stale plan gives wrong values but stays inside the arrays).
- *                            It runs one row per workgroup also where spmm_csr_f32 would group a few rows, if the
- *                            rows are long enough (the same sums as spmm_csr_f32 under DLSPM_SPLIT=4,1). Short rows,
- *                            column tiles of a B that fits one L2 and widths below 4 ignore it and run as
- *                            spmm_csr_f32(..., NULL, 0, stream); plan == NULL too. A planned launch is one kernel
- *                            (no memset, no allocation, no synchronisation): it may be captured in a HIP graph; the
- *                            plan is only read, so launches may share it.
+ * Row plan: the order in which a launch hands the rows of one matrix to its workgroups, built once per matrix
+ * structure and passed with every launch as its workspace, with DLSPM_HINT_ROW_PLAN. Small matrices with uneven rows,
+ * one row per workgroup and every workgroup on the device at once, finish when the compute unit that was handed the
+ * most nonzeros does; the plan puts the long rows first and packs the rows that start together so that every compute
+ * unit is handed about the same number of nonzeros (2048 x 512, lognormal row lengths, N = 256: 7.6 -> 6.1 us); larger
+ * matrices with uneven rows gain as much from the rows being handed out longest first. Every row is summed by one
+ * four-wave workgroup in a fixed order (no atomics): the result is bit-identical to the call with a NULL workspace
+ * wherever that runs one row per workgroup too.
+ *   dlspm_row_plan_bytes(M)  bytes of DEVICE memory for the plan of a matrix of M rows: 3 * M ints, and beyond 2048
+ *                            rows as much again and a third for the sort (the launches read the first 3 * M ints).
+ *   dlspm_row_plan_build     builds the plan from row_offsets (device) into `plan` (device, 8-byte aligned) with
+ *                            kernels on `stream`: nothing is copied to the host, nothing synchronises, and the call may
+ *                            be captured in a HIP graph together with the launches that use the plan (one launch up to
+ *                            2048 rows, 3 + log2(M / 2048) beyond). A mask whose structure changes from call to call
+ *                            can therefore be re-planned on the stream. DLSPM_E_WORKSPACE if plan_bytes is too small.
+ *   the launches             spmm_csr_f32 / sddmm_csr_f32 / fused_sddmm_spmm_f32 with workspace = plan and
+ *                            workspace_bytes = plan_bytes | DLSPM_HINT_ROW_PLAN. The plan must have been built from the
+ *                            same row_offsets (a stale plan gives wrong values but stays inside the arrays). A planned
+ *                            launch runs one row per workgroup also where the size rule would group a few rows, if the
+ *                            rows are long enough. Short rows, column tiles of a B that fits one L2, widths below 4
+ *                            (SDDMM and the fused op: widths outside 16 < D <= 512, and rows that the size rule groups
+ *                            in masks of more than 4096 rows, 8192 at D >= 128 and 128 nonzeros per row) ignore the
+ *                            plan and run as with NULL. A planned launch is one kernel (no memset, no allocation, no
+ *                            synchronisation); the plan is only read, so launches may share it.
+ *   *_planned                the same launches with the plan as a separate argument (plan == NULL: the plain call).
  * No counterpart in the reference, whose kernels take the rows in matrix order (SPMM/spmmesimd2.hpp:63-75).
  */
 size_t dlspm_row_plan_bytes(int M);
 /* 1 if a row plan is worth building for op (DLSPM_OP_*) at these sizes and this longest row (-1: unknown): the planned
- * call would use it (one column tile, rows of at least 32 nonzeros on average where the size rule would group rows;
+ * launch would use it (one column tile, rows of at least 32 nonzeros on average where the size rule would group rows;
  * SDDMM and the fused op: 16 < D <= 512), the rows are
  * not known to be even, and B is not so far beyond one L2 that the column-sliced schedule's workspace matters more;
  * else 0. Ask this before dlspm_workspace_advice: where both a plan and the flat schedule's workspace apply, the plan
@@ -200,11 +216,6 @@ int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_
 int spmm_csr_f32_planned(int M, int K, int N, int nnz, const int* row_offsets, const int* col_indices,
                          const float* values, const float* B, float* C, const void* plan, size_t plan_bytes,
                          void* stream);
-/* The same plan (it depends on row_offsets only) for the other two ops, with the arguments of sddmm_csr_f32 and
- * fused_sddmm_spmm_f32 and the plan in place of the workspace. Measured on lognormal rows against the plain calls:
- * 2048 x 2048 mask, D = 64, 100 per row: fused 12.3 -> 8.4 us, SDDMM 6.8 -> 5.0 us; 8192 x 2048, D = 128, 197 per row:
- * 77.6 -> 57.4 us and 41.5 -> 30.8 us. Widths outside 16 < D <= 512, short rows, and rows that the size rule groups in
- * masks of more than 4096 rows (8192 at D >= 128 and 128 nonzeros per row) ignore the plan. */
 int sddmm_csr_f32_planned(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* lhs,
                           const float* rhs, float* out_values, const void* plan, size_t plan_bytes, void* stream);
 int fused_sddmm_spmm_f32_planned(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices,
@@ -213,7 +224,7 @@ int fused_sddmm_spmm_f32_planned(int M, int K, int D, int nnz, const int* row_of
 
 /*
  * What to pass as `workspace` for a matrix of these sizes whose longest row has max_row_len nonzeros (from
- * dlspm_csr_row_stats, or known to the caller): DLSPM_PASS_NULL, DLSPM_PASS_ROWS_EVEN (the constant DLSPM_ROWS_EVEN)
+ * dlspm_csr_row_stats, or known to the caller): DLSPM_PASS_NULL, DLSPM_PASS_ROWS_EVEN (NULL with DLSPM_HINT_ROWS_EVEN)
  * or DLSPM_PASS_WORKSPACE (dlspm_workspace_bytes() bytes of device memory). It holds the measured rules in one place:
  * the memory where the column-sliced schedule applies (except even rows at two slices in SpMM and the fused op) or
  * where the longest row is at least four times the mean and the flat schedule applies; the constant where the
@@ -239,7 +250,7 @@ int dlspm_workspace_advice(int op, int M, int K, int N_or_D, int nnz, int max_ro
 int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape);
 
 /*
- * The same for a call that passes NULL, DLSPM_ROWS_EVEN or workspace memory (`passing` = DLSPM_PASS_NULL,
+ * The same for a call that passes NULL, the even-rows hint or workspace memory (`passing` = DLSPM_PASS_NULL,
  * DLSPM_PASS_ROWS_EVEN, DLSPM_PASS_WORKSPACE, defined with dlspm_workspace_advice): the lane layout of SpMM
  * (column tiles narrower than 128 only without memory; tiles of 128 on a B of any height only with it, where the
  * column-sliced schedule cuts the tile's slab of B) and the rows per workgroup (more for rows known to be even)
@@ -254,6 +265,38 @@ int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int pa
  * workgroup. Either pointer may be NULL. Host-only. No counterpart in the reference.
  */
 int dlspm_describe_slices(int op, int M, int K, int N_or_D, int nnz, int* slices, int* rows_per_workgroup);
+
+/*
+ * Overrides of the launch rules, for tuning sweeps and tests; production callers never need them. One set per host
+ * thread: dlspm_set_tuning changes the calling thread's, NULL goes back to the process default. That default is the
+ * rules themselves unless the environment said otherwise when the library first looked, once per process:
+ * DLSPM_SPLIT="W,R", DLSPM_FLAT, DLSPM_FLAT_CHUNK, DLSPM_SLICES, DLSPM_TILE_MAJOR, DLSPM_TILE_WIDTH, DLSPM_PLAN_ORDER
+ * (so that the drivers can be swept from a shell). No launch reads the environment. An override that names a shape
+ * the kernels are not built for is ignored. dlspm_workspace_bytes and the describe calls follow the overrides, so
+ * set them before sizing a workspace. No counterpart in the reference (its knobs are -D macros, SPMM/spmmesimd.hpp:17-21).
+ */
+typedef struct dlspm_tuning {
+    int split_w, split_r; /* waves and rows per workgroup of the row-block kernels; 0, 0 = the size rule           */
+    int flat;             /* flat schedule of a call with workspace: -1 the size rule, 0 never, 1 always            */
+    int flat_chunk;       /* nonzeros per wave of the flat schedule (>= 64); 0 = the rule                           */
+    int slices;           /* column-sliced schedule: -1 the size rule, 0 never, n >= 2 that many slices             */
+    int tile_major;       /* SpMM column tiles one after the other: -1 the rule, 0 no, 1 yes                        */
+    int tile_width;       /* SpMM column tile: 0 the rule, else 512, 256, 128, 64 or 32                             */
+    int plan_order;       /* dlspm_row_plan_build: 0 packed (the rule), 1 alternating groups, 2 longest first       */
+} dlspm_tuning;
+void dlspm_tuning_default(dlspm_tuning* t);   /* fills *t with "follow the rules" */
+int dlspm_set_tuning(const dlspm_tuning* t);  /* DLSPM_OK or DLSPM_E_INVALID_ARG (a field out of range) */
+int dlspm_get_tuning(dlspm_tuning* t);        /* what the calling thread's launches currently use */
+
+/*
+ * What the library knows about the device that the calling thread has current (read from hipDeviceProp_t once per
+ * device): compute units, bytes of one L2, and whether it is the gfx950 the kernels are built for. Any pointer may be
+ * NULL. The launch rules scale with the first two (bins of a row plan = compute units, slices and column tiles from
+ * the L2 size). Returns DLSPM_E_NO_DEVICE without a device (the figures are then those of a whole MI355X: 256, 4 MiB,
+ * which is also what the host-only size queries use there); the compute entry points return DLSPM_E_NO_DEVICE when
+ * the current device is not a gfx950.
+ */
+int dlspm_device_info(int* compute_units, long long* l2_bytes, int* is_gfx950);
 
 /* Human-readable text for a status code (never NULL). */
 const char* dlspm_status_string(int status);

@@ -32,6 +32,16 @@ def dl():
     return dlspm_hip
 
 
+@pytest.fixture(autouse=True)
+def _rules_after_every_test():
+    """Tests that override the launch rules (dl.set_tuning) must not leak the override into the next test."""
+    yield
+    import dlspm_hip
+
+    if dlspm_hip._lib is not None:
+        dlspm_hip.set_tuning()
+
+
 def random_csr(rng, M, K, kind="uniform", density=0.1):
     """Seeded CSR pattern with ascending unique columns. kind: uniform | skewed | empty_rows | full | empty."""
     if kind == "uniform":

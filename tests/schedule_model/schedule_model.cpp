@@ -350,4 +350,45 @@ int model_fused_flat(int M, int D, const int* ro, const int* ci, const float* Q,
     return model_rows_flat(M, D, nnz, ro, ci, scores, V, G, chunk, O, writes);
 }
 
+// Host model of the row plan that dlspm_row_plan_build builds on the device: rows sorted longest first (by row number
+// among equals); the first min(M, 8 x bins) of them packed into `bins` bins of equal size, longest row first into the
+// least loaded bin that still has room (ties: the lower bin), bin b becoming the positions b, b + bins, b + 2 bins, ...;
+// rows without nonzeros fill the positions still free, in ascending order; the rest follow in sorted order.
+// order 1: groups of `bins` alternate between descending and ascending length instead; order 2: plainly descending.
+// plan[0 .. M) first nonzero, plan[M .. 2M) end, plan[2M .. 3M) row. This sequential statement is the definition; the
+// device finds the same packing in parallel batches.
+void model_row_plan(int M, const int* ro, int bins, int order, int* plan)
+{
+    std::vector<int> sorted((size_t)M);
+    for (int i = 0; i < M; ++i) sorted[i] = i;
+    auto len = [&](int i) { return ro[i + 1] - ro[i] > 0 ? ro[i + 1] - ro[i] : 0; };
+    std::stable_sort(sorted.begin(), sorted.end(), [&](int a, int b) { return len(a) > len(b); });
+    const int head = M < 8 * bins ? M : 8 * bins;
+    std::vector<int> at((size_t)M);
+    for (int i = 0; i < M; ++i) at[i] = sorted[i];
+    if (order == 1) {
+        for (int g = bins; g < head; g += 2 * bins) std::reverse(at.begin() + g, at.begin() + (g + bins < head ? g + bins : head));
+    } else if (order == 0) {
+        std::vector<long long> load((size_t)bins, 0);
+        std::vector<int> cnt((size_t)bins, 0), placed((size_t)head, -1);
+        int t = 0;
+        for (; t < head && len(sorted[t]) > 0; ++t) {
+            int best = -1;
+            for (int b = 0; b < bins; ++b)
+                if ((long long)cnt[b] * bins + b < head && (best < 0 || load[b] < load[best])) best = b;
+            placed[(size_t)cnt[best] * bins + best] = sorted[t];
+            load[best] += len(sorted[t]);
+            ++cnt[best];
+        }
+        for (int p = 0; p < head; ++p)
+            if (placed[p] < 0) placed[p] = sorted[t++];
+        for (int p = 0; p < head; ++p) at[p] = placed[p];
+    }
+    for (int i = 0; i < M; ++i) {
+        plan[i] = ro[at[i]];
+        plan[(size_t)M + i] = ro[at[i] + 1];
+        plan[2 * (size_t)M + i] = at[i];
+    }
+}
+
 }  // extern "C"

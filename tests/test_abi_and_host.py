@@ -31,7 +31,9 @@ def test_header_is_plain_c(tmp_path):
     src.write_text('#include "dlspm_hip.h"\n'
                    "int use(void) { int shape[10]; return dlspm_describe_launch(DLSPM_OP_SPMM, 1, 1, 1, 1, shape)"
                    " + (int)dlspm_workspace_bytes(DLSPM_OP_FUSED, 1, 1, 1, 1)"
-                   " + spmm_csr_f32(0, 0, 0, 0, 0, 0, 0, 0, 0, DLSPM_ROWS_EVEN, 0, 0); }\n")
+                   " + spmm_csr_f32(0, 0, 0, 0, 0, 0, 0, 0, 0, DLSPM_ROWS_EVEN, 0, 0)"
+                   " + spmm_csr_f32(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, DLSPM_HINT_ROWS_EVEN | DLSPM_HINT_ROW_PLAN, 0);"
+                   " dlspm_tuning t; dlspm_tuning_default(&t); t.split_w = 4; t.split_r = 1; return dlspm_set_tuning(&t); }\n")
     inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
     r = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-fsyntax-only", "-I", inc, str(src)],
                        capture_output=True, text=True)
@@ -230,11 +232,93 @@ def test_row_plan_host_side(dl):
     assert L.dlspm_row_plan_build(-1, bogus, bogus, 0, None) == dl.E_INVALID_ARG
     assert L.dlspm_row_plan_build(8, None, bogus, 96, None) == dl.E_INVALID_ARG
     assert L.dlspm_row_plan_build(8, bogus, bogus, 95, None) == dl.E_WORKSPACE
+    assert L.dlspm_row_plan_build(4096, bogus, bogus, 3 * 4096 * 4, None) == dl.E_WORKSPACE   # beyond 2048 rows: room for the sort
     assert L.dlspm_row_plan_build(0, None, None, 0, None) == dl.OK
     assert L.spmm_csr_f32_planned(-1, 1, 1, 0, None, None, None, None, None, bogus, 0, None) == dl.E_INVALID_ARG
     assert L.spmm_csr_f32_planned(2, 2, 2, 5, None, None, None, None, None, bogus, 24, None) == dl.E_INVALID_ARG
     assert L.spmm_csr_f32_planned(2, 2, 2, 1, bogus, bogus, bogus, bogus, bogus, bogus, 23, None) == dl.E_WORKSPACE
     assert L.spmm_csr_f32_planned(2, 2, 2, 1, None, None, None, None, None, None, 0, None) == dl.E_INVALID_ARG  # as spmm_csr_f32
+
+
+def test_tuning_overrides_go_through_one_call_and_the_environment_is_read_once(dl):
+    """dlspm_set_tuning replaces the per-launch getenv knobs: per thread, validated, and visible to the host-only
+    queries; the environment only seeds the process default, once, so a later change of it changes nothing."""
+    import threading
+
+    base = dl.get_tuning()
+    assert base == {"split_w": 0, "split_r": 0, "flat": -1, "flat_chunk": 0, "slices": -1, "tile_major": -1,
+                    "tile_width": 0, "plan_order": 0}
+    sizes = (dl.OP_SPMM, 8192, 4096, 128, 8192 * 600)
+    rule = dl.describe_launch(*sizes)
+    assert (rule["W"], rule["R"]) == (4, 1)
+    dl.set_tuning(split=(8, 2))
+    assert dl.get_tuning()["split_w"] == 8 and (dl.describe_launch(*sizes)["W"], dl.describe_launch(*sizes)["R"]) == (8, 2)
+    seen = {}
+    th = threading.Thread(target=lambda: seen.update(dl.get_tuning()))   # another thread still follows the rules
+    th.start()
+    th.join()
+    assert seen == base
+    dl.set_tuning(split=(5, 3))          # not a shape the kernels are built for: ignored
+    assert (dl.describe_launch(*sizes)["W"], dl.describe_launch(*sizes)["R"]) == (4, 1)
+    os.environ["DLSPM_SPLIT"] = "16,1"   # the environment was read when the library first looked; not again
+    try:
+        dl.set_tuning()
+        assert dl.get_tuning() == base and dl.describe_launch(*sizes) == rule
+    finally:
+        del os.environ["DLSPM_SPLIT"]
+    dl.set_tuning(tile_width=128, tile_major=1)
+    sh = dl.describe_launch(dl.OP_SPMM, 4096, 512, 512, 4096 * 50)
+    assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (128, 4)
+    dl.set_tuning()
+    for bad in ({"flat": 2}, {"slices": -2}, {"plan_order": 3}, {"tile_major": 5}, {"split": (-1, 0)}, {"flat_chunk": -64}):
+        with pytest.raises(dl.DlspmError):
+            dl.set_tuning(**bad)
+    assert dl.get_tuning() == base
+    assert dl.lib().dlspm_get_tuning(None) == dl.E_INVALID_ARG
+    src = open(os.path.join(ROOT, "dlspm-esimd_amd", "csrc", "api.hip")).read()
+    sources = "".join(open(os.path.join(ROOT, "dlspm-esimd_amd", "csrc", f)).read()
+                      for f in os.listdir(os.path.join(ROOT, "dlspm-esimd_amd", "csrc")))
+    assert sources.count("getenv(") == 1 and src.count("getenv(") == 1
+
+
+def test_the_environment_seeds_the_process_default(dl):
+    """A fresh process started with DLSPM_SPLIT / DLSPM_FLAT_CHUNK in its environment starts from those overrides (how
+    the C++ drivers are swept from a shell)."""
+    code = ("import sys; sys.path.insert(0, %r); import dlspm_hip as dl; t = dl.get_tuning(); "
+            "print(t['split_w'], t['split_r'], t['flat_chunk'], t['slices'])" % os.path.join(ROOT, "dlspm-esimd_amd"))
+    env = dict(os.environ, DLSPM_SPLIT="8,1", DLSPM_FLAT_CHUNK="320", DLSPM_SLICES="0")
+    r = subprocess.run(["python", "-c", code], capture_output=True, text=True, env=env)
+    assert r.returncode == 0 and r.stdout.split() == ["8", "1", "320", "0"], r.stderr
+
+
+def test_device_info_and_hints_without_a_gpu(dl):
+    """Host-only: without a device the size rules use a whole MI355X's figures and the compute calls that would have
+    to launch say DLSPM_E_NO_DEVICE; the hint bits are no part of the workspace size."""
+    import torch
+
+    info = dl.device_info()
+    if torch.cuda.is_available():
+        assert info["status"] == dl.OK and info["gfx950"]
+    else:
+        assert info == {"status": dl.E_NO_DEVICE, "compute_units": 256, "l2_bytes": 4 << 20, "gfx950": False}
+        bogus = ctypes.c_void_p(256)   # never dereferenced: no device, no launch
+        L = dl.lib()
+        assert L.spmm_csr_f32(2, 2, 2, 1, bogus, bogus, bogus, bogus, bogus, None, 0, None) == dl.E_NO_DEVICE
+        assert L.sddmm_csr_f32(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, None, 0, None) == dl.E_NO_DEVICE
+        assert L.fused_sddmm_spmm_f32(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, 1.0, bogus, None, 0, None) == dl.E_NO_DEVICE
+        assert L.dlspm_row_plan_build(8, bogus, bogus, 96, None) == dl.E_NO_DEVICE
+        assert L.dlspm_csr_check(2, 2, 1, bogus, bogus, None) == dl.E_NO_DEVICE
+        assert L.spmm_csr_f32_static(2, 2, 2, 1, bogus, bogus, bogus, bogus, bogus, None) == dl.E_NO_DEVICE
+    assert "gfx950" in dl.status_string(dl.E_NO_DEVICE)
+    L = dl.lib()
+    bogus = ctypes.c_void_p(256)
+    # a plan hint with too little memory behind it is refused before anything else is looked at; hint bits alone are not a size
+    assert L.spmm_csr_f32(2, 2, 2, 1, bogus, bogus, bogus, bogus, bogus, bogus, 23 | dl.HINT_ROW_PLAN, None) == dl.E_WORKSPACE
+    assert L.sddmm_csr_f32(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, bogus, 23 | dl.HINT_ROW_PLAN, None) == dl.E_WORKSPACE
+    assert L.fused_sddmm_spmm_f32(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, 1.0, bogus, bogus, 23 | dl.HINT_ROW_PLAN, None) == dl.E_WORKSPACE
+    assert L.spmm_csr_f32(0, 5, 5, 0, None, None, None, None, None, None, dl.HINT_ROWS_EVEN, None) == dl.OK
+    assert L.spmm_csr_f32_planned(2, 2, 2, 1, bogus, bogus, bogus, bogus, bogus, bogus, 24 | dl.HINT_ROWS_EVEN, None) == dl.E_INVALID_ARG
+    assert dl.row_plan_bytes(2048) == 3 * 2048 * 4 and dl.row_plan_bytes(2049) == 3 * 2049 * 4 + 4 + 2 * 2049 * 8
 
 
 def test_library_exports_every_declared_symbol(dl):
@@ -261,10 +345,9 @@ def test_host_only_entry_points_answer_without_a_gpu(dl):
     assert L.sddmm_csr_f32(5, 5, 4, 0, None, None, None, None, None, None, 0, None) == dl.OK
 
 
-def test_flat_schedule_rule_and_workspace_size(dl, monkeypatch):
+def test_flat_schedule_rule_and_workspace_size(dl):
     """Host-only: the size rule of the flat schedule and the workspace it asks for (units x 2 x width floats)."""
-    monkeypatch.delenv("DLSPM_FLAT", raising=False)
-    monkeypatch.delenv("DLSPM_FLAT_CHUNK", raising=False)
+    dl.set_tuning()
     M, K, nnz = 8192, 4096, 3355443
     sh = dl.describe_launch(dl.OP_SPMM, M, K, 128, nnz)
     assert sh["flat_chunk"] == 512 and sh["flat_units"] == -(-nnz // 512)
@@ -285,9 +368,7 @@ def test_flat_schedule_rule_and_workspace_size(dl, monkeypatch):
     for cfg_sizes in [(512, 512, 128, 78643), (2048, 512, 256, 105687), (2048, 512, 392, 208896), (4096, 4096, 64, 324737)]:
         for op in (dl.OP_SPMM, dl.OP_SDDMM, dl.OP_FUSED):
             assert dl.workspace_bytes(op, *cfg_sizes) == 0 and dl.describe_launch(op, *cfg_sizes)["flat_chunk"] == 0
-    monkeypatch.setenv("DLSPM_FLAT", "1")
-    monkeypatch.setenv("DLSPM_SLICES", "0")
-    monkeypatch.setenv("DLSPM_FLAT_CHUNK", "192")
+    dl.set_tuning(flat=1, slices=0, flat_chunk=192)
     assert dl.workspace_bytes(dl.OP_SPMM, 100, 50, 7, 1000) == -(-1000 // 192) * 2 * 7 * 4
 
 

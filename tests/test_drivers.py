@@ -357,14 +357,14 @@ def test_batch_run_dlmc_script(oracle, tmp_path):
 
 @pytest.mark.gpu
 def test_drivers_pass_the_workspace_only_for_uneven_rows():
-    """3.3 M nonzeros: large enough for the flat schedule. Even rows: the driver passes DLSPM_ROWS_EVEN and no memory;
+    """3.3 M nonzeros: large enough for the flat schedule. Even rows: the driver passes DLSPM_HINT_ROWS_EVEN and no memory;
     lognormal rows (sigma 1.5): the workspace; in between (sigma 0.2) nothing; all self-check against the on-device
     gold loop."""
     rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--iters", 3)
-    assert rc == 0 and "PASS" in out and "even, DLSPM_ROWS_EVEN passed" in out and "workspace:" not in out, out
+    assert rc == 0 and "PASS" in out and "even, DLSPM_HINT_ROWS_EVEN passed" in out and "workspace:" not in out, out
     for app in ("sddmm_run", "fused_run"):
         rc, out = run(app, "--shape", 8192, 4096, 128, 0.1, "--iters", 3)
-        assert rc == 0 and "PASS" in out and "even, DLSPM_ROWS_EVEN passed" in out, out
+        assert rc == 0 and "PASS" in out and "even, DLSPM_HINT_ROWS_EVEN passed" in out, out
     rc, out = run("spmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 0.2, "--iters", 3, "--no-plan")
     assert rc == 0 and "PASS" in out and "nothing passed" in out and "workspace:" not in out, out
     rc, out = run("sddmm_run", "--shape", 8192, 4096, 128, 0.1, "--sigma", 0.2, "--iters", 3, "--no-plan")

@@ -499,10 +499,10 @@ def test_exact_integer_properties_at_large_size(torch_cuda, dl):
         check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
-def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle, monkeypatch):
+def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle):
     """spmm_csr_f32_planned hands the rows to the workgroups in the plan's order (longest first), one row per four-wave
     workgroup, and must return the bits of spmm_csr_f32 (NULL workspace) in that same shape -- which is the size rule's
-    own shape for most of these cases, and the shape forced by DLSPM_SPLIT=4,1 where the rule groups rows and the plan
+    own shape for most of these cases, and the shape forced by the tuning override split = (4, 1) where the rule groups rows and the plan
     ungroups them. The plan itself is a permutation of the rows with each row's own offsets. Short rows, column tiles of a
     B that fits the L2 and widths below 4 ignore the plan and run as without it."""
     torch = torch_cuda
@@ -526,7 +526,7 @@ def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle, mon
         ro_d, ci_d, va_d, B_d = (dev(torch, x) for x in (ro, ci, va, B))
         plan = dl.row_plan(ro_d)
         h = plan.cpu().numpy()
-        starts, ends, rows = h[:M], h[M:2 * M], h[2 * M:]
+        starts, ends, rows = h[:M], h[M:2 * M], h[2 * M:3 * M]
         assert np.array_equal(np.sort(rows), np.arange(M))
         assert np.array_equal(starts, ro[rows]) and np.array_equal(ends, ro[rows + 1])
         lens = ends - starts
@@ -535,9 +535,9 @@ def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle, mon
             assert (lens[2048:][:-1] >= lens[2048:][1:]).all()                   # after the resident part: descending
         sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size)
         want = dl.spmm(ro_d, ci_d, va_d, B_d, K=K).clone()
-        monkeypatch.setenv("DLSPM_SPLIT", "4,1")
+        dl.set_tuning(split=(4, 1))
         want_one_row = dl.spmm(ro_d, ci_d, va_d, B_d, K=K).clone()
-        monkeypatch.delenv("DLSPM_SPLIT")
+        dl.set_tuning()
         got = torch.full((M, N), float("nan"), device="cuda")
         dl.spmm(ro_d, ci_d, va_d, B_d, K=K, out=got, plan=plan)
         if dl.row_plan_advice(dl.OP_SPMM, M, K, N, ci.size, -1):   # rows unknown: 1 exactly where the planned kernel runs
@@ -555,10 +555,10 @@ def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle, mon
     assert used >= 6 and ungrouped >= 1 and tiled >= 1 and used < len(cases)
 
 
-def test_row_plan_for_sddmm_and_the_fused_op(torch_cuda, dl, oracle, monkeypatch):
+def test_row_plan_for_sddmm_and_the_fused_op(torch_cuda, dl, oracle):
     """The same plan drives sddmm_csr_f32_planned and fused_sddmm_spmm_f32_planned: one row of the mask per four-wave
     workgroup, in plan order. Their results must have the bits of the plain calls in that same shape (the size rule's
-    own, or DLSPM_SPLIT=4,1 where the rule groups rows), and agree with the oracle; widths outside 16 < D <= 512 and short
+    own, or the tuning override split = (4, 1) where the rule groups rows), and agree with the oracle; widths outside 16 < D <= 512 and short
     rows run as without a plan."""
     torch = torch_cuda
     rng = np.random.default_rng(99)
@@ -578,9 +578,9 @@ def test_row_plan_for_sddmm_and_the_fused_op(torch_cuda, dl, oracle, monkeypatch
                 (dl.OP_SDDMM, lambda: dl.sddmm(ro_d, ci_d, Q_d, K_d).clone(), lambda: dl.sddmm(ro_d, ci_d, Q_d, K_d, plan=plan).clone()),
                 (dl.OP_FUSED, lambda: dl.fused(ro_d, ci_d, Q_d, K_d, V_d, 0.25).clone(), lambda: dl.fused(ro_d, ci_d, Q_d, K_d, V_d, 0.25, plan=plan).clone())):
             want = plain()
-            monkeypatch.setenv("DLSPM_SPLIT", "4,1")
+            dl.set_tuning(split=(4, 1))
             want_one_row = plain()
-            monkeypatch.delenv("DLSPM_SPLIT")
+            dl.set_tuning()
             got = with_plan()
             if dl.row_plan_advice(op, M, K, D, ci.size, -1):
                 assert torch.equal(got, want_one_row), (kind, M, K, D, op)
@@ -611,14 +611,14 @@ def test_stale_row_plan_stays_inside_the_arrays(torch_cuda, dl):
     dl.spmm(ro_d, ci_d, va_d, B_d, K=K, out=out, plan=stale)
     torch.cuda.synchronize()
     assert torch.isfinite(out).all()
-    with pytest.raises(dl.DlspmError):   # a plan for fewer rows is refused before any launch
+    with pytest.raises((dl.DlspmError, ValueError)):   # a plan for fewer rows is refused before any launch (binding or library)
         dl.spmm(ro_d, ci_d, va_d, B_d, K=K, out=out, plan=stale[:3 * M - 3])
     # and the right plan right after gives the right bits
     good = dl.spmm(ro_d, ci_d, va_d, B_d, K=K, plan=dl.row_plan(ro_d))
     assert torch.equal(good, dl.spmm(ro_d, ci_d, va_d, B_d, K=K))
 
 
-def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
+def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl):
     """All three schedules only enqueue kernels (no memset, no allocation, no synchronisation), so a call may be captured.
     The graph is replayed several times with eager work and synchronisations in between, on changed inputs, and every
     replay must equal the eager result bit for bit."""
@@ -632,11 +632,9 @@ def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
     Q = torch.randn(M, N, device="cuda")
     for schedule in ("row-block", "flat", "sliced"):
         if schedule == "flat":
-            monkeypatch.setenv("DLSPM_FLAT", "1")
-            monkeypatch.setenv("DLSPM_SLICES", "0")
-            monkeypatch.setenv("DLSPM_FLAT_CHUNK", "128")
+            dl.set_tuning(flat=1, slices=0, flat_chunk=128)
         elif schedule == "sliced":
-            monkeypatch.setenv("DLSPM_SLICES", "3")
+            dl.set_tuning(slices=3)
         need = max(dl.workspace_bytes(op, M, K, N, ci.size) for op in (dl.OP_SPMM, dl.OP_SDDMM, dl.OP_FUSED))
         assert (need > 0) == (schedule != "row-block")
         ws = torch.empty(need, dtype=torch.uint8, device="cuda") if need else None
@@ -680,6 +678,94 @@ def test_calls_can_be_captured_in_a_hip_graph(torch_cuda, dl, monkeypatch):
             torch.cuda.synchronize()
             for g, w in zip(got, want):
                 assert torch.equal(g, w), f"replay {rep}, schedule {schedule}"
+
+
+@pytest.mark.parametrize("M", [1500, 6000])
+def test_plan_build_and_planned_launches_in_one_hip_graph(torch_cuda, dl, oracle, M):
+    """dlspm_row_plan_build is kernels only, so building the plan and launching with it can be captured together: the
+    case of a mask whose structure changes from call to call. Each replay follows an in-place change of row_offsets and
+    col_indices (same array sizes, other row lengths) and must give the bits of the eager planned calls on the new
+    structure, which in turn agree with the oracle. 1500 rows: the build is one launch; 6000: tiles, merges, packing."""
+    torch = torch_cuda
+    rng = np.random.default_rng(M)
+    K, N = 700, 128
+    structures = []
+    ro0, ci0 = random_csr(rng, M, K, "skewed", 0.25)   # long enough rows that all three ops run one row per workgroup
+    for _ in range(3):   # other structures with the same number of nonzeros: the rows' lengths permuted
+        perm = rng.permutation(M)
+        lens = np.diff(ro0)[perm]
+        ro = np.zeros(M + 1, dtype=np.int32)
+        ro[1:] = np.cumsum(lens)
+        ci = np.concatenate([ci0[ro0[r]:ro0[r + 1]] for r in perm]).astype(np.int32) if ci0.size else ci0
+        structures.append((ro, ci))
+    ro_d, ci_d = dev(torch, structures[0][0]), dev(torch, structures[0][1])
+    nnz = ci_d.numel()
+    va = torch.randn(nnz, device="cuda")
+    B = torch.randn(K, N, device="cuda")
+    Q = torch.randn(M, N, device="cuda")
+    plan = torch.zeros(dl.row_plan_bytes(M) // 4, dtype=torch.int32, device="cuda")
+    C, S, O = torch.empty(M, N, device="cuda"), torch.empty(nnz, device="cuda"), torch.empty(M, N, device="cuda")
+    assert dl.row_plan_advice(dl.OP_SPMM, M, K, N, nnz, -1) and dl.row_plan_advice(dl.OP_FUSED, M, K, N, nnz, -1)
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        dl.row_plan(ro_d, out=plan)   # warm-up outside the capture
+        dl.spmm(ro_d, ci_d, va, B, K=K, out=C, plan=plan)
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            dl.row_plan(ro_d, out=plan)
+            dl.spmm(ro_d, ci_d, va, B, K=K, out=C, plan=plan)
+            dl.sddmm(ro_d, ci_d, Q, B, out=S, plan=plan)
+            dl.fused(ro_d, ci_d, Q, B, B, 0.5, out=O, plan=plan)
+    for rep, (ro, ci) in enumerate(structures + structures[:1]):
+        ro_d.copy_(dev(torch, ro))
+        ci_d.copy_(dev(torch, ci))
+        va.copy_(torch.randn(nnz, device="cuda"))
+        plan.fill_(-1)   # whatever the last build left must not matter
+        for buf in (C, S, O):
+            buf.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got_plan = plan.clone()
+        eager_plan = dl.row_plan(ro_d)
+        assert torch.equal(got_plan[:3 * M], eager_plan[:3 * M]), f"replay {rep}: plan"
+        assert torch.equal(C, dl.spmm(ro_d, ci_d, va, B, K=K, plan=eager_plan)), f"replay {rep}: SpMM"
+        assert torch.equal(S, dl.sddmm(ro_d, ci_d, Q, B, plan=eager_plan)), f"replay {rep}: SDDMM"
+        assert torch.equal(O, dl.fused(ro_d, ci_d, Q, B, B, 0.5, plan=eager_plan)), f"replay {rep}: fused"
+        assert oracle.rel_frobenius(C.cpu().numpy(), oracle.spmm(ro, ci, va.cpu().numpy(), B.cpu().numpy(), omp=True)) <= TOL
+        rows = got_plan[2 * M:3 * M].cpu().numpy()
+        assert np.array_equal(np.sort(rows), np.arange(M))
+
+
+def test_hint_bits_and_the_deprecated_constant(torch_cuda, dl):
+    """The even-rows hint as a bit of workspace_bytes (NULL workspace) and as the deprecated pointer constant select the
+    same launch and give the same bits; the *_planned entry points are the named calls with DLSPM_HINT_ROW_PLAN."""
+    import ctypes
+
+    torch = torch_cuda
+    rng = np.random.default_rng(5)
+    M, K, N = 4096, 1024, 128
+    ro, ci = random_csr(rng, M, K, "uniform", 0.2)
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    va = torch.randn(ci.size, device="cuda")
+    B = torch.randn(K, N, device="cuda")
+    assert dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size, rows_even=True)["R"] == 4 != dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size)["R"]
+    by_bit = dl.spmm(ro_d, ci_d, va, B, workspace=dl.ROWS_EVEN).clone()
+    by_constant = torch.empty_like(by_bit)
+    L, vp = dl.lib(), ctypes.c_void_p
+    st = L.spmm_csr_f32(M, K, N, ci.size, vp(ro_d.data_ptr()), vp(ci_d.data_ptr()), vp(va.data_ptr()), vp(B.data_ptr()),
+                        vp(by_constant.data_ptr()), vp(1), 0, vp(torch.cuda.current_stream().cuda_stream))
+    assert st == dl.OK
+    plain = dl.spmm(ro_d, ci_d, va, B)
+    assert torch.equal(by_bit, by_constant) and not torch.equal(by_bit, plain) and torch.allclose(by_bit, plain, rtol=1e-4, atol=1e-4)
+    plan = dl.row_plan(ro_d)
+    via_named = dl.spmm(ro_d, ci_d, va, B, plan=plan).clone()
+    via_alias = torch.empty_like(via_named)
+    st = L.spmm_csr_f32_planned(M, K, N, ci.size, vp(ro_d.data_ptr()), vp(ci_d.data_ptr()), vp(va.data_ptr()), vp(B.data_ptr()),
+                                vp(via_alias.data_ptr()), vp(plan.data_ptr()), plan.numel() * 4,
+                                vp(torch.cuda.current_stream().cuda_stream))
+    assert st == dl.OK and torch.equal(via_named, via_alias)
 
 
 def test_concurrent_calls_from_two_threads_on_two_streams(torch_cuda, dl, oracle):

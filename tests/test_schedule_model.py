@@ -37,6 +37,8 @@ def model():
     L.model_spmm_flat.restype = ci
     L.model_fused_flat.argtypes = [ci, ci, _i, _i, _f, _f, _f, ctypes.c_float, ci, ci, ci, ci, ci, _f, _f, _i]
     L.model_fused_flat.restype = ci
+    L.model_row_plan.argtypes = [ci, _i, ci, ci, _i]
+    L.model_row_plan.restype = None
     return L
 
 
@@ -293,7 +295,7 @@ FLAT_GPU = [("uniform", 300, 200, 256, 0, 128), ("skewed", 257, 129, 64, 0, 64),
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind,M,K,N,n_long,chunk", FLAT_GPU)
-def test_gpu_flat_spmm_equals_model_bit_for_bit(model, dl, monkeypatch, kind, M, K, N, n_long, chunk):
+def test_gpu_flat_spmm_equals_model_bit_for_bit(model, dl, kind, M, K, N, n_long, chunk):
     """The flat schedule (every wave owns `chunk` consecutive nonzeros; partial rows in the workspace, added by a second
     kernel), forced on small matrices and with small chunks so that rows are shared by many waves."""
     import torch
@@ -305,9 +307,7 @@ def test_gpu_flat_spmm_equals_model_bit_for_bit(model, dl, monkeypatch, kind, M,
         ro, ci = random_csr(rng, M, K, kind, 1.0 if kind == "full" else 0.2)
     va = rng.normal(0, 1, ci.size).astype(np.float32)
     B = rng.normal(0, 1, (K, N)).astype(np.float32)
-    monkeypatch.setenv("DLSPM_FLAT", "1")
-    monkeypatch.setenv("DLSPM_SLICES", "0")
-    monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
+    dl.set_tuning(flat=1, slices=0, flat_chunk=chunk)
     sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size, with_workspace=True)
     assert sh["flat_chunk"] == chunk and sh["flat_units"] == -(-ci.size // chunk)
     need = dl.workspace_bytes(dl.OP_SPMM, M, K, N, ci.size)
@@ -333,7 +333,7 @@ def test_gpu_flat_spmm_equals_model_bit_for_bit(model, dl, monkeypatch, kind, M,
 @pytest.mark.parametrize("kind,M,K,D,n_long,chunk", [("uniform", 300, 200, 64, 0, 128), ("long_and_empty", 1500, 700, 128, 3, 256),
                                                       ("skewed", 130, 257, 49, 0, 64), ("long_and_empty", 900, 600, 256, 2, 192),
                                                       ("uniform", 40, 300, 1027, 0, 320), ("empty_rows", 500, 100, 3, 0, 64)])
-def test_gpu_flat_fused_equals_model_bit_for_bit(model, dl, monkeypatch, kind, M, K, D, n_long, chunk):
+def test_gpu_flat_fused_equals_model_bit_for_bit(model, dl, kind, M, K, D, n_long, chunk):
     import torch
 
     rng = np.random.default_rng(51 + M + D)
@@ -344,9 +344,7 @@ def test_gpu_flat_fused_equals_model_bit_for_bit(model, dl, monkeypatch, kind, M
     Q = rng.normal(0, 1, (M, D)).astype(np.float32)
     Km = rng.normal(0, 1, (K, D)).astype(np.float32)
     V = rng.normal(0, 1, (K, D)).astype(np.float32)
-    monkeypatch.setenv("DLSPM_FLAT", "1")
-    monkeypatch.setenv("DLSPM_SLICES", "0")
-    monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
+    dl.set_tuning(flat=1, slices=0, flat_chunk=chunk)
     fs = dl.describe_launch(dl.OP_FUSED, M, K, D, ci.size)
     assert fs["flat_chunk"] == chunk
     need = dl.workspace_bytes(dl.OP_FUSED, M, K, D, ci.size)
@@ -369,7 +367,7 @@ def test_gpu_flat_fused_equals_model_bit_for_bit(model, dl, monkeypatch, kind, M
 @pytest.mark.parametrize("kind,M,K,D,n_long,chunk", [("uniform", 300, 200, 64, 0, 128), ("long_and_empty", 1500, 700, 128, 3, 256),
                                                       ("skewed", 130, 257, 49, 0, 64), ("long_and_empty", 5000, 600, 32, 5, 64),
                                                       ("uniform", 40, 300, 1027, 0, 320), ("empty_rows", 500, 100, 3, 0, 64)])
-def test_gpu_flat_sddmm_equals_model_and_the_row_block_schedule_bit_for_bit(model, dl, monkeypatch, kind, M, K, D, n_long, chunk):
+def test_gpu_flat_sddmm_equals_model_and_the_row_block_schedule_bit_for_bit(model, dl, kind, M, K, D, n_long, chunk):
     """SDDMM's flat schedule changes which wave computes a dot product, not how: both schedules must give the model's bits."""
     import torch
 
@@ -386,9 +384,7 @@ def test_gpu_flat_sddmm_equals_model_and_the_row_block_schedule_bit_for_bit(mode
     model.model_sddmm(M, D, pi(ro), pi(ci), pf(Q), pf(Km), sh["vec"], sh["G1"], sh["DS"], pf(ref))
     args = (dev(torch, ro), dev(torch, ci), dev(torch, Q), dev(torch, Km))
     block = dl.sddmm(*args).cpu().numpy()
-    monkeypatch.setenv("DLSPM_FLAT", "1")
-    monkeypatch.setenv("DLSPM_SLICES", "0")
-    monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
+    dl.set_tuning(flat=1, slices=0, flat_chunk=chunk)
     assert dl.describe_launch(dl.OP_SDDMM, M, K, D, ci.size)["flat_chunk"] == chunk
     assert dl.workspace_bytes(dl.OP_SDDMM, M, K, D, ci.size) == 0
     out = torch.full((ci.size,), float("nan"), dtype=torch.float32, device="cuda")
@@ -400,7 +396,7 @@ def test_gpu_flat_sddmm_equals_model_and_the_row_block_schedule_bit_for_bit(mode
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("seed", [1, 2, 3])
-def test_gpu_random_shapes_equal_model_bit_for_bit(model, dl, monkeypatch, seed):
+def test_gpu_random_shapes_equal_model_bit_for_bit(model, dl, seed):
     """Forty random (shape, pattern, width, schedule, chunk) draws per seed, all three entry points, bit for bit."""
     import torch
 
@@ -417,9 +413,7 @@ def test_gpu_random_shapes_equal_model_bit_for_bit(model, dl, monkeypatch, seed)
         nnz = ci.size
         flat = bool(rng.integers(0, 2)) and nnz > 0
         chunk = int(rng.choice([64, 128, 192, 320, 512, 1024]))
-        monkeypatch.setenv("DLSPM_FLAT", "1" if flat else "0")
-        monkeypatch.setenv("DLSPM_SLICES", "0")
-        monkeypatch.setenv("DLSPM_FLAT_CHUNK", str(chunk))
+        dl.set_tuning(flat=1 if flat else 0, slices=0, flat_chunk=chunk)
         tag = f"seed {seed} draw {it}: M {M} K {K} N {N} {kind} {density} nnz {nnz} flat {flat} chunk {chunk}"
         print(tag, flush=True)
         va = rng.normal(0, 1, max(nnz, 1)).astype(np.float32)
@@ -493,7 +487,7 @@ SLICED_CASES = [("uniform", 300, 512, 128, 3), ("skewed", 1100, 700, 256, 2), ("
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind,M,K,N,slices", SLICED_CASES)
-def test_gpu_sliced_spmm_equals_model_bit_for_bit(model, dl, oracle, monkeypatch, kind, M, K, N, slices):
+def test_gpu_sliced_spmm_equals_model_bit_for_bit(model, dl, oracle, kind, M, K, N, slices):
     """Column-sliced SpMM = the row-block kernel's arithmetic on each column range of the matrix (the model, run on
     that range's own CSR arrays with the split the library reports), the ranges' partial rows added in range order."""
     import torch
@@ -506,7 +500,7 @@ def test_gpu_sliced_spmm_equals_model_bit_for_bit(model, dl, oracle, monkeypatch
     va = rng.normal(0, 1, ci.size).astype(np.float32)
     B = rng.normal(0, 1, (K, N)).astype(np.float32)
     assert dl.describe_slices(dl.OP_SPMM, M, K, N, ci.size)[0] == 0       # far too small for the rule
-    monkeypatch.setenv("DLSPM_SLICES", str(slices))
+    dl.set_tuning(slices=slices)
     got_slices, R = dl.describe_slices(dl.OP_SPMM, M, K, N, ci.size)
     assert got_slices == slices and R in (1, 2, 4, 8, 16)
     sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size, with_workspace=True)
@@ -537,7 +531,7 @@ def test_gpu_sliced_spmm_equals_model_bit_for_bit(model, dl, oracle, monkeypatch
                                                ("long_and_empty", 900, 600, 100, 4), ("empty_rows", 200, 300, 512, 5),
                                                ("uniform", 150, 400, 200, 16), ("skewed", 500, 700, 64, 3),
                                                ("uniform", 300, 200, 24, 4)])
-def test_gpu_sliced_fused_equals_model_bit_for_bit(model, dl, oracle, monkeypatch, kind, M, K, D, slices):
+def test_gpu_sliced_fused_equals_model_bit_for_bit(model, dl, oracle, kind, M, K, D, slices):
     import torch
 
     rng = np.random.default_rng(81 + M + D)
@@ -548,7 +542,7 @@ def test_gpu_sliced_fused_equals_model_bit_for_bit(model, dl, oracle, monkeypatc
     Q = rng.normal(0, 1, (M, D)).astype(np.float32)
     Km = rng.normal(0, 1, (K, D)).astype(np.float32)
     V = rng.normal(0, 1, (K, D)).astype(np.float32)
-    monkeypatch.setenv("DLSPM_SLICES", str(slices))
+    dl.set_tuning(slices=slices)
     got_slices, R = dl.describe_slices(dl.OP_FUSED, M, K, D, ci.size)
     assert got_slices == slices
     fs = dl.describe_launch(dl.OP_FUSED, M, K, D, ci.size)
@@ -575,7 +569,7 @@ def test_gpu_sliced_fused_equals_model_bit_for_bit(model, dl, oracle, monkeypatc
 
 
 @pytest.mark.gpu
-def test_gpu_sliced_schedule_does_not_need_ascending_columns(dl, oracle, monkeypatch):
+def test_gpu_sliced_schedule_does_not_need_ascending_columns(dl, oracle):
     """The slice boundaries are found by a search that assumes ascending columns; with any other order they are still
     a partition of every row (a running maximum), so the result stays right."""
     import torch
@@ -588,7 +582,7 @@ def test_gpu_sliced_schedule_does_not_need_ascending_columns(dl, oracle, monkeyp
         rng.shuffle(ci[ro[i]:ro[i + 1]])
     va = rng.normal(0, 1, ci.size).astype(np.float32)
     B = rng.normal(0, 1, (K, N)).astype(np.float32)
-    monkeypatch.setenv("DLSPM_SLICES", "4")
+    dl.set_tuning(slices=4)
     need = dl.workspace_bytes(dl.OP_SPMM, M, K, N, ci.size)
     ws = torch.empty(need // 4, dtype=torch.float32, device="cuda")
     got = dl.spmm(dev(torch, ro), dev(torch, ci), dev(torch, va), dev(torch, B), K=K, workspace=ws).cpu().numpy()
@@ -607,7 +601,7 @@ def test_gpu_sliced_schedule_does_not_need_ascending_columns(dl, oracle, monkeyp
                                                ("long_and_empty", 900, 600, 100, 4), ("empty_rows", 200, 300, 512, 5),
                                                ("full", 60, 256, 65, 16), ("skewed", 500, 700, 64, 3),
                                                ("uniform", 300, 200, 20, 4)])
-def test_gpu_sliced_sddmm_gives_the_same_bits(dl, oracle, monkeypatch, kind, M, K, D, slices):
+def test_gpu_sliced_sddmm_gives_the_same_bits(dl, oracle, kind, M, K, D, slices):
     """Every SDDMM result is one dot product computed by one lane group in a fixed order, whatever the schedule: the
     column-sliced call must reproduce the plain call bit for bit, and leave no slot unwritten."""
     import torch
@@ -622,7 +616,7 @@ def test_gpu_sliced_sddmm_gives_the_same_bits(dl, oracle, monkeypatch, kind, M, 
     args = (dev(torch, ro), dev(torch, ci), dev(torch, Q), dev(torch, Km))
     plain = dl.sddmm(*args)
     assert dl.workspace_bytes(dl.OP_SDDMM, M, K, D, ci.size) == 0
-    monkeypatch.setenv("DLSPM_SLICES", str(slices))
+    dl.set_tuning(slices=slices)
     assert dl.describe_slices(dl.OP_SDDMM, M, K, D, ci.size)[0] == slices
     need = dl.workspace_bytes(dl.OP_SDDMM, M, K, D, ci.size)
     assert need >= (slices + 1) * M * 4
@@ -636,3 +630,70 @@ def test_gpu_sliced_sddmm_gives_the_same_bits(dl, oracle, monkeypatch, kind, M, 
         dl.sddmm(*args, out=out, workspace=ws[: need // 4 - 1])
     assert e.value.status == dl.E_WORKSPACE
 
+
+
+# ---- row plan: the device build against its sequential definition ---------------------------------------------------
+def model_plan(L, ro, bins, order=0):
+    M = ro.size - 1
+    plan = np.empty(3 * M, dtype=np.int32)
+    L.model_row_plan(M, pi(np.ascontiguousarray(ro, dtype=np.int32)), bins, order, pi(plan))
+    return plan
+
+
+def test_model_row_plan_is_a_balanced_permutation(model, dl):
+    """CPU: the sequential definition of the plan. Every row once, with its own offsets; the first 2048 positions in
+    256 bins whose loads differ far less than in matrix order; rows without nonzeros last in their bins."""
+    c = dl.make_config(2)
+    ro = c["row_offsets"]
+    M = ro.size - 1
+    plan = model_plan(model, ro, 256)
+    starts, ends, rows = plan[:M], plan[M:2 * M], plan[2 * M:]
+    assert np.array_equal(np.sort(rows), np.arange(M))
+    assert np.array_equal(starts, ro[rows]) and np.array_equal(ends, ro[rows + 1])
+    lens = np.diff(ro)
+    packed = np.array([lens[rows[b::256]].sum() for b in range(256)])
+    plain = np.array([lens[b::256].sum() for b in range(256)])
+    assert packed.max() <= 1.1 * packed.mean() < 0.75 * plain.max()
+    # the two simpler orders
+    desc = model_plan(model, ro, 256, 2)[2 * M:]
+    assert (np.diff(lens[desc]) <= 0).all()
+    alt = model_plan(model, ro, 256, 1)[2 * M:]
+    assert np.array_equal(alt[:256], desc[:256]) and np.array_equal(alt[256:512], desc[256:512][::-1])
+    # rows without nonzeros take what is left, in order
+    ro2 = np.zeros(11, dtype=np.int32)
+    ro2[1:] = np.cumsum([5, 0, 3, 0, 0, 9, 1, 0, 2, 2])
+    assert model_plan(model, ro2, 4)[20:].tolist() == [5, 0, 2, 8, 1, 3, 6, 9, 4, 7]
+
+
+PLAN_CASES = [("cfg2", 0, 0), ("skewed", 1, 60), ("skewed", 2, 60), ("uniform", 7, 33), ("skewed", 255, 400), ("skewed", 256, 400),
+              ("empty_rows", 257, 300), ("skewed", 2047, 512), ("empty_rows", 2048, 700), ("skewed", 2049, 512),
+              ("empty", 1500, 64), ("full", 900, 37), ("skewed", 5000, 2048), ("empty_rows", 20000, 256),
+              ("skewed", 70001, 128), ("uniform", 300000, 64)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,M,K", PLAN_CASES)
+def test_gpu_row_plan_equals_its_sequential_definition(model, dl, kind, M, K):
+    """dlspm_row_plan_build builds the plan with kernels (tile sort, merge passes, batched packing); every entry must
+    equal the sequential host definition, for every order, from one row to 300000 (one launch up to 2048 rows, tiles
+    and merges beyond), with empty rows, equal rows and rows of one length only."""
+    import torch
+
+    if kind == "cfg2":
+        ro = dl.make_config(2)["row_offsets"]
+        M = ro.size - 1
+    else:
+        ro, _ = random_csr(np.random.default_rng(M + K), M, K, kind, 0.15)
+    info = dl.device_info()
+    assert info["status"] == dl.OK and info["gfx950"] and info["compute_units"] > 0 and info["l2_bytes"] >= 1 << 20
+    bins = min(info["compute_units"], 256)
+    ro_d = dev(torch, ro)
+    for order in (0, 1, 2):
+        dl.set_tuning(plan_order=order)
+        plan = torch.full((dl.row_plan_bytes(M) // 4,), -7, dtype=torch.int32, device="cuda")
+        dl.row_plan(ro_d, out=plan)
+        got = plan.cpu().numpy()[:3 * M]
+        want = model_plan(model, ro, bins, order)
+        assert np.array_equal(got, want), (kind, M, K, order, np.flatnonzero(got != want)[:10])
+    dl.set_tuning()
+    assert np.array_equal(ro_d.cpu().numpy(), ro)
