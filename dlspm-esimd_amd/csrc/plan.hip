@@ -28,6 +28,7 @@ namespace {
 constexpr int kPlanTile = 2048;     // rows sorted by one workgroup; also the most rows a head can hold
 constexpr int kPlanThreads = 1024;  // one compare-exchange per thread and stage
 constexpr int kPlanMaxBins = 256;   // 8 x bins <= kPlanTile
+static_assert(kPlanThreads == 4 * kPlanMaxBins, "the packing counts with four threads per bin");
 constexpr int kHeadPerBin = 8;      // workgroups of a four-wave kernel that a compute unit holds at once
 
 typedef unsigned long long u64;
@@ -40,8 +41,11 @@ __device__ __forceinline__ u64 plan_key(const int* __restrict__ row_offsets, int
 __device__ __forceinline__ int key_len(u64 key) { return (int)(key >> 32); }
 __device__ __forceinline__ int key_row(u64 key) { return (int)(0xFFFFFFFFu - (unsigned)(key & 0xFFFFFFFFu)); }
 
-// s_key[0 .. n) sorted descending, n a power of two <= kPlanTile, by the whole workgroup
-__device__ void sort_tile_desc(u64* s_key, int n)
+// s_key[0 .. n) sorted descending, n a power of two <= kPlanTile, by the whole workgroup (a bitonic network, one
+// compare-exchange per thread and stage). Thread t's pair of a stage with distance j < 128 lies inside the 128 keys
+// that its own wave works on in every such stage, and a wave's LDS accesses execute in order: those stages need no
+// workgroup barrier, only the stages that exchange keys between waves do (15 barriers instead of 66 for 2048 keys).
+__device__ __forceinline__ void sort_tile_desc(u64* s_key, int n)
 {
     const int t = threadIdx.x;
     for (int k = 2; k <= n; k <<= 1) {
@@ -55,26 +59,137 @@ __device__ void sort_tile_desc(u64* s_key, int n)
                     s_key[i + j] = a;
                 }
             }
-            __syncthreads();
+            // the next stage has distance j / 2, or k (the first stage of the next round) after j == 1
+            const int next = j > 1 ? j >> 1 : (k < n ? k : kPlanTile);
+            if (j >= 128 || next >= 128) __syncthreads();
+            else __builtin_amdgcn_wave_barrier();  // same wave, same 128 keys: program order is enough
         }
     }
 }
 
-struct PackShared {
-    u64 bkey[kPlanMaxBins];   // (load, bin) of a bin that can still take a row, else all ones
-    u64 skey[kPlanMaxBins];   // the same, sorted ascending
-    int sbin[kPlanMaxBins];   // bin at each sorted position
-    int load[kPlanMaxBins];   // nonzeros handed to a bin so far
-    int cnt[kPlanMaxBins];    // rows handed to a bin so far
-    int wave_free[kPlanThreads / 64];
-    int nz;                   // head rows that have nonzeros (they come first in the sorted order)
-    int batch;                // rows placed by the current batch
-    int base;
+// (load, bin) of a bin as one sortable word: 32 bits while every load stays below 2^24 (bins <= 256), else 64
+template <typename Word> struct BinKey;
+template <> struct BinKey<unsigned> {
+    static constexpr unsigned none = 0xFFFFFFFFu;
+    static __device__ __forceinline__ unsigned make(int load, int bin) { return ((unsigned)load << 8) | (unsigned)bin; }
 };
+template <> struct BinKey<u64> {
+    static constexpr u64 none = ~0ull;
+    static __device__ __forceinline__ u64 make(int load, int bin) { return ((u64)(unsigned)load << 32) | (u64)bin; }
+};
+
+struct PackShared {
+    alignas(16) u64 bkey[kPlanMaxBins];  // (load, bin) of a bin that can still take a row, else all ones (32-bit words: the first half)
+    int wave_min[kPlanThreads / 64];     // per wave: where its bins would end the batch
+    int wave_room[kPlanThreads / 64];    // per wave: bins that can still take a row
+    int wave_free[kPlanThreads / 64];
+    int nz;                              // head rows that have nonzeros (they come first in the sorted order)
+};
+
+// sum over the four lanes of a quad, in every lane of it
+__device__ __forceinline__ int quad_sum(int x)
+{
+    x += __builtin_amdgcn_update_dpp(0, x, kDppQuadSwap1, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0, x, kDppQuadSwap2, 0xF, 0xF, true);
+    return x;
+}
+// minimum over the wave, in every lane (all lanes active)
+__device__ __forceinline__ int wave_min(int x)
+{
+    x = min(x, __builtin_amdgcn_update_dpp(x, x, kDppQuadSwap1, 0xF, 0xF, false));
+    x = min(x, __builtin_amdgcn_update_dpp(x, x, kDppQuadSwap2, 0xF, 0xF, false));
+    x = min(x, __builtin_amdgcn_update_dpp(x, x, kDppRowHalfMirror, 0xF, 0xF, false));
+    x = min(x, __builtin_amdgcn_update_dpp(x, x, kDppRowMirror, 0xF, 0xF, false));
+    const auto a = __builtin_amdgcn_permlane16_swap((unsigned)x, (unsigned)x, false, false);
+    x = min((int)a[0], (int)a[1]);
+    const auto b = __builtin_amdgcn_permlane32_swap((unsigned)x, (unsigned)x, false, false);
+    return min((int)b[0], (int)b[1]);
+}
+
+// How many of the kPlanMaxBins keys lie below x, summed over the four lanes of a quad: lane q of the quad looks at the
+// 16-byte chunks q, q + 4, q + 8, ... of the key array (neighbouring lanes read neighbouring chunks: no bank conflicts).
+__device__ __forceinline__ int count_below(const unsigned* keys, int q, unsigned x)
+{
+    const uint4* chunk = reinterpret_cast<const uint4*>(keys);
+    int n = 0;
+#pragma unroll
+    for (int j = 0; j < kPlanMaxBins / 16; ++j) {
+        const uint4 k = chunk[4 * j + q];
+        n += (k.x < x ? 1 : 0) + (k.y < x ? 1 : 0) + (k.z < x ? 1 : 0) + (k.w < x ? 1 : 0);
+    }
+    return quad_sum(n);
+}
+__device__ __forceinline__ int count_below(const u64* keys, int q, u64 x)
+{
+    const ulonglong2* chunk = reinterpret_cast<const ulonglong2*>(keys);
+    int n = 0;
+#pragma unroll
+    for (int j = 0; j < kPlanMaxBins / 8; ++j) {
+        const ulonglong2 k = chunk[4 * j + q];
+        n += (k.x < x ? 1 : 0) + (k.y < x ? 1 : 0);
+    }
+    return quad_sum(n);
+}
+
+// The packing proper: rows 0 .. nz-1 of the sorted head (those with nonzeros), longest first, each into the least loaded
+// bin that has room (ties: the lower bin). In batches: with the bins ranked by (load, bin), the next rows go to the bins
+// in rank order for as long as no bin that already received a row of this batch would have been the least loaded one
+// again, i.e. up to the smallest number of keys below any participating bin's key AFTER its new row. Both steps are
+// "how many of the 256 keys lie below x", counted by the four lanes of a quad per bin, a quarter of the keys each; lane
+// 0 of the quad keeps the bin's books. Two workgroup barriers per batch.
+template <typename Word>
+__device__ __forceinline__ void pack_batches(const u64* s_key, int head, int nz, int bins, int* s_order, PackShared& sh)
+{
+    using Key = BinKey<Word>;
+    Word* bkey = reinterpret_cast<Word*>(sh.bkey);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bin = tid >> 2, q = tid & 3;  // kPlanThreads = 4 x kPlanMaxBins
+    const bool owner = q == 0 && bin < bins;
+    int load = 0, cnt = 0;  // the bin's books, kept by its owner lane
+    bool room = owner && bin < head;
+    if (q == 0) bkey[bin] = room ? Key::make(0, bin) : Key::none;  // empty bins; beyond `bins`: padding
+    unsigned long long rooms = __ballot(room);
+    if (lane == 0) sh.wave_room[wave] = __popcll(rooms);
+    __syncthreads();
+    int t = 0;  // rows placed so far; the same in every thread
+    while (t < nz) {
+        int with_room = 0;
+#pragma unroll
+        for (int x = 0; x < kPlanThreads / 64; ++x) with_room += sh.wave_room[x];
+        const int most = min(with_room, nz - t);  // >= 1: t < nz <= head rows are unplaced, so some bin has room
+        const Word mine = bkey[bin];
+        const int rank = count_below(bkey, q, mine);
+        const bool takes = mine != Key::none && rank < most;  // row t + rank would go to this bin
+        const int len = takes ? key_len(s_key[t + rank]) : 0;
+        const int load_now = __builtin_amdgcn_update_dpp(0, load, 0x00, 0xF, 0xF, true);  // quad_perm [0,0,0,0]: the owner's
+        const Word after = takes ? Key::make(load_now + len, bin) : Key::none;
+        // the batch ends before the first rank whose bin is no longer below an earlier bin of the batch with its new row
+        const int ends = takes ? count_below(bkey, q, after) : 0x7fffffff;
+        const int wave_ends = wave_min(ends);
+        if (lane == 0) sh.wave_min[wave] = wave_ends;
+        __syncthreads();
+        int batch = most;  // 1 <= batch <= most
+#pragma unroll
+        for (int x = 0; x < kPlanThreads / 64; ++x) batch = min(batch, sh.wave_min[x]);
+        if (owner) {
+            if (takes && rank < batch) {
+                s_order[cnt * bins + bin] = t + rank;
+                load += len;
+                cnt += 1;
+            }
+            room = cnt * bins + bin < head;  // the bin's next workgroup exists
+            bkey[bin] = room ? Key::make(load, bin) : Key::none;
+        }
+        rooms = __ballot(owner && room);
+        if (lane == 0) sh.wave_room[wave] = __popcll(rooms);
+        __syncthreads();
+        t += batch;
+    }
+}
 
 // s_order[p] <- which of the sorted rows 0 .. head-1 workgroup p of the head works on. order: 0 packed (above),
 // 1 groups of `bins` alternating between descending and ascending length, 2 plainly descending.
-__device__ void pack_head(const u64* s_key, int head, int bins, int order, int* s_order, PackShared& sh)
+__device__ __forceinline__ void pack_head(const u64* s_key, int head, int bins, int order, int* s_order, PackShared& sh)
 {
     const int tid = threadIdx.x;
     if (order != 0) {
@@ -86,66 +201,15 @@ __device__ void pack_head(const u64* s_key, int head, int bins, int order, int* 
         return;
     }
     for (int p = tid; p < head; p += kPlanThreads) s_order[p] = -1;
-    if (tid < bins) {
-        sh.load[tid] = 0;
-        sh.cnt[tid] = 0;
-    }
     if (tid == 0) sh.nz = 0;
     __syncthreads();
     for (int p = tid; p < head; p += kPlanThreads)  // the last row with nonzeros (lengths descend)
         if (key_len(s_key[p]) > 0 && (p + 1 == head || key_len(s_key[p + 1]) == 0)) sh.nz = p + 1;
     __syncthreads();
     const int nz = sh.nz;
-    int t = 0;  // rows placed so far; the same in every thread
-    while (t < nz) {
-        if (tid < bins) {
-            const bool room = sh.cnt[tid] * bins + tid < head;  // the bin's next workgroup exists
-            sh.bkey[tid] = room ? ((u64)(unsigned)sh.load[tid] << 32) | (u64)tid : ~0ull;
-        }
-        if (tid == 0) sh.batch = 0x7fffffff;
-        __syncthreads();
-        int with_room = 0;
-        if (tid < bins) {  // position of this bin among the bins by (load, bin), and how many bins have room
-            const u64 mine = sh.bkey[tid];
-            int rank = 0;
-            for (int k = 0; k < bins; ++k) {
-                const u64 other = sh.bkey[k];
-                rank += other < mine ? 1 : 0;
-                with_room += other != ~0ull ? 1 : 0;
-            }
-            if (mine != ~0ull) {
-                sh.sbin[rank] = tid;
-                sh.skey[rank] = mine;
-            }
-        }
-        if (tid == 0) sh.base = with_room;
-        __syncthreads();
-        const int most = min(sh.base, nz - t);  // >= 1: t < nz <= head rows are unplaced, so some bin has room
-        if (tid < most) {
-            // Row t + tid would go to the bin at sorted position tid. That holds as long as no earlier bin of this
-            // batch, with its new row, is again below a later bin: this bin ends the batch at the first later
-            // position whose (load, bin) is not below its own new (load + length, bin).
-            const int b = sh.sbin[tid];
-            const u64 after = ((u64)(unsigned)(sh.load[b] + key_len(s_key[t + tid])) << 32) | (u64)b;
-            int lo = tid + 1, hi = most;
-            while (lo < hi) {
-                const int mid = (lo + hi) >> 1;
-                if (sh.skey[mid] < after) lo = mid + 1;
-                else hi = mid;
-            }
-            atomicMin(&sh.batch, lo);
-        }
-        __syncthreads();
-        const int batch = sh.batch;  // 1 <= batch <= most
-        if (tid < batch) {
-            const int b = sh.sbin[tid];
-            s_order[sh.cnt[b] * bins + b] = t + tid;
-            sh.load[b] += key_len(s_key[t + tid]);
-            sh.cnt[b] += 1;
-        }
-        __syncthreads();
-        t += batch;
-    }
+    // a bin holds at most kHeadPerBin rows, none longer than the first: 32-bit (load, bin) words while that fits 24 bits
+    if ((long long)key_len(s_key[0]) * kHeadPerBin < (1ll << 24)) pack_batches<unsigned>(s_key, head, nz, bins, s_order, sh);
+    else pack_batches<u64>(s_key, head, nz, bins, s_order, sh);
     // rows without nonzeros: the positions still free, in ascending order, take the sorted rows nz, nz + 1, ...
     const int lane = tid & 63, wave = tid >> 6;
     int next = nz;
