@@ -25,6 +25,14 @@ template <> struct Vec<4> {
         const float4_dword_aligned t = *reinterpret_cast<const float4_dword_aligned*>(p);
         return Vec{make_float4(t.x, t.y, t.z, t.w)};
     }
+    // the same through a buffer descriptor: base + per-lane byte offset + wave-uniform byte offset, all 32-bit, summed
+    // by the load itself (no address arithmetic in the wave's instruction stream)
+    __device__ __forceinline__ static Vec bload(__amdgpu_buffer_rsrc_t rsrc, unsigned lane_bytes, unsigned row_bytes)
+    {
+        typedef unsigned u4 __attribute__((ext_vector_type(4)));
+        const u4 t = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_bytes, row_bytes, 0);
+        return Vec{make_float4(__uint_as_float(t.x), __uint_as_float(t.y), __uint_as_float(t.z), __uint_as_float(t.w))};
+    }
     __device__ __forceinline__ void gstore(float* p) const
     {
         float4_dword_aligned t = {v.x, v.y, v.z, v.w};
@@ -59,6 +67,10 @@ template <> struct Vec<1> {
     __device__ __forceinline__ static Vec load(const float* p) { return Vec{*p}; }
     __device__ __forceinline__ void store(float* p) const { *p = v; }
     __device__ __forceinline__ static Vec gload(const float* p) { return Vec{*p}; }
+    __device__ __forceinline__ static Vec bload(__amdgpu_buffer_rsrc_t rsrc, unsigned lane_bytes, unsigned row_bytes)
+    {
+        return Vec{__uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, lane_bytes, row_bytes, 0))};
+    }
     __device__ __forceinline__ void gstore(float* p) const { *p = v; }
     __device__ __forceinline__ static Vec gload_clip(const float* row, int d, int) { return Vec{row[d]}; }
     __device__ __forceinline__ void fma(float a, const Vec& b) { v = fmaf(a, b.v, v); }
@@ -234,13 +246,21 @@ struct RowBlock {
     bool aligned;          // the row-aligned split is in use (the same for every wave of the workgroup)
 
     // `prefetch()` is called right after the offsets were requested: what it asks for arrives in the same round trip
+    // `xcd_contiguous` (plain row blocks in one column tile only): workgroup 8 i + x runs on XCD x, as the hardware deals
+    // them; it then takes row block i of XCD x's own contiguous run of row blocks instead of row block 8 i + x.
     template <typename Prefetch>
     __device__ __forceinline__ void load(int rb, int M, int nnz, const int* __restrict__ row_offsets,
                                          const int* __restrict__ row_ends, const int* __restrict__ row_ids,
-                                         Prefetch&& prefetch)
+                                         Prefetch&& prefetch, int xcd_contiguous = 0)
     {
         lane = threadIdx.x & 63;
         w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        if constexpr (!SLICED && !PLANNED) {
+            if (xcd_contiguous) {
+                const int nb = (M - 1) / R + 1, x = rb & 7, each = nb >> 3, extra = nb & 7;
+                rb = x * each + min(x, extra) + (rb >> 3);  // XCD x owns each + (x < extra) row blocks
+            }
+        }
         const int r0 = rb * R;
         nr = PLANNED ? 1 : min(R, M - r0);
         row0 = r0;
@@ -501,21 +521,42 @@ __device__ __forceinline__ int window_next_row(const int* __restrict__ row_offse
 }
 
 // ---- dense-row accumulation (SpMM kernel and stage 2 of the fused kernel) -----------------------------
+// A dense operand of fewer than 4 GiB as a raw buffer (stride 0, no swizzle, 32-bit data format): the descriptor that
+// buffer loads take. Their address is base + lane offset + wave-uniform offset, so a row of B needs one scalar multiply
+// (column x row pitch) where a global load needs a 64-bit multiply, shift and add on the scalar unit plus a 64-bit add
+// per access on the vector unit.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t dense_buffer(const float* p)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p), 0, -1, 0x00020000);
+}
+
 // The wave holds `cnt` <= 64 nonzeros of one row segment, one per lane: column index `c` and value `av`
 // (lanes >= cnt hold c = 0, av = 0). Adds sum_j av_j * dense[c_j, colv[v] .. colv[v]+VEC) into acc[v].
 // G lanes cover one dense row; the S = 64/G lane groups ("slots") take different nonzeros j = t*S + slot.
 // Loads are issued U dense rows at a time before the first FMA so that U*V requests per lane are in
 // flight. `colv` must be a valid column for every lane (lanes outside the matrix pass a safe column and
 // simply never store their accumulator), so the loop body has no predicates.
-template <int VEC, int G, int V>
+// BUF (G == 64 only, dense operand below 4 GiB): the rows are read with buffer loads (dense_buffer above).
+template <int VEC, int G, int V, bool BUF = false>
 __device__ __forceinline__ void dense_rows_fma(Vec<VEC>* acc, int c, float av, int cnt, const float* __restrict__ dense,
                                                int ld, const int* colv, int lane)
 {
     using VecT = Vec<VEC>;
     constexpr int S = kWave / G;
+    static_assert(!BUF || S == 1, "buffer loads take a wave-uniform row offset");
     constexpr int U = V >= 4 ? 2 : 8 / V;
     const int slot = lane / G;
     const int full = cnt / S;  // steps in which every slot has a nonzero
+    unsigned offv[V];  // BUF: the lane's columns as byte offsets into a dense row
+#pragma unroll
+    for (int v = 0; v < V; ++v) offv[v] = (unsigned)colv[v] * (unsigned)sizeof(float);
+    const unsigned pitch = (unsigned)ld * (unsigned)sizeof(float);
+    const __amdgpu_buffer_rsrc_t rsrc = dense_buffer(dense);
+    // dense row cj, access v of this lane
+    auto row_load = [&](int cj, int v) -> VecT {
+        if constexpr (BUF) return VecT::bload(rsrc, offv[v], (unsigned)cj * pitch);
+        else return VecT::gload(dense + (size_t)cj * ld + colv[v]);
+    };
     int t = 0;
     for (; t + U <= full; t += U) {
         VecT bv[U][V];
@@ -530,9 +571,8 @@ __device__ __forceinline__ void dense_rows_fma(Vec<VEC>* acc, int c, float av, i
                 cj = lane_get(c, (t + u) * S + slot);
                 aj[u] = lane_get(av, (t + u) * S + slot);
             }
-            const float* row = dense + (size_t)cj * ld;
 #pragma unroll
-            for (int v = 0; v < V; ++v) bv[u][v] = VecT::gload(row + colv[v]);
+            for (int v = 0; v < V; ++v) bv[u][v] = row_load(cj, v);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
@@ -554,9 +594,8 @@ __device__ __forceinline__ void dense_rows_fma(Vec<VEC>* acc, int c, float av, i
                     cj = lane_get(c, (t + u) * S + slot);
                     aj[u] = lane_get(av, (t + u) * S + slot);
                 }
-                const float* row = dense + (size_t)cj * ld;
 #pragma unroll
-                for (int v = 0; v < V; ++v) bv[u][v] = VecT::gload(row + colv[v]);
+                for (int v = 0; v < V; ++v) bv[u][v] = row_load(cj, v);
             }
         }
 #pragma unroll
@@ -572,10 +611,9 @@ __device__ __forceinline__ void dense_rows_fma(Vec<VEC>* acc, int c, float av, i
             const int jj = full * S + slot;
             const int cj = lane_get(c, jj & 63);  // lanes >= cnt hold column 0: a valid row, result unused
             const float aj = lane_get(av, jj & 63);
-            const float* row = dense + (size_t)cj * ld;
             VecT bv[V];
 #pragma unroll
-            for (int v = 0; v < V; ++v) bv[v] = VecT::gload(row + colv[v]);
+            for (int v = 0; v < V; ++v) bv[v] = row_load(cj, v);
             if (jj < cnt) {
 #pragma unroll
                 for (int v = 0; v < V; ++v) acc[v].fma(aj, bv[v]);

@@ -62,13 +62,15 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
                                             const int* __restrict__ row_offsets, const int* __restrict__ row_ends,
                                             const int* __restrict__ col_indices, const float* __restrict__ Q,
                                             const float* __restrict__ Kmat, const float* __restrict__ Vmat,
-                                            float* __restrict__ O, const int* __restrict__ row_ids = nullptr, int nnz = 0)
+                                            float* __restrict__ O, const int* __restrict__ row_ids = nullptr, int nnz = 0,
+                                            int xcd_contiguous = 0)
 {
     const int row_blocks = (M - 1) / R + 1;
     const int ct = col_tiles == 1 ? 0 : bid / row_blocks;
     const int rb = bid - ct * row_blocks;
     RowBlock<W, R, SLICED, PLANNED> blk;
-    blk.load(rb, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, Q, Kmat, Vmat, O); });
+    blk.load(rb, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, Q, Kmat, Vmat, O); },
+             col_tiles == 1 ? xcd_contiguous : 0);
     dense_rows_block<VEC, G, V2>(blk, ct, D, O, [&](Vec<VEC>* acc, int r, int p, int q, const int* colv) {
         const float* q_row = Q + (size_t)(blk.row0 + r) * D;
         fused_segment<VEC, G1, DS, MASKED, G, V2>(acc, p, q, D, scale, col_indices, q_row, Kmat, Vmat, colv, blk.lane);
@@ -77,14 +79,14 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
 
 // MASKED = false: D == G1 * VEC * DS exactly, every stage-1 access of every lane falls inside the row.
 template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R>
-__global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_tiles, float scale,
+__global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_tiles, int xcd_contiguous, float scale,
                                                        const int* __restrict__ row_offsets,
                                                        const int* __restrict__ col_indices,
                                                        const float* __restrict__ Q, const float* __restrict__ Kmat,
                                                        const float* __restrict__ Vmat, float* __restrict__ O)
 {
     fused_block<VEC, G1, DS, MASKED, G, V2, W, R, false>((int)blockIdx.x, M, D, col_tiles, scale, row_offsets, nullptr,
-                                                         col_indices, Q, Kmat, Vmat, O);
+                                                         col_indices, Q, Kmat, Vmat, O, nullptr, 0, xcd_contiguous);
 }
 
 // Column-sliced schedule (see spmm_sliced_kernel): the row blocks once per slice of columns, slice after slice, so
@@ -132,13 +134,14 @@ static hipError_t launch_one(const FusedArgs& x, hipStream_t stream)
     if constexpr (DS > 0) {
         if (x.D == G1 * VEC * DS) {
             hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, false, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64),
-                               0, stream, x.M, x.D, col_tiles, x.scale, x.row_offsets, x.col_indices, x.Q, x.Kmat, x.V,
-                               x.O);
+                               0, stream, x.M, x.D, col_tiles, tuning().xcd_contiguous, x.scale, x.row_offsets, x.col_indices,
+                               x.Q, x.Kmat, x.V, x.O);
             return hipGetLastError();
         }
     }
     hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, true, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream,
-                       x.M, x.D, col_tiles, x.scale, x.row_offsets, x.col_indices, x.Q, x.Kmat, x.V, x.O);
+                       x.M, x.D, col_tiles, tuning().xcd_contiguous, x.scale, x.row_offsets, x.col_indices, x.Q, x.Kmat, x.V,
+                       x.O);
     return hipGetLastError();
 }
 

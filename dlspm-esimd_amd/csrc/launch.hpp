@@ -8,6 +8,9 @@ namespace dlspm {
 // ceil(a / b) without the overflow of (a + b - 1) for a near INT_MAX
 inline long long ceil_div(long long a, long long b) { return (a + b - 1) / b; }
 
+// A dense operand of `rows` x `width` floats can be read through a buffer descriptor (32-bit byte offsets)
+inline bool dense_fits_buffer(long long rows, long long width) { return rows * width * 4 < (1ll << 32); }
+
 // The device the calling thread has current, as far as the launch rules need it: compute units and the size of one
 // L2. Read from hipDeviceProp_t once per device and cached; without a device (host-only queries on a machine that has
 // none) the figures of a whole MI355X: 256 compute units, 4 MiB.
@@ -27,6 +30,7 @@ struct Tuning {
     int slices = -1;
     int tile_major = -1, tile_width = 0;
     int plan_order = 0;
+    int xcd_contiguous = 0;
 };
 const Tuning& tuning();
 

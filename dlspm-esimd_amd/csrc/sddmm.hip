@@ -54,10 +54,11 @@ template <int VEC, int G1, int DS, bool MASKED, int W, int R, bool SLICED, bool 
 __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __restrict__ row_offsets,
                                             const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                             const float* __restrict__ lhs, const float* __restrict__ rhs,
-                                            float* __restrict__ out, const int* __restrict__ row_ids = nullptr, int nnz = 0)
+                                            float* __restrict__ out, const int* __restrict__ row_ids = nullptr, int nnz = 0,
+                                            int xcd_contiguous = 0)
 {
     RowBlock<W, R, SLICED, PLANNED> blk;
-    blk.load(bid, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, lhs, rhs, out); });
+    blk.load(bid, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, lhs, rhs, out); }, xcd_contiguous);
     blk.for_each_segment([&](int r, int p, int q, int, int) {
         const float* lhs_row = lhs + (size_t)(blk.row0 + r) * D;
         const int shift = blk.shift(r);
@@ -67,12 +68,13 @@ __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __
 
 // MASKED = false: D == G1 * VEC * DS exactly, every access of every lane falls inside the row.
 template <int VEC, int G1, int DS, bool MASKED, int W, int R>
-__global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, const int* __restrict__ row_offsets,
+__global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, int xcd_contiguous, const int* __restrict__ row_offsets,
                                                        const int* __restrict__ col_indices,
                                                        const float* __restrict__ lhs, const float* __restrict__ rhs,
                                                        float* __restrict__ out)
 {
-    sddmm_block<VEC, G1, DS, MASKED, W, R, false>((int)blockIdx.x, M, D, row_offsets, nullptr, col_indices, lhs, rhs, out);
+    sddmm_block<VEC, G1, DS, MASKED, W, R, false>((int)blockIdx.x, M, D, row_offsets, nullptr, col_indices, lhs, rhs, out,
+                                                  nullptr, 0, xcd_contiguous);
 }
 
 // Column-sliced schedule (see spmm_sliced_kernel): the row blocks once per slice of columns, slice after slice, so that
@@ -112,12 +114,12 @@ static hipError_t launch_one(const SddmmArgs& x, hipStream_t stream)
     if constexpr (DS > 0) {
         if (x.D == G1 * VEC * DS) {
             hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, false, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M,
-                               x.D, x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
+                               x.D, tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
             return hipGetLastError();
         }
     }
     hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, true, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M, x.D,
-                       x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
+                       tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
     return hipGetLastError();
 }
 

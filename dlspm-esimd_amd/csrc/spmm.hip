@@ -25,7 +25,7 @@ namespace dlspm {
 
 // acc[v] = sum over the nonzeros [p, q) of one row (p < q, wave-uniform) of value * B[column, colv[v] ..], summed over
 // the wave's S = 64/G slots, so that every lane (slot 0 in particular) ends with the total.
-template <int VEC, int G, int V>
+template <int VEC, int G, int V, bool BUF = false>
 __device__ __forceinline__ void spmm_segment(Vec<VEC>* acc, int p, int q, const int* __restrict__ col_indices,
                                              const float* __restrict__ values, const float* __restrict__ B, int N,
                                              const int* colv, int lane)
@@ -45,7 +45,7 @@ __device__ __forceinline__ void spmm_segment(Vec<VEC>* acc, int p, int q, const 
         const int ahead = min(base + kWave + lane, q - 1);
         c_nxt = col_indices[ahead];
         a_nxt = values[ahead];
-        dense_rows_fma<VEC, G, V>(acc, c, av, min(kWave, q - base), B, N, colv, lane);
+        dense_rows_fma<VEC, G, V, BUF>(acc, c, av, min(kWave, q - base), B, N, colv, lane);
     }
     if constexpr (kWave / G > 1) slots_sum<VEC, G, V>(acc, lane);
 }
@@ -56,12 +56,13 @@ __device__ __forceinline__ void spmm_segment(Vec<VEC>* acc, int p, int q, const 
 // tile 0, then of tile 1, ...) when it does not, so that the device gathers from one K x TW slab of B at a time.
 // Measured on 512 x 4608, N = 3136 (B: 55 MiB): 708 -> 239 us tile-major; on 2048 x 1024, N = 784 (3 MiB), lognormal
 // rows: 81 us row-major, 93 us tile-major. No division in the usual case of one tile.
-template <int VEC, int G, int V, int W, int R, bool SLICED, bool PLANNED = false>
+template <int VEC, int G, int V, int W, int R, bool SLICED, bool PLANNED = false, bool BUF = false>
 __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles, int tile_major,
                                            const int* __restrict__ row_offsets,
                                            const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                            const float* __restrict__ values, const float* __restrict__ B,
-                                           float* __restrict__ C, const int* __restrict__ row_ids = nullptr, int nnz = 0)
+                                           float* __restrict__ C, const int* __restrict__ row_ids = nullptr, int nnz = 0,
+                                           int xcd_contiguous = 0)
 {
     int ct = 0, rb = bid;
     if (col_tiles != 1) {
@@ -75,21 +76,23 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
         }
     }
     RowBlock<W, R, SLICED, PLANNED> blk;
-    blk.load(rb, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, values, B, C); });
+    blk.load(rb, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, values, B, C); },
+             col_tiles == 1 ? xcd_contiguous : 0);
     dense_rows_block<VEC, G, V>(blk, ct, N, C, [&](Vec<VEC>* acc, int, int p, int q, const int* colv) {
-        spmm_segment<VEC, G, V>(acc, p, q, col_indices, values, B, N, colv, blk.lane);
+        spmm_segment<VEC, G, V, BUF>(acc, p, q, col_indices, values, B, N, colv, blk.lane);
     });
 }
 
-template <int VEC, int G, int V, int W, int R>
-__global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tiles, int tile_major,
+// BUF: B is read through a buffer descriptor (B below 4 GiB, G == 64: see dense_rows_fma)
+template <int VEC, int G, int V, int W, int R, bool BUF>
+__global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tiles, int tile_major, int xcd_contiguous,
                                                       const int* __restrict__ row_offsets,
                                                       const int* __restrict__ col_indices,
                                                       const float* __restrict__ values,
                                                       const float* __restrict__ B, float* __restrict__ C)
 {
-    spmm_block<VEC, G, V, W, R, false>((int)blockIdx.x, M, N, col_tiles, tile_major, row_offsets, nullptr, col_indices,
-                                       values, B, C);
+    spmm_block<VEC, G, V, W, R, false, false, BUF>((int)blockIdx.x, M, N, col_tiles, tile_major, row_offsets, nullptr,
+                                                   col_indices, values, B, C, nullptr, 0, xcd_contiguous);
 }
 
 // Column-sliced schedule: the grid holds the row blocks once per slice of columns, slice after slice, so that at
@@ -110,7 +113,7 @@ __global__ __launch_bounds__(4 * 64) void spmm_sliced_kernel(int M, int N, int c
 
 // Row plan: workgroup i works on the whole row rows[i] = [starts[i], ends[i]) of the CSR matrix (one row per four-wave
 // workgroup); with column tiles the plan is gone through once per tile, tile after tile.
-template <int VEC, int G, int V>
+template <int VEC, int G, int V, bool BUF>
 __global__ __launch_bounds__(4 * 64) void spmm_planned_kernel(int M, int N, int nnz, int col_tiles,
                                                               const int* __restrict__ starts,
                                                               const int* __restrict__ ends, const int* __restrict__ rows,
@@ -118,8 +121,8 @@ __global__ __launch_bounds__(4 * 64) void spmm_planned_kernel(int M, int N, int 
                                                               const float* __restrict__ values,
                                                               const float* __restrict__ B, float* __restrict__ C)
 {
-    spmm_block<VEC, G, V, 4, 1, true, true>((int)blockIdx.x, M, N, col_tiles, 1, starts, ends, col_indices, values, B, C, rows,
-                                            nnz);
+    spmm_block<VEC, G, V, 4, 1, true, true, BUF>((int)blockIdx.x, M, N, col_tiles, 1, starts, ends, col_indices, values, B, C,
+                                                 rows, nnz);
 }
 
 // ---- host side --------------------------------------------------------------------------------------
@@ -132,8 +135,15 @@ static hipError_t launch_one(const SpmmArgs& x, int tile_major, hipStream_t stre
     const long long blocks = ceil_div(x.M, R) * col_tiles;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((spmm_kernel<VEC, G, V, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream, x.M, x.N,
-                       col_tiles, tile_major, x.row_offsets, x.col_indices, x.values, x.B, x.C);
+    if constexpr (G == kWave) {
+        if (dense_fits_buffer(x.K, x.N)) {
+            hipLaunchKernelGGL((spmm_kernel<VEC, G, V, W, R, true>), dim3((unsigned)blocks), dim3(W * 64), 0, stream, x.M, x.N,
+                               col_tiles, tile_major, tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.values, x.B, x.C);
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((spmm_kernel<VEC, G, V, W, R, false>), dim3((unsigned)blocks), dim3(W * 64), 0, stream, x.M, x.N,
+                       col_tiles, tile_major, tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.values, x.B, x.C);
     return hipGetLastError();
 }
 
@@ -446,8 +456,12 @@ hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int*
         const int col_tiles = (x.N + g_ * 4 * v_ - 1) / (g_ * 4 * v_);                                                 \
         const long long blocks = (long long)x.M * col_tiles;                                                           \
         if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;                                                \
-        hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M, x.N, \
-                           x.nnz, col_tiles, starts, ends, rows, x.col_indices, x.values, x.B, x.C);                   \
+        if (g_ == kWave && dense_fits_buffer(x.K, x.N))                                                                \
+            hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_, g_ == kWave>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, \
+                               x.M, x.N, x.nnz, col_tiles, starts, ends, rows, x.col_indices, x.values, x.B, x.C);     \
+        else                                                                                                           \
+            hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_, false>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, \
+                               x.M, x.N, x.nnz, col_tiles, starts, ends, rows, x.col_indices, x.values, x.B, x.C);     \
         return hipGetLastError();                                                                                      \
     }
     DLSPM_PLANNED(64, 2)

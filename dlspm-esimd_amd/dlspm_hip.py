@@ -69,7 +69,7 @@ EXPORTS = (
 class Tuning(ctypes.Structure):
     """dlspm_tuning of include/dlspm_hip.h."""
     _fields_ = [(n, ctypes.c_int) for n in ("split_w", "split_r", "flat", "flat_chunk", "slices", "tile_major",
-                                            "tile_width", "plan_order")]
+                                            "tile_width", "plan_order", "xcd_contiguous")]
 
 
 class DlspmError(RuntimeError):

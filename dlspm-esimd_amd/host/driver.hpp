@@ -354,6 +354,8 @@ struct CaseSpec {
     int M = 0, K = 0, N = 0;
     double density = 0;
     double sigma = 0;  // > 0: row lengths lognormal around density*K with this sigma (skewed rows) instead of Bernoulli
+    int band = 0;      // > 0: every row holds a band of this many columns around its diagonal position, plus
+    int band_random = 0;  // ... this many columns anywhere (density is ignored): the pattern of sparse attention masks
     uint64_t seed = 1;
     std::string file;
 };
@@ -361,6 +363,7 @@ struct CaseSpec {
 // pattern of a --shape case
 inline Csr synthetic_pattern(const CaseSpec& s)
 {
+    if (s.band > 0) return pattern_band_plus_random(s.seed, s.M, s.K, s.band, s.band_random);
     return s.sigma > 0 ? pattern_lognormal_rows(s.seed, s.M, s.K, s.density * s.K, s.sigma)
                        : pattern_bernoulli(s.seed, s.M, s.K, s.density);
 }
@@ -397,7 +400,8 @@ inline std::string usage(const char* app, const char* width)
     u << "Usage: " << app << " <filename>.smtx <" << width << ">            one matrix from a DLMC .smtx file\n"
       << "       " << app << " --batch <list>                      lines '<filename>.smtx <" << width << ">', '#' comments\n"
       << "       " << app << " --shape M K " << width << " density [--seed S] [--sigma s]   one synthetic matrix (Bernoulli pattern;\n"
-      << "                                                     --sigma: lognormal row lengths, skewed)\n"
+      << "                                                     --sigma: lognormal row lengths, skewed;\n"
+      << "                                                     --band w [--band-random r]: a band of w columns per row plus r anywhere)\n"
       << "       " << app << " --sweep [--max-m M]                  the 12 x {32,128} x {0.3,0.2,0.1} benchmark grid\n"
       << "       " << app << " --cfg <id>                           a seeded benchmark configuration (1..5)\n"
       << "options: --iters n (20)  --warmup n (5)  --cold  --csv <file>  --dump <dir> | --dump-each <dir>  --tol x (1e-4)  --workspace | --no-workspace  --no-plan";
@@ -425,6 +429,8 @@ inline Cli parse_cli(int argc, char** argv, const char* app, const char* width)
         }
         else if (a == "--seed") { need(i, 1); const uint64_t sd = std::stoull(argv[++i]); if (!cli.cases.empty()) cli.cases.back().seed = sd; }
         else if (a == "--sigma") { need(i, 1); const double sg = std::stod(argv[++i]); if (!cli.cases.empty()) cli.cases.back().sigma = sg; }
+        else if (a == "--band") { need(i, 1); const int b = std::stoi(argv[++i]); if (!cli.cases.empty()) cli.cases.back().band = b; }
+        else if (a == "--band-random") { need(i, 1); const int b = std::stoi(argv[++i]); if (!cli.cases.empty()) cli.cases.back().band_random = b; }
         else if (a == "--no-workspace") cli.opt.workspace = Options::kNever;
         else if (a == "--workspace") cli.opt.workspace = Options::kAlways;
         else if (a == "--no-plan") cli.opt.plan = false;

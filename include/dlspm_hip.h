@@ -270,7 +270,8 @@ int dlspm_describe_slices(int op, int M, int K, int N_or_D, int nnz, int* slices
  * Overrides of the launch rules, for tuning sweeps and tests; production callers never need them. One set per host
  * thread: dlspm_set_tuning changes the calling thread's, NULL goes back to the process default. That default is the
  * rules themselves unless the environment said otherwise when the library first looked, once per process:
- * DLSPM_SPLIT="W,R", DLSPM_FLAT, DLSPM_FLAT_CHUNK, DLSPM_SLICES, DLSPM_TILE_MAJOR, DLSPM_TILE_WIDTH, DLSPM_PLAN_ORDER
+ * DLSPM_SPLIT="W,R", DLSPM_FLAT, DLSPM_FLAT_CHUNK, DLSPM_SLICES, DLSPM_TILE_MAJOR, DLSPM_TILE_WIDTH, DLSPM_PLAN_ORDER,
+ * DLSPM_XCD_CONTIGUOUS
  * (so that the drivers can be swept from a shell). No launch reads the environment. An override that names a shape
  * the kernels are not built for is ignored. dlspm_workspace_bytes and the describe calls follow the overrides, so
  * set them before sizing a workspace. No counterpart in the reference (its knobs are -D macros, SPMM/spmmesimd.hpp:17-21).
@@ -283,6 +284,11 @@ typedef struct dlspm_tuning {
     int tile_major;       /* SpMM column tiles one after the other: -1 the rule, 0 no, 1 yes                        */
     int tile_width;       /* SpMM column tile: 0 the rule, else 512, 256, 128, 64 or 32                             */
     int plan_order;       /* dlspm_row_plan_build: 0 packed (the rule), 1 alternating groups, 2 longest first       */
+    int xcd_contiguous;   /* 0 (the rule): neighbouring row blocks go to different XCDs, as the hardware deals them;   */
+                          /* 1: each of the eight XCDs works on one contiguous run of row blocks, so that a banded    */
+                          /* mask gathers a different eighth of the dense operands into each L2 (4x fewer bytes       */
+                          /* fetched, 6 % faster on a 16384-row band; unsafe as a rule: rows whose length depends on   */
+                          /* their position would load the XCDs unevenly). One column tile, no row plan, no slices.   */
 } dlspm_tuning;
 void dlspm_tuning_default(dlspm_tuning* t);   /* fills *t with "follow the rules" */
 int dlspm_set_tuning(const dlspm_tuning* t);  /* DLSPM_OK or DLSPM_E_INVALID_ARG (a field out of range) */

@@ -768,6 +768,30 @@ def test_hint_bits_and_the_deprecated_constant(torch_cuda, dl):
     assert st == dl.OK and torch.equal(via_named, via_alias)
 
 
+def test_xcd_contiguous_row_blocks_give_the_same_bits(torch_cuda, dl, oracle):
+    """dlspm_tuning.xcd_contiguous only changes which workgroup works on which row block (each XCD one contiguous run):
+    every row is summed as before, so all three ops return the bits of the default order, also where the number of
+    row blocks is no multiple of eight, where rows are grouped, and where column tiles switch it off."""
+    torch = torch_cuda
+    rng = np.random.default_rng(123)
+    for kind, M, K, N, den in (("skewed", 2048, 512, 256, 0.1), ("empty_rows", 2051, 700, 64, 0.1), ("uniform", 9, 300, 128, 0.3),
+                               ("skewed", 16390, 256, 32, 0.05), ("uniform", 5, 40, 16, 0.5), ("skewed", 1003, 512, 700, 0.1)):
+        ro, ci = random_csr(rng, M, K, kind, den)
+        va = rng.normal(0, 1, ci.size).astype(np.float32)
+        B = rng.normal(0, 1, (K, N)).astype(np.float32)
+        Q = rng.normal(0, 1, (M, N)).astype(np.float32)
+        ro_d, ci_d, va_d, B_d, Q_d = (dev(torch, x) for x in (ro, ci, va, B, Q))
+        print(f"xcd case {kind} {M}x{K} N {N} nnz {ci.size}", flush=True)
+        want = (dl.spmm(ro_d, ci_d, va_d, B_d).clone(), dl.sddmm(ro_d, ci_d, Q_d, B_d).clone(), dl.fused(ro_d, ci_d, Q_d, B_d, B_d, 0.5).clone())
+        dl.set_tuning(xcd_contiguous=1)
+        got = (dl.spmm(ro_d, ci_d, va_d, B_d).clone(), dl.sddmm(ro_d, ci_d, Q_d, B_d).clone(), dl.fused(ro_d, ci_d, Q_d, B_d, B_d, 0.5).clone())
+        dl.set_tuning()
+        for g, w in zip(got, want):
+            assert torch.equal(g, w), (kind, M, K, N)
+        assert oracle.rel_frobenius(got[0].cpu().numpy(), oracle.spmm(ro, ci, va, B, omp=True)) <= TOL
+        check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
 def test_concurrent_calls_from_two_threads_on_two_streams(torch_cuda, dl, oracle):
     """The library keeps no mutable global state: two host threads, each with its own stream, outputs and workspace."""
     import threading
