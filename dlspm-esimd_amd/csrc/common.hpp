@@ -536,14 +536,15 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t dense_buffer(const float* p)
 // Loads are issued U dense rows at a time before the first FMA so that U*V requests per lane are in
 // flight. `colv` must be a valid column for every lane (lanes outside the matrix pass a safe column and
 // simply never store their accumulator), so the loop body has no predicates.
-// BUF (G == 64 only, dense operand below 4 GiB): the rows are read with buffer loads (dense_buffer above).
+// BUF (dense operand below 4 GiB, fewer than 2^24 rows of fewer than 2^24 bytes): the rows are read with buffer loads
+// (dense_buffer above); with G < 64 every lane group has its own row, whose offset is then one 24-bit multiply-add per
+// access on the vector unit instead of a 64-bit multiply, shift and add.
 template <int VEC, int G, int V, bool BUF = false>
 __device__ __forceinline__ void dense_rows_fma(Vec<VEC>* acc, int c, float av, int cnt, const float* __restrict__ dense,
                                                int ld, const int* colv, int lane)
 {
     using VecT = Vec<VEC>;
     constexpr int S = kWave / G;
-    static_assert(!BUF || S == 1, "buffer loads take a wave-uniform row offset");
     constexpr int U = V >= 4 ? 2 : 8 / V;
     const int slot = lane / G;
     const int full = cnt / S;  // steps in which every slot has a nonzero
@@ -554,7 +555,8 @@ __device__ __forceinline__ void dense_rows_fma(Vec<VEC>* acc, int c, float av, i
     const __amdgpu_buffer_rsrc_t rsrc = dense_buffer(dense);
     // dense row cj, access v of this lane
     auto row_load = [&](int cj, int v) -> VecT {
-        if constexpr (BUF) return VecT::bload(rsrc, offv[v], (unsigned)cj * pitch);
+        if constexpr (BUF && S == 1) return VecT::bload(rsrc, offv[v], (unsigned)cj * pitch);
+        else if constexpr (BUF) return VecT::bload(rsrc, __umul24((unsigned)cj, pitch) + offv[v], 0u);
         else return VecT::gload(dense + (size_t)cj * ld + colv[v]);
     };
     int t = 0;

@@ -9,7 +9,11 @@ namespace dlspm {
 inline long long ceil_div(long long a, long long b) { return (a + b - 1) / b; }
 
 // A dense operand of `rows` x `width` floats can be read through a buffer descriptor (32-bit byte offsets)
-inline bool dense_fits_buffer(long long rows, long long width) { return rows * width * 4 < (1ll << 32); }
+// and through 24-bit multiplies of (row, row pitch in bytes)
+inline bool dense_fits_buffer(long long rows, long long width)
+{
+    return rows * width * 4 < (1ll << 32) && rows < (1 << 24) && width * 4 < (1 << 24);
+}
 
 // The device the calling thread has current, as far as the launch rules need it: compute units and the size of one
 // L2. Read from hipDeviceProp_t once per device and cached; without a device (host-only queries on a machine that has

@@ -83,7 +83,7 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
     });
 }
 
-// BUF: B is read through a buffer descriptor (B below 4 GiB, G == 64: see dense_rows_fma)
+// BUF: B is read through a buffer descriptor (B below 4 GiB: see dense_rows_fma)
 template <int VEC, int G, int V, int W, int R, bool BUF>
 __global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tiles, int tile_major, int xcd_contiguous,
                                                       const int* __restrict__ row_offsets,
@@ -135,7 +135,7 @@ static hipError_t launch_one(const SpmmArgs& x, int tile_major, hipStream_t stre
     const long long blocks = ceil_div(x.M, R) * col_tiles;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-    if constexpr (G == kWave) {
+    {
         if (dense_fits_buffer(x.K, x.N)) {
             hipLaunchKernelGGL((spmm_kernel<VEC, G, V, W, R, true>), dim3((unsigned)blocks), dim3(W * 64), 0, stream, x.M, x.N,
                                col_tiles, tile_major, tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.values, x.B, x.C);
@@ -456,8 +456,8 @@ hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int*
         const int col_tiles = (x.N + g_ * 4 * v_ - 1) / (g_ * 4 * v_);                                                 \
         const long long blocks = (long long)x.M * col_tiles;                                                           \
         if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;                                                \
-        if (g_ == kWave && dense_fits_buffer(x.K, x.N))                                                                \
-            hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_, g_ == kWave>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, \
+        if (dense_fits_buffer(x.K, x.N))                                                                               \
+            hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_, true>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, \
                                x.M, x.N, x.nnz, col_tiles, starts, ends, rows, x.col_indices, x.values, x.B, x.C);     \
         else                                                                                                           \
             hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_, false>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, \
