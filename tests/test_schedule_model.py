@@ -697,3 +697,35 @@ def test_gpu_row_plan_equals_its_sequential_definition(model, dl, kind, M, K):
         assert np.array_equal(got, want), (kind, M, K, order, np.flatnonzero(got != want)[:10])
     dl.set_tuning()
     assert np.array_equal(ro_d.cpu().numpy(), ro)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,longest,seed", [(700, 1 << 21, 1), (2048, (1 << 21) - 1, 2), (640, 3_000_000, 3), (5000, 2_500_000, 4),
+                                            (2048, 1 << 20, 5)])
+def test_gpu_row_plan_with_very_long_rows(model, dl, M, longest, seed):
+    """The plan needs row_offsets only, so rows of millions of nonzeros can be planned without a matrix behind them:
+    from 2^21 nonzeros in one row on, the tile sort and the packing work on 64-bit keys instead of 32-bit ones; both
+    forms, and the boundary between them, must give the sequential definition."""
+    import torch
+
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(0, 2000, M)
+    heavy = rng.choice(M, size=min(M, 600), replace=False)
+    lens[heavy] = rng.integers(longest // 2, longest + 1, heavy.size)
+    lens[heavy[0]] = longest
+    while lens.sum() >= (1 << 31) - 1:  # row_offsets are 32-bit
+        heavy = heavy[: heavy.size // 2]
+        lens[:] = np.minimum(lens, 2000)
+        lens[heavy] = rng.integers(longest // 2, longest + 1, heavy.size)
+        lens[heavy[0]] = longest
+    ro = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    bins = min(dl.device_info()["compute_units"], 256)
+    ro_d = dev(torch, ro)
+    for order in (0, 2):
+        dl.set_tuning(plan_order=order)
+        plan = torch.full((dl.row_plan_bytes(M) // 4,), -7, dtype=torch.int32, device="cuda")
+        dl.row_plan(ro_d, out=plan)
+        got = plan.cpu().numpy()[:3 * M]
+        want = model_plan(model, ro, bins, order)
+        assert np.array_equal(got, want), (M, longest, order, np.flatnonzero(got != want)[:10])
+    dl.set_tuning()
