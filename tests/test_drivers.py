@@ -4,6 +4,7 @@ the CPU oracle (the drivers themselves only cross-check on the device)."""
 import json
 import os
 import subprocess
+import sys
 
 import numpy as np
 import pytest
@@ -400,3 +401,19 @@ def test_spmm_driver_builds_a_row_plan_for_small_uneven_matrices():
     assert rc == 0 and "PASS" in out and "row plan:" in out, out
     rc, out = run("spmm_run", "--shape", 8192, 512, 256, 0.04, "--sigma", 0.8, "--iters", 5)    # short rows: no plan
     assert rc == 0 and "PASS" in out and "row plan:" not in out, out
+
+
+@pytest.mark.gpu
+def test_verify_dlmc_script_on_the_fixtures(tmp_path):
+    """tests/verify_dlmc.py is the wide form of the fixture tests above (any directory of .smtx files, every schedule,
+    all three ops against the oracle); here it runs over the fifteen fixtures, with a batch-size table for SpMM."""
+    table = tmp_path / "batchsizes.txt"
+    names = sorted(f[:-5] for f in os.listdir(DLMC) if f.endswith(".smtx"))
+    table.write_text("".join(f"{n},{w}\n" for n, w in zip(names, [49, 196, 64, 256, 33] * 3)))
+    report = tmp_path / "report.txt"
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "verify_dlmc.py"), DLMC, "--batch-table", str(table),
+                        "--all-schedules", "--report", str(report)], capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    assert "verify_dlmc PASS" in r.stdout and " 0 FAIL" in r.stdout
+    lines = report.read_text().splitlines()
+    assert len(lines) >= 15 * 3 * 3 and all(line.startswith("PASS ") for line in lines)

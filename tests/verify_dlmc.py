@@ -1,0 +1,179 @@
+#!/usr/bin/env python3
+"""Oracle parity over a directory of real sparsity patterns (.smtx files, the format of the reference's dlmc/ tree).
+
+    python tests/verify_dlmc.py <dir> [--batch-table rn50_batchsizes.txt | --n 256] [--d-sddmm 128] [--d-fused 64]
+                                [--ops spmm,sddmm,fused] [--every 1] [--limit 0] [--report out.txt] [--all-schedules]
+
+For every file below <dir>: the pattern is uploaded, values and dense operands are drawn from a seed, each op runs on
+the GPU through the C ABI the way the C++ drivers call it (one look at the row lengths, then a row plan, workspace
+memory, the even-rows hint or NULL as the library advises; --all-schedules runs every one of them that applies) and the
+result is compared with the CPU oracle (oracle/, the reference's gold loops: SPMM/spmm-esimd-fromfile.cpp:63-83,
+SDDMM/sddmm-esimd-fromfile.cpp:18-36, FUSED/fused.cpp:47-89): CSR arrays bit-identical after the call, values within
+1e-4 relative Frobenius error. SpMM widths come from a "<layer name>,<batch size>" table where one is given (files whose
+layer is not in it are skipped for SpMM, as in SPMM/batch-run-spmm_fromfile:16-46), else --n.
+
+This is the wide net that the fixtures under tests/golden/dlmc/ are a sample of; it needs the dataset, which is not part
+of this repository. Exit status 1 if any case fails.
+"""
+import argparse
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for sub in ("dlspm-esimd_amd", "oracle"):
+    sys.path.insert(0, os.path.join(ROOT, sub))
+
+TOLERANCE = 1e-4
+
+
+def load_smtx(path):
+    """(M, K, row_offsets, col_indices) of an .smtx file: 'M, K, nnz', then the offsets, then the column indices."""
+    with open(path) as f:
+        head = f.readline().replace(",", " ").split()
+        M, K, nnz = int(head[0]), int(head[1]), int(head[2])
+        ro = np.array(f.readline().split(), dtype=np.int64)
+        ci = np.array(f.read().split(), dtype=np.int64)  # (an empty matrix has no third line)
+    if ro.size != M + 1 or ci.size != nnz or ro[0] != 0 or ro[-1] != nnz or (np.diff(ro) < 0).any():
+        raise ValueError(f"{path}: not a CSR structure of {M} x {K} with {nnz} nonzeros")
+    if nnz and (ci.min() < 0 or ci.max() >= K):
+        raise ValueError(f"{path}: column index out of range")
+    return M, K, ro.astype(np.int32), ci.astype(np.int32)
+
+
+def schedules(dl, torch, op, M, K, N, nnz, ro_d, every):
+    """[(name, workspace, plan)]: what the drivers would pass, or every schedule that applies."""
+    longest, _ = dl.csr_row_stats(ro_d)
+    out = []
+    planned = dl.row_plan_advice(op, M, K, N, nnz, longest)
+    advice = dl.workspace_advice(op, M, K, N, nnz, longest)
+    need = dl.workspace_bytes(op, M, K, N, nnz)
+
+    def memory():
+        return torch.empty(need, dtype=torch.uint8, device="cuda")
+
+    if every:
+        out.append(("null", None, None))
+        out.append(("rows_even_hint", dl.ROWS_EVEN, None))
+        if need:
+            out.append(("workspace", memory(), None))
+        if M > 0:
+            out.append(("row_plan", None, dl.row_plan(ro_d)))
+        return out
+    if planned:
+        return [("row_plan", None, dl.row_plan(ro_d))]
+    if advice == dl.PASS_WORKSPACE and need:
+        return [("workspace", memory(), None)]
+    if advice == dl.PASS_ROWS_EVEN:
+        return [("rows_even_hint", dl.ROWS_EVEN, None)]
+    return [("null", None, None)]
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("dir")
+    ap.add_argument("--batch-table", default=None, help="'<layer name>,<batch size>' lines: the SpMM width of each layer")
+    ap.add_argument("--n", type=int, default=256, help="SpMM width without a table")
+    ap.add_argument("--d-sddmm", type=int, default=128)
+    ap.add_argument("--d-fused", type=int, default=64)
+    ap.add_argument("--ops", default="spmm,sddmm,fused")
+    ap.add_argument("--every", type=int, default=1, help="take every n-th file of the sorted list")
+    ap.add_argument("--limit", type=int, default=0, help="stop after this many files (0: all)")
+    ap.add_argument("--report", default=None, help="write one line per case to this file")
+    ap.add_argument("--all-schedules", action="store_true")
+    args = ap.parse_args()
+
+    import torch
+
+    import dlspm_hip as dl
+    import oracle
+
+    if not torch.cuda.is_available():
+        sys.exit("verify_dlmc.py needs the GPU (it checks the HIP kernels, not the oracle)")
+    oracle.lib()
+    table = None
+    if args.batch_table:
+        table = {}
+        for line in open(args.batch_table):
+            key, _, value = line.strip().partition(",")
+            if key and value:
+                table[key] = int(value)
+    files = sorted(os.path.join(d, f) for d, _, fs in os.walk(args.dir) for f in fs if f.endswith(".smtx"))
+    files = files[:: max(args.every, 1)]
+    if args.limit:
+        files = files[: args.limit]
+    ops = [o for o in args.ops.split(",") if o]
+    report = open(args.report, "w") if args.report else None
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    cases = failures = skipped = 0
+    worst = {}
+    by_schedule = {}
+    t0 = last = time.time()
+    print(f"{len(files)} files below {args.dir}; ops {ops}; oracle on {oracle.omp_threads()} threads; {dl.version()}", flush=True)
+    for index, path in enumerate(files):
+        M, K, ro, ci = load_smtx(path)
+        nnz = int(ci.size)
+        name = os.path.basename(path)[: -len(".smtx")]
+        rng = np.random.default_rng(index)
+        ro_d, ci_d = dev(ro), dev(ci)
+        for op in ops:
+            if op == "spmm":
+                N = table.get(name) if table is not None else args.n
+                if N is None:
+                    skipped += 1
+                    continue
+                code = dl.OP_SPMM
+                values = rng.standard_normal(nnz, dtype=np.float32)
+                B = rng.standard_normal((K, N), dtype=np.float32)
+                want = oracle.spmm(ro, ci, values, B, omp=True)
+                values_d, B_d = dev(values), dev(B)
+                run = lambda ws, plan: dl.spmm(ro_d, ci_d, values_d, B_d, K=K, workspace=ws, plan=plan)
+            elif op == "sddmm":
+                N, code = args.d_sddmm, dl.OP_SDDMM
+                lhs = rng.standard_normal((M, N), dtype=np.float32)
+                rhs = rng.standard_normal((K, N), dtype=np.float32)
+                want = oracle.sddmm(ro, ci, lhs, rhs, omp=True)
+                lhs_d, rhs_d = dev(lhs), dev(rhs)
+                run = lambda ws, plan: dl.sddmm(ro_d, ci_d, lhs_d, rhs_d, workspace=ws, plan=plan)
+            elif op == "fused":
+                N, code = args.d_fused, dl.OP_FUSED
+                Q = rng.standard_normal((M, N), dtype=np.float32)
+                Km = rng.standard_normal((K, N), dtype=np.float32)
+                V = rng.standard_normal((K, N), dtype=np.float32)
+                scale = float(1.0 / np.sqrt(N))
+                want = oracle.fused(ro, ci, Q, Km, V, scale, omp=True)
+                Q_d, Km_d, V_d = dev(Q), dev(Km), dev(V)
+                run = lambda ws, plan: dl.fused(ro_d, ci_d, Q_d, Km_d, V_d, scale, workspace=ws, plan=plan)
+            else:
+                sys.exit(f"unknown op {op}")
+            for schedule, ws, plan in schedules(dl, torch, code, M, K, N, nnz, ro_d, args.all_schedules):
+                got = run(ws, plan).cpu().numpy()
+                err = oracle.rel_frobenius(got, want)
+                intact = np.array_equal(ro_d.cpu().numpy(), ro) and np.array_equal(ci_d.cpu().numpy(), ci)
+                ok = bool(intact and err <= TOLERANCE)
+                cases += 1
+                failures += 0 if ok else 1
+                worst[op] = max(worst.get(op, 0.0), err)
+                by_schedule[(op, schedule)] = by_schedule.get((op, schedule), 0) + 1
+                line = f"{'PASS' if ok else 'FAIL'} {op} {schedule} {os.path.relpath(path, args.dir)} M={M} K={K} nnz={nnz} N={N} rel={err:.3e}"
+                if report:
+                    report.write(line + "\n")
+                if not ok:
+                    print(line, flush=True)
+        if time.time() - last > 30:
+            last = time.time()
+            print(f"  {index + 1}/{len(files)} files, {cases} cases, {failures} failures, {last - t0:.0f} s", flush=True)
+    if report:
+        report.close()
+    print(f"{cases} cases over {len(files)} files in {time.time() - t0:.0f} s: {cases - failures} PASS, {failures} FAIL"
+          f" ({skipped} SpMM cases skipped: layer not in the table)")
+    print("largest relative Frobenius error per op: " + ", ".join(f"{op} {worst[op]:.3e}" for op in sorted(worst)))
+    print("cases per (op, schedule): " + ", ".join(f"{op}/{s} {n}" for (op, s), n in sorted(by_schedule.items())))
+    print("verify_dlmc " + ("PASS" if failures == 0 and cases > 0 else "FAIL"))
+    sys.exit(0 if failures == 0 and cases > 0 else 1)
+
+
+if __name__ == "__main__":
+    main()
