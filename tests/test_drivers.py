@@ -417,3 +417,16 @@ def test_verify_dlmc_script_on_the_fixtures(tmp_path):
     assert "verify_dlmc PASS" in r.stdout and " 0 FAIL" in r.stdout
     lines = report.read_text().splitlines()
     assert len(lines) >= 15 * 3 * 3 and all(line.startswith("PASS ") for line in lines)
+
+
+@pytest.mark.gpu
+def test_verify_sweep_script_on_the_smallest_shapes(tmp_path):
+    """tests/verify_sweep.py checks the reference's whole benchmark grid against the oracle at full size; under pytest
+    it runs the shapes of 1024 rows (12 patterns x 3 ops, every schedule)."""
+    report = tmp_path / "report.txt"
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "verify_sweep.py"), "--max-m", "1024", "--all-schedules",
+                        "--report", str(report)], capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    assert "verify_sweep PASS" in r.stdout and " 0 FAIL" in r.stdout
+    lines = report.read_text().splitlines()
+    assert len(lines) >= 6 * 3 * 3 and all(line.startswith("PASS ") for line in lines)

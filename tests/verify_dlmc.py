@@ -71,6 +71,75 @@ def schedules(dl, torch, op, M, K, N, nnz, ro_d, every):
     return [("null", None, None)]
 
 
+def check_pattern(dl, torch, oracle, op, M, K, N, ro, ci, ro_d, ci_d, rng, all_schedules):
+    """Runs op on the pattern (ro, ci: numpy; ro_d, ci_d: the same on the GPU) with seeded operands under the schedules
+    that apply and yields (schedule, relative Frobenius error against the oracle, CSR arrays intact)."""
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    nnz = int(ci.size)
+    if op == "spmm":
+        code = dl.OP_SPMM
+        values = rng.standard_normal(nnz, dtype=np.float32)
+        B = rng.standard_normal((K, N), dtype=np.float32)
+        want = oracle.spmm(ro, ci, values, B, omp=True)
+        values_d, B_d = dev(values), dev(B)
+        run = lambda ws, plan: dl.spmm(ro_d, ci_d, values_d, B_d, K=K, workspace=ws, plan=plan)
+    elif op == "sddmm":
+        code = dl.OP_SDDMM
+        lhs = rng.standard_normal((M, N), dtype=np.float32)
+        rhs = rng.standard_normal((K, N), dtype=np.float32)
+        want = oracle.sddmm(ro, ci, lhs, rhs, omp=True)
+        lhs_d, rhs_d = dev(lhs), dev(rhs)
+        run = lambda ws, plan: dl.sddmm(ro_d, ci_d, lhs_d, rhs_d, workspace=ws, plan=plan)
+    elif op == "fused":
+        code = dl.OP_FUSED
+        Q = rng.standard_normal((M, N), dtype=np.float32)
+        Km = rng.standard_normal((K, N), dtype=np.float32)
+        V = rng.standard_normal((K, N), dtype=np.float32)
+        scale = float(1.0 / np.sqrt(N))
+        want = oracle.fused(ro, ci, Q, Km, V, scale, omp=True)
+        Q_d, Km_d, V_d = dev(Q), dev(Km), dev(V)
+        run = lambda ws, plan: dl.fused(ro_d, ci_d, Q_d, Km_d, V_d, scale, workspace=ws, plan=plan)
+    else:
+        raise ValueError(f"unknown op {op}")
+    for schedule, ws, plan in schedules(dl, torch, code, M, K, N, nnz, ro_d, all_schedules):
+        got = run(ws, plan).cpu().numpy()
+        err = oracle.rel_frobenius(got, want)
+        intact = np.array_equal(ro_d.cpu().numpy(), ro) and np.array_equal(ci_d.cpu().numpy(), ci)
+        yield schedule, err, intact
+
+
+class Tally:
+    """Counts and prints the cases of one run."""
+
+    def __init__(self, report_path):
+        self.cases = self.failures = 0
+        self.worst = {}
+        self.by_schedule = {}
+        self.report = open(report_path, "w") if report_path else None
+
+    def add(self, op, schedule, what, err, intact):
+        ok = bool(intact and err <= TOLERANCE)
+        self.cases += 1
+        self.failures += 0 if ok else 1
+        self.worst[op] = max(self.worst.get(op, 0.0), err)
+        self.by_schedule[(op, schedule)] = self.by_schedule.get((op, schedule), 0) + 1
+        line = f"{'PASS' if ok else 'FAIL'} {op} {schedule} {what} rel={err:.3e}{'' if intact else ' CSR arrays changed'}"
+        if self.report:
+            self.report.write(line + "\n")
+        if not ok:
+            print(line, flush=True)
+
+    def finish(self, name, what):
+        if self.report:
+            self.report.close()
+        print(f"{self.cases} cases over {what}: {self.cases - self.failures} PASS, {self.failures} FAIL")
+        print("largest relative Frobenius error per op: " + ", ".join(f"{op} {self.worst[op]:.3e}" for op in sorted(self.worst)))
+        print("cases per (op, schedule): " + ", ".join(f"{op}/{s} {n}" for (op, s), n in sorted(self.by_schedule.items())))
+        ok = self.failures == 0 and self.cases > 0
+        print(f"{name} " + ("PASS" if ok else "FAIL"))
+        return 0 if ok else 1
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("dir")
@@ -105,74 +174,30 @@ def main():
     if args.limit:
         files = files[: args.limit]
     ops = [o for o in args.ops.split(",") if o]
-    report = open(args.report, "w") if args.report else None
-    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
-    cases = failures = skipped = 0
-    worst = {}
-    by_schedule = {}
+    tally = Tally(args.report)
+    skipped = 0
     t0 = last = time.time()
     print(f"{len(files)} files below {args.dir}; ops {ops}; oracle on {oracle.omp_threads()} threads; {dl.version()}", flush=True)
     for index, path in enumerate(files):
         M, K, ro, ci = load_smtx(path)
-        nnz = int(ci.size)
         name = os.path.basename(path)[: -len(".smtx")]
         rng = np.random.default_rng(index)
-        ro_d, ci_d = dev(ro), dev(ci)
+        ro_d, ci_d = torch.from_numpy(ro).cuda(), torch.from_numpy(ci).cuda()
         for op in ops:
+            N = {"sddmm": args.d_sddmm, "fused": args.d_fused}.get(op)
             if op == "spmm":
                 N = table.get(name) if table is not None else args.n
                 if N is None:
                     skipped += 1
                     continue
-                code = dl.OP_SPMM
-                values = rng.standard_normal(nnz, dtype=np.float32)
-                B = rng.standard_normal((K, N), dtype=np.float32)
-                want = oracle.spmm(ro, ci, values, B, omp=True)
-                values_d, B_d = dev(values), dev(B)
-                run = lambda ws, plan: dl.spmm(ro_d, ci_d, values_d, B_d, K=K, workspace=ws, plan=plan)
-            elif op == "sddmm":
-                N, code = args.d_sddmm, dl.OP_SDDMM
-                lhs = rng.standard_normal((M, N), dtype=np.float32)
-                rhs = rng.standard_normal((K, N), dtype=np.float32)
-                want = oracle.sddmm(ro, ci, lhs, rhs, omp=True)
-                lhs_d, rhs_d = dev(lhs), dev(rhs)
-                run = lambda ws, plan: dl.sddmm(ro_d, ci_d, lhs_d, rhs_d, workspace=ws, plan=plan)
-            elif op == "fused":
-                N, code = args.d_fused, dl.OP_FUSED
-                Q = rng.standard_normal((M, N), dtype=np.float32)
-                Km = rng.standard_normal((K, N), dtype=np.float32)
-                V = rng.standard_normal((K, N), dtype=np.float32)
-                scale = float(1.0 / np.sqrt(N))
-                want = oracle.fused(ro, ci, Q, Km, V, scale, omp=True)
-                Q_d, Km_d, V_d = dev(Q), dev(Km), dev(V)
-                run = lambda ws, plan: dl.fused(ro_d, ci_d, Q_d, Km_d, V_d, scale, workspace=ws, plan=plan)
-            else:
-                sys.exit(f"unknown op {op}")
-            for schedule, ws, plan in schedules(dl, torch, code, M, K, N, nnz, ro_d, args.all_schedules):
-                got = run(ws, plan).cpu().numpy()
-                err = oracle.rel_frobenius(got, want)
-                intact = np.array_equal(ro_d.cpu().numpy(), ro) and np.array_equal(ci_d.cpu().numpy(), ci)
-                ok = bool(intact and err <= TOLERANCE)
-                cases += 1
-                failures += 0 if ok else 1
-                worst[op] = max(worst.get(op, 0.0), err)
-                by_schedule[(op, schedule)] = by_schedule.get((op, schedule), 0) + 1
-                line = f"{'PASS' if ok else 'FAIL'} {op} {schedule} {os.path.relpath(path, args.dir)} M={M} K={K} nnz={nnz} N={N} rel={err:.3e}"
-                if report:
-                    report.write(line + "\n")
-                if not ok:
-                    print(line, flush=True)
+            what = f"{os.path.relpath(path, args.dir)} M={M} K={K} nnz={ci.size} N={N}"
+            for schedule, err, intact in check_pattern(dl, torch, oracle, op, M, K, N, ro, ci, ro_d, ci_d, rng, args.all_schedules):
+                tally.add(op, schedule, what, err, intact)
         if time.time() - last > 30:
             last = time.time()
-            print(f"  {index + 1}/{len(files)} files, {cases} cases, {failures} failures, {last - t0:.0f} s", flush=True)
-    if report:
-        report.close()
-    print(f"{cases} cases over {len(files)} files in {time.time() - t0:.0f} s: {cases - failures} PASS, {failures} FAIL"
-          f" ({skipped} SpMM cases skipped: layer not in the table)")
-    print("largest relative Frobenius error per op: " + ", ".join(f"{op} {worst[op]:.3e}" for op in sorted(worst)))
-    print("cases per (op, schedule): " + ", ".join(f"{op}/{s} {n}" for (op, s), n in sorted(by_schedule.items())))
-    print("verify_dlmc " + ("PASS" if failures == 0 and cases > 0 else "FAIL"))
-    sys.exit(0 if failures == 0 and cases > 0 else 1)
+            print(f"  {index + 1}/{len(files)} files, {tally.cases} cases, {tally.failures} failures, {last - t0:.0f} s", flush=True)
+    print(f"{time.time() - t0:.0f} s; {skipped} SpMM cases skipped (layer not in the table)")
+    sys.exit(tally.finish("verify_dlmc", f"{len(files)} files"))
 
 
 if __name__ == "__main__":
