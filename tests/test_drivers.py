@@ -430,3 +430,13 @@ def test_verify_sweep_script_on_the_smallest_shapes(tmp_path):
     assert "verify_sweep PASS" in r.stdout and " 0 FAIL" in r.stdout
     lines = report.read_text().splitlines()
     assert len(lines) >= 6 * 3 * 3 and all(line.startswith("PASS ") for line in lines)
+
+
+@pytest.mark.gpu
+def test_verify_fuzz_script(tmp_path):
+    """tests/verify_fuzz.py: random shapes, widths, row-length distributions and tuning overrides, every schedule, all
+    three ops against the oracle; 40 problems of it under pytest."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "verify_fuzz.py"), "--cases", "40", "--seed", "11"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    assert "verify_fuzz PASS" in r.stdout and " 0 FAIL" in r.stdout
