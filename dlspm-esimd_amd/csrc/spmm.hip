@@ -34,18 +34,38 @@ __device__ __forceinline__ void spmm_segment(Vec<VEC>* acc, int p, int q, const 
 #pragma unroll
     for (int v = 0; v < V; ++v) acc[v] = VecT::zero();
     // 64 (column, value) pairs per pass, one per lane; the next 64 are requested (index clamped, so the
-    // loads carry no condition) before the rows of B for the current ones, and arrive behind them
+    // loads carry no condition) before the rows of B for the current ones, and arrive behind them. Narrow rows of B
+    // (lane groups of 8 or fewer: a pass is at most 8 row loads) request two passes ahead: CSR arrays beyond the
+    // Infinity Cache come from HBM, and one such pass does not cover that (24576 x 8192 at density 0.3, N = 32:
+    // 382 -> 335 us; lane groups of 16: 604 -> 627 us; of 32 and 64: -2 % and -1 %; matrices within the cache: equal).
     const int first = min(p + lane, q - 1);
     int c_nxt = col_indices[first];
     float a_nxt = values[first];
-    for (int base = p; base < q; base += kWave) {
-        const bool mine = base + lane < q;
-        const int c = mine ? c_nxt : 0;
-        const float av = mine ? a_nxt : 0.f;
-        const int ahead = min(base + kWave + lane, q - 1);
-        c_nxt = col_indices[ahead];
-        a_nxt = values[ahead];
-        dense_rows_fma<VEC, G, V, BUF>(acc, c, av, min(kWave, q - base), B, N, colv, lane);
+    if constexpr (G <= 8) {
+        const int second = min(p + kWave + lane, q - 1);
+        int c_far = col_indices[second];
+        float a_far = values[second];
+        for (int base = p; base < q; base += kWave) {
+            const bool mine = base + lane < q;
+            const int c = mine ? c_nxt : 0;
+            const float av = mine ? a_nxt : 0.f;
+            c_nxt = c_far;
+            a_nxt = a_far;
+            const int ahead = min(base + 2 * kWave + lane, q - 1);
+            c_far = col_indices[ahead];
+            a_far = values[ahead];
+            dense_rows_fma<VEC, G, V, BUF>(acc, c, av, min(kWave, q - base), B, N, colv, lane);
+        }
+    } else {
+        for (int base = p; base < q; base += kWave) {
+            const bool mine = base + lane < q;
+            const int c = mine ? c_nxt : 0;
+            const float av = mine ? a_nxt : 0.f;
+            const int ahead = min(base + kWave + lane, q - 1);
+            c_nxt = col_indices[ahead];
+            a_nxt = values[ahead];
+            dense_rows_fma<VEC, G, V, BUF>(acc, c, av, min(kWave, q - base), B, N, colv, lane);
+        }
     }
     if constexpr (kWave / G > 1) slots_sum<VEC, G, V>(acc, lane);
 }
