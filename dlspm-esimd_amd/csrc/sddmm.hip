@@ -18,11 +18,35 @@
 
 namespace dlspm {
 
+// Where the results go. Results of more bytes than the device's L2s hold together are stored with the non-temporal
+// hint: ordinary stores allocate their lines in the L2 and push out the rows of rhs that everyone gathers from
+// (24576 x 8192 at density 0.3, 60 million results: D = 32 443 -> 309 us, D = 64 715 -> 525 us, D = 128 1289 -> 1090 us;
+// 80 MB of results: +1 ... 3 %). Small results keep ordinary stores: a kernel ends when its stores have reached memory,
+// and 1 MB of them past the cache cost 5 % (2048 x 2048, D = 128: 5.6 -> 5.9 us).
+struct SampledOut {
+    float* __restrict__ at;
+    int streaming;
+    __device__ __forceinline__ void store(int j, float v) const
+    {
+        // (wave-uniform) The hinted store is written out as an instruction: __builtin_nontemporal_store on one side of
+        // this branch and a plain store on the other are merged into one store by the compiler, and the hint is lost.
+        // (A vector store like any other; the wait counts that the compiler inserts can only become stricter by it.)
+        if (streaming) asm volatile("global_store_dword %0, %1, off nt" : : "v"(at + j), "v"(v) : "memory");
+        else at[j] = v;
+    }
+};
+static inline SampledOut sampled_out(const SddmmArgs& x)
+{
+    const DeviceInfo& dev = device_info();
+    const long long all_l2 = (dev.cus >= 64 ? dev.cus / 32 : 1) * dev.l2_bytes;  // one L2 per XCD of 32 compute units
+    return SampledOut{x.out, (long long)x.nnz * (long long)sizeof(float) > all_l2 ? 1 : 0};
+}
+
 // out[j] = <lhs_row, rhs[col_indices[j]]> for the nonzeros j in [p, q) of one row (p < q, wave-uniform).
 template <int VEC, int G1, int DS, bool MASKED>
 __device__ __forceinline__ void sddmm_segment(int p, int q, int D, const int* __restrict__ col_indices,
                                               const float* __restrict__ lhs_row, const float* __restrict__ rhs,
-                                              float* __restrict__ out, int lane)
+                                              SampledOut out, int lane)
 {
     using VecT = Vec<VEC>;
     const int g = lane % G1;
@@ -43,7 +67,7 @@ __device__ __forceinline__ void sddmm_segment(int p, int q, int D, const int* __
         c_nxt = col_indices[min(base + kWave + lane, q - 1)];
         const int cnt = min(kWave, q - base);
         const float o = sddmm_chunk<VEC, G1, DS, MASKED>(D, lane, cnt, c, lhs_row, lq, rhs);
-        if (base + lane < q) out[base + lane] = o;
+        if (base + lane < q) out.store(base + lane, o);
     }
 }
 
@@ -54,11 +78,11 @@ template <int VEC, int G1, int DS, bool MASKED, int W, int R, bool SLICED, bool 
 __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __restrict__ row_offsets,
                                             const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                             const float* __restrict__ lhs, const float* __restrict__ rhs,
-                                            float* __restrict__ out, const int* __restrict__ row_ids = nullptr, int nnz = 0,
+                                            SampledOut out, const int* __restrict__ row_ids = nullptr, int nnz = 0,
                                             int xcd_contiguous = 0)
 {
     RowBlock<W, R, SLICED, PLANNED> blk;
-    blk.load(bid, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, lhs, rhs, out); }, xcd_contiguous);
+    blk.load(bid, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, lhs, rhs, out.at); }, xcd_contiguous);
     blk.for_each_segment([&](int r, int p, int q, int, int) {
         const float* lhs_row = lhs + (size_t)(blk.row0 + r) * D;
         const int shift = blk.shift(r);
@@ -71,7 +95,7 @@ template <int VEC, int G1, int DS, bool MASKED, int W, int R>
 __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, int xcd_contiguous, const int* __restrict__ row_offsets,
                                                        const int* __restrict__ col_indices,
                                                        const float* __restrict__ lhs, const float* __restrict__ rhs,
-                                                       float* __restrict__ out)
+                                                       SampledOut out)
 {
     sddmm_block<VEC, G1, DS, MASKED, W, R, false>((int)blockIdx.x, M, D, row_offsets, nullptr, col_indices, lhs, rhs, out,
                                                   nullptr, 0, xcd_contiguous);
@@ -85,7 +109,7 @@ __global__ __launch_bounds__(4 * 64) void sddmm_sliced_kernel(int M, int D, int 
                                                               const int* __restrict__ bounds,
                                                               const int* __restrict__ col_indices,
                                                               const float* __restrict__ lhs,
-                                                              const float* __restrict__ rhs, float* __restrict__ out)
+                                                              const float* __restrict__ rhs, SampledOut out)
 {
     const int sl = (int)(blockIdx.x / (unsigned)slice_blocks);
     const int bid = (int)blockIdx.x - sl * slice_blocks;
@@ -101,7 +125,7 @@ __global__ __launch_bounds__(4 * 64) void sddmm_planned_kernel(int M, int D, int
                                                                const int* __restrict__ ends, const int* __restrict__ rows,
                                                                const int* __restrict__ col_indices,
                                                                const float* __restrict__ lhs, const float* __restrict__ rhs,
-                                                               float* __restrict__ out)
+                                                               SampledOut out)
 {
     sddmm_block<VEC, G1, DS, MASKED, 4, 1, true, true>((int)blockIdx.x, M, D, starts, ends, col_indices, lhs, rhs, out, rows, nnz);
 }
@@ -114,12 +138,12 @@ static hipError_t launch_one(const SddmmArgs& x, hipStream_t stream)
     if constexpr (DS > 0) {
         if (x.D == G1 * VEC * DS) {
             hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, false, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M,
-                               x.D, tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
+                               x.D, tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
             return hipGetLastError();
         }
     }
     hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, true, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M, x.D,
-                       tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
+                       tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     return hipGetLastError();
 }
 
@@ -186,9 +210,9 @@ __global__ __launch_bounds__(kFlatWaves * 64) void sddmm_flat_kernel(int M, int 
                                                                       const int* __restrict__ row_offsets,
                                                                       const int* __restrict__ col_indices,
                                                                       const float* __restrict__ lhs,
-                                                                      const float* __restrict__ rhs, float* __restrict__ out)
+                                                                      const float* __restrict__ rhs, SampledOut out)
 {
-    fetch_args_now(row_offsets, col_indices, lhs, rhs, out);
+    fetch_args_now(row_offsets, col_indices, lhs, rhs, out.at);
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const long long a64 = ((long long)blockIdx.x * kFlatWaves + w) * chunk;
@@ -221,12 +245,12 @@ static hipError_t launch_flat(const SddmmArgs& x, int chunk, hipStream_t stream)
     if constexpr (DS > 0) {
         if (x.D == G1 * VEC * DS) {
             hipLaunchKernelGGL((sddmm_flat_kernel<VEC, G1, DS, false>), dim3(blocks), dim3(kFlatWaves * 64), 0, stream, x.M,
-                               x.D, x.nnz, chunk, x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
+                               x.D, x.nnz, chunk, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
             return hipGetLastError();
         }
     }
     hipLaunchKernelGGL((sddmm_flat_kernel<VEC, G1, DS, true>), dim3(blocks), dim3(kFlatWaves * 64), 0, stream, x.M, x.D,
-                       x.nnz, chunk, x.row_offsets, x.col_indices, x.lhs, x.rhs, x.out);
+                       x.nnz, chunk, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     return hipGetLastError();
 }
 
@@ -261,10 +285,10 @@ static hipError_t launch_sliced_r(const SddmmArgs& x, const SlicePlan& plan, con
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     if (x.D == G1 * VEC * DS)
         hipLaunchKernelGGL((sddmm_sliced_kernel<VEC, G1, DS, false, R>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream,
-                           x.M, x.D, (int)slice_blocks, bounds, x.col_indices, x.lhs, x.rhs, x.out);
+                           x.M, x.D, (int)slice_blocks, bounds, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     else
         hipLaunchKernelGGL((sddmm_sliced_kernel<VEC, G1, DS, true, R>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream,
-                           x.M, x.D, (int)slice_blocks, bounds, x.col_indices, x.lhs, x.rhs, x.out);
+                           x.M, x.D, (int)slice_blocks, bounds, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     return hipGetLastError();
 }
 
@@ -313,10 +337,10 @@ static hipError_t launch_planned(const SddmmArgs& x, const int* plan, hipStream_
     const int *starts = plan, *ends = plan + x.M, *rows = plan + 2 * (size_t)x.M;
     if (x.D == 8 * 4 * DS)
         hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, false>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M, x.D,
-                           x.nnz, starts, ends, rows, x.col_indices, x.lhs, x.rhs, x.out);
+                           x.nnz, starts, ends, rows, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     else
         hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, true>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M, x.D,
-                           x.nnz, starts, ends, rows, x.col_indices, x.lhs, x.rhs, x.out);
+                           x.nnz, starts, ends, rows, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     return hipGetLastError();
 }
 

@@ -337,6 +337,33 @@ def test_large_shape_against_oracle(torch_cuda, dl, oracle):
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
+def test_sddmm_results_beyond_the_l2_are_streamed(torch_cuda, dl, oracle):
+    """More results than the L2s hold together (here 9.4 million = 38 MB on an MI355X, whose eight L2s hold 32 MiB) are
+    stored with the non-temporal hint; the bits must be those of ordinary stores under every schedule: row blocks, the
+    even-rows hint, a row plan, and the flat schedule forced by tuning, all against the multi-threaded oracle and equal
+    to each other."""
+    torch = torch_cuda
+    M, K, D = 8192, 8192, 32
+    ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 71, M, K, 0.14)
+    info = dl.device_info()
+    assert ci.size * 4 > max(info["compute_units"] // 32, 1) * info["l2_bytes"]
+    lhs = dl.fill("normal", 72, (M, D), 0.0, 1.0)
+    rhs = dl.fill("normal", 73, (K, D), 0.0, 1.0)
+    want = oracle.sddmm(ro, ci, lhs, rhs, omp=True)
+    ro_d, ci_d, lhs_d, rhs_d = (dev(torch, x) for x in (ro, ci, lhs, rhs))
+    first = None
+    for name in ("null", "rows_even", "plan", "flat"):
+        if name == "flat":
+            dl.set_tuning(flat=1)
+        got = dl.sddmm(ro_d, ci_d, lhs_d, rhs_d, workspace=dl.ROWS_EVEN if name == "rows_even" else None,
+                       plan=dl.row_plan(ro_d) if name == "plan" else None).cpu().numpy()
+        dl.set_tuning()
+        assert oracle.rel_frobenius(got, want) <= TOL, name
+        first = got if first is None else first
+        assert np.array_equal(got, first), name
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
 @pytest.mark.parametrize("sigma", [0.0, 1.5])
 def test_flat_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
     """A matrix large enough (3.4 M nonzeros, 410 per row on average, N = 128) that a call WITH workspace takes the flat
