@@ -38,6 +38,21 @@ template <> struct Vec<4> {
         float4_dword_aligned t = {v.x, v.y, v.z, v.w};
         *reinterpret_cast<float4_dword_aligned*>(p) = t;
     }
+    // The same with the non-temporal hint where `streaming` (wave-uniform) says so. Written out as an instruction: a
+    // hinted store on one side of a branch and a plain one on the other are merged into one plain store by the
+    // compiler. (A vector store like any other; the wait counts the compiler inserts can only become stricter by it.)
+    __device__ __forceinline__ void gstore(float* p, bool streaming) const
+    {
+        if (streaming) {
+            typedef float f4 __attribute__((ext_vector_type(4)));
+            const f4 t = {v.x, v.y, v.z, v.w};
+            // s_nop: a store of more than 8 bytes reads its data one wait state after it issues, and the compiler does
+            // not know that this is one, so the next instruction might overwrite the registers of t
+            asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 0" : : "v"(p), "v"(t) : "memory");
+        } else {
+            gstore(p);
+        }
+    }
     // elements [d, d+4) of a row of D >= 4 floats, d < D, for sums over the row: a lane whose four elements
     // would run past D reads the last four instead and zeroes the ones its left neighbour already covers
     __device__ __forceinline__ static Vec gload_clip(const float* row, int d, int D)
@@ -72,6 +87,11 @@ template <> struct Vec<1> {
         return Vec{__uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, lane_bytes, row_bytes, 0))};
     }
     __device__ __forceinline__ void gstore(float* p) const { *p = v; }
+    __device__ __forceinline__ void gstore(float* p, bool streaming) const
+    {
+        if (streaming) asm volatile("global_store_dword %0, %1, off nt" : : "v"(p), "v"(v) : "memory");
+        else *p = v;
+    }
     __device__ __forceinline__ static Vec gload_clip(const float* row, int d, int) { return Vec{row[d]}; }
     __device__ __forceinline__ void fma(float a, const Vec& b) { v = fmaf(a, b.v, v); }
     __device__ __forceinline__ void add(const Vec& b) { v += b.v; }
@@ -239,6 +259,7 @@ template <int W, int R, bool SLICED, bool PLANNED>
 struct RowBlock {
     static_assert(!PLANNED || (SLICED && R == 1), "a row plan names one row per workgroup");
     int lane, w;
+    int rows_total;  // rows of the matrix
     int nr;    // rows in this block (fewer than R at the end of the matrix)
     int row0;  // row of the dense operands and of the output that belongs to the block's first row
     int off_lo, off_hi, off_win, start_lo, start_win;
@@ -255,6 +276,7 @@ struct RowBlock {
     {
         lane = threadIdx.x & 63;
         w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        rows_total = M;
         if constexpr (!SLICED && !PLANNED) {
             if (xcd_contiguous) {
                 const int nb = (M - 1) / R + 1, x = rb & 7, each = nb >> 3, extra = nb & 7;
@@ -365,6 +387,14 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
     }
     auto s_off = [&](int i) { return blk.off(i); };
     const int T0 = blk.T0, T = blk.T, per = blk.per, a = blk.a;
+    // Results of kStreamedOutputFloats and more are stored with the non-temporal hint: they are written once, and
+    // ordinary stores allocate their lines in the L2 beside the dense rows that are gathered from it, to be written
+    // back when the kernel ends. Measured (SpMM): 2048 x 512, N = 256 (2 MiB) 6.07 -> 5.96 us; 16384 x 4096 at 10 %,
+    // N = 128 (8 MiB) 133 -> 128 us; 65536 x 1024 at 2 %, N = 256 (64 MiB) 52.5 -> 49.7 us; 131072 x 512, N = 128
+    // 41.6 -> 39.1 us. Smaller results lose by it when rows end inside a cache line (512 x 2048, N = 49: 4.72 -> 5.04 us;
+    // 2048 x 1024, N = 33: 4.66 -> 5.03 us). Not for the partial rows of the column-sliced schedule, which are read again.
+    constexpr long long kStreamedOutputFloats = 512 * 1024;
+    const bool streaming = (!SLICED || PLANNED) && (long long)blk.rows_total * width >= kStreamedOutputFloats;
 
     blk.for_each_segment([&](int r, int p, int q, int rs, int re) {
         VecT acc[V];
@@ -376,7 +406,7 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
                 float* orow = out + (size_t)(blk.row0 + r) * width;
 #pragma unroll
                 for (int v = 0; v < V; ++v)
-                    if (act[v]) acc[v].gstore(orow + colv[v]);
+                    if (act[v]) acc[v].gstore(orow + colv[v], streaming);
             } else {
                 float* part = s_part[w][(NP == 1 || p == a) ? 0 : 1];
 #pragma unroll
@@ -393,7 +423,7 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
                     float* orow = out + (size_t)(blk.row0 + r) * width;
 #pragma unroll
                     for (int v = 0; v < V; ++v)
-                        if (act[v]) VecT::zero().gstore(orow + colv[v]);
+                        if (act[v]) VecT::zero().gstore(orow + colv[v], streaming);
                 }
             }
         } else {
@@ -412,7 +442,7 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
 #pragma unroll
                         for (int j = 0; j < m; ++j)
                             if (j * part < len) sum.add(VecT::load(&s_part[r * m + j][0][(v * G + g) * VEC]));
-                        if (act[v]) sum.gstore(orow + colv[v]);
+                        if (act[v]) sum.gstore(orow + colv[v], streaming);
                     }
                 }
             }
@@ -429,7 +459,7 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
             if (T == 0) {
 #pragma unroll
                 for (int v = 0; v < V; ++v)
-                    if (act[v]) VecT::zero().gstore(orow + colv[v]);
+                    if (act[v]) VecT::zero().gstore(orow + colv[v], streaming);
             } else if (T > per) {  // T <= per: wave 0 held the whole row and has stored it
 #pragma unroll
                 for (int v = 0; v < V; ++v) {
@@ -437,7 +467,7 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
 #pragma unroll
                     for (int x = 0; x < W; ++x)
                         if (x * per < T) sum.add(VecT::load(&s_part[x][0][(v * G + g) * VEC]));
-                    if (act[v]) sum.gstore(orow + colv[v]);
+                    if (act[v]) sum.gstore(orow + colv[v], streaming);
                 }
             }
         }
@@ -452,7 +482,7 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
             if (rs == re) {
 #pragma unroll
                 for (int v = 0; v < V; ++v)
-                    if (act[v]) VecT::zero().gstore(orow + colv[v]);
+                    if (act[v]) VecT::zero().gstore(orow + colv[v], streaming);
                 continue;
             }
             const int wl = (rs - T0) / per;
@@ -465,7 +495,7 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
                     const int k = (NP == 2 && x == wl && T0 + x * per != rs) ? 1 : 0;
                     sum.add(VecT::load(&s_part[x][k][(v * G + g) * VEC]));
                 }
-                if (act[v]) sum.gstore(orow + colv[v]);
+                if (act[v]) sum.gstore(orow + colv[v], streaming);
             }
         }
     }
