@@ -106,12 +106,14 @@ struct WorkspaceArg {
     size_t bytes;
     bool rows_even;
     bool row_plan;
+    bool banded;
 };
 static WorkspaceArg workspace_arg(void* workspace, size_t workspace_bytes)
 {
     WorkspaceArg a{};
     a.rows_even = (workspace_bytes & DLSPM_HINT_ROWS_EVEN) != 0 || workspace == DLSPM_ROWS_EVEN;
     a.row_plan = (workspace_bytes & DLSPM_HINT_ROW_PLAN) != 0;
+    a.banded = (workspace_bytes & DLSPM_HINT_BANDED) != 0;
     a.bytes = workspace_bytes & ~DLSPM_HINT_MASK;
     a.mem = workspace == DLSPM_ROWS_EVEN ? nullptr : workspace;
     if (!a.mem || a.bytes == 0) {
@@ -402,7 +404,7 @@ int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int
     if (nnz > 0 && (!col_indices || !values || !B)) return DLSPM_E_INVALID_ARG;
     if (const int st = require_device()) return st;
     const bool vec4 = N >= 4;  // dwordx4 accesses need only dword alignment
-    const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C};
+    const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C, ws.banded ? 1 : 0};
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipError_t e;
     if (ws.row_plan && ws.mem) {
@@ -412,8 +414,10 @@ int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int
                                                 : spmm_launch(args, shape, st);
         return e == hipSuccess ? DLSPM_OK : fail_hip(e);
     }
-    const bool memory = !ws.rows_even && ws.mem != nullptr;
-    const SpmmShape shape = spmm_choose(M, K, N, nnz, vec4, ws.rows_even, !memory);
+    // a banded matrix (DLSPM_HINT_BANDED) runs as row blocks whatever memory came with the call: column slices and
+    // the flat schedule are answers to columns spread over all of K and to uneven rows
+    const bool memory = !ws.rows_even && !ws.banded && ws.mem != nullptr;
+    const SpmmShape shape = spmm_choose(M, K, N, nnz, vec4, ws.rows_even, !memory, ws.banded);
     if (memory) {
         const SlicePlan sliced = spmm_slice_plan(M, K, N, nnz, shape);
         const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(M, nnz, N, shape.G);
@@ -570,7 +574,7 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
         return e0 == hipSuccess ? DLSPM_OK : fail_hip(e0);
     }
     const bool vec4 = D >= 4;  // dwordx4 accesses need only dword alignment
-    const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values};
+    const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values, ws.banded ? 1 : 0};
     if (ws.row_plan && ws.mem) {
         SddmmShape shape = sddmm_choose(M, D, nnz, vec4);
         if (sddmm_plan_applies(shape, M, D, nnz)) {
@@ -582,7 +586,7 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
     const SddmmShape shape = sddmm_choose(M, D, nnz, vec4, ws.rows_even);
     // the flat schedule needs no workspace here (nothing to combine), so the size rule alone decides; it has no
     // width condition for SDDMM (measured for D = 32 ... 256: equal on uniform rows, 15-33 % faster on skewed ones)
-    if (ws.mem && !ws.rows_even && !ws.row_plan) {
+    if (ws.mem && !ws.rows_even && !ws.row_plan && !ws.banded) {
         // with a workspace for the slice boundaries: the column-sliced schedule where the rhs operand exceeds one L2
         const SlicePlan sliced = sddmm_slice_plan(M, K, D, nnz, shape);
         if (ws.bytes < sliced.bytes) return DLSPM_E_WORKSPACE;
@@ -591,7 +595,7 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
             return es == hipSuccess ? DLSPM_OK : fail_hip(es);
         }
     }
-    const FlatPlan plan = sddmm_flat_plan(M, nnz, D);
+    const FlatPlan plan = ws.banded ? FlatPlan{0, 0, 0} : sddmm_flat_plan(M, nnz, D);
     const hipError_t e = plan.chunk > 0 ? sddmm_flat_launch(args, shape, plan.chunk, st) : sddmm_launch(args, shape, st);
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }
@@ -610,7 +614,7 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz, const int* row_offsets, c
     if (const int st = require_device()) return st;
     const bool vec4 = D >= 4;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const FusedArgs args{M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O};
+    const FusedArgs args{M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O, ws.banded ? 1 : 0};
     hipError_t e;
     if (ws.row_plan && ws.mem) {
         FusedShape shape = fused_choose(M, D, nnz, vec4);
@@ -619,7 +623,7 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz, const int* row_offsets, c
         return e == hipSuccess ? DLSPM_OK : fail_hip(e);
     }
     const FusedShape shape = fused_choose(M, D, nnz, vec4, ws.rows_even);
-    if (!ws.rows_even && ws.mem) {
+    if (!ws.rows_even && !ws.banded && ws.mem) {
         const SlicePlan sliced = fused_slice_plan(M, K, D, nnz, shape);
         const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(M, nnz, D, shape.G);
         if (ws.bytes < (sliced.slices > 0 ? sliced.bytes : plan.bytes)) return DLSPM_E_WORKSPACE;

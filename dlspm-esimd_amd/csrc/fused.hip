@@ -134,13 +134,13 @@ static hipError_t launch_one(const FusedArgs& x, hipStream_t stream)
     if constexpr (DS > 0) {
         if (x.D == G1 * VEC * DS) {
             hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, false, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64),
-                               0, stream, x.M, x.D, col_tiles, tuning().xcd_contiguous, x.scale, x.row_offsets, x.col_indices,
+                               0, stream, x.M, x.D, col_tiles, (x.xcd_contiguous | tuning().xcd_contiguous), x.scale, x.row_offsets, x.col_indices,
                                x.Q, x.Kmat, x.V, x.O);
             return hipGetLastError();
         }
     }
     hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, true, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream,
-                       x.M, x.D, col_tiles, tuning().xcd_contiguous, x.scale, x.row_offsets, x.col_indices, x.Q, x.Kmat, x.V,
+                       x.M, x.D, col_tiles, (x.xcd_contiguous | tuning().xcd_contiguous), x.scale, x.row_offsets, x.col_indices, x.Q, x.Kmat, x.V,
                        x.O);
     return hipGetLastError();
 }

@@ -55,6 +55,7 @@ struct SpmmArgs {
     const float* values;
     const float* B;
     float* C;
+    int xcd_contiguous = 0;  // deal the row blocks to the XCDs in contiguous runs (DLSPM_HINT_BANDED)
 };
 struct SddmmArgs {
     int M, K, D, nnz;
@@ -63,6 +64,7 @@ struct SddmmArgs {
     const float* lhs;
     const float* rhs;
     float* out;
+    int xcd_contiguous = 0;
 };
 struct FusedArgs {
     int M, K, D, nnz;
@@ -73,6 +75,7 @@ struct FusedArgs {
     const float* V;
     float scale;
     float* O;
+    int xcd_contiguous = 0;
 };
 
 // Flat schedule: `units` waves of `chunk` consecutive nonzeros each; `bytes` of device workspace for the partial
@@ -108,7 +111,7 @@ hipError_t slice_bounds_launch(int M, int K, int slices, const int* row_offsets,
 hipError_t slice_sum_launch(long long count, int slices, const float* partial, float* out, hipStream_t stream);
 
 // narrow_tiles: the call passes no workspace memory (column tiles below 128 columns are then allowed)
-SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles);
+SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles, bool banded = false);
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
 // Row plan (3 x M ints on the device: first nonzero, end and row number of the row that workgroup i works on): only for
 // shapes of one row per four-wave workgroup and one column tile

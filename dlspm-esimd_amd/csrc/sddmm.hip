@@ -138,12 +138,12 @@ static hipError_t launch_one(const SddmmArgs& x, hipStream_t stream)
     if constexpr (DS > 0) {
         if (x.D == G1 * VEC * DS) {
             hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, false, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M,
-                               x.D, tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+                               x.D, (x.xcd_contiguous | tuning().xcd_contiguous), x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
             return hipGetLastError();
         }
     }
     hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, true, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M, x.D,
-                       tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+                       (x.xcd_contiguous | tuning().xcd_contiguous), x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     return hipGetLastError();
 }
 

@@ -158,12 +158,12 @@ static hipError_t launch_one(const SpmmArgs& x, int tile_major, hipStream_t stre
     {
         if (dense_fits_buffer(x.K, x.N)) {
             hipLaunchKernelGGL((spmm_kernel<VEC, G, V, W, R, true>), dim3((unsigned)blocks), dim3(W * 64), 0, stream, x.M, x.N,
-                               col_tiles, tile_major, tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.values, x.B, x.C);
+                               col_tiles, tile_major, (x.xcd_contiguous | tuning().xcd_contiguous), x.row_offsets, x.col_indices, x.values, x.B, x.C);
             return hipGetLastError();
         }
     }
     hipLaunchKernelGGL((spmm_kernel<VEC, G, V, W, R, false>), dim3((unsigned)blocks), dim3(W * 64), 0, stream, x.M, x.N,
-                       col_tiles, tile_major, tuning().xcd_contiguous, x.row_offsets, x.col_indices, x.values, x.B, x.C);
+                       col_tiles, tile_major, (x.xcd_contiguous | tuning().xcd_contiguous), x.row_offsets, x.col_indices, x.values, x.B, x.C);
     return hipGetLastError();
 }
 
@@ -229,11 +229,12 @@ static int spmm_tile_width(int M, int K, int N, int nnz, bool narrow_tiles)
 }
 
 // Chooses the lane layout from N (and the height of B) and the (W, R) split from the mean row length.
-SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles)
+SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles, bool banded)
 {
     SpmmShape s{};
     s.vec = vec4 ? 4 : 1;
-    const int tile = vec4 ? spmm_tile_width(M, K, N, nnz, narrow_tiles) : 0;
+    // banded (DLSPM_HINT_BANDED): no L2-sized column tiles, each XCD gathers from its own part of B anyway
+    const int tile = vec4 && !banded ? spmm_tile_width(M, K, N, nnz, narrow_tiles) : 0;
     s.tile_major = tile > 0 ? 1 : 0;
     if (vec4) {
         if (tile == 512) { s.G = 64; s.V = 2; }

@@ -25,6 +25,7 @@ OP_SPMM, OP_SDDMM, OP_FUSED = 0, 1, 2
 
 HINT_ROWS_EVEN = 1 << 62
 HINT_ROW_PLAN = 1 << 61
+HINT_BANDED = 1 << 60
 
 
 class _RowsEven:
@@ -235,22 +236,26 @@ def _csr_sizes(row_offsets, col_indices):
     return row_offsets.numel() - 1, col_indices.numel()
 
 
-def _workspace_args(workspace, plan, M):
-    """(pointer, size with hint bits) for the pair (workspace, workspace_bytes) of the three compute entry points."""
+def _workspace_args(workspace, plan, M, banded=False):
+    """(pointer, size with hint bits) for the pair (workspace, workspace_bytes) of the three compute entry points.
+    banded: the caller knows that every row's columns lie in a narrow window that moves with the row (DLSPM_HINT_BANDED)."""
     import torch
 
+    hint = HINT_BANDED if banded else 0
     if plan is not None:
         if workspace is not None:
             raise ValueError("pass a row plan or a workspace, not both")
         need = row_plan_bytes(M) // 4
-        return _ptr(plan, torch.int32, "plan", need), (plan.numel() * 4) | HINT_ROW_PLAN
-    return _workspace(workspace)
+        return _ptr(plan, torch.int32, "plan", need), (plan.numel() * 4) | HINT_ROW_PLAN | hint
+    pointer, size = _workspace(workspace)
+    return pointer, size | hint
 
 
-def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None, plan=None):
+def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None, plan=None, banded=False):
     """C = A_csr @ B on the current stream (spmm_csr_f32). row_offsets/col_indices int32, values/B float32, all on
     the GPU. `workspace`: optional GPU tensor of at least workspace_bytes(OP_SPMM, ...) bytes, or ROWS_EVEN.
-    `plan`: optional row plan of this matrix (row_plan()), passed as the workspace with DLSPM_HINT_ROW_PLAN."""
+    `plan`: optional row plan of this matrix (row_plan()), passed as the workspace with DLSPM_HINT_ROW_PLAN.
+    `banded`: every row's columns lie in a narrow window that moves with the row (DLSPM_HINT_BANDED)."""
     import torch
 
     M, nnz = _csr_sizes(row_offsets, col_indices)
@@ -262,7 +267,7 @@ def spmm(row_offsets, col_indices, values, B, K=None, out=None, workspace=None, 
         raise ValueError(f"B has {Kd} rows, the matrix has K = {K} columns")
     if out is None:
         out = torch.empty((M, N), dtype=torch.float32, device=B.device)
-    wp, wb = _workspace_args(workspace, plan, M)
+    wp, wb = _workspace_args(workspace, plan, M, banded)
     st = lib().spmm_csr_f32(M, K, N, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
                             _ptr(col_indices, torch.int32, "col_indices"), _ptr(values, torch.float32, "values", nnz),
                             _ptr(B, torch.float32, "B"), _ptr(out, torch.float32, "C", M * N), wp, wb, _stream())
@@ -296,7 +301,7 @@ def spmm_static(row_offsets, col_indices, values, B, K=None, out=None):
     return out
 
 
-def sddmm(row_offsets, col_indices, lhs, rhs, out=None, workspace=None, plan=None):
+def sddmm(row_offsets, col_indices, lhs, rhs, out=None, workspace=None, plan=None, banded=False):
     """out[j] = <lhs[i], rhs[col[j]]> for each CSR slot j of row i, on the current stream (sddmm_csr_f32).
     `workspace`: None, ROWS_EVEN, or a GPU tensor of workspace_bytes(OP_SDDMM, ...) bytes (the slice boundaries of the
     column-sliced schedule; 0 bytes where that schedule does not apply). `plan`: a row plan of the mask instead."""
@@ -310,7 +315,7 @@ def sddmm(row_offsets, col_indices, lhs, rhs, out=None, workspace=None, plan=Non
         raise ValueError(f"lhs has {lhs.shape[0]} rows, the mask has {M}")
     if out is None:
         out = torch.empty((nnz,), dtype=torch.float32, device=lhs.device)
-    wp, wb = _workspace_args(workspace, plan, M)
+    wp, wb = _workspace_args(workspace, plan, M, banded)
     st = lib().sddmm_csr_f32(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
                              _ptr(col_indices, torch.int32, "col_indices"), _ptr(lhs, torch.float32, "lhs"),
                              _ptr(rhs, torch.float32, "rhs"), _ptr(out, torch.float32, "out", nnz), wp, wb, _stream())
@@ -319,7 +324,7 @@ def sddmm(row_offsets, col_indices, lhs, rhs, out=None, workspace=None, plan=Non
     return out
 
 
-def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None, workspace=None, plan=None):
+def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None, workspace=None, plan=None, banded=False):
     """O = (S .* (Q Kmat^T) * scale) V on the current stream (fused_sddmm_spmm_f32); the scores are never stored.
     `workspace`: optional GPU tensor of at least workspace_bytes(OP_FUSED, ...) bytes, or ROWS_EVEN.
     `plan`: optional row plan of the mask (row_plan()), passed as the workspace with DLSPM_HINT_ROW_PLAN."""
@@ -333,7 +338,7 @@ def fused(row_offsets, col_indices, Q, Kmat, V, scale=1.0, out=None, workspace=N
         raise ValueError(f"Q has {Q.shape[0]} rows, the mask has {M}")
     if out is None:
         out = torch.empty((M, D), dtype=torch.float32, device=Q.device)
-    wp, wb = _workspace_args(workspace, plan, M)
+    wp, wb = _workspace_args(workspace, plan, M, banded)
     st = lib().fused_sddmm_spmm_f32(M, K, D, nnz, _ptr(row_offsets, torch.int32, "row_offsets"),
                                     _ptr(col_indices, torch.int32, "col_indices"), _ptr(Q, torch.float32, "Q"),
                                     _ptr(Kmat, torch.float32, "Kmat"), _ptr(V, torch.float32, "V"),

@@ -222,14 +222,25 @@ struct WorkspaceChoice {
     size_t bytes = 0;        // device memory to allocate and pass
     bool rows_even = false;  // pass NULL with DLSPM_HINT_ROWS_EVEN instead
     bool plan = false;       // build a row plan and pass it as the workspace, with DLSPM_HINT_ROW_PLAN
+    bool banded = false;     // the pattern is a band (--band without --band-random): DLSPM_HINT_BANDED
     void* arg(void* buffer) const { return bytes ? buffer : nullptr; }
-    size_t size() const { return rows_even ? DLSPM_HINT_ROWS_EVEN : bytes; }
+    size_t size() const { return (rows_even ? DLSPM_HINT_ROWS_EVEN : bytes) | (banded ? DLSPM_HINT_BANDED : 0); }
 };
 inline WorkspaceChoice workspace_to_pass(const Options& opt, int op, int M, int K, int width, int nnz,
-                                         const int* row_offsets_dev, bool plan_allowed = false)
+                                         const int* row_offsets_dev, bool plan_allowed = false, bool banded = false)
 {
     WorkspaceChoice c;
     if (opt.workspace == Options::kNever || M <= 0 || nnz <= 0) return c;
+    if (banded && opt.workspace == Options::kAuto) {
+        // what the generator knows and dlspm_workspace_advice cannot see: no memory, the hint instead
+        int longest = 0, empty = 0;
+        if (dlspm_csr_row_stats(M, row_offsets_dev, nullptr, &longest, &empty) != DLSPM_OK) throw std::runtime_error("dlspm_csr_row_stats failed");
+        c.banded = true;
+        c.rows_even = (long long)longest * 2 * M <= 3ll * nnz;  // longest row at most 1.5 x the mean
+        std::printf("rows: longest %d, mean %.1f, empty %d -> banded, DLSPM_HINT_BANDED passed%s\n", longest, (double)nnz / M, empty,
+                    c.rows_even ? " with DLSPM_HINT_ROWS_EVEN" : "");
+        return c;
+    }
     const size_t want = dlspm_workspace_bytes(op, M, K, width, nnz);
     int longest = 0, empty = 0;
     if (dlspm_csr_row_stats(M, row_offsets_dev, nullptr, &longest, &empty) != DLSPM_OK) throw std::runtime_error("dlspm_csr_row_stats failed");

@@ -44,7 +44,8 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     if (dlspm_csr_check(M, K, nnz, ro_d.p, ci_d.p, nullptr) != DLSPM_OK) throw std::invalid_argument("malformed CSR structure");
     DLSPM_HIP_CHECK(hipMemset(O_d.p, 0xFF, (size_t)M * D * sizeof(float)));
 
-    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_FUSED, M, K, D, nnz, ro_d.p, opt.plan);  // 0 bytes for small problems
+    const bool banded = s.kind == CaseSpec::kShape && s.band > 0 && s.band_random == 0;
+    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_FUSED, M, K, D, nnz, ro_d.p, opt.plan, banded);  // 0 bytes for small problems
     DevBuf<char> ws(wc.bytes);
     if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
     DevBuf<char> plan = wc.plan ? build_row_plan(M, ro_d.p) : DevBuf<char>(0);

@@ -41,7 +41,8 @@ static bool run_case(const CaseSpec& s, const Options& opt)
 
     // SDDMM needs memory only for the slice boundaries of the column-sliced schedule; otherwise the argument only
     // carries what is known about the rows
-    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_SDDMM, M, K, D, nnz, ro_d.p, opt.plan);
+    const bool banded = s.kind == CaseSpec::kShape && s.band > 0 && s.band_random == 0;
+    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_SDDMM, M, K, D, nnz, ro_d.p, opt.plan, banded);
     DevBuf<char> ws(wc.bytes);
     if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
     DevBuf<char> plan = wc.plan ? build_row_plan(M, ro_d.p) : DevBuf<char>(0);

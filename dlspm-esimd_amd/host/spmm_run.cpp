@@ -45,7 +45,8 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     // the caller owns the workspace, as it owns every other buffer: 0 bytes for small problems
     // uneven rows that are not short: a row plan, built once per matrix like the look at the row lengths, hands the
     // rows out by length, one per workgroup (dlspm_row_plan_advice); otherwise what dlspm_workspace_advice says
-    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_SPMM, M, K, N, nnz, ro_d.p, opt.plan);
+    const bool banded = s.kind == CaseSpec::kShape && s.band > 0 && s.band_random == 0;
+    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_SPMM, M, K, N, nnz, ro_d.p, opt.plan, banded);
     DevBuf<char> ws(wc.bytes);
     if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
     const bool planned = wc.plan;

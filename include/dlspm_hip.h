@@ -39,7 +39,7 @@
  *     workspace smaller than that is refused with DLSPM_E_WORKSPACE. The contents need no
  *     initialisation and mean nothing afterwards; two calls that share a workspace must not overlap
  *     in time.
- *   - Two more things travel through the same pair of arguments, as hint bits in the upper byte of `workspace_bytes`
+ *   - Three more things travel through the same pair of arguments, as hint bits in the upper byte of `workspace_bytes`
  *     (DLSPM_HINT_*, or-ed into the size; they are no part of the size):
  *       DLSPM_HINT_ROWS_EVEN, with workspace NULL: the caller knows that no row is much longer than the mean (longest
  *         row at most one and a half times nnz / M). Tall matrices of long rows then run one whole row per wave, which
@@ -49,6 +49,16 @@
  *       DLSPM_HINT_ROW_PLAN: `workspace` holds the row plan of this matrix (dlspm_row_plan_build, below; at least
  *         dlspm_row_plan_bytes(M) bytes, else DLSPM_E_WORKSPACE) and the launch hands the rows out in the plan's order.
  *         The plan is only read.
+ *       DLSPM_HINT_BANDED: the caller knows that the columns of every row lie in a window much narrower than K that
+ *         moves down the columns with the row (sliding-window and block-diagonal attention masks, banded matrices).
+ *         Neighbouring rows then gather neighbouring dense rows: the row blocks are dealt to the XCDs in contiguous
+ *         runs, so that each L2 fetches its own share of the K-side operands and not all of them, and the call runs as
+ *         row blocks whatever memory comes with it (column slices and column tiles are answers to columns spread over
+ *         all of K). Measured on MI355X, K = V = 16384 x 128 floats (8 MiB each), 128 columns per row: the fused op
+ *         104 us as dlspm_workspace_advice, which cannot see the band, says (three column slices), 77 us with NULL,
+ *         74 us with this hint; the L2s fetch 33 MiB per launch instead of 145 MiB. A wrong hint costs time (rows whose
+ *         length depends on their position load the XCDs unevenly), never correctness: the bits are those of the call
+ *         with NULL. May be combined with DLSPM_HINT_ROWS_EVEN; a row plan takes precedence.
  * Calls on different streams may run concurrently from different host threads (each with its own
  * workspace). The library's only mutable state is per host thread (the tuning overrides of dlspm_set_tuning and the
  * last HIP error), a cache of the devices' properties, and the static scratch array of spmm_csr_f32_static.
@@ -74,6 +84,7 @@ extern "C" {
 /* hints, or-ed into `workspace_bytes` (see above); the size proper is workspace_bytes & ~DLSPM_HINT_MASK */
 #define DLSPM_HINT_ROWS_EVEN ((size_t)1 << 62)
 #define DLSPM_HINT_ROW_PLAN  ((size_t)1 << 61)
+#define DLSPM_HINT_BANDED    ((size_t)1 << 60)
 #define DLSPM_HINT_MASK      ((size_t)0xFF << 56)
 
 /* Deprecated spelling of DLSPM_HINT_ROWS_EVEN, still accepted: this constant as `workspace` with workspace_bytes 0.

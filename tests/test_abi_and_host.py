@@ -32,7 +32,7 @@ def test_header_is_plain_c(tmp_path):
                    "int use(void) { int shape[10]; return dlspm_describe_launch(DLSPM_OP_SPMM, 1, 1, 1, 1, shape)"
                    " + (int)dlspm_workspace_bytes(DLSPM_OP_FUSED, 1, 1, 1, 1)"
                    " + spmm_csr_f32(0, 0, 0, 0, 0, 0, 0, 0, 0, DLSPM_ROWS_EVEN, 0, 0)"
-                   " + spmm_csr_f32(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, DLSPM_HINT_ROWS_EVEN | DLSPM_HINT_ROW_PLAN, 0);"
+                   " + spmm_csr_f32(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, DLSPM_HINT_ROWS_EVEN | DLSPM_HINT_ROW_PLAN | DLSPM_HINT_BANDED, 0);"
                    " dlspm_tuning t; dlspm_tuning_default(&t); t.split_w = 4; t.split_r = 1; return dlspm_set_tuning(&t); }\n")
     inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
     r = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-fsyntax-only", "-I", inc, str(src)],

@@ -795,6 +795,47 @@ def test_hint_bits_and_the_deprecated_constant(torch_cuda, dl):
     assert st == dl.OK and torch.equal(via_named, via_alias)
 
 
+def test_banded_hint(torch_cuda, dl, oracle):
+    """DLSPM_HINT_BANDED on a sliding-window mask whose K-side operands exceed one L2, where dlspm_workspace_advice (which
+    cannot see the band) recommends column slices: the call runs as row blocks dealt to the XCDs in contiguous runs,
+    with or without memory, and returns the bits of the call with NULL for SDDMM and the fused op; SpMM drops its
+    L2-sized column tiles (another, equally fixed order of the same sums, so equal to a tile-free launch and within
+    tolerance of the oracle). Combined with the even-rows hint it is that hint's launch."""
+    torch = torch_cuda
+    M = K = 16384
+    D = 128
+    ro, ci = dl.make_pattern(dl.PATTERN_BAND_RANDOM, 91, M, K, 96, 0)
+    lens = np.diff(ro)
+    assert lens.max() <= 96 and (np.abs(ci - np.repeat(np.arange(M), lens)) <= 96).all()
+    nnz = ci.size
+    assert dl.describe_slices(dl.OP_FUSED, M, K, D, nnz)[0] >= 2  # a call with memory (and no hint) would work in column slices
+    rng = np.random.default_rng(92)
+    Q, Km, V = (rng.standard_normal(s, dtype=np.float32) for s in ((M, D), (K, D), (K, D)))
+    va = rng.standard_normal(nnz, dtype=np.float32)
+    ro_d, ci_d, Q_d, Km_d, V_d, va_d = (dev(torch, x) for x in (ro, ci, Q, Km, V, va))
+    # fused and SDDMM: the same bits as with NULL, with and without memory behind the hint
+    for op, run, want in (
+        (dl.OP_FUSED, lambda **kw: dl.fused(ro_d, ci_d, Q_d, Km_d, V_d, 0.125, **kw), lambda: oracle.fused(ro, ci, Q, Km, V, 0.125, omp=True)),
+        (dl.OP_SDDMM, lambda **kw: dl.sddmm(ro_d, ci_d, Q_d, Km_d, **kw), lambda: oracle.sddmm(ro, ci, Q, Km, omp=True)),
+    ):
+        plain = run().cpu().numpy()
+        assert oracle.rel_frobenius(plain, want()) <= TOL
+        assert np.array_equal(run(banded=True).cpu().numpy(), plain)
+        ws = torch.empty(max(dl.workspace_bytes(op, M, K, D, nnz), 16), dtype=torch.uint8, device="cuda")
+        assert np.array_equal(run(banded=True, workspace=ws).cpu().numpy(), plain)
+        even = run(workspace=dl.ROWS_EVEN).cpu().numpy()
+        assert np.array_equal(run(banded=True, workspace=dl.ROWS_EVEN).cpu().numpy(), even)
+    # SpMM: B (8 MiB) would be cut into column tiles; with the hint it is one tile, as tile_major = 0 gives without it
+    want = oracle.spmm(ro, ci, va, Km, omp=True)
+    hinted = dl.spmm(ro_d, ci_d, va_d, Km_d, banded=True).cpu().numpy()
+    assert oracle.rel_frobenius(hinted, want) <= TOL
+    dl.set_tuning(tile_major=0)
+    untiled = dl.spmm(ro_d, ci_d, va_d, Km_d).cpu().numpy()
+    dl.set_tuning()
+    assert np.array_equal(hinted, untiled)
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
 def test_xcd_contiguous_row_blocks_give_the_same_bits(torch_cuda, dl, oracle):
     """dlspm_tuning.xcd_contiguous only changes which workgroup works on which row block (each XCD one contiguous run):
     every row is summed as before, so all three ops return the bits of the default order, also where the number of
