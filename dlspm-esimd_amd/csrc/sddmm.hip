@@ -18,11 +18,12 @@
 
 namespace dlspm {
 
-// Where the results go. Results of more bytes than the device's L2s hold together are stored with the non-temporal
-// hint: ordinary stores allocate their lines in the L2 and push out the rows of rhs that everyone gathers from
-// (24576 x 8192 at density 0.3, 60 million results: D = 32 443 -> 309 us, D = 64 715 -> 525 us, D = 128 1289 -> 1090 us;
-// 80 MB of results: +1 ... 3 %). Small results keep ordinary stores: a kernel ends when its stores have reached memory,
-// and 1 MB of them past the cache cost 5 % (2048 x 2048, D = 128: 5.6 -> 5.9 us).
+// Where the results go. Results of more bytes than one L2 holds are stored with the non-temporal hint: ordinary stores
+// allocate their lines in the L2 and push out the rows of rhs that everyone gathers from (24576 x 8192 at density 0.3,
+// 60 million results: D = 32 443 -> 309 us, D = 64 715 -> 525 us, D = 128 1289 -> 1090 us; 8192 x 2048 at 0.3, 19 MiB:
+// D = 32 32.9 -> 29.2 us, D = 128 90.1 -> 88.0 us; 5 MiB: equal). Small results keep ordinary stores: a kernel ends when
+// its stores have reached memory, and neighbouring waves share cache lines here (2048 x 2048 at 5 %, D = 128, 0.8 MiB:
+// 5.6 -> 5.9 us with the hint).
 struct SampledOut {
     float* __restrict__ at;
     int streaming;
@@ -37,9 +38,7 @@ struct SampledOut {
 };
 static inline SampledOut sampled_out(const SddmmArgs& x)
 {
-    const DeviceInfo& dev = device_info();
-    const long long all_l2 = (dev.cus >= 64 ? dev.cus / 32 : 1) * dev.l2_bytes;  // one L2 per XCD of 32 compute units
-    return SampledOut{x.out, (long long)x.nnz * (long long)sizeof(float) > all_l2 ? 1 : 0};
+    return SampledOut{x.out, (long long)x.nnz * (long long)sizeof(float) > device_info().l2_bytes ? 1 : 0};
 }
 
 // out[j] = <lhs_row, rhs[col_indices[j]]> for the nonzeros j in [p, q) of one row (p < q, wave-uniform).
