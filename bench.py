@@ -12,6 +12,9 @@ events recorded on the launching stream, and the MEDIAN replay gives every figur
 ms_per_step and roofline all come from the same event interval; the host's wall time around the same replay is
 reported separately). R is 5 for K >= 1000 and grows for small K so that a 20-step run is not at the mercy of one
 replay. --no-graph launches the K steps from the host instead (Python + ctypes per launch enter the figure then).
+For K below 1000 a replay's own cost (its start and its drain, about 15 us) is a visible share of K launches of 6 us:
+`timing.steady_state_launch_us` then gives the time per launch between a graph of 2 K and a graph of K steps, and
+`timing.replay_overhead_us` what is left per replay; `value` and `ms_per_step` stay those of the K-step replay.
 
 Prints ONE JSON line:
   value / unit      GFLOP/s with the reference's flop formula (2*nnz - M)*N  (SPMM/spmm-esimd-fromfile2.cpp:253)
@@ -123,9 +126,13 @@ def timed_replays(torch, stream, run, replays):
     return ev, wall
 
 
-def time_steps(torch, step, steps, warmup, replays, use_graph):
-    """{'per_step_s' (median replay), 'wall_per_step_s' (same replay), 'all_us' per replay, 'mode'} for K = `steps`."""
+def time_steps(torch, step, steps, warmup, replays, use_graph, split_overhead=False):
+    """{'per_step_s' (median replay), 'wall_per_step_s' (same replay), 'all_us' per replay, 'mode'} for K = `steps`.
+    split_overhead (graph mode, small K): a graph of 2 K steps is timed the same way, and the difference of the two
+    medians is K steps without what one replay costs by itself ('steady_per_step_s', 'replay_overhead_s'): reported
+    beside the K-step figure, never instead of it."""
     stream = torch.cuda.Stream()
+    extra = {}
     with torch.cuda.stream(stream):
         for _ in range(warmup):
             step()
@@ -133,10 +140,16 @@ def time_steps(torch, step, steps, warmup, replays, use_graph):
         graph = capture(torch, stream, lambda: [step() for _ in range(steps)]) if use_graph else None
         run = graph.replay if graph is not None else (lambda: [step() for _ in range(steps)])
         ev, wall = timed_replays(torch, stream, run, replays)
+        if split_overhead and graph is not None:
+            twice = capture(torch, stream, lambda: [step() for _ in range(2 * steps)])
+            if twice is not None:
+                ev2, _ = timed_replays(torch, stream, twice.replay, replays)
+                m1, m2 = sorted(ev)[replays // 2], sorted(ev2)[replays // 2]
+                extra = {"steady_per_step_s": (m2 - m1) / steps, "replay_overhead_s": 2 * m1 - m2}
     order = sorted(range(replays), key=lambda i: ev[i])
     mid = order[replays // 2]
     return {"per_step_s": ev[mid] / steps, "wall_per_step_s": wall[mid] / steps,
-            "all_us": [round(x / steps * 1e6, 3) for x in ev], "mode": "hipgraph" if graph is not None else "host"}
+            "all_us": [round(x / steps * 1e6, 3) for x in ev], "mode": "hipgraph" if graph is not None else "host", **extra}
 
 
 def cold_launch_us(torch, step, pairs=24, replays=5):
@@ -261,7 +274,7 @@ def measure(dl, torch, np, c, args, steps, warmup, replays, ceiling_gbps, with_c
     acct = dl.account(c["op"], c["M"], c["K"], c["N"], c["nnz"])
     info = {}
     step, out = make_step(dl, torch, c, not args.no_plan, info)
-    t = time_steps(torch, step, steps, warmup, replays, not args.no_graph)
+    t = time_steps(torch, step, steps, warmup, replays, not args.no_graph, split_overhead=steps < 1000)
     s = t["per_step_s"]
     traffic = None
     pmc_path = os.path.join(ROOT, "profiles", "pmc_traffic.json")
@@ -283,6 +296,9 @@ def measure(dl, torch, np, c, args, steps, warmup, replays, ceiling_gbps, with_c
         "frac_of_gather_ceiling": round(eff_gbps / ceiling_gbps, 3) if ceiling_gbps else None,
         "warm_us": round(s * 1e6, 3),
     }
+    if "steady_per_step_s" in t:
+        r["steady_state_launch_us"] = round(t["steady_per_step_s"] * 1e6, 3)
+        r["replay_overhead_us"] = round(t["replay_overhead_s"] * 1e6, 2)
     cold = cold_launch_us(torch, step) if not args.no_graph else None
     r["cold_us"] = cold["us"] if cold else None
     r["cold_detail"] = cold
@@ -344,7 +360,10 @@ def main():
                    "N_or_D": c["N"], "nnz": c["nnz"], "launch": head["launch"], "row_plan": head["row_plan"]},
         "timing": {"clock": "HIP events on the launching stream around each replay of the K-step graph; median replay",
                    "replays": replays, "replay_launch_us": head["replay_launch_us"],
-                   "host_wall_ms_per_step": round(head["host_wall_us_per_step"] * 1e-3, 6)},
+                   "host_wall_ms_per_step": round(head["host_wall_us_per_step"] * 1e-3, 6),
+                   # small K only: what one replay costs beside its K launches (graph of 2 K steps minus graph of K steps)
+                   "steady_state_launch_us": head.get("steady_state_launch_us"),
+                   "replay_overhead_us": head.get("replay_overhead_us")},
         "roofline": head["roofline"],
         "effective_GBps": head["effective_GBps"], "effective_fraction": head["effective_fraction"],
         "effective_bytes": head["effective_bytes"],
