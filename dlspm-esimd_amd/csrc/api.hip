@@ -28,7 +28,7 @@ static int fail_hip(hipError_t e)
 // ---- tuning overrides ------------------------------------------------------------------------------------------------
 // One set per host thread (dlspm_set_tuning). A thread that never called it uses the process default, which is read
 // from the environment exactly once: DLSPM_SPLIT="W,R", DLSPM_FLAT=0|1, DLSPM_FLAT_CHUNK=n, DLSPM_SLICES=0|n,
-// DLSPM_TILE_MAJOR=0|1, DLSPM_TILE_WIDTH=512|..|32, DLSPM_PLAN_ORDER=0|1|2, DLSPM_XCD_CONTIGUOUS=0|1 (so that the drivers can be swept from a
+// DLSPM_TILE_MAJOR=0|1, DLSPM_TILE_WIDTH=512|..|32, DLSPM_PLAN_ORDER=0|1|2, DLSPM_XCD_CONTIGUOUS=0|1, DLSPM_STREAM_RESULTS=0|1 (so that the drivers can be swept from a
 // shell without a rebuild). No launch path reads the environment.
 static Tuning tuning_from_environment()
 {
@@ -51,6 +51,7 @@ static Tuning tuning_from_environment()
     number("DLSPM_TILE_WIDTH", t.tile_width);
     number("DLSPM_PLAN_ORDER", t.plan_order);
     number("DLSPM_XCD_CONTIGUOUS", t.xcd_contiguous);
+    number("DLSPM_STREAM_RESULTS", t.stream_results);
     return t;
 }
 static const Tuning& process_tuning()
@@ -348,7 +349,7 @@ void dlspm_tuning_default(dlspm_tuning* t)
     if (!t) return;
     const Tuning d;
     *t = dlspm_tuning{d.split_w, d.split_r, d.flat, d.flat_chunk, d.slices, d.tile_major, d.tile_width, d.plan_order,
-                      d.xcd_contiguous};
+                      d.xcd_contiguous, d.stream_results};
 }
 
 int dlspm_set_tuning(const dlspm_tuning* t)
@@ -359,7 +360,7 @@ int dlspm_set_tuning(const dlspm_tuning* t)
     }
     if (t->split_w < 0 || t->split_r < 0 || t->flat < -1 || t->flat > 1 || t->flat_chunk < 0 || t->slices < -1 ||
         t->tile_major < -1 || t->tile_major > 1 || t->tile_width < 0 || t->plan_order < 0 || t->plan_order > 2 ||
-        t->xcd_contiguous < 0 || t->xcd_contiguous > 1)
+        t->xcd_contiguous < 0 || t->xcd_contiguous > 1 || t->stream_results < -1 || t->stream_results > 1)
         return DLSPM_E_INVALID_ARG;
     t_tuning.split_w = t->split_w;
     t_tuning.split_r = t->split_r;
@@ -370,6 +371,7 @@ int dlspm_set_tuning(const dlspm_tuning* t)
     t_tuning.tile_width = t->tile_width;
     t_tuning.plan_order = t->plan_order;
     t_tuning.xcd_contiguous = t->xcd_contiguous;
+    t_tuning.stream_results = t->stream_results;
     t_tuning_set = true;
     return DLSPM_OK;
 }
@@ -379,7 +381,7 @@ int dlspm_get_tuning(dlspm_tuning* t)
     if (!t) return DLSPM_E_INVALID_ARG;
     const Tuning& c = tuning();
     *t = dlspm_tuning{c.split_w, c.split_r, c.flat, c.flat_chunk, c.slices, c.tile_major, c.tile_width, c.plan_order,
-                      c.xcd_contiguous};
+                      c.xcd_contiguous, c.stream_results};
     return DLSPM_OK;
 }
 

@@ -260,6 +260,7 @@ struct RowBlock {
     static_assert(!PLANNED || (SLICED && R == 1), "a row plan names one row per workgroup");
     int lane, w;
     int rows_total;  // rows of the matrix
+    int stream_rule;  // results with the non-temporal hint: 0 by the size rule, 1 never, 2 always (launch flags, bits 1-2)
     int nr;    // rows in this block (fewer than R at the end of the matrix)
     int row0;  // row of the dense operands and of the output that belongs to the block's first row
     int off_lo, off_hi, off_win, start_lo, start_win;
@@ -267,18 +268,20 @@ struct RowBlock {
     bool aligned;          // the row-aligned split is in use (the same for every wave of the workgroup)
 
     // `prefetch()` is called right after the offsets were requested: what it asks for arrives in the same round trip
-    // `xcd_contiguous` (plain row blocks in one column tile only): workgroup 8 i + x runs on XCD x, as the hardware deals
-    // them; it then takes row block i of XCD x's own contiguous run of row blocks instead of row block 8 i + x.
+    // `flags`: the launch flags (launch.hpp). Bit 0, XCD-contiguous (plain row blocks in one column tile only): workgroup
+    // 8 i + x runs on XCD x, as the hardware deals them; it then takes row block i of XCD x's own contiguous run of row
+    // blocks instead of row block 8 i + x.
     template <typename Prefetch>
     __device__ __forceinline__ void load(int rb, int M, int nnz, const int* __restrict__ row_offsets,
                                          const int* __restrict__ row_ends, const int* __restrict__ row_ids,
-                                         Prefetch&& prefetch, int xcd_contiguous = 0)
+                                         Prefetch&& prefetch, int flags = 0)
     {
         lane = threadIdx.x & 63;
         w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
         rows_total = M;
+        stream_rule = (flags >> 1) & 3;
         if constexpr (!SLICED && !PLANNED) {
-            if (xcd_contiguous) {
+            if (flags & 1) {
                 const int nb = (M - 1) / R + 1, x = rb & 7, each = nb >> 3, extra = nb & 7;
                 rb = x * each + min(x, extra) + (rb >> 3);  // XCD x owns each + (x < extra) row blocks
             }
@@ -388,8 +391,8 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
     auto s_off = [&](int i) { return blk.off(i); };
     const int T0 = blk.T0, T = blk.T, per = blk.per, a = blk.a;
     // Results of kStreamedOutputFloats and more are stored with the non-temporal hint: they are written once, and
-    // ordinary stores allocate their lines in the L2 beside the dense rows that are gathered from it, to be written
-    // back when the kernel ends. Measured (SpMM): 2048 x 512, N = 256 (2 MiB) 6.07 -> 5.96 us; 16384 x 4096 at 10 %,
+    // ordinary stores are held in the L2 as dirty lines to be written back later, where hinted ones drain as they are
+    // issued (hits, misses and fetched bytes of the L2 stay the same; the time does not). Measured (SpMM): 2048 x 512, N = 256 (2 MiB) 6.07 -> 5.96 us; 16384 x 4096 at 10 %,
     // N = 128 (8 MiB) 133 -> 128 us; 65536 x 1024 at 2 %, N = 256 (64 MiB) 52.5 -> 49.7 us; 131072 x 512, N = 128
     // 41.6 -> 39.1 us. Smaller results lose by it when rows end inside a cache line (512 x 2048, N = 49: 4.72 -> 5.04 us;
     // 2048 x 1024, N = 33: 4.66 -> 5.03 us). Not for the partial rows of the column-sliced schedule, which are read again.
@@ -397,8 +400,10 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
     // fused 9.60 -> 9.35 us).
     constexpr long long kStreamedOutputFloats = 512 * 1024, kStreamedWholeLineFloats = 128 * 1024;
     const long long out_floats = (long long)blk.rows_total * width;
-    const bool streaming = (!SLICED || PLANNED) &&
-                           (out_floats >= kStreamedOutputFloats || (width % 32 == 0 && out_floats >= kStreamedWholeLineFloats));
+    // (dlspm_tuning.stream_results switches the rule off or on for sweeps and tests: blk.stream_rule)
+    const bool streaming = (!SLICED || PLANNED) && blk.stream_rule != 1 &&
+                           (blk.stream_rule == 2 || out_floats >= kStreamedOutputFloats ||
+                            (width % 32 == 0 && out_floats >= kStreamedWholeLineFloats));
 
     blk.for_each_segment([&](int r, int p, int q, int rs, int re) {
         VecT acc[V];

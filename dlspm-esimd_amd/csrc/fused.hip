@@ -63,14 +63,14 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
                                             const int* __restrict__ col_indices, const float* __restrict__ Q,
                                             const float* __restrict__ Kmat, const float* __restrict__ Vmat,
                                             float* __restrict__ O, const int* __restrict__ row_ids = nullptr, int nnz = 0,
-                                            int xcd_contiguous = 0)
+                                            int flags = 0)
 {
     const int row_blocks = (M - 1) / R + 1;
     const int ct = col_tiles == 1 ? 0 : bid / row_blocks;
     const int rb = bid - ct * row_blocks;
     RowBlock<W, R, SLICED, PLANNED> blk;
     blk.load(rb, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, Q, Kmat, Vmat, O); },
-             col_tiles == 1 ? xcd_contiguous : 0);
+             col_tiles == 1 ? flags : flags & ~1);
     dense_rows_block<VEC, G, V2>(blk, ct, D, O, [&](Vec<VEC>* acc, int r, int p, int q, const int* colv) {
         const float* q_row = Q + (size_t)(blk.row0 + r) * D;
         fused_segment<VEC, G1, DS, MASKED, G, V2>(acc, p, q, D, scale, col_indices, q_row, Kmat, Vmat, colv, blk.lane);
@@ -79,14 +79,14 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
 
 // MASKED = false: D == G1 * VEC * DS exactly, every stage-1 access of every lane falls inside the row.
 template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R>
-__global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_tiles, int xcd_contiguous, float scale,
+__global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_tiles, int flags, float scale,
                                                        const int* __restrict__ row_offsets,
                                                        const int* __restrict__ col_indices,
                                                        const float* __restrict__ Q, const float* __restrict__ Kmat,
                                                        const float* __restrict__ Vmat, float* __restrict__ O)
 {
     fused_block<VEC, G1, DS, MASKED, G, V2, W, R, false>((int)blockIdx.x, M, D, col_tiles, scale, row_offsets, nullptr,
-                                                         col_indices, Q, Kmat, Vmat, O, nullptr, 0, xcd_contiguous);
+                                                         col_indices, Q, Kmat, Vmat, O, nullptr, 0, flags);
 }
 
 // Column-sliced schedule (see spmm_sliced_kernel): the row blocks once per slice of columns, slice after slice, so
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(4 * 64) void fused_sliced_kernel(int M, int D, int 
 // Row plan: workgroup i works on the whole row rows[i] = [starts[i], ends[i]) (one row per four-wave workgroup, one
 // column tile).
 template <int VEC, int G1, int DS, bool MASKED, int G, int V2>
-__global__ __launch_bounds__(4 * 64) void fused_planned_kernel(int M, int D, int nnz, float scale,
+__global__ __launch_bounds__(4 * 64) void fused_planned_kernel(int M, int D, int nnz, int flags, float scale,
                                                                const int* __restrict__ starts, const int* __restrict__ ends,
                                                                const int* __restrict__ rows,
                                                                const int* __restrict__ col_indices,
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(4 * 64) void fused_planned_kernel(int M, int D, int
                                                                const float* __restrict__ Vmat, float* __restrict__ O)
 {
     fused_block<VEC, G1, DS, MASKED, G, V2, 4, 1, true, true>((int)blockIdx.x, M, D, 1, scale, starts, ends, col_indices, Q,
-                                                              Kmat, Vmat, O, rows, nnz);
+                                                              Kmat, Vmat, O, rows, nnz, flags);
 }
 
 // ---- host side --------------------------------------------------------------------------------------
@@ -134,13 +134,13 @@ static hipError_t launch_one(const FusedArgs& x, hipStream_t stream)
     if constexpr (DS > 0) {
         if (x.D == G1 * VEC * DS) {
             hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, false, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64),
-                               0, stream, x.M, x.D, col_tiles, (x.xcd_contiguous | tuning().xcd_contiguous), x.scale, x.row_offsets, x.col_indices,
+                               0, stream, x.M, x.D, col_tiles, launch_flags(x.xcd_contiguous), x.scale, x.row_offsets, x.col_indices,
                                x.Q, x.Kmat, x.V, x.O);
             return hipGetLastError();
         }
     }
     hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, true, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream,
-                       x.M, x.D, col_tiles, (x.xcd_contiguous | tuning().xcd_contiguous), x.scale, x.row_offsets, x.col_indices, x.Q, x.Kmat, x.V,
+                       x.M, x.D, col_tiles, launch_flags(x.xcd_contiguous), x.scale, x.row_offsets, x.col_indices, x.Q, x.Kmat, x.V,
                        x.O);
     return hipGetLastError();
 }
@@ -387,10 +387,10 @@ static hipError_t launch_planned(const FusedArgs& x, const int* plan, hipStream_
     const int *starts = plan, *ends = plan + x.M, *rows = plan + 2 * (size_t)x.M;
     if (x.D == 8 * 4 * DS)
         hipLaunchKernelGGL((fused_planned_kernel<4, 8, DS, false, G, V2>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M,
-                           x.D, x.nnz, x.scale, starts, ends, rows, x.col_indices, x.Q, x.Kmat, x.V, x.O);
+                           x.D, x.nnz, launch_flags(0), x.scale, starts, ends, rows, x.col_indices, x.Q, x.Kmat, x.V, x.O);
     else
         hipLaunchKernelGGL((fused_planned_kernel<4, 8, DS, true, G, V2>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M,
-                           x.D, x.nnz, x.scale, starts, ends, rows, x.col_indices, x.Q, x.Kmat, x.V, x.O);
+                           x.D, x.nnz, launch_flags(0), x.scale, starts, ends, rows, x.col_indices, x.Q, x.Kmat, x.V, x.O);
     return hipGetLastError();
 }
 

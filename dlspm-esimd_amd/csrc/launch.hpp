@@ -35,8 +35,20 @@ struct Tuning {
     int tile_major = -1, tile_width = 0;
     int plan_order = 0;
     int xcd_contiguous = 0;
+    int stream_results = -1;
 };
 const Tuning& tuning();
+
+// What a row-block kernel is told about its launch in one int: bit 0 = deal the row blocks to the XCDs in contiguous
+// runs (DLSPM_HINT_BANDED or the tuning knob), bits 1-2 = results with the non-temporal hint: 0 by the size rule,
+// 1 never, 2 wherever the rule could say so (dlspm_tuning.stream_results).
+constexpr int kFlagXcdContiguous = 1, kFlagStreamShift = 1, kFlagStreamNever = 1, kFlagStreamAlways = 2;
+inline int launch_flags(int xcd_contiguous_hint)
+{
+    const Tuning& t = tuning();
+    const int stream = t.stream_results < 0 ? 0 : t.stream_results == 0 ? kFlagStreamNever : kFlagStreamAlways;
+    return ((xcd_contiguous_hint | t.xcd_contiguous) ? kFlagXcdContiguous : 0) | (stream << kFlagStreamShift);
+}
 
 // Lane layout and work split of one launch.
 //   vec : floats per lane per access (4 = dwordx4 when the dense width is at least 4, else 1 = dword)

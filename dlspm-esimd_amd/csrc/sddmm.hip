@@ -19,8 +19,9 @@
 namespace dlspm {
 
 // Where the results go. Results of more bytes than one L2 holds are stored with the non-temporal hint: ordinary stores
-// allocate their lines in the L2 and push out the rows of rhs that everyone gathers from (24576 x 8192 at density 0.3,
-// 60 million results: D = 32 443 -> 309 us, D = 64 715 -> 525 us, D = 128 1289 -> 1090 us; 8192 x 2048 at 0.3, 19 MiB:
+// are held in the L2 as dirty lines and written back later, hinted ones drain as they are issued. (The L2's hit rate
+// and the bytes fetched do not change by it; the time does.) Measured: 24576 x 8192 at density 0.3,
+// 60 million results, D = 32 443 -> 309 us, D = 64 715 -> 525 us, D = 128 1289 -> 1090 us; 8192 x 2048 at 0.3, 19 MiB:
 // D = 32 32.9 -> 29.2 us, D = 128 90.1 -> 88.0 us; 5 MiB: equal). Small results keep ordinary stores: a kernel ends when
 // its stores have reached memory, and neighbouring waves share cache lines here (2048 x 2048 at 5 %, D = 128, 0.8 MiB:
 // 5.6 -> 5.9 us with the hint).
@@ -38,7 +39,9 @@ struct SampledOut {
 };
 static inline SampledOut sampled_out(const SddmmArgs& x)
 {
-    return SampledOut{x.out, (long long)x.nnz * (long long)sizeof(float) > device_info().l2_bytes ? 1 : 0};
+    const int forced = tuning().stream_results;  // -1: the size rule (sweeps and tests switch it off or on)
+    const bool by_rule = (long long)x.nnz * (long long)sizeof(float) > device_info().l2_bytes;
+    return SampledOut{x.out, (forced < 0 ? by_rule : forced != 0) ? 1 : 0};
 }
 
 // out[j] = <lhs_row, rhs[col_indices[j]]> for the nonzeros j in [p, q) of one row (p < q, wave-uniform).
@@ -78,10 +81,10 @@ __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __
                                             const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                             const float* __restrict__ lhs, const float* __restrict__ rhs,
                                             SampledOut out, const int* __restrict__ row_ids = nullptr, int nnz = 0,
-                                            int xcd_contiguous = 0)
+                                            int flags = 0)
 {
     RowBlock<W, R, SLICED, PLANNED> blk;
-    blk.load(bid, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, lhs, rhs, out.at); }, xcd_contiguous);
+    blk.load(bid, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, lhs, rhs, out.at); }, flags);
     blk.for_each_segment([&](int r, int p, int q, int, int) {
         const float* lhs_row = lhs + (size_t)(blk.row0 + r) * D;
         const int shift = blk.shift(r);
@@ -91,13 +94,13 @@ __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __
 
 // MASKED = false: D == G1 * VEC * DS exactly, every access of every lane falls inside the row.
 template <int VEC, int G1, int DS, bool MASKED, int W, int R>
-__global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, int xcd_contiguous, const int* __restrict__ row_offsets,
+__global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, int flags, const int* __restrict__ row_offsets,
                                                        const int* __restrict__ col_indices,
                                                        const float* __restrict__ lhs, const float* __restrict__ rhs,
                                                        SampledOut out)
 {
     sddmm_block<VEC, G1, DS, MASKED, W, R, false>((int)blockIdx.x, M, D, row_offsets, nullptr, col_indices, lhs, rhs, out,
-                                                  nullptr, 0, xcd_contiguous);
+                                                  nullptr, 0, flags);
 }
 
 // Column-sliced schedule (see spmm_sliced_kernel): the row blocks once per slice of columns, slice after slice, so that
@@ -137,12 +140,12 @@ static hipError_t launch_one(const SddmmArgs& x, hipStream_t stream)
     if constexpr (DS > 0) {
         if (x.D == G1 * VEC * DS) {
             hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, false, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M,
-                               x.D, (x.xcd_contiguous | tuning().xcd_contiguous), x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+                               x.D, launch_flags(x.xcd_contiguous), x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
             return hipGetLastError();
         }
     }
     hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, true, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M, x.D,
-                       (x.xcd_contiguous | tuning().xcd_contiguous), x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+                       launch_flags(x.xcd_contiguous), x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     return hipGetLastError();
 }
 

@@ -82,7 +82,7 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
                                            const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                            const float* __restrict__ values, const float* __restrict__ B,
                                            float* __restrict__ C, const int* __restrict__ row_ids = nullptr, int nnz = 0,
-                                           int xcd_contiguous = 0)
+                                           int flags = 0)
 {
     int ct = 0, rb = bid;
     if (col_tiles != 1) {
@@ -97,7 +97,7 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
     }
     RowBlock<W, R, SLICED, PLANNED> blk;
     blk.load(rb, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, values, B, C); },
-             col_tiles == 1 ? xcd_contiguous : 0);
+             col_tiles == 1 ? flags : flags & ~1);
     dense_rows_block<VEC, G, V>(blk, ct, N, C, [&](Vec<VEC>* acc, int, int p, int q, const int* colv) {
         spmm_segment<VEC, G, V, BUF>(acc, p, q, col_indices, values, B, N, colv, blk.lane);
     });
@@ -105,14 +105,14 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
 
 // BUF: B is read through a buffer descriptor (B below 4 GiB: see dense_rows_fma)
 template <int VEC, int G, int V, int W, int R, bool BUF>
-__global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tiles, int tile_major, int xcd_contiguous,
+__global__ __launch_bounds__(W * 64) void spmm_kernel(int M, int N, int col_tiles, int tile_major, int flags,
                                                       const int* __restrict__ row_offsets,
                                                       const int* __restrict__ col_indices,
                                                       const float* __restrict__ values,
                                                       const float* __restrict__ B, float* __restrict__ C)
 {
     spmm_block<VEC, G, V, W, R, false, false, BUF>((int)blockIdx.x, M, N, col_tiles, tile_major, row_offsets, nullptr,
-                                                   col_indices, values, B, C, nullptr, 0, xcd_contiguous);
+                                                   col_indices, values, B, C, nullptr, 0, flags);
 }
 
 // Column-sliced schedule: the grid holds the row blocks once per slice of columns, slice after slice, so that at
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(4 * 64) void spmm_sliced_kernel(int M, int N, int c
 // Row plan: workgroup i works on the whole row rows[i] = [starts[i], ends[i]) of the CSR matrix (one row per four-wave
 // workgroup); with column tiles the plan is gone through once per tile, tile after tile.
 template <int VEC, int G, int V, bool BUF>
-__global__ __launch_bounds__(4 * 64) void spmm_planned_kernel(int M, int N, int nnz, int col_tiles,
+__global__ __launch_bounds__(4 * 64) void spmm_planned_kernel(int M, int N, int nnz, int col_tiles, int flags,
                                                               const int* __restrict__ starts,
                                                               const int* __restrict__ ends, const int* __restrict__ rows,
                                                               const int* __restrict__ col_indices,
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(4 * 64) void spmm_planned_kernel(int M, int N, int 
                                                               const float* __restrict__ B, float* __restrict__ C)
 {
     spmm_block<VEC, G, V, 4, 1, true, true, BUF>((int)blockIdx.x, M, N, col_tiles, 1, starts, ends, col_indices, values, B, C,
-                                                 rows, nnz);
+                                                 rows, nnz, flags);
 }
 
 // ---- host side --------------------------------------------------------------------------------------
@@ -158,12 +158,12 @@ static hipError_t launch_one(const SpmmArgs& x, int tile_major, hipStream_t stre
     {
         if (dense_fits_buffer(x.K, x.N)) {
             hipLaunchKernelGGL((spmm_kernel<VEC, G, V, W, R, true>), dim3((unsigned)blocks), dim3(W * 64), 0, stream, x.M, x.N,
-                               col_tiles, tile_major, (x.xcd_contiguous | tuning().xcd_contiguous), x.row_offsets, x.col_indices, x.values, x.B, x.C);
+                               col_tiles, tile_major, launch_flags(x.xcd_contiguous), x.row_offsets, x.col_indices, x.values, x.B, x.C);
             return hipGetLastError();
         }
     }
     hipLaunchKernelGGL((spmm_kernel<VEC, G, V, W, R, false>), dim3((unsigned)blocks), dim3(W * 64), 0, stream, x.M, x.N,
-                       col_tiles, tile_major, (x.xcd_contiguous | tuning().xcd_contiguous), x.row_offsets, x.col_indices, x.values, x.B, x.C);
+                       col_tiles, tile_major, launch_flags(x.xcd_contiguous), x.row_offsets, x.col_indices, x.values, x.B, x.C);
     return hipGetLastError();
 }
 
@@ -479,10 +479,10 @@ hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int*
         if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;                                                \
         if (dense_fits_buffer(x.K, x.N))                                                                               \
             hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_, true>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, \
-                               x.M, x.N, x.nnz, col_tiles, starts, ends, rows, x.col_indices, x.values, x.B, x.C);     \
+                               x.M, x.N, x.nnz, col_tiles, launch_flags(0), starts, ends, rows, x.col_indices, x.values, x.B, x.C);     \
         else                                                                                                           \
             hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_, false>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, \
-                               x.M, x.N, x.nnz, col_tiles, starts, ends, rows, x.col_indices, x.values, x.B, x.C);     \
+                               x.M, x.N, x.nnz, col_tiles, launch_flags(0), starts, ends, rows, x.col_indices, x.values, x.B, x.C);     \
         return hipGetLastError();                                                                                      \
     }
     DLSPM_PLANNED(64, 2)

@@ -70,7 +70,7 @@ EXPORTS = (
 class Tuning(ctypes.Structure):
     """dlspm_tuning of include/dlspm_hip.h."""
     _fields_ = [(n, ctypes.c_int) for n in ("split_w", "split_r", "flat", "flat_chunk", "slices", "tile_major",
-                                            "tile_width", "plan_order", "xcd_contiguous")]
+                                            "tile_width", "plan_order", "xcd_contiguous", "stream_results")]
 
 
 class DlspmError(RuntimeError):
@@ -151,7 +151,7 @@ def version() -> str:
 
 def set_tuning(**fields) -> None:
     """Overrides of the launch rules for the calling thread (dlspm_set_tuning): split=(W, R), flat, flat_chunk, slices,
-    tile_major, tile_width, plan_order; fields not named follow the rules. No argument: back to the process default."""
+    tile_major, tile_width, plan_order, xcd_contiguous, stream_results; fields not named follow the rules. No argument: back to the process default."""
     if not fields:
         st = lib().dlspm_set_tuning(None)
     else:

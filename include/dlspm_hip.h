@@ -282,7 +282,7 @@ int dlspm_describe_slices(int op, int M, int K, int N_or_D, int nnz, int* slices
  * thread: dlspm_set_tuning changes the calling thread's, NULL goes back to the process default. That default is the
  * rules themselves unless the environment said otherwise when the library first looked, once per process:
  * DLSPM_SPLIT="W,R", DLSPM_FLAT, DLSPM_FLAT_CHUNK, DLSPM_SLICES, DLSPM_TILE_MAJOR, DLSPM_TILE_WIDTH, DLSPM_PLAN_ORDER,
- * DLSPM_XCD_CONTIGUOUS
+ * DLSPM_XCD_CONTIGUOUS, DLSPM_STREAM_RESULTS
  * (so that the drivers can be swept from a shell). No launch reads the environment. An override that names a shape
  * the kernels are not built for is ignored. dlspm_workspace_bytes and the describe calls follow the overrides, so
  * set them before sizing a workspace. No counterpart in the reference (its knobs are -D macros, SPMM/spmmesimd.hpp:17-21).
@@ -300,6 +300,9 @@ typedef struct dlspm_tuning {
                           /* mask gathers a different eighth of the dense operands into each L2 (4x fewer bytes       */
                           /* fetched, 6 % faster on a 16384-row band; unsafe as a rule: rows whose length depends on   */
                           /* their position would load the XCDs unevenly). One column tile, no row plan, no slices.   */
+                          /* (DLSPM_HINT_BANDED asks for the same per call.)                                          */
+    int stream_results;   /* results stored with the non-temporal hint: -1 the size rule (SDDMM: more than one L2's    */
+                          /* worth; dense rows: from 2 MiB, whole cache lines from 0.5 MiB), 0 never, 1 always         */
 } dlspm_tuning;
 void dlspm_tuning_default(dlspm_tuning* t);   /* fills *t with "follow the rules" */
 int dlspm_set_tuning(const dlspm_tuning* t);  /* DLSPM_OK or DLSPM_E_INVALID_ARG (a field out of range) */

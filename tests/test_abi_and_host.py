@@ -247,7 +247,7 @@ def test_tuning_overrides_go_through_one_call_and_the_environment_is_read_once(d
 
     base = dl.get_tuning()
     assert base == {"split_w": 0, "split_r": 0, "flat": -1, "flat_chunk": 0, "slices": -1, "tile_major": -1,
-                    "tile_width": 0, "plan_order": 0, "xcd_contiguous": 0}
+                    "tile_width": 0, "plan_order": 0, "xcd_contiguous": 0, "stream_results": -1}
     sizes = (dl.OP_SPMM, 8192, 4096, 128, 8192 * 600)
     rule = dl.describe_launch(*sizes)
     assert (rule["W"], rule["R"]) == (4, 1)
@@ -271,7 +271,7 @@ def test_tuning_overrides_go_through_one_call_and_the_environment_is_read_once(d
     assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (128, 4)
     dl.set_tuning()
     for bad in ({"flat": 2}, {"slices": -2}, {"plan_order": 3}, {"tile_major": 5}, {"split": (-1, 0)}, {"flat_chunk": -64},
-                {"xcd_contiguous": 2}):
+                {"xcd_contiguous": 2}, {"stream_results": 2}, {"stream_results": -2}):
         with pytest.raises(dl.DlspmError):
             dl.set_tuning(**bad)
     assert dl.get_tuning() == base

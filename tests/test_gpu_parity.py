@@ -795,6 +795,45 @@ def test_hint_bits_and_the_deprecated_constant(torch_cuda, dl):
     assert st == dl.OK and torch.equal(via_named, via_alias)
 
 
+def test_streamed_results_have_the_bits_of_ordinary_stores(torch_cuda, dl, oracle):
+    """Large results are stored with the non-temporal hint (instructions written out in the kernels); the size rule
+    switches it on only for results of megabytes. dlspm_tuning.stream_results forces it for any size: every width from 1
+    float (dword stores) over widths that are no multiple of 4 (rows that end inside a cache line, lanes that store the
+    same columns twice) to column tiles, empty rows, shared rows, row plans and grouped rows must give the bits of the
+    run with ordinary stores, for all three ops."""
+    torch = torch_cuda
+    rng = np.random.default_rng(77)
+    cases = [("skewed", 300, 200, 1, 0.1), ("uniform", 257, 100, 3, 0.2), ("empty_rows", 1000, 300, 5, 0.1), ("skewed", 2048, 512, 49, 0.1),
+             ("uniform", 700, 256, 64, 0.2), ("skewed", 513, 700, 129, 0.05), ("empty_rows", 2051, 512, 256, 0.1), ("uniform", 64, 147, 1030, 0.3),
+             ("skewed", 9000, 256, 33, 0.05), ("full", 40, 300, 196, 1.0)]
+    for kind, M, K, N, den in cases:
+        ro, ci = random_csr(rng, M, K, kind, den)
+        va = rng.normal(0, 1, ci.size).astype(np.float32)
+        B = rng.normal(0, 1, (K, N)).astype(np.float32)
+        Q = rng.normal(0, 1, (M, N)).astype(np.float32)
+        V = rng.normal(0, 1, (K, N)).astype(np.float32)
+        ro_d, ci_d, va_d, B_d, Q_d, V_d = (dev(torch, x) for x in (ro, ci, va, B, Q, V))
+        plan = dl.row_plan(ro_d)
+        runs = {
+            "spmm": lambda **kw: dl.spmm(ro_d, ci_d, va_d, B_d, K=K, **kw),
+            "sddmm": lambda **kw: dl.sddmm(ro_d, ci_d, Q_d, B_d, **kw),
+            "fused": lambda **kw: dl.fused(ro_d, ci_d, Q_d, B_d, V_d, 0.25, **kw),
+        }
+        for op, run in runs.items():
+            for schedule in ({}, {"workspace": dl.ROWS_EVEN}, {"plan": plan}):
+                dl.set_tuning(stream_results=0)
+                plain = run(**schedule).cpu().numpy()
+                dl.set_tuning(stream_results=1)
+                streamed = run(**schedule).cpu().numpy()
+                dl.set_tuning()
+                assert np.array_equal(plain, streamed), (op, kind, M, K, N, list(schedule))
+        want = oracle.spmm(ro, ci, va, B, omp=True)
+        dl.set_tuning(stream_results=1)
+        assert oracle.rel_frobenius(dl.spmm(ro_d, ci_d, va_d, B_d, K=K).cpu().numpy(), want) <= TOL
+        dl.set_tuning()
+        check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
 def test_banded_hint(torch_cuda, dl, oracle):
     """DLSPM_HINT_BANDED on a sliding-window mask whose K-side operands exceed one L2, where dlspm_workspace_advice (which
     cannot see the band) recommends column slices: the call runs as row blocks dealt to the XCDs in contiguous runs,

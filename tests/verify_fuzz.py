@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Seeded random cases against the CPU oracle: odd shapes and widths, four kinds of row-length distribution, every
 schedule, with the library's launch rules overridden at random (dlspm_set_tuning: work split, flat schedule and its
-chunk, column slices, tile order and width, plan order, XCD-contiguous row blocks).
+chunk, column slices, tile order and width, plan order, XCD-contiguous row blocks, streamed results).
 
     python tests/verify_fuzz.py [--cases 1000] [--seed 1] [--report out.txt]
 
@@ -46,6 +46,8 @@ def random_tuning(rng):
         t["plan_order"] = pick([0, 1, 2])
     if rng.random() < 0.5:
         t["xcd_contiguous"] = 1
+    if rng.random() < 0.5:
+        t["stream_results"] = pick([0, 1])
     return t
 
 
