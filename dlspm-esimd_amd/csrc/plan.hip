@@ -4,7 +4,7 @@
 // A planned launch runs one row per four-wave workgroup. Workgroups are dispatched in index order, so the rows that
 // take longest should come first, and the first 8 x bins workgroups (bins = compute units of the device) all start at
 // once, workgroup i of them on compute unit i mod bins: those rows ("the head") are packed into `bins` bins of equal
-// size, longest row first into the least loaded bin that still has room, and bin b becomes the workgroups b, b + bins,
+// size, longest row first into the least loaded bin (of its group, see below) that still has room, and bin b becomes the workgroups b, b + bins,
 // b + 2 bins, ... so that a compute unit's rows add up to about the same number of nonzeros. The rows after the head
 // follow longest first (whatever compute unit frees up takes the longest row left).
 //
@@ -15,11 +15,12 @@
 //   sort     longest first and by row number among equals: a bitonic network over the 2048 keys of a tile, two per
 //            thread in registers (32-bit keys; 64-bit keys in LDS when a row has 2^21 nonzeros or more); merging by rank
 //            (every key finds its place in the sibling run by binary search).
-//   packing  exactly the sequential rule above, but in batches: with the bins sorted by (load, bin), the next rows go
-//            to the bins in that order for as long as no bin that already received a row of this batch would have
-//            been the least loaded one again; each batch is found in parallel (one search per bin in the sorted bins)
-//            and the sorted order is carried from batch to batch. Rows without nonzeros fill the positions that are
-//            left, in order.
+//   packing  the bins in groups of at most 64, one wave per group (sorted row t and bin b in group t % groups and
+//            b % groups), each group exactly by the sequential rule above, but in batches: with the bins sorted by
+//            (load, bin), the next rows go to the bins in that order for as long as no bin that already received a row of
+//            this batch would have been the least loaded one again; each batch is found in parallel (one search per bin
+//            in the sorted bins) and the sorted order is carried from batch to batch. Rows without nonzeros fill the
+//            positions that are left, in order.
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -246,31 +247,35 @@ template <> struct BinKey<u64> {
     static __device__ __forceinline__ u64 make(int load, int bin) { return ((u64)(unsigned)load << 32) | (u64)bin; }
 };
 
-constexpr int kSortedPad = 64;  // the search below looks up to 63 places past the last key
-template <typename Word> struct PackKeys {
-    alignas(16) Word sorted[2][kPlanMaxBins + kSortedPad];  // the keys of the bins that can take a row, ascending, then all ones
-    alignas(16) Word fresh[kPlanMaxBins];                   // the new keys of the bins of one batch
+// The bins are packed in groups of at most kGroupBins, one wave per group, each lane of the wave keeping the books of
+// one bin: sorted row t and bin b belong to group t % groups and b % groups. A group's rows are every groups-th of the
+// sorted rows, so the groups hold the same mix of long and short rows, and what is lost against packing all bins
+// together is small (the benchmark matrix: heaviest bin 451 nonzeros instead of 445, mean 413) beside what is won:
+// nothing in the loop below leaves the wave -- no workgroup barrier, the ranking of 64 keys instead of 256.
+constexpr int kGroupBins = 64;
+__host__ __device__ inline int plan_groups(int bins)
+{
+    int groups = (bins + kGroupBins - 1) / kGroupBins;
+    while (bins % groups != 0) ++groups;  // so that row t's group, (t % bins) % groups, is t % groups
+    return groups;
+}
+
+constexpr int kSortedPad = 8;
+template <typename Word> struct GroupKeys {
+    alignas(16) Word sorted[kGroupBins + kSortedPad];  // the keys of the bins that can take a row, ascending, then all ones
+    alignas(16) Word fresh[kGroupBins];                // the new keys of the bins of one batch
 };
 struct PackShared {
     union {
-        PackKeys<unsigned> narrow;
-        PackKeys<u64> wide;
+        GroupKeys<unsigned> narrow[kPlanThreads / 64];  // one set per wave
+        GroupKeys<u64> wide[kPlanThreads / 64];
     } keys;
-    alignas(16) int wave_min[kPlanThreads / 64];   // per wave: where its bins would end the batch
-    alignas(16) int wave_room[kPlanThreads / 64];  // per wave: bins that can still take a row
     alignas(16) int wave_free[2][kPlanThreads / 64];
-    template <typename Word> __device__ __forceinline__ PackKeys<Word>& of();
+    template <typename Word> __device__ __forceinline__ GroupKeys<Word>& of(int wave);
 };
-template <> __device__ __forceinline__ PackKeys<unsigned>& PackShared::of<unsigned>() { return keys.narrow; }
-template <> __device__ __forceinline__ PackKeys<u64>& PackShared::of<u64>() { return keys.wide; }
+template <> __device__ __forceinline__ GroupKeys<unsigned>& PackShared::of<unsigned>(int wave) { return keys.narrow[wave]; }
+template <> __device__ __forceinline__ GroupKeys<u64>& PackShared::of<u64>(int wave) { return keys.wide[wave]; }
 
-// sum over the four lanes of a quad, in every lane of it
-__device__ __forceinline__ int quad_sum(int x)
-{
-    x += __builtin_amdgcn_update_dpp(0, x, kDppQuadSwap1, 0xF, 0xF, true);
-    x += __builtin_amdgcn_update_dpp(0, x, kDppQuadSwap2, 0xF, 0xF, true);
-    return x;
-}
 // minimum over the wave, in every lane (all lanes active)
 __device__ __forceinline__ int wave_min(int x)
 {
@@ -284,104 +289,104 @@ __device__ __forceinline__ int wave_min(int x)
     return min((int)b[0], (int)b[1]);
 }
 
-// How many keys of the ascending array `sorted` (kPlanMaxBins keys, then kSortedPad times all ones) lie below x: a
-// search by the four lanes of a quad in two steps of sixteen. First the last key of each sixteenth of the array, four per
-// lane: as many of them as lie below x, so many whole sixteenths do; then the sixteen keys that follow, four per lane.
-template <typename Word> __device__ __forceinline__ int count_below_sorted(const Word* sorted, int q, Word x)
+// How many of the kGroupBins keys of the ascending array `sorted` lie below x (all ones never do): two steps of eight.
+// First the last key of each eighth: as many of them as lie below x, so many whole eighths do; then the eight keys
+// that follow (they exist: padding). Two round trips to LDS, where a binary search makes seven.
+template <typename Word> __device__ __forceinline__ int count_below_sorted(const Word* sorted, Word x)
 {
-    static_assert(kPlanMaxBins == 256 && kSortedPad >= 16, "two steps of sixteen");
+    static_assert(kGroupBins == 64 && kSortedPad >= 8, "two steps of eight");
     int n = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) n += sorted[16 * (4 * q + i) + 15] < x ? 1 : 0;
-    const int lo = 16 * quad_sum(n);  // <= 256: the sixteen keys from there on exist (padding)
+    for (int i = 0; i < 8; ++i) n += sorted[8 * i + 7] < x ? 1 : 0;
+    const int lo = 8 * n;  // <= 64
     n = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) n += sorted[lo + 4 * q + i] < x ? 1 : 0;
-    return lo + quad_sum(n);
+    for (int i = 0; i < 8; ++i) n += sorted[lo + i] < x ? 1 : 0;
+    return lo + n;
 }
 
-// How many of fresh[0 .. n) lie below x (n a multiple of the keys in 64 bytes), summed over the four lanes of a quad:
-// lane q looks at the 16-byte chunks q, q + 4, ... (neighbouring lanes read neighbouring chunks: no bank conflicts).
-__device__ __forceinline__ int count_below_fresh(const unsigned* fresh, int n, int q, unsigned x)
+// How many of the kGroupBins keys of fresh[] lie below x (entries that hold no key of the batch are all ones). Every
+// lane reads every key -- the addresses are the same for the whole wave -- and all the reads are issued before the first
+// comparison: one round trip to LDS, not sixteen.
+__device__ __forceinline__ int count_below_fresh(const unsigned* fresh, unsigned x)
 {
     const uint4* chunk = reinterpret_cast<const uint4*>(fresh);
+    uint4 k[kGroupBins / 4];
+#pragma unroll
+    for (int j = 0; j < kGroupBins / 4; ++j) k[j] = chunk[j];
     int below = 0;
-    for (int j = 0; 16 * j < n; ++j) {
-        const uint4 k = chunk[4 * j + q];
-        below += (k.x < x ? 1 : 0) + (k.y < x ? 1 : 0) + (k.z < x ? 1 : 0) + (k.w < x ? 1 : 0);
-    }
-    return quad_sum(below);
+#pragma unroll
+    for (int j = 0; j < kGroupBins / 4; ++j) below += (k[j].x < x ? 1 : 0) + (k[j].y < x ? 1 : 0) + (k[j].z < x ? 1 : 0) + (k[j].w < x ? 1 : 0);
+    return below;
 }
-__device__ __forceinline__ int count_below_fresh(const u64* fresh, int n, int q, u64 x)
+__device__ __forceinline__ int count_below_fresh(const u64* fresh, u64 x)
 {
     const ulonglong2* chunk = reinterpret_cast<const ulonglong2*>(fresh);
     int below = 0;
-    for (int j = 0; 8 * j < n; ++j) {
-        const ulonglong2 k = chunk[4 * j + q];
-        below += (k.x < x ? 1 : 0) + (k.y < x ? 1 : 0);
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {  // 32 keys in registers at a time
+        ulonglong2 k[kGroupBins / 4];
+#pragma unroll
+        for (int j = 0; j < kGroupBins / 4; ++j) k[j] = chunk[half * (kGroupBins / 4) + j];
+#pragma unroll
+        for (int j = 0; j < kGroupBins / 4; ++j) below += (k[j].x < x ? 1 : 0) + (k[j].y < x ? 1 : 0);
     }
-    return quad_sum(below);
+    return below;
 }
 
-// The packing proper: rows 0 .. nz-1 of the sorted head (those with nonzeros), longest first, each into the least loaded
-// bin that has room (ties: the lower bin). In batches: with the bins ranked by (load, bin), the next rows go to the bins
-// in rank order for as long as no bin that already received a row of this batch would have been the least loaded one
-// again, i.e. up to the smallest number of keys below any participating bin's key AFTER its new row (a search in the
-// sorted keys). The four lanes of a quad keep the books of one bin (identically) and share its searches and counts.
-// The order is carried from batch to batch: a bin that took no row moves down by the batch and up by the number of new
-// keys below its own; a bin that took one lands behind the untouched keys that its search found below its new key, plus
-// the new keys below it. Only the new keys of a batch are counted one by one. Three workgroup barriers per batch.
+// The packing of one group by one wave: the group's rows (sorted rows g, g + groups, ... with nonzeros), longest first,
+// each into the least loaded bin of the group that has room (ties: the lower bin). In batches: with the bins ranked by
+// (load, bin), the next rows go to the bins in rank order for as long as no bin that already received a row of this
+// batch would have been the least loaded one again, i.e. up to the smallest number of keys below any participating
+// bin's key AFTER its new row (a search in the sorted keys). The order is carried from batch to batch: a bin that took
+// no row moves down by the batch and up by the number of new keys below its own; a bin that took one lands behind the
+// untouched keys that its search found below its new key, plus the new keys below it. Lane l keeps the books of the
+// group's bin l; LDS accesses of one wave execute in order, so wave barriers (for the compiler) are all it takes.
 template <typename Word>
-__device__ __forceinline__ void pack_batches(const int* s_len, int head, int nz, int bins, int* s_order, PackShared& sh)
+__device__ __forceinline__ void pack_group(const int* s_len, int head, int nz, int bins, int groups, int g, int* s_order,
+                                           GroupKeys<Word>& keys)
 {
     using Key = BinKey<Word>;
-    constexpr int kFreshPad = 64 / (int)sizeof(Word);  // one 16-byte chunk per lane of a quad
-    PackKeys<Word>& keys = sh.of<Word>();
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int bin = tid >> 2, q = tid & 3;  // kPlanThreads = 4 x kPlanMaxBins
-    const int open = min(bins, head);       // bins that exist and have a first workgroup
+    const int lane = threadIdx.x & 63;
+    const int bin = lane * groups + g;                           // this lane's bin, if it exists
+    const bool exists = lane < bins / groups && bin < head;      // ... and has a first workgroup
+    const int rows = nz > g ? (nz - g + groups - 1) / groups : 0;  // rows of this group
     int load = 0, cnt = 0;
-    Word mine = bin < open ? Key::make(0, bin) : Key::none;  // all ones: cannot take a row (any more)
-    int rank = bin;                                          // empty bins rank by number
-    for (int i = tid; i < kPlanMaxBins + kSortedPad; i += kPlanThreads) keys.sorted[0][i] = i < open ? Key::make(0, i) : Key::none;
-    __syncthreads();
-    int with_room = open;  // bins that can still take a row
-    int cur = 0;
-    int t = 0;  // rows placed so far; the same in every thread
-    while (t < nz) {
-        const int most = min(with_room, nz - t);  // >= 1: t < nz <= head rows are unplaced, so some bin has room
-        const bool takes = mine != Key::none && rank < most;  // row t + rank would go to this bin
-        const int len = takes ? s_len[t + rank] : 0;
-        const Word after = takes ? Key::make(load + len, bin) : Key::none;
+    Word mine = exists ? Key::make(0, lane) : Key::none;  // all ones: cannot take a row (any more)
+    int rank = lane;                                      // empty bins rank by number
+    keys.sorted[lane] = mine;
+    if (lane < kSortedPad) keys.sorted[kGroupBins + lane] = Key::none;
+    __builtin_amdgcn_wave_barrier();
+    int t = 0;  // rows of the group placed so far
+    while (t < rows) {
+        const int with_room = __popcll(__ballot(mine != Key::none));
+        const int most = min(with_room, rows - t);  // >= 1: the rows left have a place, so some bin has room
+        const bool takes = mine != Key::none && rank < most;  // the group's row t + rank would go to this bin
+        const int row = (t + rank) * groups + g;              // ... which is this one of the sorted rows
+        const int len = takes ? s_len[row] : 0;
+        const Word after = takes ? Key::make(load + len, lane) : Key::none;
         // the batch ends before the first rank whose bin is no longer below an earlier bin of the batch with its new row
-        const int found = count_below_sorted(keys.sorted[cur], q, after);
-        const int wave_ends = wave_min(takes ? found : 0x7fffffff);
-        if (lane == 0) sh.wave_min[wave] = wave_ends;
-        for (int i = tid; i < kPlanMaxBins + kSortedPad; i += kPlanThreads) keys.sorted[cur ^ 1][i] = Key::none;
-        __syncthreads();
-        const int batch = min(most, min_of_waves(sh.wave_min));  // 1 <= batch <= most
+        const int found = count_below_sorted(keys.sorted, after);
+        const int batch = min(most, wave_min(takes ? found : 0x7fffffff));  // 1 <= batch <= most
         const bool took = takes && rank < batch;
         if (took) {
-            if (q == 0) s_order[cnt * bins + bin] = t + rank;
+            s_order[cnt * bins + bin] = row;
             load += len;
             cnt += 1;
         }
         const bool room = mine != Key::none && cnt * bins + bin < head;  // the bin's next workgroup exists
-        const Word next = room ? Key::make(load, bin) : Key::none;
-        // the bins that took a row are the ranks 0 .. batch-1
-        if (took && q == 0) keys.fresh[rank] = next;
-        const int padded = (batch + kFreshPad - 1) / kFreshPad * kFreshPad;
-        if (tid >= batch && tid < padded) keys.fresh[tid] = Key::none;
-        const unsigned long long rooms = __ballot(q == 0 && room);
-        if (lane == 0) sh.wave_room[wave] = __popcll(rooms);
-        __syncthreads();
-        with_room = sum_of_waves(sh.wave_room);
-        const int place = (took ? found : rank) - batch + count_below_fresh(keys.fresh, padded, q, next);
-        if (room && q == 0) keys.sorted[cur ^ 1][place] = next;
-        __syncthreads();
+        const Word next = room ? Key::make(load, lane) : Key::none;
+        // the bins that took a row are the ranks 0 .. batch-1; the rest of fresh[] holds no key
+        if (took) keys.fresh[rank] = next;
+        if (lane >= batch) keys.fresh[lane] = Key::none;
+        __builtin_amdgcn_wave_barrier();
+        const int place = (took ? found : rank) - batch + count_below_fresh(keys.fresh, next);
+        keys.sorted[lane] = Key::none;
+        __builtin_amdgcn_wave_barrier();
+        if (room) keys.sorted[place] = next;
+        __builtin_amdgcn_wave_barrier();
         mine = next;
         rank = place;
-        cur ^= 1;
         t += batch;
     }
 }
@@ -400,10 +405,17 @@ __device__ __forceinline__ void pack_head(const int* s_len, int head, int nz, in
         __syncthreads();
         return;
     }
-    // a bin holds at most kHeadPerBin rows, none longer than the first
-    if (s_len[0] < (1 << kNarrowLenBits)) pack_batches<unsigned>(s_len, head, nz, bins, s_order, sh);
-    else pack_batches<u64>(s_len, head, nz, bins, s_order, sh);
-    if (nz == head) return;  // (the loop above ended with a barrier)
+    // a bin holds at most kHeadPerBin rows, none longer than the first: 32-bit (load, bin) words below 2^21 nonzeros
+    {
+        const int groups = plan_groups(bins), wave = tid >> 6;
+        const bool narrow = s_len[0] < (1 << kNarrowLenBits);
+        for (int g = wave; g < groups; g += kPlanThreads / 64) {  // wave-uniform
+            if (narrow) pack_group<unsigned>(s_len, head, nz, bins, groups, g, s_order, sh.of<unsigned>(wave));
+            else pack_group<u64>(s_len, head, nz, bins, groups, g, s_order, sh.of<u64>(wave));
+        }
+        __syncthreads();
+    }
+    if (nz == head) return;
     // rows without nonzeros: the positions still free, in ascending order, take the sorted rows nz, nz + 1, ...
     static_assert(kPlanTile == 2 * kPlanThreads, "two positions per thread: tid and tid + kPlanThreads");
     const int lane = tid & 63, wave = tid >> 6;
@@ -509,10 +521,10 @@ __global__ __launch_bounds__(kPlanThreads) void plan_emit_kernel(int M, const in
             mine += wide_len(key) > 0 ? 1 : 0;
         }
         for (int m = 32; m >= 1; m >>= 1) mine += __shfl_xor(mine, m);
-        if (lane == 0) hs.pack.wave_room[wave] = mine;
+        if (lane == 0) hs.pack.wave_free[0][wave] = mine;
         __syncthreads();
-        const int nz = sum_of_waves(hs.pack.wave_room);
-        __syncthreads();  // wave_room is written again by the packing
+        const int nz = sum_of_waves(hs.pack.wave_free[0]);
+        __syncthreads();  // wave_free is written again after the packing
         pack_head(hs.len, head, nz, bins, order, hs.order, hs.pack);
         for (int p = threadIdx.x; p < head; p += kPlanThreads) emit(plan, M, p, hs.row[hs.order[p]], row_offsets);
         return;

@@ -352,7 +352,9 @@ int model_fused_flat(int M, int D, const int* ro, const int* ci, const float* Q,
 
 // Host model of the row plan that dlspm_row_plan_build builds on the device: rows sorted longest first (by row number
 // among equals); the first min(M, 8 x bins) of them packed into `bins` bins of equal size, longest row first into the
-// least loaded bin that still has room (ties: the lower bin), bin b becoming the positions b, b + bins, b + 2 bins, ...;
+// least loaded bin OF ITS GROUP that still has room (ties: the lower bin), bin b becoming the positions b, b + bins,
+// b + 2 bins, ...; the groups -- at most 64 bins each, sorted row t and bin b in group t % groups and b % groups --
+// are packed independently of each other (one wave each on the device);
 // rows without nonzeros fill the positions still free, in ascending order; the rest follow in sorted order.
 // order 1: groups of `bins` alternate between descending and ascending length instead; order 2: plainly descending.
 // plan[0 .. M) first nonzero, plan[M .. 2M) end, plan[2M .. 3M) row. This sequential statement is the definition; the
@@ -369,12 +371,15 @@ void model_row_plan(int M, const int* ro, int bins, int order, int* plan)
     if (order == 1) {
         for (int g = bins; g < head; g += 2 * bins) std::reverse(at.begin() + g, at.begin() + (g + bins < head ? g + bins : head));
     } else if (order == 0) {
+        // groups: the smallest number g >= bins / 64 that divides bins; sorted row t and bin b belong to group t % g, b % g
+        int groups = (bins + 63) / 64;
+        while (bins % groups != 0) ++groups;
         std::vector<long long> load((size_t)bins, 0);
         std::vector<int> cnt((size_t)bins, 0), placed((size_t)head, -1);
         int t = 0;
         for (; t < head && len(sorted[t]) > 0; ++t) {
             int best = -1;
-            for (int b = 0; b < bins; ++b)
+            for (int b = t % groups; b < bins; b += groups)
                 if ((long long)cnt[b] * bins + b < head && (best < 0 || load[b] < load[best])) best = b;
             placed[(size_t)cnt[best] * bins + best] = sorted[t];
             load[best] += len(sorted[t]);
