@@ -7,10 +7,11 @@
 A "step" is one launch of the configuration's kernel through the library's named entry point (default:
 BASELINE.json's configs[1], fp32 CSR SpMM 2048x512 * 512x256 at 90 % sparsity with lognormal-skewed rows, through
 spmm_csr_f32) on inputs that already sit in device memory. After W untimed steps, exactly K steps are captured in one
-HIP graph and that graph is replayed R times; every replay is bracketed by a device synchronisation and by two HIP
-events recorded on the launching stream, and the MEDIAN replay gives every figure of the line (one clock: value,
-ms_per_step and roofline all come from the same event interval; the host's wall time around the same replay is
-reported separately). R is 5 for K >= 1000 and grows for small K so that a 20-step run is not at the mercy of one
+HIP graph and that graph is replayed R times back to back; every replay is bracketed by two HIP events recorded on
+the launching stream (the device is synchronised before the first replay and after the last), and the MEDIAN replay
+gives every figure of the line (one clock: value,
+ms_per_step and roofline all come from the same event interval; the host's wall time around all replays, per
+replay, is reported separately). R is 5 for K >= 1000 and grows for small K so that a 20-step run is not at the mercy of one
 replay. --no-graph launches the K steps from the host instead (Python + ctypes per launch enter the figure then).
 For K below 1000 a replay's own cost (its start and its drain, about 15 us) is a visible share of K launches of 6 us:
 `timing.steady_state_launch_us` then gives the time per launch between a graph of 2 K and a graph of K steps, and
@@ -109,21 +110,20 @@ def capture(torch, stream, body):
 
 
 def timed_replays(torch, stream, run, replays):
-    """`replays` executions of run(), each between two device synchronisations and two HIP events on `stream`:
-    ([event seconds], [host wall seconds])."""
-    ev, wall = [], []
-    for _ in range(replays):
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        e0.record(stream)
+    """`replays` executions of run(), enqueued back to back on `stream`, each between its own pair of HIP events; the
+    device is synchronised before the first and after the last, so a replay starts on a device that is at work, as
+    every launch but the first of a long run does: ([event seconds per replay], [host wall seconds / replays] * replays)."""
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(replays)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(replays)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(replays):
+        starts[i].record(stream)
         run()
-        e1.record(stream)
-        torch.cuda.synchronize()
-        wall.append(time.perf_counter() - t0)
-        ev.append(e0.elapsed_time(e1) * 1e-3)
-    return ev, wall
+        ends[i].record(stream)
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / replays
+    return [starts[i].elapsed_time(ends[i]) * 1e-3 for i in range(replays)], [wall] * replays
 
 
 def time_steps(torch, step, steps, warmup, replays, use_graph, split_overhead=False):
