@@ -31,7 +31,6 @@ namespace {
 constexpr int kPlanTile = 2048;     // rows sorted by one workgroup; also the most rows a head can hold
 constexpr int kPlanThreads = 1024;  // two keys per thread
 constexpr int kPlanMaxBins = 256;   // 8 x bins <= kPlanTile
-static_assert(kPlanThreads == 4 * kPlanMaxBins, "the packing counts with four threads per bin");
 static_assert(kPlanTile == 2 * kPlanThreads, "the register sort holds two keys per thread");
 constexpr int kHeadPerBin = 8;      // workgroups of a four-wave kernel that a compute unit holds at once
 // While every row of a tile is shorter than 2^21 its sort keys fit 32 bits (length << 11 | 2047 - row in tile) and are
