@@ -390,20 +390,18 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
     }
     auto s_off = [&](int i) { return blk.off(i); };
     const int T0 = blk.T0, T = blk.T, per = blk.per, a = blk.a;
-    // Results of kStreamedOutputFloats and more are stored with the non-temporal hint: they are written once, and
-    // ordinary stores are held in the L2 as dirty lines to be written back later, where hinted ones drain as they are
-    // issued (hits, misses and fetched bytes of the L2 stay the same; the time does not). Measured (SpMM): 2048 x 512, N = 256 (2 MiB) 6.07 -> 5.96 us; 16384 x 4096 at 10 %,
-    // N = 128 (8 MiB) 133 -> 128 us; 65536 x 1024 at 2 %, N = 256 (64 MiB) 52.5 -> 49.7 us; 131072 x 512, N = 128
-    // 41.6 -> 39.1 us. Smaller results lose by it when rows end inside a cache line (512 x 2048, N = 49: 4.72 -> 5.04 us;
-    // 2048 x 1024, N = 33: 4.66 -> 5.03 us). Not for the partial rows of the column-sliced schedule, which are read again.
-    // Rows that are whole cache lines (a multiple of 32 floats) gain from 0.5 MiB on (4096 x 4096 at 2 %, D = 64, 1 MiB:
-    // fused 9.60 -> 9.35 us).
-    constexpr long long kStreamedOutputFloats = 512 * 1024, kStreamedWholeLineFloats = 128 * 1024;
+    // Results of kStreamedOutputFloats (4 MiB, one L2's worth) and more are stored with the non-temporal hint: they are
+    // written once, and ordinary stores are held in the L2 as dirty lines to be written back later, where hinted ones
+    // drain as they are issued (hits, misses and fetched bytes of the L2 stay the same; the time does not). Measured with
+    // both kinds of store in one process (SpMM): 4-8 MiB -0.5 ... -1.3 %; 8192 x 1024 at 5 %, N = 1024 (32 MiB)
+    // 58.3 -> 56.9 us; 65536 x 1024 at 2 %, N = 256 (64 MiB) 52.3 -> 49.2 us; 131072 x 512, N = 128 41.2 -> 38.8 us;
+    // fused 65536 x 2048, D = 64 (16 MiB) 42.3 -> 40.8 us. Below 4 MiB there is nothing to gain (+-0.8 %). Not for the
+    // partial rows of the column-sliced schedule, which are read again.
+    constexpr long long kStreamedOutputFloats = 1024 * 1024;
     const long long out_floats = (long long)blk.rows_total * width;
     // (dlspm_tuning.stream_results switches the rule off or on for sweeps and tests: blk.stream_rule)
     const bool streaming = (!SLICED || PLANNED) && blk.stream_rule != 1 &&
-                           (blk.stream_rule == 2 || out_floats >= kStreamedOutputFloats ||
-                            (width % 32 == 0 && out_floats >= kStreamedWholeLineFloats));
+                           (blk.stream_rule == 2 || out_floats >= kStreamedOutputFloats);
 
     blk.for_each_segment([&](int r, int p, int q, int rs, int re) {
         VecT acc[V];

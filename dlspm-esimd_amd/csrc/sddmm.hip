@@ -18,13 +18,14 @@
 
 namespace dlspm {
 
-// Where the results go. Results of more bytes than one L2 holds are stored with the non-temporal hint: ordinary stores
-// are held in the L2 as dirty lines and written back later, hinted ones drain as they are issued. (The L2's hit rate
-// and the bytes fetched do not change by it; the time does.) Measured: 24576 x 8192 at density 0.3,
-// 60 million results, D = 32 443 -> 309 us, D = 64 715 -> 525 us, D = 128 1289 -> 1090 us; 8192 x 2048 at 0.3, 19 MiB:
-// D = 32 32.9 -> 29.2 us, D = 128 90.1 -> 88.0 us; 5 MiB: equal). Small results keep ordinary stores: a kernel ends when
-// its stores have reached memory, and neighbouring waves share cache lines here (2048 x 2048 at 5 %, D = 128, 0.8 MiB:
-// 5.6 -> 5.9 us with the hint).
+// Where the results go. Results of more than one and a half times what one L2 holds (6 MiB on an MI355X) are stored with
+// the non-temporal hint: ordinary stores are held in the L2 as dirty lines and written back later, hinted ones drain as
+// they are issued. (The L2's hit rate and the bytes fetched do not change by it; the time does.) Measured with both
+// kinds of store in one process, D = 32 / 128: 24576 x 8192 at density 0.3 (230 MiB of results) 443 -> 297 us /
+// 1287 -> 1089 us; 8192 x 2048 at 0.3 (19 MiB) 32.5 -> 28.1 us / 90.6 -> 88.3 us; 6144 x 2048 at 0.2 (9.6 MiB) -3.5 % /
+// -4.4 %; 6.4 MiB -1.2 % / -1.8 %; 4.8 MiB +0.4 ... +2.2 % / equal. Small results lose by the hint -- neighbouring waves
+// share cache lines here, and a kernel ends when its stores have reached memory -- (2048 x 2048 at 5 %, 0.8 MiB: +8 % /
+// +4 %) and keep ordinary stores.
 struct SampledOut {
     float* __restrict__ at;
     int streaming;
@@ -40,7 +41,8 @@ struct SampledOut {
 static inline SampledOut sampled_out(const SddmmArgs& x)
 {
     const int forced = tuning().stream_results;  // -1: the size rule (sweeps and tests switch it off or on)
-    const bool by_rule = (long long)x.nnz * (long long)sizeof(float) > device_info().l2_bytes;
+    const long long l2 = device_info().l2_bytes;
+    const bool by_rule = (long long)x.nnz * (long long)sizeof(float) > l2 + l2 / 2;
     return SampledOut{x.out, (forced < 0 ? by_rule : forced != 0) ? 1 : 0};
 }
 

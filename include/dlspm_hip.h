@@ -301,8 +301,8 @@ typedef struct dlspm_tuning {
                           /* fetched, 6 % faster on a 16384-row band; unsafe as a rule: rows whose length depends on   */
                           /* their position would load the XCDs unevenly). One column tile, no row plan, no slices.   */
                           /* (DLSPM_HINT_BANDED asks for the same per call.)                                          */
-    int stream_results;   /* results stored with the non-temporal hint: -1 the size rule (SDDMM: more than one L2's    */
-                          /* worth; dense rows: from 2 MiB, whole cache lines from 0.5 MiB), 0 never, 1 always         */
+    int stream_results;   /* results stored with the non-temporal hint: -1 the size rule (dense result rows from one   */
+                          /* L2's worth on, SDDMM results from one and a half), 0 never, 1 always                      */
 } dlspm_tuning;
 void dlspm_tuning_default(dlspm_tuning* t);   /* fills *t with "follow the rules" */
 int dlspm_set_tuning(const dlspm_tuning* t);  /* DLSPM_OK or DLSPM_E_INVALID_ARG (a field out of range) */

@@ -338,7 +338,7 @@ def test_large_shape_against_oracle(torch_cuda, dl, oracle):
 
 
 def test_sddmm_results_beyond_the_l2_are_streamed(torch_cuda, dl, oracle):
-    """More results than one L2 holds (here 9.4 million = 38 MB; an MI355X's L2 is 4 MiB) are stored with the
+    """More results than one and a half L2s hold (here 9.4 million = 38 MB; an MI355X's L2 is 4 MiB) are stored with the
     non-temporal hint; the bits must be those of ordinary stores under every schedule: row blocks, the
     even-rows hint, a row plan, and the flat schedule forced by tuning, all against the multi-threaded oracle and equal
     to each other."""
@@ -346,7 +346,7 @@ def test_sddmm_results_beyond_the_l2_are_streamed(torch_cuda, dl, oracle):
     M, K, D = 8192, 8192, 32
     ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 71, M, K, 0.14)
     info = dl.device_info()
-    assert ci.size * 4 > info["l2_bytes"]
+    assert ci.size * 4 > 1.5 * info["l2_bytes"]
     lhs = dl.fill("normal", 72, (M, D), 0.0, 1.0)
     rhs = dl.fill("normal", 73, (K, D), 0.0, 1.0)
     want = oracle.sddmm(ro, ci, lhs, rhs, omp=True)
