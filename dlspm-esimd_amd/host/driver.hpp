@@ -200,11 +200,13 @@ inline Diff compare(const std::vector<float>& ref, const std::vector<float>& gpu
 struct Timing {
     double min_ms = 0, median_ms = 0;
     double cold_min_ms = -1;  // with the caches flushed before every launch; -1 when not measured
+    double graph_ms = -1;     // per launch inside a HIP graph of Options::graph launches (median replay); -1 when not measured
 };
 struct Options {
     int warmup = 5;
     int iters = 20;  // the reference keeps the minimum of 20 launches (SPMM/spmm-esimd-fromfile2.cpp:194-243)
     bool cold = false;
+    int graph = 0;  // --graph n: also time a HIP graph of n launches, replayed five times (no event between the launches)
     // what to pass as `workspace`: by default the memory dlspm_workspace_bytes asks for when the column-sliced schedule
     // applies or the longest row is at least four times the mean row (dlspm_csr_row_stats), DLSPM_HINT_ROWS_EVEN when it is
     // at most one and a half times the mean;
@@ -286,17 +288,23 @@ inline DevBuf<char> build_row_plan(int M, const int* row_offsets_dev)
     return plan;
 }
 
+// `launch(stream)` enqueues one call of the op. Every launch is timed between its own pair of HIP events (the minimum is
+// the reference's figure; the pair itself costs about 3 us that a sequence of launches does not pay); with --graph n the
+// same launch is also captured n times into a HIP graph, whose replay is timed as a whole.
 template <typename Launch> Timing time_launches(const Options& opt, Launch&& launch)
 {
     hipEvent_t e0, e1;
     DLSPM_HIP_CHECK(hipEventCreate(&e0));
     DLSPM_HIP_CHECK(hipEventCreate(&e1));
+    auto check = [](int st) {
+        if (st != DLSPM_OK) throw std::runtime_error(std::string("libdlspm_hip: ") + dlspm_status_string(st));
+    };
     auto one = [&]() {
         DLSPM_HIP_CHECK(hipEventRecord(e0, nullptr));
-        const int st = launch();
+        const int st = launch(static_cast<hipStream_t>(nullptr));
         DLSPM_HIP_CHECK(hipEventRecord(e1, nullptr));
         DLSPM_HIP_CHECK(hipEventSynchronize(e1));
-        if (st != DLSPM_OK) throw std::runtime_error(std::string("libdlspm_hip: ") + dlspm_status_string(st));
+        check(st);
         float ms = 0;
         DLSPM_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
         return (double)ms;
@@ -317,6 +325,46 @@ template <typename Launch> Timing time_launches(const Options& opt, Launch&& lau
             best = std::min(best, one());
         }
         r.cold_min_ms = best;
+    }
+    if (opt.graph > 0) {
+        constexpr int kReplays = 5;
+        hipStream_t stream;
+        hipGraph_t graph;
+        hipGraphExec_t exec;
+        DLSPM_HIP_CHECK(hipDeviceSynchronize());
+        DLSPM_HIP_CHECK(hipStreamCreate(&stream));
+        DLSPM_HIP_CHECK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+        int st = DLSPM_OK;
+        for (int i = 0; i < opt.graph && st == DLSPM_OK; ++i) st = launch(stream);
+        DLSPM_HIP_CHECK(hipStreamEndCapture(stream, &graph));
+        check(st);
+        DLSPM_HIP_CHECK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+        DLSPM_HIP_CHECK(hipGraphLaunch(exec, stream));  // untimed: first-use set-up of the graph
+        DLSPM_HIP_CHECK(hipStreamSynchronize(stream));
+        hipEvent_t begin[kReplays], end[kReplays];
+        for (int i = 0; i < kReplays; ++i) {
+            DLSPM_HIP_CHECK(hipEventCreate(&begin[i]));
+            DLSPM_HIP_CHECK(hipEventCreate(&end[i]));
+        }
+        for (int i = 0; i < kReplays; ++i) {  // enqueued back to back: a replay starts on a device that is at work
+            DLSPM_HIP_CHECK(hipEventRecord(begin[i], stream));
+            DLSPM_HIP_CHECK(hipGraphLaunch(exec, stream));
+            DLSPM_HIP_CHECK(hipEventRecord(end[i], stream));
+        }
+        DLSPM_HIP_CHECK(hipStreamSynchronize(stream));
+        std::vector<double> replay;
+        for (int i = 0; i < kReplays; ++i) {
+            float ms = 0;
+            DLSPM_HIP_CHECK(hipEventElapsedTime(&ms, begin[i], end[i]));
+            replay.push_back((double)ms / opt.graph);
+            (void)hipEventDestroy(begin[i]);
+            (void)hipEventDestroy(end[i]);
+        }
+        std::sort(replay.begin(), replay.end());
+        r.graph_ms = replay[kReplays / 2];
+        (void)hipGraphExecDestroy(exec);
+        (void)hipGraphDestroy(graph);
+        (void)hipStreamDestroy(stream);
     }
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
@@ -342,6 +390,9 @@ inline void report(const char* opname, Op op, int M, int K, int N, int nnz, cons
     std::printf("GFLOPS:  %8.2f\n", a.flops / s * 1e-9);
     std::printf("median kernel time %f ms over %d launches (%d warm-up)\n", t.median_ms, opt.iters, opt.warmup);
     if (t.cold_min_ms >= 0) std::printf("cold-cache kernel time %f ms (1 GiB streamed through the caches before each launch)\n", t.cold_min_ms);
+    if (t.graph_ms >= 0)
+        std::printf("in a HIP graph of %d launches: %f ms per launch, GFLOPS: %8.2f (median of 5 replays)\n", opt.graph, t.graph_ms,
+                    a.flops / (t.graph_ms * 1e-3) * 1e-9);
     std::printf("effective (application) bandwidth: %9.1f GB/s = %5.1f %% of 8000 GB/s HBM peak  [%.0f bytes]\n",
                 a.effective_B / s * 1e-9, a.effective_B / s * 1e-9 / 80.0, a.effective_B);
     std::printf("algorithmic bandwidth:             %9.1f GB/s = %5.2f %% of 8000 GB/s HBM peak  [%.0f bytes]\n",
@@ -415,7 +466,7 @@ inline std::string usage(const char* app, const char* width)
       << "                                                     --band w [--band-random r]: a band of w columns per row plus r anywhere)\n"
       << "       " << app << " --sweep [--max-m M]                  the 12 x {32,128} x {0.3,0.2,0.1} benchmark grid\n"
       << "       " << app << " --cfg <id>                           a seeded benchmark configuration (1..5)\n"
-      << "options: --iters n (20)  --warmup n (5)  --cold  --csv <file>  --dump <dir> | --dump-each <dir>  --tol x (1e-4)  --workspace | --no-workspace  --no-plan";
+      << "options: --iters n (20)  --warmup n (5)  --cold  --graph n  --csv <file>  --dump <dir> | --dump-each <dir>  --tol x (1e-4)  --workspace | --no-workspace  --no-plan";
     return u.str();
 }
 
@@ -462,6 +513,7 @@ inline Cli parse_cli(int argc, char** argv, const char* app, const char* width)
         }
         else if (a == "--iters") { need(i, 1); cli.opt.iters = std::max(1, std::stoi(argv[++i])); }
         else if (a == "--warmup") { need(i, 1); cli.opt.warmup = std::max(0, std::stoi(argv[++i])); }
+        else if (a == "--graph") { need(i, 1); cli.opt.graph = std::max(0, std::stoi(argv[++i])); }
         else if (a == "--cold") cli.opt.cold = true;
         else if (a == "--csv") { need(i, 1); cli.opt.csv = argv[++i]; }
         else if (a == "--dump") { need(i, 1); cli.opt.dump = argv[++i]; }

@@ -49,10 +49,10 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     DevBuf<char> ws(wc.bytes);
     if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
     DevBuf<char> plan = wc.plan ? build_row_plan(M, ro_d.p) : DevBuf<char>(0);
-    const Timing t = time_launches(opt, [&]() {
-        if (wc.plan) return fused_sddmm_spmm_f32(M, K, D, nnz, ro_d.p, ci_d.p, Q_d.p, K_d.p, V_d.p, scale, O_d.p, plan.p, plan.n | DLSPM_HINT_ROW_PLAN, nullptr);
+    const Timing t = time_launches(opt, [&](hipStream_t stream) {
+        if (wc.plan) return fused_sddmm_spmm_f32(M, K, D, nnz, ro_d.p, ci_d.p, Q_d.p, K_d.p, V_d.p, scale, O_d.p, plan.p, plan.n | DLSPM_HINT_ROW_PLAN, stream);
         return fused_sddmm_spmm_f32(M, K, D, nnz, ro_d.p, ci_d.p, Q_d.p, K_d.p, V_d.p, scale, O_d.p, wc.arg(ws.p),
-                                    wc.size(), nullptr);
+                                    wc.size(), stream);
     });
     hipLaunchKernelGGL(check_row_of_slot_kernel, dim3(blocks_for(M)), dim3(256), 0, nullptr, M, ro_d.p, rowof_d.p);
     hipLaunchKernelGGL(check_sddmm_kernel, dim3(blocks_for(nnz)), dim3(256), 0, nullptr, nnz, D, rowof_d.p, ci_d.p, Q_d.p, K_d.p,

@@ -51,9 +51,9 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
     const bool planned = wc.plan;
     DevBuf<char> plan = planned ? build_row_plan(M, ro_d.p) : DevBuf<char>(0);
-    const Timing t = time_launches(opt, [&]() {
-        if (planned) return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, plan.p, plan.n | DLSPM_HINT_ROW_PLAN, nullptr);
-        return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, wc.arg(ws.p), wc.size(), nullptr);
+    const Timing t = time_launches(opt, [&](hipStream_t stream) {
+        if (planned) return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, plan.p, plan.n | DLSPM_HINT_ROW_PLAN, stream);
+        return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, wc.arg(ws.p), wc.size(), stream);
     });
     hipLaunchKernelGGL(check_spmm_kernel, dim3(blocks_for((long long)M * N)), dim3(256), 0, nullptr, M, N, ro_d.p, ci_d.p,
                        va_d.p, B_d.p, Cref_d.p);

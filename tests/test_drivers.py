@@ -140,6 +140,26 @@ def test_driver_shape_and_small_sweep():
     assert rc == 0 and out.count("PASS") == 6  # (1024,1024) x N in {32,128} x density in {0.3,0.2,0.1}
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("app,cfg", [("spmm_run", 2), ("sddmm_run", 3), ("fused_run", 5)])
+def test_driver_graph_timing(oracle, app, cfg, tmp_path):
+    """--graph n: the launch is also captured n times into a HIP graph (row plan or workspace included) and the replay
+    timed as a whole; the result is checked and dumped after those replays, and a launch inside the graph does not take
+    longer than a launch between its own pair of events."""
+    import re
+
+    d = tmp_path / "dump"
+    d.mkdir()
+    rc, out = run(app, "--cfg", cfg, "--graph", 40, "--dump", d)
+    assert rc == 0 and "PASS" in out, out[-800:]
+    m = re.search(r"in a HIP graph of 40 launches: ([0-9.]+) ms per launch, GFLOPS: +([0-9.]+)", out)
+    assert m, out[-800:]
+    single = float(re.search(r"Total kernel time was ([0-9.]+) ms", out).group(1))
+    assert 0 < float(m.group(1)) <= single * 1.05
+    meta, err = verify_dump(oracle, str(d))
+    assert err <= 1e-4
+
+
 def verify_dump(oracle, d):
     """Relative Frobenius error of one driver dump (inputs and the kernel's output) against the CPU oracle."""
     meta, arr = load_dump(d)
