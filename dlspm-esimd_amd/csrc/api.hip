@@ -234,9 +234,14 @@ void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bo
     // four-wave workgroups win whenever the matrix has enough rows to fill the device (16-wave workgroups were up
     // to 2x slower on long rows: their barrier makes every wave wait for the slowest of sixteen), and rows are
     // grouped only as far as the grid keeps `blocks_per_cu` workgroups per compute unit and a workgroup stays below ~512 nonzeros.
+    // Fewer rows than two per compute unit: eight waves per row from about a hundred nonzeros per row on, four below
+    // (the reference's ResNet-50 and transformer layers of 64 ... 256 rows, 200 launches in a graph, four / eight /
+    // sixteen waves: 128 x 512 with 26 per row, SpMM at N = 256 2.6 / 2.7 / 3.2 us, SDDMM 2.1 / 2.1 / 2.6 us;
+    // 256 x 2304 with 208 per row: 5.4 / 5.2 / 5.5 us, 3.8 / 3.4 / 3.9 us): more waves than a row has passes for only add
+    // to the partial sums behind the barrier.
     const double avg = M > 0 ? (double)nnz / M : 0.0;
     const long long work_rows = (long long)M * col_tiles;
-    W = work_rows >= 2 * cus ? 4 : work_rows >= cus ? 8 : 16;
+    W = work_rows < 2 * cus && avg >= 96.0 ? 8 : 4;
     // very long rows in a tall matrix: sixteen waves per row gain 5-8 % in SpMM (24576 and 32768 rows of ~2000
     // nonzeros); with 8192 rows they lose as much, and the fused kernel loses 25-50 % with them at any height
     if (rule.w16_long_rows && avg >= 1536.0 && work_rows >= 64 * cus) W = 16;
@@ -518,6 +523,11 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
     }
     // rows known to be even gain nothing from another order (and the even-rows hint may serve them better)
     if (max_row_len >= 0 && max_row_len <= 1.5 * ((double)nnz / M)) return 0;
+    // SDDMM on short rows groups them by the size rule, and gives that up for the plan's order only where they are far
+    // from even (2048 x 512 of the reference's data set, 10 per row, D = 128: longest 158, 3.56 -> 2.65 us; longest 23,
+    // 3.34 -> 3.66 us; over the files of that shape: a longest row of 4 ... 8 times the mean +4 ... 6 %, of 8 ... 12 times
+    // -4 %, beyond that -8 ... 14 %)
+    if (op == DLSPM_OP_SDDMM && (long long)nnz < 32ll * M && max_row_len >= 0 && max_row_len < 8.0 * ((double)nnz / M)) return 0;
     // dense operands well beyond one L2 need the column-sliced schedule's workspace more than they need balance; the
     // flat schedule, though, is behind the plan wherever both apply (SpMM, lognormal rows, sigma 1 ... 2, row-block /
     // flat / plan: 8192 x 2048, N = 128: 45.4 / 41.2 / 30.8 us; 16384 x 4096: 121 / 105 / 86.6 us; 32768 x 8192: 525 / 466

@@ -181,7 +181,11 @@ FusedShape fused_choose(int M, int D, int nnz, bool vec4, bool rows_even)
         s.G1 = 4; s.DS = 1; s.G = 8; s.V = 1;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(M, (D + tw - 1) / tw, nnz, SplitRule{2, tw >= 1024 ? 4 : 16, kWave / s.G, false}, rows_even, s.W, s.R);
+    // rows are grouped while the grid keeps three workgroups per compute unit (lognormal rows of 8 ... 40 nonzeros, D = 64,
+    // rows per workgroup 1 / 2 / 4 / 8 / 16: 1024 rows 3.3 / 4.4 / 5.5 / 6.9 / 10.9 us; 2048 rows 4.8 / 4.9 / 6.1 / 7.8 /
+    // 11.7 us; 4096 rows 7.3 / 7.2 / 6.5 / 8.0 / 11.6 us; 8192 rows 12.1 / 10.4 / 8.3 / 7.2 / 9.2 us; 16384 rows: sixteen;
+    // 3072 rows of 102, even: two per workgroup 8.5 us, four 7.2 us)
+    choose_split(M, (D + tw - 1) / tw, nnz, SplitRule{3, tw >= 1024 ? 4 : 16, kWave / s.G, false}, rows_even, s.W, s.R);
     return s;
 }
 

@@ -70,6 +70,33 @@ def test_split_rule_and_the_even_rows_hint(dl):
     assert dl.describe_launch(dl.OP_FUSED, 300, 8192, 32, 300 * 7000)["W"] == 16  # few rows, very long: still sixteen
 
 
+def test_split_rule_for_small_matrices(dl):
+    """The reference's layer shapes of 64 ... 2048 rows. Fewer rows than two per compute unit: four waves per row,
+    eight from about a hundred nonzeros per row on, sixteen only for very long rows. The fused op keeps three
+    workgroups per compute unit when it groups rows (SDDMM two, SpMM eight). SDDMM and the fused op take a row plan for
+    short rows up to eight rows per compute unit; the advice gives SDDMM's grouping up only for a longest row of eight
+    times the mean."""
+    for op in (dl.OP_SPMM, dl.OP_SDDMM, dl.OP_FUSED):
+        width = 256 if op == dl.OP_SPMM else 64
+        assert dl.describe_launch(op, 128, 512, width, 128 * 26)["W"] == 4
+        assert dl.describe_launch(op, 64, 576, width, 64 * 58)["W"] == 4
+        assert dl.describe_launch(op, 256, 2304, width, 256 * 208)["W"] == 8
+        assert dl.describe_launch(op, 511, 2304, width, 511 * 96)["W"] == 8
+        assert dl.describe_launch(op, 512, 2304, width, 512 * 208)["W"] == 4
+    assert dl.describe_launch(dl.OP_SPMM, 64, 4608, 256, 64 * 800)["W"] == 16
+    rows_per_workgroup = lambda op, M, avg: dl.describe_launch(op, M, 1024, 64, M * avg)["R"]
+    assert [rows_per_workgroup(dl.OP_FUSED, M, 20) for M in (1024, 2048, 3072, 4096, 8192, 16384)] == [1, 2, 4, 4, 8, 16]
+    assert [rows_per_workgroup(dl.OP_SDDMM, M, 20) for M in (1024, 2048, 4096, 8192)] == [2, 4, 8, 16]
+    assert [rows_per_workgroup(dl.OP_SPMM, M, 20) for M in (1024, 2048, 4096, 8192)] == [1, 1, 2, 4]
+    M, K, nnz = 2048, 512, 2048 * 10
+    assert dl.row_plan_advice(dl.OP_FUSED, M, K, 64, nnz, 23) == 1  # short rows: any unevenness
+    assert dl.row_plan_advice(dl.OP_FUSED, M, K, 64, nnz, 14) == 0  # even
+    assert dl.row_plan_advice(dl.OP_SDDMM, M, K, 128, nnz, 52) == 0
+    assert dl.row_plan_advice(dl.OP_SDDMM, M, K, 128, nnz, 158) == 1
+    assert dl.row_plan_advice(dl.OP_SDDMM, M, K, 128, 2048 * 64, 209) == 1  # rows of 32 and more: as before
+    assert dl.row_plan_advice(dl.OP_FUSED, 4096, K, 64, 4096 * 10, 158) == 0  # more rows: short rows stay grouped
+
+
 def test_column_tiles_narrow_with_the_height_of_the_dense_operand(dl):
     """Dense rows wider than 512 floats are covered by several column tiles, worked through one after the other: the
     widest tile whose K x tile slab of B fits 4 MiB."""
