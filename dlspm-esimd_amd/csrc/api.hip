@@ -234,14 +234,15 @@ void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bo
     // four-wave workgroups win whenever the matrix has enough rows to fill the device (16-wave workgroups were up
     // to 2x slower on long rows: their barrier makes every wave wait for the slowest of sixteen), and rows are
     // grouped only as far as the grid keeps `blocks_per_cu` workgroups per compute unit and a workgroup stays below ~512 nonzeros.
-    // Fewer rows than two per compute unit: eight waves per row from about a hundred nonzeros per row on, four below
-    // (the reference's ResNet-50 and transformer layers of 64 ... 256 rows, 200 launches in a graph, four / eight /
-    // sixteen waves: 128 x 512 with 26 per row, SpMM at N = 256 2.6 / 2.7 / 3.2 us, SDDMM 2.1 / 2.1 / 2.6 us;
-    // 256 x 2304 with 208 per row: 5.4 / 5.2 / 5.5 us, 3.8 / 3.4 / 3.9 us): more waves than a row has passes for only add
-    // to the partial sums behind the barrier.
+    // Fewer rows than two per compute unit: four waves per row; SDDMM and the fused op take eight from about a hundred
+    // nonzeros per row on (the reference's ResNet-50 and transformer layers of 64 ... 256 rows, 200 launches in a graph,
+    // four / eight / sixteen waves: 128 x 512 with 26 per row, SpMM at N = 256 2.6 / 2.7 / 3.2 us, SDDMM 2.1 / 2.1 / 2.6 us;
+    // 256 x 2304 with 208 per row: SpMM 5.4 / 5.2 / 5.5 us, SDDMM 3.8 / 3.4 / 3.9 us, fused 4.7 / 4.3 / 4.7 us; SpMM in
+    // column tiles, 64 x 576 with 414 per row at N = 3136: 18.7 / 22.2 / 24.5 us): more waves than a row has passes for
+    // only add to the partial sums behind the barrier.
     const double avg = M > 0 ? (double)nnz / M : 0.0;
     const long long work_rows = (long long)M * col_tiles;
-    W = work_rows < 2 * cus && avg >= 96.0 ? 8 : 4;
+    W = rule.w8_few_rows_avg > 0 && work_rows < 2 * cus && avg >= rule.w8_few_rows_avg ? 8 : 4;
     // very long rows in a tall matrix: sixteen waves per row gain 5-8 % in SpMM (24576 and 32768 rows of ~2000
     // nonzeros); with 8192 rows they lose as much, and the fused kernel loses 25-50 % with them at any height
     if (rule.w16_long_rows && avg >= 1536.0 && work_rows >= 64 * cus) W = 16;

@@ -185,7 +185,7 @@ FusedShape fused_choose(int M, int D, int nnz, bool vec4, bool rows_even)
     // rows per workgroup 1 / 2 / 4 / 8 / 16: 1024 rows 3.3 / 4.4 / 5.5 / 6.9 / 10.9 us; 2048 rows 4.8 / 4.9 / 6.1 / 7.8 /
     // 11.7 us; 4096 rows 7.3 / 7.2 / 6.5 / 8.0 / 11.6 us; 8192 rows 12.1 / 10.4 / 8.3 / 7.2 / 9.2 us; 16384 rows: sixteen;
     // 3072 rows of 102, even: two per workgroup 8.5 us, four 7.2 us)
-    choose_split(M, (D + tw - 1) / tw, nnz, SplitRule{3, tw >= 1024 ? 4 : 16, kWave / s.G, false}, rows_even, s.W, s.R);
+    choose_split(M, (D + tw - 1) / tw, nnz, SplitRule{3, tw >= 1024 ? 4 : 16, kWave / s.G, false, 96}, rows_even, s.W, s.R);
     return s;
 }
 

@@ -183,7 +183,7 @@ SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4, bool rows_even)
         s.G1 = 4;
         s.DS = 1;
     }
-    choose_split(M, 1, nnz, SplitRule{2, 16, kWave / s.G1, true}, rows_even, s.W, s.R);
+    choose_split(M, 1, nnz, SplitRule{2, 16, kWave / s.G1, true, 96}, rows_even, s.W, s.R);
     return s;
 }
 

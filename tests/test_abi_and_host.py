@@ -71,8 +71,8 @@ def test_split_rule_and_the_even_rows_hint(dl):
 
 
 def test_split_rule_for_small_matrices(dl):
-    """The reference's layer shapes of 64 ... 2048 rows. Fewer rows than two per compute unit: four waves per row,
-    eight from about a hundred nonzeros per row on, sixteen only for very long rows. The fused op keeps three
+    """The reference's layer shapes of 64 ... 2048 rows. Fewer rows than two per compute unit: four waves per row, in
+    SDDMM and the fused op eight from about a hundred nonzeros per row on, sixteen only for very long rows. The fused op keeps three
     workgroups per compute unit when it groups rows (SDDMM two, SpMM eight). SDDMM and the fused op take a row plan for
     short rows up to eight rows per compute unit; the advice gives SDDMM's grouping up only for a longest row of eight
     times the mean."""
@@ -80,9 +80,11 @@ def test_split_rule_for_small_matrices(dl):
         width = 256 if op == dl.OP_SPMM else 64
         assert dl.describe_launch(op, 128, 512, width, 128 * 26)["W"] == 4
         assert dl.describe_launch(op, 64, 576, width, 64 * 58)["W"] == 4
-        assert dl.describe_launch(op, 256, 2304, width, 256 * 208)["W"] == 8
-        assert dl.describe_launch(op, 511, 2304, width, 511 * 96)["W"] == 8
+        eight = 4 if op == dl.OP_SPMM else 8  # SpMM: only by the rule for very long rows
+        assert dl.describe_launch(op, 256, 2304, width, 256 * 208)["W"] == eight
+        assert dl.describe_launch(op, 511, 2304, width, 511 * 96)["W"] == eight
         assert dl.describe_launch(op, 512, 2304, width, 512 * 208)["W"] == 4
+    assert dl.describe_launch(dl.OP_SPMM, 256, 2304, 196, 256 * 461)["W"] == 8
     assert dl.describe_launch(dl.OP_SPMM, 64, 4608, 256, 64 * 800)["W"] == 16
     rows_per_workgroup = lambda op, M, avg: dl.describe_launch(op, M, 1024, 64, M * avg)["R"]
     assert [rows_per_workgroup(dl.OP_FUSED, M, 20) for M in (1024, 2048, 3072, 4096, 8192, 16384)] == [1, 2, 4, 4, 8, 16]
