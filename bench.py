@@ -32,6 +32,8 @@ Prints ONE JSON line:
   row_plan          (uneven rows) the steps pass the row plan as their workspace (DLSPM_HINT_ROW_PLAN); the plan is built
                     once per matrix, on the device, before the timed region; this object gives what building it costs
                     and the time of the same launches in matrix order (--no-plan measures those as the headline)
+  rows_even_hint    (per configuration) the steps pass DLSPM_HINT_ROWS_EVEN: dlspm_workspace_advice said so for the
+                    longest row that one look at the row lengths found (dlspm_csr_row_stats), as the C++ drivers do
   all_configs       the same measurement for every benchmark configuration (shorter runs)
 """
 import argparse
@@ -75,6 +77,10 @@ def make_step(dl, torch, c, use_plan=True, info=None):
     need = dl.workspace_bytes(c["op"], c["M"], c["K"], c["N"], c["nnz"])  # 0 at the sizes of the five configurations
     ws = torch.empty(need, dtype=torch.uint8, device="cuda") if need else None
     longest, _ = dl.csr_row_stats(ro)
+    if not need and dl.workspace_advice(c["op"], c["M"], c["K"], c["N"], c["nnz"], longest) == dl.PASS_ROWS_EVEN:
+        ws = dl.ROWS_EVEN  # no memory: the hint that no row is much longer than the mean (cfg1, cfg3, cfg4)
+        if info is not None:
+            info["rows_even"] = True
     plan = None
     if use_plan and dl.row_plan_advice(c["op"], c["M"], c["K"], c["N"], c["nnz"], longest):
         plan = dl.row_plan(ro)
@@ -285,7 +291,7 @@ def measure(dl, torch, np, c, args, steps, warmup, replays, ceiling_gbps, with_c
         "workload": c["name"], "op": OP_NAMES[c["op"]], "entry_point": ["spmm_csr_f32", "sddmm_csr_f32", "fused_sddmm_spmm_f32"][c["op"]],
         "M": c["M"], "K": c["K"], "N_or_D": c["N"], "nnz": c["nnz"], "steps": steps, "replays": replays,
         "launch_us": round(s * 1e6, 3), "replay_launch_us": t["all_us"], "host_wall_us_per_step": round(t["wall_per_step_s"] * 1e6, 3),
-        "launch": t["mode"], "row_plan": "plan" in info,
+        "launch": t["mode"], "row_plan": "plan" in info, "rows_even_hint": "rows_even" in info,
         "GFLOPs": round(acct["flops"] / s / 1e9, 2),
         "roofline": {"bound": "hbm", "achieved": round(acct["algorithmic_bytes"] / s / 1e9, 2), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(acct["algorithmic_bytes"] / s / 1e9 / HBM_PEAK_GBPS, 5), "traffic": traffic,

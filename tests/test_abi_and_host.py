@@ -42,8 +42,8 @@ def test_header_is_plain_c(tmp_path):
 
 def test_split_rule_and_the_even_rows_hint(dl):
     """Rows per workgroup: one for long rows of unknown evenness, four (a whole row per wave) once the caller says the
-    rows are even and the matrix has at least 2048 rows; the hint changes nothing for the benchmark configurations'
-    sizes or for short rows. Sixteen waves per row: never in the fused op on tall matrices, in SpMM only from
+    rows are even and the matrix has at least 2048 rows; the hint changes nothing for short rows or for the benchmark
+    configurations' sizes but the fourth. Sixteen waves per row: never in the fused op on tall matrices, in SpMM only from
     16384 rows on."""
     for op in (dl.OP_SPMM, dl.OP_SDDMM, dl.OP_FUSED):
         for width in (32, 128, 256):
@@ -60,9 +60,13 @@ def test_split_rule_and_the_even_rows_hint(dl):
         b = dl.describe_launch(op, 65536, 1024, 64, 65536 * 20, rows_even=True)
         assert a == b and a["R"] == 16
     for cfg in ((dl.OP_SPMM, 512, 512, 128, 78848), (dl.OP_SPMM, 2048, 512, 256, 105687),
-                (dl.OP_SDDMM, 2048, 2048, 128, 209715), (dl.OP_SPMM, 2048, 512, 392, 208896),
-                (dl.OP_FUSED, 4096, 4096, 64, 323000)):
+                (dl.OP_SDDMM, 2048, 2048, 128, 209715), (dl.OP_FUSED, 4096, 4096, 64, 323000)):
         assert dl.describe_launch(*cfg) == dl.describe_launch(*cfg, rows_even=True)
+    # where a row of the dense operand takes a whole wave (SpMM from 256 columns on), even rows are grouped from about a
+    # hundred nonzeros on: the fourth benchmark configuration (102 per row), not the same rows at N = 128
+    cfg4 = (dl.OP_SPMM, 2048, 512, 392, 208896)
+    assert dl.describe_launch(*cfg4)["R"] == 1 and dl.describe_launch(*cfg4, rows_even=True)["R"] == 4
+    assert dl.describe_launch(dl.OP_SPMM, 2048, 512, 128, 208896, rows_even=True)["R"] == 1
     long_rows = 2000
     assert dl.describe_launch(dl.OP_SPMM, 8192, 8192, 128, 8192 * long_rows)["W"] == 4
     assert dl.describe_launch(dl.OP_SPMM, 24576, 8192, 128, 24576 * long_rows)["W"] == 16
