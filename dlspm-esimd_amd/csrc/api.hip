@@ -191,7 +191,9 @@ SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial
     if (M <= 0 || K <= 0 || nnz <= 0 || width <= 0 || G <= 0) return p;  // G == 0: no sliced kernel for this layout
     const int force = tuning().slices;
     const long long l2 = device_info().l2_bytes;
-    const long long bytes = (long long)K * width * (long long)sizeof(float) * operands;
+    // (sizes no device holds are cut off at 2^50 bytes: they take the largest number of slices either way)
+    const double bytes_exact = (double)K * (double)width * (double)sizeof(float) * (double)operands;
+    const long long bytes = bytes_exact < (double)(1ll << 50) ? (long long)bytes_exact : (1ll << 50);
     long long slices = ceil_div(bytes * (partial_rows ? kSlicesPer2L2Partial : kSlicesPer2L2), 2 * l2);
     if (slices > kSliceMaxSlices) slices = kSliceMaxSlices;
     // Slices that leave a row its minimum share: 16 nonzeros per slice for dense rows of 256 floats and more, in
@@ -744,7 +746,7 @@ int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int pa
     if (op == DLSPM_OP_SPMM) {
         const SpmmShape s = spmm_choose(M, K, n, nnz, vec4, even, !memory);
         const int tw = s.G * s.vec * s.V;
-        shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[5] = s.W; shape[6] = s.R; shape[7] = (n + tw - 1) / tw;
+        shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[5] = s.W; shape[6] = s.R; shape[7] = (int)ceil_div(n, tw);
         const FlatPlan fp = flat_plan(M, nnz, n, s.G);
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_SDDMM) {
@@ -756,7 +758,7 @@ int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int pa
         const FusedShape s = fused_choose(M, n, nnz, vec4, even);
         const int tw = s.G * s.vec * s.V;
         shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R;
-        shape[7] = (n + tw - 1) / tw;
+        shape[7] = (int)ceil_div(n, tw);
         const FlatPlan fp = flat_plan(M, nnz, n, s.G);
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else {

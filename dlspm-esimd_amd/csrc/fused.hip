@@ -127,7 +127,7 @@ template <int VEC, int G1, int DS, int G, int V2, int W, int R>
 static hipError_t launch_one(const FusedArgs& x, hipStream_t stream)
 {
     constexpr int TW = G * VEC * V2;
-    const int col_tiles = (x.D + TW - 1) / TW;
+    const int col_tiles = (int)ceil_div(x.D, TW);
     const long long blocks = ceil_div(x.M, R) * col_tiles;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
@@ -185,7 +185,7 @@ FusedShape fused_choose(int M, int D, int nnz, bool vec4, bool rows_even)
     // rows per workgroup 1 / 2 / 4 / 8 / 16: 1024 rows 3.3 / 4.4 / 5.5 / 6.9 / 10.9 us; 2048 rows 4.8 / 4.9 / 6.1 / 7.8 /
     // 11.7 us; 4096 rows 7.3 / 7.2 / 6.5 / 8.0 / 11.6 us; 8192 rows 12.1 / 10.4 / 8.3 / 7.2 / 9.2 us; 16384 rows: sixteen;
     // 3072 rows of 102, even: two per workgroup 8.5 us, four 7.2 us)
-    choose_split(M, (D + tw - 1) / tw, nnz, SplitRule{3, tw >= 1024 ? 4 : 16, kWave / s.G, false, 96}, rows_even, s.W, s.R);
+    choose_split(M, ceil_div(D, tw), nnz, SplitRule{3, tw >= 1024 ? 4 : 16, kWave / s.G, false, 96}, rows_even, s.W, s.R);
     return s;
 }
 
@@ -274,7 +274,7 @@ template <int VEC, int G1, int DS, int G, int V2>
 static hipError_t launch_flat(const FusedArgs& x, const FlatPlan& plan, float* partial, hipStream_t stream)
 {
     constexpr int TW = G * VEC * V2;
-    const int col_tiles = (x.D + TW - 1) / TW;
+    const int col_tiles = (int)ceil_div(x.D, TW);
     const long long waves = (long long)plan.units * col_tiles;
     const long long blocks = (waves + kFlatWaves - 1) / kFlatWaves;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
@@ -319,7 +319,7 @@ static hipError_t launch_sliced_r(const FusedArgs& x, const SlicePlan& plan, con
                                   hipStream_t stream)
 {
     constexpr int TW = G * VEC * V2;
-    const int col_tiles = (x.D + TW - 1) / TW;
+    const int col_tiles = (int)ceil_div(x.D, TW);
     const long long slice_blocks = ceil_div(x.M, R) * col_tiles;
     const long long blocks = slice_blocks * plan.slices;
     if (blocks <= 0) return hipSuccess;

@@ -151,7 +151,7 @@ template <int VEC, int G, int V, int W, int R>
 static hipError_t launch_one(const SpmmArgs& x, int tile_major, hipStream_t stream)
 {
     constexpr int TW = G * VEC * V;
-    const int col_tiles = (x.N + TW - 1) / TW;
+    const int col_tiles = (int)ceil_div(x.N, TW);
     const long long blocks = ceil_div(x.M, R) * col_tiles;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
@@ -205,7 +205,7 @@ static int spmm_tile_width(int M, int K, int N, int nnz, bool narrow_tiles)
     const long long l2 = device_info().l2_bytes;
     const int min_tile = narrow_tiles ? 32 : 128;
     if (N <= min_tile) return 0;
-    bool on = (long long)K * N * (long long)sizeof(float) > l2 && (long long)M * ((N + 511) / 512) >= 8ll * device_info().cus;
+    bool on = (double)K * (double)N * (double)sizeof(float) > (double)l2 && (long long)M * ceil_div(N, 512) >= 8ll * device_info().cus;
     if (tuning().tile_major >= 0) on = tuning().tile_major != 0;
     if (!on) return 0;
     int tile = min_tile;
@@ -252,7 +252,7 @@ SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, b
         s.V = 1;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(M, (N + tw - 1) / tw, nnz, SplitRule{8, 16, kWave / s.G, true}, rows_even, s.W, s.R);
+    choose_split(M, ceil_div(N, tw), nnz, SplitRule{8, 16, kWave / s.G, true}, rows_even, s.W, s.R);
     return s;
 }
 
@@ -354,7 +354,7 @@ template <int VEC, int G, int V>
 static hipError_t launch_flat(const SpmmArgs& x, const FlatPlan& plan, int tile_major, float* partial, hipStream_t stream)
 {
     constexpr int TW = G * VEC * V;
-    const int col_tiles = (x.N + TW - 1) / TW;
+    const int col_tiles = (int)ceil_div(x.N, TW);
     const long long waves = (long long)plan.units * col_tiles;
     const long long blocks = (waves + kFlatWaves - 1) / kFlatWaves;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
@@ -387,7 +387,7 @@ static hipError_t launch_sliced_r(const SpmmArgs& x, const SlicePlan& plan, int 
                                   float* partial, hipStream_t stream)
 {
     constexpr int TW = G * VEC * V;
-    const int col_tiles = (x.N + TW - 1) / TW;
+    const int col_tiles = (int)ceil_div(x.N, TW);
     const long long slice_blocks = ceil_div(x.M, R) * col_tiles;
     const long long blocks = slice_blocks * plan.slices;
     if (blocks <= 0) return hipSuccess;
@@ -478,7 +478,7 @@ hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int*
     const int *starts = plan, *ends = plan + x.M, *rows = plan + 2 * (size_t)x.M;
 #define DLSPM_PLANNED(g_, v_)                                                                                          \
     if (s.G == g_ && s.V == v_) {                                                                                      \
-        const int col_tiles = (x.N + g_ * 4 * v_ - 1) / (g_ * 4 * v_);                                                 \
+        const int col_tiles = (int)ceil_div(x.N, g_ * 4 * v_);                                                         \
         const long long blocks = (long long)x.M * col_tiles;                                                           \
         if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;                                                \
         if (dense_fits_buffer(x.K, x.N))                                                                               \

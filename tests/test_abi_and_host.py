@@ -456,3 +456,13 @@ def test_accounting_formulas(dl):
     f = dl.account(dl.OP_FUSED, 4096, 4096, 64, 327680)
     assert f["flops"] == (2 * 327680 - 4096) * 64 + 327680 * (2 * 64 - 1) + 327680
     assert f["algorithmic_bytes"] == 4 * 4097 + 4 * 327680 + 4 * 4096 * 64 + 8 * 4096 * 64 + 4 * 4096 * 64
+
+
+def test_host_entry_points_over_edge_and_random_sizes():
+    """tests/host_fuzz: every host-side entry point (and, where there is no device, the compute entry points, which
+    must answer with a status) over edge values and random sizes up to INT_MAX; `make -C tests/host_fuzz san` runs
+    the same program against a build of the library with ASan and UBSan on the host side."""
+    d = os.path.join(ROOT, "tests", "host_fuzz")
+    r = subprocess.run(["make", "-C", d, "run"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "nothing reported" in r.stdout
