@@ -42,7 +42,8 @@
  *   - Three more things travel through the same pair of arguments, as hint bits in the upper byte of `workspace_bytes`
  *     (DLSPM_HINT_*, or-ed into the size; they are no part of the size):
  *       DLSPM_HINT_ROWS_EVEN, with workspace NULL: the caller knows that no row is much longer than the mean (longest
- *         row at most one and a half times nnz / M). Tall matrices of long rows then run one whole row per wave, which
+ *         row at most one and a half times nnz / M). Tall matrices of long rows (from 2048 rows of 128 nonzeros; SpMM
+ *         from 256 columns on: of about a hundred) then run one whole row per wave, which
  *         is the faster split for even rows and the slower one for uneven rows. It is a hint about speed only: a wrong
  *         one costs time, never correctness (a row's products are added in a different, equally fixed order), and
  *         other sizes ignore it.
@@ -207,10 +208,11 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
  *                            workspace_bytes = plan_bytes | DLSPM_HINT_ROW_PLAN. The plan must have been built from the
  *                            same row_offsets (a stale plan gives wrong values but stays inside the arrays). A planned
  *                            launch runs one row per workgroup also where the size rule would group a few rows, if the
- *                            rows are long enough. Short rows, column tiles of a B that fits one L2, widths below 4
- *                            (SDDMM and the fused op: widths outside 16 < D <= 512, and rows that the size rule groups
- *                            in masks of more than 4096 rows, 8192 at D >= 128 and 128 nonzeros per row) ignore the
- *                            plan and run as with NULL. A planned launch is one kernel (no memset, no allocation, no
+ *                            rows are long enough (SDDMM and the fused op up to 2048 rows: whatever their length).
+ *                            Short rows, column tiles of a B that fits one L2, widths below 4 (SDDMM and the fused
+ *                            op: widths outside 16 < D <= 512, and rows that the size rule groups in masks of more
+ *                            than 4096 rows, 8192 at D >= 128 and 128 nonzeros per row) ignore the plan and run as
+ *                            with NULL. A planned launch is one kernel (no memset, no allocation, no
  *                            synchronisation); the plan is only read, so launches may share it.
  *   *_planned                the same launches with the plan as a separate argument (plan == NULL: the plain call).
  * No counterpart in the reference, whose kernels take the rows in matrix order (SPMM/spmmesimd2.hpp:63-75).
@@ -218,9 +220,9 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
 size_t dlspm_row_plan_bytes(int M);
 /* 1 if a row plan is worth building for op (DLSPM_OP_*) at these sizes and this longest row (-1: unknown): the planned
  * launch would use it (one column tile, rows of at least 32 nonzeros on average where the size rule would group rows;
- * SDDMM and the fused op: 16 < D <= 512), the rows are
- * not known to be even, and B is not so far beyond one L2 that the column-sliced schedule's workspace matters more;
- * else 0. Ask this before dlspm_workspace_advice: where both a plan and the flat schedule's workspace apply, the plan
+ * SDDMM and the fused op: 16 < D <= 512, up to 2048 rows also shorter rows), the rows are not known to be even (SDDMM
+ * on rows below 32 nonzeros: the longest is at least eight times the mean), and B is not so far beyond one L2 that the
+ * column-sliced schedule's workspace matters more; else 0. Ask this before dlspm_workspace_advice: where both a plan and the flat schedule's workspace apply, the plan
  * is 10-40 % faster. */
 int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row_len);
 int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_bytes, void* stream);
