@@ -268,11 +268,10 @@ void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bo
         // floats twice in the fused op), because waves that start together then sweep the columns together. With
         // uneven rows the same grouping is 5-20 % slower (four rows of work per workgroup make the tail of the
         // launch coarser), hence only on the caller's word. Rows below 128 nonzeros keep the grouping of the size rule
-        // (4096 rows of ~100: four per workgroup measured 6 % slower than two) -- except where a row of the dense operand
-        // takes a whole wave (slots == 1, SpMM from 256 columns on): there the grouping pays from about a hundred
-        // nonzeros per row (2048 x 512 with 102 per row: N = 392 14.9 -> 14.5 us, N = 256 9.7 -> 8.9 us).
-        const double even_from = rule.slots == 1 ? 96.0 : 128.0;
-        if (rows_even && R < 4 && avg >= even_from && ceil_div(M, 4) * col_tiles >= 2 * cus) R = 4;
+        // (4096 rows of ~100: four per workgroup measured 6 % slower than two) -- except in SpMM where a row of the dense
+        // operand takes a whole wave (from 256 columns on; rule.even_rows_avg): there the grouping pays from about a
+        // hundred nonzeros per row (2048 x 512 with 102 per row: N = 392 14.9 -> 14.5 us, N = 256 9.7 -> 8.9 us).
+        if (rows_even && R < 4 && avg >= rule.even_rows_avg && ceil_div(M, 4) * col_tiles >= 2 * cus) R = 4;
     }
 }
 

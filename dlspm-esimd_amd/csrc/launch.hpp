@@ -161,6 +161,7 @@ struct SplitRule {
     int slots;
     bool w16_long_rows;
     int w8_few_rows_avg = 0;  // > 0: eight waves per row from this many nonzeros per row on where there are few rows
+    int even_rows_avg = 128;  // rows known to be even are grouped four to a workgroup from this many nonzeros per row on
 };
 void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bool rows_even, int& W, int& R);
 

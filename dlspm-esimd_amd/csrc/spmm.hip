@@ -252,7 +252,7 @@ SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, b
         s.V = 1;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(M, ceil_div(N, tw), nnz, SplitRule{8, 16, kWave / s.G, true}, rows_even, s.W, s.R);
+    choose_split(M, ceil_div(N, tw), nnz, SplitRule{8, 16, kWave / s.G, true, 0, s.G == kWave ? 96 : 128}, rows_even, s.W, s.R);
     return s;
 }
 
