@@ -2,7 +2,7 @@
 """Benchmark of the sparse hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--replays R] [--no-graph] [--no-cpu] [--no-plan]
-                    [--headline-only]
+                    [--headline-only] [--no-cold] [--no-null]
 
 A "step" is one launch of the configuration's kernel through the library's named entry point (default:
 BASELINE.json's configs[1], fp32 CSR SpMM 2048x512 * 512x256 at 90 % sparsity with lognormal-skewed rows, through
@@ -29,11 +29,15 @@ Prints ONE JSON line:
                     loop over all cores; one per configuration in all_configs
   warm_us / cold_us per-launch time back to back (the graph above) and with the caches flushed before every launch:
                     [1 GiB fill -> launch] pairs replayed from one graph, minus the same graph without the launches
-  row_plan          (uneven rows) the steps pass the row plan as their workspace (DLSPM_HINT_ROW_PLAN); the plan is built
-                    once per matrix, on the device, before the timed region; this object gives what building it costs
-                    and the time of the same launches in matrix order (--no-plan measures those as the headline)
-  rows_even_hint    (per configuration) the steps pass DLSPM_HINT_ROWS_EVEN: dlspm_workspace_advice said so for the
-                    longest row that one look at the row lengths found (dlspm_csr_row_stats), as the C++ drivers do
+  prepared          what the steps pass as (workspace, workspace_bytes): the answer of dlspm_advise to one look at the
+                    matrix (dlspm_analyze), as the C++ drivers do -- a row plan for the uneven rows of the headline
+                    (DLSPM_HINT_ROW_PLAN; built once per matrix, on the device, before the timed region),
+                    DLSPM_HINT_ROWS_EVEN for the even rows of three others. `prepare_us` says what that costs once per
+                    matrix (the synchronising analysis, on the host's clock, and the plan build, on the device's);
+                    --no-plan measures the launches that pass NULL as the headline
+  null_call_us      the same K-step graph with workspace = NULL, 0 (the plain drop-in call), beside launch_us
+  host_enqueue_us   what one call costs the host outside a graph (200 calls issued without synchronising, wall time per
+                    call): the plain call, the prepared call, and an empty kernel launch (the runtime's own share)
   all_configs       the same measurement for every benchmark configuration (shorter runs)
 """
 import argparse
@@ -61,6 +65,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-plan", action="store_true", help="launch in matrix order, without the row plan")
     ap.add_argument("--headline-only", action="store_true", help="skip the other four configurations")
+    ap.add_argument("--no-cold", action="store_true", help="skip the cold-cache leg (kernel traces of the timed graph alone)")
+    ap.add_argument("--no-null", action="store_true", help="skip the legs that time the plain call (NULL workspace) and the plan build")
     return ap.parse_args()
 
 
@@ -69,36 +75,38 @@ def median(xs):
     return s[len(s) // 2]
 
 
-def make_step(dl, torch, c, use_plan=True, info=None):
+def make_step(dl, torch, c, prepared=True, info=None):
     """Uploads configuration c and returns (step_fn, output tensor). What a caller does once per matrix happens here,
-    outside the timed steps: one look at the row lengths and, on uneven rows, the row plan (built on the device)."""
+    outside the timed steps: one look at the matrix (dlspm_analyze), the library's answer for this op and width
+    (dlspm_advise), and what that answer asks to allocate and build. prepared=False: the plain call, workspace = NULL."""
     d = lambda a: torch.from_numpy(a).cuda()
     ro, ci = d(c["row_offsets"]), d(c["col_indices"])
-    need = dl.workspace_bytes(c["op"], c["M"], c["K"], c["N"], c["nnz"])  # 0 at the sizes of the five configurations
-    ws = torch.empty(need, dtype=torch.uint8, device="cuda") if need else None
-    longest, _ = dl.csr_row_stats(ro)
-    if not need and dl.workspace_advice(c["op"], c["M"], c["K"], c["N"], c["nnz"], longest) == dl.PASS_ROWS_EVEN:
-        ws = dl.ROWS_EVEN  # no memory: the hint that no row is much longer than the mean (cfg1, cfg3, cfg4)
+    prep = None
+    if prepared:
+        t0 = time.perf_counter()
+        mi = dl.analyze(ro, ci, c["K"])
+        t1 = time.perf_counter()
+        prep = dl.prepare(ro, ci, c["K"], c["op"], c["N"], info=mi)
         if info is not None:
-            info["rows_even"] = True
-    plan = None
-    if use_plan and dl.row_plan_advice(c["op"], c["M"], c["K"], c["N"], c["nnz"], longest):
-        plan = dl.row_plan(ro)
-        ws = None
-        if info is not None:
-            info["row_offsets"] = ro
-            info["plan"] = plan
+            info.update({"row_offsets": ro, "prepared": prep, "matrix_info": mi.as_dict(), "analyze_host_us": (t1 - t0) * 1e6})
     if c["op"] == dl.OP_SPMM:
         va, B = d(c["values"]), d(c["d0"])
         out = torch.empty((c["M"], c["N"]), dtype=torch.float32, device="cuda")
-        return (lambda: dl.spmm(ro, ci, va, B, K=c["K"], out=out, workspace=ws, plan=plan)), out
-    if c["op"] == dl.OP_SDDMM:
+        step = lambda: dl.spmm(ro, ci, va, B, K=c["K"], out=out, plan=prep)
+        raw = ("spmm", (c["M"], c["K"], c["N"], c["nnz"], ro, ci, va, B, out))
+    elif c["op"] == dl.OP_SDDMM:
         lhs, rhs = d(c["d0"]), d(c["d1"])
         out = torch.empty((c["nnz"],), dtype=torch.float32, device="cuda")
-        return (lambda: dl.sddmm(ro, ci, lhs, rhs, out=out, workspace=ws, plan=plan)), out
-    Q, Km, V = d(c["d0"]), d(c["d1"]), d(c["d2"])
-    out = torch.empty((c["M"], c["N"]), dtype=torch.float32, device="cuda")
-    return (lambda: dl.fused(ro, ci, Q, Km, V, c["scale"], out=out, workspace=ws, plan=plan)), out
+        step = lambda: dl.sddmm(ro, ci, lhs, rhs, out=out, plan=prep)
+        raw = ("sddmm", (c["M"], c["K"], c["N"], c["nnz"], ro, ci, lhs, rhs, out))
+    else:
+        Q, Km, V = d(c["d0"]), d(c["d1"]), d(c["d2"])
+        out = torch.empty((c["M"], c["N"]), dtype=torch.float32, device="cuda")
+        step = lambda: dl.fused(ro, ci, Q, Km, V, c["scale"], out=out, plan=prep)
+        raw = ("fused", (c["M"], c["K"], c["N"], c["nnz"], ro, ci, Q, Km, V, c["scale"], out))
+    if info is not None:
+        info["raw"] = raw
+    return step, out
 
 
 def capture(torch, stream, body):
@@ -234,6 +242,46 @@ class Probe:
         self.lib.dlspm_probe_gather.restype = ctypes.c_int
         self.lib.dlspm_probe_copy.argtypes = [vp, vp, ctypes.c_size_t, vp]
         self.lib.dlspm_probe_copy.restype = ctypes.c_int
+        ci, sz, st = ctypes.c_int, ctypes.c_size_t, ctypes.POINTER(ctypes.c_int)
+        for name, args in (("spmm", [vp] * 5), ("sddmm", [vp] * 5), ("fused", [vp] * 5 + [ctypes.c_float, vp])):
+            f = getattr(self.lib, "dlspm_probe_enqueue_" + name)
+            f.restype = ctypes.c_double
+            f.argtypes = [vp, ci, ci, ci, ci, ci] + args + [vp, sz, vp, st]
+        self.lib.dlspm_probe_enqueue_empty.restype = ctypes.c_double
+        self.lib.dlspm_probe_enqueue_empty.argtypes = [ci, vp]
+
+    def host_enqueue_us(self, dl, torch, raw, prepared, calls=200, reps=5):
+        """Host microseconds per call of the entry point, issued `calls` times without synchronising, outside a graph
+        (median of `reps` such runs): the plain call (NULL, 0), the prepared call, and an empty kernel launch."""
+        name, a = raw
+        fn = ctypes.cast(getattr(dl.lib(), {"spmm": "spmm_csr_f32", "sddmm": "sddmm_csr_f32", "fused": "fused_sddmm_spmm_f32"}[name]),
+                         ctypes.c_void_p)
+        ptr = lambda t: t.data_ptr() if hasattr(t, "data_ptr") else t
+        status = ctypes.c_int(0)
+        run = getattr(self.lib, "dlspm_probe_enqueue_" + name)
+
+        def one(ws, size):
+            xs = []
+            for _ in range(reps):
+                torch.cuda.synchronize()
+                xs.append(run(fn, calls, *[ptr(x) for x in a], ws, size, None, ctypes.byref(status)))
+                torch.cuda.synchronize()
+                if status.value != 0:
+                    raise RuntimeError(f"{name}: status {status.value} in the host-enqueue leg")
+            return round(median(xs), 2)
+
+        def empty():
+            xs = []
+            for _ in range(reps):
+                torch.cuda.synchronize()
+                xs.append(self.lib.dlspm_probe_enqueue_empty(calls, None))
+                torch.cuda.synchronize()
+            return round(median(xs), 2)
+
+        out = {"plain_call": one(None, 0), "empty_kernel_launch": empty(), "calls": calls}
+        if prepared is not None:
+            out["prepared_call"] = one(prepared.memory.data_ptr() if prepared.memory is not None else None, prepared.size_and_hints)
+        return out
 
     def gather_ceiling(self, torch, use_graph=True):
         """TB/s of whole-wave 1 KiB row gathers: random rows of a 512 KiB table (fits every L2: the ceiling the
@@ -275,26 +323,55 @@ class Probe:
         return {"kernel": "dlspm_probe_copy_kernel", "launches": reps, "bytes_read": n * 4, "bytes_written": n * 4}
 
 
-def measure(dl, torch, np, c, args, steps, warmup, replays, ceiling_gbps, with_cpu, cpu_budget):
+HINT_NAMES = (("HINT_ROW_PLAN", "DLSPM_HINT_ROW_PLAN"), ("HINT_CUT_PLAN", "DLSPM_HINT_CUT_PLAN"), ("HINT_ROWS_EVEN", "DLSPM_HINT_ROWS_EVEN"),
+              ("HINT_BANDED", "DLSPM_HINT_BANDED"), ("HINT_ROWS_SKEWED", "DLSPM_HINT_ROWS_SKEWED"))
+
+
+def launch_signature(dl, c, prep):
+    """What identifies the launch a traffic figure was recorded for: op, lane layout, split and the hints passed."""
+    sh = dl.describe_launch(c["op"], c["M"], c["K"], c["N"], c["nnz"], rows_even=bool(prep and prep.call_plan.hints & dl.HINT_ROWS_EVEN))
+    hints = "+".join(n for a, n in HINT_NAMES if prep and prep.call_plan.hints & getattr(dl, a)) or "NULL"
+    planned = bool(prep and prep.call_plan.build)
+    return (f"{OP_NAMES[c['op']]}:vec{sh['vec']}:row-lanes{sh['G']}x{sh['V']}:dot-lanes{sh['G1']}x{sh['DS']}:"
+            f"W{sh['W']}:R{1 if planned else sh['R']}:{hints}")
+
+
+def measure(dl, torch, np, c, args, probe, steps, warmup, replays, ceiling_gbps, with_cpu, cpu_budget):
     """Every figure of one configuration."""
     acct = dl.account(c["op"], c["M"], c["K"], c["N"], c["nnz"])
     info = {}
     step, out = make_step(dl, torch, c, not args.no_plan, info)
+    prep = info.get("prepared")
     t = time_steps(torch, step, steps, warmup, replays, not args.no_graph, split_overhead=steps < 1000)
     s = t["per_step_s"]
-    traffic = None
+    # HBM-side traffic: recorded by rocprofv3 --pmc runs (profiles/pmc_traffic.json), valid for the launch it names only
+    traffic, traffic_source = None, None
+    signature = launch_signature(dl, c, prep)
     pmc_path = os.path.join(ROOT, "profiles", "pmc_traffic.json")
     if os.path.exists(pmc_path):
-        traffic = json.load(open(pmc_path)).get(c["name"], {}).get("traffic_bytes_per_launch")
+        rec = json.load(open(pmc_path)).get(c["name"], {})
+        if rec.get("launch") == signature:
+            traffic = rec.get("traffic_bytes_per_launch")
+            traffic_source = f"recorded@{rec.get('commit', '?')} for {rec.get('kernel', '?')}"
+        elif rec:
+            traffic_source = f"stale: recorded for {rec.get('launch', 'an unnamed launch')}, this run launches {signature}"
     eff_gbps = acct["effective_bytes"] / s / 1e9
+    entry = ["spmm_csr_f32", "sddmm_csr_f32", "fused_sddmm_spmm_f32"][c["op"]]
+    hints = [n for a, n in HINT_NAMES if prep and prep.call_plan.hints & getattr(dl, a)]
     r = {
-        "workload": c["name"], "op": OP_NAMES[c["op"]], "entry_point": ["spmm_csr_f32", "sddmm_csr_f32", "fused_sddmm_spmm_f32"][c["op"]],
+        "workload": c["name"], "op": OP_NAMES[c["op"]], "entry_point": entry + "".join(" + " + h for h in hints),
         "M": c["M"], "K": c["K"], "N_or_D": c["N"], "nnz": c["nnz"], "steps": steps, "replays": replays,
         "launch_us": round(s * 1e6, 3), "replay_launch_us": t["all_us"], "host_wall_us_per_step": round(t["wall_per_step_s"] * 1e6, 3),
-        "launch": t["mode"], "row_plan": "plan" in info, "rows_even_hint": "rows_even" in info,
+        "launch": t["mode"], "launch_signature": signature,
+        "prepared": {"build": ["nothing", "dlspm_row_plan_build", "dlspm_row_plan_build_cut"][prep.call_plan.build],
+                     "workspace_bytes": int(prep.call_plan.bytes), "hints": hints} if prep else None,
+        "row_plan": bool(prep and prep.call_plan.build == dl.BUILD_ROW_PLAN),
+        "rows_even_hint": bool(prep and prep.call_plan.hints & dl.HINT_ROWS_EVEN),
+        "matrix_info": info.get("matrix_info"),
         "GFLOPs": round(acct["flops"] / s / 1e9, 2),
         "roofline": {"bound": "hbm", "achieved": round(acct["algorithmic_bytes"] / s / 1e9, 2), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(acct["algorithmic_bytes"] / s / 1e9 / HBM_PEAK_GBPS, 5), "traffic": traffic,
+                     "traffic_source": traffic_source,
                      "traffic_over_algorithmic": round(traffic / acct["algorithmic_bytes"], 2) if traffic else None,
                      "algorithmic_bytes": acct["algorithmic_bytes"], "launch_us": round(s * 1e6, 3)},
         "effective_GBps": round(eff_gbps, 1), "effective_fraction": round(eff_gbps / HBM_PEAK_GBPS, 4),
@@ -305,21 +382,46 @@ def measure(dl, torch, np, c, args, steps, warmup, replays, ceiling_gbps, with_c
     if "steady_per_step_s" in t:
         r["steady_state_launch_us"] = round(t["steady_per_step_s"] * 1e6, 3)
         r["replay_overhead_us"] = round(t["replay_overhead_s"] * 1e6, 2)
-    cold = cold_launch_us(torch, step) if not args.no_graph else None
+    cold = cold_launch_us(torch, step) if not (args.no_graph or args.no_cold) else None
     r["cold_us"] = cold["us"] if cold else None
     r["cold_detail"] = cold
-    if "plan" in info:
-        # what the plan costs once per matrix (kernels on the stream, no synchronisation), and the same launches without it
-        ro, plan = info["row_offsets"], info["plan"]
-        build = time_steps(torch, lambda: dl.row_plan(ro, out=plan), 20, 3, 5, not args.no_graph)
-        plain, _ = make_step(dl, torch, c, False)
+    if not args.no_null:
+        # the plain drop-in call (workspace = NULL, 0) in the same kind of graph, and what the preparation costs once per matrix
         k = min(steps, 500)
-        without = time_steps(torch, plain, k, min(warmup, 50), replays, not args.no_graph)
-        r["row_plan_detail"] = {"build_us_once_per_matrix": round(build["per_step_s"] * 1e6, 2),
+        if prep is not None and (prep.memory is not None or prep.call_plan.hints):
+            plain, _ = make_step(dl, torch, c, False)
+            without = time_steps(torch, plain, k, min(warmup, 50), replays, not args.no_graph)
+            r["null_call_us"] = round(without["per_step_s"] * 1e6, 3)
+        else:
+            r["null_call_us"] = r["launch_us"]  # nothing is passed: the timed launches are the plain call
+        prepare = {"analyze_host_us": round(info.get("analyze_host_us", 0.0), 1),
+                   "analyze": "dlspm_analyze: one pass over the CSR structure on the device, synchronises, host wall time"}
+        if prep is not None and prep.call_plan.build:
+            ro, mem = info["row_offsets"], prep.memory
+            build_fn = dl.lib().dlspm_row_plan_build if prep.call_plan.build == dl.BUILD_ROW_PLAN else dl.lib().dlspm_row_plan_build_cut
+            M = c["M"]
+
+            def build():
+                st = build_fn(M, ctypes.c_void_p(ro.data_ptr()), ctypes.c_void_p(mem.data_ptr()), mem.numel() * 4,
+                              ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+                if st != 0:
+                    raise RuntimeError(f"plan build: status {st}")
+
+            built = time_steps(torch, build, 20, 3, 5, not args.no_graph)
+            prepare["build_us"] = round(built["per_step_s"] * 1e6, 2)
+            prepare["build"] = "kernels on the stream, no host copy, no synchronisation (capturable); HIP events, graph of 20 builds"
+            gain = (r["null_call_us"] - r["launch_us"])
+            prepare["launches_until_the_build_pays"] = round(prepare["build_us"] / gain, 1) if gain > 0 else None
+        r["prepare_us"] = prepare
+        r["host_enqueue_us"] = probe.host_enqueue_us(dl, torch, info["raw"], prep)
+    if r.get("row_plan") and "prepare_us" in r:
+        r["row_plan_detail"] = {"build_us_once_per_matrix": r["prepare_us"].get("build_us"),
                                 "build": "dlspm_row_plan_build: kernels on the stream, no host copy, no synchronisation",
-                                "launch_us_without_plan": round(without["per_step_s"] * 1e6, 3)}
+                                "launch_us_without_plan": r["null_call_us"]}
     if with_cpu:
         r["cpu_baseline"], ref = cpu_baseline(dl, c, acct, *cpu_budget)
+        torch.cuda.synchronize()
+        step()
         torch.cuda.synchronize()
         got = out.cpu().numpy()
         num = float(np.linalg.norm(got.astype(np.float64).ravel() - ref.astype(np.float64).ravel()))
@@ -351,7 +453,7 @@ def main():
 
     ceiling = probe.gather_ceiling(torch, not args.no_graph)
     c = dl.make_config(args.config)
-    head, acct = measure(dl, torch, np, c, args, args.steps, args.warmup, replays, ceiling["value"], not args.no_cpu, (6.0, 3.0))
+    head, acct = measure(dl, torch, np, c, args, probe, args.steps, args.warmup, replays, ceiling["value"], not args.no_cpu, (6.0, 3.0))
     s = head["launch_us"] * 1e-6
 
     result = {
@@ -381,6 +483,9 @@ def main():
         result["rel_frobenius_vs_cpu"] = head["rel_frobenius_vs_cpu"]
     if "row_plan_detail" in head:
         result["row_plan"] = head["row_plan_detail"]
+    for key in ("null_call_us", "prepare_us", "host_enqueue_us", "prepared", "matrix_info"):
+        if key in head:
+            result[key] = head[key]
     info = dl.device_info()
     result["device"] = {"compute_units": info["compute_units"], "l2_bytes": info["l2_bytes"], "name": torch.cuda.get_device_name(0)}
 
@@ -392,7 +497,7 @@ def main():
                 continue
             cc = dl.make_config(cfg)
             k = min(args.steps, 500)
-            rr, _ = measure(dl, torch, np, cc, args, k, min(args.warmup, 50), replays, ceiling["value"], not args.no_cpu, (2.5, 1.5))
+            rr, _ = measure(dl, torch, np, cc, args, probe, k, min(args.warmup, 50), replays, ceiling["value"], not args.no_cpu, (2.5, 1.5))
             others[cc["name"]] = {k2: v for k2, v in rr.items() if k2 not in ("replay_launch_us",)}
         result["all_configs"] = others
 

@@ -18,7 +18,7 @@ namespace dlspm {
 
 static thread_local int t_last_hip_error = 0;
 
-static int fail_hip(hipError_t e)
+int fail_hip(hipError_t e)
 {
     t_last_hip_error = (int)e;
     return DLSPM_E_LAUNCH;
@@ -52,6 +52,8 @@ static Tuning tuning_from_environment()
     number("DLSPM_PLAN_ORDER", t.plan_order);
     number("DLSPM_XCD_CONTIGUOUS", t.xcd_contiguous);
     number("DLSPM_STREAM_RESULTS", t.stream_results);
+    number("DLSPM_CUT_PIECE_PCT", t.cut_piece_pct);
+    number("DLSPM_CUT_LONGEST_PCT", t.cut_longest_pct);
     return t;
 }
 static const Tuning& process_tuning()
@@ -76,6 +78,10 @@ const DeviceInfo& device_info()
         (void)hipGetLastError();  // a machine without a device is not an error of the caller's next HIP call
         return kNoDevice;
     }
+    // the device this thread asked about last: no lock on that path (an entry of the cache never changes once written)
+    static thread_local int t_last_dev = -1;
+    static thread_local const DeviceInfo* t_last_info = nullptr;
+    if (dev == t_last_dev) return *t_last_info;
     std::lock_guard<std::mutex> lock(mutex);
     if (!known[dev]) {
         DeviceInfo d = kNoDevice;
@@ -92,14 +98,12 @@ const DeviceInfo& device_info()
         cache[dev] = d;
         known[dev] = true;
     }
+    t_last_dev = dev;
+    t_last_info = &cache[dev];
     return cache[dev];
 }
 // DLSPM_OK if the current device can run the kernels
-static int require_device()
-{
-    const DeviceInfo& d = device_info();
-    return d.present && d.gfx950 ? DLSPM_OK : DLSPM_E_NO_DEVICE;
-}
+static int require_device(const DeviceInfo& d) { return d.present && d.gfx950 ? DLSPM_OK : DLSPM_E_NO_DEVICE; }
 
 // What the caller passed as (workspace, workspace_bytes): device memory, and the hints in the upper bits of the size.
 struct WorkspaceArg {
@@ -107,15 +111,26 @@ struct WorkspaceArg {
     size_t bytes;
     bool rows_even;
     bool row_plan;
+    bool cut_plan;
     bool banded;
+    bool skewed;
+    bool bad_hint;  // a bit of the hint byte that means nothing, or a row plan of a size no plan has
 };
 static WorkspaceArg workspace_arg(void* workspace, size_t workspace_bytes)
 {
     WorkspaceArg a{};
     a.rows_even = (workspace_bytes & DLSPM_HINT_ROWS_EVEN) != 0 || workspace == DLSPM_ROWS_EVEN;
     a.row_plan = (workspace_bytes & DLSPM_HINT_ROW_PLAN) != 0;
+    a.cut_plan = (workspace_bytes & DLSPM_HINT_CUT_PLAN) != 0;
     a.banded = (workspace_bytes & DLSPM_HINT_BANDED) != 0;
+    a.skewed = (workspace_bytes & DLSPM_HINT_ROWS_SKEWED) != 0;
     a.bytes = workspace_bytes & ~DLSPM_HINT_MASK;
+    // A caller that passes "plenty" (SIZE_MAX) as the size of scratch memory would set every hint bit: bits without a
+    // meaning are refused, and so is a plan of 2^48 bytes and more (no plan is that large; a size with stray upper bits is)
+    constexpr size_t known =
+        DLSPM_HINT_ROWS_EVEN | DLSPM_HINT_ROW_PLAN | DLSPM_HINT_CUT_PLAN | DLSPM_HINT_BANDED | DLSPM_HINT_ROWS_SKEWED;
+    a.bad_hint = (workspace_bytes & DLSPM_HINT_MASK & ~known) != 0 || ((a.row_plan || a.cut_plan) && a.bytes >= ((size_t)1 << 48)) ||
+                 (a.row_plan && a.cut_plan) || (a.rows_even && a.skewed) || (workspace == DLSPM_ROWS_EVEN && a.bytes != 0);
     a.mem = workspace == DLSPM_ROWS_EVEN ? nullptr : workspace;
     if (!a.mem || a.bytes == 0) {
         a.mem = nullptr;
@@ -141,7 +156,7 @@ constexpr int kFlatUnitsPerCu = 128;     // waves wanted at least: four rounds o
 constexpr int kFlatMinNnzSddmm = 1 << 21;
 constexpr int kFlatMinRowSddmm = 256;
 
-FlatPlan flat_plan(int M, int nnz, int width, int G)
+FlatPlan flat_plan(const DeviceInfo& dev, int M, int nnz, int width, int G)
 {
     FlatPlan p{0, 0, 0};
     if (M <= 0 || nnz <= 0 || width <= 0) return p;
@@ -149,7 +164,7 @@ FlatPlan flat_plan(int M, int nnz, int width, int G)
     const bool by_rule = nnz >= kFlatMinNnz && (long long)nnz >= (long long)kFlatMinRow * M && G >= kFlatMinLanes;
     if (force == 0 || (force < 0 && !by_rule)) return p;
     long long chunk = nnz >= (1 << 21) ? 512 : 256;  // at least eight (four) passes of 64 nonzeros per wave
-    const long long target_units = (long long)kFlatUnitsPerCu * device_info().cus;
+    const long long target_units = (long long)kFlatUnitsPerCu * dev.cus;
     const long long even = ceil_div(nnz, target_units);
     if (even > chunk) chunk = (even + 63) / 64 * 64;
     if (tuning().flat_chunk >= 64) chunk = tuning().flat_chunk;
@@ -159,11 +174,11 @@ FlatPlan flat_plan(int M, int nnz, int width, int G)
     return p;
 }
 
-static FlatPlan sddmm_flat_plan(int M, int nnz, int D)
+static FlatPlan sddmm_flat_plan(const DeviceInfo& dev, int M, int nnz, int D)
 {
     const int force = tuning().flat;
     if (force < 0 && (nnz < kFlatMinNnzSddmm || (long long)nnz < (long long)kFlatMinRowSddmm * M)) return FlatPlan{0, 0, 0};
-    return flat_plan(M, nnz, D, kWave);
+    return flat_plan(dev, M, nnz, D, kWave);
 }
 
 // Column-sliced schedule (the device works through the column ranges of the sparse matrix one after the other, partial
@@ -184,13 +199,13 @@ constexpr int kSliceMaxSlices = 16;
 constexpr int kSliceMinRow = 16;  // least mean nonzeros of a row inside one slice; fewer slices rather than shorter shares
 constexpr int kSliceMinRowAtL2 = 256;  // the same for an operand that just fills one L2
 
-SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial_width, int G, bool partial_rows,
+SlicePlan slice_plan(const DeviceInfo& dev, int M, int K, int width, int nnz, int operands, int partial_width, int G, bool partial_rows,
                      int slots, int blocks_per_cu)
 {
     SlicePlan p{0, 1, 0, 0};
     if (M <= 0 || K <= 0 || nnz <= 0 || width <= 0 || G <= 0) return p;  // G == 0: no sliced kernel for this layout
     const int force = tuning().slices;
-    const long long l2 = device_info().l2_bytes;
+    const long long l2 = dev.l2_bytes;
     // (sizes no device holds are cut off at 2^50 bytes: they take the largest number of slices either way)
     const double bytes_exact = (double)K * (double)width * (double)sizeof(float) * (double)operands;
     const long long bytes = bytes_exact < (double)(1ll << 50) ? (long long)bytes_exact : (1ll << 50);
@@ -213,14 +228,14 @@ SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial
     if (slices < 2) return p;
     p.slices = (int)slices;
     int W = 4;
-    choose_split(M, 1, (int)(nnz / slices), SplitRule{blocks_per_cu, 4, slots, false}, false, W, p.R);
+    choose_split(dev, M, 1, (int)(nnz / slices), SplitRule{blocks_per_cu, 4, slots, false}, false, W, p.R);
     if (W != 4) p.R = 1;  // only four-wave workgroups are built for this schedule
     p.bounds_bytes = (((size_t)(slices + 1) * M * sizeof(int)) + 255) / 256 * 256;
     p.bytes = p.bounds_bytes + (size_t)slices * M * (size_t)partial_width * sizeof(float);
     return p;
 }
 
-void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bool rows_even, int& W, int& R)
+void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, const SplitRule& rule, bool rows_even, int& W, int& R)
 {
     static const int kPairs[][2] = {{4, 16}, {4, 8}, {4, 4}, {4, 2}, {4, 1}, {8, 4}, {8, 2}, {8, 1}, {16, 1}};
     if (tuning().split_w > 0) {
@@ -231,7 +246,7 @@ void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bo
                 return;
             }
     }
-    const long long cus = device_info().cus;  // the thresholds below were measured on 256 compute units and scale with them
+    const long long cus = dev.cus;  // the thresholds below were measured on 256 compute units and scale with them
     // Measured on MI355X over the benchmark configurations and the 12 x {32,128} x {0.3,0.2,0.1} sweep grid:
     // four-wave workgroups win whenever the matrix has enough rows to fill the device (16-wave workgroups were up
     // to 2x slower on long rows: their barrier makes every wave wait for the slowest of sixteen), and rows are
@@ -274,6 +289,10 @@ void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bo
         if (rows_even && R < 4 && avg >= rule.even_rows_avg && ceil_div(M, 4) * col_tiles >= 2 * cus) R = 4;
     }
 }
+
+constexpr int kCutPlanAdviceMaxRows = 16384;     // the cut rule is one workgroup's work: 16 rounds of 1024 rows
+constexpr double kCutPlanMinGainNs = 2500.0;      // SpMM, fused: the kernel that adds the pieces must be paid for
+constexpr double kCutPlanMinGainNsSddmm = 300.0;  // SDDMM: no second kernel
 
 // longest row and number of rows without nonzeros (dlspm_csr_row_stats); stats[0] = max, stats[1] = empty rows
 __global__ void row_stats_kernel(int M, const int* __restrict__ row_offsets, int* __restrict__ stats)
@@ -325,27 +344,27 @@ __global__ void csr_check_kernel(int M, int K, int nnz, const int* __restrict__ 
 }
 
 // the sliced plan of each op, from its lane layout (0 slices: not used)
-static SlicePlan spmm_slice_plan(int M, int K, int N, int nnz, const SpmmShape& s)
+static SlicePlan spmm_slice_plan(const DeviceInfo& dev, int M, int K, int N, int nnz, const SpmmShape& s)
 {
     const int tw = s.G * s.vec * s.V;
     // the column tiles are worked through one after the other: one tile's slab of B is what is gathered from at a time
     // and the workgroups of one (slice, tile) pair should fill the device by themselves, or it gathers from several
     // slabs at once: rows per workgroup as if there were one tile (4096 x 65536, N = 3136, 25 tiles of 128, 131 or
     // 656 nonzeros per row: 856 -> 716 us and 2320 -> 2133 us)
-    SlicePlan p = slice_plan(M, K, N < tw ? N : tw, nnz, 1, 0, s.vec == 4 ? s.G : 0, true, kWave / s.G, 8);
+    SlicePlan p = slice_plan(dev, M, K, N < tw ? N : tw, nnz, 1, 0, s.vec == 4 ? s.G : 0, true, kWave / s.G, 8);
     p.bytes = p.slices > 0 ? p.bounds_bytes + (size_t)p.slices * M * (size_t)N * sizeof(float) : 0;
     return p;
 }
-static SlicePlan fused_slice_plan(int M, int K, int D, int nnz, const FusedShape& s)
+static SlicePlan fused_slice_plan(const DeviceInfo& dev, int M, int K, int D, int nnz, const FusedShape& s)
 {
     const int tw = s.G * s.vec * s.V;
     const bool built = s.vec == 4 && s.G1 == 8 && s.DS > 0 && tw >= D;  // the widths the sliced kernels are built for (17 .. 512)
-    return slice_plan(M, K, D, nnz, 2, D, built ? s.G : 0, true, kWave / s.G, 2);
+    return slice_plan(dev, M, K, D, nnz, 2, D, built ? s.G : 0, true, kWave / s.G, 2);
 }
-static SlicePlan sddmm_slice_plan(int M, int K, int D, int nnz, const SddmmShape& s)
+static SlicePlan sddmm_slice_plan(const DeviceInfo& dev, int M, int K, int D, int nnz, const SddmmShape& s)
 {
     const bool built = s.vec == 4 && s.G1 == 8 && s.DS >= 1;  // 16 < D <= 512
-    return slice_plan(M, K, D, nnz, 1, 0, built ? kWave : 0, false, kWave / s.G1, 2);
+    return slice_plan(dev, M, K, D, nnz, 1, 0, built ? kWave : 0, false, kWave / s.G1, 2);
 }
 
 }  // namespace dlspm
@@ -359,7 +378,7 @@ void dlspm_tuning_default(dlspm_tuning* t)
     if (!t) return;
     const Tuning d;
     *t = dlspm_tuning{d.split_w, d.split_r, d.flat, d.flat_chunk, d.slices, d.tile_major, d.tile_width, d.plan_order,
-                      d.xcd_contiguous, d.stream_results};
+                      d.xcd_contiguous, d.stream_results, d.cut_piece_pct, d.cut_longest_pct};
 }
 
 int dlspm_set_tuning(const dlspm_tuning* t)
@@ -370,7 +389,9 @@ int dlspm_set_tuning(const dlspm_tuning* t)
     }
     if (t->split_w < 0 || t->split_r < 0 || t->flat < -1 || t->flat > 1 || t->flat_chunk < 0 || t->slices < -1 ||
         t->tile_major < -1 || t->tile_major > 1 || t->tile_width < 0 || t->plan_order < 0 || t->plan_order > 2 ||
-        t->xcd_contiguous < 0 || t->xcd_contiguous > 1 || t->stream_results < -1 || t->stream_results > 1)
+        t->xcd_contiguous < 0 || t->xcd_contiguous > 1 || t->stream_results < -1 || t->stream_results > 1 ||
+        (t->cut_piece_pct != 0 && (t->cut_piece_pct < 10 || t->cut_piece_pct > 1000)) ||
+        (t->cut_longest_pct != 0 && (t->cut_longest_pct < 10 || t->cut_longest_pct > 1000)))
         return DLSPM_E_INVALID_ARG;
     t_tuning.split_w = t->split_w;
     t_tuning.split_r = t->split_r;
@@ -382,6 +403,8 @@ int dlspm_set_tuning(const dlspm_tuning* t)
     t_tuning.plan_order = t->plan_order;
     t_tuning.xcd_contiguous = t->xcd_contiguous;
     t_tuning.stream_results = t->stream_results;
+    t_tuning.cut_piece_pct = t->cut_piece_pct;
+    t_tuning.cut_longest_pct = t->cut_longest_pct;
     t_tuning_set = true;
     return DLSPM_OK;
 }
@@ -391,7 +414,7 @@ int dlspm_get_tuning(dlspm_tuning* t)
     if (!t) return DLSPM_E_INVALID_ARG;
     const Tuning& c = tuning();
     *t = dlspm_tuning{c.split_w, c.split_r, c.flat, c.flat_chunk, c.slices, c.tile_major, c.tile_width, c.plan_order,
-                      c.xcd_contiguous, c.stream_results};
+                      c.xcd_contiguous, c.stream_results, c.cut_piece_pct, c.cut_longest_pct};
     return DLSPM_OK;
 }
 
@@ -410,29 +433,39 @@ int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int
     if (M < 0 || K < 0 || N < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
     const WorkspaceArg ws = workspace_arg(workspace, workspace_bytes);
+    if (ws.bad_hint) return DLSPM_E_INVALID_ARG;
     if (ws.row_plan && ws.mem && ws.bytes < row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
     if (M == 0 || N == 0) return DLSPM_OK;
     if (!row_offsets || !C) return DLSPM_E_INVALID_ARG;
     if (nnz > 0 && (!col_indices || !values || !B)) return DLSPM_E_INVALID_ARG;
-    if (const int st = require_device()) return st;
+    const DeviceInfo& dev = device_info();
+    if (const int st = require_device(dev)) return st;
     const bool vec4 = N >= 4;  // dwordx4 accesses need only dword alignment
     const SpmmArgs args{M, K, N, nnz, row_offsets, col_indices, values, B, C, ws.banded ? 1 : 0};
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipError_t e;
+    if (ws.cut_plan && ws.mem) {
+        // the memory holds the cut plan of this matrix and room for the partial rows of its pieces
+        const CutPlan cp = cut_plan_layout(M, N, dev.cus);
+        if (cp.bytes == 0 || ws.bytes < cp.bytes) return DLSPM_E_WORKSPACE;
+        SpmmShape shape = spmm_choose(dev, M, K, N, nnz, vec4, false, true);
+        e = spmm_plan_applies(dev, shape, M, N, nnz) ? spmm_pieces_launch(args, shape, cp, ws.mem, st) : spmm_launch(args, shape, st);
+        return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+    }
     if (ws.row_plan && ws.mem) {
         // the memory holds the row plan of this matrix; sizes a planned launch is not built for run as with NULL
-        SpmmShape shape = spmm_choose(M, K, N, nnz, vec4, false, true);
-        e = spmm_plan_applies(shape, M, N, nnz) ? spmm_planned_launch(args, shape, static_cast<const int*>(ws.mem), st)
+        SpmmShape shape = spmm_choose(dev, M, K, N, nnz, vec4, false, true);
+        e = spmm_plan_applies(dev, shape, M, N, nnz) ? spmm_planned_launch(args, shape, static_cast<const int*>(ws.mem), st)
                                                 : spmm_launch(args, shape, st);
         return e == hipSuccess ? DLSPM_OK : fail_hip(e);
     }
     // a banded matrix (DLSPM_HINT_BANDED) runs as row blocks whatever memory came with the call: column slices and
     // the flat schedule are answers to columns spread over all of K and to uneven rows
     const bool memory = !ws.rows_even && !ws.banded && ws.mem != nullptr;
-    const SpmmShape shape = spmm_choose(M, K, N, nnz, vec4, ws.rows_even, !memory, ws.banded);
+    const SpmmShape shape = spmm_choose(dev, M, K, N, nnz, vec4, ws.rows_even, !memory, ws.banded);
     if (memory) {
-        const SlicePlan sliced = spmm_slice_plan(M, K, N, nnz, shape);
-        const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(M, nnz, N, shape.G);
+        const SlicePlan sliced = spmm_slice_plan(dev, M, K, N, nnz, shape);
+        const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(dev, M, nnz, N, shape.G);
         if (ws.bytes < (sliced.slices > 0 ? sliced.bytes : plan.bytes)) return DLSPM_E_WORKSPACE;
         if (sliced.slices > 0)
             e = spmm_sliced_launch(args, shape, sliced, ws.mem, st);
@@ -497,32 +530,79 @@ int spmm_csr_f32_static(int M, int K, int N, int nnz, const int* row_offsets, co
 
 size_t dlspm_row_plan_bytes(int M) { return row_plan_bytes(M); }
 
+static int cut_plan_width(int op, int N_or_D) { return op == DLSPM_OP_SDDMM ? 0 : N_or_D; }
+
+size_t dlspm_row_plan_bytes_for(int op, int M, int N_or_D)
+{
+    const DeviceInfo& dev = device_info();
+    if ((op != DLSPM_OP_SPMM && op != DLSPM_OP_SDDMM && op != DLSPM_OP_FUSED) || N_or_D < 0) return 0;
+    return cut_plan_layout(M, cut_plan_width(op, N_or_D), dev.cus).bytes;
+}
+
+int dlspm_row_plan_build_cut(int M, const int* row_offsets, void* plan, size_t plan_bytes, void* stream)
+{
+    if (M < 0 || M > kCutPlanMaxRows) return DLSPM_E_INVALID_ARG;
+    if (M == 0) return DLSPM_OK;
+    if (!row_offsets || !plan) return DLSPM_E_INVALID_ARG;
+    const DeviceInfo& dev = device_info();
+    if (const int st = require_device(dev)) return st;
+    const CutPlan cp = cut_plan_layout(M, 0, dev.cus);  // what the build writes ends where the partial rows begin
+    if (plan_bytes < cp.bytes) return DLSPM_E_WORKSPACE;
+    const hipError_t e = cut_plan_build_launch(M, row_offsets, cp, plan, tuning().plan_order, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+}
+
 int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_bytes, void* stream)
 {
     if (M < 0) return DLSPM_E_INVALID_ARG;
     if (M == 0) return DLSPM_OK;
     if (!row_offsets || !plan) return DLSPM_E_INVALID_ARG;
     if (plan_bytes < row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
-    if (const int st = require_device()) return st;
+    const DeviceInfo& dev = device_info();
+    if (const int st = require_device(dev)) return st;
     // one bin per compute unit: the first 8 x bins workgroups of a launch start together, eight on each compute unit
-    const hipError_t e = row_plan_build_launch(M, row_offsets, static_cast<int*>(plan), device_info().cus,
+    const hipError_t e = row_plan_build_launch(M, row_offsets, static_cast<int*>(plan), dev.cus,
                                                tuning().plan_order, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }
 
+// Whether cutting the longest rows (a cut plan) is expected to beat the plan over whole rows. The longest row runs on
+// one compute unit, which gathers about 48 bytes per clock (115 bytes per nanosecond at 2.4 GHz) of dense rows; cut, no
+// entry is longer than one and a half shares. What that saves is set against what the cut plan costs: for SpMM and the
+// fused op the second kernel that adds the pieces (about 2 us between two graph nodes), for SDDMM only a grid that is
+// `compute units` entries larger.
+static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int nnz, int max_row_len)
+{
+    if (max_row_len <= 0 || M > kCutPlanAdviceMaxRows) return false;
+    const long long cus = dev.cus;
+    const long long share = std::max<long long>(ceil_div(nnz, cus), 1);
+    const long long longest_whole = (share * kCutLongestPct + 99) / 100;
+    if (max_row_len <= longest_whole) return false;
+    const double bytes_per_nonzero = (op == DLSPM_OP_FUSED ? 2.0 : 1.0) * (double)std::min(width, 512) * sizeof(float);
+    const double saved_ns = (double)(max_row_len - longest_whole) * bytes_per_nonzero / 115.0;
+    return saved_ns >= (op == DLSPM_OP_SDDMM ? kCutPlanMinGainNsSddmm : kCutPlanMinGainNs);
+}
+
+// the longest row at least twenty times the mean: what DLSPM_HINT_ROWS_SKEWED says
+static bool rows_are_skewed(int M, int nnz, int max_row_len)
+{
+    return M > 0 && max_row_len >= 0 && (double)max_row_len * M >= 20.0 * (double)nnz;
+}
+
 int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row_len)
 {
+    const DeviceInfo& dev = device_info();
     if (M <= 0 || K <= 0 || N_or_D <= 0 || nnz <= 0) return 0;
     const bool vec4 = N_or_D >= 4;
     if (op == DLSPM_OP_SPMM) {
-        SpmmShape shape = spmm_choose(M, K, N_or_D, nnz, vec4, false, true);
-        if (!spmm_plan_applies(shape, M, N_or_D, nnz)) return 0;
+        SpmmShape shape = spmm_choose(dev, M, K, N_or_D, nnz, vec4, false, true);
+        if (!spmm_plan_applies(dev, shape, M, N_or_D, nnz)) return 0;
     } else if (op == DLSPM_OP_SDDMM) {
-        SddmmShape shape = sddmm_choose(M, N_or_D, nnz, vec4);
-        if (!sddmm_plan_applies(shape, M, N_or_D, nnz)) return 0;
+        SddmmShape shape = sddmm_choose(dev, M, N_or_D, nnz, vec4);
+        if (!sddmm_plan_applies(dev, shape, M, N_or_D, nnz, rows_are_skewed(M, nnz, max_row_len))) return 0;
     } else if (op == DLSPM_OP_FUSED) {
-        FusedShape shape = fused_choose(M, N_or_D, nnz, vec4);
-        if (!fused_plan_applies(shape, M, N_or_D, nnz)) return 0;
+        FusedShape shape = fused_choose(dev, M, N_or_D, nnz, vec4);
+        if (!fused_plan_applies(dev, shape, M, N_or_D, nnz, rows_are_skewed(M, nnz, max_row_len))) return 0;
     } else {
         return 0;
     }
@@ -539,7 +619,8 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
     // / 424 us)
     int slices = 0;
     (void)dlspm_describe_slices(op, M, K, N_or_D, nnz, &slices, nullptr);
-    return slices >= 3 ? 0 : 1;
+    if (slices >= 3) return 0;
+    return cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len) ? 2 : 1;
 }
 
 // the *_planned entry points: the named call with the plan as its workspace and the hint that says so
@@ -578,11 +659,13 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
     if (M < 0 || K < 0 || D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
     const WorkspaceArg ws = workspace_arg(workspace, workspace_bytes);
+    if (ws.bad_hint) return DLSPM_E_INVALID_ARG;
     if (ws.row_plan && ws.mem && ws.bytes < row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
     if (M == 0 || nnz == 0) return DLSPM_OK;
     if (!row_offsets || !col_indices || !out_values) return DLSPM_E_INVALID_ARG;
     if (D > 0 && (!lhs || !rhs)) return DLSPM_E_INVALID_ARG;
-    if (const int st = require_device()) return st;
+    const DeviceInfo& dev = device_info();
+    if (const int st = require_device(dev)) return st;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (D == 0) {
         const unsigned blocks = (unsigned)ceil_div(nnz, 256);
@@ -591,28 +674,37 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
         return e0 == hipSuccess ? DLSPM_OK : fail_hip(e0);
     }
     const bool vec4 = D >= 4;  // dwordx4 accesses need only dword alignment
-    const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values, ws.banded ? 1 : 0};
+    const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values, ws.banded ? 1 : 0, dev.l2_bytes};
+    if (ws.cut_plan && ws.mem) {
+        const CutPlan cp = cut_plan_layout(M, 0, dev.cus);
+        if (cp.bytes == 0 || ws.bytes < cp.bytes) return DLSPM_E_WORKSPACE;
+        SddmmShape shape = sddmm_choose(dev, M, D, nnz, vec4);
+        if (sddmm_plan_applies(dev, shape, M, D, nnz)) {
+            const hipError_t e = sddmm_pieces_launch(args, shape, cp, ws.mem, st);
+            return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+        }
+    }
     if (ws.row_plan && ws.mem) {
-        SddmmShape shape = sddmm_choose(M, D, nnz, vec4);
-        if (sddmm_plan_applies(shape, M, D, nnz)) {
+        SddmmShape shape = sddmm_choose(dev, M, D, nnz, vec4);
+        if (sddmm_plan_applies(dev, shape, M, D, nnz, ws.skewed)) {
             const hipError_t e = sddmm_planned_launch(args, shape, static_cast<const int*>(ws.mem), st);
             return e == hipSuccess ? DLSPM_OK : fail_hip(e);
         }
         // sizes a planned launch is not built for run as with NULL
     }
-    const SddmmShape shape = sddmm_choose(M, D, nnz, vec4, ws.rows_even);
+    const SddmmShape shape = sddmm_choose(dev, M, D, nnz, vec4, ws.rows_even);
     // the flat schedule needs no workspace here (nothing to combine), so the size rule alone decides; it has no
     // width condition for SDDMM (measured for D = 32 ... 256: equal on uniform rows, 15-33 % faster on skewed ones)
-    if (ws.mem && !ws.rows_even && !ws.row_plan && !ws.banded) {
+    if (ws.mem && !ws.rows_even && !ws.row_plan && !ws.cut_plan && !ws.banded) {
         // with a workspace for the slice boundaries: the column-sliced schedule where the rhs operand exceeds one L2
-        const SlicePlan sliced = sddmm_slice_plan(M, K, D, nnz, shape);
+        const SlicePlan sliced = sddmm_slice_plan(dev, M, K, D, nnz, shape);
         if (ws.bytes < sliced.bytes) return DLSPM_E_WORKSPACE;
         if (sliced.slices > 0) {
             const hipError_t es = sddmm_sliced_launch(args, shape, sliced, ws.mem, st);
             return es == hipSuccess ? DLSPM_OK : fail_hip(es);
         }
     }
-    const FlatPlan plan = ws.banded ? FlatPlan{0, 0, 0} : sddmm_flat_plan(M, nnz, D);
+    const FlatPlan plan = ws.banded ? FlatPlan{0, 0, 0} : sddmm_flat_plan(dev, M, nnz, D);
     const hipError_t e = plan.chunk > 0 ? sddmm_flat_launch(args, shape, plan.chunk, st) : sddmm_launch(args, shape, st);
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }
@@ -624,25 +716,34 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz, const int* row_offsets, c
     if (M < 0 || K < 0 || D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_ARG;
     const WorkspaceArg ws = workspace_arg(workspace, workspace_bytes);
+    if (ws.bad_hint) return DLSPM_E_INVALID_ARG;
     if (ws.row_plan && ws.mem && ws.bytes < row_plan_bytes(M)) return DLSPM_E_WORKSPACE;
     if (M == 0 || D == 0) return DLSPM_OK;
     if (!row_offsets || !O) return DLSPM_E_INVALID_ARG;
     if (nnz > 0 && (!col_indices || !Q || !Kmat || !V)) return DLSPM_E_INVALID_ARG;
-    if (const int st = require_device()) return st;
+    const DeviceInfo& dev = device_info();
+    if (const int st = require_device(dev)) return st;
     const bool vec4 = D >= 4;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const FusedArgs args{M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O, ws.banded ? 1 : 0};
     hipError_t e;
+    if (ws.cut_plan && ws.mem) {
+        const CutPlan cp = cut_plan_layout(M, D, dev.cus);
+        if (cp.bytes == 0 || ws.bytes < cp.bytes) return DLSPM_E_WORKSPACE;
+        FusedShape shape = fused_choose(dev, M, D, nnz, vec4);
+        e = fused_plan_applies(dev, shape, M, D, nnz) ? fused_pieces_launch(args, shape, cp, ws.mem, st) : fused_launch(args, shape, st);
+        return e == hipSuccess ? DLSPM_OK : fail_hip(e);
+    }
     if (ws.row_plan && ws.mem) {
-        FusedShape shape = fused_choose(M, D, nnz, vec4);
-        e = fused_plan_applies(shape, M, D, nnz) ? fused_planned_launch(args, shape, static_cast<const int*>(ws.mem), st)
+        FusedShape shape = fused_choose(dev, M, D, nnz, vec4);
+        e = fused_plan_applies(dev, shape, M, D, nnz, ws.skewed) ? fused_planned_launch(args, shape, static_cast<const int*>(ws.mem), st)
                                                  : fused_launch(args, shape, st);
         return e == hipSuccess ? DLSPM_OK : fail_hip(e);
     }
-    const FusedShape shape = fused_choose(M, D, nnz, vec4, ws.rows_even);
+    const FusedShape shape = fused_choose(dev, M, D, nnz, vec4, ws.rows_even);
     if (!ws.rows_even && !ws.banded && ws.mem) {
-        const SlicePlan sliced = fused_slice_plan(M, K, D, nnz, shape);
-        const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(M, nnz, D, shape.G);
+        const SlicePlan sliced = fused_slice_plan(dev, M, K, D, nnz, shape);
+        const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(dev, M, nnz, D, shape.G);
         if (ws.bytes < (sliced.slices > 0 ? sliced.bytes : plan.bytes)) return DLSPM_E_WORKSPACE;
         if (sliced.slices > 0)
             e = fused_sliced_launch(args, shape, sliced, ws.mem, st);
@@ -658,23 +759,24 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz, const int* row_offsets, c
 
 size_t dlspm_workspace_bytes(int op, int M, int K, int N_or_D, int nnz)
 {
+    const DeviceInfo& dev = device_info();
     // The workgroup-per-row-block schedule splits the work from row_offsets alone and keeps partial sums in LDS: no
     // scratch. Where flat_plan's rule selects the flat schedule for SpMM or the fused op, its partial rows live in the
     // workspace; a call without workspace runs the row-block schedule instead.
     if (M <= 0 || N_or_D <= 0 || nnz <= 0) return 0;
     if (op == DLSPM_OP_SPMM) {
-        const SpmmShape s = spmm_choose(M, K, N_or_D, nnz, N_or_D >= 4, false, false);  // a call with memory
-        const SlicePlan sliced = spmm_slice_plan(M, K, N_or_D, nnz, s);
-        return sliced.slices > 0 ? sliced.bytes : flat_plan(M, nnz, N_or_D, s.G).bytes;
+        const SpmmShape s = spmm_choose(dev, M, K, N_or_D, nnz, N_or_D >= 4, false, false);  // a call with memory
+        const SlicePlan sliced = spmm_slice_plan(dev, M, K, N_or_D, nnz, s);
+        return sliced.slices > 0 ? sliced.bytes : flat_plan(dev, M, nnz, N_or_D, s.G).bytes;
     }
     if (op == DLSPM_OP_FUSED) {
-        const FusedShape s = fused_choose(M, N_or_D, nnz, N_or_D >= 4);
-        const SlicePlan sliced = fused_slice_plan(M, K, N_or_D, nnz, s);
-        return sliced.slices > 0 ? sliced.bytes : flat_plan(M, nnz, N_or_D, s.G).bytes;
+        const FusedShape s = fused_choose(dev, M, N_or_D, nnz, N_or_D >= 4);
+        const SlicePlan sliced = fused_slice_plan(dev, M, K, N_or_D, nnz, s);
+        return sliced.slices > 0 ? sliced.bytes : flat_plan(dev, M, nnz, N_or_D, s.G).bytes;
     }
     if (op == DLSPM_OP_SDDMM) {  // every result goes into its own CSR slot: only the slice boundaries need memory
-        const SddmmShape s = sddmm_choose(M, N_or_D, nnz, N_or_D >= 4);
-        return sddmm_slice_plan(M, K, N_or_D, nnz, s).bytes;
+        const SddmmShape s = sddmm_choose(dev, M, N_or_D, nnz, N_or_D >= 4);
+        return sddmm_slice_plan(dev, M, K, N_or_D, nnz, s).bytes;
     }
     return 0;
 }
@@ -685,7 +787,8 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
     if ((long long)nnz > (long long)M * K) return DLSPM_E_INVALID_CSR;
     if (!row_offsets) return DLSPM_E_INVALID_ARG;
     if (nnz > 0 && !col_indices) return DLSPM_E_INVALID_ARG;
-    if (const int st = require_device()) return st;
+    const DeviceInfo& dev = device_info();
+    if (const int st = require_device(dev)) return st;
     hipStream_t s = static_cast<hipStream_t>(stream);
     int* d_flags = nullptr;
     hipError_t e = hipMalloc(&d_flags, sizeof(int));
@@ -711,7 +814,8 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
     if (M < 0 || (M > 0 && !row_offsets)) return DLSPM_E_INVALID_ARG;
     int h[2] = {0, 0};
     if (M > 0) {
-        if (const int st = require_device()) return st;
+        const DeviceInfo& dev = device_info();
+    if (const int st = require_device(dev)) return st;
         hipStream_t s = static_cast<hipStream_t>(stream);
         int* d = nullptr;
         hipError_t e = hipMalloc(&d, 2 * sizeof(int));
@@ -734,6 +838,7 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
 
 int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int passing, int* shape)
 {
+    const DeviceInfo& dev = device_info();
     if (passing != DLSPM_PASS_NULL && passing != DLSPM_PASS_ROWS_EVEN && passing != DLSPM_PASS_WORKSPACE)
         return DLSPM_E_INVALID_ARG;
     const bool even = passing == DLSPM_PASS_ROWS_EVEN;
@@ -743,22 +848,22 @@ int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int pa
     const bool vec4 = n >= 4;
     for (int i = 0; i < 10; ++i) shape[i] = 0;
     if (op == DLSPM_OP_SPMM) {
-        const SpmmShape s = spmm_choose(M, K, n, nnz, vec4, even, !memory);
+        const SpmmShape s = spmm_choose(dev, M, K, n, nnz, vec4, even, !memory);
         const int tw = s.G * s.vec * s.V;
         shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[5] = s.W; shape[6] = s.R; shape[7] = (int)ceil_div(n, tw);
-        const FlatPlan fp = flat_plan(M, nnz, n, s.G);
+        const FlatPlan fp = flat_plan(dev, M, nnz, n, s.G);
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_SDDMM) {
-        const SddmmShape s = sddmm_choose(M, n, nnz, vec4, even);
+        const SddmmShape s = sddmm_choose(dev, M, n, nnz, vec4, even);
         shape[0] = s.vec; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R; shape[7] = 1;
-        const FlatPlan fp = sddmm_flat_plan(M, nnz, n);
+        const FlatPlan fp = sddmm_flat_plan(dev, M, nnz, n);
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_FUSED) {
-        const FusedShape s = fused_choose(M, n, nnz, vec4, even);
+        const FusedShape s = fused_choose(dev, M, n, nnz, vec4, even);
         const int tw = s.G * s.vec * s.V;
         shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R;
         shape[7] = (int)ceil_div(n, tw);
-        const FlatPlan fp = flat_plan(M, nnz, n, s.G);
+        const FlatPlan fp = flat_plan(dev, M, nnz, n, s.G);
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else {
         return DLSPM_E_INVALID_ARG;
@@ -773,6 +878,7 @@ int dlspm_describe_launch(int op, int M, int K, int N_or_D, int nnz, int* shape)
 
 int dlspm_workspace_advice(int op, int M, int K, int N_or_D, int nnz, int max_row_len)
 {
+    const DeviceInfo& dev = device_info();
     if (M <= 0 || K <= 0 || N_or_D <= 0 || nnz <= 0) return DLSPM_PASS_NULL;
     if (op != DLSPM_OP_SPMM && op != DLSPM_OP_SDDMM && op != DLSPM_OP_FUSED) return DLSPM_PASS_NULL;
     int slices = 0;
@@ -789,8 +895,8 @@ int dlspm_workspace_advice(int op, int M, int K, int N_or_D, int nnz, int max_ro
     // 32768 x 32768, N = 256: 228 against 282 us at 128; 16384 x 32768, N = 1024: 418 against 459 us at 70,
     // 788 against 590 us at 140)
     if (sliced && op == DLSPM_OP_SPMM && mean < 128.0) {
-        const SpmmShape without = spmm_choose(M, K, N_or_D, nnz, N_or_D >= 4, false, true);
-        const SpmmShape with = spmm_choose(M, K, N_or_D, nnz, N_or_D >= 4, false, false);
+        const SpmmShape without = spmm_choose(dev, M, K, N_or_D, nnz, N_or_D >= 4, false, true);
+        const SpmmShape with = spmm_choose(dev, M, K, N_or_D, nnz, N_or_D >= 4, false, false);
         if (without.tile_major && without.G * without.V < with.G * with.V) sliced = false;
     }
     if (sliced || (uneven && want > 0 && slices == 0)) return DLSPM_PASS_WORKSPACE;
@@ -799,11 +905,12 @@ int dlspm_workspace_advice(int op, int M, int K, int N_or_D, int nnz, int max_ro
 
 int dlspm_describe_slices(int op, int M, int K, int N_or_D, int nnz, int* slices, int* rows_per_workgroup)
 {
+    const DeviceInfo& dev = device_info();
     if (M < 0 || K < 0 || N_or_D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     SlicePlan p{0, 1, 0, 0};
-    if (op == DLSPM_OP_SPMM) p = spmm_slice_plan(M, K, N_or_D, nnz, spmm_choose(M, K, N_or_D, nnz, N_or_D >= 4, false, false));
-    else if (op == DLSPM_OP_FUSED) p = fused_slice_plan(M, K, N_or_D, nnz, fused_choose(M, N_or_D, nnz, N_or_D >= 4));
-    else if (op == DLSPM_OP_SDDMM) p = sddmm_slice_plan(M, K, N_or_D, nnz, sddmm_choose(M, N_or_D, nnz, N_or_D >= 4));
+    if (op == DLSPM_OP_SPMM) p = spmm_slice_plan(dev, M, K, N_or_D, nnz, spmm_choose(dev, M, K, N_or_D, nnz, N_or_D >= 4, false, false));
+    else if (op == DLSPM_OP_FUSED) p = fused_slice_plan(dev, M, K, N_or_D, nnz, fused_choose(dev, M, N_or_D, nnz, N_or_D >= 4));
+    else if (op == DLSPM_OP_SDDMM) p = sddmm_slice_plan(dev, M, K, N_or_D, nnz, sddmm_choose(dev, M, N_or_D, nnz, N_or_D >= 4));
     else return DLSPM_E_INVALID_ARG;
     if (slices) *slices = p.slices;
     if (rows_per_workgroup) *rows_per_workgroup = p.R;

@@ -46,9 +46,13 @@ template <> struct Vec<4> {
         if (streaming) {
             typedef float f4 __attribute__((ext_vector_type(4)));
             const f4 t = {v.x, v.y, v.z, v.w};
-            // s_nop: a store of more than 8 bytes reads its data one wait state after it issues, and the compiler does
-            // not know that this is one, so the next instruction might overwrite the registers of t
-            asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 0" : : "v"(p), "v"(t) : "memory");
+            // s_nop 1: on the gfx940 family a vector-memory store of more than 8 bytes still reads its data registers for
+            // two wait states after it issues, and a VALU write of those registers must not come earlier (the "VMEM store
+            // of more than 64 bits, then a write of the VGPRs holding its data" row of the ISA guide's table of wait
+            // states the program must insert; the compiler keeps two independent instructions or `s_nop 1` there for its
+            // own dwordx4 stores). It cannot see that this asm is such a store, so the two wait states are spent here,
+            // whatever it schedules behind. (The dword store below reads its data as it issues and needs none.)
+            asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(p), "v"(t) : "memory");
         } else {
             gstore(p);
         }
@@ -253,12 +257,19 @@ __host__ __device__ __forceinline__ void wave_range(bool aligned, Off&& off, int
 //                   back to where it lies in memory.
 //   PLANNED (with SLICED and R == 1): workgroup i works on row row_ids[i], whose nonzeros are
 //                   [row_offsets[i], row_ends[i]): a row plan hands the rows out in an order of its own.
+//                   kPlanPieces: the entry may be a PIECE of a row (a row longer than one compute unit's share of the
+//                   nonzeros is cut into several entries): row_slots[i] is -1 for a whole row, s >= 0 for a piece whose
+//                   partial row goes to slot s of a buffer of partial rows (a second kernel adds the pieces of a row
+//                   in order), and below -1 for an entry that holds nothing (the plan has room for the most pieces
+//                   any matrix of its height can need).
 // The R + 1 offsets are read without LDS or a barrier: with R == 1 they are the same two words for every lane (scalar
 // loads); otherwise lane i of every wave holds offset i and v_readlane picks one.
-template <int W, int R, bool SLICED, bool PLANNED>
+constexpr int kPlanNone = 0, kPlanRows = 1, kPlanPieces = 2;
+template <int W, int R, bool SLICED, int PLANNED>
 struct RowBlock {
     static_assert(!PLANNED || (SLICED && R == 1), "a row plan names one row per workgroup");
     int lane, w;
+    int piece = -1;  // kPlanPieces: the entry's slot among the partial rows, -1 a whole row, below -1 nothing
     int rows_total;  // rows of the matrix
     int stream_rule;  // results with the non-temporal hint: 0 by the size rule, 1 never, 2 always (launch flags, bits 1-2)
     int nr;    // rows in this block (fewer than R at the end of the matrix)
@@ -274,7 +285,8 @@ struct RowBlock {
     template <typename Prefetch>
     __device__ __forceinline__ void load(int rb, int M, int nnz, const int* __restrict__ row_offsets,
                                          const int* __restrict__ row_ends, const int* __restrict__ row_ids,
-                                         Prefetch&& prefetch, int flags = 0)
+                                         Prefetch&& prefetch, int flags = 0, const int* __restrict__ row_slots = nullptr,
+                                         int slots = 0)
     {
         lane = threadIdx.x & 63;
         w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -307,6 +319,7 @@ struct RowBlock {
                     row0 = min(max(row_ids[r0], 0), M - 1);
                     start_lo = min(max(start_lo, 0), nnz);
                     off_hi = min(max(off_hi, 0), nnz - start_lo);
+                    if constexpr (PLANNED == kPlanPieces) piece = min(row_slots[r0], slots - 1);
                 }
             } else {
                 static_assert(R + 1 <= 32, "the running sum covers 32 lanes");
@@ -366,10 +379,16 @@ struct RowBlock {
 // wave are stored straight to `out` (row blk.row0 + r, `width` floats per row); rows shared by several waves leave
 // per-wave partial sums in LDS which are added in wave order after one barrier, so the result does not depend on
 // timing (no atomics, no pre-zeroed output); rows without nonzeros are written as zeros.
-template <int VEC, int G, int V, int W, int R, bool SLICED, bool PLANNED, typename Segment>
+// kPlanPieces: an entry that is a piece of a row stores its sum to `pieces` (slot blk.piece) instead, with ordinary stores
+// (it is read again), and an entry that holds nothing leaves at once (the whole workgroup, before any barrier).
+template <int VEC, int G, int V, int W, int R, bool SLICED, int PLANNED, typename Segment>
 __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PLANNED>& blk, int ct, int width,
-                                                 float* __restrict__ out, Segment&& segment)
+                                                 float* __restrict__ out, Segment&& segment,
+                                                 float* __restrict__ pieces = nullptr)
 {
+    if constexpr (PLANNED == kPlanPieces) {
+        if (blk.piece < -1) return;
+    }
     constexpr int TW = G * VEC * V;  // columns covered by one wave
     constexpr int NP = R == 1 ? 1 : 2;  // with one row per workgroup a wave never ends a second segment
     using VecT = Vec<VEC>;
@@ -400,8 +419,15 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
     constexpr long long kStreamedOutputFloats = 1024 * 1024;
     const long long out_floats = (long long)blk.rows_total * width;
     // (dlspm_tuning.stream_results switches the rule off or on for sweeps and tests: blk.stream_rule)
-    const bool streaming = (!SLICED || PLANNED) && blk.stream_rule != 1 &&
+    const bool streaming = (!SLICED || PLANNED) && blk.stream_rule != 1 && (PLANNED != kPlanPieces || blk.piece < 0) &&
                            (blk.stream_rule == 2 || out_floats >= kStreamedOutputFloats);
+    // where row r of the block is stored
+    auto out_row = [&](int r) -> float* {
+        if constexpr (PLANNED == kPlanPieces) {
+            if (blk.piece >= 0) return pieces + (size_t)blk.piece * width;
+        }
+        return out + (size_t)(blk.row0 + r) * width;
+    };
 
     blk.for_each_segment([&](int r, int p, int q, int rs, int re) {
         VecT acc[V];
@@ -410,7 +436,7 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
         const bool whole_row = (p == rs) && (q == re);
         if (slot == 0) {
             if (whole_row) {
-                float* orow = out + (size_t)(blk.row0 + r) * width;
+                float* orow = out_row(r);
 #pragma unroll
                 for (int v = 0; v < V; ++v)
                     if (act[v]) acc[v].gstore(orow + colv[v], streaming);
@@ -462,7 +488,7 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
         // one row per workgroup: wave x had nonzeros iff x * per < T, and wave 0 adds them up (no division, the
         // partial sums of all waves are requested from LDS together)
         if (w == 0 && slot == 0) {
-            float* orow = out + (size_t)blk.row0 * width;
+            float* orow = out_row(0);
             if (T == 0) {
 #pragma unroll
                 for (int v = 0; v < V; ++v)

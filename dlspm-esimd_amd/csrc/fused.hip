@@ -57,24 +57,28 @@ __device__ __forceinline__ void fused_segment(Vec<VEC>* acc, int p, int q, int D
 // The work of workgroup `bid` (RowBlock in common.hpp explains SLICED and PLANNED: with PLANNED workgroup i works on row
 // row_ids[i] of Q, O and the mask). Column tiles (D > 1024) tile-major, as in spmm_block; no division in the usual
 // case of one tile.
-template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R, bool SLICED, bool PLANNED = false>
+template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R, bool SLICED, int PLANNED = kPlanNone>
 __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles, float scale,
                                             const int* __restrict__ row_offsets, const int* __restrict__ row_ends,
                                             const int* __restrict__ col_indices, const float* __restrict__ Q,
                                             const float* __restrict__ Kmat, const float* __restrict__ Vmat,
                                             float* __restrict__ O, const int* __restrict__ row_ids = nullptr, int nnz = 0,
-                                            int flags = 0)
+                                            int flags = 0, const int* __restrict__ row_slots = nullptr,
+                                            float* __restrict__ pieces = nullptr, int slots = 0)
 {
-    const int row_blocks = (M - 1) / R + 1;
+    const int row_blocks = (M - 1) / R + 1;  // (planned launches have one column tile)
     const int ct = col_tiles == 1 ? 0 : bid / row_blocks;
     const int rb = bid - ct * row_blocks;
     RowBlock<W, R, SLICED, PLANNED> blk;
     blk.load(rb, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, Q, Kmat, Vmat, O); },
-             col_tiles == 1 ? flags : flags & ~1);
-    dense_rows_block<VEC, G, V2>(blk, ct, D, O, [&](Vec<VEC>* acc, int r, int p, int q, const int* colv) {
-        const float* q_row = Q + (size_t)(blk.row0 + r) * D;
-        fused_segment<VEC, G1, DS, MASKED, G, V2>(acc, p, q, D, scale, col_indices, q_row, Kmat, Vmat, colv, blk.lane);
-    });
+             col_tiles == 1 ? flags : flags & ~1, row_slots, slots);
+    dense_rows_block<VEC, G, V2>(
+        blk, ct, D, O,
+        [&](Vec<VEC>* acc, int r, int p, int q, const int* colv) {
+            const float* q_row = Q + (size_t)(blk.row0 + r) * D;
+            fused_segment<VEC, G1, DS, MASKED, G, V2>(acc, p, q, D, scale, col_indices, q_row, Kmat, Vmat, colv, blk.lane);
+        },
+        pieces);
 }
 
 // MASKED = false: D == G1 * VEC * DS exactly, every stage-1 access of every lane falls inside the row.
@@ -117,8 +121,23 @@ __global__ __launch_bounds__(4 * 64) void fused_planned_kernel(int M, int D, int
                                                                const float* __restrict__ Q, const float* __restrict__ Kmat,
                                                                const float* __restrict__ Vmat, float* __restrict__ O)
 {
-    fused_block<VEC, G1, DS, MASKED, G, V2, 4, 1, true, true>((int)blockIdx.x, M, D, 1, scale, starts, ends, col_indices, Q,
-                                                              Kmat, Vmat, O, rows, nnz, flags);
+    fused_block<VEC, G1, DS, MASKED, G, V2, 4, 1, true, kPlanRows>((int)blockIdx.x, M, D, 1, scale, starts, ends, col_indices,
+                                                                   Q, Kmat, Vmat, O, rows, nnz, flags);
+}
+
+// Row plan with cut rows (see spmm_pieces_kernel): entry i is the whole row rows[i], a piece of it whose partial row of O
+// goes to pieces[slot_of[i]], or nothing.
+template <int VEC, int G1, int DS, bool MASKED, int G, int V2>
+__global__ __launch_bounds__(4 * 64) void fused_pieces_kernel(int M, int D, int nnz, int flags, int slots, float scale,
+                                                              const int* __restrict__ starts, const int* __restrict__ ends,
+                                                              const int* __restrict__ rows, const int* __restrict__ slot_of,
+                                                              const int* __restrict__ col_indices,
+                                                              const float* __restrict__ Q, const float* __restrict__ Kmat,
+                                                              const float* __restrict__ Vmat, float* __restrict__ O,
+                                                              float* __restrict__ pieces)
+{
+    fused_block<VEC, G1, DS, MASKED, G, V2, 4, 1, true, kPlanPieces>((int)blockIdx.x, M, D, 1, scale, starts, ends, col_indices,
+                                                                     Q, Kmat, Vmat, O, rows, nnz, flags, slot_of, pieces, slots);
 }
 
 // ---- host side --------------------------------------------------------------------------------------
@@ -165,7 +184,7 @@ static hipError_t launch_wr(const FusedArgs& x, int W, int R, hipStream_t stream
     return hipErrorInvalidValue;
 }
 
-FusedShape fused_choose(int M, int D, int nnz, bool vec4, bool rows_even)
+FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even)
 {
     FusedShape s{};
     s.vec = vec4 ? 4 : 1;
@@ -185,7 +204,7 @@ FusedShape fused_choose(int M, int D, int nnz, bool vec4, bool rows_even)
     // rows per workgroup 1 / 2 / 4 / 8 / 16: 1024 rows 3.3 / 4.4 / 5.5 / 6.9 / 10.9 us; 2048 rows 4.8 / 4.9 / 6.1 / 7.8 /
     // 11.7 us; 4096 rows 7.3 / 7.2 / 6.5 / 8.0 / 11.6 us; 8192 rows 12.1 / 10.4 / 8.3 / 7.2 / 9.2 us; 16384 rows: sixteen;
     // 3072 rows of 102, even: two per workgroup 8.5 us, four 7.2 us)
-    choose_split(M, ceil_div(D, tw), nnz, SplitRule{3, tw >= 1024 ? 4 : 16, kWave / s.G, false, 96}, rows_even, s.W, s.R);
+    choose_split(dev, M, ceil_div(D, tw), nnz, SplitRule{3, tw >= 1024 ? 4 : 16, kWave / s.G, false, 96}, rows_even, s.W, s.R);
     return s;
 }
 
@@ -375,12 +394,12 @@ hipError_t fused_sliced_launch(const FusedArgs& x, const FusedShape& s, const Sl
 
 // ---- row plan ---------------------------------------------------------------------------------------
 
-bool fused_plan_applies(FusedShape& s, int M, int D, int nnz)
+bool fused_plan_applies(const DeviceInfo& dev, FusedShape& s, int M, int D, int nnz, bool skewed)
 {
     // built for 16 < D <= 512 (the shapes of the column-sliced kernels): one column tile
     if (s.vec != 4 || s.G1 != 8 || s.DS < 1 || s.W != 4 || s.G * s.vec * s.V < D) return false;
     if (s.R == 1) return true;
-    if (!plan_ungroups_dots(M, D, nnz)) return false;
+    if (!plan_ungroups_dots(dev, M, D, nnz) && !(skewed && plan_ungroups_skewed(dev, M, nnz))) return false;
     s.R = 1;
     return true;
 }
@@ -396,6 +415,37 @@ static hipError_t launch_planned(const FusedArgs& x, const int* plan, hipStream_
         hipLaunchKernelGGL((fused_planned_kernel<4, 8, DS, true, G, V2>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M,
                            x.D, x.nnz, launch_flags(0), x.scale, starts, ends, rows, x.col_indices, x.Q, x.Kmat, x.V, x.O);
     return hipGetLastError();
+}
+
+template <int DS, int G, int V2>
+static hipError_t launch_pieces(const FusedArgs& x, const CutPlan& cp, void* plan, hipStream_t stream)
+{
+    const int* base = static_cast<const int*>(plan);
+    const int *starts = base, *ends = base + cp.entries, *rows = base + 2 * (size_t)cp.entries,
+              *slot_of = base + 3 * (size_t)cp.entries;
+    float* pieces = reinterpret_cast<float*>(static_cast<char*>(plan) + cp.off_pieces);
+    if (x.D == 8 * 4 * DS)
+        hipLaunchKernelGGL((fused_pieces_kernel<4, 8, DS, false, G, V2>), dim3((unsigned)cp.entries), dim3(4 * 64), 0, stream,
+                           x.M, x.D, x.nnz, launch_flags(0), cp.slots, x.scale, starts, ends, rows, slot_of, x.col_indices, x.Q,
+                           x.Kmat, x.V, x.O, pieces);
+    else
+        hipLaunchKernelGGL((fused_pieces_kernel<4, 8, DS, true, G, V2>), dim3((unsigned)cp.entries), dim3(4 * 64), 0, stream,
+                           x.M, x.D, x.nnz, launch_flags(0), cp.slots, x.scale, starts, ends, rows, slot_of, x.col_indices, x.Q,
+                           x.Kmat, x.V, x.O, pieces);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return cut_rows_sum_launch(x.M, x.D, cp, plan, x.O, stream);
+}
+
+hipError_t fused_pieces_launch(const FusedArgs& x, const FusedShape& s, const CutPlan& cp, void* plan, hipStream_t stream)
+{
+    if (x.M <= 0) return hipSuccess;
+    if (s.DS == 1 && s.G == 8 && s.V == 1) return launch_pieces<1, 8, 1>(x, cp, plan, stream);
+    if (s.DS == 2 && s.G == 16 && s.V == 1) return launch_pieces<2, 16, 1>(x, cp, plan, stream);
+    if (s.DS == 4 && s.G == 32 && s.V == 1) return launch_pieces<4, 32, 1>(x, cp, plan, stream);
+    if (s.DS == 8 && s.G == 64 && s.V == 1) return launch_pieces<8, 64, 1>(x, cp, plan, stream);
+    if (s.DS == 16 && s.G == 64 && s.V == 2) return launch_pieces<16, 64, 2>(x, cp, plan, stream);
+    return hipErrorInvalidValue;
 }
 
 hipError_t fused_planned_launch(const FusedArgs& x, const FusedShape& s, const int* plan, hipStream_t stream)

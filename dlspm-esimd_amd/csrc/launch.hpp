@@ -15,6 +15,9 @@ inline bool dense_fits_buffer(long long rows, long long width)
     return rows * width * 4 < (1ll << 32) && rows < (1 << 24) && width * 4 < (1 << 24);
 }
 
+// DLSPM_E_LAUNCH, after noting e as the calling thread's last HIP error (dlspm_last_hip_error)
+int fail_hip(hipError_t e);
+
 // The device the calling thread has current, as far as the launch rules need it: compute units and the size of one
 // L2. Read from hipDeviceProp_t once per device and cached; without a device (host-only queries on a machine that has
 // none) the figures of a whole MI355X: 256 compute units, 4 MiB.
@@ -24,7 +27,7 @@ struct DeviceInfo {
     bool present;  // a HIP device is current
     bool gfx950;   // ... and it is the architecture the kernels are built for
 };
-const DeviceInfo& device_info();
+const DeviceInfo& device_info();  // one look-up per entry-point call; everything below takes the result as `dev`
 
 // Overrides of the launch rules for tuning sweeps and tests (dlspm_set_tuning; one set per host thread, initialised from
 // the environment once per process). The fields and their "follow the rule" values are those of dlspm_tuning.
@@ -36,6 +39,7 @@ struct Tuning {
     int plan_order = 0;
     int xcd_contiguous = 0;
     int stream_results = -1;
+    int cut_piece_pct = 0, cut_longest_pct = 0;
 };
 const Tuning& tuning();
 
@@ -77,6 +81,7 @@ struct SddmmArgs {
     const float* rhs;
     float* out;
     int xcd_contiguous = 0;
+    long long l2_bytes = 4ll << 20;  // of the device the call runs on (DeviceInfo::l2_bytes): results beyond it are streamed
 };
 struct FusedArgs {
     int M, K, D, nnz;
@@ -99,7 +104,7 @@ struct FlatPlan {
     int units;
     size_t bytes;
 };
-FlatPlan flat_plan(int M, int nnz, int width, int G);
+FlatPlan flat_plan(const DeviceInfo& dev, int M, int nnz, int width, int G);
 hipError_t row_fixup_launch(int M, int N, int chunk, const int* row_offsets, const float* partial, float* out,
                             hipStream_t stream);
 
@@ -116,35 +121,35 @@ struct SlicePlan {
 // `operands`: dense operands gathered per nonzero (1 SpMM and SDDMM, 2 fused); `partial_width`: floats of a partial
 // row that `bytes` accounts for (0: SDDMM has none, SpMM adds its own); `partial_rows`: the op writes partial rows at
 // all (its slices are then a third larger); G, slots: the op's lane layout
-SlicePlan slice_plan(int M, int K, int width, int nnz, int operands, int partial_width, int G, bool partial_rows,
+SlicePlan slice_plan(const DeviceInfo& dev, int M, int K, int width, int nnz, int operands, int partial_width, int G, bool partial_rows,
                      int slots, int blocks_per_cu);
 hipError_t slice_bounds_launch(int M, int K, int slices, const int* row_offsets, const int* col_indices, int* bounds,
                                hipStream_t stream);
 hipError_t slice_sum_launch(long long count, int slices, const float* partial, float* out, hipStream_t stream);
 
 // narrow_tiles: the call passes no workspace memory (column tiles below 128 columns are then allowed)
-SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles, bool banded = false);
+SpmmShape spmm_choose(const DeviceInfo& dev, int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles, bool banded = false);
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
 // Row plan (3 x M ints on the device: first nonzero, end and row number of the row that workgroup i works on): only for
 // shapes of one row per four-wave workgroup and one column tile
 hipError_t row_plan_build_launch(int M, const int* row_offsets, int* plan, int bins, int order, hipStream_t stream);
 size_t row_plan_bytes(int M);
-bool plan_ungroups(int M, int width, int nnz);  // SpMM: rows long enough that a plan runs them one per workgroup against the size rule
-bool plan_ungroups_dots(int M, int D, int nnz);  // the same for SDDMM and the fused op
-bool spmm_plan_applies(SpmmShape& s, int M, int N, int nnz);  // true: s is the shape of the planned launch (R = 1)
+bool plan_ungroups(const DeviceInfo& dev, int M, int width, int nnz);  // SpMM: rows long enough that a plan runs them one per workgroup against the size rule
+bool plan_ungroups_dots(const DeviceInfo& dev, int M, int D, int nnz);  // the same for SDDMM and the fused op
+bool spmm_plan_applies(const DeviceInfo& dev, SpmmShape& s, int M, int N, int nnz);  // true: s is the shape of the planned launch (R = 1)
 hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int* plan, hipStream_t stream);
 hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPlan& plan, float* partial,
                             hipStream_t stream);
 hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const SlicePlan& plan, void* workspace,
                               hipStream_t stream);
 
-SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4, bool rows_even = false);
+SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even = false);
 hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t stream);
 hipError_t sddmm_flat_launch(const SddmmArgs& x, const SddmmShape& s, int chunk, hipStream_t stream);
 hipError_t sddmm_sliced_launch(const SddmmArgs& x, const SddmmShape& s, const SlicePlan& plan, void* workspace,
                                hipStream_t stream);
 
-FusedShape fused_choose(int M, int D, int nnz, bool vec4, bool rows_even = false);
+FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even = false);
 hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream);
 hipError_t fused_flat_launch(const FusedArgs& x, const FusedShape& s, const FlatPlan& plan, float* partial,
                              hipStream_t stream);
@@ -163,12 +168,41 @@ struct SplitRule {
     int w8_few_rows_avg = 0;  // > 0: eight waves per row from this many nonzeros per row on where there are few rows
     int even_rows_avg = 128;  // rows known to be even are grouped four to a workgroup from this many nonzeros per row on
 };
-void choose_split(int M, long long col_tiles, int nnz, const SplitRule& rule, bool rows_even, int& W, int& R);
+void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, const SplitRule& rule, bool rows_even, int& W, int& R);
+
+// Row plan with cut rows ("cut plan"): rows longer than `longest_pct` per cent of a share (a share = the nonzeros of the
+// matrix over the compute units) are cut into pieces of at most `piece_pct` per cent of a share, and the plan hands out
+// `entries` = M + extra entries, each a whole row, a piece of a row, or nothing (no matrix can need more: see plan.hip).
+// All offsets are bytes from the start of the plan's memory; the launches read the first 4 x entries ints (first
+// nonzero, end, row, slot) and, SpMM and the fused op, the partial rows of the pieces and the list of cut rows.
+constexpr int kCutPlanMaxRows = 1 << 20;  // a cut plan is built by one workgroup: not for taller matrices
+constexpr int kCutPiecePct = 100, kCutLongestPct = 150;  // the rule (dlspm_tuning.cut_piece_pct / .cut_longest_pct override it)
+struct CutPlan {
+    int entries;      // M + ceil(bins x 100 / piece_pct)
+    int bins;         // compute units the plan was sized for (at most 256)
+    int piece_pct, longest_pct;
+    int slots;        // partial rows the plan has room for (more than the pieces of any matrix)
+    int max_cut;      // rows that can be cut (ceil(bins x 100 / longest_pct): more than any matrix has above the limit)
+    size_t off_keys;      // sort keys of the build (2 x entries 64-bit words; only beyond 2048 entries)
+    size_t off_virtual;   // the rows and pieces in matrix order: entries + 1 offsets, entries rows, entries slots
+    size_t off_cut;       // [0] number of cut rows, [1] share, [2] entries in use, [3] unused; then max_cut records of (row, first slot, pieces, in use)
+    size_t off_pieces;    // slots x width floats
+    size_t bytes;
+};
+CutPlan cut_plan_layout(int M, int width, int cus);
+hipError_t cut_plan_build_launch(int M, const int* row_offsets, const CutPlan& cp, void* plan, int order, hipStream_t stream);
+hipError_t cut_rows_sum_launch(int M, int width, const CutPlan& cp, const void* plan, float* out, hipStream_t stream);
+hipError_t spmm_pieces_launch(const SpmmArgs& x, const SpmmShape& s, const CutPlan& cp, void* plan, hipStream_t stream);
 
 // the same plan for the other two ops (16 < D <= 512, one row per four-wave workgroup)
-bool sddmm_plan_applies(SddmmShape& s, int M, int D, int nnz);
+// skewed (DLSPM_HINT_ROWS_SKEWED): the caller knows that the longest row is at least twenty times the mean
+bool plan_ungroups_skewed(const DeviceInfo& dev, int M, int nnz);
+bool sddmm_plan_applies(const DeviceInfo& dev, SddmmShape& s, int M, int D, int nnz, bool skewed = false);
 hipError_t sddmm_planned_launch(const SddmmArgs& x, const SddmmShape& s, const int* plan, hipStream_t stream);
-bool fused_plan_applies(FusedShape& s, int M, int D, int nnz);
+bool fused_plan_applies(const DeviceInfo& dev, FusedShape& s, int M, int D, int nnz, bool skewed = false);
 hipError_t fused_planned_launch(const FusedArgs& x, const FusedShape& s, const int* plan, hipStream_t stream);
+// with a cut plan: SDDMM needs neither partial rows nor a second kernel (every piece writes its own CSR slots)
+hipError_t sddmm_pieces_launch(const SddmmArgs& x, const SddmmShape& s, const CutPlan& cp, const void* plan, hipStream_t stream);
+hipError_t fused_pieces_launch(const FusedArgs& x, const FusedShape& s, const CutPlan& cp, void* plan, hipStream_t stream);
 
 }  // namespace dlspm

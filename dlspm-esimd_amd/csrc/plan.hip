@@ -439,13 +439,20 @@ __device__ __forceinline__ void pack_head(const int* s_len, int head, int nz, in
     __syncthreads();
 }
 
-// plan entry p <- `row`
-__device__ __forceinline__ void emit(int* __restrict__ plan, int M, long long p, long long row, const int* __restrict__ row_offsets)
+// plan entry p <- `row`. A cut plan (v_row != nullptr) is built over the rows and pieces in matrix order ("virtual rows":
+// row_offsets are then their offsets, M their number): entry p names the matrix row v_row[row] and the slot v_slot[row].
+__device__ __forceinline__ void emit(int* __restrict__ plan, int M, long long p, long long row, const int* __restrict__ row_offsets,
+                                     const int* __restrict__ v_row, const int* __restrict__ v_slot)
 {
     const int r = (int)min(max(row, 0ll), (long long)M - 1);
     plan[p] = row_offsets[r];
     plan[(size_t)M + p] = row_offsets[r + 1];
-    plan[2 * (size_t)M + p] = r;
+    if (v_row == nullptr) {
+        plan[2 * (size_t)M + p] = r;
+    } else {
+        plan[2 * (size_t)M + p] = v_row[r];
+        plan[3 * (size_t)M + p] = v_slot[r];
+    }
 }
 
 struct HeadShared {
@@ -457,7 +464,9 @@ struct HeadShared {
 
 // M <= kPlanTile: the whole build in one workgroup
 __global__ __launch_bounds__(kPlanThreads) void plan_one_block_kernel(int M, const int* __restrict__ row_offsets,
-                                                                      int* __restrict__ plan, int bins, int order)
+                                                                      int* __restrict__ plan, int bins, int order,
+                                                                      const int* __restrict__ v_row,
+                                                                      const int* __restrict__ v_slot)
 {
     __shared__ SortShared sort;
     __shared__ HeadShared hs;
@@ -469,7 +478,8 @@ __global__ __launch_bounds__(kPlanThreads) void plan_one_block_kernel(int M, con
     __syncthreads();
     const int head = min(M, kHeadPerBin * bins);
     pack_head(hs.len, head, min(nonzero_rows, head), bins, order, hs.order, hs.pack);
-    for (int p = threadIdx.x; p < M; p += kPlanThreads) emit(plan, M, p, hs.row[p < head ? hs.order[p] : p], row_offsets);
+    for (int p = threadIdx.x; p < M; p += kPlanThreads)
+        emit(plan, M, p, hs.row[p < head ? hs.order[p] : p], row_offsets, v_row, v_slot);
 }
 
 // M > kPlanTile, step 1: workgroup x sorts the keys of rows [x * kPlanTile, (x + 1) * kPlanTile)
@@ -505,7 +515,8 @@ __global__ __launch_bounds__(256) void plan_merge_kernel(long long M, long long 
 // step 3: workgroup 0 packs the head and writes its entries, the others write the entries behind it
 __global__ __launch_bounds__(kPlanThreads) void plan_emit_kernel(int M, const int* __restrict__ row_offsets,
                                                                  const u64* __restrict__ sorted, int* __restrict__ plan,
-                                                                 int bins, int order)
+                                                                 int bins, int order, const int* __restrict__ v_row,
+                                                                 const int* __restrict__ v_slot)
 {
     const int head = min(M, kHeadPerBin * bins);
     if (blockIdx.x == 0) {
@@ -525,12 +536,148 @@ __global__ __launch_bounds__(kPlanThreads) void plan_emit_kernel(int M, const in
         const int nz = sum_of_waves(hs.pack.wave_free[0]);
         __syncthreads();  // wave_free is written again after the packing
         pack_head(hs.len, head, nz, bins, order, hs.order, hs.pack);
-        for (int p = threadIdx.x; p < head; p += kPlanThreads) emit(plan, M, p, hs.row[hs.order[p]], row_offsets);
+        for (int p = threadIdx.x; p < head; p += kPlanThreads)
+            emit(plan, M, p, hs.row[hs.order[p]], row_offsets, v_row, v_slot);
         return;
     }
     const long long stride = (long long)(gridDim.x - 1) * kPlanThreads;
     for (long long p = head + (long long)(blockIdx.x - 1) * kPlanThreads + threadIdx.x; p < M; p += stride)
-        emit(plan, M, p, wide_row(sorted[p]), row_offsets);
+        emit(plan, M, p, wide_row(sorted[p]), row_offsets, v_row, v_slot);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Cut rows
+//
+// A row longer than one compute unit's share of the nonzeros sets the time of the whole launch through the one compute
+// unit it runs on. With share = ceil(nnz / bins) (at least 1), piece = ceil(share x piece_pct / 100) and longest =
+// max(piece, ceil(share x longest_pct / 100)) (the rule: 100 and 150 per cent), a row of more than `longest` nonzeros is
+// cut into c = ceil(length / piece) pieces of ceil(length / c) nonzeros (the last one what is left; none is empty), and
+// the plan is built over the "virtual rows" -- the rows and pieces in matrix order -- like a plan over rows. How many
+// there can be: the cut rows hold at most nnz <= share x bins nonzeros, so their pieces number at most
+// bins x 100 / piece_pct + (cut rows), and fewer than bins x 100 / longest_pct rows can exceed `longest`; hence at most
+// ceil(bins x 100 / piece_pct) entries more than rows, whatever the matrix. The plan is sized for those bounds (entries
+// that are not needed hold nothing), so its size and the grids of its launches depend on M and the device alone.
+// One workgroup: pass 1 counts the nonzeros (from the offsets themselves, so the bounds hold for any array), pass 2
+// numbers the virtual rows, the pieces' slots and the cut rows with one running sum over (entries | slots << 32 | cut
+// rows << 48), 1024 rows per round.
+__global__ __launch_bounds__(kPlanThreads) void plan_cut_kernel(int M, const int* __restrict__ row_offsets, int bins,
+                                                                int piece_pct, int longest_pct, int entries, int slots,
+                                                                int max_cut,
+                                                                int* __restrict__ v_off, int* __restrict__ v_row,
+                                                                int* __restrict__ v_slot, int* __restrict__ cut)
+{
+    __shared__ long long s_nnz[kPlanThreads / 64];
+    __shared__ u64 s_scan[kPlanThreads / 64];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    long long mine = 0;
+    for (int i = t; i < M; i += kPlanThreads) mine += max(row_offsets[i + 1] - row_offsets[i], 0);
+    for (int m = 32; m >= 1; m >>= 1) mine += __shfl_xor(mine, m);
+    if (lane == 0) s_nnz[wave] = mine;
+    __syncthreads();
+    long long total = 0;
+#pragma unroll
+    for (int x = 0; x < kPlanThreads / 64; ++x) total += s_nnz[x];
+    const long long share = max((total + bins - 1) / bins, 1ll);
+    const long long piece_max = max((share * piece_pct + 99) / 100, 1ll);
+    const long long longest_whole = max((share * longest_pct + 99) / 100, piece_max);
+
+    u64 carry = 0;  // virtual rows | slots << 32 | cut rows << 48 of the rows before this round
+    for (int base = 0; base < M; base += kPlanThreads) {
+        const int i = base + t;
+        int rs = 0, len = 0, c = 0;
+        bool cut_it = false;
+        if (i < M) {
+            rs = row_offsets[i];
+            len = max(row_offsets[i + 1] - rs, 0);
+            cut_it = len > longest_whole;
+            c = cut_it ? (int)((len + piece_max - 1) / piece_max) : 1;
+        }
+        const u64 x = (u64)c | (cut_it ? ((u64)c << 32) | (1ull << 48) : 0ull);
+        u64 inc = x;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const u64 y = __shfl_up(inc, d);
+            inc += lane >= d ? y : 0ull;
+        }
+        if (lane == 63) s_scan[wave] = inc;
+        __syncthreads();
+        u64 before = carry, round = 0;
+#pragma unroll
+        for (int xw = 0; xw < kPlanThreads / 64; ++xw) {
+            const u64 w = s_scan[xw];
+            before += xw < wave ? w : 0ull;
+            round += w;
+        }
+        const u64 ex = before + inc - x;
+        const int e0 = (int)(ex & 0xFFFFFFFFull), s0 = (int)((ex >> 32) & 0xFFFFull), j = (int)(ex >> 48);
+        if (i < M) {
+            if (!cut_it) {
+                if (e0 < entries) {
+                    v_off[e0] = rs;
+                    v_row[e0] = i;
+                    v_slot[e0] = -1;
+                }
+            } else {
+                const int piece = (len + c - 1) / c;
+                for (int k = 0; k < c && e0 + k < entries; ++k) {
+                    v_off[e0 + k] = rs + min(len, k * piece);
+                    v_row[e0 + k] = i;
+                    v_slot[e0 + k] = s0 + k < slots ? s0 + k : -2;  // (beyond the bound: only if the offsets changed under the build)
+                }
+                if (j < max_cut) {  // one record of four ints per cut row: row, first slot, pieces, 1
+                    cut[4 + 4 * j] = i;
+                    cut[4 + 4 * j + 1] = s0;
+                    cut[4 + 4 * j + 2] = c;
+                    cut[4 + 4 * j + 3] = 1;
+                }
+            }
+        }
+        carry += round;
+        __syncthreads();  // s_scan is written again in the next round
+    }
+    const long long used = min((long long)(carry & 0xFFFFFFFFull), (long long)entries);
+    const int end = M > 0 ? row_offsets[M] : 0;
+    for (long long e = used + t; e <= entries; e += kPlanThreads) {
+        v_off[e] = end;
+        if (e < entries) {
+            v_row[e] = -1;
+            v_slot[e] = -2;
+        }
+    }
+    const int cut_rows = min((int)(carry >> 48), max_cut);
+    for (int j = cut_rows + t; j < max_cut; j += kPlanThreads)  // the records that are not in use say so
+        reinterpret_cast<int4*>(cut + 4)[j] = make_int4(0, 0, 0, 0);
+    if (t == 0) {
+        cut[0] = cut_rows;
+        cut[1] = (int)min(share, 0x7fffffffll);
+        cut[2] = (int)used;
+        cut[3] = 0;
+    }
+}
+
+// out[row] <- the sum of the row's pieces, in piece order, for every cut row (one workgroup per cut row that the plan has
+// room for; those beyond the matrix's own number leave at once). Everything read from the plan is clamped to the arrays.
+template <int VEC, int THREADS>
+__global__ __launch_bounds__(THREADS) void cut_rows_sum_kernel(int M, int width, int slots,
+                                                           const int* __restrict__ cut, const float* __restrict__ pieces,
+                                                           float* __restrict__ out)
+{
+    using VecT = Vec<VEC>;
+    // (row, first slot, pieces, in use) of cut row blockIdx.x: one scalar load, the first of two round trips to memory
+    const int4 rec = reinterpret_cast<const int4*>(cut + 4)[blockIdx.x];
+    if (rec.w == 0) return;
+    const int row = min(max(rec.x, 0), M - 1);
+    const int first = min(max(rec.y, 0), slots);
+    const int cnt = min(max(rec.z, 0), slots - first);
+    const float* part = pieces + (size_t)first * width;
+    float* orow = out + (size_t)row * width;
+    for (int col = threadIdx.x * VEC; col < width; col += THREADS * VEC) {
+        const int c = min(col, width - VEC);  // the last thread of a row moves back to the row's last VEC floats
+        VecT sum = VecT::zero();
+#pragma unroll 4
+        for (int k = 0; k < cnt; ++k) sum.add(VecT::gload(part + (size_t)k * width + c));
+        sum.gstore(orow + c);
+    }
 }
 
 }  // namespace
@@ -543,15 +690,19 @@ size_t row_plan_bytes(int M)
     return M <= kPlanTile ? plan : (plan + 7) / 8 * 8 + (size_t)2 * (size_t)M * sizeof(u64);
 }
 
-hipError_t row_plan_build_launch(int M, const int* row_offsets, int* plan, int bins, int order, hipStream_t stream)
+// The plan of M rows (or virtual rows, with v_row and v_slot) with offsets row_offsets; `keys`: 2 x M words for the sort
+// beyond one tile.
+static hipError_t build_plan(int M, const int* row_offsets, int* plan, u64* keys, int bins, int order, const int* v_row,
+                             const int* v_slot, hipStream_t stream)
 {
     if (M <= 0) return hipSuccess;
     bins = bins < 1 ? 1 : bins > kPlanMaxBins ? kPlanMaxBins : bins;
     if (M <= kPlanTile) {
-        hipLaunchKernelGGL(plan_one_block_kernel, dim3(1), dim3(kPlanThreads), 0, stream, M, row_offsets, plan, bins, order);
+        hipLaunchKernelGGL(plan_one_block_kernel, dim3(1), dim3(kPlanThreads), 0, stream, M, row_offsets, plan, bins, order,
+                           v_row, v_slot);
         return hipGetLastError();
     }
-    u64* keys_a = reinterpret_cast<u64*>(reinterpret_cast<char*>(plan) + ((size_t)3 * (size_t)M * sizeof(int) + 7) / 8 * 8);
+    u64* keys_a = keys;
     u64* keys_b = keys_a + M;
     const unsigned tiles = (unsigned)ceil_div(M, kPlanTile);
     hipLaunchKernelGGL(plan_tile_sort_kernel, dim3(tiles), dim3(kPlanThreads), 0, stream, M, row_offsets, keys_a);
@@ -568,7 +719,72 @@ hipError_t row_plan_build_launch(int M, const int* row_offsets, int* plan, int b
     }
     const long long tail_blocks = ceil_div(M, kPlanThreads);
     const unsigned blocks = 1 + (unsigned)(tail_blocks < 2048 ? tail_blocks : 2048);
-    hipLaunchKernelGGL(plan_emit_kernel, dim3(blocks), dim3(kPlanThreads), 0, stream, M, row_offsets, in, plan, bins, order);
+    hipLaunchKernelGGL(plan_emit_kernel, dim3(blocks), dim3(kPlanThreads), 0, stream, M, row_offsets, in, plan, bins, order,
+                       v_row, v_slot);
+    return hipGetLastError();
+}
+
+hipError_t row_plan_build_launch(int M, const int* row_offsets, int* plan, int bins, int order, hipStream_t stream)
+{
+    u64* keys = reinterpret_cast<u64*>(reinterpret_cast<char*>(plan) + ((size_t)3 * (size_t)M * sizeof(int) + 7) / 8 * 8);
+    return build_plan(M, row_offsets, plan, keys, bins, order, nullptr, nullptr, stream);
+}
+
+// ---- cut plan: layout, build, and the sum of the pieces ------------------------------------------------------------
+
+CutPlan cut_plan_layout(int M, int width, int cus)
+{
+    CutPlan cp{};
+    if (M <= 0 || M > kCutPlanMaxRows || width < 0) return cp;  // bytes == 0: no cut plan for this height
+    cp.bins = cus < 1 ? 1 : cus > kPlanMaxBins ? kPlanMaxBins : cus;
+    const Tuning& t = tuning();
+    cp.piece_pct = t.cut_piece_pct > 0 ? t.cut_piece_pct : kCutPiecePct;
+    cp.longest_pct = t.cut_longest_pct > 0 ? t.cut_longest_pct : kCutLongestPct;
+    const int extra = (cp.bins * 100 + cp.piece_pct - 1) / cp.piece_pct;
+    cp.max_cut = (cp.bins * 100 + cp.longest_pct - 1) / cp.longest_pct;
+    cp.entries = M + extra;
+    cp.slots = extra + cp.max_cut;
+    auto align = [](size_t x, size_t a) { return (x + a - 1) / a * a; };
+    size_t at = align((size_t)4 * cp.entries * sizeof(int), 8);
+    cp.off_keys = at;
+    if (cp.entries > kPlanTile) at += (size_t)2 * cp.entries * sizeof(u64);
+    cp.off_virtual = at;
+    at = align(at + ((size_t)3 * cp.entries + 1) * sizeof(int), 16);
+    cp.off_cut = at;
+    at = align(at + ((size_t)4 + 4 * (size_t)cp.max_cut) * sizeof(int), 256);
+    cp.off_pieces = at;
+    cp.bytes = at + (size_t)cp.slots * (size_t)width * sizeof(float);
+    return cp;
+}
+
+hipError_t cut_plan_build_launch(int M, const int* row_offsets, const CutPlan& cp, void* plan, int order, hipStream_t stream)
+{
+    if (M <= 0 || cp.bytes == 0) return hipErrorInvalidValue;
+    char* base = static_cast<char*>(plan);
+    int* v_off = reinterpret_cast<int*>(base + cp.off_virtual);
+    int* v_row = v_off + cp.entries + 1;
+    int* v_slot = v_row + cp.entries;
+    int* cut = reinterpret_cast<int*>(base + cp.off_cut);
+    hipLaunchKernelGGL(plan_cut_kernel, dim3(1), dim3(kPlanThreads), 0, stream, M, row_offsets, cp.bins, cp.piece_pct,
+                       cp.longest_pct, cp.entries, cp.slots, cp.max_cut, v_off, v_row, v_slot, cut);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return build_plan(cp.entries, v_off, reinterpret_cast<int*>(base), reinterpret_cast<u64*>(base + cp.off_keys), cp.bins, order,
+                      v_row, v_slot, stream);
+}
+
+hipError_t cut_rows_sum_launch(int M, int width, const CutPlan& cp, const void* plan, float* out, hipStream_t stream)
+{
+    if (M <= 0 || width <= 0) return hipSuccess;
+    const char* base = static_cast<const char*>(plan);
+    const int* cut = reinterpret_cast<const int*>(base + cp.off_cut);
+    const float* pieces = reinterpret_cast<const float*>(base + cp.off_pieces);
+    if (width > 256)
+        hipLaunchKernelGGL((cut_rows_sum_kernel<4, 256>), dim3(cp.max_cut), dim3(256), 0, stream, M, width, cp.slots, cut, pieces, out);
+    else if (width >= 4)  // one wave covers the row
+        hipLaunchKernelGGL((cut_rows_sum_kernel<4, 64>), dim3(cp.max_cut), dim3(64), 0, stream, M, width, cp.slots, cut, pieces, out);
+    else
+        hipLaunchKernelGGL((cut_rows_sum_kernel<1, 64>), dim3(cp.max_cut), dim3(64), 0, stream, M, width, cp.slots, cut, pieces, out);
     return hipGetLastError();
 }
 

@@ -41,7 +41,7 @@ struct SampledOut {
 static inline SampledOut sampled_out(const SddmmArgs& x)
 {
     const int forced = tuning().stream_results;  // -1: the size rule (sweeps and tests switch it off or on)
-    const long long l2 = device_info().l2_bytes;
+    const long long l2 = x.l2_bytes;
     const bool by_rule = (long long)x.nnz * (long long)sizeof(float) > l2 + l2 / 2;
     return SampledOut{x.out, (forced < 0 ? by_rule : forced != 0) ? 1 : 0};
 }
@@ -78,7 +78,7 @@ __device__ __forceinline__ void sddmm_segment(int p, int q, int D, const int* __
 // The work of workgroup `bid` (RowBlock in common.hpp explains SLICED and PLANNED; a segment's results go where its
 // nonzeros lie, so a sliced or planned launch writes the same slots as any other). This kernel has neither LDS nor a
 // barrier.
-template <int VEC, int G1, int DS, bool MASKED, int W, int R, bool SLICED, bool PLANNED = false>
+template <int VEC, int G1, int DS, bool MASKED, int W, int R, bool SLICED, int PLANNED = kPlanNone>
 __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __restrict__ row_offsets,
                                             const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                             const float* __restrict__ lhs, const float* __restrict__ rhs,
@@ -131,7 +131,8 @@ __global__ __launch_bounds__(4 * 64) void sddmm_planned_kernel(int M, int D, int
                                                                const float* __restrict__ lhs, const float* __restrict__ rhs,
                                                                SampledOut out)
 {
-    sddmm_block<VEC, G1, DS, MASKED, 4, 1, true, true>((int)blockIdx.x, M, D, starts, ends, col_indices, lhs, rhs, out, rows, nnz);
+    sddmm_block<VEC, G1, DS, MASKED, 4, 1, true, kPlanRows>((int)blockIdx.x, M, D, starts, ends, col_indices, lhs, rhs, out, rows,
+                                                            nnz);
 }
 
 template <int VEC, int G1, int DS, int W, int R>
@@ -169,7 +170,7 @@ static hipError_t launch_wr(const SddmmArgs& x, int W, int R, hipStream_t stream
     return hipErrorInvalidValue;
 }
 
-SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4, bool rows_even)
+SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even)
 {
     SddmmShape s{};
     s.vec = vec4 ? 4 : 1;
@@ -183,7 +184,7 @@ SddmmShape sddmm_choose(int M, int D, int nnz, bool vec4, bool rows_even)
         s.G1 = 4;
         s.DS = 1;
     }
-    choose_split(M, 1, nnz, SplitRule{2, 16, kWave / s.G1, true, 96}, rows_even, s.W, s.R);
+    choose_split(dev, M, 1, nnz, SplitRule{2, 16, kWave / s.G1, true, 96}, rows_even, s.W, s.R);
     return s;
 }
 
@@ -326,39 +327,52 @@ hipError_t sddmm_sliced_launch(const SddmmArgs& x, const SddmmShape& s, const Sl
 
 // ---- row plan ---------------------------------------------------------------------------------------
 
-bool sddmm_plan_applies(SddmmShape& s, int M, int D, int nnz)
+bool sddmm_plan_applies(const DeviceInfo& dev, SddmmShape& s, int M, int D, int nnz, bool skewed)
 {
     if (s.vec != 4 || s.G1 != 8 || s.DS < 1 || s.W != 4) return false;  // built for 16 < D <= 512
     if (s.R == 1) return true;
-    if (!plan_ungroups_dots(M, D, nnz)) return false;
+    if (!plan_ungroups_dots(dev, M, D, nnz) && !(skewed && plan_ungroups_skewed(dev, M, nnz))) return false;
     s.R = 1;
     return true;
 }
 
+// `entries` workgroups: M for a plan over whole rows; a cut plan's M + bins, each a row, a piece of a row (its results go
+// to its own CSR slots like any others: no partial rows, no second kernel, the same bits) or nothing (first nonzero ==
+// end, which writes nothing)
 template <int DS>
-static hipError_t launch_planned(const SddmmArgs& x, const int* plan, hipStream_t stream)
+static hipError_t launch_planned(const SddmmArgs& x, const int* plan, int entries, hipStream_t stream)
 {
-    const int *starts = plan, *ends = plan + x.M, *rows = plan + 2 * (size_t)x.M;
+    const int *starts = plan, *ends = plan + entries, *rows = plan + 2 * (size_t)entries;
     if (x.D == 8 * 4 * DS)
-        hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, false>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M, x.D,
+        hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, false>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
                            x.nnz, starts, ends, rows, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     else
-        hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, true>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M, x.D,
+        hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, true>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
                            x.nnz, starts, ends, rows, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     return hipGetLastError();
 }
 
-hipError_t sddmm_planned_launch(const SddmmArgs& x, const SddmmShape& s, const int* plan, hipStream_t stream)
+static hipError_t launch_planned_ds(const SddmmArgs& x, const SddmmShape& s, const int* plan, int entries, hipStream_t stream)
 {
     if (x.M <= 0) return hipSuccess;
     switch (s.DS) {
-        case 1: return launch_planned<1>(x, plan, stream);
-        case 2: return launch_planned<2>(x, plan, stream);
-        case 4: return launch_planned<4>(x, plan, stream);
-        case 8: return launch_planned<8>(x, plan, stream);
-        case 16: return launch_planned<16>(x, plan, stream);
+        case 1: return launch_planned<1>(x, plan, entries, stream);
+        case 2: return launch_planned<2>(x, plan, entries, stream);
+        case 4: return launch_planned<4>(x, plan, entries, stream);
+        case 8: return launch_planned<8>(x, plan, entries, stream);
+        case 16: return launch_planned<16>(x, plan, entries, stream);
     }
     return hipErrorInvalidValue;
+}
+
+hipError_t sddmm_planned_launch(const SddmmArgs& x, const SddmmShape& s, const int* plan, hipStream_t stream)
+{
+    return launch_planned_ds(x, s, plan, x.M, stream);
+}
+
+hipError_t sddmm_pieces_launch(const SddmmArgs& x, const SddmmShape& s, const CutPlan& cp, const void* plan, hipStream_t stream)
+{
+    return launch_planned_ds(x, s, static_cast<const int*>(plan), cp.entries, stream);
 }
 
 }  // namespace dlspm

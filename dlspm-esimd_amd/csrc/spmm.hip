@@ -76,18 +76,19 @@ __device__ __forceinline__ void spmm_segment(Vec<VEC>* acc, int p, int q, const 
 // tile 0, then of tile 1, ...) when it does not, so that the device gathers from one K x TW slab of B at a time.
 // Measured on 512 x 4608, N = 3136 (B: 55 MiB): 708 -> 239 us tile-major; on 2048 x 1024, N = 784 (3 MiB), lognormal
 // rows: 81 us row-major, 93 us tile-major. No division in the usual case of one tile.
-template <int VEC, int G, int V, int W, int R, bool SLICED, bool PLANNED = false, bool BUF = false>
+template <int VEC, int G, int V, int W, int R, bool SLICED, int PLANNED = kPlanNone, bool BUF = false>
 __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles, int tile_major,
                                            const int* __restrict__ row_offsets,
                                            const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                            const float* __restrict__ values, const float* __restrict__ B,
                                            float* __restrict__ C, const int* __restrict__ row_ids = nullptr, int nnz = 0,
-                                           int flags = 0)
+                                           int flags = 0, int row_blocks = 0, const int* __restrict__ row_slots = nullptr,
+                                           float* __restrict__ pieces = nullptr, int slots = 0)
 {
     int ct = 0, rb = bid;
     if (col_tiles != 1) {
         if (tile_major) {
-            const int row_blocks = (M - 1) / R + 1;
+            if constexpr (!PLANNED) row_blocks = (M - 1) / R + 1;  // (a plan has as many entries as its launch says)
             ct = bid / row_blocks;
             rb = bid - ct * row_blocks;
         } else {
@@ -97,10 +98,13 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
     }
     RowBlock<W, R, SLICED, PLANNED> blk;
     blk.load(rb, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, values, B, C); },
-             col_tiles == 1 ? flags : flags & ~1);
-    dense_rows_block<VEC, G, V>(blk, ct, N, C, [&](Vec<VEC>* acc, int, int p, int q, const int* colv) {
-        spmm_segment<VEC, G, V, BUF>(acc, p, q, col_indices, values, B, N, colv, blk.lane);
-    });
+             col_tiles == 1 ? flags : flags & ~1, row_slots, slots);
+    dense_rows_block<VEC, G, V>(
+        blk, ct, N, C,
+        [&](Vec<VEC>* acc, int, int p, int q, const int* colv) {
+            spmm_segment<VEC, G, V, BUF>(acc, p, q, col_indices, values, B, N, colv, blk.lane);
+        },
+        pieces);
 }
 
 // BUF: B is read through a buffer descriptor (B below 4 GiB: see dense_rows_fma)
@@ -141,8 +145,25 @@ __global__ __launch_bounds__(4 * 64) void spmm_planned_kernel(int M, int N, int 
                                                               const float* __restrict__ values,
                                                               const float* __restrict__ B, float* __restrict__ C)
 {
-    spmm_block<VEC, G, V, 4, 1, true, true, BUF>((int)blockIdx.x, M, N, col_tiles, 1, starts, ends, col_indices, values, B, C,
-                                                 rows, nnz, flags);
+    spmm_block<VEC, G, V, 4, 1, true, kPlanRows, BUF>((int)blockIdx.x, M, N, col_tiles, 1, starts, ends, col_indices, values,
+                                                      B, C, rows, nnz, flags, M);
+}
+
+// Row plan with cut rows: `entries` workgroups per column tile, entry i = the nonzeros [starts[i], ends[i]) of row rows[i],
+// which is the whole row (slot_of[i] == -1: stored to C), a piece of it (slot_of[i] = s >= 0: the piece's sum goes to
+// pieces[s][0 .. N) and cut_rows_sum_kernel adds the pieces of each cut row afterwards), or nothing (below -1).
+template <int VEC, int G, int V, bool BUF>
+__global__ __launch_bounds__(4 * 64) void spmm_pieces_kernel(int M, int N, int nnz, int col_tiles, int flags, int entries,
+                                                             int slots, const int* __restrict__ starts,
+                                                             const int* __restrict__ ends, const int* __restrict__ rows,
+                                                             const int* __restrict__ slot_of,
+                                                             const int* __restrict__ col_indices,
+                                                             const float* __restrict__ values,
+                                                             const float* __restrict__ B, float* __restrict__ C,
+                                                             float* __restrict__ pieces)
+{
+    spmm_block<VEC, G, V, 4, 1, true, kPlanPieces, BUF>((int)blockIdx.x, M, N, col_tiles, 1, starts, ends, col_indices, values,
+                                                        B, C, rows, nnz, flags, entries, slot_of, pieces, slots);
 }
 
 // ---- host side --------------------------------------------------------------------------------------
@@ -200,12 +221,12 @@ static hipError_t launch_wr(const SpmmArgs& x, int W, int R, int tile_major, hip
 // equal; K = 65536, slab 8 MiB, 655 per row: 330 -> 236 us).
 // dlspm_tuning.tile_major = 0|1 and .tile_width = 512|...|32 override the rule for tuning sweeps. "The L2" is the
 // device's own figure for one of them (4 MiB on MI355X), "all at once" eight workgroups on each compute unit.
-static int spmm_tile_width(int M, int K, int N, int nnz, bool narrow_tiles)
+static int spmm_tile_width(const DeviceInfo& dev, int M, int K, int N, int nnz, bool narrow_tiles)
 {
-    const long long l2 = device_info().l2_bytes;
+    const long long l2 = dev.l2_bytes;
     const int min_tile = narrow_tiles ? 32 : 128;
     if (N <= min_tile) return 0;
-    bool on = (double)K * (double)N * (double)sizeof(float) > (double)l2 && (long long)M * ceil_div(N, 512) >= 8ll * device_info().cus;
+    bool on = (double)K * (double)N * (double)sizeof(float) > (double)l2 && (long long)M * ceil_div(N, 512) >= 8ll * dev.cus;
     if (tuning().tile_major >= 0) on = tuning().tile_major != 0;
     if (!on) return 0;
     int tile = min_tile;
@@ -229,12 +250,12 @@ static int spmm_tile_width(int M, int K, int N, int nnz, bool narrow_tiles)
 }
 
 // Chooses the lane layout from N (and the height of B) and the (W, R) split from the mean row length.
-SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles, bool banded)
+SpmmShape spmm_choose(const DeviceInfo& dev, int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles, bool banded)
 {
     SpmmShape s{};
     s.vec = vec4 ? 4 : 1;
     // banded (DLSPM_HINT_BANDED): no L2-sized column tiles, each XCD gathers from its own part of B anyway
-    const int tile = vec4 && !banded ? spmm_tile_width(M, K, N, nnz, narrow_tiles) : 0;
+    const int tile = vec4 && !banded ? spmm_tile_width(dev, M, K, N, nnz, narrow_tiles) : 0;
     s.tile_major = tile > 0 ? 1 : 0;
     if (vec4) {
         if (tile == 512) { s.G = 64; s.V = 2; }
@@ -252,7 +273,7 @@ SpmmShape spmm_choose(int M, int K, int N, int nnz, bool vec4, bool rows_even, b
         s.V = 1;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(M, ceil_div(N, tw), nnz, SplitRule{8, 16, kWave / s.G, true, 0, s.G == kWave ? 96 : 128}, rows_even, s.W, s.R);
+    choose_split(dev, M, ceil_div(N, tw), nnz, SplitRule{8, 16, kWave / s.G, true, 0, s.G == kWave ? 96 : 128}, rows_even, s.W, s.R);
     return s;
 }
 
@@ -440,10 +461,10 @@ hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const Slice
 // 18.3 against 24.6 us; 8192 x 2048, 199 per row, N = 128: 29.1 against 37.5 us; 16384 x 512, 51 per row, N = 256: 31.4
 // against 35.3 us; 65536 x 2048, 197 per row, N = 128: 223 against 232 us; but 32768 x 1024, 32 per row, N = 256: 46.6
 // against 43.9 us; 16384 x 2048, 101 per row, N = 32: 17.7 against 14.2 us; rows below 32 nonzeros lose everywhere.
-bool plan_ungroups(int M, int width, int nnz)
+bool plan_ungroups(const DeviceInfo& dev, int M, int width, int nnz)
 {
     const long long avg32 = 32ll * M, avg48 = 48ll * M, avg128 = 128ll * M;
-    const long long cus = device_info().cus;  // measured on 256 compute units: 4096, 8192 and 16384 rows
+    const long long cus = dev.cus;  // measured on 256 compute units: 4096, 8192 and 16384 rows
     return nnz >= avg32 && (M <= 16 * cus || (width >= 128 && (M <= 32 * cus || (nnz >= avg48 && M <= 64 * cus) || nnz >= avg128)));
 }
 
@@ -454,20 +475,32 @@ bool plan_ungroups(int M, int width, int nnz)
 // Up to eight rows per compute unit the plan's order wins whatever the length of the rows (lognormal rows, sigma 0.8,
 // D = 64 / 128, rule's grouping against one row per workgroup in plan order: 2048 x 1024, 8 per row: fused 4.86 -> 4.44 us,
 // SDDMM 3.71 -> 3.57 us; 24 per row: 6.04 -> 4.97 us, 4.26 -> 4.03 us; from 4096 rows on short rows lose).
-bool plan_ungroups_dots(int M, int D, int nnz)
+bool plan_ungroups_dots(const DeviceInfo& dev, int M, int D, int nnz)
 {
-    const long long cus = device_info().cus;  // measured on 256 compute units: 2048, 4096 and 8192 rows
+    const long long cus = dev.cus;  // measured on 256 compute units: 2048, 4096 and 8192 rows
     if (M <= 8 * cus) return true;
     return (long long)nnz >= 32ll * M && (M <= 16 * cus || (D >= 128 && M <= 32 * cus && (long long)nnz >= 128ll * M));
 }
 
-bool spmm_plan_applies(SpmmShape& s, int M, int N, int nnz)
+// Very uneven rows (the longest at least twenty times the mean: lognormal row lengths from sigma = 1 on) in masks of 16 to
+// 64 rows per compute unit: SDDMM and the fused op, which the size rule runs several rows per workgroup there, take
+// 0.63 ... 0.93 of the time with one row per workgroup in plan order (8192 x 2048, 60 per row, sigma = 1: fused at D = 64
+// 27.3 -> 17.5 us, SDDMM at D = 128 24.0 -> 17.6 us; 16384 x 4096, sigma = 1.5: 58.8 -> 44.1 and 59.2 -> 41.3 us); at
+// sigma <= 0.6, or from 128 rows per compute unit on, the same choice loses 4 ... 100 %. The sizes cannot tell the two
+// apart, so this applies on the caller's word only (DLSPM_HINT_ROWS_SKEWED; dlspm_advise says it from the longest row).
+bool plan_ungroups_skewed(const DeviceInfo& dev, int M, int nnz)
+{
+    const long long cus = dev.cus;  // measured on 256 compute units: 8192 and 16384 rows
+    return M > 16 * cus && M <= 64 * cus && (long long)nnz >= 32ll * M;
+}
+
+bool spmm_plan_applies(const DeviceInfo& dev, SpmmShape& s, int M, int N, int nnz)
 {
     // one column tile, or tiles in tile-major order (a B beyond one L2): there the workgroups of one tile are consecutive,
     // as the plan's packing assumes; tiles in row-major order (B within the L2) keep the matrix order
     if (s.vec != 4 || s.W != 4 || (s.G * s.vec * s.V < N && !s.tile_major)) return false;
     if (s.R == 1) return true;
-    if (!plan_ungroups(M, N, nnz)) return false;
+    if (!plan_ungroups(dev, M, N, nnz)) return false;
     s.R = 1;
     return true;
 }
@@ -496,6 +529,41 @@ hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int*
     DLSPM_PLANNED(8, 1)
 #undef DLSPM_PLANNED
     return hipErrorInvalidValue;
+}
+
+// The same with a cut plan (CutPlan, launch.hpp): one workgroup per entry and column tile, then the kernel that adds the
+// pieces of the cut rows in piece order.
+hipError_t spmm_pieces_launch(const SpmmArgs& x, const SpmmShape& s, const CutPlan& cp, void* plan, hipStream_t stream)
+{
+    if (x.M <= 0) return hipSuccess;
+    const int* base = static_cast<const int*>(plan);
+    const int *starts = base, *ends = base + cp.entries, *rows = base + 2 * (size_t)cp.entries,
+              *slot_of = base + 3 * (size_t)cp.entries;
+    float* pieces = reinterpret_cast<float*>(static_cast<char*>(plan) + cp.off_pieces);
+    hipError_t e = hipErrorInvalidValue;
+#define DLSPM_PIECES(g_, v_)                                                                                              \
+    if (s.G == g_ && s.V == v_) {                                                                                         \
+        const int col_tiles = (int)ceil_div(x.N, g_ * 4 * v_);                                                            \
+        const long long blocks = (long long)cp.entries * col_tiles;                                                       \
+        if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;                                                   \
+        if (dense_fits_buffer(x.K, x.N))                                                                                  \
+            hipLaunchKernelGGL((spmm_pieces_kernel<4, g_, v_, true>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M, \
+                               x.N, x.nnz, col_tiles, launch_flags(0), cp.entries, cp.slots, starts, ends, rows, slot_of, \
+                               x.col_indices, x.values, x.B, x.C, pieces);                                                \
+        else                                                                                                              \
+            hipLaunchKernelGGL((spmm_pieces_kernel<4, g_, v_, false>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream,   \
+                               x.M, x.N, x.nnz, col_tiles, launch_flags(0), cp.entries, cp.slots, starts, ends, rows,     \
+                               slot_of, x.col_indices, x.values, x.B, x.C, pieces);                                       \
+        e = hipGetLastError();                                                                                            \
+    }
+    DLSPM_PIECES(64, 2)
+    DLSPM_PIECES(64, 1)
+    DLSPM_PIECES(32, 1)
+    DLSPM_PIECES(16, 1)
+    DLSPM_PIECES(8, 1)
+#undef DLSPM_PIECES
+    if (e != hipSuccess) return e;
+    return cut_rows_sum_launch(x.M, x.N, cp, plan, x.C, stream);
 }
 
 }  // namespace dlspm

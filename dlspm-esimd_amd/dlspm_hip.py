@@ -26,6 +26,8 @@ OP_SPMM, OP_SDDMM, OP_FUSED = 0, 1, 2
 HINT_ROWS_EVEN = 1 << 62
 HINT_ROW_PLAN = 1 << 61
 HINT_BANDED = 1 << 60
+HINT_CUT_PLAN = 1 << 59
+HINT_ROWS_SKEWED = 1 << 58
 
 
 class _RowsEven:
@@ -52,6 +54,10 @@ EXPORTS = (
     "dlspm_row_plan_bytes",
     "dlspm_row_plan_advice",
     "dlspm_row_plan_build",
+    "dlspm_row_plan_bytes_for",
+    "dlspm_analyze",
+    "dlspm_advise",
+    "dlspm_row_plan_build_cut",
     "dlspm_tuning_default",
     "dlspm_set_tuning",
     "dlspm_get_tuning",
@@ -70,7 +76,25 @@ EXPORTS = (
 class Tuning(ctypes.Structure):
     """dlspm_tuning of include/dlspm_hip.h."""
     _fields_ = [(n, ctypes.c_int) for n in ("split_w", "split_r", "flat", "flat_chunk", "slices", "tile_major",
-                                            "tile_width", "plan_order", "xcd_contiguous", "stream_results")]
+                                            "tile_width", "plan_order", "xcd_contiguous", "stream_results",
+                                            "cut_piece_pct", "cut_longest_pct")]
+
+
+class MatrixInfo(ctypes.Structure):
+    """dlspm_matrix_info of include/dlspm_hip.h."""
+    _fields_ = [(n, ctypes.c_int) for n in ("M", "K", "nnz", "max_row_len", "empty_rows", "max_col_span",
+                                            "eighths_cover_permille", "eighths_nnz_permille")]
+
+    def as_dict(self):
+        return {n: getattr(self, n) for n, _ in self._fields_}
+
+
+class CallPlan(ctypes.Structure):
+    """dlspm_call_plan of include/dlspm_hip.h."""
+    _fields_ = [("build", ctypes.c_int), ("bytes", ctypes.c_size_t), ("hints", ctypes.c_size_t)]
+
+
+BUILD_NOTHING, BUILD_ROW_PLAN, BUILD_CUT_PLAN = 0, 1, 2
 
 
 class DlspmError(RuntimeError):
@@ -116,6 +140,14 @@ def lib() -> ctypes.CDLL:
         L.dlspm_row_plan_advice.restype = ci
         L.dlspm_row_plan_build.argtypes = [ci, vp, vp, sz, vp]
         L.dlspm_row_plan_build.restype = ci
+        L.dlspm_row_plan_bytes_for.argtypes = [ci, ci, ci]
+        L.dlspm_row_plan_bytes_for.restype = sz
+        L.dlspm_row_plan_build_cut.argtypes = [ci, vp, vp, sz, vp]
+        L.dlspm_row_plan_build_cut.restype = ci
+        L.dlspm_analyze.argtypes = [ci, ci, ci, vp, vp, vp, ctypes.POINTER(MatrixInfo)]
+        L.dlspm_analyze.restype = ci
+        L.dlspm_advise.argtypes = [ci, ci, ctypes.POINTER(MatrixInfo), ctypes.POINTER(CallPlan)]
+        L.dlspm_advise.restype = ci
         L.spmm_csr_f32_planned.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, sz, vp]
         L.spmm_csr_f32_planned.restype = ci
         L.sddmm_csr_f32_planned.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, sz, vp]
@@ -205,9 +237,10 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def row_plan_advice(op, M, K, N_or_D, nnz, max_row_len=-1) -> bool:
-    """Whether a row plan is worth building for op at these sizes (see dlspm_row_plan_advice)."""
-    return bool(lib().dlspm_row_plan_advice(op, M, K, N_or_D, nnz, max_row_len))
+def row_plan_advice(op, M, K, N_or_D, nnz, max_row_len=-1) -> int:
+    """Whether a row plan is worth building for op at these sizes (dlspm_row_plan_advice): 0 no, 1 a plan over whole rows
+    (row_plan), 2 a plan that cuts the longest rows (cut_plan)."""
+    return int(lib().dlspm_row_plan_advice(op, M, K, N_or_D, nnz, max_row_len))
 
 
 def row_plan_bytes(M: int) -> int:
@@ -230,6 +263,85 @@ def row_plan(row_offsets, out=None):
     return plan
 
 
+class CutPlan:
+    """A row plan that cuts rows longer than one compute unit's share of the nonzeros into pieces (cut_plan()): the
+    device memory, and the op and width it has room for."""
+
+    def __init__(self, memory, op, width):
+        self.memory, self.op, self.width = memory, op, width
+
+
+def row_plan_bytes_for(op: int, M: int, width: int) -> int:
+    return int(lib().dlspm_row_plan_bytes_for(op, M, width))
+
+
+def cut_plan(row_offsets, op, width, out=None) -> CutPlan:
+    """The cut plan of one matrix for op at dense width `width` (dlspm_row_plan_build_cut into
+    dlspm_row_plan_bytes_for(op, M, width) bytes), built by kernels on the current stream. Pass it as plan=... ."""
+    import torch
+
+    M = row_offsets.numel() - 1
+    need = (row_plan_bytes_for(op, M, width) + 3) // 4
+    if need == 0:
+        raise ValueError(f"no cut plan for a matrix of {M} rows")
+    mem = out if out is not None else torch.empty((need,), dtype=torch.int32, device=row_offsets.device)
+    st = lib().dlspm_row_plan_build_cut(M, _ptr(row_offsets, torch.int32, "row_offsets", M + 1), _ptr(mem, torch.int32, "plan", need),
+                                        mem.numel() * 4, _stream())
+    if st != OK:
+        raise DlspmError(st, "dlspm_row_plan_build_cut")
+    return CutPlan(mem, op, width)
+
+
+def analyze(row_offsets, col_indices, K) -> MatrixInfo:
+    """dlspm_analyze: one synchronising pass over the CSR structure on the GPU."""
+    import torch
+
+    M, nnz = row_offsets.numel() - 1, col_indices.numel()
+    info = MatrixInfo()
+    st = lib().dlspm_analyze(M, K, nnz, _ptr(row_offsets, torch.int32, "row_offsets", M + 1),
+                             _ptr(col_indices, torch.int32, "col_indices"), _stream(), ctypes.byref(info))
+    if st != OK:
+        raise DlspmError(st, "dlspm_analyze")
+    return info
+
+
+def advise(op, width, info: MatrixInfo) -> CallPlan:
+    """dlspm_advise (host only): what to allocate, build and hint for op at this dense width."""
+    cp = CallPlan()
+    st = lib().dlspm_advise(op, width, ctypes.byref(info), ctypes.byref(cp))
+    if st != OK:
+        raise DlspmError(st, "dlspm_advise")
+    return cp
+
+
+class Prepared:
+    """What dlspm_advise said for one matrix, op and width, allocated and built (prepare()): pass as prepared=... ."""
+
+    def __init__(self, memory, size_and_hints, call_plan):
+        self.memory, self.size_and_hints, self.call_plan = memory, size_and_hints, call_plan
+
+
+def prepare(row_offsets, col_indices, K, op, width, info=None) -> Prepared:
+    """The lead path of a caller: dlspm_analyze (unless `info` is given) -> dlspm_advise -> allocate -> build."""
+    import torch
+
+    info = info if info is not None else analyze(row_offsets, col_indices, K)
+    cp = advise(op, width, info)
+    M = row_offsets.numel() - 1
+    mem = torch.empty(((cp.bytes + 3) // 4,), dtype=torch.int32, device=row_offsets.device) if cp.bytes else None
+    if cp.build == BUILD_ROW_PLAN:
+        st = lib().dlspm_row_plan_build(M, _ptr(row_offsets, torch.int32, "row_offsets", M + 1), ctypes.c_void_p(mem.data_ptr()),
+                                        mem.numel() * 4, _stream())
+    elif cp.build == BUILD_CUT_PLAN:
+        st = lib().dlspm_row_plan_build_cut(M, _ptr(row_offsets, torch.int32, "row_offsets", M + 1), ctypes.c_void_p(mem.data_ptr()),
+                                            mem.numel() * 4, _stream())
+    else:
+        st = OK
+    if st != OK:
+        raise DlspmError(st, "dlspm_row_plan_build")
+    return Prepared(mem, (mem.numel() * 4 if mem is not None else 0) | cp.hints, cp)
+
+
 def _csr_sizes(row_offsets, col_indices):
     if row_offsets.numel() < 1:
         raise ValueError("row_offsets must hold M + 1 >= 1 entries")
@@ -242,6 +354,14 @@ def _workspace_args(workspace, plan, M, banded=False):
     import torch
 
     hint = HINT_BANDED if banded else 0
+    if isinstance(plan, Prepared):
+        if workspace is not None:
+            raise ValueError("pass what prepare() returned or a workspace, not both")
+        return (ctypes.c_void_p(plan.memory.data_ptr()) if plan.memory is not None else None), plan.size_and_hints | hint
+    if isinstance(plan, CutPlan):
+        if workspace is not None:
+            raise ValueError("pass a row plan or a workspace, not both")
+        return _ptr(plan.memory, torch.int32, "plan"), (plan.memory.numel() * 4) | HINT_CUT_PLAN | hint
     if plan is not None:
         if workspace is not None:
             raise ValueError("pass a row plan or a workspace, not both")

@@ -207,85 +207,82 @@ struct Options {
     int iters = 20;  // the reference keeps the minimum of 20 launches (SPMM/spmm-esimd-fromfile2.cpp:194-243)
     bool cold = false;
     int graph = 0;  // --graph n: also time a HIP graph of n launches, replayed five times (no event between the launches)
-    // what to pass as `workspace`: by default the memory dlspm_workspace_bytes asks for when the column-sliced schedule
-    // applies or the longest row is at least four times the mean row (dlspm_csr_row_stats), DLSPM_HINT_ROWS_EVEN when it is
-    // at most one and a half times the mean;
-    // --workspace: always the memory, --no-workspace: always NULL
+    // what to pass as `workspace`: by default what dlspm_advise says after one look at the matrix (dlspm_analyze);
+    // --workspace: always the schedule memory of dlspm_workspace_bytes, --no-workspace: always NULL
     enum Workspace { kAuto, kAlways, kNever } workspace = kAuto;
-    bool plan = true;  // build a row plan where dlspm_row_plan_advice says so (--no-plan: never)
+    bool plan = true;  // build a row plan or a cut plan where dlspm_advise says so (--no-plan: never)
     std::string csv, dump;
     std::string dump_each;  // --dump-each DIR: every case dumps into its own sub-directory DIR/case_000, DIR/case_001, ...
     double tol = 1e-4;  // relative Frobenius error allowed between the kernel and the check kernel
 };
 
-// What this run passes as `workspace`: what dlspm_workspace_advice says for the sizes and the longest row
-// (dlspm_csr_row_stats, one look per matrix) -- device memory, the hint DLSPM_HINT_ROWS_EVEN, or nothing.
-struct WorkspaceChoice {
-    size_t bytes = 0;        // device memory to allocate and pass
-    bool rows_even = false;  // pass NULL with DLSPM_HINT_ROWS_EVEN instead
-    bool plan = false;       // build a row plan and pass it as the workspace, with DLSPM_HINT_ROW_PLAN
-    bool banded = false;     // the pattern is a band (--band without --band-random): DLSPM_HINT_BANDED
-    void* arg(void* buffer) const { return bytes ? buffer : nullptr; }
-    size_t size() const { return (rows_even ? DLSPM_HINT_ROWS_EVEN : bytes) | (banded ? DLSPM_HINT_BANDED : 0); }
+// What this run passes as (workspace, workspace_bytes): one look at the matrix (dlspm_analyze, once per matrix structure)
+// and the library's answer for the op and the width (dlspm_advise) -- nothing, a hint, schedule memory, a row plan or a
+// cut plan -- allocated and, for the plans, built on the device here, with the time that took.
+struct PreparedCall {
+    DevBuf<char> memory{0};
+    size_t hints = 0;
+    int build = DLSPM_BUILD_NOTHING;
+    void* arg() const { return memory.n ? memory.p : nullptr; }
+    size_t size() const { return memory.n | hints; }
 };
-inline WorkspaceChoice workspace_to_pass(const Options& opt, int op, int M, int K, int width, int nnz,
-                                         const int* row_offsets_dev, bool plan_allowed = false, bool banded = false)
+inline PreparedCall prepare_call(const Options& opt, int op, int M, int K, int width, int nnz, const int* row_offsets_dev,
+                                 const int* col_indices_dev)
 {
-    WorkspaceChoice c;
-    if (opt.workspace == Options::kNever || M <= 0 || nnz <= 0) return c;
-    if (banded && opt.workspace == Options::kAuto) {
-        // what the generator knows and dlspm_workspace_advice cannot see: no memory, the hint instead
-        int longest = 0, empty = 0;
-        if (dlspm_csr_row_stats(M, row_offsets_dev, nullptr, &longest, &empty) != DLSPM_OK) throw std::runtime_error("dlspm_csr_row_stats failed");
-        c.banded = true;
-        c.rows_even = (long long)longest * 2 * M <= 3ll * nnz;  // longest row at most 1.5 x the mean
-        std::printf("rows: longest %d, mean %.1f, empty %d -> banded, DLSPM_HINT_BANDED passed%s\n", longest, (double)nnz / M, empty,
-                    c.rows_even ? " with DLSPM_HINT_ROWS_EVEN" : "");
-        return c;
+    PreparedCall pc;
+    if (opt.workspace == Options::kNever || M <= 0 || nnz <= 0) return pc;
+    dlspm_matrix_info mi;
+    if (dlspm_analyze(M, K, nnz, row_offsets_dev, col_indices_dev, nullptr, &mi) != DLSPM_OK) throw std::runtime_error("dlspm_analyze failed");
+    dlspm_call_plan cp{DLSPM_BUILD_NOTHING, 0, 0};
+    if (opt.workspace == Options::kAlways) {
+        cp.bytes = dlspm_workspace_bytes(op, M, K, width, nnz);
+    } else {
+        if (dlspm_advise(op, width, &mi, &cp) != DLSPM_OK) throw std::runtime_error("dlspm_advise failed");
+        if (!opt.plan && cp.build != DLSPM_BUILD_NOTHING) {  // --no-plan: what the advice says without plans
+            const int passing = dlspm_workspace_advice(op, M, K, width, nnz, mi.max_row_len);
+            cp = dlspm_call_plan{DLSPM_BUILD_NOTHING, passing == DLSPM_PASS_WORKSPACE ? dlspm_workspace_bytes(op, M, K, width, nnz) : 0,
+                                 passing == DLSPM_PASS_ROWS_EVEN ? DLSPM_HINT_ROWS_EVEN : 0};
+        }
     }
-    const size_t want = dlspm_workspace_bytes(op, M, K, width, nnz);
-    int longest = 0, empty = 0;
-    if (dlspm_csr_row_stats(M, row_offsets_dev, nullptr, &longest, &empty) != DLSPM_OK) throw std::runtime_error("dlspm_csr_row_stats failed");
-    if (plan_allowed && opt.workspace == Options::kAuto && dlspm_row_plan_advice(op, M, K, width, nnz, longest) == 1) {
-        c.plan = true;
-        std::printf("rows: longest %d, mean %.1f, empty %d -> uneven, row plan (one row per workgroup, handed out by length)\n",
-                    longest, (double)nnz / M, empty);
-        return c;
-    }
-    const int advice = dlspm_workspace_advice(op, M, K, width, nnz, longest);
     int slices = 0;
     (void)dlspm_describe_slices(op, M, K, width, nnz, &slices, nullptr);
-    if (opt.workspace == Options::kAlways || advice == DLSPM_PASS_WORKSPACE) c.bytes = want;
-    else c.rows_even = advice == DLSPM_PASS_ROWS_EVEN;
-    std::printf("rows: longest %d, mean %.1f, empty %d -> %s\n", longest, (double)nnz / M, empty,
-                opt.workspace == Options::kAlways ? "workspace passed (--workspace)"
-                : c.bytes && slices > 0           ? "dense operands beyond one L2, workspace passed (column-sliced schedule)"
-                : c.bytes                         ? "uneven, workspace passed (flat schedule)"
-                : c.rows_even                     ? "even, DLSPM_HINT_ROWS_EVEN passed"
-                                                  : "nothing passed");
-    return c;
-}
-
-// The row plan of one matrix (dlspm_row_plan_build: once per matrix, kernels on the stream), with what it cost on the
-// device (HIP events around the second of two builds: the first pays for loading the kernels).
-inline DevBuf<char> build_row_plan(int M, const int* row_offsets_dev)
-{
-    DevBuf<char> plan(dlspm_row_plan_bytes(M));
-    hipEvent_t e0, e1;
-    DLSPM_HIP_CHECK(hipEventCreate(&e0));
-    DLSPM_HIP_CHECK(hipEventCreate(&e1));
-    float ms = 0;
-    for (int rep = 0; rep < 2; ++rep) {
-        DLSPM_HIP_CHECK(hipEventRecord(e0, nullptr));
-        if (dlspm_row_plan_build(M, row_offsets_dev, plan.p, plan.n, nullptr) != DLSPM_OK) throw std::runtime_error("dlspm_row_plan_build failed");
-        DLSPM_HIP_CHECK(hipEventRecord(e1, nullptr));
-        DLSPM_HIP_CHECK(hipEventSynchronize(e1));
-        DLSPM_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+    std::printf("rows: longest %d, mean %.1f, empty %d; columns: widest row %d, eighths span %.2f x K -> %s%s%s\n", mi.max_row_len,
+                (double)nnz / M, mi.empty_rows, mi.max_col_span, mi.eighths_cover_permille * 1e-3,
+                opt.workspace == Options::kAlways           ? "workspace passed (--workspace)"
+                : cp.build == DLSPM_BUILD_CUT_PLAN          ? "a row above one and a half shares, cut plan (long rows handed out in pieces)"
+                : cp.build == DLSPM_BUILD_ROW_PLAN          ? "uneven, row plan (one row per workgroup, handed out by length)"
+                : (cp.hints & DLSPM_HINT_BANDED)            ? "banded, DLSPM_HINT_BANDED passed"
+                : cp.bytes && slices > 0                    ? "dense operands beyond one L2, workspace passed (column-sliced schedule)"
+                : cp.bytes                                  ? "uneven, workspace passed (flat schedule)"
+                : (cp.hints & DLSPM_HINT_ROWS_EVEN)         ? "even, DLSPM_HINT_ROWS_EVEN passed"
+                                                            : "nothing passed",
+                (cp.hints & DLSPM_HINT_BANDED) && (cp.hints & DLSPM_HINT_ROWS_EVEN) ? " with DLSPM_HINT_ROWS_EVEN" : "",
+                (cp.hints & DLSPM_HINT_ROWS_SKEWED) ? " with DLSPM_HINT_ROWS_SKEWED" : "");
+    pc.memory = DevBuf<char>(cp.bytes);
+    pc.hints = cp.hints;
+    pc.build = cp.build;
+    if (cp.bytes && cp.build == DLSPM_BUILD_NOTHING) std::printf("workspace: %zu bytes\n", cp.bytes);
+    if (cp.build != DLSPM_BUILD_NOTHING) {
+        // what the plan costs on the device: HIP events around the second of two builds (the first pays for loading the kernels)
+        hipEvent_t e0, e1;
+        DLSPM_HIP_CHECK(hipEventCreate(&e0));
+        DLSPM_HIP_CHECK(hipEventCreate(&e1));
+        float ms = 0;
+        for (int rep = 0; rep < 2; ++rep) {
+            DLSPM_HIP_CHECK(hipEventRecord(e0, nullptr));
+            const int st = cp.build == DLSPM_BUILD_CUT_PLAN ? dlspm_row_plan_build_cut(M, row_offsets_dev, pc.memory.p, pc.memory.n, nullptr)
+                                                            : dlspm_row_plan_build(M, row_offsets_dev, pc.memory.p, pc.memory.n, nullptr);
+            if (st != DLSPM_OK) throw std::runtime_error("building the row plan failed");
+            DLSPM_HIP_CHECK(hipEventRecord(e1, nullptr));
+            DLSPM_HIP_CHECK(hipEventSynchronize(e1));
+            DLSPM_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+        }
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+        std::printf("%s: %zu bytes, built on the device in %.1f us (once per matrix)\n",
+                    cp.build == DLSPM_BUILD_CUT_PLAN ? "cut plan" : "row plan", pc.memory.n, ms * 1e3);
     }
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
-    std::printf("row plan: %zu bytes, built on the device in %.1f us (once per matrix)\n", plan.n, ms * 1e3);
-    return plan;
+    return pc;
 }
 
 // `launch(stream)` enqueues one call of the op. Every launch is timed between its own pair of HIP events (the minimum is

@@ -44,15 +44,9 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     if (dlspm_csr_check(M, K, nnz, ro_d.p, ci_d.p, nullptr) != DLSPM_OK) throw std::invalid_argument("malformed CSR structure");
     DLSPM_HIP_CHECK(hipMemset(O_d.p, 0xFF, (size_t)M * D * sizeof(float)));
 
-    const bool banded = s.kind == CaseSpec::kShape && s.band > 0 && s.band_random == 0;
-    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_FUSED, M, K, D, nnz, ro_d.p, opt.plan, banded);  // 0 bytes for small problems
-    DevBuf<char> ws(wc.bytes);
-    if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
-    DevBuf<char> plan = wc.plan ? build_row_plan(M, ro_d.p) : DevBuf<char>(0);
+    const PreparedCall pc = prepare_call(opt, DLSPM_OP_FUSED, M, K, D, nnz, ro_d.p, ci_d.p);  // nothing for small, even problems
     const Timing t = time_launches(opt, [&](hipStream_t stream) {
-        if (wc.plan) return fused_sddmm_spmm_f32(M, K, D, nnz, ro_d.p, ci_d.p, Q_d.p, K_d.p, V_d.p, scale, O_d.p, plan.p, plan.n | DLSPM_HINT_ROW_PLAN, stream);
-        return fused_sddmm_spmm_f32(M, K, D, nnz, ro_d.p, ci_d.p, Q_d.p, K_d.p, V_d.p, scale, O_d.p, wc.arg(ws.p),
-                                    wc.size(), stream);
+        return fused_sddmm_spmm_f32(M, K, D, nnz, ro_d.p, ci_d.p, Q_d.p, K_d.p, V_d.p, scale, O_d.p, pc.arg(), pc.size(), stream);
     });
     hipLaunchKernelGGL(check_row_of_slot_kernel, dim3(blocks_for(M)), dim3(256), 0, nullptr, M, ro_d.p, rowof_d.p);
     hipLaunchKernelGGL(check_sddmm_kernel, dim3(blocks_for(nnz)), dim3(256), 0, nullptr, nnz, D, rowof_d.p, ci_d.p, Q_d.p, K_d.p,

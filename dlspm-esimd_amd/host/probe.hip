@@ -1,4 +1,4 @@
-// libdlspm_probe.so: two measurement kernels for bench.py, behind a C ABI. Not part of libdlspm_hip and not used by it.
+// libdlspm_probe.so: measurement legs of bench.py, behind a C ABI. Not part of libdlspm_hip and not used by it.
 //   gather  what the device delivers for the access pattern the sparse kernels are made of -- whole waves fetching
 //           1 KiB dense rows at random (or consecutive) positions of a table -- so that kernel times can be judged
 //           against a measured ceiling instead of the HBM figure, which these cache-resident problems never touch.
@@ -7,9 +7,14 @@
 //           fit every XCD's L2 (B of the 2048 x 512 x 256 benchmark), 8192 rows = 8 MiB do not.
 //   copy    a plain float4 copy of known size: the kernel whose rocprofv3 FETCH_SIZE / WRITE_SIZE readings scale the
 //           counters of the other kernels.
+//   enqueue what a call of one of the three entry points costs the HOST when it is issued outside a graph, the way the
+//           reference times its kernels (20 single launches, SPMM/spmm-esimd-fromfile2.cpp:194-243): n calls through
+//           the function pointer, no synchronisation in between, wall time / n; and the same loop over an empty
+//           kernel, which is what the HIP runtime's launch alone costs.
 // The reference's nearest relative is the cache-flush copy kernel of SDDMM/tprint.cpp:65-72.
 #include <hip/hip_runtime.h>
 #include <stddef.h>
+#include <chrono>
 
 namespace {
 
@@ -52,9 +57,59 @@ __global__ __launch_bounds__(256) void dlspm_probe_copy_kernel(const float4* __r
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) dst[i] = src[i];
 }
 
+__global__ void dlspm_probe_empty_kernel(int) {}
+
+template <typename F> double per_call_us(int n, F&& call)
+{
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < n; ++i) call();
+    const auto t1 = std::chrono::steady_clock::now();
+    return std::chrono::duration<double, std::micro>(t1 - t0).count() / (n > 0 ? n : 1);
+}
+
 }  // namespace
 
 extern "C" {
+
+typedef int (*dlspm_probe_spmm_fn)(int, int, int, int, const int*, const int*, const float*, const float*, float*, void*,
+                                   size_t, void*);
+typedef int (*dlspm_probe_sddmm_fn)(int, int, int, int, const int*, const int*, const float*, const float*, float*, void*,
+                                    size_t, void*);
+typedef int (*dlspm_probe_fused_fn)(int, int, int, int, const int*, const int*, const float*, const float*, const float*,
+                                    float, float*, void*, size_t, void*);
+
+// Host microseconds per call of n calls of `fn` (spmm_csr_f32 or an entry point of its signature) issued back to back on
+// `stream` without synchronising; *status receives the last call's status. The caller synchronises afterwards.
+double dlspm_probe_enqueue_spmm(void* fn, int n, int M, int K, int N, int nnz, const int* ro, const int* ci, const float* va,
+                                const float* B, float* C, void* ws, size_t ws_bytes, void* stream, int* status)
+{
+    int st = 0;
+    const double us = per_call_us(n, [&] { st = ((dlspm_probe_spmm_fn)fn)(M, K, N, nnz, ro, ci, va, B, C, ws, ws_bytes, stream); });
+    if (status) *status = st;
+    return us;
+}
+double dlspm_probe_enqueue_sddmm(void* fn, int n, int M, int K, int D, int nnz, const int* ro, const int* ci, const float* lhs,
+                                 const float* rhs, float* out, void* ws, size_t ws_bytes, void* stream, int* status)
+{
+    int st = 0;
+    const double us = per_call_us(n, [&] { st = ((dlspm_probe_sddmm_fn)fn)(M, K, D, nnz, ro, ci, lhs, rhs, out, ws, ws_bytes, stream); });
+    if (status) *status = st;
+    return us;
+}
+double dlspm_probe_enqueue_fused(void* fn, int n, int M, int K, int D, int nnz, const int* ro, const int* ci, const float* Q,
+                                 const float* Km, const float* V, float scale, float* O, void* ws, size_t ws_bytes, void* stream,
+                                 int* status)
+{
+    int st = 0;
+    const double us = per_call_us(n, [&] { st = ((dlspm_probe_fused_fn)fn)(M, K, D, nnz, ro, ci, Q, Km, V, scale, O, ws, ws_bytes, stream); });
+    if (status) *status = st;
+    return us;
+}
+// the same loop over an empty kernel: the launch cost of the runtime by itself
+double dlspm_probe_enqueue_empty(int n, void* stream)
+{
+    return per_call_us(n, [&] { hipLaunchKernelGGL(dlspm_probe_empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), 0); });
+}
 
 // One launch: `blocks` workgroups of four waves, every wave gathers iters x 8 rows of 256 floats from `table`
 // ((rows_mask + 1) x 256 floats on the device). Returns the hipError_t of the launch as int (0 = ok).

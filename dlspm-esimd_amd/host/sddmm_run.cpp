@@ -39,16 +39,11 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     if (dlspm_csr_check(M, K, nnz, ro_d.p, ci_d.p, nullptr) != DLSPM_OK) throw std::invalid_argument("malformed CSR structure");
     DLSPM_HIP_CHECK(hipMemset(out_d.p, 0xFF, std::max(nnz, 1) * sizeof(float)));
 
-    // SDDMM needs memory only for the slice boundaries of the column-sliced schedule; otherwise the argument only
-    // carries what is known about the rows
-    const bool banded = s.kind == CaseSpec::kShape && s.band > 0 && s.band_random == 0;
-    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_SDDMM, M, K, D, nnz, ro_d.p, opt.plan, banded);
-    DevBuf<char> ws(wc.bytes);
-    if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
-    DevBuf<char> plan = wc.plan ? build_row_plan(M, ro_d.p) : DevBuf<char>(0);
+    // SDDMM needs memory only for the slice boundaries of the column-sliced schedule or for a plan; otherwise the
+    // argument only carries what dlspm_advise found out about the rows and columns
+    const PreparedCall pc = prepare_call(opt, DLSPM_OP_SDDMM, M, K, D, nnz, ro_d.p, ci_d.p);
     const Timing t = time_launches(opt, [&](hipStream_t stream) {
-        if (wc.plan) return sddmm_csr_f32(M, K, D, nnz, ro_d.p, ci_d.p, lhs_d.p, rhs_d.p, out_d.p, plan.p, plan.n | DLSPM_HINT_ROW_PLAN, stream);
-        return sddmm_csr_f32(M, K, D, nnz, ro_d.p, ci_d.p, lhs_d.p, rhs_d.p, out_d.p, wc.arg(ws.p), wc.size(), stream);
+        return sddmm_csr_f32(M, K, D, nnz, ro_d.p, ci_d.p, lhs_d.p, rhs_d.p, out_d.p, pc.arg(), pc.size(), stream);
     });
     hipLaunchKernelGGL(check_row_of_slot_kernel, dim3(blocks_for(M)), dim3(256), 0, nullptr, M, ro_d.p, rowof_d.p);
     hipLaunchKernelGGL(check_sddmm_kernel, dim3(blocks_for(nnz)), dim3(256), 0, nullptr, nnz, D, rowof_d.p, ci_d.p, lhs_d.p,

@@ -42,18 +42,11 @@ static bool run_case(const CaseSpec& s, const Options& opt)
     if (dlspm_csr_check(M, K, nnz, ro_d.p, ci_d.p, nullptr) != DLSPM_OK) throw std::invalid_argument("malformed CSR structure");
     DLSPM_HIP_CHECK(hipMemset(C_d.p, 0xFF, (size_t)M * N * sizeof(float)));  // NaN pattern: every element must be written
 
-    // the caller owns the workspace, as it owns every other buffer: 0 bytes for small problems
-    // uneven rows that are not short: a row plan, built once per matrix like the look at the row lengths, hands the
-    // rows out by length, one per workgroup (dlspm_row_plan_advice); otherwise what dlspm_workspace_advice says
-    const bool banded = s.kind == CaseSpec::kShape && s.band > 0 && s.band_random == 0;
-    const WorkspaceChoice wc = workspace_to_pass(opt, DLSPM_OP_SPMM, M, K, N, nnz, ro_d.p, opt.plan, banded);
-    DevBuf<char> ws(wc.bytes);
-    if (wc.bytes) std::printf("workspace: %zu bytes\n", wc.bytes);
-    const bool planned = wc.plan;
-    DevBuf<char> plan = planned ? build_row_plan(M, ro_d.p) : DevBuf<char>(0);
+    // the caller owns the workspace, as it owns every other buffer. Once per matrix: one look at it (dlspm_analyze) and
+    // the library's answer for this op and width (dlspm_advise) -- nothing, a hint, schedule memory, or a plan built here
+    const PreparedCall pc = prepare_call(opt, DLSPM_OP_SPMM, M, K, N, nnz, ro_d.p, ci_d.p);
     const Timing t = time_launches(opt, [&](hipStream_t stream) {
-        if (planned) return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, plan.p, plan.n | DLSPM_HINT_ROW_PLAN, stream);
-        return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, wc.arg(ws.p), wc.size(), stream);
+        return spmm_csr_f32(M, K, N, nnz, ro_d.p, ci_d.p, va_d.p, B_d.p, C_d.p, pc.arg(), pc.size(), stream);
     });
     hipLaunchKernelGGL(check_spmm_kernel, dim3(blocks_for((long long)M * N)), dim3(256), 0, nullptr, M, N, ro_d.p, ci_d.p,
                        va_d.p, B_d.p, Cref_d.p);

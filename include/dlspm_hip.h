@@ -60,6 +60,13 @@
  *         74 us with this hint; the L2s fetch 33 MiB per launch instead of 145 MiB. A wrong hint costs time (rows whose
  *         length depends on their position load the XCDs unevenly), never correctness: the bits are those of the call
  *         with NULL. May be combined with DLSPM_HINT_ROWS_EVEN; a row plan takes precedence.
+ *       DLSPM_HINT_CUT_PLAN: `workspace` holds a cut plan (dlspm_row_plan_build_cut, below).
+ *       DLSPM_HINT_ROWS_SKEWED, with a row plan: the caller knows that the longest row is at least twenty times the mean.
+ *         SDDMM and the fused op then run one row per workgroup in plan order also for masks of 16 to 64 rows per compute
+ *         unit (4096 < M <= 16384 on an MI355X), where the sizes alone would group several rows per workgroup (faster for
+ *         moderately uneven rows, 0.63-0.93 of the time for very uneven ones). Speed only; other sizes ignore it.
+ *     A bit of that byte that has no meaning, or a combination that has none (both kinds of plan, a plan of 2^48 bytes and
+ *     more, even and skewed rows at once), is refused with DLSPM_E_INVALID_ARG.
  * Calls on different streams may run concurrently from different host threads (each with its own
  * workspace). The library's only mutable state is per host thread (the tuning overrides of dlspm_set_tuning and the
  * last HIP error), a cache of the devices' properties, and the static scratch array of spmm_csr_f32_static.
@@ -86,6 +93,8 @@ extern "C" {
 #define DLSPM_HINT_ROWS_EVEN ((size_t)1 << 62)
 #define DLSPM_HINT_ROW_PLAN  ((size_t)1 << 61)
 #define DLSPM_HINT_BANDED    ((size_t)1 << 60)
+#define DLSPM_HINT_CUT_PLAN  ((size_t)1 << 59)
+#define DLSPM_HINT_ROWS_SKEWED ((size_t)1 << 58)
 #define DLSPM_HINT_MASK      ((size_t)0xFF << 56)
 
 /* Deprecated spelling of DLSPM_HINT_ROWS_EVEN, still accepted: this constant as `workspace` with workspace_bytes 0.
@@ -178,6 +187,52 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
                     void* stream);
 
 /*
+ * One look at the matrix, one answer. The compute calls see sizes only; how a matrix should be launched also depends on
+ * how uneven its rows are and on whether neighbouring rows gather neighbouring dense rows. These two calls hold every
+ * such rule in one place (the thresholds live in the library's code, once):
+ *   dlspm_analyze   one pass over the CSR structure on the device (synchronises `stream`; once per matrix structure, like
+ *                   dlspm_csr_check): the longest row, the rows without nonzeros, the widest row (largest - smallest
+ *                   column + 1), and, with the rows cut into eight contiguous eighths (the share of one XCD under
+ *                   DLSPM_HINT_BANDED): the columns that the eighths span, summed, in thousandths of K (1000: a band that
+ *                   moves down the columns with the row; 8000: every eighth reaches all columns), and the nonzeros of
+ *                   the heaviest eighth in thousandths of the mean eighth.
+ *   dlspm_advise    host only: for op (DLSPM_OP_*) at dense width N_or_D, what to allocate (`bytes` of device memory, 0:
+ *                   pass NULL), what to build into it (`build`: nothing, dlspm_row_plan_build or
+ *                   dlspm_row_plan_build_cut; nothing with bytes > 0: plain schedule memory, no initialisation), and
+ *                   the hint bits to or into workspace_bytes (`hints`). A band is detected, not hinted; very uneven rows
+ *                   in masks of 16 to 64 rows per compute unit get DLSPM_HINT_ROWS_SKEWED with their plan.
+ * Use:  dlspm_matrix_info mi; dlspm_call_plan cp;
+ *       dlspm_analyze(M, K, nnz, row_offsets, col_indices, stream, &mi);   dlspm_advise(DLSPM_OP_SPMM, N, &mi, &cp);
+ *       void* ws = NULL; if (cp.bytes) hipMalloc(&ws, cp.bytes);
+ *       if (cp.build == DLSPM_BUILD_ROW_PLAN) dlspm_row_plan_build(M, row_offsets, ws, cp.bytes, stream);
+ *       if (cp.build == DLSPM_BUILD_CUT_PLAN) dlspm_row_plan_build_cut(M, row_offsets, ws, cp.bytes, stream);
+ *       spmm_csr_f32(M, K, N, nnz, ..., ws, cp.bytes | cp.hints, stream);    // as often as the structure is used
+ * The finer-grained queries below (dlspm_csr_row_stats, dlspm_workspace_advice, dlspm_row_plan_advice,
+ * dlspm_describe_*) remain for callers that know their matrices and for tuning reports.
+ * No counterpart in the reference, whose launch sizing needs no knowledge of the matrix (SPMM/spmmesimd2.hpp:30-60) and
+ * takes the rows as they come.
+ */
+typedef struct dlspm_matrix_info {
+    int M, K, nnz;
+    int max_row_len;             /* longest row                                                               */
+    int empty_rows;              /* rows without nonzeros                                                     */
+    int max_col_span;            /* widest row: largest - smallest column index + 1                           */
+    int eighths_cover_permille;  /* sum over the eight eighths of the rows of the columns each spans, x 1000 / K */
+    int eighths_nnz_permille;    /* nonzeros of the heaviest eighth x 1000 / those of the mean eighth         */
+} dlspm_matrix_info;
+#define DLSPM_BUILD_NOTHING   0
+#define DLSPM_BUILD_ROW_PLAN  1
+#define DLSPM_BUILD_CUT_PLAN  2
+typedef struct dlspm_call_plan {
+    int build;     /* DLSPM_BUILD_*: what to build into the memory before the first launch */
+    size_t bytes;  /* device memory to pass as `workspace` (0: NULL)                       */
+    size_t hints;  /* DLSPM_HINT_* bits to or into `workspace_bytes`                       */
+} dlspm_call_plan;
+int dlspm_analyze(int M, int K, int nnz, const int* row_offsets, const int* col_indices, void* stream,
+                  dlspm_matrix_info* info);
+int dlspm_advise(int op, int N_or_D, const dlspm_matrix_info* info, dlspm_call_plan* plan);
+
+/*
  * Longest row and number of rows without nonzeros of a CSR structure that lives on the device (either result
  * pointer may be NULL). Synchronises `stream`; meant to be called once per matrix, like dlspm_csr_check. It
  * has no counterpart in the reference, whose launch sizing looks at M and N only
@@ -214,10 +269,38 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
  *                            than 4096 rows, 8192 at D >= 128 and 128 nonzeros per row) ignore the plan and run as
  *                            with NULL. A planned launch is one kernel (no memset, no allocation, no
  *                            synchronisation); the plan is only read, so launches may share it.
- *   *_planned                the same launches with the plan as a separate argument (plan == NULL: the plain call).
+ *   *_planned                DEPRECATED aliases: the same launches with the plan as a separate argument (plan == NULL: the
+ *                            plain call). New code passes the plan as the workspace with DLSPM_HINT_ROW_PLAN.
  * No counterpart in the reference, whose kernels take the rows in matrix order (SPMM/spmmesimd2.hpp:63-75).
  */
 size_t dlspm_row_plan_bytes(int M);
+/*
+ * Cut plan: a row plan that also cuts rows. A row that holds more than one and a half times a compute unit's share of
+ * the nonzeros (share = nnz / compute units) sets the time of the launch by itself, through the one compute unit it
+ * runs on, whatever the order of the rows. A cut plan hands such a row out as ceil(length / share) pieces to as many
+ * workgroups. SDDMM pieces write their own CSR slots (nothing else changes: same bits as any other schedule); SpMM and
+ * the fused op write one partial row per piece into memory that follows the plan, and a second small kernel adds the
+ * pieces of every cut row in piece order (no atomics, no fences: deterministic; rows that are not cut are summed as by
+ * the plain plan). The plan has room for the most pieces any matrix of M rows can need -- M + compute units entries --
+ * so its size and the launches' grids depend on M, the width and the device only, never on the matrix, and building it
+ * needs no look at the matrix from the host.
+ *   dlspm_row_plan_bytes_for(op, M, N_or_D)  bytes of DEVICE memory for the cut plan of a matrix of M rows and the
+ *                            partial rows of op at that dense width (SDDMM: none, the width is ignored). 0: no cut plan
+ *                            at this height (more than 2^20 rows).
+ *   dlspm_row_plan_build_cut builds it from row_offsets (device) into `plan` (device, 256-byte aligned) with kernels on
+ *                            `stream` only, like dlspm_row_plan_build (two launches up to 2048 - compute units rows).
+ *                            plan_bytes must be at least dlspm_row_plan_bytes_for(DLSPM_OP_SDDMM, M, 0); a plan that is
+ *                            to serve SpMM or the fused op must have been sized for that op and width.
+ *   the launches             the three compute entry points with workspace = plan and
+ *                            workspace_bytes = plan_bytes | DLSPM_HINT_CUT_PLAN (DLSPM_E_WORKSPACE below
+ *                            dlspm_row_plan_bytes_for(op, M, width)). SpMM and the fused op write the partial rows
+ *                            behind the plan: launches that share a cut plan must not overlap in time. Sizes a planned
+ *                            launch is not built for run as with NULL. SpMM and fused: two kernels per launch.
+ * dlspm_row_plan_advice returns 2 where it expects the cut plan to beat the plain one.
+ * No counterpart in the reference (one hardware thread per row or row slice, SPMM/spmmesimd2.hpp:63-75).
+ */
+size_t dlspm_row_plan_bytes_for(int op, int M, int N_or_D);
+int dlspm_row_plan_build_cut(int M, const int* row_offsets, void* plan, size_t plan_bytes, void* stream);
 /* 1 if a row plan is worth building for op (DLSPM_OP_*) at these sizes and this longest row (-1: unknown): the planned
  * launch would use it (one column tile, rows of at least 32 nonzeros on average where the size rule would group rows;
  * SDDMM and the fused op: 16 < D <= 512, up to 2048 rows also shorter rows), the rows are not known to be even (SDDMM
@@ -305,6 +388,9 @@ typedef struct dlspm_tuning {
                           /* (DLSPM_HINT_BANDED asks for the same per call.)                                          */
     int stream_results;   /* results stored with the non-temporal hint: -1 the size rule (dense result rows from one   */
                           /* L2's worth on, SDDMM results from one and a half), 0 never, 1 always                      */
+    int cut_piece_pct;    /* cut plans: the longest piece, in per cent of a share (nnz / compute units); 0 = the rule, 100 */
+    int cut_longest_pct;  /* ... and the longest row that stays whole; 0 = the rule, 150. Both 10 ... 1000; they enter the  */
+                          /* size of a cut plan, so set them before dlspm_row_plan_bytes_for and keep them for the launches */
 } dlspm_tuning;
 void dlspm_tuning_default(dlspm_tuning* t);   /* fills *t with "follow the rules" */
 int dlspm_set_tuning(const dlspm_tuning* t);  /* DLSPM_OK or DLSPM_E_INVALID_ARG (a field out of range) */

@@ -396,4 +396,67 @@ void model_row_plan(int M, const int* ro, int bins, int order, int* plan)
     }
 }
 
+// Host model of the cut rule of a cut plan (plan_cut_kernel): with share = max(1, ceil(nnz / bins)), piece_max =
+// ceil(share x piece_pct / 100) and longest = max(piece_max, ceil(share x longest_pct / 100)), a row of more than
+// `longest` nonzeros becomes c = ceil(length / piece_max) pieces of ceil(length / c) nonzeros each (the last one what
+// is left); the rows and pieces in matrix order are the "virtual rows" 0 .. used-1 of `entries` = M + extra, extra =
+// ceil(bins x 100 / piece_pct); the others hold nothing. v_off[entries + 1], v_row[entries] (-1: nothing),
+// v_slot[entries] (-1 a whole row, s >= 0 piece number s among all pieces in matrix order, -2 nothing); cut[0] = cut
+// rows, cut[1] = share, cut[2] = used, cut[3] = 0, then max_cut = ceil(bins x 100 / longest_pct) records of four ints
+// (row, first slot, pieces, 1; records beyond cut[0] are zeros). Returns 0, or 1 if a bound that the plan's size relies
+// on does not hold (more than entries virtual rows, extra + max_cut pieces or max_cut cut rows).
+int model_cut_rows(int M, const int* ro, int bins, int piece_pct, int longest_pct, int* v_off, int* v_row, int* v_slot, int* cut)
+{
+    const int extra = (bins * 100 + piece_pct - 1) / piece_pct, max_cut = (bins * 100 + longest_pct - 1) / longest_pct;
+    const int entries = M + extra, slots = extra + max_cut;
+    long long nnz = 0;
+    for (int i = 0; i < M; ++i) nnz += std::max(ro[i + 1] - ro[i], 0);
+    const long long share = std::max((nnz + bins - 1) / bins, 1ll);
+    const long long piece_max = std::max((share * piece_pct + 99) / 100, 1ll);
+    const long long longest_whole = std::max((share * longest_pct + 99) / 100, piece_max);
+    int e = 0, s = 0, j = 0;
+    for (int i = 0; i < M; ++i) {
+        const int len = std::max(ro[i + 1] - ro[i], 0);
+        if (len <= longest_whole) {
+            if (e >= entries) return 1;
+            v_off[e] = ro[i]; v_row[e] = i; v_slot[e] = -1;
+            ++e;
+            continue;
+        }
+        const int c = (int)((len + piece_max - 1) / piece_max), piece = (len + c - 1) / c;
+        if (e + c > entries || s + c > slots || j >= max_cut) return 1;
+        cut[4 + 4 * j] = i; cut[4 + 4 * j + 1] = s; cut[4 + 4 * j + 2] = c; cut[4 + 4 * j + 3] = 1;
+        for (int k = 0; k < c; ++k) {
+            v_off[e] = ro[i] + std::min(len, k * piece); v_row[e] = i; v_slot[e] = s;
+            ++e; ++s;
+        }
+        ++j;
+    }
+    cut[0] = j; cut[1] = (int)share; cut[2] = e; cut[3] = 0;
+    for (; j < max_cut; ++j) cut[4 + 4 * j] = cut[4 + 4 * j + 1] = cut[4 + 4 * j + 2] = cut[4 + 4 * j + 3] = 0;
+    for (; e <= entries; ++e) {
+        v_off[e] = ro[M];
+        if (e < entries) { v_row[e] = -1; v_slot[e] = -2; }
+    }
+    return 0;
+}
+
+// The cut plan that dlspm_row_plan_build_cut builds: the row plan (model_row_plan) of the virtual rows, each entry then
+// naming its matrix row and its slot. plan[4 x entries]: first nonzero, end, row, slot.
+int model_row_plan_cut(int M, const int* ro, int bins, int piece_pct, int longest_pct, int order, int* plan, int* cut)
+{
+    const int entries = M + (bins * 100 + piece_pct - 1) / piece_pct;
+    std::vector<int> v_off((size_t)entries + 1), v_row((size_t)entries), v_slot((size_t)entries), vp((size_t)3 * entries);
+    if (model_cut_rows(M, ro, bins, piece_pct, longest_pct, v_off.data(), v_row.data(), v_slot.data(), cut)) return 1;
+    model_row_plan(entries, v_off.data(), bins, order, vp.data());
+    for (int p = 0; p < entries; ++p) {
+        const int v = vp[2 * (size_t)entries + p];
+        plan[p] = vp[p];
+        plan[(size_t)entries + p] = vp[(size_t)entries + p];
+        plan[2 * (size_t)entries + p] = v_row[v];
+        plan[3 * (size_t)entries + p] = v_slot[v];
+    }
+    return 0;
+}
+
 }  // extern "C"

@@ -280,7 +280,8 @@ def test_tuning_overrides_go_through_one_call_and_the_environment_is_read_once(d
 
     base = dl.get_tuning()
     assert base == {"split_w": 0, "split_r": 0, "flat": -1, "flat_chunk": 0, "slices": -1, "tile_major": -1,
-                    "tile_width": 0, "plan_order": 0, "xcd_contiguous": 0, "stream_results": -1}
+                    "tile_width": 0, "plan_order": 0, "xcd_contiguous": 0, "stream_results": -1, "cut_piece_pct": 0,
+                    "cut_longest_pct": 0}
     sizes = (dl.OP_SPMM, 8192, 4096, 128, 8192 * 600)
     rule = dl.describe_launch(*sizes)
     assert (rule["W"], rule["R"]) == (4, 1)
@@ -353,6 +354,27 @@ def test_device_info_and_hints_without_a_gpu(dl):
     assert L.spmm_csr_f32(0, 5, 5, 0, None, None, None, None, None, None, dl.HINT_ROWS_EVEN, None) == dl.OK
     assert L.spmm_csr_f32_planned(2, 2, 2, 1, bogus, bogus, bogus, bogus, bogus, bogus, 24 | dl.HINT_ROWS_EVEN, None) == dl.E_INVALID_ARG
     assert dl.row_plan_bytes(2048) == 3 * 2048 * 4 and dl.row_plan_bytes(2049) == 3 * 2049 * 4 + 4 + 2 * 2049 * 8
+    # Bits of the hint byte that mean nothing are refused, so a "plenty of scratch" size such as SIZE_MAX cannot turn
+    # scratch memory into a row plan; so are a plan of 2^48 bytes and more, both kinds of plan at once, and the
+    # deprecated pointer constant together with a size.
+    size_max = (1 << 64) - 1
+    spmm = lambda ws, size: L.spmm_csr_f32(2, 2, 2, 1, bogus, bogus, bogus, bogus, bogus, ws, size, None)
+    sddmm = lambda ws, size: L.sddmm_csr_f32(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, ws, size, None)
+    fused = lambda ws, size: L.fused_sddmm_spmm_f32(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, 1.0, bogus, ws, size, None)
+    for call in (spmm, sddmm, fused):
+        assert call(bogus, size_max) == dl.E_INVALID_ARG
+        assert call(bogus, 4096 | (1 << 63)) == dl.E_INVALID_ARG
+        assert call(bogus, 4096 | (1 << 57)) == dl.E_INVALID_ARG
+        assert call(None, dl.HINT_ROWS_EVEN | dl.HINT_ROWS_SKEWED) == dl.E_INVALID_ARG
+        assert call(bogus, (1 << 48) | dl.HINT_ROW_PLAN) == dl.E_INVALID_ARG
+        assert call(bogus, 4096 | dl.HINT_ROW_PLAN | dl.HINT_CUT_PLAN) == dl.E_INVALID_ARG
+        assert call(ctypes.c_void_p(1), 4096) == dl.E_INVALID_ARG
+        assert call(bogus, 23 | dl.HINT_CUT_PLAN) in (dl.E_WORKSPACE, dl.E_NO_DEVICE)
+    # cut plans: argument checks come before anything touches the device
+    assert L.dlspm_row_plan_build_cut(-1, bogus, bogus, 0, None) == dl.E_INVALID_ARG
+    assert L.dlspm_row_plan_build_cut((1 << 20) + 1, bogus, bogus, 1 << 40, None) == dl.E_INVALID_ARG
+    assert L.dlspm_row_plan_build_cut(8, None, bogus, 1 << 20, None) == dl.E_INVALID_ARG
+    assert L.dlspm_row_plan_build_cut(0, None, None, 0, None) == dl.OK
 
 
 def test_library_exports_every_declared_symbol(dl):
