@@ -575,6 +575,10 @@ static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int n
 {
     if (max_row_len <= 0 || M > kCutPlanAdviceMaxRows) return false;
     const long long cus = dev.cus;
+    // SpMM and the fused op: only where a share holds at least two mean rows, so that the rows above one and a half
+    // shares are the exception and the kernel that adds their pieces has little to do (the reference's layers of 64 ...
+    // 256 rows, where most rows would be cut: 0.85 ... 1.5 times the time of the plan over whole rows; 512 rows: 0.66 ... 1.0)
+    if (op != DLSPM_OP_SDDMM && M < 2 * cus) return false;
     const long long share = std::max<long long>(ceil_div(nnz, cus), 1);
     const long long longest_whole = (share * kCutLongestPct + 99) / 100;
     if (max_row_len <= longest_whole) return false;
@@ -599,7 +603,11 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
         if (!spmm_plan_applies(dev, shape, M, N_or_D, nnz)) return 0;
     } else if (op == DLSPM_OP_SDDMM) {
         SddmmShape shape = sddmm_choose(dev, M, N_or_D, nnz, vec4);
-        if (!sddmm_plan_applies(dev, shape, M, N_or_D, nnz, rows_are_skewed(M, nnz, max_row_len))) return 0;
+        if (!sddmm_plan_applies(dev, shape, M, N_or_D, nnz, rows_are_skewed(M, nnz, max_row_len))) {
+            // fewer rows than compute units: only a cut plan helps (its pieces fill the device)
+            SddmmShape few = sddmm_choose(dev, M, N_or_D, nnz, vec4);
+            return sddmm_cut_plan_applies(dev, few, M, N_or_D, nnz) && cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len) ? 2 : 0;
+        }
     } else if (op == DLSPM_OP_FUSED) {
         FusedShape shape = fused_choose(dev, M, N_or_D, nnz, vec4);
         if (!fused_plan_applies(dev, shape, M, N_or_D, nnz, rows_are_skewed(M, nnz, max_row_len))) return 0;
@@ -679,7 +687,7 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
         const CutPlan cp = cut_plan_layout(M, 0, dev.cus);
         if (cp.bytes == 0 || ws.bytes < cp.bytes) return DLSPM_E_WORKSPACE;
         SddmmShape shape = sddmm_choose(dev, M, D, nnz, vec4);
-        if (sddmm_plan_applies(dev, shape, M, D, nnz)) {
+        if (sddmm_cut_plan_applies(dev, shape, M, D, nnz)) {
             const hipError_t e = sddmm_pieces_launch(args, shape, cp, ws.mem, st);
             return e == hipSuccess ? DLSPM_OK : fail_hip(e);
         }

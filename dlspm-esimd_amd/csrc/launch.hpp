@@ -198,6 +198,7 @@ hipError_t spmm_pieces_launch(const SpmmArgs& x, const SpmmShape& s, const CutPl
 // skewed (DLSPM_HINT_ROWS_SKEWED): the caller knows that the longest row is at least twenty times the mean
 bool plan_ungroups_skewed(const DeviceInfo& dev, int M, int nnz);
 bool sddmm_plan_applies(const DeviceInfo& dev, SddmmShape& s, int M, int D, int nnz, bool skewed = false);
+bool sddmm_cut_plan_applies(const DeviceInfo& dev, SddmmShape& s, int M, int D, int nnz);  // also few rows of eight waves each
 hipError_t sddmm_planned_launch(const SddmmArgs& x, const SddmmShape& s, const int* plan, hipStream_t stream);
 bool fused_plan_applies(const DeviceInfo& dev, FusedShape& s, int M, int D, int nnz, bool skewed = false);
 hipError_t fused_planned_launch(const FusedArgs& x, const FusedShape& s, const int* plan, hipStream_t stream);

@@ -180,6 +180,14 @@ def test_cut_plan_sizes_and_advice(dl):
     assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 256, 52000, -1) == 1     # unknown rows: never a cut plan
     assert dl.row_plan_advice(dl.OP_SPMM, 2048, 512, 256, 105687, 312) == 1   # the headline matrix: below one share
     assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 256, 52000, 110) == 0    # even rows: no plan at all
+    # fewer rows than compute units (eight waves per row by the size rule): SDDMM takes a cut plan, whose pieces fill the
+    # device at no cost; SpMM and the fused op, which would cut most rows and pay for adding the pieces, do not
+    assert dl.describe_launch(dl.OP_SDDMM, 128, 1152, 128, 29510)["W"] == 8
+    assert dl.row_plan_advice(dl.OP_SDDMM, 128, 1152, 128, 29510, 455) == 2
+    assert dl.row_plan_advice(dl.OP_SDDMM, 64, 576, 128, 31919, 547) == 2
+    assert dl.row_plan_advice(dl.OP_SDDMM, 256, 2304, 128, 118041, 900) == 0   # 256 rows: as many as compute units
+    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 256, 29510, 455) in (0, 1)
+    assert dl.row_plan_advice(dl.OP_FUSED, 128, 1152, 64, 29510, 455) in (0, 1)
 
 
 def load_smtx(path):

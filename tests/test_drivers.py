@@ -426,17 +426,28 @@ def test_spmm_driver_builds_a_row_plan_for_small_uneven_matrices():
 @pytest.mark.gpu
 def test_verify_dlmc_script_on_the_fixtures(tmp_path):
     """tests/verify_dlmc.py is the wide form of the fixture tests above (any directory of .smtx files, every schedule,
-    all three ops against the oracle); here it runs over the fifteen fixtures, with a batch-size table for SpMM."""
+    all three ops against the oracle); here it runs over the eighteen fixtures, with a batch-size table for SpMM, and once
+    more the way a driver would call (dlspm_analyze -> dlspm_advise), from a pack of the same patterns, with timing."""
     table = tmp_path / "batchsizes.txt"
     names = sorted(f[:-5] for f in os.listdir(DLMC) if f.endswith(".smtx"))
-    table.write_text("".join(f"{n},{w}\n" for n, w in zip(names, [49, 196, 64, 256, 33] * 3)))
+    table.write_text("".join(f"{n},{w}\n" for n, w in zip(names, [49, 196, 64, 256, 33] * 4)))
     report = tmp_path / "report.txt"
     r = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "verify_dlmc.py"), DLMC, "--batch-table", str(table),
                         "--all-schedules", "--report", str(report)], capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
     assert "verify_dlmc PASS" in r.stdout and " 0 FAIL" in r.stdout
     lines = report.read_text().splitlines()
-    assert len(lines) >= 15 * 3 * 3 and all(line.startswith("PASS ") for line in lines)
+    assert len(lines) >= 18 * 3 * 3 and all(line.startswith("PASS ") for line in lines)
+    assert any(" cut_plan " in line for line in lines)
+    pack = tmp_path / "patterns.npz"
+    subprocess.run([sys.executable, os.path.join(DLMC, "pack_patterns.py"), DLMC, str(pack), "--min-nnz", "20000"], check=True)
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "verify_dlmc.py"), str(pack), "--time", "--report", str(report)],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    assert "verify_dlmc PASS" in r.stdout and "geometric means" in r.stdout
+    lines = report.read_text().splitlines()   # the four patterns of 20 000 nonzeros and more: three of them with a very long row
+    assert len(lines) == 4 * 3 and all(line.startswith("PASS ") and " us=" in line for line in lines)
+    assert sum(" cut_plan " in line for line in lines) >= 4
 
 
 @pytest.mark.gpu

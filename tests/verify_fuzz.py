@@ -87,7 +87,7 @@ def main():
         dl.set_tuning(**tuning)
         ro_d, ci_d = torch.from_numpy(ro).cuda(), torch.from_numpy(ci).cuda()
         for op in ("spmm", "sddmm", "fused"):
-            for schedule, err, intact in check_pattern(dl, torch, oracle, op, M, K, N, ro, ci, ro_d, ci_d, rng, True):
+            for schedule, err, intact, _, _ in check_pattern(dl, torch, oracle, op, M, K, N, ro, ci, ro_d, ci_d, rng, True):
                 tally.add(op, schedule, what, err, intact)
         dl.set_tuning()
     print(f"{time.time() - t0:.0f} s")

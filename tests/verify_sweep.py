@@ -62,7 +62,7 @@ def main():
                     if op == "fused" and M > args.fused_max_m:
                         continue
                     what = f"M={M} K={K} N={N} density={density} nnz={ci.size}"
-                    for schedule, err, intact in check_pattern(dl, torch, oracle, op, M, K, N, ro, ci, ro_d, ci_d, rng, args.all_schedules):
+                    for schedule, err, intact, _, _ in check_pattern(dl, torch, oracle, op, M, K, N, ro, ci, ro_d, ci_d, rng, args.all_schedules):
                         tally.add(op, schedule, what, err, intact)
                 print(f"  {M} x {K}, N = {N}, density {density}: {tally.cases} cases, {tally.failures} failures, {time.time() - t0:.0f} s",
                       flush=True)
