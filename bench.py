@@ -146,6 +146,7 @@ def time_steps(torch, step, steps, warmup, replays, use_graph, split_overhead=Fa
     medians is K steps without what one replay costs by itself ('steady_per_step_s', 'replay_overhead_s'): reported
     beside the K-step figure, never instead of it."""
     stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())  # what was enqueued so far (uploads, a plan build) comes first
     extra = {}
     with torch.cuda.stream(stream):
         for _ in range(warmup):
@@ -172,6 +173,7 @@ def cold_launch_us(torch, step, pairs=24, replays=5):
     node would not do), and 1 GiB is four times the 256 MiB Infinity Cache."""
     scratch = torch.empty(256 * 1024 * 1024, dtype=torch.float32, device="cuda")
     stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(stream):
         scratch.fill_(0.0)
         step()

@@ -54,6 +54,7 @@ static Tuning tuning_from_environment()
     number("DLSPM_STREAM_RESULTS", t.stream_results);
     number("DLSPM_CUT_PIECE_PCT", t.cut_piece_pct);
     number("DLSPM_CUT_LONGEST_PCT", t.cut_longest_pct);
+    number("DLSPM_RULES_OFF", t.rules_off);
     return t;
 }
 static const Tuning& process_tuning()
@@ -237,14 +238,10 @@ SlicePlan slice_plan(const DeviceInfo& dev, int M, int K, int width, int nnz, in
 
 void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, const SplitRule& rule, bool rows_even, int& W, int& R)
 {
-    static const int kPairs[][2] = {{4, 16}, {4, 8}, {4, 4}, {4, 2}, {4, 1}, {8, 4}, {8, 2}, {8, 1}, {16, 1}};
-    if (tuning().split_w > 0) {
-        for (const auto& pr : kPairs)
-            if (pr[0] == tuning().split_w && pr[1] == tuning().split_r && pr[0] <= rule.max_w) {
-                W = pr[0];
-                R = pr[1];
-                return;
-            }
+    if (tuning().split_w > 0 && split_is_built(tuning().split_w, tuning().split_r, rule.max_w)) {  // (else: ignored)
+        W = tuning().split_w;
+        R = tuning().split_r;
+        return;
     }
     const long long cus = dev.cus;  // the thresholds below were measured on 256 compute units and scale with them
     // Measured on MI355X over the benchmark configurations and the 12 x {32,128} x {0.3,0.2,0.1} sweep grid:
@@ -259,20 +256,20 @@ void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, co
     // only add to the partial sums behind the barrier.
     const double avg = M > 0 ? (double)nnz / M : 0.0;
     const long long work_rows = (long long)M * col_tiles;
-    W = rule.w8_few_rows_avg > 0 && work_rows < 2 * cus && avg >= rule.w8_few_rows_avg ? 8 : 4;
+    W = rule.w8_few_rows_avg > 0 && work_rows < 2 * cus && avg >= rule.w8_few_rows_avg && rule_on(kRuleEightWavesFewRows) ? 8 : 4;
     // very long rows in a tall matrix: sixteen waves per row gain 5-8 % in SpMM (24576 and 32768 rows of ~2000
     // nonzeros); with 8192 rows they lose as much, and the fused kernel loses 25-50 % with them at any height
-    if (rule.w16_long_rows && avg >= 1536.0 && work_rows >= 64 * cus) W = 16;
+    if (rule.w16_long_rows && avg >= 1536.0 && work_rows >= 64 * cus && rule_on(kRuleSixteenWavesTallLongRows)) W = 16;
     // few rows, each long (pruned ResNet-50 layers at small batch): four waves per row leave the device with a
     // couple of waves per SIMD, each walking hundreds of steps in sequence (measured 15-25 % slower); a step
     // takes `slots` nonzeros of the row at once
     const double steps = avg / (rule.slots > 0 ? rule.slots : 1);
-    if (work_rows < 4 * cus && steps >= 768.0) W = 16;
-    else if (work_rows < 4 * cus && steps >= 384.0 && W < 8) W = 8;
+    if (work_rows < 4 * cus && steps >= 768.0 && rule_on(kRuleMoreWavesFewLongRows)) W = 16;
+    else if (work_rows < 4 * cus && steps >= 384.0 && W < 8 && rule_on(kRuleMoreWavesFewLongRows)) W = 8;
     if (W > rule.max_w) W = rule.max_w;
     R = 1;
     if (W == 4) {
-        for (int r = 2; r <= 16; r *= 2) {
+        for (int r = 2; r <= 16 && rule_on(kRuleGroupRows); r *= 2) {
             const long long blocks = ceil_div(M, r) * col_tiles;
             if (blocks < rule.blocks_per_cu * cus || avg * r > 512.0) break;
             R = r;
@@ -293,6 +290,7 @@ void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, co
 constexpr int kCutPlanAdviceMaxRows = 16384;     // the cut rule is one workgroup's work: 16 rounds of 1024 rows
 constexpr double kCutPlanMinGainNs = 2500.0;      // SpMM, fused: the kernel that adds the pieces must be paid for
 constexpr double kCutPlanMinGainNsSddmm = 300.0;  // SDDMM: no second kernel
+constexpr double kCutPlanMinGainNsSddmmOneRowEach = 1000.0;  // ... one to two rows per compute unit: eight waves per row do nearly as well
 
 // longest row and number of rows without nonzeros (dlspm_csr_row_stats); stats[0] = max, stats[1] = empty rows
 __global__ void row_stats_kernel(int M, const int* __restrict__ row_offsets, int* __restrict__ stats)
@@ -378,7 +376,7 @@ void dlspm_tuning_default(dlspm_tuning* t)
     if (!t) return;
     const Tuning d;
     *t = dlspm_tuning{d.split_w, d.split_r, d.flat, d.flat_chunk, d.slices, d.tile_major, d.tile_width, d.plan_order,
-                      d.xcd_contiguous, d.stream_results, d.cut_piece_pct, d.cut_longest_pct};
+                      d.xcd_contiguous, d.stream_results, d.cut_piece_pct, d.cut_longest_pct, d.rules_off};
 }
 
 int dlspm_set_tuning(const dlspm_tuning* t)
@@ -391,7 +389,7 @@ int dlspm_set_tuning(const dlspm_tuning* t)
         t->tile_major < -1 || t->tile_major > 1 || t->tile_width < 0 || t->plan_order < 0 || t->plan_order > 2 ||
         t->xcd_contiguous < 0 || t->xcd_contiguous > 1 || t->stream_results < -1 || t->stream_results > 1 ||
         (t->cut_piece_pct != 0 && (t->cut_piece_pct < 10 || t->cut_piece_pct > 1000)) ||
-        (t->cut_longest_pct != 0 && (t->cut_longest_pct < 10 || t->cut_longest_pct > 1000)))
+        (t->cut_longest_pct != 0 && (t->cut_longest_pct < 10 || t->cut_longest_pct > 1000)) || t->rules_off < 0 || t->rules_off > 127)
         return DLSPM_E_INVALID_ARG;
     t_tuning.split_w = t->split_w;
     t_tuning.split_r = t->split_r;
@@ -405,6 +403,7 @@ int dlspm_set_tuning(const dlspm_tuning* t)
     t_tuning.stream_results = t->stream_results;
     t_tuning.cut_piece_pct = t->cut_piece_pct;
     t_tuning.cut_longest_pct = t->cut_longest_pct;
+    t_tuning.rules_off = t->rules_off;
     t_tuning_set = true;
     return DLSPM_OK;
 }
@@ -414,7 +413,7 @@ int dlspm_get_tuning(dlspm_tuning* t)
     if (!t) return DLSPM_E_INVALID_ARG;
     const Tuning& c = tuning();
     *t = dlspm_tuning{c.split_w, c.split_r, c.flat, c.flat_chunk, c.slices, c.tile_major, c.tile_width, c.plan_order,
-                      c.xcd_contiguous, c.stream_results, c.cut_piece_pct, c.cut_longest_pct};
+                      c.xcd_contiguous, c.stream_results, c.cut_piece_pct, c.cut_longest_pct, c.rules_off};
     return DLSPM_OK;
 }
 
@@ -584,7 +583,8 @@ static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int n
     if (max_row_len <= longest_whole) return false;
     const double bytes_per_nonzero = (op == DLSPM_OP_FUSED ? 2.0 : 1.0) * (double)std::min(width, 512) * sizeof(float);
     const double saved_ns = (double)(max_row_len - longest_whole) * bytes_per_nonzero / 115.0;
-    return saved_ns >= (op == DLSPM_OP_SDDMM ? kCutPlanMinGainNsSddmm : kCutPlanMinGainNs);
+    if (op == DLSPM_OP_SDDMM) return saved_ns >= (M >= cus && M < 2 * cus ? kCutPlanMinGainNsSddmmOneRowEach : kCutPlanMinGainNsSddmm);
+    return saved_ns >= kCutPlanMinGainNs;
 }
 
 // the longest row at least twenty times the mean: what DLSPM_HINT_ROWS_SKEWED says
@@ -712,7 +712,9 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
             return es == hipSuccess ? DLSPM_OK : fail_hip(es);
         }
     }
-    const FlatPlan plan = ws.banded ? FlatPlan{0, 0, 0} : sddmm_flat_plan(dev, M, nnz, D);
+    // (rows known to be even have nothing to gain from the flat schedule, which costs them 4 ... 12 % today: the reference's
+    // grid at density 0.1, 12288 ... 32768 rows of 410 ... 819 nonzeros, D = 32 and 128)
+    const FlatPlan plan = ws.banded || ws.rows_even ? FlatPlan{0, 0, 0} : sddmm_flat_plan(dev, M, nnz, D);
     const hipError_t e = plan.chunk > 0 ? sddmm_flat_launch(args, shape, plan.chunk, st) : sddmm_launch(args, shape, st);
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }
@@ -864,7 +866,7 @@ int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int pa
     } else if (op == DLSPM_OP_SDDMM) {
         const SddmmShape s = sddmm_choose(dev, M, n, nnz, vec4, even);
         shape[0] = s.vec; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R; shape[7] = 1;
-        const FlatPlan fp = sddmm_flat_plan(dev, M, nnz, n);
+        const FlatPlan fp = even ? FlatPlan{0, 0, 0} : sddmm_flat_plan(dev, M, nnz, n);  // as sddmm_csr_f32 decides
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_FUSED) {
         const FusedShape s = fused_choose(dev, M, n, nnz, vec4, even);

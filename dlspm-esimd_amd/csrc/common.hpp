@@ -333,7 +333,7 @@ struct RowBlock {
         T = off(nr) - T0;
         per = split_per_wave(T, W);
         auto o = [&](int i) { return off(i); };
-        aligned = split_is_row_aligned<W, R>(o, nr, per);
+        aligned = (flags & 8) == 0 && split_is_row_aligned<W, R>(o, nr, per);  // (bit 3: the rule is switched off for a measurement)
         int a_, b_;
         wave_range<W, R>(aligned, o, nr, w, T0, T, per, a_, b_);
         a = __builtin_amdgcn_readfirstlane(a_);

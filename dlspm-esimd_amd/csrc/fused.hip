@@ -151,7 +151,7 @@ static hipError_t launch_one(const FusedArgs& x, hipStream_t stream)
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     if constexpr (DS > 0) {
-        if (x.D == G1 * VEC * DS) {
+        if (x.D == G1 * VEC * DS && rule_on(kRuleExactWidthKernels)) {
             hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, false, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64),
                                0, stream, x.M, x.D, col_tiles, launch_flags(x.xcd_contiguous), x.scale, x.row_offsets, x.col_indices,
                                x.Q, x.Kmat, x.V, x.O);
@@ -164,25 +164,14 @@ static hipError_t launch_one(const FusedArgs& x, hipStream_t stream)
     return hipGetLastError();
 }
 
-template <int VEC, int G1, int DS, int G, int V2>
-static hipError_t launch_wr(const FusedArgs& x, int W, int R, hipStream_t stream)
+// the layout of shape s among FusedLayouts
+template <typename Launch> static hipError_t dispatch_layout(const FusedShape& s, Launch&& launch)
 {
-#define DLSPM_WR(w_, r_) \
-    if (W == w_ && R == r_) return launch_one<VEC, G1, DS, G, V2, w_, r_>(x, stream);
-    DLSPM_WR(4, 16)
-    DLSPM_WR(4, 8)
-    DLSPM_WR(4, 4)
-    DLSPM_WR(4, 2)
-    DLSPM_WR(4, 1)
-    if constexpr (G * VEC * V2 < 1024) {  // wider tiles: the per-wave partial sums of 8 or 16 waves do not fit in LDS
-        DLSPM_WR(8, 4)
-        DLSPM_WR(8, 2)
-        DLSPM_WR(8, 1)
-        DLSPM_WR(16, 1)
-    }
-#undef DLSPM_WR
-    return hipErrorInvalidValue;
+    return dispatch<FusedLayouts>(
+        [&](auto l) { return l.VEC == s.vec && l.G1 == s.G1 && l.DS == s.DS && l.G == s.G && l.V == s.V; }, launch);
 }
+// the layouts the column-sliced and planned kernels are built for: 16 < D <= 512 in one column tile
+template <typename L> constexpr bool kOneTileLayout = L::VEC == 4 && L::G1 == 8 && L::DS >= 1;
 
 FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even)
 {
@@ -210,18 +199,15 @@ FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
 
 hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream)
 {
-    if (s.vec == 4) {
-        if (s.G1 == 4 && s.DS == 1 && s.G == 8 && s.V == 1) return launch_wr<4, 4, 1, 8, 1>(x, s.W, s.R, stream);
-        if (s.G1 == 8 && s.DS == 1 && s.G == 8 && s.V == 1) return launch_wr<4, 8, 1, 8, 1>(x, s.W, s.R, stream);
-        if (s.G1 == 8 && s.DS == 2 && s.G == 16 && s.V == 1) return launch_wr<4, 8, 2, 16, 1>(x, s.W, s.R, stream);
-        if (s.G1 == 8 && s.DS == 4 && s.G == 32 && s.V == 1) return launch_wr<4, 8, 4, 32, 1>(x, s.W, s.R, stream);
-        if (s.G1 == 8 && s.DS == 8 && s.G == 64 && s.V == 1) return launch_wr<4, 8, 8, 64, 1>(x, s.W, s.R, stream);
-        if (s.G1 == 8 && s.DS == 16 && s.G == 64 && s.V == 2) return launch_wr<4, 8, 16, 64, 2>(x, s.W, s.R, stream);
-        if (s.G1 == 8 && s.DS == 0 && s.G == 64 && s.V == 4) return launch_wr<4, 8, 0, 64, 4>(x, s.W, s.R, stream);
-    } else if (s.G1 == 4 && s.DS == 1 && s.G == 8 && s.V == 1) {
-        return launch_wr<1, 4, 1, 8, 1>(x, s.W, s.R, stream);
-    }
-    return hipErrorInvalidValue;
+    return dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        return dispatch_split(s.W, s.R, [&](auto split) {
+            using S = decltype(split);
+            // column tiles of 1024: the per-wave partial sums of 8 or 16 waves do not fit in LDS
+            if constexpr (S::W > 4 && L::G * L::VEC * L::V >= 1024) return hipErrorInvalidValue;
+            else return launch_one<L::VEC, L::G1, L::DS, L::G, L::V, S::W, S::R>(x, stream);
+        });
+    });
 }
 
 // ---- flat schedule (see spmm.hip): every wave owns `chunk` consecutive nonzeros of the mask ------------------------
@@ -317,18 +303,10 @@ static hipError_t launch_flat(const FusedArgs& x, const FlatPlan& plan, float* p
 hipError_t fused_flat_launch(const FusedArgs& x, const FusedShape& s, const FlatPlan& plan, float* partial,
                              hipStream_t stream)
 {
-    if (s.vec == 4) {
-        if (s.G1 == 4 && s.DS == 1 && s.G == 8 && s.V == 1) return launch_flat<4, 4, 1, 8, 1>(x, plan, partial, stream);
-        if (s.G1 == 8 && s.DS == 1 && s.G == 8 && s.V == 1) return launch_flat<4, 8, 1, 8, 1>(x, plan, partial, stream);
-        if (s.G1 == 8 && s.DS == 2 && s.G == 16 && s.V == 1) return launch_flat<4, 8, 2, 16, 1>(x, plan, partial, stream);
-        if (s.G1 == 8 && s.DS == 4 && s.G == 32 && s.V == 1) return launch_flat<4, 8, 4, 32, 1>(x, plan, partial, stream);
-        if (s.G1 == 8 && s.DS == 8 && s.G == 64 && s.V == 1) return launch_flat<4, 8, 8, 64, 1>(x, plan, partial, stream);
-        if (s.G1 == 8 && s.DS == 16 && s.G == 64 && s.V == 2) return launch_flat<4, 8, 16, 64, 2>(x, plan, partial, stream);
-        if (s.G1 == 8 && s.DS == 0 && s.G == 64 && s.V == 4) return launch_flat<4, 8, 0, 64, 4>(x, plan, partial, stream);
-    } else if (s.G1 == 4 && s.DS == 1 && s.G == 8 && s.V == 1) {
-        return launch_flat<1, 4, 1, 8, 1>(x, plan, partial, stream);
-    }
-    return hipErrorInvalidValue;
+    return dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        return launch_flat<L::VEC, L::G1, L::DS, L::G, L::V>(x, plan, partial, stream);
+    });
 }
 
 // ---- column-sliced schedule ------------------------------------------------------------------------
@@ -344,7 +322,7 @@ static hipError_t launch_sliced_r(const FusedArgs& x, const SlicePlan& plan, con
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     if constexpr (DS > 0) {
-        if (x.D == G1 * VEC * DS) {
+        if (x.D == G1 * VEC * DS && rule_on(kRuleExactWidthKernels)) {
             hipLaunchKernelGGL((fused_sliced_kernel<VEC, G1, DS, false, G, V2, R>), dim3((unsigned)blocks), dim3(4 * 64), 0,
                                stream, x.M, x.D, col_tiles, (int)slice_blocks, x.scale, bounds, x.col_indices, x.Q, x.Kmat,
                                x.V, partial);
@@ -360,14 +338,9 @@ template <int VEC, int G1, int DS, int G, int V2>
 static hipError_t launch_sliced(const FusedArgs& x, const SlicePlan& plan, const int* bounds, float* partial,
                                 hipStream_t stream)
 {
-    switch (plan.R) {
-        case 1: return launch_sliced_r<VEC, G1, DS, G, V2, 1>(x, plan, bounds, partial, stream);
-        case 2: return launch_sliced_r<VEC, G1, DS, G, V2, 2>(x, plan, bounds, partial, stream);
-        case 4: return launch_sliced_r<VEC, G1, DS, G, V2, 4>(x, plan, bounds, partial, stream);
-        case 8: return launch_sliced_r<VEC, G1, DS, G, V2, 8>(x, plan, bounds, partial, stream);
-        case 16: return launch_sliced_r<VEC, G1, DS, G, V2, 16>(x, plan, bounds, partial, stream);
-    }
-    return hipErrorInvalidValue;
+    return dispatch_sliced_rows(plan.R, [&](auto r) {
+        return launch_sliced_r<VEC, G1, DS, G, V2, decltype(r)::R>(x, plan, bounds, partial, stream);
+    });
 }
 
 hipError_t fused_sliced_launch(const FusedArgs& x, const FusedShape& s, const SlicePlan& plan, void* workspace,
@@ -377,17 +350,11 @@ hipError_t fused_sliced_launch(const FusedArgs& x, const FusedShape& s, const Sl
     float* partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + plan.bounds_bytes);
     hipError_t e = slice_bounds_launch(x.M, x.K, plan.slices, x.row_offsets, x.col_indices, bounds, stream);
     if (e != hipSuccess) return e;
-    e = hipErrorInvalidValue;
-    // built for 16 < D <= 512: the layouts fused_choose gives those widths
-#define DLSPM_SLICED(g1_, ds_, g_, v_)                                                \
-    if (s.vec == 4 && s.G1 == g1_ && s.DS == ds_ && s.G == g_ && s.V == v_)           \
-        e = launch_sliced<4, g1_, ds_, g_, v_>(x, plan, bounds, partial, stream);
-    DLSPM_SLICED(8, 1, 8, 1)
-    DLSPM_SLICED(8, 2, 16, 1)
-    DLSPM_SLICED(8, 4, 32, 1)
-    DLSPM_SLICED(8, 8, 64, 1)
-    DLSPM_SLICED(8, 16, 64, 2)
-#undef DLSPM_SLICED
+    e = dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        if constexpr (kOneTileLayout<L>) return launch_sliced<4, 8, L::DS, L::G, L::V>(x, plan, bounds, partial, stream);
+        else return hipErrorInvalidValue;
+    });
     if (e != hipSuccess) return e;
     return slice_sum_launch((long long)x.M * x.D, plan.slices, partial, x.O, stream);
 }
@@ -440,23 +407,21 @@ static hipError_t launch_pieces(const FusedArgs& x, const CutPlan& cp, void* pla
 hipError_t fused_pieces_launch(const FusedArgs& x, const FusedShape& s, const CutPlan& cp, void* plan, hipStream_t stream)
 {
     if (x.M <= 0) return hipSuccess;
-    if (s.DS == 1 && s.G == 8 && s.V == 1) return launch_pieces<1, 8, 1>(x, cp, plan, stream);
-    if (s.DS == 2 && s.G == 16 && s.V == 1) return launch_pieces<2, 16, 1>(x, cp, plan, stream);
-    if (s.DS == 4 && s.G == 32 && s.V == 1) return launch_pieces<4, 32, 1>(x, cp, plan, stream);
-    if (s.DS == 8 && s.G == 64 && s.V == 1) return launch_pieces<8, 64, 1>(x, cp, plan, stream);
-    if (s.DS == 16 && s.G == 64 && s.V == 2) return launch_pieces<16, 64, 2>(x, cp, plan, stream);
-    return hipErrorInvalidValue;
+    return dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        if constexpr (kOneTileLayout<L>) return launch_pieces<L::DS, L::G, L::V>(x, cp, plan, stream);
+        else return hipErrorInvalidValue;
+    });
 }
 
 hipError_t fused_planned_launch(const FusedArgs& x, const FusedShape& s, const int* plan, hipStream_t stream)
 {
     if (x.M <= 0) return hipSuccess;
-    if (s.DS == 1 && s.G == 8 && s.V == 1) return launch_planned<1, 8, 1>(x, plan, stream);
-    if (s.DS == 2 && s.G == 16 && s.V == 1) return launch_planned<2, 16, 1>(x, plan, stream);
-    if (s.DS == 4 && s.G == 32 && s.V == 1) return launch_planned<4, 32, 1>(x, plan, stream);
-    if (s.DS == 8 && s.G == 64 && s.V == 1) return launch_planned<8, 64, 1>(x, plan, stream);
-    if (s.DS == 16 && s.G == 64 && s.V == 2) return launch_planned<16, 64, 2>(x, plan, stream);
-    return hipErrorInvalidValue;
+    return dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        if constexpr (kOneTileLayout<L>) return launch_planned<L::DS, L::G, L::V>(x, plan, stream);
+        else return hipErrorInvalidValue;
+    });
 }
 
 }  // namespace dlspm

@@ -3,7 +3,60 @@
 
 #include <hip/hip_runtime.h>
 
+#include <tuple>
+
 namespace dlspm {
+
+// ---- the shapes the kernels are built for, as compile-time tables, and the run-time dispatch onto them ---------------
+// One table per kind of shape; a kernel family instantiates itself for every entry of the tables it is launched over
+// (dispatch below calls `launch` with each entry type), and the size rules choose among the same entries, so a shape is
+// added in one place.
+template <int W_, int R_> struct Split { static constexpr int W = W_, R = R_; };  // waves, consecutive rows per workgroup
+using Splits = std::tuple<Split<4, 16>, Split<4, 8>, Split<4, 4>, Split<4, 2>, Split<4, 1>, Split<8, 4>, Split<8, 2>, Split<8, 1>,
+                          Split<16, 1>>;
+template <int R_> struct Rows { static constexpr int R = R_; };  // rows per four-wave workgroup of the column-sliced kernels
+using SlicedRows = std::tuple<Rows<1>, Rows<2>, Rows<4>, Rows<8>, Rows<16>>;
+// SpMM: floats per lane and access, lanes per dense row, accesses per lane (the last entry: widths below 4)
+template <int VEC_, int G_, int V_> struct RowLanes { static constexpr int VEC = VEC_, G = G_, V = V_; };
+using SpmmLayouts = std::tuple<RowLanes<4, 64, 2>, RowLanes<4, 64, 1>, RowLanes<4, 32, 1>, RowLanes<4, 16, 1>, RowLanes<4, 8, 1>,
+                               RowLanes<1, 8, 1>>;
+// SDDMM: floats per lane and access, lanes per dot product, accesses per lane (0: a run-time loop)
+template <int VEC_, int G1_, int DS_> struct DotLanes { static constexpr int VEC = VEC_, G1 = G1_, DS = DS_; };
+using SddmmLayouts = std::tuple<DotLanes<4, 4, 1>, DotLanes<4, 8, 1>, DotLanes<4, 8, 2>, DotLanes<4, 8, 4>, DotLanes<4, 8, 8>,
+                                DotLanes<4, 8, 16>, DotLanes<4, 8, 0>, DotLanes<1, 4, 1>>;
+// fused: both stages
+template <int VEC_, int G1_, int DS_, int G_, int V_> struct FusedLanes {
+    static constexpr int VEC = VEC_, G1 = G1_, DS = DS_, G = G_, V = V_;
+};
+using FusedLayouts = std::tuple<FusedLanes<4, 4, 1, 8, 1>, FusedLanes<4, 8, 1, 8, 1>, FusedLanes<4, 8, 2, 16, 1>, FusedLanes<4, 8, 4, 32, 1>,
+                                FusedLanes<4, 8, 8, 64, 1>, FusedLanes<4, 8, 16, 64, 2>, FusedLanes<4, 8, 0, 64, 4>, FusedLanes<1, 4, 1, 8, 1>>;
+
+// launch(entry) for the first entry of Table that `match` accepts; hipErrorInvalidValue if there is none
+template <typename Table, typename Match, typename Launch> hipError_t dispatch(Match&& match, Launch&& launch)
+{
+    hipError_t e = hipErrorInvalidValue;
+    bool found = false;
+    auto one = [&](auto entry) {
+        if (!found && match(entry)) {
+            found = true;
+            e = launch(entry);
+        }
+    };
+    std::apply([&](auto... entry) { (one(entry), ...); }, Table{});
+    return e;
+}
+template <typename Launch> hipError_t dispatch_split(int W, int R, Launch&& launch)
+{
+    return dispatch<Splits>([&](auto s) { return s.W == W && s.R == R; }, launch);
+}
+template <typename Launch> hipError_t dispatch_sliced_rows(int R, Launch&& launch)
+{
+    return dispatch<SlicedRows>([&](auto r) { return r.R == R; }, launch);
+}
+inline bool split_is_built(int W, int R, int max_w)
+{
+    return dispatch_split(W, R, [&](auto s) { return s.W <= max_w ? hipSuccess : hipErrorInvalidValue; }) == hipSuccess;
+}
 
 // ceil(a / b) without the overflow of (a + b - 1) for a near INT_MAX
 inline long long ceil_div(long long a, long long b) { return (a + b - 1) / b; }
@@ -40,18 +93,26 @@ struct Tuning {
     int xcd_contiguous = 0;
     int stream_results = -1;
     int cut_piece_pct = 0, cut_longest_pct = 0;
+    int rules_off = 0;  // DLSPM_RULE_* bits: size rules switched off, to measure what each is worth
 };
+// (the values of DLSPM_RULE_* in the header)
+constexpr int kRuleEightWavesFewRows = 1, kRuleSixteenWavesTallLongRows = 2, kRuleMoreWavesFewLongRows = 4, kRuleGroupRows = 8,
+              kRuleRowAlignedSplit = 16, kRulePlanUngroups = 32, kRuleExactWidthKernels = 64;
+
 const Tuning& tuning();
+inline bool rule_on(int rule) { return (tuning().rules_off & rule) == 0; }
 
 // What a row-block kernel is told about its launch in one int: bit 0 = deal the row blocks to the XCDs in contiguous
 // runs (DLSPM_HINT_BANDED or the tuning knob), bits 1-2 = results with the non-temporal hint: 0 by the size rule,
 // 1 never, 2 wherever the rule could say so (dlspm_tuning.stream_results).
-constexpr int kFlagXcdContiguous = 1, kFlagStreamShift = 1, kFlagStreamNever = 1, kFlagStreamAlways = 2;
+// bit 3 = never take the row-aligned split (DLSPM_RULE_ROW_ALIGNED_SPLIT switched off).
+constexpr int kFlagXcdContiguous = 1, kFlagStreamShift = 1, kFlagStreamNever = 1, kFlagStreamAlways = 2, kFlagNoAlignedSplit = 8;
 inline int launch_flags(int xcd_contiguous_hint)
 {
     const Tuning& t = tuning();
     const int stream = t.stream_results < 0 ? 0 : t.stream_results == 0 ? kFlagStreamNever : kFlagStreamAlways;
-    return ((xcd_contiguous_hint | t.xcd_contiguous) ? kFlagXcdContiguous : 0) | (stream << kFlagStreamShift);
+    return ((xcd_contiguous_hint | t.xcd_contiguous) ? kFlagXcdContiguous : 0) | (stream << kFlagStreamShift) |
+           ((t.rules_off & 16) ? kFlagNoAlignedSplit : 0);
 }
 
 // Lane layout and work split of one launch.

@@ -141,7 +141,7 @@ static hipError_t launch_one(const SddmmArgs& x, hipStream_t stream)
     const int blocks = (int)ceil_div(x.M, R);
     if (blocks <= 0) return hipSuccess;
     if constexpr (DS > 0) {
-        if (x.D == G1 * VEC * DS) {
+        if (x.D == G1 * VEC * DS && rule_on(kRuleExactWidthKernels)) {
             hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, false, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M,
                                x.D, launch_flags(x.xcd_contiguous), x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
             return hipGetLastError();
@@ -152,22 +152,10 @@ static hipError_t launch_one(const SddmmArgs& x, hipStream_t stream)
     return hipGetLastError();
 }
 
-template <int VEC, int G1, int DS>
-static hipError_t launch_wr(const SddmmArgs& x, int W, int R, hipStream_t stream)
+// the layout of shape s among SddmmLayouts
+template <typename Launch> static hipError_t dispatch_layout(const SddmmShape& s, Launch&& launch)
 {
-#define DLSPM_WR(w_, r_) \
-    if (W == w_ && R == r_) return launch_one<VEC, G1, DS, w_, r_>(x, stream);
-    DLSPM_WR(4, 16)
-    DLSPM_WR(4, 8)
-    DLSPM_WR(4, 4)
-    DLSPM_WR(4, 2)
-    DLSPM_WR(4, 1)
-    DLSPM_WR(8, 4)
-    DLSPM_WR(8, 2)
-    DLSPM_WR(8, 1)
-    DLSPM_WR(16, 1)
-#undef DLSPM_WR
-    return hipErrorInvalidValue;
+    return dispatch<SddmmLayouts>([&](auto l) { return l.VEC == s.vec && l.G1 == s.G1 && l.DS == s.DS; }, launch);
 }
 
 SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even)
@@ -190,22 +178,13 @@ SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
 
 hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t stream)
 {
-    if (s.vec == 4) {
-        if (s.G1 == 4 && s.DS == 1) return launch_wr<4, 4, 1>(x, s.W, s.R, stream);
-        if (s.G1 == 8) {
-            switch (s.DS) {
-                case 1: return launch_wr<4, 8, 1>(x, s.W, s.R, stream);
-                case 2: return launch_wr<4, 8, 2>(x, s.W, s.R, stream);
-                case 4: return launch_wr<4, 8, 4>(x, s.W, s.R, stream);
-                case 8: return launch_wr<4, 8, 8>(x, s.W, s.R, stream);
-                case 16: return launch_wr<4, 8, 16>(x, s.W, s.R, stream);
-                case 0: return launch_wr<4, 8, 0>(x, s.W, s.R, stream);
-            }
-        }
-    } else if (s.G1 == 4 && s.DS == 1) {
-        return launch_wr<1, 4, 1>(x, s.W, s.R, stream);
-    }
-    return hipErrorInvalidValue;
+    return dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        return dispatch_split(s.W, s.R, [&](auto split) {
+            using S = decltype(split);
+            return launch_one<L::VEC, L::G1, L::DS, S::W, S::R>(x, stream);
+        });
+    });
 }
 
 // ---- flat schedule: every wave owns `chunk` consecutive nonzeros of the mask, whatever rows they belong to ---------
@@ -248,7 +227,7 @@ static hipError_t launch_flat(const SddmmArgs& x, int chunk, hipStream_t stream)
     const long long units = ((long long)x.nnz + chunk - 1) / chunk;
     const unsigned blocks = (unsigned)((units + kFlatWaves - 1) / kFlatWaves);
     if constexpr (DS > 0) {
-        if (x.D == G1 * VEC * DS) {
+        if (x.D == G1 * VEC * DS && rule_on(kRuleExactWidthKernels)) {
             hipLaunchKernelGGL((sddmm_flat_kernel<VEC, G1, DS, false>), dim3(blocks), dim3(kFlatWaves * 64), 0, stream, x.M,
                                x.D, x.nnz, chunk, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
             return hipGetLastError();
@@ -261,22 +240,10 @@ static hipError_t launch_flat(const SddmmArgs& x, int chunk, hipStream_t stream)
 
 hipError_t sddmm_flat_launch(const SddmmArgs& x, const SddmmShape& s, int chunk, hipStream_t stream)
 {
-    if (s.vec == 4) {
-        if (s.G1 == 4 && s.DS == 1) return launch_flat<4, 4, 1>(x, chunk, stream);
-        if (s.G1 == 8) {
-            switch (s.DS) {
-                case 1: return launch_flat<4, 8, 1>(x, chunk, stream);
-                case 2: return launch_flat<4, 8, 2>(x, chunk, stream);
-                case 4: return launch_flat<4, 8, 4>(x, chunk, stream);
-                case 8: return launch_flat<4, 8, 8>(x, chunk, stream);
-                case 16: return launch_flat<4, 8, 16>(x, chunk, stream);
-                case 0: return launch_flat<4, 8, 0>(x, chunk, stream);
-            }
-        }
-    } else if (s.G1 == 4 && s.DS == 1) {
-        return launch_flat<1, 4, 1>(x, chunk, stream);
-    }
-    return hipErrorInvalidValue;
+    return dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        return launch_flat<L::VEC, L::G1, L::DS>(x, chunk, stream);
+    });
 }
 
 // ---- column-sliced schedule ------------------------------------------------------------------------
@@ -300,14 +267,7 @@ static hipError_t launch_sliced_r(const SddmmArgs& x, const SlicePlan& plan, con
 template <int VEC, int G1, int DS>
 static hipError_t launch_sliced(const SddmmArgs& x, const SlicePlan& plan, const int* bounds, hipStream_t stream)
 {
-    switch (plan.R) {
-        case 1: return launch_sliced_r<VEC, G1, DS, 1>(x, plan, bounds, stream);
-        case 2: return launch_sliced_r<VEC, G1, DS, 2>(x, plan, bounds, stream);
-        case 4: return launch_sliced_r<VEC, G1, DS, 4>(x, plan, bounds, stream);
-        case 8: return launch_sliced_r<VEC, G1, DS, 8>(x, plan, bounds, stream);
-        case 16: return launch_sliced_r<VEC, G1, DS, 16>(x, plan, bounds, stream);
-    }
-    return hipErrorInvalidValue;
+    return dispatch_sliced_rows(plan.R, [&](auto r) { return launch_sliced_r<VEC, G1, DS, decltype(r)::R>(x, plan, bounds, stream); });
 }
 
 // built for 16 < D <= 512 (G1 = 8 with 1 to 16 accesses per lane)
@@ -317,12 +277,11 @@ hipError_t sddmm_sliced_launch(const SddmmArgs& x, const SddmmShape& s, const Sl
     int* bounds = static_cast<int*>(workspace);
     const hipError_t e = slice_bounds_launch(x.M, x.K, plan.slices, x.row_offsets, x.col_indices, bounds, stream);
     if (e != hipSuccess) return e;
-    if (s.vec == 4 && s.G1 == 8 && s.DS == 4) return launch_sliced<4, 8, 4>(x, plan, bounds, stream);
-    if (s.vec == 4 && s.G1 == 8 && s.DS == 8) return launch_sliced<4, 8, 8>(x, plan, bounds, stream);
-    if (s.vec == 4 && s.G1 == 8 && s.DS == 16) return launch_sliced<4, 8, 16>(x, plan, bounds, stream);
-    if (s.vec == 4 && s.G1 == 8 && s.DS == 2) return launch_sliced<4, 8, 2>(x, plan, bounds, stream);
-    if (s.vec == 4 && s.G1 == 8 && s.DS == 1) return launch_sliced<4, 8, 1>(x, plan, bounds, stream);
-    return hipErrorInvalidValue;
+    return dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        if constexpr (L::VEC == 4 && L::G1 == 8 && L::DS >= 1) return launch_sliced<4, 8, L::DS>(x, plan, bounds, stream);
+        else return hipErrorInvalidValue;
+    });
 }
 
 // ---- row plan ---------------------------------------------------------------------------------------
@@ -343,10 +302,12 @@ bool sddmm_plan_applies(const DeviceInfo& dev, SddmmShape& s, int M, int D, int 
 // which a plan over whole rows cannot help (every row has a compute unit to itself, half of the device idles): cut, the
 // pieces of the rows fill the device, at no cost to SDDMM, whose pieces write their own CSR slots. Measured on the
 // reference's ResNet-50 layers of 64 and 128 rows (36 ... 900 nonzeros per row, D = 128, in a graph): 0.74 ... 0.93 of the
-// time (64 x 576 with 499 per row: 4.30 -> 3.20 us; 128 x 1152 with 231: 3.78 -> 3.15 us); with 256 rows 0.93 ... 1.06.
+// time (64 x 576 with 499 per row: 4.30 -> 3.20 us; 128 x 1152 with 231: 3.78 -> 3.15 us); with 256 rows 0.93 ... 1.06 on
+// those layers, whose longest rows hold two to three shares, and 0.66 where one holds three and a half (256 x 2304,
+// lognormal rows of 200 on average): from as many rows as compute units on, the advice asks for a longer row.
 bool sddmm_cut_plan_applies(const DeviceInfo& dev, SddmmShape& s, int M, int D, int nnz)
 {
-    if (s.vec == 4 && s.G1 == 8 && s.DS >= 1 && s.W == 8 && M < dev.cus) {
+    if (s.vec == 4 && s.G1 == 8 && s.DS >= 1 && s.W == 8 && M < 2 * dev.cus) {
         s.W = 4;
         s.R = 1;
         return true;
@@ -370,14 +331,11 @@ static hipError_t launch_planned(const SddmmArgs& x, const int* plan, int entrie
 static hipError_t launch_planned_ds(const SddmmArgs& x, const SddmmShape& s, const int* plan, int entries, hipStream_t stream)
 {
     if (x.M <= 0) return hipSuccess;
-    switch (s.DS) {
-        case 1: return launch_planned<1>(x, plan, entries, stream);
-        case 2: return launch_planned<2>(x, plan, entries, stream);
-        case 4: return launch_planned<4>(x, plan, entries, stream);
-        case 8: return launch_planned<8>(x, plan, entries, stream);
-        case 16: return launch_planned<16>(x, plan, entries, stream);
-    }
-    return hipErrorInvalidValue;
+    return dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        if constexpr (L::VEC == 4 && L::G1 == 8 && L::DS >= 1) return launch_planned<L::DS>(x, plan, entries, stream);
+        else return hipErrorInvalidValue;
+    });
 }
 
 hipError_t sddmm_planned_launch(const SddmmArgs& x, const SddmmShape& s, const int* plan, hipStream_t stream)

@@ -188,22 +188,10 @@ static hipError_t launch_one(const SpmmArgs& x, int tile_major, hipStream_t stre
     return hipGetLastError();
 }
 
-template <int VEC, int G, int V>
-static hipError_t launch_wr(const SpmmArgs& x, int W, int R, int tile_major, hipStream_t stream)
+// the layout of shape s among SpmmLayouts
+template <typename Launch> static hipError_t dispatch_layout(const SpmmShape& s, Launch&& launch)
 {
-#define DLSPM_WR(w_, r_) \
-    if (W == w_ && R == r_) return launch_one<VEC, G, V, w_, r_>(x, tile_major, stream);
-    DLSPM_WR(4, 16)
-    DLSPM_WR(4, 8)
-    DLSPM_WR(4, 4)
-    DLSPM_WR(8, 4)
-    DLSPM_WR(8, 2)
-    DLSPM_WR(8, 1)
-    DLSPM_WR(16, 1)
-    DLSPM_WR(4, 2)
-    DLSPM_WR(4, 1)
-#undef DLSPM_WR
-    return hipErrorInvalidValue;
+    return dispatch<SpmmLayouts>([&](auto l) { return l.VEC == s.vec && l.G == s.G && l.V == s.V; }, launch);
 }
 
 // Width of the column tiles of B that the grid works through one after the other (tile-major order), or 0: one tile
@@ -279,16 +267,13 @@ SpmmShape spmm_choose(const DeviceInfo& dev, int M, int K, int N, int nnz, bool 
 
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream)
 {
-    if (s.vec == 4) {
-        if (s.G == 64 && s.V == 1) return launch_wr<4, 64, 1>(x, s.W, s.R, s.tile_major, stream);
-        if (s.G == 64 && s.V == 2) return launch_wr<4, 64, 2>(x, s.W, s.R, s.tile_major, stream);
-        if (s.G == 32 && s.V == 1) return launch_wr<4, 32, 1>(x, s.W, s.R, s.tile_major, stream);
-        if (s.G == 16 && s.V == 1) return launch_wr<4, 16, 1>(x, s.W, s.R, s.tile_major, stream);
-        if (s.G == 8 && s.V == 1) return launch_wr<4, 8, 1>(x, s.W, s.R, s.tile_major, stream);
-    } else {
-        if (s.G == 8 && s.V == 1) return launch_wr<1, 8, 1>(x, s.W, s.R, s.tile_major, stream);
-    }
-    return hipErrorInvalidValue;
+    return dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        return dispatch_split(s.W, s.R, [&](auto split) {
+            using S = decltype(split);
+            return launch_one<L::VEC, L::G, L::V, S::W, S::R>(x, s.tile_major, stream);
+        });
+    });
 }
 
 // ---- flat schedule ----------------------------------------------------------------------------------
@@ -389,16 +374,10 @@ static hipError_t launch_flat(const SpmmArgs& x, const FlatPlan& plan, int tile_
 hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPlan& plan, float* partial,
                             hipStream_t stream)
 {
-    if (s.vec == 4) {
-        if (s.G == 64 && s.V == 1) return launch_flat<4, 64, 1>(x, plan, s.tile_major, partial, stream);
-        if (s.G == 64 && s.V == 2) return launch_flat<4, 64, 2>(x, plan, s.tile_major, partial, stream);
-        if (s.G == 32 && s.V == 1) return launch_flat<4, 32, 1>(x, plan, s.tile_major, partial, stream);
-        if (s.G == 16 && s.V == 1) return launch_flat<4, 16, 1>(x, plan, s.tile_major, partial, stream);
-        if (s.G == 8 && s.V == 1) return launch_flat<4, 8, 1>(x, plan, s.tile_major, partial, stream);
-    } else if (s.G == 8 && s.V == 1) {
-        return launch_flat<1, 8, 1>(x, plan, s.tile_major, partial, stream);
-    }
-    return hipErrorInvalidValue;
+    return dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        return launch_flat<L::VEC, L::G, L::V>(x, plan, s.tile_major, partial, stream);
+    });
 }
 
 // ---- column-sliced schedule ------------------------------------------------------------------------
@@ -422,14 +401,9 @@ template <int VEC, int G, int V>
 static hipError_t launch_sliced(const SpmmArgs& x, const SlicePlan& plan, int tile_major, const int* bounds,
                                 float* partial, hipStream_t stream)
 {
-    switch (plan.R) {
-        case 1: return launch_sliced_r<VEC, G, V, 1>(x, plan, tile_major, bounds, partial, stream);
-        case 2: return launch_sliced_r<VEC, G, V, 2>(x, plan, tile_major, bounds, partial, stream);
-        case 4: return launch_sliced_r<VEC, G, V, 4>(x, plan, tile_major, bounds, partial, stream);
-        case 8: return launch_sliced_r<VEC, G, V, 8>(x, plan, tile_major, bounds, partial, stream);
-        case 16: return launch_sliced_r<VEC, G, V, 16>(x, plan, tile_major, bounds, partial, stream);
-    }
-    return hipErrorInvalidValue;
+    return dispatch_sliced_rows(plan.R, [&](auto r) {
+        return launch_sliced_r<VEC, G, V, decltype(r)::R>(x, plan, tile_major, bounds, partial, stream);
+    });
 }
 
 hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const SlicePlan& plan, void* workspace,
@@ -439,16 +413,12 @@ hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const Slice
     float* partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + plan.bounds_bytes);
     hipError_t e = slice_bounds_launch(x.M, x.K, plan.slices, x.row_offsets, x.col_indices, bounds, stream);
     if (e != hipSuccess) return e;
-    e = hipErrorInvalidValue;
     // built for every dwordx4 layout spmm_choose gives (N >= 4)
-#define DLSPM_SLICED(g_, v_) \
-    if (s.vec == 4 && s.G == g_ && s.V == v_) e = launch_sliced<4, g_, v_>(x, plan, s.tile_major, bounds, partial, stream);
-    DLSPM_SLICED(64, 2)
-    DLSPM_SLICED(64, 1)
-    DLSPM_SLICED(32, 1)
-    DLSPM_SLICED(16, 1)
-    DLSPM_SLICED(8, 1)
-#undef DLSPM_SLICED
+    e = dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        if constexpr (L::VEC == 4) return launch_sliced<4, L::G, L::V>(x, plan, s.tile_major, bounds, partial, stream);
+        else return hipErrorInvalidValue;
+    });
     if (e != hipSuccess) return e;
     return slice_sum_launch((long long)x.M * x.N, plan.slices, partial, x.C, stream);
 }
@@ -465,6 +435,7 @@ bool plan_ungroups(const DeviceInfo& dev, int M, int width, int nnz)
 {
     const long long avg32 = 32ll * M, avg48 = 48ll * M, avg128 = 128ll * M;
     const long long cus = dev.cus;  // measured on 256 compute units: 4096, 8192 and 16384 rows
+    if (!rule_on(kRulePlanUngroups)) return false;
     return nnz >= avg32 && (M <= 16 * cus || (width >= 128 && (M <= 32 * cus || (nnz >= avg48 && M <= 64 * cus) || nnz >= avg128)));
 }
 
@@ -478,6 +449,7 @@ bool plan_ungroups(const DeviceInfo& dev, int M, int width, int nnz)
 bool plan_ungroups_dots(const DeviceInfo& dev, int M, int D, int nnz)
 {
     const long long cus = dev.cus;  // measured on 256 compute units: 2048, 4096 and 8192 rows
+    if (!rule_on(kRulePlanUngroups)) return false;
     if (M <= 8 * cus) return true;
     return (long long)nnz >= 32ll * M && (M <= 16 * cus || (D >= 128 && M <= 32 * cus && (long long)nnz >= 128ll * M));
 }
@@ -509,26 +481,23 @@ hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int*
 {
     if (x.M <= 0) return hipSuccess;
     const int *starts = plan, *ends = plan + x.M, *rows = plan + 2 * (size_t)x.M;
-#define DLSPM_PLANNED(g_, v_)                                                                                          \
-    if (s.G == g_ && s.V == v_) {                                                                                      \
-        const int col_tiles = (int)ceil_div(x.N, g_ * 4 * v_);                                                         \
-        const long long blocks = (long long)x.M * col_tiles;                                                           \
-        if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;                                                \
-        if (dense_fits_buffer(x.K, x.N))                                                                               \
-            hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_, true>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, \
-                               x.M, x.N, x.nnz, col_tiles, launch_flags(0), starts, ends, rows, x.col_indices, x.values, x.B, x.C);     \
-        else                                                                                                           \
-            hipLaunchKernelGGL((spmm_planned_kernel<4, g_, v_, false>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, \
-                               x.M, x.N, x.nnz, col_tiles, launch_flags(0), starts, ends, rows, x.col_indices, x.values, x.B, x.C);     \
-        return hipGetLastError();                                                                                      \
-    }
-    DLSPM_PLANNED(64, 2)
-    DLSPM_PLANNED(64, 1)
-    DLSPM_PLANNED(32, 1)
-    DLSPM_PLANNED(16, 1)
-    DLSPM_PLANNED(8, 1)
-#undef DLSPM_PLANNED
-    return hipErrorInvalidValue;
+    return dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        if constexpr (L::VEC != 4) {
+            return hipErrorInvalidValue;
+        } else {
+            const int col_tiles = (int)ceil_div(x.N, L::G * 4 * L::V);
+            const long long blocks = (long long)x.M * col_tiles;
+            if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+            if (dense_fits_buffer(x.K, x.N))
+                hipLaunchKernelGGL((spmm_planned_kernel<4, L::G, L::V, true>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M,
+                                   x.N, x.nnz, col_tiles, launch_flags(0), starts, ends, rows, x.col_indices, x.values, x.B, x.C);
+            else
+                hipLaunchKernelGGL((spmm_planned_kernel<4, L::G, L::V, false>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M,
+                                   x.N, x.nnz, col_tiles, launch_flags(0), starts, ends, rows, x.col_indices, x.values, x.B, x.C);
+            return hipGetLastError();
+        }
+    });
 }
 
 // The same with a cut plan (CutPlan, launch.hpp): one workgroup per entry and column tile, then the kernel that adds the
@@ -540,28 +509,25 @@ hipError_t spmm_pieces_launch(const SpmmArgs& x, const SpmmShape& s, const CutPl
     const int *starts = base, *ends = base + cp.entries, *rows = base + 2 * (size_t)cp.entries,
               *slot_of = base + 3 * (size_t)cp.entries;
     float* pieces = reinterpret_cast<float*>(static_cast<char*>(plan) + cp.off_pieces);
-    hipError_t e = hipErrorInvalidValue;
-#define DLSPM_PIECES(g_, v_)                                                                                              \
-    if (s.G == g_ && s.V == v_) {                                                                                         \
-        const int col_tiles = (int)ceil_div(x.N, g_ * 4 * v_);                                                            \
-        const long long blocks = (long long)cp.entries * col_tiles;                                                       \
-        if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;                                                   \
-        if (dense_fits_buffer(x.K, x.N))                                                                                  \
-            hipLaunchKernelGGL((spmm_pieces_kernel<4, g_, v_, true>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M, \
-                               x.N, x.nnz, col_tiles, launch_flags(0), cp.entries, cp.slots, starts, ends, rows, slot_of, \
-                               x.col_indices, x.values, x.B, x.C, pieces);                                                \
-        else                                                                                                              \
-            hipLaunchKernelGGL((spmm_pieces_kernel<4, g_, v_, false>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream,   \
-                               x.M, x.N, x.nnz, col_tiles, launch_flags(0), cp.entries, cp.slots, starts, ends, rows,     \
-                               slot_of, x.col_indices, x.values, x.B, x.C, pieces);                                       \
-        e = hipGetLastError();                                                                                            \
-    }
-    DLSPM_PIECES(64, 2)
-    DLSPM_PIECES(64, 1)
-    DLSPM_PIECES(32, 1)
-    DLSPM_PIECES(16, 1)
-    DLSPM_PIECES(8, 1)
-#undef DLSPM_PIECES
+    const hipError_t e = dispatch_layout(s, [&](auto l) {
+        using L = decltype(l);
+        if constexpr (L::VEC != 4) {
+            return hipErrorInvalidValue;
+        } else {
+            const int col_tiles = (int)ceil_div(x.N, L::G * 4 * L::V);
+            const long long blocks = (long long)cp.entries * col_tiles;
+            if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+            if (dense_fits_buffer(x.K, x.N))
+                hipLaunchKernelGGL((spmm_pieces_kernel<4, L::G, L::V, true>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M,
+                                   x.N, x.nnz, col_tiles, launch_flags(0), cp.entries, cp.slots, starts, ends, rows, slot_of,
+                                   x.col_indices, x.values, x.B, x.C, pieces);
+            else
+                hipLaunchKernelGGL((spmm_pieces_kernel<4, L::G, L::V, false>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M,
+                                   x.N, x.nnz, col_tiles, launch_flags(0), cp.entries, cp.slots, starts, ends, rows, slot_of,
+                                   x.col_indices, x.values, x.B, x.C, pieces);
+            return hipGetLastError();
+        }
+    });
     if (e != hipSuccess) return e;
     return cut_rows_sum_launch(x.M, x.N, cp, plan, x.C, stream);
 }

@@ -391,7 +391,16 @@ typedef struct dlspm_tuning {
     int cut_piece_pct;    /* cut plans: the longest piece, in per cent of a share (nnz / compute units); 0 = the rule, 100 */
     int cut_longest_pct;  /* ... and the longest row that stays whole; 0 = the rule, 150. Both 10 ... 1000; they enter the  */
                           /* size of a cut plan, so set them before dlspm_row_plan_bytes_for and keep them for the launches */
+    int rules_off;        /* DLSPM_RULE_* bits: size rules switched off, to measure what each is worth; 0 = all on        */
 } dlspm_tuning;
+/* rules that dlspm_tuning.rules_off can switch off (the others have a field of their own above) */
+#define DLSPM_RULE_EIGHT_WAVES_FEW_ROWS         1  /* SDDMM, fused: eight waves per row below two rows per compute unit     */
+#define DLSPM_RULE_SIXTEEN_WAVES_TALL_LONG_ROWS 2  /* sixteen waves per row for very long rows in a tall matrix             */
+#define DLSPM_RULE_MORE_WAVES_FEW_LONG_ROWS     4  /* eight or sixteen waves per row for few rows of very many nonzeros     */
+#define DLSPM_RULE_GROUP_ROWS                   8  /* several short rows per workgroup in tall matrices                     */
+#define DLSPM_RULE_ROW_ALIGNED_SPLIT           16  /* whole rows per wave where that is nearly as even as the even split    */
+#define DLSPM_RULE_PLAN_UNGROUPS               32  /* a planned launch runs one row per workgroup where the size rule groups */
+#define DLSPM_RULE_EXACT_WIDTH_KERNELS         64  /* SDDMM, fused: kernels without bounds handling for D = 16, 32, ... 512  */
 void dlspm_tuning_default(dlspm_tuning* t);   /* fills *t with "follow the rules" */
 int dlspm_set_tuning(const dlspm_tuning* t);  /* DLSPM_OK or DLSPM_E_INVALID_ARG (a field out of range) */
 int dlspm_get_tuning(dlspm_tuning* t);        /* what the calling thread's launches currently use */

@@ -185,7 +185,8 @@ def test_cut_plan_sizes_and_advice(dl):
     assert dl.describe_launch(dl.OP_SDDMM, 128, 1152, 128, 29510)["W"] == 8
     assert dl.row_plan_advice(dl.OP_SDDMM, 128, 1152, 128, 29510, 455) == 2
     assert dl.row_plan_advice(dl.OP_SDDMM, 64, 576, 128, 31919, 547) == 2
-    assert dl.row_plan_advice(dl.OP_SDDMM, 256, 2304, 128, 118041, 900) == 0   # 256 rows: as many as compute units
+    assert dl.row_plan_advice(dl.OP_SDDMM, 256, 2304, 128, 118041, 900) == 0   # 256 rows, longest below two shares: no
+    assert dl.row_plan_advice(dl.OP_SDDMM, 256, 2304, 128, 53000, 800) == 2    # ... of nearly four shares: yes
     assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 256, 29510, 455) in (0, 1)
     assert dl.row_plan_advice(dl.OP_FUSED, 128, 1152, 64, 29510, 455) in (0, 1)
 

@@ -89,6 +89,7 @@ def schedules(dl, torch, op, M, K, N, nnz, ro_d, ci_d, every):
 def graph_us(torch, step, launches=20, replays=7):
     """Microseconds per launch of step() inside a HIP graph of `launches` launches (median of `replays` double replays)."""
     stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())  # what was enqueued so far (a plan build, say) comes first
     with torch.cuda.stream(stream):
         for _ in range(3):
             step()
