@@ -51,7 +51,13 @@ def test_split_rule_and_the_even_rows_hint(dl):
             a = dl.describe_launch(op, 8192, 4096, width, nnz)
             b = dl.describe_launch(op, 8192, 4096, width, nnz, rows_even=True)
             assert (a["W"], a["R"]) == (4, 1) and (b["W"], b["R"]) == (4, 4)
-            assert {k: v for k, v in a.items() if k != "R"} == {k: v for k, v in b.items() if k != "R"}
+            same = lambda d: {k: v for k, v in d.items() if k not in ("R", "flat_chunk", "flat_units")}
+            assert same(a) == same(b)
+            # SDDMM needs no memory for its flat schedule and takes it by the sizes alone -- except for rows known to be even
+            if op == dl.OP_SDDMM:
+                assert a["flat_chunk"] > 0 and b["flat_chunk"] == 0
+            else:
+                assert (a["flat_chunk"], a["flat_units"]) == (b["flat_chunk"], b["flat_units"])
             # too few rows for 512 workgroups of four rows: unchanged
             assert dl.describe_launch(op, 2048, 4096, width, 2048 * 600, rows_even=True)["R"] == 4
             assert dl.describe_launch(op, 1536, 4096, width, 1536 * 600, rows_even=True)["R"] == 1
