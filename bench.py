@@ -38,6 +38,11 @@ Prints ONE JSON line:
   null_call_us      the same K-step graph with workspace = NULL, 0 (the plain drop-in call), beside launch_us
   host_enqueue_us   what one call costs the host outside a graph (200 calls issued without synchronising, wall time per
                     call): the plain call, the prepared call, and an empty kernel launch (the runtime's own share)
+  launch_floor      measured in this run, between the nodes of a HIP graph like the ops: an empty kernel of 256 ...
+                    8192 workgroups of 256 threads, and a kernel that only walks the dependent loads every row-block
+                    kernel starts with (row offsets -> column indices -> one dense row -> one store) on the grid of the
+                    headline's launch: what a launch costs the device before any arithmetic. `floor_us` of every
+                    configuration is the empty kernel at that configuration's number of workgroups (interpolated)
   all_configs       the same measurement for every benchmark configuration (shorter runs)
 """
 import argparse
@@ -83,12 +88,16 @@ def make_step(dl, torch, c, prepared=True, info=None):
     ro, ci = d(c["row_offsets"]), d(c["col_indices"])
     prep = None
     if prepared:
-        t0 = time.perf_counter()
-        mi = dl.analyze(ro, ci, c["K"])
-        t1 = time.perf_counter()
+        torch.cuda.synchronize()
+        walls = []
+        for _ in range(6):  # the first call of a process also loads the kernel: reported by itself
+            t0 = time.perf_counter()
+            mi = dl.analyze(ro, ci, c["K"])
+            walls.append((time.perf_counter() - t0) * 1e6)
         prep = dl.prepare(ro, ci, c["K"], c["op"], c["N"], info=mi)
         if info is not None:
-            info.update({"row_offsets": ro, "prepared": prep, "matrix_info": mi.as_dict(), "analyze_host_us": (t1 - t0) * 1e6})
+            info.update({"row_offsets": ro, "prepared": prep, "matrix_info": mi.as_dict(), "analyze_host_us": median(walls[1:]),
+                         "analyze_first_call_us": walls[0]})
     if c["op"] == dl.OP_SPMM:
         va, B = d(c["values"]), d(c["d0"])
         out = torch.empty((c["M"], c["N"]), dtype=torch.float32, device="cuda")
@@ -251,6 +260,38 @@ class Probe:
             f.argtypes = [vp, ci, ci, ci, ci, ci] + args + [vp, sz, vp, st]
         self.lib.dlspm_probe_enqueue_empty.restype = ctypes.c_double
         self.lib.dlspm_probe_enqueue_empty.argtypes = [ci, vp]
+        self.lib.dlspm_probe_floor.restype = ctypes.c_int
+        self.lib.dlspm_probe_floor.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp]
+
+    def launch_floor(self, dl, torch, c, use_graph=True, launches=200):
+        """Microseconds per launch between the nodes of a graph of `launches`: the empty kernel against the number of
+        workgroups, and the chain kernel (depth 0 ... 3) on configuration c's matrix at one workgroup per row."""
+        ro, ci = torch.from_numpy(c["row_offsets"]).cuda(), torch.from_numpy(c["col_indices"]).cuda()
+        B = torch.zeros((c["K"], 256), dtype=torch.float32, device="cuda")
+        C = torch.empty((c["M"], 256), dtype=torch.float32, device="cuda")
+        stream = torch.cuda.Stream()
+
+        def timed(workgroups, depth):
+            def one():
+                st = self.lib.dlspm_probe_floor(workgroups, 256, depth, c["M"], ro.data_ptr(), ci.data_ptr(), B.data_ptr(),
+                                                C.data_ptr(), torch.cuda.current_stream().cuda_stream)
+                if st != 0:
+                    raise RuntimeError(f"dlspm_probe_floor: hip error {st}")
+            with torch.cuda.stream(stream):
+                stream.wait_stream(torch.cuda.current_stream())
+                for _ in range(3):
+                    one()
+                stream.synchronize()
+                g = capture(torch, stream, lambda: [one() for _ in range(launches)]) if use_graph else None
+                ev, _ = timed_replays(torch, stream, g.replay if g else (lambda: [one() for _ in range(launches)]), 7)
+            return round(median(ev) / launches * 1e6, 2)
+
+        grids = [256, 512, 1024, 2048, 4096, 8192]
+        return {"what": f"us per launch between the nodes of a graph of {launches} (median of 7 replays); 256 threads per workgroup",
+                "workgroups": grids, "empty_kernel_us": [timed(g, -1) for g in grids],
+                "dependent_loads": {"matrix": c["name"], "workgroups": c["M"],
+                                    "row_offsets_us": timed(c["M"], 0), "plus_column_indices_us": timed(c["M"], 1),
+                                    "plus_one_dense_row_us": timed(c["M"], 2), "plus_store_us": timed(c["M"], 3)}}
 
     def host_enqueue_us(self, dl, torch, raw, prepared, calls=200, reps=5):
         """Host microseconds per call of the entry point, issued `calls` times without synchronising, outside a graph
@@ -338,7 +379,18 @@ def launch_signature(dl, c, prep):
             f"W{sh['W']}:R{1 if planned else sh['R']}:{hints}")
 
 
-def measure(dl, torch, np, c, args, probe, steps, warmup, replays, ceiling_gbps, with_cpu, cpu_budget):
+def floor_at(floor, workgroups):
+    """The empty-kernel time of the floor table at `workgroups` (linear between its points, flat outside them)."""
+    xs, ys = floor["workgroups"], floor["empty_kernel_us"]
+    if workgroups <= xs[0]:
+        return ys[0]
+    for (x0, y0), (x1, y1) in zip(zip(xs, ys), zip(xs[1:], ys[1:])):
+        if workgroups <= x1:
+            return round(y0 + (y1 - y0) * (workgroups - x0) / (x1 - x0), 2)
+    return ys[-1]
+
+
+def measure(dl, torch, np, c, args, probe, steps, warmup, replays, ceiling_gbps, with_cpu, cpu_budget, floor=None):
     """Every figure of one configuration."""
     acct = dl.account(c["op"], c["M"], c["K"], c["N"], c["nnz"])
     info = {}
@@ -381,6 +433,12 @@ def measure(dl, torch, np, c, args, probe, steps, warmup, replays, ceiling_gbps,
         "frac_of_gather_ceiling": round(eff_gbps / ceiling_gbps, 3) if ceiling_gbps else None,
         "warm_us": round(s * 1e6, 3),
     }
+    if floor is not None:
+        # one workgroup per R rows and column tile (a row plan without grouping: one per row)
+        shape = dl.describe_launch(c["op"], c["M"], c["K"], c["N"], c["nnz"], rows_even=r["rows_even_hint"])
+        rows_each = 1 if prep and prep.call_plan.build else max(shape["R"], 1)
+        r["workgroups"] = -(-c["M"] // rows_each) * max(shape["col_tiles"], 1)
+        r["floor_us"] = floor_at(floor, r["workgroups"])
     if "steady_per_step_s" in t:
         r["steady_state_launch_us"] = round(t["steady_per_step_s"] * 1e6, 3)
         r["replay_overhead_us"] = round(t["replay_overhead_s"] * 1e6, 2)
@@ -397,7 +455,9 @@ def measure(dl, torch, np, c, args, probe, steps, warmup, replays, ceiling_gbps,
         else:
             r["null_call_us"] = r["launch_us"]  # nothing is passed: the timed launches are the plain call
         prepare = {"analyze_host_us": round(info.get("analyze_host_us", 0.0), 1),
-                   "analyze": "dlspm_analyze: one pass over the CSR structure on the device, synchronises, host wall time"}
+                   "analyze_first_call_us": round(info.get("analyze_first_call_us", 0.0), 1),
+                   "analyze": "dlspm_analyze: one pass over the CSR structure on the device, synchronises; host wall time, median of "
+                              "five calls after the first (which may load the kernel)"}
         if prep is not None and prep.call_plan.build:
             ro, mem = info["row_offsets"], prep.memory
             build_fn = dl.lib().dlspm_row_plan_build if prep.call_plan.build == dl.BUILD_ROW_PLAN else dl.lib().dlspm_row_plan_build_cut
@@ -414,6 +474,8 @@ def measure(dl, torch, np, c, args, probe, steps, warmup, replays, ceiling_gbps,
             prepare["build"] = "kernels on the stream, no host copy, no synchronisation (capturable); HIP events, graph of 20 builds"
             gain = (r["null_call_us"] - r["launch_us"])
             prepare["launches_until_the_build_pays"] = round(prepare["build_us"] / gain, 1) if gain > 0 else None
+            prepare["launches_until_analysis_and_build_pay"] = (round((prepare["build_us"] + prepare["analyze_host_us"]) / gain, 1)
+                                                                if gain > 0 else None)
         r["prepare_us"] = prepare
         r["host_enqueue_us"] = probe.host_enqueue_us(dl, torch, info["raw"], prep)
     if r.get("row_plan") and "prepare_us" in r:
@@ -455,7 +517,8 @@ def main():
 
     ceiling = probe.gather_ceiling(torch, not args.no_graph)
     c = dl.make_config(args.config)
-    head, acct = measure(dl, torch, np, c, args, probe, args.steps, args.warmup, replays, ceiling["value"], not args.no_cpu, (6.0, 3.0))
+    floor = probe.launch_floor(dl, torch, c, not args.no_graph)
+    head, acct = measure(dl, torch, np, c, args, probe, args.steps, args.warmup, replays, ceiling["value"], not args.no_cpu, (6.0, 3.0), floor)
     s = head["launch_us"] * 1e-6
 
     result = {
@@ -478,6 +541,7 @@ def main():
         "effective_GBps": head["effective_GBps"], "effective_fraction": head["effective_fraction"],
         "effective_bytes": head["effective_bytes"],
         "gather_ceiling": ceiling, "frac_of_gather_ceiling": head["frac_of_gather_ceiling"],
+        "launch_floor": floor,
         "warm_us": head["warm_us"], "cold_us": head["cold_us"], "cold_detail": head["cold_detail"],
         "cpu_baseline": head["cpu_baseline"],
     }
@@ -485,7 +549,7 @@ def main():
         result["rel_frobenius_vs_cpu"] = head["rel_frobenius_vs_cpu"]
     if "row_plan_detail" in head:
         result["row_plan"] = head["row_plan_detail"]
-    for key in ("null_call_us", "prepare_us", "host_enqueue_us", "prepared", "matrix_info"):
+    for key in ("null_call_us", "prepare_us", "host_enqueue_us", "prepared", "matrix_info", "workgroups", "floor_us"):
         if key in head:
             result[key] = head[key]
     info = dl.device_info()
@@ -499,7 +563,7 @@ def main():
                 continue
             cc = dl.make_config(cfg)
             k = min(args.steps, 500)
-            rr, _ = measure(dl, torch, np, cc, args, probe, k, min(args.warmup, 50), replays, ceiling["value"], not args.no_cpu, (2.5, 1.5))
+            rr, _ = measure(dl, torch, np, cc, args, probe, k, min(args.warmup, 50), replays, ceiling["value"], not args.no_cpu, (2.5, 1.5), floor)
             others[cc["name"]] = {k2: v for k2, v in rr.items() if k2 not in ("replay_launch_us",)}
         result["all_configs"] = others
 

@@ -5,6 +5,7 @@
 #include "../../include/dlspm_hip.h"
 
 #include <algorithm>
+#include <mutex>
 
 #include "common.hpp"
 #include "launch.hpp"
@@ -17,6 +18,55 @@ constexpr int kEighths = 8;  // the row blocks are dealt to eight XCDs; DLSPM_HI
 // stats: [0] longest row, [1] rows without nonzeros, [2] widest row (largest - smallest column + 1),
 // [3 .. 10] smallest column of each eighth of the rows, [11 .. 18] largest, [19 .. 26] nonzeros of each eighth
 constexpr int kStats = 3 + 3 * kEighths;
+
+// Where the kernel leaves its figures: one of 64 slots of a static device array (32 ints each), taken for the length of
+// one call. An allocation per call would cost the host ten times what the pass itself does (hipMalloc + hipFree: about
+// 0.4 ms). With all 64 slots in use at once (64 host threads inside dlspm_analyze) a call allocates after all.
+constexpr int kSlots = 64, kSlotInts = 32;
+static_assert(kStats <= kSlotInts, "a slot holds the figures of one call");
+static __device__ __align__(256) int g_analyze_slots[kSlots * kSlotInts];
+
+struct SlotPool {
+    std::mutex mutex;
+    unsigned long long busy[64] = {};  // per device: bit s set = slot s is in use
+    int* base[64] = {};                // per device: the array's address on that device
+};
+SlotPool& slot_pool()
+{
+    static SlotPool pool;
+    return pool;
+}
+// A free slot of the current device's array (nullptr: none free, or the address cannot be had); *slot names it for release.
+int* acquire_slot(int dev, int* slot)
+{
+    *slot = -1;
+    if (dev < 0 || dev >= 64) return nullptr;
+    SlotPool& pool = slot_pool();
+    std::lock_guard<std::mutex> lock(pool.mutex);
+    if (!pool.base[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_analyze_slots)) != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        pool.base[dev] = static_cast<int*>(p);
+    }
+    for (int s = 0; s < kSlots; ++s) {
+        if (!(pool.busy[dev] >> s & 1ull)) {
+            pool.busy[dev] |= 1ull << s;
+            *slot = s;
+            return pool.base[dev] + s * kSlotInts;
+        }
+    }
+    return nullptr;
+}
+void release_slot(int dev, int slot)
+{
+    if (slot < 0) return;
+    SlotPool& pool = slot_pool();
+    std::lock_guard<std::mutex> lock(pool.mutex);
+    pool.busy[dev] &= ~(1ull << slot);
+}
 
 __global__ void analyze_init_kernel(int* __restrict__ stats)
 {
@@ -113,9 +163,14 @@ int dlspm_analyze(int M, int K, int nnz, const int* row_offsets, const int* col_
     const DeviceInfo& dev = device_info();
     if (!dev.present || !dev.gfx950) return DLSPM_E_NO_DEVICE;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    int* d = nullptr;
-    hipError_t e = hipMalloc(&d, kStats * sizeof(int));
+    int device = -1, slot = -1;
+    hipError_t e = hipGetDevice(&device);
     if (e != hipSuccess) return fail_hip(e);
+    int* d = acquire_slot(device, &slot);
+    if (!d) {
+        e = hipMalloc(&d, kStats * sizeof(int));
+        if (e != hipSuccess) return fail_hip(e);
+    }
     int h[kStats] = {};
     hipLaunchKernelGGL(analyze_init_kernel, dim3(1), dim3(64), 0, s, d);
     e = hipGetLastError();
@@ -130,7 +185,8 @@ int dlspm_analyze(int M, int K, int nnz, const int* row_offsets, const int* col_
     }
     if (e == hipSuccess) e = hipMemcpyAsync(h, d, kStats * sizeof(int), hipMemcpyDeviceToHost, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);
-    (void)hipFree(d);
+    if (slot >= 0) release_slot(device, slot);
+    else (void)hipFree(d);
     if (e != hipSuccess) return fail_hip(e);
     info->max_row_len = h[0];
     info->empty_rows = h[1];

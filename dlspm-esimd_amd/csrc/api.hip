@@ -257,15 +257,23 @@ void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, co
     const double avg = M > 0 ? (double)nnz / M : 0.0;
     const long long work_rows = (long long)M * col_tiles;
     W = rule.w8_few_rows_avg > 0 && work_rows < 2 * cus && avg >= rule.w8_few_rows_avg && rule_on(kRuleEightWavesFewRows) ? 8 : 4;
-    // very long rows in a tall matrix: sixteen waves per row gain 5-8 % in SpMM (24576 and 32768 rows of ~2000
-    // nonzeros); with 8192 rows they lose as much, and the fused kernel loses 25-50 % with them at any height
-    if (rule.w16_long_rows && avg >= 1536.0 && work_rows >= 64 * cus && rule_on(kRuleSixteenWavesTallLongRows)) W = 16;
-    // few rows, each long (pruned ResNet-50 layers at small batch): four waves per row leave the device with a
-    // couple of waves per SIMD, each walking hundreds of steps in sequence (measured 15-25 % slower); a step
-    // takes `slots` nonzeros of the row at once
-    const double steps = avg / (rule.slots > 0 ? rule.slots : 1);
-    if (work_rows < 4 * cus && steps >= 768.0 && rule_on(kRuleMoreWavesFewLongRows)) W = 16;
-    else if (work_rows < 4 * cus && steps >= 384.0 && W < 8 && rule_on(kRuleMoreWavesFewLongRows)) W = 8;
+    // Very long rows (SpMM only; times inside a graph, rule on / off):
+    //  * in a tall matrix sixteen waves per row gain 4-13 % from 24576 rows of ~1600 nonzeros on (24576 x 8192 at density
+    //    0.2, N = 128: 792 / 840 us; 32768 x 8192 at 0.3, N = 32: 475 / 551 us); at 16384 rows they gain nothing and keep
+    //    the even-rows grouping from applying (N = 128: 490 / 453 us under the hint), hence from 96 rows per compute unit on;
+    //  * in few rows (pruned ResNet-50 layers at small batch): four waves per row leave the device with a couple of waves
+    //    per SIMD, each walking hundreds of steps in sequence (256 x 8192 at 0.5, N = 128: 23.4 / 32.3 us; 128 x 4608,
+    //    N = 256: 24.1 / 34.3 us); with two rows per compute unit the same choice loses (512 x 8192 at 0.25, N = 256:
+    //    45.9 / 39.9 us), hence up to one and a half. A step takes `slots` nonzeros of the row at once.
+    // SDDMM is indifferent to both (within 1 %) and loses the even-rows grouping to the first (24576 x 8192 at 0.2, D = 256,
+    // under the hint: 2586 / 1577 us); the fused op loses 3-17 % with the second (512 x 8192, D = 256: 87.2 / 72.8 us) and
+    // 25-50 % with the first.
+    if (rule.more_waves_long_rows) {
+        if (avg >= 1536.0 && work_rows >= 96 * cus && rule_on(kRuleSixteenWavesTallLongRows)) W = 16;
+        const double steps = avg / (rule.slots > 0 ? rule.slots : 1);
+        if (2 * work_rows <= 3 * cus && steps >= 768.0 && rule_on(kRuleMoreWavesFewLongRows)) W = 16;
+        else if (2 * work_rows <= 3 * cus && steps >= 384.0 && W < 8 && rule_on(kRuleMoreWavesFewLongRows)) W = 8;
+    }
     if (W > rule.max_w) W = rule.max_w;
     R = 1;
     if (W == 4) {

@@ -218,14 +218,14 @@ hipError_t fused_sliced_launch(const FusedArgs& x, const FusedShape& s, const Sl
                                hipStream_t stream);
 
 // Picks (W, R), W <= max_w: waves per workgroup from the number of rows, rows per workgroup as large as keeps
-// `blocks_per_cu` workgroups per compute unit in the grid. `slots` = nonzeros of a row a wave works on at once (64 / G); `w16_long_rows`:
-// the op gains from sixteen waves per row on tall matrices of very long rows; `w8_few_rows_avg`: see below. `rows_even`: the caller knows that no
+// `blocks_per_cu` workgroups per compute unit in the grid. `slots` = nonzeros of a row a wave works on at once (64 / G); `more_waves_long_rows`:
+// the op gains from more waves per row where rows are very long (SpMM only, see choose_split); `w8_few_rows_avg`: see below. `rows_even`: the caller knows that no
 // row is much longer than the mean. Only the pairs the kernels are instantiated for are returned.
 struct SplitRule {
     int blocks_per_cu;
     int max_w;
     int slots;
-    bool w16_long_rows;
+    bool more_waves_long_rows;
     int w8_few_rows_avg = 0;  // > 0: eight waves per row from this many nonzeros per row on where there are few rows
     int even_rows_avg = 128;  // rows known to be even are grouped four to a workgroup from this many nonzeros per row on
 };

@@ -172,7 +172,7 @@ SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
         s.G1 = 4;
         s.DS = 1;
     }
-    choose_split(dev, M, 1, nnz, SplitRule{2, 16, kWave / s.G1, true, 96}, rows_even, s.W, s.R);
+    choose_split(dev, M, 1, nnz, SplitRule{2, 16, kWave / s.G1, false, 96}, rows_even, s.W, s.R);
     return s;
 }
 

@@ -11,6 +11,9 @@
 //           reference times its kernels (20 single launches, SPMM/spmm-esimd-fromfile2.cpp:194-243): n calls through
 //           the function pointer, no synchronisation in between, wall time / n; and the same loop over an empty
 //           kernel, which is what the HIP runtime's launch alone costs.
+//   floor   what a launch costs the DEVICE before any arithmetic: an empty kernel of a given grid, and a kernel that only
+//           walks the dependent loads every row-block kernel starts with (two row offsets -> 64 column indices -> one
+//           1 KiB dense row -> one store). Timed by bench.py between the nodes of a HIP graph, like the ops themselves.
 // The reference's nearest relative is the cache-flush copy kernel of SDDMM/tprint.cpp:65-72.
 #include <hip/hip_runtime.h>
 #include <stddef.h>
@@ -58,6 +61,25 @@ __global__ __launch_bounds__(256) void dlspm_probe_copy_kernel(const float4* __r
 }
 
 __global__ void dlspm_probe_empty_kernel(int) {}
+
+// depth 0: the row offsets only; 1: + 64 column indices per wave; 2: + the dense row of the first of them; 3: + the store
+__global__ __launch_bounds__(256) void dlspm_probe_chain_kernel(int M, const int* __restrict__ ro, const int* __restrict__ ci,
+                                                                const float* __restrict__ B, float* __restrict__ C, int depth)
+{
+    const int row = blockIdx.x % M, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int rs = ro[row], re = ro[row + 1];
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (depth >= 1 && re > rs) {
+        const int c = ci[min(rs + lane + 64 * w, re - 1)];
+        if (depth >= 2) {
+            const int first = __builtin_amdgcn_readfirstlane(c);
+            acc = *reinterpret_cast<const float4*>(B + (size_t)first * 256 + lane * 4);
+        } else {
+            acc.x = (float)c;
+        }
+    }
+    if ((depth >= 3 || acc.x == 12345.678f) && w == 0) *reinterpret_cast<float4*>(C + (size_t)row * 256 + lane * 4) = acc;
+}
 
 template <typename F> double per_call_us(int n, F&& call)
 {
@@ -109,6 +131,23 @@ double dlspm_probe_enqueue_fused(void* fn, int n, int M, int K, int D, int nnz, 
 double dlspm_probe_enqueue_empty(int n, void* stream)
 {
     return per_call_us(n, [&] { hipLaunchKernelGGL(dlspm_probe_empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), 0); });
+}
+
+// One launch of the floor kernels. depth < 0: the empty kernel with `workgroups` x `threads`; depth 0 ... 3: the chain kernel
+// (256 threads) over a CSR matrix of M rows whose column indices are < the rows of B (B and C have 256 floats per row, C has M rows).
+int dlspm_probe_floor(int workgroups, int threads, int depth, int M, const int* ro, const int* ci, const float* B, float* C,
+                      void* stream)
+{
+    if (workgroups < 1 || depth > 3) return (int)hipErrorInvalidValue;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (depth < 0) {
+        if (threads < 1 || threads > 1024) return (int)hipErrorInvalidValue;
+        hipLaunchKernelGGL(dlspm_probe_empty_kernel, dim3(workgroups), dim3(threads), 0, st, 0);
+    } else {
+        if (M < 1 || !ro || !ci || !B || !C) return (int)hipErrorInvalidValue;
+        hipLaunchKernelGGL(dlspm_probe_chain_kernel, dim3(workgroups), dim3(256), 0, st, M, ro, ci, B, C, depth);
+    }
+    return (int)hipGetLastError();
 }
 
 // One launch: `blocks` workgroups of four waves, every wave gathers iters x 8 rows of 256 floats from `table`

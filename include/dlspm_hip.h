@@ -24,49 +24,35 @@
  *     SDDMM/sddmm-esimd-fromfile_v4.hpp:161,175);
  *   - errors are returned as a negative status, nothing is thrown across the ABI (the reference
  *     throws std::invalid_argument / std::logic_error on the host before launching).
- *   - `workspace` is optional device memory owned by the caller. NULL (or 0 bytes) is always valid and
- *     selects the schedule that needs none. A caller that passes at least dlspm_workspace_bytes()
- *     bytes lets SpMM and the fused op use the flat schedule where the library's size rule allows it
- *     (from about half a million nonzeros, 64 per row on average, dense width above 64: every wave then
- *     owns a fixed run of nonzeros, however they are spread over the rows, and a second kernel adds the
- *     partial rows kept in the workspace, in a fixed order), or, when the dense operands gathered per
- *     nonzero exceed 4 MiB together (K x N floats in SpMM, K x D in SDDMM, twice K x D in the fused op), the
- *     column-sliced schedule (the column ranges of the sparse matrix one after the other, so that the
- *     part of the dense operands in use fits the cache; partial rows per range in the workspace, added
- *     in range order; SDDMM keeps only the range boundaries there). The flat schedule is the faster one when row
- *     lengths are uneven and the slower one when they are even, so pass the workspace for matrices
- *     whose longest row is several times the mean (dlspm_csr_row_stats) and NULL otherwise. A non-NULL
- *     workspace smaller than that is refused with DLSPM_E_WORKSPACE. The contents need no
- *     initialisation and mean nothing afterwards; two calls that share a workspace must not overlap
- *     in time.
- *   - Three more things travel through the same pair of arguments, as hint bits in the upper byte of `workspace_bytes`
- *     (DLSPM_HINT_*, or-ed into the size; they are no part of the size):
+ *   - `workspace` is optional device memory owned by the caller. NULL (or 0 bytes) is always valid and selects the
+ *     schedule that needs none. What else can travel through (workspace, workspace_bytes) -- schedule memory, a row plan,
+ *     a cut plan, or hints about the matrix in the upper byte of the size -- is decided in one place: dlspm_analyze looks
+ *     at the matrix once, dlspm_advise says what to allocate, build and pass for an op and a width (below). The
+ *     thresholds behind that advice live in the library's code only. A non-NULL workspace smaller than the call needs is
+ *     refused with DLSPM_E_WORKSPACE. Schedule memory needs no initialisation and means nothing afterwards; two calls that
+ *     share it must not overlap in time.
+ *       schedule memory (dlspm_workspace_bytes() bytes, no hint): lets SpMM and the fused op use the flat schedule on large
+ *         matrices (every wave owns a fixed run of nonzeros, however they are spread over the rows; a second kernel adds
+ *         the partial rows kept in the workspace, in a fixed order: the faster schedule for very uneven rows, the slower
+ *         one for even rows), and all three ops the column-sliced schedule where the dense operands gathered per nonzero
+ *         exceed one L2 (the column ranges of the sparse matrix one after the other, so that the part of the operands in
+ *         use fits the cache; partial rows per range in the workspace, added in range order; SDDMM keeps only the range
+ *         boundaries there).
  *       DLSPM_HINT_ROWS_EVEN, with workspace NULL: the caller knows that no row is much longer than the mean (longest
- *         row at most one and a half times nnz / M). Tall matrices of long rows (from 2048 rows of 128 nonzeros; SpMM
- *         from 256 columns on: of about a hundred) then run one whole row per wave, which
- *         is the faster split for even rows and the slower one for uneven rows. It is a hint about speed only: a wrong
- *         one costs time, never correctness (a row's products are added in a different, equally fixed order), and
- *         other sizes ignore it.
+ *         row at most one and a half times nnz / M). Tall matrices of long rows then run one whole row per wave, which
+ *         is the faster split for even rows and the slower one for uneven rows. A hint about speed only: a wrong one
+ *         costs time, never correctness (a row's products are added in a different, equally fixed order).
  *       DLSPM_HINT_ROW_PLAN: `workspace` holds the row plan of this matrix (dlspm_row_plan_build, below; at least
  *         dlspm_row_plan_bytes(M) bytes, else DLSPM_E_WORKSPACE) and the launch hands the rows out in the plan's order.
  *         The plan is only read.
- *       DLSPM_HINT_BANDED: the caller knows that the columns of every row lie in a window much narrower than K that
- *         moves down the columns with the row (sliding-window and block-diagonal attention masks, banded matrices).
- *         Neighbouring rows then gather neighbouring dense rows: the row blocks are dealt to the XCDs in contiguous
- *         runs, so that each L2 fetches its own share of the K-side operands and not all of them, and the call runs as
- *         row blocks whatever memory comes with it (column slices and column tiles are answers to columns spread over
- *         all of K). Measured on MI355X, K = V = 16384 x 128 floats (8 MiB each), 128 columns per row: the fused op
- *         104 us as dlspm_workspace_advice, which cannot see the band, says (three column slices), 77 us with NULL,
- *         74 us with this hint; the L2s fetch 33 MiB per launch instead of 145 MiB. A wrong hint costs time (rows whose
- *         length depends on their position load the XCDs unevenly), never correctness: the bits are those of the call
- *         with NULL. May be combined with DLSPM_HINT_ROWS_EVEN; a row plan takes precedence.
- *       DLSPM_HINT_CUT_PLAN: `workspace` holds a cut plan (dlspm_row_plan_build_cut, below).
- *       DLSPM_HINT_ROWS_SKEWED, with a row plan: the caller knows that the longest row is at least twenty times the mean.
- *         SDDMM and the fused op then run one row per workgroup in plan order also for masks of 16 to 64 rows per compute
- *         unit (4096 < M <= 16384 on an MI355X), where the sizes alone would group several rows per workgroup (faster for
- *         moderately uneven rows, 0.63-0.93 of the time for very uneven ones). Speed only; other sizes ignore it.
- *     A bit of that byte that has no meaning, or a combination that has none (both kinds of plan, a plan of 2^48 bytes and
- *     more, even and skewed rows at once), is refused with DLSPM_E_INVALID_ARG.
+ *       DLSPM_HINT_BANDED: the columns of every row lie in a window much narrower than K that moves down the columns
+ *         with the row (sliding-window and block-diagonal attention masks, banded matrices). Neighbouring rows then
+ *         gather neighbouring dense rows: the row blocks are dealt to the XCDs in contiguous runs, so that each L2
+ *         fetches its own share of the K-side operands and not all of them, and the call runs as row blocks whatever
+ *         memory comes with it. Measured on MI355X, K = V = 16384 x 128 floats, 128 columns per row: the fused op 104 us
+ *         in column slices, 77 us with NULL, 74 us with this hint; the L2s fetch 33 MiB per launch instead of 145 MiB.
+ *         A wrong hint costs time, never correctness: the bits are those of the call with NULL. May be combined with
+ *         DLSPM_HINT_ROWS_EVEN; a row plan takes precedence. dlspm_advise detects bands from the matrix.
  * Calls on different streams may run concurrently from different host threads (each with its own
  * workspace). The library's only mutable state is per host thread (the tuning overrides of dlspm_set_tuning and the
  * last HIP error), a cache of the devices' properties, and the static scratch array of spmm_csr_f32_static.
@@ -237,9 +223,7 @@ int dlspm_advise(int op, int N_or_D, const dlspm_matrix_info* info, dlspm_call_p
  * pointer may be NULL). Synchronises `stream`; meant to be called once per matrix, like dlspm_csr_check. It
  * has no counterpart in the reference, whose launch sizing looks at M and N only
  * (SPMM/spmmesimd2.hpp:30-60).
- * Use: the compute calls cannot see how evenly the nonzeros are spread over the rows; a caller who finds
- * max_row_len at least four times nnz / M should pass a workspace, one who finds it at most one and a half times
- * nnz / M may pass DLSPM_HINT_ROWS_EVEN (see above), anyone else NULL.
+ * Use: dlspm_workspace_advice and dlspm_row_plan_advice take the longest row (dlspm_analyze returns it too).
  */
 int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_row_len, int* empty_rows);
 
@@ -301,12 +285,11 @@ size_t dlspm_row_plan_bytes(int M);
  */
 size_t dlspm_row_plan_bytes_for(int op, int M, int N_or_D);
 int dlspm_row_plan_build_cut(int M, const int* row_offsets, void* plan, size_t plan_bytes, void* stream);
-/* 1 if a row plan is worth building for op (DLSPM_OP_*) at these sizes and this longest row (-1: unknown): the planned
- * launch would use it (one column tile, rows of at least 32 nonzeros on average where the size rule would group rows;
- * SDDMM and the fused op: 16 < D <= 512, up to 2048 rows also shorter rows), the rows are not known to be even (SDDMM
- * on rows below 32 nonzeros: the longest is at least eight times the mean), and B is not so far beyond one L2 that the
- * column-sliced schedule's workspace matters more; else 0. Ask this before dlspm_workspace_advice: where both a plan and the flat schedule's workspace apply, the plan
- * is 10-40 % faster. */
+/* Whether a plan is worth building for op (DLSPM_OP_*) at these sizes and this longest row (-1: unknown): 0 no (the
+ * planned launch is not built for the shape, the rows are known to be even, or the dense operands are so far beyond one
+ * L2 that the column-sliced schedule's workspace matters more), 1 a row plan, 2 a cut plan. One of the questions
+ * dlspm_advise asks; a caller that passes DLSPM_HINT_ROWS_SKEWED with the plan (longest row at least twenty times the
+ * mean) gets the answer for that launch by passing such a longest row here. */
 int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row_len);
 int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_bytes, void* stream);
 int spmm_csr_f32_planned(int M, int K, int N, int nnz, const int* row_offsets, const int* col_indices,
@@ -321,11 +304,11 @@ int fused_sddmm_spmm_f32_planned(int M, int K, int D, int nnz, const int* row_of
 /*
  * What to pass as `workspace` for a matrix of these sizes whose longest row has max_row_len nonzeros (from
  * dlspm_csr_row_stats, or known to the caller): DLSPM_PASS_NULL, DLSPM_PASS_ROWS_EVEN (NULL with DLSPM_HINT_ROWS_EVEN)
- * or DLSPM_PASS_WORKSPACE (dlspm_workspace_bytes() bytes of device memory). It holds the measured rules in one place:
- * the memory where the column-sliced schedule applies (except even rows at two slices in SpMM and the fused op) or
- * where the longest row is at least four times the mean and the flat schedule applies; the constant where the
- * longest row is at most one and a half times the mean; NULL otherwise. Host-only; a negative max_row_len means
- * "unknown" and gives the memory only for the column-sliced schedule. No counterpart in the reference.
+ * or DLSPM_PASS_WORKSPACE (dlspm_workspace_bytes() bytes of device memory): the memory where the column-sliced schedule
+ * applies, or where the rows are very uneven and the flat schedule applies; the hint where the rows are even; NULL
+ * otherwise. Host-only; a negative max_row_len means "unknown" and gives the memory only for the column-sliced
+ * schedule. One of the questions dlspm_advise asks (after dlspm_row_plan_advice: where a plan applies it is the faster
+ * answer). No counterpart in the reference.
  */
 #define DLSPM_PASS_NULL       0
 #define DLSPM_PASS_ROWS_EVEN  1

@@ -6,7 +6,8 @@ the same launches are timed again.
 
 Cases: the five benchmark configurations; the reference's 12-shape benchmark grid (SPMM/spmm-esimd-allbenchs.cpp:252-255)
 at density 0.1 with N = D = 32 and 128 (Bernoulli patterns); lognormal row lengths (sigma 1) on 2048 ... 16384 rows; layer
-shapes of 64 ... 512 rows as in the reference's dlmc/ tree. Every case is launched as a driver would (dlspm_analyze ->
+shapes of 64 ... 512 rows as in the reference's dlmc/ tree; very long rows in a tall matrix (16384 x 8192 at density 0.2) and in
+few rows (256 ... 512 rows of 2048 ... 4096 nonzeros), which is where the rules that add waves per row apply. Every case is launched as a driver would (dlspm_analyze ->
 dlspm_advise -> allocate -> build), inside a HIP graph of 20 launches (median of 7 double replays). With a rule off the
 preparation is repeated, so that sizes and advice follow the changed rules. The launches with all rules on are timed
 before and after the others (after one untimed run) and their mean is the reference. One line per rule and op: the geometric mean
@@ -55,6 +56,13 @@ def cases(dl, quick):
     for (M, K, mean) in ((64, 576, 400.0), (128, 1152, 200.0), (256, 2304, 200.0), (512, 512, 50.0), (512, 2048, 100.0)):
         ro, ci = dl.make_pattern(dl.PATTERN_LOGNORMAL_ROWS, 9, M, K, mean, 0.5)
         out.append((f"layer {M}x{K} mean {mean:.0f} sigma 0.5 width 256/128/64", None, M, K, -1, ro, ci))
+    if not quick:
+        ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 11, 16384, 8192, 0.2)
+        for width in (32, 128):
+            out.append((f"tall, long rows 16384x8192 density 0.2 width {width}", None, 16384, 8192, width, ro, ci))
+        for (M, K, density) in ((256, 8192, 0.5), (512, 8192, 0.25)):
+            ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 13, M, K, density)
+            out.append((f"few long rows {M}x{K} density {density} width 256/128/64", None, M, K, -1, ro, ci))
     return out
 
 

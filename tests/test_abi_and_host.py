@@ -76,8 +76,15 @@ def test_split_rule_and_the_even_rows_hint(dl):
     long_rows = 2000
     assert dl.describe_launch(dl.OP_SPMM, 8192, 8192, 128, 8192 * long_rows)["W"] == 4
     assert dl.describe_launch(dl.OP_SPMM, 24576, 8192, 128, 24576 * long_rows)["W"] == 16
-    assert dl.describe_launch(dl.OP_FUSED, 24576, 8192, 128, 24576 * long_rows)["W"] == 4
-    assert dl.describe_launch(dl.OP_FUSED, 300, 8192, 32, 300 * 7000)["W"] == 16  # few rows, very long: still sixteen
+    assert dl.describe_launch(dl.OP_SPMM, 16384, 8192, 128, 16384 * long_rows)["W"] == 4  # sixteen only from 96 rows per compute unit on
+    for op in (dl.OP_SDDMM, dl.OP_FUSED):  # the rules that add waves for very long rows are SpMM's alone
+        assert dl.describe_launch(op, 24576, 8192, 128, 24576 * long_rows)["W"] == 4
+        assert dl.describe_launch(op, 24576, 8192, 128, 24576 * long_rows, rows_even=True)["R"] == 4
+        assert dl.describe_launch(op, 300, 8192, 32, 300 * 7000)["W"] == 8  # (eight: few rows of a hundred nonzeros and more)
+    # few rows, very long: sixteen waves per row in SpMM, up to one and a half rows per compute unit
+    assert dl.describe_launch(dl.OP_SPMM, 300, 8192, 32, 300 * 7000)["W"] == 16
+    assert dl.describe_launch(dl.OP_SPMM, 384, 8192, 256, 384 * 2048)["W"] == 16
+    assert dl.describe_launch(dl.OP_SPMM, 512, 8192, 256, 512 * 2048)["W"] == 4
 
 
 def test_split_rule_for_small_matrices(dl):
