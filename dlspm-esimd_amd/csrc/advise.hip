@@ -20,8 +20,10 @@ constexpr int kEighths = 8;  // the row blocks are dealt to eight XCDs; DLSPM_HI
 constexpr int kStats = 3 + 3 * kEighths;
 
 // Where the kernel leaves its figures: one of 64 slots of a static device array (32 ints each), taken for the length of
-// one call. An allocation per call would cost the host ten times what the pass itself does (hipMalloc + hipFree: about
-// 0.4 ms). With all 64 slots in use at once (64 host threads inside dlspm_analyze) a call allocates after all.
+// one call, and the same slot of a pinned host array (8 KiB per device, allocated at the first call on that device and
+// kept) for the copy back. An allocation per call would cost the host several times what the pass itself does
+// (hipMalloc + hipFree: about 0.4 ms; a copy into pageable memory: 0.06 ms). With all 64 slots in use at once (64 host
+// threads inside dlspm_analyze) a call allocates after all.
 constexpr int kSlots = 64, kSlotInts = 32;
 static_assert(kStats <= kSlotInts, "a slot holds the figures of one call");
 static __device__ __align__(256) int g_analyze_slots[kSlots * kSlotInts];
@@ -30,16 +32,19 @@ struct SlotPool {
     std::mutex mutex;
     unsigned long long busy[64] = {};  // per device: bit s set = slot s is in use
     int* base[64] = {};                // per device: the array's address on that device
+    int* host[64] = {};                // per device: pinned host memory, slot for slot (nullptr: could not be had)
 };
 SlotPool& slot_pool()
 {
     static SlotPool pool;
     return pool;
 }
-// A free slot of the current device's array (nullptr: none free, or the address cannot be had); *slot names it for release.
-int* acquire_slot(int dev, int* slot)
+// A free slot of the current device's array (nullptr: none free, or the address cannot be had); *slot names it for
+// release, *pinned is the slot's host side (nullptr: copy into ordinary memory).
+int* acquire_slot(int dev, int* slot, int** pinned)
 {
     *slot = -1;
+    *pinned = nullptr;
     if (dev < 0 || dev >= 64) return nullptr;
     SlotPool& pool = slot_pool();
     std::lock_guard<std::mutex> lock(pool.mutex);
@@ -50,11 +55,15 @@ int* acquire_slot(int dev, int* slot)
             return nullptr;
         }
         pool.base[dev] = static_cast<int*>(p);
+        void* h = nullptr;
+        if (hipHostMalloc(&h, sizeof(int) * kSlots * kSlotInts, hipHostMallocDefault) == hipSuccess) pool.host[dev] = static_cast<int*>(h);
+        else (void)hipGetLastError();
     }
     for (int s = 0; s < kSlots; ++s) {
         if (!(pool.busy[dev] >> s & 1ull)) {
             pool.busy[dev] |= 1ull << s;
             *slot = s;
+            if (pool.host[dev]) *pinned = pool.host[dev] + s * kSlotInts;
             return pool.base[dev] + s * kSlotInts;
         }
     }
@@ -166,18 +175,22 @@ int dlspm_analyze(int M, int K, int nnz, const int* row_offsets, const int* col_
     int device = -1, slot = -1;
     hipError_t e = hipGetDevice(&device);
     if (e != hipSuccess) return fail_hip(e);
-    int* d = acquire_slot(device, &slot);
+    int* pinned = nullptr;
+    int* d = acquire_slot(device, &slot, &pinned);
     if (!d) {
         e = hipMalloc(&d, kStats * sizeof(int));
         if (e != hipSuccess) return fail_hip(e);
     }
-    int h[kStats] = {};
+    int pageable[kStats] = {};
+    int* h = pinned ? pinned : pageable;
     hipLaunchKernelGGL(analyze_init_kernel, dim3(1), dim3(64), 0, s, d);
     e = hipGetLastError();
     if (e == hipSuccess) {
-        // about 16 waves per compute unit, each a run of rows
-        const long long waves_wanted = std::max<long long>(16ll * dev.cus, 1);
-        const int rows_per_wave = (int)std::max<long long>(ceil_div(M, waves_wanted), 1);
+        // One to sixteen waves per compute unit, each a run of rows, about 2048 nonzeros per wave: every wave ends with a
+        // handful of atomic operations on the same few words, which is what a small matrix would otherwise wait for
+        // (2048 rows of 50 nonzeros: 117 us of host time per call with a wave per row, 44 us with eight rows per wave).
+        const long long waves_wanted = std::min<long long>(16ll * dev.cus, std::max<long long>(dev.cus, nnz / 2048));
+        const int rows_per_wave = (int)std::max<long long>(ceil_div(M, std::max<long long>(waves_wanted, 1)), 1);
         const long long waves = ceil_div(M, rows_per_wave);
         hipLaunchKernelGGL(analyze_kernel, dim3((unsigned)ceil_div(waves, 4)), dim3(256), 0, s, M, K, rows_per_wave, row_offsets,
                            col_indices, d);
@@ -185,6 +198,9 @@ int dlspm_analyze(int M, int K, int nnz, const int* row_offsets, const int* col_
     }
     if (e == hipSuccess) e = hipMemcpyAsync(h, d, kStats * sizeof(int), hipMemcpyDeviceToHost, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);
+    int got[kStats];
+    for (int i = 0; i < kStats; ++i) got[i] = h[i];
+    h = got;  // (the slot, and with it the pinned memory, goes back before the figures are used)
     if (slot >= 0) release_slot(device, slot);
     else (void)hipFree(d);
     if (e != hipSuccess) return fail_hip(e);

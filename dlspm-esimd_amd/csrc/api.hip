@@ -55,6 +55,8 @@ static Tuning tuning_from_environment()
     number("DLSPM_CUT_PIECE_PCT", t.cut_piece_pct);
     number("DLSPM_CUT_LONGEST_PCT", t.cut_longest_pct);
     number("DLSPM_RULES_OFF", t.rules_off);
+    number("DLSPM_COMPUTE_UNITS", t.compute_units);
+    if (t.compute_units < 8 || t.compute_units > 1024 || t.compute_units % 8 != 0) t.compute_units = 0;
     return t;
 }
 static const Tuning& process_tuning()
@@ -69,7 +71,7 @@ const Tuning& tuning() { return t_tuning_set ? t_tuning : process_tuning(); }
 // ---- the current device ----------------------------------------------------------------------------------------------
 constexpr int kMaxDevices = 64;
 static const DeviceInfo kNoDevice{256, 4ll << 20, false, false};
-const DeviceInfo& device_info()
+static const DeviceInfo& current_device_info()
 {
     static std::mutex mutex;
     static DeviceInfo cache[kMaxDevices];
@@ -102,6 +104,17 @@ const DeviceInfo& device_info()
     t_last_dev = dev;
     t_last_info = &cache[dev];
     return cache[dev];
+}
+// (with dlspm_tuning.compute_units set: the same device with that many compute units, for this host thread)
+const DeviceInfo& device_info()
+{
+    const DeviceInfo& real = current_device_info();
+    const int cus = tuning().compute_units;
+    if (cus <= 0) return real;
+    static thread_local DeviceInfo t_resized;
+    t_resized = real;
+    t_resized.cus = cus;
+    return t_resized;
 }
 // DLSPM_OK if the current device can run the kernels
 static int require_device(const DeviceInfo& d) { return d.present && d.gfx950 ? DLSPM_OK : DLSPM_E_NO_DEVICE; }
@@ -384,7 +397,7 @@ void dlspm_tuning_default(dlspm_tuning* t)
     if (!t) return;
     const Tuning d;
     *t = dlspm_tuning{d.split_w, d.split_r, d.flat, d.flat_chunk, d.slices, d.tile_major, d.tile_width, d.plan_order,
-                      d.xcd_contiguous, d.stream_results, d.cut_piece_pct, d.cut_longest_pct, d.rules_off};
+                      d.xcd_contiguous, d.stream_results, d.cut_piece_pct, d.cut_longest_pct, d.rules_off, d.compute_units};
 }
 
 int dlspm_set_tuning(const dlspm_tuning* t)
@@ -397,7 +410,8 @@ int dlspm_set_tuning(const dlspm_tuning* t)
         t->tile_major < -1 || t->tile_major > 1 || t->tile_width < 0 || t->plan_order < 0 || t->plan_order > 2 ||
         t->xcd_contiguous < 0 || t->xcd_contiguous > 1 || t->stream_results < -1 || t->stream_results > 1 ||
         (t->cut_piece_pct != 0 && (t->cut_piece_pct < 10 || t->cut_piece_pct > 1000)) ||
-        (t->cut_longest_pct != 0 && (t->cut_longest_pct < 10 || t->cut_longest_pct > 1000)) || t->rules_off < 0 || t->rules_off > 127)
+        (t->cut_longest_pct != 0 && (t->cut_longest_pct < 10 || t->cut_longest_pct > 1000)) || t->rules_off < 0 || t->rules_off > 127 ||
+        (t->compute_units != 0 && (t->compute_units < 8 || t->compute_units > 1024 || t->compute_units % 8 != 0)))
         return DLSPM_E_INVALID_ARG;
     t_tuning.split_w = t->split_w;
     t_tuning.split_r = t->split_r;
@@ -412,6 +426,7 @@ int dlspm_set_tuning(const dlspm_tuning* t)
     t_tuning.cut_piece_pct = t->cut_piece_pct;
     t_tuning.cut_longest_pct = t->cut_longest_pct;
     t_tuning.rules_off = t->rules_off;
+    t_tuning.compute_units = t->compute_units;
     t_tuning_set = true;
     return DLSPM_OK;
 }
@@ -421,7 +436,7 @@ int dlspm_get_tuning(dlspm_tuning* t)
     if (!t) return DLSPM_E_INVALID_ARG;
     const Tuning& c = tuning();
     *t = dlspm_tuning{c.split_w, c.split_r, c.flat, c.flat_chunk, c.slices, c.tile_major, c.tile_width, c.plan_order,
-                      c.xcd_contiguous, c.stream_results, c.cut_piece_pct, c.cut_longest_pct, c.rules_off};
+                      c.xcd_contiguous, c.stream_results, c.cut_piece_pct, c.cut_longest_pct, c.rules_off, c.compute_units};
     return DLSPM_OK;
 }
 

@@ -94,6 +94,7 @@ struct Tuning {
     int stream_results = -1;
     int cut_piece_pct = 0, cut_longest_pct = 0;
     int rules_off = 0;  // DLSPM_RULE_* bits: size rules switched off, to measure what each is worth
+    int compute_units = 0;  // > 0: device_info() reports this many compute units instead of the device's own
 };
 // (the values of DLSPM_RULE_* in the header)
 constexpr int kRuleEightWavesFewRows = 1, kRuleSixteenWavesTallLongRows = 2, kRuleMoreWavesFewLongRows = 4, kRuleGroupRows = 8,

@@ -77,7 +77,7 @@ class Tuning(ctypes.Structure):
     """dlspm_tuning of include/dlspm_hip.h."""
     _fields_ = [(n, ctypes.c_int) for n in ("split_w", "split_r", "flat", "flat_chunk", "slices", "tile_major",
                                             "tile_width", "plan_order", "xcd_contiguous", "stream_results",
-                                            "cut_piece_pct", "cut_longest_pct", "rules_off")]
+                                            "cut_piece_pct", "cut_longest_pct", "rules_off", "compute_units")]
 
 RULES = {"eight_waves_few_rows": 1, "sixteen_waves_tall_long_rows": 2, "more_waves_few_long_rows": 4, "group_rows": 8,
          "row_aligned_split": 16, "plan_ungroups": 32, "exact_width_kernels": 64}

@@ -375,11 +375,14 @@ typedef struct dlspm_tuning {
     int cut_longest_pct;  /* ... and the longest row that stays whole; 0 = the rule, 150. Both 10 ... 1000; they enter the  */
                           /* size of a cut plan, so set them before dlspm_row_plan_bytes_for and keep them for the launches */
     int rules_off;        /* DLSPM_RULE_* bits: size rules switched off, to measure what each is worth; 0 = all on        */
+    int compute_units;    /* 0 = the device's own; n (8 ... 1024, a multiple of 8): rules, grids and plans as on a device of n  */
+                          /* compute units -- for tests of the rules on another size of device (a partition of an MI355X); */
+                          /* results are right for any n, times are best for the true one                                  */
 } dlspm_tuning;
 /* rules that dlspm_tuning.rules_off can switch off (the others have a field of their own above) */
 #define DLSPM_RULE_EIGHT_WAVES_FEW_ROWS         1  /* SDDMM, fused: eight waves per row below two rows per compute unit     */
-#define DLSPM_RULE_SIXTEEN_WAVES_TALL_LONG_ROWS 2  /* sixteen waves per row for very long rows in a tall matrix             */
-#define DLSPM_RULE_MORE_WAVES_FEW_LONG_ROWS     4  /* eight or sixteen waves per row for few rows of very many nonzeros     */
+#define DLSPM_RULE_SIXTEEN_WAVES_TALL_LONG_ROWS 2  /* SpMM: sixteen waves per row for very long rows in a tall matrix       */
+#define DLSPM_RULE_MORE_WAVES_FEW_LONG_ROWS     4  /* SpMM: eight or sixteen waves per row for few rows of very many nonzeros */
 #define DLSPM_RULE_GROUP_ROWS                   8  /* several short rows per workgroup in tall matrices                     */
 #define DLSPM_RULE_ROW_ALIGNED_SPLIT           16  /* whole rows per wave where that is nearly as even as the even split    */
 #define DLSPM_RULE_PLAN_UNGROUPS               32  /* a planned launch runs one row per workgroup where the size rule groups */

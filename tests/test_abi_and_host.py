@@ -294,7 +294,7 @@ def test_tuning_overrides_go_through_one_call_and_the_environment_is_read_once(d
     base = dl.get_tuning()
     assert base == {"split_w": 0, "split_r": 0, "flat": -1, "flat_chunk": 0, "slices": -1, "tile_major": -1,
                     "tile_width": 0, "plan_order": 0, "xcd_contiguous": 0, "stream_results": -1, "cut_piece_pct": 0,
-                    "cut_longest_pct": 0, "rules_off": 0}
+                    "cut_longest_pct": 0, "rules_off": 0, "compute_units": 0}
     sizes = (dl.OP_SPMM, 8192, 4096, 128, 8192 * 600)
     rule = dl.describe_launch(*sizes)
     assert (rule["W"], rule["R"]) == (4, 1)
