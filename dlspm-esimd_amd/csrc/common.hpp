@@ -265,6 +265,19 @@ __host__ __device__ __forceinline__ void wave_range(bool aligned, Off&& off, int
 // The R + 1 offsets are read without LDS or a barrier: with R == 1 they are the same two words for every lane (scalar
 // loads); otherwise lane i of every wave holds offset i and v_readlane picks one.
 constexpr int kPlanNone = 0, kPlanRows = 1, kPlanPieces = 2;
+// What a cut plan says of an entry that is a piece of a row, in one word: the slot of its partial row | which piece of the
+// row it is << 15 | log2 of the number of pieces << 23. A row is cut into 2, 4, ... 256 equal pieces, and the entry
+// holds the range of the WHOLE row: piece k of c takes the nonzeros piece_range() says, or 1/c of the columns.
+constexpr int kPieceSlotMask = 0x7FFF, kPieceNumberShift = 15, kPieceNumberMask = 0xFF, kPieceCountShift = 23, kPieceCountMask = 0xF;
+constexpr int kMaxPiecesOfARow = 256;
+// piece k of 1 << lg of a row of len nonzeros: [*first, *first + *count) of the row
+__device__ __forceinline__ void piece_range(int len, int word, int* first, int* count)
+{
+    const int k = (word >> kPieceNumberShift) & kPieceNumberMask, lg = (word >> kPieceCountShift) & kPieceCountMask;
+    const int piece = (len + (1 << lg) - 1) >> lg;
+    *first = min(len, k * piece);
+    *count = min(piece, len - *first);
+}
 template <int W, int R, bool SLICED, int PLANNED>
 struct RowBlock {
     static_assert(!PLANNED || (SLICED && R == 1), "a row plan names one row per workgroup");
@@ -319,7 +332,16 @@ struct RowBlock {
                     row0 = min(max(row_ids[r0], 0), M - 1);
                     start_lo = min(max(start_lo, 0), nnz);
                     off_hi = min(max(off_hi, 0), nnz - start_lo);
-                    if constexpr (PLANNED == kPlanPieces) piece = min(row_slots[r0], slots - 1);
+                    if constexpr (PLANNED == kPlanPieces) {
+                        const int word = row_slots[r0];  // -1 a whole row, -2 nothing, else a piece of the row entered here
+                        piece = word < 0 ? word : min(word & kPieceSlotMask, slots - 1);
+                        if (word >= 0) {
+                            int first, count;
+                            piece_range(off_hi, word, &first, &count);
+                            start_lo += first;
+                            off_hi = count;
+                        }
+                    }
                 }
             } else {
                 static_assert(R + 1 <= 32, "the running sum covers 32 lanes");
@@ -329,6 +351,11 @@ struct RowBlock {
             }
         }
         prefetch();
+        split(flags);
+    }
+    // the work split of the block over its waves, from the offsets that load() left
+    __device__ __forceinline__ void split(int flags)
+    {
         T0 = off(0);
         T = off(nr) - T0;
         per = split_per_wave(T, W);
@@ -381,10 +408,22 @@ struct RowBlock {
 // timing (no atomics, no pre-zeroed output); rows without nonzeros are written as zeros.
 // kPlanPieces: an entry that is a piece of a row stores its sum to `pieces` (slot blk.piece) instead, with ordinary stores
 // (it is read again), and an entry that holds nothing leaves at once (the whole workgroup, before any barrier).
+// The window form works on the columns [col0, col_end) of rows of `width` floats, col_end - col0 <= G * VEC * V and >= VEC;
+// the tile form on column tile ct of the whole width.
+template <int VEC, int G, int V, int W, int R, bool SLICED, int PLANNED, typename Segment>
+__device__ __forceinline__ void dense_rows_window(const RowBlock<W, R, SLICED, PLANNED>& blk, int col0, int col_end, int width,
+                                                  float* __restrict__ out, Segment&& segment,
+                                                  float* __restrict__ pieces = nullptr);
 template <int VEC, int G, int V, int W, int R, bool SLICED, int PLANNED, typename Segment>
 __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PLANNED>& blk, int ct, int width,
                                                  float* __restrict__ out, Segment&& segment,
                                                  float* __restrict__ pieces = nullptr)
+{
+    dense_rows_window<VEC, G, V>(blk, ct * (G * VEC * V), width, width, out, static_cast<Segment&&>(segment), pieces);
+}
+template <int VEC, int G, int V, int W, int R, bool SLICED, int PLANNED, typename Segment>
+__device__ __forceinline__ void dense_rows_window(const RowBlock<W, R, SLICED, PLANNED>& blk, int col0, int col_end, int width,
+                                                  float* __restrict__ out, Segment&& segment, float* __restrict__ pieces)
 {
     if constexpr (PLANNED == kPlanPieces) {
         if (blk.piece < -1) return;
@@ -401,11 +440,11 @@ __device__ __forceinline__ void dense_rows_block(const RowBlock<W, R, SLICED, PL
     bool act[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-        const int col = ct * TW + (v * G + g) * VEC;
-        act[v] = col < width;
-        // a lane whose VEC columns would run past the width moves back to end there: it then repeats columns of its
-        // left neighbour, with the same operations, and stores the same values there (width >= VEC)
-        colv[v] = act[v] ? min(col, width - VEC) : 0;
+        const int col = col0 + (v * G + g) * VEC;
+        act[v] = col < col_end;
+        // a lane whose VEC columns would run past the end moves back to end there: it then repeats columns of its
+        // left neighbour, with the same operations, and stores the same values there (col_end - col0 >= VEC)
+        colv[v] = act[v] ? min(col, col_end - VEC) : 0;
     }
     auto s_off = [&](int i) { return blk.off(i); };
     const int T0 = blk.T0, T = blk.T, per = blk.per, a = blk.a;

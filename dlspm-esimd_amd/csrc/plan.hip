@@ -445,13 +445,23 @@ __device__ __forceinline__ void emit(int* __restrict__ plan, int M, long long p,
                                      const int* __restrict__ v_row, const int* __restrict__ v_slot)
 {
     const int r = (int)min(max(row, 0ll), (long long)M - 1);
-    plan[p] = row_offsets[r];
-    plan[(size_t)M + p] = row_offsets[r + 1];
     if (v_row == nullptr) {
+        plan[p] = row_offsets[r];
+        plan[(size_t)M + p] = row_offsets[r + 1];
         plan[2 * (size_t)M + p] = r;
     } else {
+        // a piece is entered with the range of its WHOLE row: the word says which of how many equal pieces it is, and a
+        // launch takes from that the piece's share of the nonzeros (piece_range) or of the columns
+        const int word = v_slot[r];
+        int first = r, last = r + 1;
+        if (word >= 0) {
+            first = max(r - ((word >> kPieceNumberShift) & kPieceNumberMask), 0);
+            last = min(first + (1 << ((word >> kPieceCountShift) & kPieceCountMask)), M);
+        }
+        plan[p] = row_offsets[first];
+        plan[(size_t)M + p] = row_offsets[last];
         plan[2 * (size_t)M + p] = v_row[r];
-        plan[3 * (size_t)M + p] = v_slot[r];
+        plan[3 * (size_t)M + p] = word;
     }
 }
 
@@ -551,12 +561,15 @@ __global__ __launch_bounds__(kPlanThreads) void plan_emit_kernel(int M, const in
 // A row longer than one compute unit's share of the nonzeros sets the time of the whole launch through the one compute
 // unit it runs on. With share = ceil(nnz / bins) (at least 1), piece = ceil(share x piece_pct / 100) and longest =
 // max(piece, ceil(share x longest_pct / 100)) (the rule: 100 and 150 per cent), a row of more than `longest` nonzeros is
-// cut into c = ceil(length / piece) pieces of ceil(length / c) nonzeros (the last one what is left; none is empty), and
+// cut into c pieces of ceil(length / c) nonzeros (the last one what is left; rows of a few nonzeros can end in empty ones), c the smallest power of two
+// with pieces of at most `piece` nonzeros (256 at most) -- a power of two, so that a launch can also give each piece the
+// row's whole length and 1/c of the COLUMNS (SpMM), and so that a piece's range follows from its row's by a shift -- and
 // the plan is built over the "virtual rows" -- the rows and pieces in matrix order -- like a plan over rows. How many
-// there can be: the cut rows hold at most nnz <= share x bins nonzeros, so their pieces number at most
-// bins x 100 / piece_pct + (cut rows), and fewer than bins x 100 / longest_pct rows can exceed `longest`; hence at most
-// ceil(bins x 100 / piece_pct) entries more than rows, whatever the matrix. The plan is sized for those bounds (entries
-// that are not needed hold nothing), so its size and the grids of its launches depend on M and the device alone.
+// there can be: ceil(length / piece) - 1 < length / piece, summed over the cut rows at most nnz / piece <= bins x 100 /
+// piece_pct =: extra; rounding up to a power of two at most doubles (pieces - 1) of a row; and fewer than max_cut =
+// bins x 100 / longest_pct rows can exceed `longest`. Hence at most 2 x extra entries more than rows and 2 x extra +
+// max_cut pieces, whatever the matrix. The plan is sized for those bounds (entries that are not needed hold nothing),
+// so its size and the grids of its launches depend on M and the device alone.
 // One workgroup: pass 1 counts the nonzeros (from the offsets themselves, so the bounds hold for any array), pass 2
 // numbers the virtual rows, the pieces' slots and the cut rows with one running sum over (entries | slots << 32 | cut
 // rows << 48), 1024 rows per round.
@@ -590,7 +603,13 @@ __global__ __launch_bounds__(kPlanThreads) void plan_cut_kernel(int M, const int
             rs = row_offsets[i];
             len = max(row_offsets[i + 1] - rs, 0);
             cut_it = len > longest_whole;
-            c = cut_it ? (int)((len + piece_max - 1) / piece_max) : 1;
+            if (cut_it) {  // the smallest power of two of pieces that are no longer than piece_max, 256 at most
+                const long long need = (len + piece_max - 1) / piece_max;
+                c = 2;
+                while (c < need && c < kMaxPiecesOfARow) c *= 2;
+            } else {
+                c = 1;
+            }
         }
         const u64 x = (u64)c | (cut_it ? ((u64)c << 32) | (1ull << 48) : 0ull);
         u64 inc = x;
@@ -618,11 +637,14 @@ __global__ __launch_bounds__(kPlanThreads) void plan_cut_kernel(int M, const int
                     v_slot[e0] = -1;
                 }
             } else {
-                const int piece = (len + c - 1) / c;
+                const int lg = 31 - __clz(c);
+                const int piece = (len + c - 1) >> lg;
                 for (int k = 0; k < c && e0 + k < entries; ++k) {
                     v_off[e0 + k] = rs + min(len, k * piece);
                     v_row[e0 + k] = i;
-                    v_slot[e0 + k] = s0 + k < slots ? s0 + k : -2;  // (beyond the bound: only if the offsets changed under the build)
+                    // the slot of the piece's partial row | which piece of its row it is | log2 of how many there are
+                    v_slot[e0 + k] = s0 + k < slots ? ((s0 + k) & kPieceSlotMask) | k << kPieceNumberShift | lg << kPieceCountShift
+                                                    : -2;  // (beyond the bound: only if the offsets changed under the build)
                 }
                 if (j < max_cut) {  // one record of four ints per cut row: row, first slot, pieces, 1
                     cut[4 + 4 * j] = i;
@@ -742,8 +764,8 @@ CutPlan cut_plan_layout(int M, int width, int cus)
     cp.longest_pct = t.cut_longest_pct > 0 ? t.cut_longest_pct : kCutLongestPct;
     const int extra = (cp.bins * 100 + cp.piece_pct - 1) / cp.piece_pct;
     cp.max_cut = (cp.bins * 100 + cp.longest_pct - 1) / cp.longest_pct;
-    cp.entries = M + extra;
-    cp.slots = extra + cp.max_cut;
+    cp.entries = M + 2 * extra;
+    cp.slots = 2 * extra + cp.max_cut;
     auto align = [](size_t x, size_t a) { return (x + a - 1) / a * a; };
     size_t at = align((size_t)4 * cp.entries * sizeof(int), 8);
     cp.off_keys = at;

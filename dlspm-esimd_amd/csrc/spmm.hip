@@ -166,6 +166,58 @@ __global__ __launch_bounds__(4 * 64) void spmm_pieces_kernel(int M, int N, int n
                                                         B, C, rows, nnz, flags, entries, slot_of, pieces, slots);
 }
 
+// The same plan with the cut rows shared out by COLUMNS instead (widths that one wave covers with all its lanes, 129 ... 512
+// columns): an entry that is piece k of a row cut into c works on ALL nonzeros of the row -- the plan enters a piece with
+// its whole row's range -- and on the k-th of c equal shares of the columns (a multiple of four each), and stores to C
+// directly: no partial rows, no second kernel. The share is gone through in passes of GW x 4 columns with GW lanes per
+// dense row, GW = 32, 16 or 8 for shares of more than 64, more than 32, and fewer columns: a pass then costs the piece
+// as many load instructions as its share of the nonzeros would have (64 / GW nonzeros per instruction instead of
+// one; c is a power of two, so 256 columns are shared out exactly down to 32 per piece). Every share of a row is summed in
+// the same order (that of a row in the GW layout), so the result does not depend on the plan.
+template <int VEC, int GW, bool BUF, typename Block>
+__device__ __forceinline__ void spmm_share_passes(const Block& blk, int col0, int col_end, int N,
+                                                  const int* __restrict__ col_indices, const float* __restrict__ values,
+                                                  const float* __restrict__ B, float* __restrict__ C)
+{
+    constexpr int TWW = GW * VEC;
+    for (int c0 = col0; c0 < col_end; c0 += TWW) {
+        dense_rows_window<VEC, GW, 1>(blk, c0, min(col_end, c0 + TWW), N, C,
+                                      [&](Vec<VEC>* acc, int, int p, int q, const int* colv) {
+                                          spmm_segment<VEC, GW, 1, BUF>(acc, p, q, col_indices, values, B, N, colv, blk.lane);
+                                      });
+        if (c0 + TWW < col_end) __syncthreads();  // the partial sums in LDS are written again by the next pass
+    }
+}
+
+template <int VEC, int G, int V, bool BUF>
+__global__ __launch_bounds__(4 * 64) void spmm_shares_kernel(int M, int N, int nnz, int flags, int entries,
+                                                             const int* __restrict__ starts, const int* __restrict__ ends,
+                                                             const int* __restrict__ rows, const int* __restrict__ slot_of,
+                                                             const int* __restrict__ col_indices,
+                                                             const float* __restrict__ values,
+                                                             const float* __restrict__ B, float* __restrict__ C)
+{
+    const int word = slot_of[blockIdx.x];
+    if (word < -1) return;  // an entry that holds nothing
+    RowBlock<4, 1, true, kPlanRows> blk;
+    blk.load((int)blockIdx.x, M, nnz, starts, ends, rows, [&]() { fetch_args_now(col_indices, values, B, C); }, flags);
+    if (word < 0) {  // a whole row
+        dense_rows_block<VEC, G, V>(blk, 0, N, C, [&](Vec<VEC>* acc, int, int p, int q, const int* colv) {
+            spmm_segment<VEC, G, V, BUF>(acc, p, q, col_indices, values, B, N, colv, blk.lane);
+        });
+        return;
+    }
+    const int k = (word >> kPieceNumberShift) & kPieceNumberMask, lg = (word >> kPieceCountShift) & kPieceCountMask;
+    const int share = max((((N + (1 << lg) - 1) >> lg) + 3) & ~3, 4);
+    const int col0 = k * share, col_end = min(N, col0 + share);
+    if (col0 >= N) return;  // more pieces than the width has shares of four columns
+    // (a width that is no multiple of four: the last share's lanes move back to end with the width, as everywhere; where
+    // that takes them into the share before, they store what its own piece stores there)
+    if (share > 64) spmm_share_passes<VEC, 32, BUF>(blk, col0, col_end, N, col_indices, values, B, C);
+    else if (share > 32) spmm_share_passes<VEC, 16, BUF>(blk, col0, col_end, N, col_indices, values, B, C);
+    else spmm_share_passes<VEC, 8, BUF>(blk, col0, col_end, N, col_indices, values, B, C);
+}
+
 // ---- host side --------------------------------------------------------------------------------------
 
 template <int VEC, int G, int V, int W, int R>
@@ -502,6 +554,13 @@ hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int*
 
 // The same with a cut plan (CutPlan, launch.hpp): one workgroup per entry and column tile, then the kernel that adds the
 // pieces of the cut rows in piece order.
+// Cut rows are shared out by columns (spmm_shares_kernel) where one wave covers the width with all its lanes.
+bool spmm_cut_by_columns(const SpmmArgs& x, const SpmmShape& s, const CutPlan& cp)
+{
+    (void)cp;
+    return rule_on(kRuleCutRowsByColumns) && s.vec == 4 && s.G == kWave && x.N <= s.G * 4 * s.V;
+}
+
 hipError_t spmm_pieces_launch(const SpmmArgs& x, const SpmmShape& s, const CutPlan& cp, void* plan, hipStream_t stream)
 {
     if (x.M <= 0) return hipSuccess;
@@ -509,6 +568,7 @@ hipError_t spmm_pieces_launch(const SpmmArgs& x, const SpmmShape& s, const CutPl
     const int *starts = base, *ends = base + cp.entries, *rows = base + 2 * (size_t)cp.entries,
               *slot_of = base + 3 * (size_t)cp.entries;
     float* pieces = reinterpret_cast<float*>(static_cast<char*>(plan) + cp.off_pieces);
+    const bool by_columns = spmm_cut_by_columns(x, s, cp);
     const hipError_t e = dispatch_layout(s, [&](auto l) {
         using L = decltype(l);
         if constexpr (L::VEC != 4) {
@@ -517,6 +577,19 @@ hipError_t spmm_pieces_launch(const SpmmArgs& x, const SpmmShape& s, const CutPl
             const int col_tiles = (int)ceil_div(x.N, L::G * 4 * L::V);
             const long long blocks = (long long)cp.entries * col_tiles;
             if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+            if constexpr (L::G == kWave) {
+                if (by_columns) {
+                    if (dense_fits_buffer(x.K, x.N))
+                        hipLaunchKernelGGL((spmm_shares_kernel<4, L::G, L::V, true>), dim3((unsigned)cp.entries), dim3(4 * 64), 0,
+                                           stream, x.M, x.N, x.nnz, launch_flags(0), cp.entries, starts, ends, rows, slot_of,
+                                           x.col_indices, x.values, x.B, x.C);
+                    else
+                        hipLaunchKernelGGL((spmm_shares_kernel<4, L::G, L::V, false>), dim3((unsigned)cp.entries), dim3(4 * 64), 0,
+                                           stream, x.M, x.N, x.nnz, launch_flags(0), cp.entries, starts, ends, rows, slot_of,
+                                           x.col_indices, x.values, x.B, x.C);
+                    return hipGetLastError();
+                }
+            }
             if (dense_fits_buffer(x.K, x.N))
                 hipLaunchKernelGGL((spmm_pieces_kernel<4, L::G, L::V, true>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M,
                                    x.N, x.nnz, col_tiles, launch_flags(0), cp.entries, cp.slots, starts, ends, rows, slot_of,
@@ -528,7 +601,7 @@ hipError_t spmm_pieces_launch(const SpmmArgs& x, const SpmmShape& s, const CutPl
             return hipGetLastError();
         }
     });
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess || by_columns) return e;
     return cut_rows_sum_launch(x.M, x.N, cp, plan, x.C, stream);
 }
 

@@ -387,6 +387,8 @@ typedef struct dlspm_tuning {
 #define DLSPM_RULE_ROW_ALIGNED_SPLIT           16  /* whole rows per wave where that is nearly as even as the even split    */
 #define DLSPM_RULE_PLAN_UNGROUPS               32  /* a planned launch runs one row per workgroup where the size rule groups */
 #define DLSPM_RULE_EXACT_WIDTH_KERNELS         64  /* SDDMM, fused: kernels without bounds handling for D = 16, 32, ... 512  */
+#define DLSPM_RULE_CUT_ROWS_BY_COLUMNS        128  /* SpMM with a cut plan, 132 ... 512 columns: the pieces of a cut row share */
+                                                   /* its columns, not its nonzeros (no partial rows, no second kernel)       */
 void dlspm_tuning_default(dlspm_tuning* t);   /* fills *t with "follow the rules" */
 int dlspm_set_tuning(const dlspm_tuning* t);  /* DLSPM_OK or DLSPM_E_INVALID_ARG (a field out of range) */
 int dlspm_get_tuning(dlspm_tuning* t);        /* what the calling thread's launches currently use */

@@ -398,17 +398,18 @@ void model_row_plan(int M, const int* ro, int bins, int order, int* plan)
 
 // Host model of the cut rule of a cut plan (plan_cut_kernel): with share = max(1, ceil(nnz / bins)), piece_max =
 // ceil(share x piece_pct / 100) and longest = max(piece_max, ceil(share x longest_pct / 100)), a row of more than
-// `longest` nonzeros becomes c = ceil(length / piece_max) pieces of ceil(length / c) nonzeros each (the last one what
-// is left); the rows and pieces in matrix order are the "virtual rows" 0 .. used-1 of `entries` = M + extra, extra =
-// ceil(bins x 100 / piece_pct); the others hold nothing. v_off[entries + 1], v_row[entries] (-1: nothing),
-// v_slot[entries] (-1 a whole row, s >= 0 piece number s among all pieces in matrix order, -2 nothing); cut[0] = cut
-// rows, cut[1] = share, cut[2] = used, cut[3] = 0, then max_cut = ceil(bins x 100 / longest_pct) records of four ints
-// (row, first slot, pieces, 1; records beyond cut[0] are zeros). Returns 0, or 1 if a bound that the plan's size relies
-// on does not hold (more than entries virtual rows, extra + max_cut pieces or max_cut cut rows).
+// `longest` nonzeros becomes c pieces of ceil(length / c) nonzeros each (the last ones what is left, possibly nothing),
+// c the smallest power of two >= ceil(length / piece_max), 256 at most; the rows and pieces in matrix order are the
+// "virtual rows" 0 .. used-1 of `entries` = M + 2 x extra, extra = ceil(bins x 100 / piece_pct); the others hold nothing.
+// v_off[entries + 1], v_row[entries] (-1: nothing), v_slot[entries] (-1 a whole row, s >= 0 piece number s among all
+// pieces in matrix order, -2 nothing); cut[0] = cut rows, cut[1] = share, cut[2] = used, cut[3] = 0, then max_cut =
+// ceil(bins x 100 / longest_pct) records of four ints (row, first slot, pieces, 1; records beyond cut[0] are zeros).
+// Returns 0, or 1 if a bound that the plan's size relies on does not hold (more than entries virtual rows, 2 x extra +
+// max_cut pieces or max_cut cut rows).
 int model_cut_rows(int M, const int* ro, int bins, int piece_pct, int longest_pct, int* v_off, int* v_row, int* v_slot, int* cut)
 {
     const int extra = (bins * 100 + piece_pct - 1) / piece_pct, max_cut = (bins * 100 + longest_pct - 1) / longest_pct;
-    const int entries = M + extra, slots = extra + max_cut;
+    const int entries = M + 2 * extra, slots = 2 * extra + max_cut;
     long long nnz = 0;
     for (int i = 0; i < M; ++i) nnz += std::max(ro[i + 1] - ro[i], 0);
     const long long share = std::max((nnz + bins - 1) / bins, 1ll);
@@ -423,7 +424,10 @@ int model_cut_rows(int M, const int* ro, int bins, int piece_pct, int longest_pc
             ++e;
             continue;
         }
-        const int c = (int)((len + piece_max - 1) / piece_max), piece = (len + c - 1) / c;
+        const long long need = (len + piece_max - 1) / piece_max;
+        int c = 2;
+        while (c < need && c < 256) c *= 2;
+        const int piece = (len + c - 1) / c;
         if (e + c > entries || s + c > slots || j >= max_cut) return 1;
         cut[4 + 4 * j] = i; cut[4 + 4 * j + 1] = s; cut[4 + 4 * j + 2] = c; cut[4 + 4 * j + 3] = 1;
         for (int k = 0; k < c; ++k) {
@@ -442,10 +446,13 @@ int model_cut_rows(int M, const int* ro, int bins, int piece_pct, int longest_pc
 }
 
 // The cut plan that dlspm_row_plan_build_cut builds: the row plan (model_row_plan) of the virtual rows, each entry then
-// naming its matrix row and its slot. plan[4 x entries]: first nonzero, end, row, slot.
+// naming its matrix row and its slot. plan[4 x entries]: first nonzero, end, row, slot word. The slot word of piece k of
+// a row cut into c = 1 << lg is slot | k << 15 | lg << 23, and such an entry holds the range of its WHOLE row (a launch
+// takes the piece's share of the nonzeros, or of the columns, from the word); -1 for a whole row, -2 for an entry that
+// holds nothing.
 int model_row_plan_cut(int M, const int* ro, int bins, int piece_pct, int longest_pct, int order, int* plan, int* cut)
 {
-    const int entries = M + (bins * 100 + piece_pct - 1) / piece_pct;
+    const int entries = M + 2 * ((bins * 100 + piece_pct - 1) / piece_pct);
     std::vector<int> v_off((size_t)entries + 1), v_row((size_t)entries), v_slot((size_t)entries), vp((size_t)3 * entries);
     if (model_cut_rows(M, ro, bins, piece_pct, longest_pct, v_off.data(), v_row.data(), v_slot.data(), cut)) return 1;
     model_row_plan(entries, v_off.data(), bins, order, vp.data());
@@ -454,7 +461,18 @@ int model_row_plan_cut(int M, const int* ro, int bins, int piece_pct, int longes
         plan[p] = vp[p];
         plan[(size_t)entries + p] = vp[(size_t)entries + p];
         plan[2 * (size_t)entries + p] = v_row[v];
-        plan[3 * (size_t)entries + p] = v_slot[v];
+        int word = v_slot[v];
+        if (word >= 0) {
+            int first = v, last = v;  // the virtual rows of one matrix row are neighbours
+            while (first > 0 && v_row[first - 1] == v_row[v]) --first;
+            while (last + 1 < entries && v_row[last + 1] == v_row[v]) ++last;
+            int lg = 0;
+            while ((1 << lg) < last - first + 1) ++lg;
+            word = (word & 0x7fff) | (v - first) << 15 | lg << 23;
+            plan[p] = v_off[first];
+            plan[(size_t)entries + p] = v_off[last + 1];
+        }
+        plan[3 * (size_t)entries + p] = word;
     }
     return 0;
 }

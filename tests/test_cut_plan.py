@@ -63,7 +63,7 @@ def run_spmm(L, ro, ci, va, B, G, W, R):
 
 def sizes(M, bins, piece_pct=100, longest_pct=150):
     """(entries, most cut rows) of a cut plan of M rows."""
-    return M + -(-bins * 100 // piece_pct), -(-bins * 100 // longest_pct)
+    return M + 2 * -(-bins * 100 // piece_pct), -(-bins * 100 // longest_pct)
 
 
 def cut_list_offset(M, bins, piece_pct=100, longest_pct=150):
@@ -120,8 +120,9 @@ ROW_CASES = [
                                                         (104, 200, 150), (256, 1000, 10)])
 def test_cut_rule_partitions_rows_within_its_bounds(model, name, make, bins, piece_pct, longest_pct):
     """CPU: every row is covered by its virtual rows exactly, in order; only rows above one and a half shares are cut,
-    into pieces of at most one share; no more than M + bins virtual rows, fewer than 2 x bins pieces, fewer than bins cut
-    rows (the bounds the plan's size is made of), for any matrix; the plan is a permutation of the virtual rows."""
+    into a power of two (at most 256) of equal pieces of at most one share; no more than M + 2 x bins virtual rows, 2 x bins
+    more pieces than cut rows, fewer than bins cut rows (the bounds the plan's size is made of), for any matrix; the plan
+    holds every virtual row once, a piece with the range of its whole row and a word that says which piece of how many it is."""
     ro, _ = make(np.random.default_rng(len(name) * 131 + bins))
     M = ro.size - 1
     E, max_cut = sizes(M, bins, piece_pct, longest_pct)
@@ -143,10 +144,13 @@ def test_cut_rule_partitions_rows_within_its_bounds(model, name, make, bins, pie
             assert v_row[e] == i and v_slot[e] == -1 and v_off[e] == ro[i] and vlen[e] == lens[i]
             e += 1
             continue
-        c = -(-int(lens[i]) // piece_max)
-        assert c >= 2
+        need = -(-int(lens[i]) // piece_max)
+        assert need >= 2
+        c = min(256, 1 << (need - 1).bit_length())  # the smallest power of two of pieces that are short enough
         assert (v_row[e:e + c] == i).all() and v_off[e] == ro[i] and v_off[e + c] == ro[i + 1]
-        assert (vlen[e:e + c] > 0).all() and vlen[e:e + c].max() <= piece_max and vlen[e:e + c].sum() == lens[i]
+        piece = -(-int(lens[i]) // c)
+        assert np.array_equal(vlen[e:e + c], np.clip(lens[i] - piece * np.arange(c), 0, piece))
+        assert vlen[e:e + c].sum() == lens[i] and (need > 256 or piece <= piece_max)
         assert np.array_equal(v_slot[e:e + c], np.arange(pieces, pieces + c))
         cut_rows.append((i, pieces, c))
         pieces += c
@@ -155,10 +159,22 @@ def test_cut_rule_partitions_rows_within_its_bounds(model, name, make, bins, pie
     for j, (i, s, c) in enumerate(cut_rows):
         assert cut[4 + 4 * j:8 + 4 * j].tolist() == [i, s, c, 1]
     assert not cut[4 + 4 * len(cut_rows):].any()
-    # the plan: every virtual row once, with its own range, row and slot
-    starts, ends, rows, slots = plan[:E], plan[E:2 * E], plan[2 * E:3 * E], plan[3 * E:]
+    # the plan: every virtual row once, with its row and slot; a whole row with its own range, a piece with its row's
+    starts, ends, rows, words = plan[:E], plan[E:2 * E], plan[2 * E:3 * E], plan[3 * E:]
     key = lambda a, b, c, d: sorted(zip(a.tolist(), b.tolist(), c.tolist(), d.tolist()))
-    assert key(starts, ends, rows, slots) == key(v_off[:-1], v_off[1:], v_row, v_slot)
+    of_row = {i: (s, c) for (i, s, c) in cut_rows}
+    got_starts, got_ends = starts.copy(), ends.copy()
+    for p, (word, row) in enumerate(zip(words.tolist(), rows.tolist())):
+        if word >= 0:
+            first, c = of_row[row]
+            k = (word >> 15) & 255
+            assert k == (word & 0x7FFF) - first and 1 << ((word >> 23) & 15) == c
+            assert (starts[p], ends[p]) == (ro[row], ro[row + 1])
+            piece = -(-int(lens[row]) // c)  # what a launch takes from the word: the piece's share of the row's nonzeros
+            got_starts[p] = ro[row] + min(int(lens[row]), k * piece)
+            got_ends[p] = min(int(ro[row + 1]), got_starts[p] + piece)
+    piece_number = np.where(words >= 0, words & 0x7FFF, words)
+    assert key(got_starts, got_ends, rows, piece_number) == key(v_off[:-1], v_off[1:], v_row, v_slot)
 
 
 def test_cut_plan_sizes_and_advice(dl):
@@ -168,7 +184,7 @@ def test_cut_plan_sizes_and_advice(dl):
     b0 = dl.row_plan_bytes_for(dl.OP_SDDMM, 512, 128)
     assert b0 > 0 and b0 == dl.row_plan_bytes_for(dl.OP_SDDMM, 512, 7)
     b1, b2 = dl.row_plan_bytes_for(dl.OP_SPMM, 512, 128), dl.row_plan_bytes_for(dl.OP_SPMM, 512, 256)
-    assert b0 < b1 < b2 and b2 - b1 == (256 + 171) * 128 * 4   # room for 256 x 100 / 100 + ceil(256 x 100 / 150) pieces
+    assert b0 < b1 < b2 and b2 - b1 == (2 * 256 + 171) * 128 * 4   # room for 2 x 256 x 100 / 100 + ceil(256 x 100 / 150) pieces
     assert dl.row_plan_bytes_for(dl.OP_FUSED, 512, 256) == b2
     assert dl.row_plan_bytes_for(dl.OP_SPMM, (1 << 20) + 1, 64) == 0 and dl.row_plan_bytes_for(7, 512, 64) == 0
     assert dl.row_plan_bytes_for(dl.OP_SPMM, 0, 64) == 0
@@ -285,15 +301,33 @@ def test_gpu_launches_with_a_cut_plan(model, dl, oracle, width, piece_pct, longe
         V = rng.normal(0, 1, (K, width)).astype(np.float32)
         # one plan, sized for SpMM / fused at this width, serves all three ops
         cp = dl.cut_plan(ro_d, dl.OP_SPMM, width)
-        # SpMM
+        # SpMM. Widths that one wave covers with all its lanes (129 ... 512 columns) share a cut row out by columns: every
+        # piece sums the whole row, in the lane layout of its share's width; the other widths (and the rule switched off)
+        # by nonzeros, with partial rows that a second kernel adds
         sh = dl.describe_launch(dl.OP_SPMM, M, K, width, nnz)
-        got = dl.spmm(ro_d, ci_d, dev(torch, va), dev(torch, B), K=K, plan=cp).cpu().numpy()
         want = oracle.spmm(ro, ci, va, B)
-        assert oracle.rel_frobenius(got, want) <= TOL, (name, "spmm")
-        if dl.row_plan_advice(dl.OP_SPMM, M, K, width, nnz, -1) and sh["col_tiles"] == 1 and sh["vec"] == 4:
-            rc, Cv, _ = run_spmm(model, v_off, ci, va, B, sh["G"], 4, 1)
-            assert rc == 0
-            assert np.array_equal(got, combine(Cv, M, v_row, v_slot, cut, max_cut)), (name, "spmm against the model")
+        by_columns = sh["vec"] == 4 and sh["G"] == 64 and sh["col_tiles"] == 1
+        for shares in (("columns", "nonzeros") if by_columns else ("nonzeros",)):
+            dl.set_tuning(cut_piece_pct=piece_pct, cut_longest_pct=longest_pct,
+                          rules_off=dl.RULES["cut_rows_by_columns"] if by_columns and shares == "nonzeros" else 0)
+            got = dl.spmm(ro_d, ci_d, dev(torch, va), dev(torch, B), K=K, plan=cp).cpu().numpy()
+            assert oracle.rel_frobenius(got, want) <= TOL, (name, "spmm", shares)
+            if dl.row_plan_advice(dl.OP_SPMM, M, K, width, nnz, -1) and sh["col_tiles"] == 1 and sh["vec"] == 4:
+                rc, Cv, _ = run_spmm(model, v_off, ci, va, B, sh["G"], 4, 1)
+                assert rc == 0
+                expect = combine(Cv, M, v_row, v_slot, cut, max_cut)
+                if shares == "columns":
+                    whole_rows = {}
+                    for j in range(cut[0]):
+                        row, _, c = cut[4 + 4 * j:7 + 4 * j]
+                        share = max(4, (-(-width // c) + 3) & ~3)
+                        lanes = 32 if share > 64 else 16 if share > 32 else 8
+                        if lanes not in whole_rows:
+                            rc, whole_rows[lanes], _ = run_spmm(model, ro, ci, va, B, lanes, 4, 1)
+                            assert rc == 0
+                        expect[row] = whole_rows[lanes][row]
+                assert np.array_equal(got, expect), (name, "spmm against the model", shares)
+        dl.set_tuning(cut_piece_pct=piece_pct, cut_longest_pct=longest_pct)
         # SDDMM: the same bits as the plain call, whatever the plan
         if width <= 512:
             plain = dl.sddmm(ro_d, ci_d, dev(torch, Q), dev(torch, B))
