@@ -83,10 +83,11 @@ __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __
                                             const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                             const float* __restrict__ lhs, const float* __restrict__ rhs,
                                             SampledOut out, const int* __restrict__ row_ids = nullptr, int nnz = 0,
-                                            int flags = 0)
+                                            int flags = 0, const int* __restrict__ row_slots = nullptr, int slots = 0)
 {
     RowBlock<W, R, SLICED, PLANNED> blk;
-    blk.load(bid, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, lhs, rhs, out.at); }, flags);
+    blk.load(bid, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, lhs, rhs, out.at); }, flags,
+             row_slots, slots);
     blk.for_each_segment([&](int r, int p, int q, int, int) {
         const float* lhs_row = lhs + (size_t)(blk.row0 + r) * D;
         const int shift = blk.shift(r);
@@ -133,6 +134,21 @@ __global__ __launch_bounds__(4 * 64) void sddmm_planned_kernel(int M, int D, int
 {
     sddmm_block<VEC, G1, DS, MASKED, 4, 1, true, kPlanRows>((int)blockIdx.x, M, D, starts, ends, col_indices, lhs, rhs, out, rows,
                                                             nnz);
+}
+
+// Row plan with cut rows: entry i is a whole row (slot_of[i] == -1), a piece of one -- entered with its row's whole range,
+// slot_of[i] says which piece of how many: that share of the row's nonzeros, whose results go to their own CSR slots like
+// any others -- or nothing (an empty range).
+template <int VEC, int G1, int DS, bool MASKED>
+__global__ __launch_bounds__(4 * 64) void sddmm_pieces_kernel(int M, int D, int nnz, int slots, const int* __restrict__ starts,
+                                                              const int* __restrict__ ends, const int* __restrict__ rows,
+                                                              const int* __restrict__ slot_of,
+                                                              const int* __restrict__ col_indices,
+                                                              const float* __restrict__ lhs, const float* __restrict__ rhs,
+                                                              SampledOut out)
+{
+    sddmm_block<VEC, G1, DS, MASKED, 4, 1, true, kPlanPieces>((int)blockIdx.x, M, D, starts, ends, col_indices, lhs, rhs, out, rows,
+                                                              nnz, 0, slot_of, slots);
 }
 
 template <int VEC, int G1, int DS, int W, int R>
@@ -316,9 +332,18 @@ bool sddmm_cut_plan_applies(const DeviceInfo& dev, SddmmShape& s, int M, int D, 
 }
 
 template <int DS>
-static hipError_t launch_planned(const SddmmArgs& x, const int* plan, int entries, hipStream_t stream)
+static hipError_t launch_planned(const SddmmArgs& x, const int* plan, int entries, int slots, hipStream_t stream)
 {
-    const int *starts = plan, *ends = plan + entries, *rows = plan + 2 * (size_t)entries;
+    const int *starts = plan, *ends = plan + entries, *rows = plan + 2 * (size_t)entries, *slot_of = plan + 3 * (size_t)entries;
+    if (slots > 0) {  // a cut plan
+        if (x.D == 8 * 4 * DS)
+            hipLaunchKernelGGL((sddmm_pieces_kernel<4, 8, DS, false>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
+                               x.nnz, slots, starts, ends, rows, slot_of, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+        else
+            hipLaunchKernelGGL((sddmm_pieces_kernel<4, 8, DS, true>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
+                               x.nnz, slots, starts, ends, rows, slot_of, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+        return hipGetLastError();
+    }
     if (x.D == 8 * 4 * DS)
         hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, false>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
                            x.nnz, starts, ends, rows, x.col_indices, x.lhs, x.rhs, sampled_out(x));
@@ -328,24 +353,25 @@ static hipError_t launch_planned(const SddmmArgs& x, const int* plan, int entrie
     return hipGetLastError();
 }
 
-static hipError_t launch_planned_ds(const SddmmArgs& x, const SddmmShape& s, const int* plan, int entries, hipStream_t stream)
+static hipError_t launch_planned_ds(const SddmmArgs& x, const SddmmShape& s, const int* plan, int entries, int slots,
+                                    hipStream_t stream)
 {
     if (x.M <= 0) return hipSuccess;
     return dispatch_layout(s, [&](auto l) {
         using L = decltype(l);
-        if constexpr (L::VEC == 4 && L::G1 == 8 && L::DS >= 1) return launch_planned<L::DS>(x, plan, entries, stream);
+        if constexpr (L::VEC == 4 && L::G1 == 8 && L::DS >= 1) return launch_planned<L::DS>(x, plan, entries, slots, stream);
         else return hipErrorInvalidValue;
     });
 }
 
 hipError_t sddmm_planned_launch(const SddmmArgs& x, const SddmmShape& s, const int* plan, hipStream_t stream)
 {
-    return launch_planned_ds(x, s, plan, x.M, stream);
+    return launch_planned_ds(x, s, plan, x.M, 0, stream);
 }
 
 hipError_t sddmm_pieces_launch(const SddmmArgs& x, const SddmmShape& s, const CutPlan& cp, const void* plan, hipStream_t stream)
 {
-    return launch_planned_ds(x, s, static_cast<const int*>(plan), cp.entries, stream);
+    return launch_planned_ds(x, s, static_cast<const int*>(plan), cp.entries, cp.slots, stream);
 }
 
 }  // namespace dlspm
