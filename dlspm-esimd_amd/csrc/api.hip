@@ -309,8 +309,8 @@ void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, co
 }
 
 constexpr int kCutPlanAdviceMaxRows = 16384;     // the cut rule is one workgroup's work: 16 rounds of 1024 rows
-constexpr double kCutPlanMinGainNs = 2500.0;      // SpMM, fused: the kernel that adds the pieces must be paid for
-constexpr double kCutPlanMinGainNsSddmm = 300.0;  // SDDMM: no second kernel
+constexpr double kCutPlanMinGainNs = 2500.0;      // fused, SpMM with partial rows: the kernel that adds the pieces must be paid for
+constexpr double kCutPlanMinGainNsOneKernel = 300.0;  // SDDMM, and SpMM where the pieces share the columns: no second kernel
 constexpr double kCutPlanMinGainNsSddmmOneRowEach = 1000.0;  // ... one to two rows per compute unit: eight waves per row do nearly as well
 
 // longest row and number of rows without nonzeros (dlspm_csr_row_stats); stats[0] = max, stats[1] = empty rows
@@ -590,24 +590,29 @@ int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_
 
 // Whether cutting the longest rows (a cut plan) is expected to beat the plan over whole rows. The longest row runs on
 // one compute unit, which gathers about 48 bytes per clock (115 bytes per nanosecond at 2.4 GHz) of dense rows; cut, no
-// entry is longer than one and a half shares. What that saves is set against what the cut plan costs: for SpMM and the
-// fused op the second kernel that adds the pieces (about 2 us between two graph nodes), for SDDMM only a grid that is
-// `compute units` entries larger.
-static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int nnz, int max_row_len)
+// entry is longer than one and a half shares. What that saves is set against what the cut plan costs: where the pieces
+// leave partial rows (the fused op; SpMM outside 65 ... 512 columns) the second kernel that adds them (about 2 us between
+// two graph nodes), else (SDDMM; SpMM where the pieces share the row's columns) only a grid that is two entries per
+// compute unit larger.
+static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int nnz, int max_row_len, bool second_kernel)
 {
     if (max_row_len <= 0 || M > kCutPlanAdviceMaxRows) return false;
     const long long cus = dev.cus;
-    // SpMM and the fused op: only where a share holds at least two mean rows, so that the rows above one and a half
+    // With a second kernel: only where a share holds at least two mean rows, so that the rows above one and a half
     // shares are the exception and the kernel that adds their pieces has little to do (the reference's layers of 64 ...
     // 256 rows, where most rows would be cut: 0.85 ... 1.5 times the time of the plan over whole rows; 512 rows: 0.66 ... 1.0)
-    if (op != DLSPM_OP_SDDMM && M < 2 * cus) return false;
+    if (second_kernel && M < 2 * cus) return false;
     const long long share = std::max<long long>(ceil_div(nnz, cus), 1);
     const long long longest_whole = (share * kCutLongestPct + 99) / 100;
     if (max_row_len <= longest_whole) return false;
     const double bytes_per_nonzero = (op == DLSPM_OP_FUSED ? 2.0 : 1.0) * (double)std::min(width, 512) * sizeof(float);
     const double saved_ns = (double)(max_row_len - longest_whole) * bytes_per_nonzero / 115.0;
-    if (op == DLSPM_OP_SDDMM) return saved_ns >= (M >= cus && M < 2 * cus ? kCutPlanMinGainNsSddmmOneRowEach : kCutPlanMinGainNsSddmm);
-    return saved_ns >= kCutPlanMinGainNs;
+    if (second_kernel) return saved_ns >= kCutPlanMinGainNs;
+    // (SpMM, N = 256, the 302 files of the reference's data set with a row above one and a half shares, against the better
+    // of NULL and the plan over whole rows: 0.99 of the time below 300 ns by this model, 0.96 / 0.91 / 0.84 / 0.81 from 300 /
+    // 600 / 1000 / 2500 ns on, at every height from 64 to 2048 rows)
+    if (op == DLSPM_OP_SDDMM && M >= cus && M < 2 * cus) return saved_ns >= kCutPlanMinGainNsSddmmOneRowEach;
+    return saved_ns >= kCutPlanMinGainNsOneKernel;
 }
 
 // the longest row at least twenty times the mean: what DLSPM_HINT_ROWS_SKEWED says
@@ -621,15 +626,17 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
     const DeviceInfo& dev = device_info();
     if (M <= 0 || K <= 0 || N_or_D <= 0 || nnz <= 0) return 0;
     const bool vec4 = N_or_D >= 4;
+    bool second_kernel = op == DLSPM_OP_FUSED;  // a cut plan's pieces leave partial rows for a second kernel to add
     if (op == DLSPM_OP_SPMM) {
         SpmmShape shape = spmm_choose(dev, M, K, N_or_D, nnz, vec4, false, true);
         if (!spmm_plan_applies(dev, shape, M, N_or_D, nnz)) return 0;
+        second_kernel = !spmm_cut_by_columns(shape, N_or_D);
     } else if (op == DLSPM_OP_SDDMM) {
         SddmmShape shape = sddmm_choose(dev, M, N_or_D, nnz, vec4);
         if (!sddmm_plan_applies(dev, shape, M, N_or_D, nnz, rows_are_skewed(M, nnz, max_row_len))) {
             // fewer rows than compute units: only a cut plan helps (its pieces fill the device)
             SddmmShape few = sddmm_choose(dev, M, N_or_D, nnz, vec4);
-            return sddmm_cut_plan_applies(dev, few, M, N_or_D, nnz) && cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len) ? 2 : 0;
+            return sddmm_cut_plan_applies(dev, few, M, N_or_D, nnz) && cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len, false) ? 2 : 0;
         }
     } else if (op == DLSPM_OP_FUSED) {
         FusedShape shape = fused_choose(dev, M, N_or_D, nnz, vec4);
@@ -651,7 +658,7 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
     int slices = 0;
     (void)dlspm_describe_slices(op, M, K, N_or_D, nnz, &slices, nullptr);
     if (slices >= 3) return 0;
-    return cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len) ? 2 : 1;
+    return cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len, second_kernel) ? 2 : 1;
 }
 
 // the *_planned entry points: the named call with the plan as its workspace and the hint that says so

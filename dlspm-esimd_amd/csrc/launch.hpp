@@ -255,6 +255,7 @@ CutPlan cut_plan_layout(int M, int width, int cus);
 hipError_t cut_plan_build_launch(int M, const int* row_offsets, const CutPlan& cp, void* plan, int order, hipStream_t stream);
 hipError_t cut_rows_sum_launch(int M, int width, const CutPlan& cp, const void* plan, float* out, hipStream_t stream);
 hipError_t spmm_pieces_launch(const SpmmArgs& x, const SpmmShape& s, const CutPlan& cp, void* plan, hipStream_t stream);
+bool spmm_cut_by_columns(const SpmmShape& s, int N);  // the pieces of a cut row share its columns: one kernel, no partial rows
 
 // the same plan for the other two ops (16 < D <= 512, one row per four-wave workgroup)
 // skewed (DLSPM_HINT_ROWS_SKEWED): the caller knows that the longest row is at least twenty times the mean
