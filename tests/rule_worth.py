@@ -7,7 +7,8 @@ the same launches are timed again.
 Cases: the five benchmark configurations; the reference's 12-shape benchmark grid (SPMM/spmm-esimd-allbenchs.cpp:252-255)
 at density 0.1 with N = D = 32 and 128 (Bernoulli patterns); lognormal row lengths (sigma 1) on 2048 ... 16384 rows; layer
 shapes of 64 ... 512 rows as in the reference's dlmc/ tree; very long rows in a tall matrix (16384 x 8192 at density 0.2) and in
-few rows (256 ... 512 rows of 2048 ... 4096 nonzeros), which is where the rules that add waves per row apply. Every case is launched as a driver would (dlspm_analyze ->
+few rows (256 ... 512 rows of 2048 ... 4096 nonzeros), which is where the rules that add waves per row apply; the three
+patterns of tests/golden/dlmc whose longest row holds four compute units' shares of the nonzeros (cut plans). Every case is launched as a driver would (dlspm_analyze ->
 dlspm_advise -> allocate -> build), inside a HIP graph of 20 launches (median of 7 double replays). With a rule off the
 preparation is repeated, so that sizes and advice follow the changed rules. The launches with all rules on are timed
 before and after the others (after one untimed run) and their mean is the reference. One line per rule and op: the geometric mean
@@ -63,6 +64,10 @@ def cases(dl, quick):
         for (M, K, density) in ((256, 8192, 0.5), (512, 8192, 0.25)):
             ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 13, M, K, density)
             out.append((f"few long rows {M}x{K} density {density} width 256/128/64", None, M, K, -1, ro, ci))
+    from test_cut_plan import DLMC, LONG_ROW_FILES, load_smtx
+    for f in LONG_ROW_FILES:
+        M, K, ro, ci = load_smtx(os.path.join(DLMC, f))
+        out.append((f"dlmc {f[:28]} {M}x{K} width 256/128/64", None, M, K, -1, ro, ci))
     return out
 
 
