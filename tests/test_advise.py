@@ -110,6 +110,41 @@ def test_analyze_against_numpy(dl):
 
 
 @pytest.mark.gpu
+def test_analyze_from_several_threads_at_once(dl):
+    """dlspm_analyze keeps the figures of a call in a slot of a static device array for the length of the call: four host
+    threads, each on a stream of its own, analyse different matrices a hundred times at once and get their own answers."""
+    import threading
+
+    import torch
+
+    rng = np.random.default_rng(11)
+    problems = []
+    for kind, M, K, density in (("uniform", 900, 700, 0.1), ("skewed", 3000, 1024, 0.03), ("empty_rows", 500, 400, 0.2),
+                                ("uniform", 64, 3000, 0.4)):
+        ro, ci = random_csr(rng, M, K, kind, density)
+        problems.append((dev(torch, ro), dev(torch, ci), K, numpy_info(ro, ci, K)))
+    torch.cuda.synchronize()
+    wrong = []
+
+    def work(index):
+        ro_d, ci_d, K, want = problems[index]
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            for _ in range(100):
+                got = dl.analyze(ro_d, ci_d, K).as_dict()
+                if got != want:
+                    wrong.append((index, got, want))
+                    return
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(problems))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not wrong, wrong[:1]
+
+
+@pytest.mark.gpu
 def test_prepared_calls_follow_the_matrix(dl, oracle):
     """analyze -> advise -> allocate -> build -> launch, with no knowledge of the matrix on the caller's side: the
     sliding-window mask gets the banded launch (the bits of the call with DLSPM_HINT_BANDED), the matrix with one very
