@@ -286,7 +286,7 @@ def combine(per_virtual_row, M, v_row, v_slot, cut, max_cut):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("width,piece_pct,longest_pct", [(256, 100, 150), (128, 100, 150), (64, 100, 150), (49, 100, 150), (392, 100, 150),
-                                                         (256, 50, 100), (64, 25, 30)])
+                                                         (256, 50, 100), (64, 25, 30), (250, 100, 150), (100, 100, 150), (130, 10, 10)])
 def test_gpu_launches_with_a_cut_plan(model, dl, oracle, width, piece_pct, longest_pct):
     """All three ops with DLSPM_HINT_CUT_PLAN against the host model (bit for bit) and the oracle (1e-4); SDDMM also
     against the plain call (bit for bit: pieces write their own CSR slots)."""

@@ -1,12 +1,13 @@
 #!/usr/bin/env python3
 """Seeded random cases against the CPU oracle: odd shapes and widths, four kinds of row-length distribution, every
 schedule, with the library's launch rules overridden at random (dlspm_set_tuning: work split, flat schedule and its
-chunk, column slices, tile order and width, plan order, XCD-contiguous row blocks, streamed results).
+chunk, column slices, tile order and width, plan order, XCD-contiguous row blocks, streamed results, single size rules
+switched off, the cut rule's percentages, the number of compute units the rules and plans are sized for).
 
     python tests/verify_fuzz.py [--cases 1000] [--seed 1] [--report out.txt]
 
 Each case runs all three ops on the GPU through the C ABI under every schedule that applies (NULL, the even-rows hint,
-workspace memory, a row plan) and compares with the oracle: CSR arrays bit-identical after the call, values within 1e-4
+workspace memory, a row plan, a cut plan) and compares with the oracle: CSR arrays bit-identical after the call, values within 1e-4
 relative Frobenius error. No tuning value may change a result beyond the summation order, and none may make a launch
 fail. The case is printed before it runs. Exit status 1 if any case fails.
 """
@@ -48,6 +49,12 @@ def random_tuning(rng):
         t["xcd_contiguous"] = 1
     if rng.random() < 0.5:
         t["stream_results"] = pick([0, 1])
+    if rng.random() < 0.5:
+        t["rules_off"] = int(rng.integers(0, 256))
+    if rng.random() < 0.3:
+        t["cut_piece_pct"], t["cut_longest_pct"] = pick([(100, 150), (50, 75), (25, 30), (200, 150), (10, 10), (1000, 1000)])
+    if rng.random() < 0.3:
+        t["compute_units"] = pick([8, 32, 64, 128, 304, 1024])
     return t
 
 
