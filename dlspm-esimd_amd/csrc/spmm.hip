@@ -197,10 +197,12 @@ __global__ __launch_bounds__(4 * 64) void spmm_shares_kernel(int M, int N, int n
                                                              const float* __restrict__ values,
                                                              const float* __restrict__ B, float* __restrict__ C)
 {
+    // (the word is asked for together with the rest of the entry: looking at it first would put one more round trip to
+    // memory in front of every workgroup's work)
     const int word = slot_of[blockIdx.x];
-    if (word < -1) return;  // an entry that holds nothing
     RowBlock<4, 1, true, kPlanRows> blk;
     blk.load((int)blockIdx.x, M, nnz, starts, ends, rows, [&]() { fetch_args_now(col_indices, values, B, C); }, flags);
+    if (word < -1) return;  // an entry that holds nothing
     if (word < 0) {  // a whole row
         dense_rows_block<VEC, G, V>(blk, 0, N, C, [&](Vec<VEC>* acc, int, int p, int q, const int* colv) {
             spmm_segment<VEC, G, V, BUF>(acc, p, q, col_indices, values, B, N, colv, blk.lane);
