@@ -973,6 +973,6 @@ const char* dlspm_status_string(int status)
 
 int dlspm_last_hip_error(void) { return t_last_hip_error; }
 
-const char* dlspm_version(void) { return "dlspm_hip 0.2 gfx950"; }
+const char* dlspm_version(void) { return "dlspm_hip 0.3 gfx950"; }
 
 }  // extern "C"
