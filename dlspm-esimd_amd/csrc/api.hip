@@ -591,7 +591,7 @@ int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_
 // Whether cutting the longest rows (a cut plan) is expected to beat the plan over whole rows. The longest row runs on
 // one compute unit, which gathers about 48 bytes per clock (115 bytes per nanosecond at 2.4 GHz) of dense rows; cut, no
 // entry is longer than one and a half shares. What that saves is set against what the cut plan costs: where the pieces
-// leave partial rows (the fused op; SpMM outside 65 ... 512 columns) the second kernel that adds them (about 2 us between
+// leave partial rows (the fused op; SpMM outside 33 ... 512 columns) the second kernel that adds them (about 2 us between
 // two graph nodes), else (SDDMM; SpMM where the pieces share the row's columns) only a grid that is two entries per
 // compute unit larger.
 static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int nnz, int max_row_len, bool second_kernel)

@@ -166,8 +166,8 @@ __global__ __launch_bounds__(4 * 64) void spmm_pieces_kernel(int M, int N, int n
                                                         B, C, rows, nnz, flags, entries, slot_of, pieces, slots);
 }
 
-// The same plan with the cut rows shared out by COLUMNS instead (widths that one wave covers with lane groups of 32 or 64,
-// 65 ... 512 columns): an entry that is piece k of a row cut into c works on ALL nonzeros of the row -- the plan enters a piece with
+// The same plan with the cut rows shared out by COLUMNS instead (widths that one wave covers with lane groups of 16 to 64,
+// 33 ... 512 columns): an entry that is piece k of a row cut into c works on ALL nonzeros of the row -- the plan enters a piece with
 // its whole row's range -- and on the k-th of c equal shares of the columns (a multiple of four each), and stores to C
 // directly: no partial rows, no second kernel. The share is gone through in passes of GW x 4 columns with GW lanes per
 // dense row, GW = 32, 16 or 8 for shares of more than 64, more than 32, and fewer columns: a pass then costs the piece
@@ -556,11 +556,11 @@ hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int*
 
 // The same with a cut plan (CutPlan, launch.hpp): one workgroup per entry and column tile, then the kernel that adds the
 // pieces of the cut rows in piece order.
-// Cut rows are shared out by columns (spmm_shares_kernel) where one wave covers the width with lane groups of 32 or 64
-// (65 ... 512 columns).
+// Cut rows are shared out by columns (spmm_shares_kernel) where one wave covers the width with lane groups of 16 to 64
+// (33 ... 512 columns).
 bool spmm_cut_by_columns(const SpmmShape& s, int N)
 {
-    return rule_on(kRuleCutRowsByColumns) && s.vec == 4 && s.G >= 32 && N <= s.G * 4 * s.V;
+    return rule_on(kRuleCutRowsByColumns) && s.vec == 4 && s.G >= 16 && N <= s.G * 4 * s.V;
 }
 
 hipError_t spmm_pieces_launch(const SpmmArgs& x, const SpmmShape& s, const CutPlan& cp, void* plan, hipStream_t stream)
@@ -579,7 +579,7 @@ hipError_t spmm_pieces_launch(const SpmmArgs& x, const SpmmShape& s, const CutPl
             const int col_tiles = (int)ceil_div(x.N, L::G * 4 * L::V);
             const long long blocks = (long long)cp.entries * col_tiles;
             if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-            if constexpr (L::G >= 32) {
+            if constexpr (L::G >= 16) {
                 if (by_columns) {
                     if (dense_fits_buffer(x.K, x.N))
                         hipLaunchKernelGGL((spmm_shares_kernel<4, L::G, L::V, true>), dim3((unsigned)cp.entries), dim3(4 * 64), 0,

@@ -263,7 +263,7 @@ size_t dlspm_row_plan_bytes(int M);
  * the nonzeros (share = nnz / compute units) sets the time of the launch by itself, through the one compute unit it
  * runs on, whatever the order of the rows. A cut plan hands such a row out in 2, 4, ... 256 equal pieces (the fewest
  * that are no longer than a share) to as many workgroups. SDDMM pieces take a share of the row's nonzeros and write
- * their own CSR slots (same bits as any other schedule). SpMM at 65 ... 512 columns gives every piece ALL nonzeros of the
+ * their own CSR slots (same bits as any other schedule). SpMM at 33 ... 512 columns gives every piece ALL nonzeros of the
  * row and a share of its columns: one kernel, nothing to combine. The fused op, and SpMM at other widths, write one
  * partial row per piece into memory that follows the plan, and a second small kernel adds the pieces of every cut row
  * in piece order. No atomics, no fences anywhere: deterministic; rows that are not cut are summed as by the plain plan.
@@ -281,7 +281,7 @@ size_t dlspm_row_plan_bytes(int M);
  *                            workspace_bytes = plan_bytes | DLSPM_HINT_CUT_PLAN (DLSPM_E_WORKSPACE below
  *                            dlspm_row_plan_bytes_for(op, M, width)). SpMM and the fused op write the partial rows
  *                            behind the plan: launches that share a cut plan must not overlap in time. Sizes a planned
- *                            launch is not built for run as with NULL. The fused op (SpMM outside 65 ... 512 columns):
+ *                            launch is not built for run as with NULL. The fused op (SpMM outside 33 ... 512 columns):
  *                            two kernels per launch.
  * dlspm_row_plan_advice returns 2 where it expects the cut plan to beat the plain one.
  * No counterpart in the reference (one hardware thread per row or row slice, SPMM/spmmesimd2.hpp:63-75).
@@ -390,7 +390,7 @@ typedef struct dlspm_tuning {
 #define DLSPM_RULE_ROW_ALIGNED_SPLIT           16  /* whole rows per wave where that is nearly as even as the even split    */
 #define DLSPM_RULE_PLAN_UNGROUPS               32  /* a planned launch runs one row per workgroup where the size rule groups */
 #define DLSPM_RULE_EXACT_WIDTH_KERNELS         64  /* SDDMM, fused: kernels without bounds handling for D = 16, 32, ... 512  */
-#define DLSPM_RULE_CUT_ROWS_BY_COLUMNS        128  /* SpMM with a cut plan, 65 ... 512 columns: the pieces of a cut row share  */
+#define DLSPM_RULE_CUT_ROWS_BY_COLUMNS        128  /* SpMM with a cut plan, 33 ... 512 columns: the pieces of a cut row share  */
                                                    /* its columns, not its nonzeros (no partial rows, no second kernel)       */
 void dlspm_tuning_default(dlspm_tuning* t);   /* fills *t with "follow the rules" */
 int dlspm_set_tuning(const dlspm_tuning* t);  /* DLSPM_OK or DLSPM_E_INVALID_ARG (a field out of range) */

@@ -197,7 +197,7 @@ def test_cut_plan_sizes_and_advice(dl):
     assert dl.row_plan_advice(dl.OP_SPMM, 2048, 512, 256, 105687, 312) == 1   # the headline matrix: below one share
     assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 256, 52000, 110) == 0    # even rows: no plan at all
     # fewer rows than compute units (eight waves per row by the size rule): SDDMM takes a cut plan, whose pieces fill the
-    # device at no cost, and so does SpMM at widths where the pieces of a row share its columns (65 ... 512); the fused op and
+    # device at no cost, and so does SpMM at widths where the pieces of a row share its columns (33 ... 512); the fused op and
     # SpMM at the other widths, which would cut most rows and pay for adding the pieces, do not
     assert dl.describe_launch(dl.OP_SDDMM, 128, 1152, 128, 29510)["W"] == 8
     assert dl.row_plan_advice(dl.OP_SDDMM, 128, 1152, 128, 29510, 455) == 2
@@ -206,9 +206,10 @@ def test_cut_plan_sizes_and_advice(dl):
     assert dl.row_plan_advice(dl.OP_SDDMM, 256, 2304, 128, 53000, 800) == 2    # ... of nearly four shares: yes
     assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 256, 29510, 455) == 2
     assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 128, 29510, 455) == 2
-    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 64, 29510, 455) in (0, 1)
-    assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 64, 52000, 2000) == 2     # (with partial rows: only from a large gain on
-    assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 64, 52000, 500) == 1      # ... and two rows per compute unit)
+    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 64, 29510, 455) == 2
+    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 32, 29510, 455) in (0, 1)
+    assert dl.row_plan_advice(dl.OP_SPMM, 512, 8192, 32, 52000, 3000) == 2     # (with partial rows: only from a large gain on
+    assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 32, 52000, 700) == 1      # ... and two rows per compute unit)
     assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 256, 52000, 500) == 2
     assert dl.row_plan_advice(dl.OP_FUSED, 128, 1152, 64, 29510, 455) in (0, 1)
 
@@ -307,12 +308,12 @@ def test_gpu_launches_with_a_cut_plan(model, dl, oracle, width, piece_pct, longe
         V = rng.normal(0, 1, (K, width)).astype(np.float32)
         # one plan, sized for SpMM / fused at this width, serves all three ops
         cp = dl.cut_plan(ro_d, dl.OP_SPMM, width)
-        # SpMM. Widths that one wave covers with lane groups of 32 or 64 (65 ... 512 columns) share a cut row out by columns: every
+        # SpMM. Widths that one wave covers with lane groups of 16 to 64 (33 ... 512 columns) share a cut row out by columns: every
         # piece sums the whole row, in the lane layout of its share's width; the other widths (and the rule switched off)
         # by nonzeros, with partial rows that a second kernel adds
         sh = dl.describe_launch(dl.OP_SPMM, M, K, width, nnz)
         want = oracle.spmm(ro, ci, va, B)
-        by_columns = sh["vec"] == 4 and sh["G"] >= 32 and sh["col_tiles"] == 1
+        by_columns = sh["vec"] == 4 and sh["G"] >= 16 and sh["col_tiles"] == 1
         for shares in (("columns", "nonzeros") if by_columns else ("nonzeros",)):
             dl.set_tuning(cut_piece_pct=piece_pct, cut_longest_pct=longest_pct,
                           rules_off=dl.RULES["cut_rows_by_columns"] if by_columns and shares == "nonzeros" else 0)
