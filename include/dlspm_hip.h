@@ -274,7 +274,7 @@ size_t dlspm_row_plan_bytes(int M);
  *                            partial rows of op at that dense width (SDDMM: none, the width is ignored). 0: no cut plan
  *                            at this height (more than 2^20 rows).
  *   dlspm_row_plan_build_cut builds it from row_offsets (device) into `plan` (device, 256-byte aligned) with kernels on
- *                            `stream` only, like dlspm_row_plan_build (two launches up to 2048 - compute units rows).
+ *                            `stream` only, like dlspm_row_plan_build (two launches up to 2048 - 2 x compute units rows).
  *                            plan_bytes must be at least dlspm_row_plan_bytes_for(DLSPM_OP_SDDMM, M, 0); a plan that is
  *                            to serve SpMM or the fused op must have been sized for that op and width.
  *   the launches             the three compute entry points with workspace = plan and
