@@ -712,7 +712,7 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
         return e0 == hipSuccess ? DLSPM_OK : fail_hip(e0);
     }
     const bool vec4 = D >= 4;  // dwordx4 accesses need only dword alignment
-    const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values, ws.banded ? 1 : 0, dev.l2_bytes};
+    const SddmmArgs args{M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values, ws.banded ? 1 : 0, dev.l2_bytes, dev.cus};
     if (ws.cut_plan && ws.mem) {
         const CutPlan cp = cut_plan_layout(M, 0, dev.cus);
         if (cp.bytes == 0 || ws.bytes < cp.bytes) return DLSPM_E_WORKSPACE;

@@ -106,8 +106,10 @@ inline bool rule_on(int rule) { return (tuning().rules_off & rule) == 0; }
 // What a row-block kernel is told about its launch in one int: bit 0 = deal the row blocks to the XCDs in contiguous
 // runs (DLSPM_HINT_BANDED or the tuning knob), bits 1-2 = results with the non-temporal hint: 0 by the size rule,
 // 1 never, 2 wherever the rule could say so (dlspm_tuning.stream_results).
-// bit 3 = never take the row-aligned split (DLSPM_RULE_ROW_ALIGNED_SPLIT switched off).
-constexpr int kFlagXcdContiguous = 1, kFlagStreamShift = 1, kFlagStreamNever = 1, kFlagStreamAlways = 2, kFlagNoAlignedSplit = 8;
+// bit 3 = never take the row-aligned split (DLSPM_RULE_ROW_ALIGNED_SPLIT switched off); bit 4 (SDDMM, one row per
+// workgroup) = the waves of a row take whole passes of 64 nonzeros in turn (sddmm_row_interleaved).
+constexpr int kFlagXcdContiguous = 1, kFlagStreamShift = 1, kFlagStreamNever = 1, kFlagStreamAlways = 2, kFlagNoAlignedSplit = 8,
+              kFlagFullPasses = 16;
 inline int launch_flags(int xcd_contiguous_hint)
 {
     const Tuning& t = tuning();
@@ -144,6 +146,7 @@ struct SddmmArgs {
     float* out;
     int xcd_contiguous = 0;
     long long l2_bytes = 4ll << 20;  // of the device the call runs on (DeviceInfo::l2_bytes): results beyond it are streamed
+    int cus = 256;                   // ... and its compute units
 };
 struct FusedArgs {
     int M, K, D, nnz;
