@@ -661,36 +661,6 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
     return cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len, second_kernel) ? 2 : 1;
 }
 
-// the *_planned entry points: the named call with the plan as its workspace and the hint that says so
-int spmm_csr_f32_planned(int M, int K, int N, int nnz, const int* row_offsets, const int* col_indices,
-                         const float* values, const float* B, float* C, const void* plan, size_t plan_bytes,
-                         void* stream)
-{
-    if (!plan) return spmm_csr_f32(M, K, N, nnz, row_offsets, col_indices, values, B, C, nullptr, 0, stream);
-    if (plan_bytes & DLSPM_HINT_MASK) return DLSPM_E_INVALID_ARG;
-    return spmm_csr_f32(M, K, N, nnz, row_offsets, col_indices, values, B, C, const_cast<void*>(plan),
-                        plan_bytes | DLSPM_HINT_ROW_PLAN, stream);
-}
-
-int sddmm_csr_f32_planned(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* lhs,
-                          const float* rhs, float* out_values, const void* plan, size_t plan_bytes, void* stream)
-{
-    if (!plan) return sddmm_csr_f32(M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values, nullptr, 0, stream);
-    if (plan_bytes & DLSPM_HINT_MASK) return DLSPM_E_INVALID_ARG;
-    return sddmm_csr_f32(M, K, D, nnz, row_offsets, col_indices, lhs, rhs, out_values, const_cast<void*>(plan),
-                         plan_bytes | DLSPM_HINT_ROW_PLAN, stream);
-}
-
-int fused_sddmm_spmm_f32_planned(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* Q,
-                                 const float* Kmat, const float* V, float scale, float* O, const void* plan,
-                                 size_t plan_bytes, void* stream)
-{
-    if (!plan) return fused_sddmm_spmm_f32(M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O, nullptr, 0, stream);
-    if (plan_bytes & DLSPM_HINT_MASK) return DLSPM_E_INVALID_ARG;
-    return fused_sddmm_spmm_f32(M, K, D, nnz, row_offsets, col_indices, Q, Kmat, V, scale, O, const_cast<void*>(plan),
-                                plan_bytes | DLSPM_HINT_ROW_PLAN, stream);
-}
-
 int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* lhs,
                   const float* rhs, float* out_values, void* workspace, size_t workspace_bytes, void* stream)
 {

@@ -62,9 +62,6 @@ EXPORTS = (
     "dlspm_set_tuning",
     "dlspm_get_tuning",
     "dlspm_device_info",
-    "spmm_csr_f32_planned",
-    "sddmm_csr_f32_planned",
-    "fused_sddmm_spmm_f32_planned",
     "spmm_csr_f32_static",
     "dlspm_static_scratch_bytes",
     "dlspm_status_string",
@@ -151,12 +148,6 @@ def lib() -> ctypes.CDLL:
         L.dlspm_analyze.restype = ci
         L.dlspm_advise.argtypes = [ci, ci, ctypes.POINTER(MatrixInfo), ctypes.POINTER(CallPlan)]
         L.dlspm_advise.restype = ci
-        L.spmm_csr_f32_planned.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, sz, vp]
-        L.spmm_csr_f32_planned.restype = ci
-        L.sddmm_csr_f32_planned.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, sz, vp]
-        L.sddmm_csr_f32_planned.restype = ci
-        L.fused_sddmm_spmm_f32_planned.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, cf, vp, vp, sz, vp]
-        L.fused_sddmm_spmm_f32_planned.restype = ci
         L.spmm_csr_f32_static.argtypes = [ci, ci, ci, ci, vp, vp, vp, vp, vp, vp]
         L.spmm_csr_f32_static.restype = ci
         L.dlspm_static_scratch_bytes.restype = sz

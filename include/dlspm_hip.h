@@ -65,6 +65,9 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+#if defined(__GNUC__) || defined(__clang__)
+#pragma GCC visibility push(default) /* what this header declares is what the library exports */
+#endif
 
 /* status codes */
 #define DLSPM_OK              0
@@ -253,8 +256,6 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
  *                            than 4096 rows, 8192 at D >= 128 and 128 nonzeros per row) ignore the plan and run as
  *                            with NULL. A planned launch is one kernel (no memset, no allocation, no
  *                            synchronisation); the plan is only read, so launches may share it.
- *   *_planned                DEPRECATED aliases: the same launches with the plan as a separate argument (plan == NULL: the
- *                            plain call). New code passes the plan as the workspace with DLSPM_HINT_ROW_PLAN.
  * No counterpart in the reference, whose kernels take the rows in matrix order (SPMM/spmmesimd2.hpp:63-75).
  */
 size_t dlspm_row_plan_bytes(int M);
@@ -295,14 +296,6 @@ int dlspm_row_plan_build_cut(int M, const int* row_offsets, void* plan, size_t p
  * mean) gets the answer for that launch by passing such a longest row here. */
 int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row_len);
 int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_bytes, void* stream);
-int spmm_csr_f32_planned(int M, int K, int N, int nnz, const int* row_offsets, const int* col_indices,
-                         const float* values, const float* B, float* C, const void* plan, size_t plan_bytes,
-                         void* stream);
-int sddmm_csr_f32_planned(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* lhs,
-                          const float* rhs, float* out_values, const void* plan, size_t plan_bytes, void* stream);
-int fused_sddmm_spmm_f32_planned(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices,
-                                 const float* Q, const float* Kmat, const float* V, float scale, float* O,
-                                 const void* plan, size_t plan_bytes, void* stream);
 
 /*
  * What to pass as `workspace` for a matrix of these sizes whose longest row has max_row_len nonzeros (from
@@ -415,6 +408,9 @@ int dlspm_last_hip_error(void);
 /* "dlspm_hip <major>.<minor> gfx950" */
 const char* dlspm_version(void);
 
+#if defined(__GNUC__) || defined(__clang__)
+#pragma GCC visibility pop
+#endif
 #ifdef __cplusplus
 }
 #endif

@@ -269,21 +269,22 @@ def test_row_plan_host_side(dl):
     assert not dl.row_plan_advice(dl.OP_FUSED, 8192, 8192, 128, 8192 * 800, 8000)   # Kmat and V of 8 MiB: the slices first
     assert not dl.row_plan_advice(7, 2048, 2048, 64, 2048 * 100, 500)
     bogus = ctypes.c_void_p(256)   # never dereferenced: the checks come first
-    assert L.sddmm_csr_f32_planned(2, 2, -4, 1, None, None, None, None, None, bogus, 24, None) == dl.E_INVALID_ARG
-    assert L.sddmm_csr_f32_planned(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, bogus, 23, None) == dl.E_WORKSPACE
-    assert L.sddmm_csr_f32_planned(2, 2, 32, 1, None, None, None, None, None, None, 0, None) == dl.E_INVALID_ARG
-    assert L.fused_sddmm_spmm_f32_planned(2, 2, 32, 9, None, None, None, None, None, 1.0, None, bogus, 24, None) == dl.E_INVALID_ARG
-    assert L.fused_sddmm_spmm_f32_planned(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, 1.0, bogus, bogus, 23, None) == dl.E_WORKSPACE
-    assert L.fused_sddmm_spmm_f32_planned(2, 2, 32, 1, None, None, None, None, None, 1.0, None, None, 0, None) == dl.E_INVALID_ARG
+    plan_of = lambda n: n | dl.HINT_ROW_PLAN   # (a row plan of n bytes as the workspace of the named entry points)
+    assert L.sddmm_csr_f32(2, 2, -4, 1, None, None, None, None, None, bogus, plan_of(24), None) == dl.E_INVALID_ARG
+    assert L.sddmm_csr_f32(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, bogus, plan_of(23), None) == dl.E_WORKSPACE
+    assert L.sddmm_csr_f32(2, 2, 32, 1, None, None, None, None, None, None, 0, None) == dl.E_INVALID_ARG
+    assert L.fused_sddmm_spmm_f32(2, 2, 32, 9, None, None, None, None, None, 1.0, None, bogus, plan_of(24), None) == dl.E_INVALID_ARG
+    assert L.fused_sddmm_spmm_f32(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, 1.0, bogus, bogus, plan_of(23), None) == dl.E_WORKSPACE
+    assert L.fused_sddmm_spmm_f32(2, 2, 32, 1, None, None, None, None, None, 1.0, None, None, 0, None) == dl.E_INVALID_ARG
     assert L.dlspm_row_plan_build(-1, bogus, bogus, 0, None) == dl.E_INVALID_ARG
     assert L.dlspm_row_plan_build(8, None, bogus, 96, None) == dl.E_INVALID_ARG
     assert L.dlspm_row_plan_build(8, bogus, bogus, 95, None) == dl.E_WORKSPACE
     assert L.dlspm_row_plan_build(4096, bogus, bogus, 3 * 4096 * 4, None) == dl.E_WORKSPACE   # beyond 2048 rows: room for the sort
     assert L.dlspm_row_plan_build(0, None, None, 0, None) == dl.OK
-    assert L.spmm_csr_f32_planned(-1, 1, 1, 0, None, None, None, None, None, bogus, 0, None) == dl.E_INVALID_ARG
-    assert L.spmm_csr_f32_planned(2, 2, 2, 5, None, None, None, None, None, bogus, 24, None) == dl.E_INVALID_ARG
-    assert L.spmm_csr_f32_planned(2, 2, 2, 1, bogus, bogus, bogus, bogus, bogus, bogus, 23, None) == dl.E_WORKSPACE
-    assert L.spmm_csr_f32_planned(2, 2, 2, 1, None, None, None, None, None, None, 0, None) == dl.E_INVALID_ARG  # as spmm_csr_f32
+    assert L.spmm_csr_f32(-1, 1, 1, 0, None, None, None, None, None, bogus, plan_of(0), None) == dl.E_INVALID_ARG
+    assert L.spmm_csr_f32(2, 2, 2, 5, None, None, None, None, None, bogus, plan_of(24), None) == dl.E_INVALID_ARG
+    assert L.spmm_csr_f32(2, 2, 2, 1, bogus, bogus, bogus, bogus, bogus, bogus, plan_of(23), None) == dl.E_WORKSPACE
+    assert L.spmm_csr_f32(2, 2, 2, 1, None, None, None, None, None, None, 0, None) == dl.E_INVALID_ARG
 
 
 def test_tuning_overrides_go_through_one_call_and_the_environment_is_read_once(dl):
@@ -365,7 +366,6 @@ def test_device_info_and_hints_without_a_gpu(dl):
     assert L.sddmm_csr_f32(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, bogus, 23 | dl.HINT_ROW_PLAN, None) == dl.E_WORKSPACE
     assert L.fused_sddmm_spmm_f32(2, 2, 32, 1, bogus, bogus, bogus, bogus, bogus, 1.0, bogus, bogus, 23 | dl.HINT_ROW_PLAN, None) == dl.E_WORKSPACE
     assert L.spmm_csr_f32(0, 5, 5, 0, None, None, None, None, None, None, dl.HINT_ROWS_EVEN, None) == dl.OK
-    assert L.spmm_csr_f32_planned(2, 2, 2, 1, bogus, bogus, bogus, bogus, bogus, bogus, 24 | dl.HINT_ROWS_EVEN, None) == dl.E_INVALID_ARG
     assert dl.row_plan_bytes(2048) == 3 * 2048 * 4 and dl.row_plan_bytes(2049) == 3 * 2049 * 4 + 4 + 2 * 2049 * 8
     # Bits of the hint byte that mean nothing are refused, so a "plenty of scratch" size such as SIZE_MAX cannot turn
     # scratch memory into a row plan; so are a plan of 2^48 bytes and more, both kinds of plan at once, and the

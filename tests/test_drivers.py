@@ -408,7 +408,7 @@ def test_drivers_pass_the_workspace_only_for_uneven_rows():
 @pytest.mark.gpu
 def test_spmm_driver_builds_a_row_plan_for_small_uneven_matrices():
     """The headline configuration (2048 x 512, lognormal rows, one row per workgroup): the driver builds the row plan
-    once and launches spmm_csr_f32_planned; with --no-plan, or on even rows, it does not; all self-check."""
+    once and launches spmm_csr_f32 with it; with --no-plan, or on even rows, it does not; all self-check."""
     rc, out = run("spmm_run", "--cfg", 2, "--iters", 5)
     assert rc == 0 and "PASS" in out and "row plan:" in out and "uneven, row plan" in out, out
     rc, out = run("spmm_run", "--cfg", 2, "--iters", 5, "--no-plan")

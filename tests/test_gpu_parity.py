@@ -527,7 +527,7 @@ def test_exact_integer_properties_at_large_size(torch_cuda, dl):
 
 
 def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle):
-    """spmm_csr_f32_planned hands the rows to the workgroups in the plan's order (longest first), one row per four-wave
+    """spmm_csr_f32 with a row plan hands the rows to the workgroups in the plan's order (longest first), one row per four-wave
     workgroup, and must return the bits of spmm_csr_f32 (NULL workspace) in that same shape -- which is the size rule's
     own shape for most of these cases, and the shape forced by the tuning override split = (4, 1) where the rule groups rows and the plan
     ungroups them. The plan itself is a permutation of the rows with each row's own offsets. Short rows, column tiles of a
@@ -583,7 +583,7 @@ def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle):
 
 
 def test_row_plan_for_sddmm_and_the_fused_op(torch_cuda, dl, oracle):
-    """The same plan drives sddmm_csr_f32_planned and fused_sddmm_spmm_f32_planned: one row of the mask per four-wave
+    """The same plan drives sddmm_csr_f32 and fused_sddmm_spmm_f32: one row of the mask per four-wave
     workgroup, in plan order. Their results must have the bits of the plain calls in that same shape (the size rule's
     own, or the tuning override split = (4, 1) where the rule groups rows), and agree with the oracle; widths outside 16 < D <= 512 and short
     rows run as without a plan."""
@@ -767,7 +767,7 @@ def test_plan_build_and_planned_launches_in_one_hip_graph(torch_cuda, dl, oracle
 
 def test_hint_bits_and_the_deprecated_constant(torch_cuda, dl):
     """The even-rows hint as a bit of workspace_bytes (NULL workspace) and as the deprecated pointer constant select the
-    same launch and give the same bits; the *_planned entry points are the named calls with DLSPM_HINT_ROW_PLAN."""
+    same launch and give the same bits; a row plan is passed as the workspace with DLSPM_HINT_ROW_PLAN."""
     import ctypes
 
     torch = torch_cuda
@@ -788,11 +788,11 @@ def test_hint_bits_and_the_deprecated_constant(torch_cuda, dl):
     assert torch.equal(by_bit, by_constant) and not torch.equal(by_bit, plain) and torch.allclose(by_bit, plain, rtol=1e-4, atol=1e-4)
     plan = dl.row_plan(ro_d)
     via_named = dl.spmm(ro_d, ci_d, va, B, plan=plan).clone()
-    via_alias = torch.empty_like(via_named)
-    st = L.spmm_csr_f32_planned(M, K, N, ci.size, vp(ro_d.data_ptr()), vp(ci_d.data_ptr()), vp(va.data_ptr()), vp(B.data_ptr()),
-                                vp(via_alias.data_ptr()), vp(plan.data_ptr()), plan.numel() * 4,
-                                vp(torch.cuda.current_stream().cuda_stream))
-    assert st == dl.OK and torch.equal(via_named, via_alias)
+    via_abi = torch.empty_like(via_named)
+    st = L.spmm_csr_f32(M, K, N, ci.size, vp(ro_d.data_ptr()), vp(ci_d.data_ptr()), vp(va.data_ptr()), vp(B.data_ptr()),
+                        vp(via_abi.data_ptr()), vp(plan.data_ptr()), (plan.numel() * 4) | dl.HINT_ROW_PLAN,
+                        vp(torch.cuda.current_stream().cuda_stream))
+    assert st == dl.OK and torch.equal(via_named, via_abi) and not torch.equal(via_named, torch.zeros_like(via_named))
 
 
 def test_streamed_results_have_the_bits_of_ordinary_stores(torch_cuda, dl, oracle):
