@@ -395,6 +395,14 @@ def test_library_exports_every_declared_symbol(dl):
     for name in declared_functions():
         assert hasattr(lib, name), f"{name} is declared in include/dlspm_hip.h but not exported"
     assert set(declared_functions()) == set(dl.EXPORTS)
+    # ... and nothing else: the rest of the library has hidden visibility
+    import shutil
+    import subprocess
+
+    if shutil.which("nm"):
+        out = subprocess.run(["nm", "-D", "--defined-only", dl.LIB_PATH], capture_output=True, text=True, check=True).stdout
+        exported = {line.split()[2] for line in out.splitlines() if len(line.split()) == 3 and line.split()[1] in "TW"}
+        assert exported == set(declared_functions()), sorted(exported ^ set(declared_functions()))
 
 
 def test_host_only_entry_points_answer_without_a_gpu(dl):
