@@ -603,7 +603,7 @@ static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int n
     // 256 rows, where most rows would be cut: 0.85 ... 1.5 times the time of the plan over whole rows; 512 rows: 0.66 ... 1.0)
     if (second_kernel && M < 2 * cus) return false;
     const long long share = std::max<long long>(ceil_div(nnz, cus), 1);
-    const long long longest_whole = (share * kCutLongestPct + 99) / 100;
+    const long long longest_whole = (share * kCutAdvicePct + 99) / 100;
     if (max_row_len <= longest_whole) return false;
     const double bytes_per_nonzero = (op == DLSPM_OP_FUSED ? 2.0 : 1.0) * (double)std::min(width, 512) * sizeof(float);
     const double saved_ns = (double)(max_row_len - longest_whole) * bytes_per_nonzero / 115.0;

@@ -241,7 +241,13 @@ void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, co
 // All offsets are bytes from the start of the plan's memory; the launches read the first 4 x entries ints (first
 // nonzero, end, row, slot) and, SpMM and the fused op, the partial rows of the pieces and the list of cut rows.
 constexpr int kCutPlanMaxRows = 1 << 20;  // a cut plan is built by one workgroup: not for taller matrices
-constexpr int kCutPiecePct = 100, kCutLongestPct = 150;  // the rule (dlspm_tuning.cut_piece_pct / .cut_longest_pct override it)
+// The rule (dlspm_tuning.cut_piece_pct / .cut_longest_pct override it): rows above one share in pieces of at most three
+// quarters of a share. Against pieces of a share for rows above one and a half (every fourth of the 302 long-row files of
+// the reference's data set, geometric means): SpMM at N = 256 4.95 -> 4.83 us, SDDMM at D = 128 3.54 -> 3.45 us, the fused
+// op at D = 64 5.59 -> 5.62 us; 512 x 2048 with a row of 4.7 shares: SpMM 5.59 -> 5.18 us. Half a share (and 75 %): 4.90 /
+// 3.54 / 5.68 us.
+constexpr int kCutPiecePct = 75, kCutLongestPct = 100;
+constexpr int kCutAdvicePct = 150;  // a cut plan is advised from a longest row of this many per cent of a share on
 struct CutPlan {
     int entries;      // M + ceil(bins x 100 / piece_pct)
     int bins;         // compute units the plan was sized for (at most 256)

@@ -560,7 +560,7 @@ __global__ __launch_bounds__(kPlanThreads) void plan_emit_kernel(int M, const in
 //
 // A row longer than one compute unit's share of the nonzeros sets the time of the whole launch through the one compute
 // unit it runs on. With share = ceil(nnz / bins) (at least 1), piece = ceil(share x piece_pct / 100) and longest =
-// max(piece, ceil(share x longest_pct / 100)) (the rule: 100 and 150 per cent), a row of more than `longest` nonzeros is
+// max(piece, ceil(share x longest_pct / 100)) (the rule: 75 and 100 per cent), a row of more than `longest` nonzeros is
 // cut into c pieces of ceil(length / c) nonzeros (the last one what is left; rows of a few nonzeros can end in empty ones), c the smallest power of two
 // with pieces of at most `piece` nonzeros (256 at most) -- a power of two, so that a launch can also give each piece the
 // row's whole length and 1/c of the COLUMNS (SpMM), and so that a piece's range follows from its row's by a shift -- and

@@ -260,15 +260,15 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
  */
 size_t dlspm_row_plan_bytes(int M);
 /*
- * Cut plan: a row plan that also cuts rows. A row that holds more than one and a half times a compute unit's share of
- * the nonzeros (share = nnz / compute units) sets the time of the launch by itself, through the one compute unit it
- * runs on, whatever the order of the rows. A cut plan hands such a row out in 2, 4, ... 256 equal pieces (the fewest
- * that are no longer than a share) to as many workgroups. SDDMM pieces take a share of the row's nonzeros and write
+ * Cut plan: a row plan that also cuts rows. A row that holds much more than a compute unit's share of the nonzeros
+ * (share = nnz / compute units) sets the time of the launch by itself, through the one compute unit it runs on,
+ * whatever the order of the rows. A cut plan hands every row above one share out in 2, 4, ... 256 equal pieces (the
+ * fewest that are no longer than three quarters of a share) to as many workgroups. SDDMM pieces take a share of the row's nonzeros and write
  * their own CSR slots (same bits as any other schedule). SpMM at 33 ... 512 columns gives every piece ALL nonzeros of the
  * row and a share of its columns: one kernel, nothing to combine. The fused op, and SpMM at other widths, write one
  * partial row per piece into memory that follows the plan, and a second small kernel adds the pieces of every cut row
  * in piece order. No atomics, no fences anywhere: deterministic; rows that are not cut are summed as by the plain plan.
- * The plan has room for the most pieces any matrix of M rows can need -- M + 2 x compute units entries -- so its size
+ * The plan has room for the most pieces any matrix of M rows can need -- M + 8/3 x compute units entries -- so its size
  * and the launches' grids depend on M, the width and the device only, never on the matrix, and building it needs no
  * look at the matrix from the host.
  *   dlspm_row_plan_bytes_for(op, M, N_or_D)  bytes of DEVICE memory for the cut plan of a matrix of M rows and the
@@ -367,8 +367,8 @@ typedef struct dlspm_tuning {
                           /* (DLSPM_HINT_BANDED asks for the same per call.)                                          */
     int stream_results;   /* results stored with the non-temporal hint: -1 the size rule (dense result rows from one   */
                           /* L2's worth on, SDDMM results from one and a half), 0 never, 1 always                      */
-    int cut_piece_pct;    /* cut plans: the longest piece, in per cent of a share (nnz / compute units); 0 = the rule, 100 */
-    int cut_longest_pct;  /* ... and the longest row that stays whole; 0 = the rule, 150. Both 10 ... 1000; they enter the  */
+    int cut_piece_pct;    /* cut plans: the longest piece, in per cent of a share (nnz / compute units); 0 = the rule, 75  */
+    int cut_longest_pct;  /* ... and the longest row that stays whole; 0 = the rule, 100. Both 10 ... 1000; they enter the  */
                           /* size of a cut plan, so set them before dlspm_row_plan_bytes_for and keep them for the launches */
     int rules_off;        /* DLSPM_RULE_* bits: size rules switched off, to measure what each is worth; 0 = all on        */
     int compute_units;    /* 0 = the device's own; n (8 ... 1024, a multiple of 8): rules, grids and plans as on a device of n  */

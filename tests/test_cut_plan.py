@@ -61,12 +61,12 @@ def run_spmm(L, ro, ci, va, B, G, W, R):
     return rc, C, writes
 
 
-def sizes(M, bins, piece_pct=100, longest_pct=150):
+def sizes(M, bins, piece_pct=75, longest_pct=100):
     """(entries, most cut rows) of a cut plan of M rows."""
     return M + 2 * -(-bins * 100 // piece_pct), -(-bins * 100 // longest_pct)
 
 
-def cut_list_offset(M, bins, piece_pct=100, longest_pct=150):
+def cut_list_offset(M, bins, piece_pct=75, longest_pct=100):
     """Where the list of cut rows lies in a cut plan, in ints (the layout of cut_plan_layout in csrc/plan.hip: 4 x entries
     ints of plan, the sort keys beyond 2048 entries, the virtual rows, then the list)."""
     E, _ = sizes(M, bins, piece_pct, longest_pct)
@@ -77,7 +77,7 @@ def cut_list_offset(M, bins, piece_pct=100, longest_pct=150):
     return at // 4
 
 
-def cut_model(L, ro, bins, order=0, piece_pct=100, longest_pct=150):
+def cut_model(L, ro, bins, order=0, piece_pct=75, longest_pct=100):
     """(plan[4 x entries], cut list, v_off, v_row, v_slot) by the host definition."""
     ro = np.ascontiguousarray(ro, dtype=np.int32)
     M = ro.size - 1
@@ -116,7 +116,7 @@ ROW_CASES = [
 
 
 @pytest.mark.parametrize("name,make", ROW_CASES, ids=[c[0] for c in ROW_CASES])
-@pytest.mark.parametrize("bins,piece_pct,longest_pct", [(256, 100, 150), (64, 100, 150), (7, 100, 150), (256, 50, 100), (256, 33, 40),
+@pytest.mark.parametrize("bins,piece_pct,longest_pct", [(256, 75, 100), (256, 100, 150), (64, 75, 100), (7, 100, 150), (256, 50, 100), (256, 33, 40),
                                                         (104, 200, 150), (256, 1000, 10)])
 def test_cut_rule_partitions_rows_within_its_bounds(model, name, make, bins, piece_pct, longest_pct):
     """CPU: every row is covered by its virtual rows exactly, in order; only rows above one and a half shares are cut,
@@ -184,7 +184,7 @@ def test_cut_plan_sizes_and_advice(dl):
     b0 = dl.row_plan_bytes_for(dl.OP_SDDMM, 512, 128)
     assert b0 > 0 and b0 == dl.row_plan_bytes_for(dl.OP_SDDMM, 512, 7)
     b1, b2 = dl.row_plan_bytes_for(dl.OP_SPMM, 512, 128), dl.row_plan_bytes_for(dl.OP_SPMM, 512, 256)
-    assert b0 < b1 < b2 and b2 - b1 == (2 * 256 + 171) * 128 * 4   # room for 2 x 256 x 100 / 100 + ceil(256 x 100 / 150) pieces
+    assert b0 < b1 < b2 and b2 - b1 == (2 * 342 + 256) * 128 * 4   # room for 2 x ceil(256 x 100 / 75) + 256 x 100 / 100 pieces
     assert dl.row_plan_bytes_for(dl.OP_FUSED, 512, 256) == b2
     assert dl.row_plan_bytes_for(dl.OP_SPMM, (1 << 20) + 1, 64) == 0 and dl.row_plan_bytes_for(7, 512, 64) == 0
     assert dl.row_plan_bytes_for(dl.OP_SPMM, 0, 64) == 0
@@ -256,7 +256,7 @@ def test_gpu_cut_plan_equals_its_sequential_definition(model, dl):
     for name, K, ro, ci in gpu_cases():
         M = ro.size - 1
         print(f"cut plan build: {name} {M}x{K} nnz {ci.size}", flush=True)
-        for order, piece_pct, longest_pct in ((0, 100, 150), (2, 100, 150), (0, 50, 100), (0, 25, 30)):
+        for order, piece_pct, longest_pct in ((0, 75, 100), (2, 100, 150), (0, 50, 100), (0, 25, 30)):
             E, max_cut = sizes(M, bins, piece_pct, longest_pct)
             dl.set_tuning(plan_order=order, cut_piece_pct=piece_pct, cut_longest_pct=longest_pct)
             mem = torch.full(((dl.row_plan_bytes_for(dl.OP_SDDMM, M, 0) + 3) // 4,), -7, dtype=torch.int32, device="cuda")
@@ -286,7 +286,7 @@ def combine(per_virtual_row, M, v_row, v_slot, cut, max_cut):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("width,piece_pct,longest_pct", [(256, 100, 150), (128, 100, 150), (64, 100, 150), (49, 100, 150), (392, 100, 150),
+@pytest.mark.parametrize("width,piece_pct,longest_pct", [(256, 75, 100), (128, 75, 100), (64, 100, 150), (49, 75, 100), (392, 100, 150),
                                                          (256, 50, 100), (64, 25, 30), (250, 100, 150), (100, 100, 150), (130, 10, 10)])
 def test_gpu_launches_with_a_cut_plan(model, dl, oracle, width, piece_pct, longest_pct):
     """All three ops with DLSPM_HINT_CUT_PLAN against the host model (bit for bit) and the oracle (1e-4); SDDMM also

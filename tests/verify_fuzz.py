@@ -52,7 +52,7 @@ def random_tuning(rng):
     if rng.random() < 0.5:
         t["rules_off"] = int(rng.integers(0, 256))
     if rng.random() < 0.3:
-        t["cut_piece_pct"], t["cut_longest_pct"] = pick([(100, 150), (50, 75), (25, 30), (200, 150), (10, 10), (1000, 1000)])
+        t["cut_piece_pct"], t["cut_longest_pct"] = pick([(100, 150), (75, 100), (50, 75), (25, 30), (200, 150), (10, 10), (1000, 1000)])
     if rng.random() < 0.3:
         t["compute_units"] = pick([8, 32, 64, 128, 304, 1024])
     return t
