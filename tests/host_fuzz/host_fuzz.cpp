@@ -28,8 +28,13 @@ int main()
         (void)dlspm_describe_launch_rows(op, M, K, W, nnz, DLSPM_PASS_ROWS_EVEN, shape);
         (void)dlspm_describe_launch_rows(op, M, K, W, nnz, DLSPM_PASS_WORKSPACE, shape);
         volatile size_t pb = dlspm_row_plan_bytes(M);
-        (void)b; (void)a; (void)p; (void)pb;
-        if (!no_device) { calls += 8; return; }
+        volatile size_t cb = dlspm_row_plan_bytes_for(op, M, W);
+        // the one-look advice on a matrix description of these sizes (any figures: it must answer or refuse, never crash)
+        dlspm_matrix_info mi = {M, K, nnz, longest, (int)(nnz % 7), K / 3 + 1, (int)((unsigned)nnz % 8001u), (int)((unsigned)M % 8001u)};
+        dlspm_call_plan cp;
+        volatile int ad = dlspm_advise(op, W, &mi, &cp);
+        (void)b; (void)a; (void)p; (void)pb; (void)cb; (void)ad;
+        if (!no_device) { calls += 10; return; }
         // the compute entry points without a device and with pointers that must not be touched: a status, nothing else
         float* bad = reinterpret_cast<float*>(16);
         int* badi = reinterpret_cast<int*>(16);
@@ -38,8 +43,12 @@ int main()
         volatile int e3 = fused_sddmm_spmm_f32(M, K, W, nnz, badi, badi, bad, bad, bad, 0.5f, bad, bad, (size_t)longest | DLSPM_HINT_ROW_PLAN, nullptr);
         volatile int e4 = dlspm_row_plan_build(M, badi, bad, (size_t)nnz, nullptr);
         volatile int e5 = spmm_csr_f32_static(M, K, W, nnz, badi, badi, bad, bad, bad, nullptr);
-        (void)e1; (void)e2; (void)e3; (void)e4; (void)e5;
-        calls += 13;
+        volatile int e6 = dlspm_row_plan_build_cut(M, badi, bad, (size_t)nnz, nullptr);
+        volatile int e7 = sddmm_csr_f32(M, K, W, nnz, badi, badi, bad, bad, bad, bad, (size_t)longest | DLSPM_HINT_CUT_PLAN, nullptr);
+        dlspm_matrix_info got;
+        volatile int e8 = dlspm_analyze(M, K, nnz, badi, badi, nullptr, &got);
+        (void)e1; (void)e2; (void)e3; (void)e4; (void)e5; (void)e6; (void)e7; (void)e8;
+        calls += 18;
     };
     for (int op = 0; op < 4; ++op)
         for (int i = 0; i < ne; ++i)
@@ -47,6 +56,17 @@ int main()
                 for (int k = 0; k < ne; k += 2)
                     for (int l = 0; l < ne; l += 3) one(op, edge[i], edge[j], edge[k], edge[l], edge[(i + l) % ne]);
     for (int t = 0; t < 200000; ++t) {
+        if (t % 1000 == 0) {  // the rules and plans as for devices of other sizes, and other cut rules
+            dlspm_tuning tune;
+            dlspm_tuning_default(&tune);
+            const int units[] = {0, 8, 32, 64, 304, 1024};
+            const int pcts[] = {0, 10, 33, 75, 100, 1000};
+            tune.compute_units = units[rng() % 6];
+            tune.cut_piece_pct = pcts[rng() % 6];
+            tune.cut_longest_pct = pcts[rng() % 6];
+            tune.rules_off = (int)(rng() % 256);
+            if (dlspm_set_tuning(&tune) != DLSPM_OK) return 1;
+        }
         const int op = (int)(rng() % 3);
         const int M = (int)(rng() % (1u << (1 + rng() % 30)));
         const int K = (int)(rng() % (1u << (1 + rng() % 30)));
