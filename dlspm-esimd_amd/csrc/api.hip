@@ -750,7 +750,7 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz, const int* row_offsets, c
                                                  : fused_launch(args, shape, st);
         return e == hipSuccess ? DLSPM_OK : fail_hip(e);
     }
-    const FusedShape shape = fused_choose(dev, M, D, nnz, vec4, ws.rows_even);
+    const FusedShape shape = fused_choose(dev, M, D, nnz, vec4, ws.rows_even, K);
     if (!ws.rows_even && !ws.banded && ws.mem) {
         const SlicePlan sliced = fused_slice_plan(dev, M, K, D, nnz, shape);
         const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(dev, M, nnz, D, shape.G);
@@ -869,7 +869,7 @@ int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int pa
         const FlatPlan fp = even ? FlatPlan{0, 0, 0} : sddmm_flat_plan(dev, M, nnz, n);  // as sddmm_csr_f32 decides
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_FUSED) {
-        const FusedShape s = fused_choose(dev, M, n, nnz, vec4, even);
+        const FusedShape s = fused_choose(dev, M, n, nnz, vec4, even, K);
         const int tw = s.G * s.vec * s.V;
         shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R;
         shape[7] = (int)ceil_div(n, tw);

@@ -173,7 +173,7 @@ template <typename Launch> static hipError_t dispatch_layout(const FusedShape& s
 // the layouts the column-sliced and planned kernels are built for: 16 < D <= 512 in one column tile
 template <typename L> constexpr bool kOneTileLayout = L::VEC == 4 && L::G1 == 8 && L::DS >= 1;
 
-FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even)
+FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even, int K)
 {
     FusedShape s{};
     s.vec = vec4 ? 4 : 1;
@@ -193,7 +193,16 @@ FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
     // rows per workgroup 1 / 2 / 4 / 8 / 16: 1024 rows 3.3 / 4.4 / 5.5 / 6.9 / 10.9 us; 2048 rows 4.8 / 4.9 / 6.1 / 7.8 /
     // 11.7 us; 4096 rows 7.3 / 7.2 / 6.5 / 8.0 / 11.6 us; 8192 rows 12.1 / 10.4 / 8.3 / 7.2 / 9.2 us; 16384 rows: sixteen;
     // 3072 rows of 102, even: two per workgroup 8.5 us, four 7.2 us)
-    choose_split(dev, M, ceil_div(D, tw), nnz, SplitRule{3, tw >= 1024 ? 4 : 16, kWave / s.G, false, 96}, rows_even, s.W, s.R);
+    // Kmat and V beyond one L2 (K known: a plain call or one with the even-rows hint): long rows are grouped four to a
+    // workgroup, one whole row per wave, as under the even-rows hint, whatever the caller said. Waves that live for a whole row
+    // and start together sweep the sorted columns together, so the rows of Kmat and V they gather are in L2 at the same
+    // time: even rows (Bernoulli patterns, D = 128 / 256) 8192 x 8192 398 -> 243 us and 1159 -> 638 us, 16384 x 8192 462 ->
+    // 283 us, 4096 x 16384 300 -> 144 us; lognormal rows (sigma 0.3 ... 1.0) lose nothing to 8 % (8192 x 8192: 470 -> 475,
+    // 486 -> 514, 545 -> 577 us), which is what a caller with such rows gets back several times over from a row plan or the
+    // column slices. Within one L2 the same grouping gains 6 % on even rows and loses 7 % on uneven ones: only on the hint.
+    const bool beyond_l2 = K > 0 && 2.0 * (double)K * (double)D * sizeof(float) > (double)dev.l2_bytes;
+    choose_split(dev, M, ceil_div(D, tw), nnz, SplitRule{3, tw >= 1024 ? 4 : 16, kWave / s.G, false, 96}, rows_even || beyond_l2, s.W,
+                 s.R);
     return s;
 }
 

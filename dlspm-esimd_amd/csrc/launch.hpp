@@ -214,7 +214,8 @@ hipError_t sddmm_flat_launch(const SddmmArgs& x, const SddmmShape& s, int chunk,
 hipError_t sddmm_sliced_launch(const SddmmArgs& x, const SddmmShape& s, const SlicePlan& plan, void* workspace,
                                hipStream_t stream);
 
-FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even = false);
+// K > 0: the height of Kmat and V is known and may count (operands beyond one L2 group long rows as under the even-rows hint)
+FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even = false, int K = 0);
 hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream);
 hipError_t fused_flat_launch(const FusedArgs& x, const FusedShape& s, const FlatPlan& plan, float* partial,
                              hipStream_t stream);

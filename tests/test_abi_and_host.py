@@ -50,7 +50,8 @@ def test_split_rule_and_the_even_rows_hint(dl):
             nnz = 8192 * 600
             a = dl.describe_launch(op, 8192, 4096, width, nnz)
             b = dl.describe_launch(op, 8192, 4096, width, nnz, rows_even=True)
-            assert (a["W"], a["R"]) == (4, 1) and (b["W"], b["R"]) == (4, 4)
+            # (the fused op groups long rows by itself where Kmat and V together exceed one L2: 2 x 4096 x 256 floats)
+            assert (a["W"], a["R"]) == ((4, 4) if op == dl.OP_FUSED and width == 256 else (4, 1)) and (b["W"], b["R"]) == (4, 4)
             same = lambda d: {k: v for k, v in d.items() if k not in ("R", "flat_chunk", "flat_units")}
             assert same(a) == same(b)
             # SDDMM needs no memory for its flat schedule and takes it by the sizes alone -- except for rows known to be even
@@ -65,6 +66,11 @@ def test_split_rule_and_the_even_rows_hint(dl):
         a = dl.describe_launch(op, 65536, 1024, 64, 65536 * 20)
         b = dl.describe_launch(op, 65536, 1024, 64, 65536 * 20, rows_even=True)
         assert a == b and a["R"] == 16
+    # the fused op, Kmat and V together beyond one L2 (2 x K x D floats > 4 MiB): long rows four to a workgroup without the hint
+    assert dl.describe_launch(dl.OP_FUSED, 8192, 8192, 128, 8192 * 819)["R"] == 4
+    assert dl.describe_launch(dl.OP_FUSED, 8192, 4096, 128, 8192 * 410)["R"] == 1      # exactly one L2: only on the hint
+    assert dl.describe_launch(dl.OP_FUSED, 8192, 8192, 128, 8192 * 40)["R"] == dl.describe_launch(dl.OP_FUSED, 8192, 1024, 128, 8192 * 40)["R"]  # short rows: the size rule
+    assert dl.describe_launch(dl.OP_SDDMM, 8192, 16384, 128, 8192 * 819)["R"] == 1     # SDDMM: its flat schedule instead
     for cfg in ((dl.OP_SPMM, 512, 512, 128, 78848), (dl.OP_SPMM, 2048, 512, 256, 105687),
                 (dl.OP_SDDMM, 2048, 2048, 128, 209715), (dl.OP_FUSED, 4096, 4096, 64, 323000)):
         assert dl.describe_launch(*cfg) == dl.describe_launch(*cfg, rows_even=True)
