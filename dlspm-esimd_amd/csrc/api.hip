@@ -235,7 +235,13 @@ SlicePlan slice_plan(const DeviceInfo& dev, int M, int K, int width, int nnz, in
     if (just_fills && width < 128) slices = 0;
     const long long fit = (long long)nnz / ((long long)min_row * M);
     if (slices > fit) slices = fit;
-    const bool by_rule = bytes >= l2 && nnz >= kSlicedMinNnz && slices >= 2;
+    // Fewer than four rows per compute unit: one slice's share of the rows does not fill the device and the launches that
+    // follow each other cost more than the cache misses they save (512 rows of ~2050 nonzeros, K = 8192 / 32768, without /
+    // with slices: SpMM at N = 256 42.7 / 48.7 and 53.2 / 62.7 us, SDDMM at D = 128 23.4 / 27.8 and 29.8 / 33.9 us, fused at
+    // D = 128 40.8 / 48.4 and 57.3 / 61.0 us; 1024 rows: 84.5 / 80.7 and 178.8 / 94.7 us, 40.9 / 44.8 and 114.0 / 51.9 us,
+    // 86.2 / 80.8 and 169.0 / 96.7 us).
+    const bool rows_fill = (long long)M >= kSlicedMinRowsPerCu * dev.cus;
+    const bool by_rule = bytes >= l2 && nnz >= kSlicedMinNnz && slices >= 2 && rows_fill;
     if (force == 0 || force == 1 || (force < 0 && !by_rule)) return p;
     if (force >= 2) slices = force < kSliceMaxSlices ? force : kSliceMaxSlices;
     if (slices > K) slices = K;

@@ -163,6 +163,7 @@ struct FusedArgs {
 // Flat schedule: `units` waves of `chunk` consecutive nonzeros each; `bytes` of device workspace for the partial
 // rows (units x 2 x width floats). chunk == 0: not used for this problem.
 constexpr int kSlicedMinNnz = 1 << 19;  // the column-sliced schedule (two more launches) only from this many nonzeros on
+constexpr long long kSlicedMinRowsPerCu = 4;  // ... and from this many rows per compute unit on (one slice's workgroups must fill the device)
 constexpr int kFlatWaves = 4;  // waves per workgroup of the flat kernels (the waves are independent)
 struct FlatPlan {
     int chunk;

@@ -280,7 +280,7 @@ static int spmm_tile_width(const DeviceInfo& dev, int M, int K, int N, int nnz, 
     // with workspace memory the column-sliced schedule cuts a taller slab along K as well, from two slices of 32
     // nonzeros per row on (8192 x 32768, N = 1024: 925 us in tiles of 32 without memory, 807 us in 16 slices of tiles
     // of 512, 533 us in 8 slices of tiles of 128; 2048 x 131072, N = 512: 384 / 324 / 250 us)
-    const bool sliced_too = !narrow_tiles && nnz >= kSlicedMinNnz && (long long)nnz >= 64ll * M;
+    const bool sliced_too = !narrow_tiles && nnz >= kSlicedMinNnz && (long long)nnz >= 64ll * M && (long long)M >= kSlicedMinRowsPerCu * dev.cus;
     const bool narrow_ok =
         (long long)nnz >= 32ll * M && ((long long)K * tile * (long long)sizeof(float) <= 2 * l2 || sliced_too);
     if (!narrow_ok) tile = 512;

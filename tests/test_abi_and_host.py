@@ -201,6 +201,12 @@ def test_column_sliced_schedule_rule(dl):
     assert dl.describe_slices(dl.OP_SDDMM, M, K, 256, nnz)[0] == 4      # rhs: 8 MiB in slices of 2 MiB (no partial rows); only the boundaries need memory
     assert dl.workspace_bytes(dl.OP_SDDMM, M, K, 256, nnz) == -(-5 * M * 4 // 256) * 256
     assert dl.describe_slices(dl.OP_SDDMM, M, K, 100, nnz)[0] == 0 and dl.workspace_bytes(dl.OP_SDDMM, M, K, 100, nnz) == 0
+    # fewer than four rows per compute unit (1024 on this device): one slice's workgroups would not fill it
+    for op, width in ((dl.OP_SPMM, 256), (dl.OP_SDDMM, 128), (dl.OP_FUSED, 128)):
+        assert dl.describe_slices(op, 512, 4 * K, width, 512 * 2048)[0] == 0
+        assert dl.describe_slices(op, 1023, 4 * K, width, 1023 * 2048)[0] == 0
+        assert dl.describe_slices(op, 1024, 4 * K, width, 1024 * 2048)[0] >= 6
+    assert dl.workspace_bytes(dl.OP_SDDMM, 512, 4 * K, 128, 512 * 2048) == 0
     slices, R = dl.describe_slices(dl.OP_FUSED, M, K, 256, nnz)
     assert R == 2                                                       # 133 nonzeros per row and slice
     bounds = -(-(slices + 1) * M * 4 // 256) * 256
@@ -223,7 +229,10 @@ def test_workspace_advice(dl):
     assert A(dl.OP_SPMM, M, K, 128, nnz, mean + 10) == dl.PASS_ROWS_EVEN
     assert A(dl.OP_SPMM, M, K, 128, nnz, 3 * mean) == dl.PASS_WORKSPACE
     assert A(dl.OP_SDDMM, M, K, 128, nnz, mean + 10) == dl.PASS_WORKSPACE
-    # SpMM on rows below 128 nonzeros: narrower column tiles without memory beat the slices
+    # few rows: no slices, and even rows take the hint (SpMM, 256 x 8192 half full at N = 256: 42.8 us against 48.2 us with memory)
+    assert A(dl.OP_SPMM, 256, K, 256, 256 * 4096, 4200) == dl.PASS_ROWS_EVEN
+    assert A(dl.OP_SDDMM, 512, K, 128, 512 * 2048, 2150) == dl.PASS_ROWS_EVEN
+    assert A(dl.OP_SDDMM, 1024, 4 * K, 128, 1024 * 2048, 2150) == dl.PASS_WORKSPACE
     assert dl.describe_slices(dl.OP_SPMM, M, 4 * K, 256, M * 120)[0] == 3
     assert A(dl.OP_SPMM, M, 4 * K, 256, M * 120, 3 * 120) == dl.PASS_NULL
     assert A(dl.OP_SPMM, M, 4 * K, 256, M * 120, 130) == dl.PASS_ROWS_EVEN
