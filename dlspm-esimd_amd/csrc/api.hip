@@ -416,7 +416,7 @@ int dlspm_set_tuning(const dlspm_tuning* t)
         t->tile_major < -1 || t->tile_major > 1 || t->tile_width < 0 || t->plan_order < 0 || t->plan_order > 2 ||
         t->xcd_contiguous < 0 || t->xcd_contiguous > 1 || t->stream_results < -1 || t->stream_results > 1 ||
         (t->cut_piece_pct != 0 && (t->cut_piece_pct < 10 || t->cut_piece_pct > 1000)) ||
-        (t->cut_longest_pct != 0 && (t->cut_longest_pct < 10 || t->cut_longest_pct > 1000)) || t->rules_off < 0 || t->rules_off > 255 ||
+        (t->cut_longest_pct != 0 && (t->cut_longest_pct < 10 || t->cut_longest_pct > 1000)) || t->rules_off < 0 || t->rules_off > 511 ||
         (t->compute_units != 0 && (t->compute_units < 8 || t->compute_units > 1024 || t->compute_units % 8 != 0)))
         return DLSPM_E_INVALID_ARG;
     t_tuning.split_w = t->split_w;
@@ -477,20 +477,21 @@ int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int
         const CutPlan cp = cut_plan_layout(M, N, dev.cus);
         if (cp.bytes == 0 || ws.bytes < cp.bytes) return DLSPM_E_WORKSPACE;
         SpmmShape shape = spmm_choose(dev, M, K, N, nnz, vec4, false, true);
-        e = spmm_plan_applies(dev, shape, M, N, nnz) ? spmm_pieces_launch(args, shape, cp, ws.mem, st) : spmm_launch(args, shape, st);
+        e = spmm_plan_applies(dev, shape, M, N, nnz) ? spmm_pieces_launch(args, shape, cp, ws.mem, st)
+                                                : spmm_launch(args, spmm_choose(dev, M, K, N, nnz, vec4, false, true, false, true), st);
         return e == hipSuccess ? DLSPM_OK : fail_hip(e);
     }
     if (ws.row_plan && ws.mem) {
         // the memory holds the row plan of this matrix; sizes a planned launch is not built for run as with NULL
         SpmmShape shape = spmm_choose(dev, M, K, N, nnz, vec4, false, true);
         e = spmm_plan_applies(dev, shape, M, N, nnz) ? spmm_planned_launch(args, shape, static_cast<const int*>(ws.mem), st)
-                                                : spmm_launch(args, shape, st);
+                                                : spmm_launch(args, spmm_choose(dev, M, K, N, nnz, vec4, false, true, false, true), st);
         return e == hipSuccess ? DLSPM_OK : fail_hip(e);
     }
     // a banded matrix (DLSPM_HINT_BANDED) runs as row blocks whatever memory came with the call: column slices and
     // the flat schedule are answers to columns spread over all of K and to uneven rows
     const bool memory = !ws.rows_even && !ws.banded && ws.mem != nullptr;
-    const SpmmShape shape = spmm_choose(dev, M, K, N, nnz, vec4, ws.rows_even, !memory, ws.banded);
+    const SpmmShape shape = spmm_choose(dev, M, K, N, nnz, vec4, ws.rows_even, !memory, ws.banded, !memory);
     if (memory) {
         const SlicePlan sliced = spmm_slice_plan(dev, M, K, N, nnz, shape);
         const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(dev, M, nnz, N, shape.G);
@@ -864,7 +865,7 @@ int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int pa
     const bool vec4 = n >= 4;
     for (int i = 0; i < 10; ++i) shape[i] = 0;
     if (op == DLSPM_OP_SPMM) {
-        const SpmmShape s = spmm_choose(dev, M, K, n, nnz, vec4, even, !memory);
+        const SpmmShape s = spmm_choose(dev, M, K, n, nnz, vec4, even, !memory, false, !memory);
         const int tw = s.G * s.vec * s.V;
         shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[5] = s.W; shape[6] = s.R; shape[7] = (int)ceil_div(n, tw);
         const FlatPlan fp = flat_plan(dev, M, nnz, n, s.G);

@@ -98,7 +98,8 @@ struct Tuning {
 };
 // (the values of DLSPM_RULE_* in the header)
 constexpr int kRuleEightWavesFewRows = 1, kRuleSixteenWavesTallLongRows = 2, kRuleMoreWavesFewLongRows = 4, kRuleGroupRows = 8,
-              kRuleRowAlignedSplit = 16, kRulePlanUngroups = 32, kRuleExactWidthKernels = 64, kRuleCutRowsByColumns = 128;
+              kRuleRowAlignedSplit = 16, kRulePlanUngroups = 32, kRuleExactWidthKernels = 64, kRuleCutRowsByColumns = 128,
+              kRuleFinerColumnTiles = 256;
 
 const Tuning& tuning();
 inline bool rule_on(int rule) { return (tuning().rules_off & rule) == 0; }
@@ -194,7 +195,8 @@ hipError_t slice_bounds_launch(int M, int K, int slices, const int* row_offsets,
 hipError_t slice_sum_launch(long long count, int slices, const float* partial, float* out, hipStream_t stream);
 
 // narrow_tiles: the call passes no workspace memory (column tiles below 128 columns are then allowed)
-SpmmShape spmm_choose(const DeviceInfo& dev, int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles, bool banded = false);
+SpmmShape spmm_choose(const DeviceInfo& dev, int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles, bool banded = false,
+                      bool plain = false);
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
 // Row plan (3 x M ints on the device: first nonzero, end and row number of the row that workgroup i works on): only for
 // shapes of one row per four-wave workgroup and one column tile

@@ -261,16 +261,57 @@ template <typename Launch> static hipError_t dispatch_layout(const SpmmShape& s,
 // for rows of at least 32 nonzeros on average, and only while the slab is at most twice the L2 (measured on graph-
 // like shapes, K = 262144 ... 1048576, 8 nonzeros per row: tiles of 32 up to 2x slower than one tile; 32 per row:
 // equal; K = 65536, slab 8 MiB, 655 per row: 330 -> 236 us).
-// dlspm_tuning.tile_major = 0|1 and .tile_width = 512|...|32 override the rule for tuning sweeps. "The L2" is the
-// device's own figure for one of them (4 MiB on MI355X), "all at once" eight workgroups on each compute unit.
-static int spmm_tile_width(const DeviceInfo& dev, int M, int K, int N, int nnz, bool narrow_tiles)
+// dlspm_tuning.tile_major = 0|1 and .tile_width = 512|...|32 override the rule for tuning sweeps (tile_major = 0 with a
+// width: tiles of that width in row-major order). "The L2" is the device's own figure for one of them (4 MiB on MI355X),
+// "all at once" eight workgroups on each compute unit.
+//
+// Finer tiles for a call without memory or plan (`plain`; kRuleFinerColumnTiles, rows of 16 nonzeros and more on average).
+// Such a call does not know how even the rows are; finer tiles cost even rows little and spread a long row over
+// several compute units. Times in us inside a graph, rule off / on:
+//  * few rows (up to three quarters of a compute unit's worth of row x tile pairs): the widest tile that gives two pairs
+//    per compute unit, row-major. Bernoulli rows, M = 16 / 64 / 128, mean over six shapes: N = 128: 4.20 / 3.40, 4.3 / 3.5,
+//    4.38 / 3.80; N = 256: 4.89 / 3.44, 5.0 / 3.7, 5.28 / 4.50; N = 512: 6.93 / 3.51, 7.3 / 4.6, 7.59 / 5.74; lognormal
+//    rows (sigma 0.8): times 0.35 ... 0.9; at 160 and 192 rows even rows gain nothing (0.96 ... 1.13, the losses at widths
+//    that are not a multiple of the tile) and lognormal ones 10-40 %. The reference's 128 x 1152 and 128 x 512 ResNet-50
+//    layers at N = 256 (26 files): 6.08 / 4.80; at N = 512: 8.81 / 6.51.
+//  * N above 512 and up to eight rows per compute unit: row-major tiles of 256 instead of 512 (200 x 2304, N = 784:
+//    12.2 / 11.5 even, 42.1 / 19.7 lognormal; 1500 x 512, N = 600: 24.8 / 19.3 and 34.4 / 25.6; taller matrices lose:
+//    8192 x 512, N = 784: 57.4 / 62.0).
+//  * B beyond the L2 and N above 512: tile-major order from three pairs per compute unit on (instead of eight) for
+//    matrices of at least half a compute unit's count of rows, in tiles of 64: the finer the tile, the smaller the slab of B
+//    in use at a time and the more evenly long rows spread (256 x 2304, N = 3136: 86.8 / 39.8 even, 134 / 93 lognormal;
+//    1024 x 1152, N = 12544: 212 / 220 and 645 / 251; 2048 x 2304, N = 3136: 225 / 206 and 404 / 234; 4096 x 4096,
+//    N = 3136: 453 / 375 and 679 / 422; even rows lose at most 6 %, at K = 512).
+//  Rows below 16 nonzeros pay the start of a row once more per tile: 256 x 64 with 3 ... 13 per row at N = 3136 lost 13-33 %
+//  to tiles of 256, 512 x 128 with 6 per row at N = 784 10-18 %.
+struct TileChoice { int width, major; };  // width 0: no tiles narrower than a wave covers (or than 512)
+
+// widest tile that one wave covers N with: what a launch without tiles works in
+static int spmm_one_wave_tile(int N) { return N > 256 ? 512 : N > 128 ? 256 : N > 64 ? 128 : N > 32 ? 64 : 32; }
+
+static TileChoice spmm_tile_width(const DeviceInfo& dev, int M, int K, int N, int nnz, bool narrow_tiles, bool plain)
 {
     const long long l2 = dev.l2_bytes;
     const int min_tile = narrow_tiles ? 32 : 128;
-    if (N <= min_tile) return 0;
-    bool on = (double)K * (double)N * (double)sizeof(float) > (double)l2 && (long long)M * ceil_div(N, 512) >= 8ll * dev.cus;
+    if (N <= min_tile) return {0, 0};
+    const bool finer = plain && narrow_tiles && rule_on(kRuleFinerColumnTiles);
+    const bool beyond_l2 = (double)K * (double)N * (double)sizeof(float) > (double)l2;
+    bool on = beyond_l2 && (long long)M * ceil_div(N, 512) >= (finer && N > 512 && 2ll * M >= dev.cus ? 3ll : 8ll) * dev.cus;
     if (tuning().tile_major >= 0) on = tuning().tile_major != 0;
-    if (!on) return 0;
+    if (!on) {
+        const int t = tuning().tile_width;
+        if (tuning().tile_major == 0)  // tuning: tiles of this width in row-major order
+            return (t == 512 || t == 256 || t == 128 || t == 64 || t == 32) && t >= min_tile && t < N ? TileChoice{t, 0} : TileChoice{0, 0};
+        if (!finer || (long long)nnz < 16ll * M) return {0, 0};
+        const int one = spmm_one_wave_tile(N);
+        if (4ll * M * ceil_div(N, one) <= 3ll * dev.cus) {  // few rows
+            int tile = one;
+            while (tile > 32 && (long long)M * ceil_div(N, tile) < 2ll * dev.cus) tile /= 2;
+            if (2 * (N - (int)(ceil_div(N, tile) - 1) * tile) < tile) tile *= 2;  // a last tile less than half full: wider tiles
+            return tile < one && tile < N ? TileChoice{tile, 0} : TileChoice{0, 0};
+        }
+        return N > 512 && M <= 8ll * dev.cus ? TileChoice{256, 0} : TileChoice{0, 0};
+    }
     int tile = min_tile;
     for (int t = 512; t > min_tile; t /= 2)
         if ((long long)K * t * (long long)sizeof(float) <= l2) {
@@ -284,21 +325,24 @@ static int spmm_tile_width(const DeviceInfo& dev, int M, int K, int N, int nnz, 
     const bool narrow_ok =
         (long long)nnz >= 32ll * M && ((long long)K * tile * (long long)sizeof(float) <= 2 * l2 || sliced_too);
     if (!narrow_ok) tile = 512;
+    else if (finer && tile > 64 && N > 512) tile = 64;
     {
         const int t = tuning().tile_width;
         if ((t == 512 || t == 256 || t == 128 || t == 64 || t == 32) && t >= min_tile) tile = t;
     }
-    return tile < N ? tile : 0;  // a single tile: nothing to order
+    return tile < N ? TileChoice{tile, 1} : TileChoice{0, 0};  // a single tile: nothing to order
 }
 
 // Chooses the lane layout from N (and the height of B) and the (W, R) split from the mean row length.
-SpmmShape spmm_choose(const DeviceInfo& dev, int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles, bool banded)
+SpmmShape spmm_choose(const DeviceInfo& dev, int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles, bool banded,
+                      bool plain)
 {
     SpmmShape s{};
     s.vec = vec4 ? 4 : 1;
     // banded (DLSPM_HINT_BANDED): no L2-sized column tiles, each XCD gathers from its own part of B anyway
-    const int tile = vec4 && !banded ? spmm_tile_width(dev, M, K, N, nnz, narrow_tiles) : 0;
-    s.tile_major = tile > 0 ? 1 : 0;
+    const TileChoice tiles = vec4 && !banded ? spmm_tile_width(dev, M, K, N, nnz, narrow_tiles, plain) : TileChoice{0, 0};
+    const int tile = tiles.width;
+    s.tile_major = tiles.major;
     if (vec4) {
         if (tile == 512) { s.G = 64; s.V = 2; }
         else if (tile == 256) { s.G = 64; s.V = 1; }

@@ -77,7 +77,8 @@ class Tuning(ctypes.Structure):
                                             "cut_piece_pct", "cut_longest_pct", "rules_off", "compute_units")]
 
 RULES = {"eight_waves_few_rows": 1, "sixteen_waves_tall_long_rows": 2, "more_waves_few_long_rows": 4, "group_rows": 8,
-         "row_aligned_split": 16, "plan_ungroups": 32, "exact_width_kernels": 64, "cut_rows_by_columns": 128}
+         "row_aligned_split": 16, "plan_ungroups": 32, "exact_width_kernels": 64, "cut_rows_by_columns": 128,
+         "finer_column_tiles": 256}
 
 
 class MatrixInfo(ctypes.Structure):

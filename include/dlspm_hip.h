@@ -357,7 +357,8 @@ typedef struct dlspm_tuning {
     int flat_chunk;       /* nonzeros per wave of the flat schedule (>= 64); 0 = the rule                           */
     int slices;           /* column-sliced schedule: -1 the size rule, 0 never, n >= 2 that many slices             */
     int tile_major;       /* SpMM column tiles one after the other: -1 the rule, 0 no, 1 yes                        */
-    int tile_width;       /* SpMM column tile: 0 the rule, else 512, 256, 128, 64 or 32                             */
+    int tile_width;       /* SpMM column tile: 0 the rule, else 512, 256, 128, 64 or 32 (with tile_major = 0: tiles */
+                          /* of this width in row-major order)                                                       */
     int plan_order;       /* dlspm_row_plan_build: 0 packed (the rule), 1 alternating groups, 2 longest first       */
     int xcd_contiguous;   /* 0 (the rule): neighbouring row blocks go to different XCDs, as the hardware deals them;   */
                           /* 1: each of the eight XCDs works on one contiguous run of row blocks, so that a banded    */
@@ -385,6 +386,8 @@ typedef struct dlspm_tuning {
 #define DLSPM_RULE_EXACT_WIDTH_KERNELS         64  /* SDDMM, fused: kernels without bounds handling for D = 16, 32, ... 512  */
 #define DLSPM_RULE_CUT_ROWS_BY_COLUMNS        128  /* SpMM with a cut plan, 33 ... 512 columns: the pieces of a cut row share  */
                                                    /* its columns, not its nonzeros (no partial rows, no second kernel)       */
+#define DLSPM_RULE_FINER_COLUMN_TILES         256  /* SpMM without memory or plan: narrower column tiles of B for few rows,   */
+                                                   /* and for N above 512 in matrices of up to eight rows per compute unit   */
 void dlspm_tuning_default(dlspm_tuning* t);   /* fills *t with "follow the rules" */
 int dlspm_set_tuning(const dlspm_tuning* t);  /* DLSPM_OK or DLSPM_E_INVALID_ARG (a field out of range) */
 int dlspm_get_tuning(dlspm_tuning* t);        /* what the calling thread's launches currently use */

@@ -108,7 +108,14 @@ def test_split_rule_for_small_matrices(dl):
         assert dl.describe_launch(op, 511, 2304, width, 511 * 96)["W"] == eight
         assert dl.describe_launch(op, 512, 2304, width, 512 * 208)["W"] == 4
     assert dl.describe_launch(dl.OP_SPMM, 256, 2304, 196, 256 * 461)["W"] == 8
-    assert dl.describe_launch(dl.OP_SPMM, 64, 4608, 256, 64 * 800)["W"] == 16
+    # few rows in a plain SpMM call: narrower column tiles of B instead of more waves per row (64 rows x 8 tiles of 32)
+    sh = dl.describe_launch(dl.OP_SPMM, 64, 4608, 256, 64 * 800)
+    assert (sh["W"], sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (4, 32, 8)
+    dl.set_tuning(rules_off=dl.RULES["finer_column_tiles"])
+    try:
+        assert dl.describe_launch(dl.OP_SPMM, 64, 4608, 256, 64 * 800)["W"] == 16
+    finally:
+        dl.set_tuning()
     rows_per_workgroup = lambda op, M, avg: dl.describe_launch(op, M, 1024, 64, M * avg)["R"]
     assert [rows_per_workgroup(dl.OP_FUSED, M, 20) for M in (1024, 2048, 3072, 4096, 8192, 16384)] == [1, 2, 4, 4, 8, 16]
     assert [rows_per_workgroup(dl.OP_SDDMM, M, 20) for M in (1024, 2048, 4096, 8192)] == [2, 4, 8, 16]
@@ -122,13 +129,65 @@ def test_split_rule_for_small_matrices(dl):
     assert dl.row_plan_advice(dl.OP_FUSED, 4096, K, 64, 4096 * 10, 158) == 0  # more rows: short rows stay grouped
 
 
+def test_finer_column_tiles_for_plain_spmm_calls(dl):
+    """A SpMM call without memory or plan does not know how even the rows are: few rows are covered by the widest column
+    tile of B that gives two (row, tile) pairs per compute unit; N above 512 is covered in tiles of 256 instead of 512 up
+    to eight rows per compute unit, and in tile-major tiles of 64 where B exceeds the L2. Not for rows below 16 nonzeros,
+    not with memory or a plan."""
+    tile = lambda M, K, N, per_row, **kw: (lambda sh: (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]))(
+        dl.describe_launch(dl.OP_SPMM, M, K, N, M * per_row, **kw))
+    assert tile(128, 1152, 256, 200) == (64, 4)      # 128 rows x 4 tiles = 512 pairs
+    assert tile(128, 1152, 128, 200) == (32, 4)
+    assert tile(64, 576, 256, 100) == (32, 8)
+    assert tile(64, 576, 512, 100) == (64, 8)
+    assert tile(16, 576, 512, 100) == (32, 16)       # never narrower than 32
+    assert tile(192, 1152, 256, 200) == (64, 4)      # up to three quarters of a compute unit's count of pairs
+    assert tile(193, 1152, 256, 200) == (256, 1)
+    assert tile(128, 1152, 196, 200) == (128, 2)     # tiles of 64 would leave a last tile of 4 columns
+    assert tile(128, 1152, 100, 200) == (64, 2)      # (64 + 36: more than half full)
+    assert tile(128, 1152, 32, 200) == (32, 1)
+    assert tile(128, 1152, 256, 15) == (256, 1)      # short rows pay their start once more per tile
+    assert tile(128, 1152, 256, 200, with_workspace=True) == (256, 1)
+    assert tile(128, 1152, 256, 200, rows_even=True) == (64, 4)   # the hint changes the grouping of rows, not the tiles
+    # N above 512
+    assert tile(1000, 512, 784, 100) == (256, 4)
+    assert tile(2048, 512, 784, 100) == (256, 4)
+    assert tile(2049, 512, 784, 100) == (512, 2)
+    assert tile(1000, 512, 784, 15) == (512, 2)
+    assert tile(64, 576, 3136, 100) == (256, 13)     # 64 x 7 pairs: no longer "few rows"
+    # B beyond the L2 (K x N x 4 > 4 MiB): tile-major tiles of 64 from three pairs per compute unit on, 128 rows and more
+    assert tile(300, 1152, 3136, 100) == (64, 49)
+    assert tile(64, 1152, 12544, 100) == (256, 49)     # fewer rows than half the compute units: row-major tiles of 256
+    assert tile(4096, 4096, 3136, 100) == (64, 49)
+    assert tile(4096, 4096, 3136, 20) == (512, 7)    # rows below 32 nonzeros keep the widest tile, as before
+    dl.set_tuning(rules_off=dl.RULES["finer_column_tiles"])
+    try:
+        assert tile(128, 1152, 256, 200) == (256, 1) and tile(1000, 512, 784, 100) == (512, 2)
+        assert tile(300, 1152, 3136, 100) == (512, 7) and tile(4096, 4096, 3136, 100) == (256, 13)
+    finally:
+        dl.set_tuning()
+    # the tuning fields: tile_major = 0 with a width gives row-major tiles of that width
+    dl.set_tuning(tile_major=0, tile_width=128)
+    try:
+        assert tile(4096, 4096, 3136, 100) == (128, 25) and tile(4096, 4096, 100, 100) == (128, 1)
+    finally:
+        dl.set_tuning()
+
+
 def test_column_tiles_narrow_with_the_height_of_the_dense_operand(dl):
     """Dense rows wider than 512 floats are covered by several column tiles, worked through one after the other: the
     widest tile whose K x tile slab of B fits 4 MiB."""
     nnz = 4096 * 100
     for K, tile in ((512, 512), (2048, 512), (2049, 256), (4096, 256), (4097, 128), (8193, 64), (1 << 16, 32)):
-        sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz)
+        dl.set_tuning(rules_off=dl.RULES["finer_column_tiles"])
+        try:
+            sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz)
+        finally:
+            dl.set_tuning()
         assert sh["G"] * sh["vec"] * sh["V"] == tile and sh["col_tiles"] == -(-3136 // tile), (K, sh)
+        # a call without memory takes tiles of 64 at most (N above 512): long rows spread over more workgroups
+        sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz)
+        assert sh["G"] * sh["vec"] * sh["V"] == min(tile, 64) and sh["col_tiles"] == -(-3136 // min(tile, 64)), (K, sh)
         sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz, with_workspace=True)
         assert sh["G"] * sh["vec"] * sh["V"] == (max(tile, 128) if K * 128 * 4 <= (8 << 20) else 512)
     # ... with memory and rows long enough for the column-sliced schedule (64 nonzeros per row, half a million in

@@ -445,6 +445,43 @@ def test_column_sliced_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
+@pytest.mark.parametrize("M,K,N,per_row,tile,tiles", [
+    (128, 1152, 256, 200, 64, 4), (64, 576, 512, 100, 64, 8), (16, 576, 500, 100, 32, 16), (128, 1152, 196, 200, 128, 2),
+    (5, 300, 50, 40, 32, 2), (1000, 512, 784, 100, 256, 4), (300, 1152, 3140, 100, 64, 50), (130, 2304, 1030, 60, 256, 5)])
+@pytest.mark.parametrize("sigma", [0.0, 0.8])
+def test_finer_column_tiles_of_plain_spmm_calls(torch_cuda, dl, oracle, M, K, N, per_row, tile, tiles, sigma):
+    """The column tiles a SpMM call without memory takes for few rows and for wide dense rows (row-major tiles of
+    32 ... 256 columns, tile-major tiles of 64 where B exceeds the L2; last tiles of 4, 5 and 6 columns among them):
+    NULL and the even-rows hint against the oracle, and against the same call with the rule switched off."""
+    torch = torch_cuda
+    if sigma == 0.0:
+        ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 171, M, K, per_row / K)
+    else:
+        ro, ci = dl.make_pattern(dl.PATTERN_LOGNORMAL_ROWS, 172, M, K, float(per_row), sigma)
+    nnz = ci.size
+    va = dl.fill("uniform", 173, (nnz,), -1.0, 1.0)
+    B = dl.fill("uniform", 174, (K, N), -1.0, 1.0)
+    ro_d, ci_d, va_d, B_d = (dev(torch, x) for x in (ro, ci, va, B))
+    sh = dl.describe_launch(dl.OP_SPMM, M, K, N, nnz)
+    if nnz >= 16 * M:
+        assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (tile, tiles)
+    ref = oracle.spmm(ro, ci, va, B, omp=True)
+    out = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    dl.spmm(ro_d, ci_d, va_d, B_d, K=K, out=out)
+    assert oracle.rel_frobenius(out.cpu().numpy(), ref) <= TOL
+    out.fill_(float("nan"))
+    dl.spmm(ro_d, ci_d, va_d, B_d, K=K, out=out, workspace=dl.ROWS_EVEN)
+    assert oracle.rel_frobenius(out.cpu().numpy(), ref) <= TOL
+    dl.set_tuning(rules_off=dl.RULES["finer_column_tiles"])
+    try:
+        assert dl.describe_launch(dl.OP_SPMM, M, K, N, nnz)["col_tiles"] < tiles
+        off = dl.spmm(ro_d, ci_d, va_d, B_d, K=K)
+    finally:
+        dl.set_tuning()
+    assert oracle.rel_frobenius(off.cpu().numpy(), ref) <= TOL
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
 @pytest.mark.parametrize("sigma", [0.0, 1.0])
 def test_sliced_column_tiles_on_a_tall_wide_dense_operand(torch_cuda, dl, oracle, sigma):
     """B of 24576 x 392 floats (37 MiB; not even a tile of 128 columns fits twice the L2) under rows of ~130 nonzeros:
@@ -562,7 +599,7 @@ def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle):
             assert (lens[2048:][:-1] >= lens[2048:][1:]).all()                   # after the resident part: descending
         sh = dl.describe_launch(dl.OP_SPMM, M, K, N, ci.size)
         want = dl.spmm(ro_d, ci_d, va_d, B_d, K=K).clone()
-        dl.set_tuning(split=(4, 1))
+        dl.set_tuning(split=(4, 1), rules_off=dl.RULES["finer_column_tiles"])   # (a planned launch takes the column tiles of the other calls)
         want_one_row = dl.spmm(ro_d, ci_d, va_d, B_d, K=K).clone()
         dl.set_tuning()
         got = torch.full((M, N), float("nan"), device="cuda")
