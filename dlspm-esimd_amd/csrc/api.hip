@@ -416,7 +416,7 @@ int dlspm_set_tuning(const dlspm_tuning* t)
         t->tile_major < -1 || t->tile_major > 1 || t->tile_width < 0 || t->plan_order < 0 || t->plan_order > 2 ||
         t->xcd_contiguous < 0 || t->xcd_contiguous > 1 || t->stream_results < -1 || t->stream_results > 1 ||
         (t->cut_piece_pct != 0 && (t->cut_piece_pct < 10 || t->cut_piece_pct > 1000)) ||
-        (t->cut_longest_pct != 0 && (t->cut_longest_pct < 10 || t->cut_longest_pct > 1000)) || t->rules_off < 0 || t->rules_off > 511 ||
+        (t->cut_longest_pct != 0 && (t->cut_longest_pct < 10 || t->cut_longest_pct > 1000)) || t->rules_off < 0 || t->rules_off > 1023 ||
         (t->compute_units != 0 && (t->compute_units < 8 || t->compute_units > 1024 || t->compute_units % 8 != 0)))
         return DLSPM_E_INVALID_ARG;
     t_tuning.split_w = t->split_w;
@@ -600,8 +600,9 @@ int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_
 // entry is longer than one and a half shares. What that saves is set against what the cut plan costs: where the pieces
 // leave partial rows (the fused op; SpMM outside 33 ... 512 columns) the second kernel that adds them (about 2 us between
 // two graph nodes), else (SDDMM; SpMM where the pieces share the row's columns) only a grid that is two entries per
-// compute unit larger.
-static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int nnz, int max_row_len, bool second_kernel)
+// compute unit larger. `spread`: the workgroups over which a call without plan spreads every row by itself (few rows: SpMM's
+// column tiles, SDDMM's row pieces); the longest row then keeps one compute unit busy for that fraction of its length only.
+static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int nnz, int max_row_len, bool second_kernel, int spread = 1)
 {
     if (max_row_len <= 0 || M > kCutPlanAdviceMaxRows) return false;
     const long long cus = dev.cus;
@@ -611,9 +612,10 @@ static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int n
     if (second_kernel && M < 2 * cus) return false;
     const long long share = std::max<long long>(ceil_div(nnz, cus), 1);
     const long long longest_whole = (share * kCutAdvicePct + 99) / 100;
-    if (max_row_len <= longest_whole) return false;
+    const long long longest_unit = ceil_div(max_row_len, std::max(spread, 1));
+    if (longest_unit <= longest_whole) return false;
     const double bytes_per_nonzero = (op == DLSPM_OP_FUSED ? 2.0 : 1.0) * (double)std::min(width, 512) * sizeof(float);
-    const double saved_ns = (double)(max_row_len - longest_whole) * bytes_per_nonzero / 115.0;
+    const double saved_ns = (double)(longest_unit - longest_whole) * bytes_per_nonzero / 115.0;
     if (second_kernel) return saved_ns >= kCutPlanMinGainNs;
     // (SpMM, N = 256, the 302 files of the reference's data set with a row above one and a half shares, against the better
     // of NULL and the plan over whole rows: 0.99 of the time below 300 ns by this model, 0.96 / 0.91 / 0.84 / 0.81 from 300 /
@@ -634,16 +636,25 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
     if (M <= 0 || K <= 0 || N_or_D <= 0 || nnz <= 0) return 0;
     const bool vec4 = N_or_D >= 4;
     bool second_kernel = op == DLSPM_OP_FUSED;  // a cut plan's pieces leave partial rows for a second kernel to add
+    int spread = 1;  // workgroups over which a call without plan spreads each row by itself
     if (op == DLSPM_OP_SPMM) {
         SpmmShape shape = spmm_choose(dev, M, K, N_or_D, nnz, vec4, false, true);
         if (!spmm_plan_applies(dev, shape, M, N_or_D, nnz)) return 0;
         second_kernel = !spmm_cut_by_columns(shape, N_or_D);
+        // few rows: a call without plan works in narrower column tiles than a planned launch does
+        const SpmmShape plain = spmm_choose(dev, M, K, N_or_D, nnz, vec4, false, true, false, true);
+        const long long tiles = ceil_div(N_or_D, shape.G * shape.vec * shape.V), tiles_plain = ceil_div(N_or_D, plain.G * plain.vec * plain.V);
+        if (!plain.tile_major && tiles_plain > tiles) spread = (int)(tiles_plain / tiles);
     } else if (op == DLSPM_OP_SDDMM) {
         SddmmShape shape = sddmm_choose(dev, M, N_or_D, nnz, vec4);
         if (!sddmm_plan_applies(dev, shape, M, N_or_D, nnz, rows_are_skewed(M, nnz, max_row_len))) {
             // fewer rows than compute units: only a cut plan helps (its pieces fill the device)
-            SddmmShape few = sddmm_choose(dev, M, N_or_D, nnz, vec4);
-            return sddmm_cut_plan_applies(dev, few, M, N_or_D, nnz) && cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len, false) ? 2 : 0;
+            SddmmShape few = sddmm_choose(dev, M, N_or_D, nnz, vec4), plain = few;
+            sddmm_few_rows_pieces(dev, plain, M, nnz);  // what a call without plan does by itself
+            return sddmm_cut_plan_applies(dev, few, M, N_or_D, nnz) &&
+                           cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len, false, 1 << plain.pieces_lg)
+                       ? 2
+                       : 0;
         }
     } else if (op == DLSPM_OP_FUSED) {
         FusedShape shape = fused_choose(dev, M, N_or_D, nnz, vec4);
@@ -665,7 +676,8 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
     int slices = 0;
     (void)dlspm_describe_slices(op, M, K, N_or_D, nnz, &slices, nullptr);
     if (slices >= 3) return 0;
-    return cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len, second_kernel) ? 2 : 1;
+    if (cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len, second_kernel, spread)) return 2;
+    return spread > 1 ? 0 : 1;  // (a plan over whole rows would undo the spread)
 }
 
 int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const int* col_indices, const float* lhs,
@@ -722,7 +734,9 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
     // (rows known to be even have nothing to gain from the flat schedule, which costs them 4 ... 12 % today: the reference's
     // grid at density 0.1, 12288 ... 32768 rows of 410 ... 819 nonzeros, D = 32 and 128)
     const FlatPlan plan = ws.banded || ws.rows_even ? FlatPlan{0, 0, 0} : sddmm_flat_plan(dev, M, nnz, D);
-    const hipError_t e = plan.chunk > 0 ? sddmm_flat_launch(args, shape, plan.chunk, st) : sddmm_launch(args, shape, st);
+    SddmmShape plain = shape;
+    if (plan.chunk == 0) sddmm_few_rows_pieces(dev, plain, M, nnz);
+    const hipError_t e = plan.chunk > 0 ? sddmm_flat_launch(args, shape, plan.chunk, st) : sddmm_launch(args, plain, st);
     return e == hipSuccess ? DLSPM_OK : fail_hip(e);
 }
 
@@ -871,9 +885,11 @@ int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int pa
         const FlatPlan fp = flat_plan(dev, M, nnz, n, s.G);
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_SDDMM) {
-        const SddmmShape s = sddmm_choose(dev, M, n, nnz, vec4, even);
-        shape[0] = s.vec; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R; shape[7] = 1;
+        SddmmShape s = sddmm_choose(dev, M, n, nnz, vec4, even);
         const FlatPlan fp = even ? FlatPlan{0, 0, 0} : sddmm_flat_plan(dev, M, nnz, n);  // as sddmm_csr_f32 decides
+        if (!memory && fp.chunk == 0) sddmm_few_rows_pieces(dev, s, M, nnz);
+        // ([7]: the workgroups that share a row -- SDDMM has no column tiles)
+        shape[0] = s.vec; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R; shape[7] = 1 << s.pieces_lg;
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_FUSED) {
         const FusedShape s = fused_choose(dev, M, n, nnz, vec4, even, K);

@@ -99,7 +99,7 @@ struct Tuning {
 // (the values of DLSPM_RULE_* in the header)
 constexpr int kRuleEightWavesFewRows = 1, kRuleSixteenWavesTallLongRows = 2, kRuleMoreWavesFewLongRows = 4, kRuleGroupRows = 8,
               kRuleRowAlignedSplit = 16, kRulePlanUngroups = 32, kRuleExactWidthKernels = 64, kRuleCutRowsByColumns = 128,
-              kRuleFinerColumnTiles = 256;
+              kRuleFinerColumnTiles = 256, kRuleRowPiecesFewRows = 512;
 
 const Tuning& tuning();
 inline bool rule_on(int rule) { return (tuning().rules_off & rule) == 0; }
@@ -110,7 +110,7 @@ inline bool rule_on(int rule) { return (tuning().rules_off & rule) == 0; }
 // bit 3 = never take the row-aligned split (DLSPM_RULE_ROW_ALIGNED_SPLIT switched off); bit 4 (SDDMM, one row per
 // workgroup) = the waves of a row take whole passes of 64 nonzeros in turn (sddmm_row_interleaved).
 constexpr int kFlagXcdContiguous = 1, kFlagStreamShift = 1, kFlagStreamNever = 1, kFlagStreamAlways = 2, kFlagNoAlignedSplit = 8,
-              kFlagFullPasses = 16;
+              kFlagFullPasses = 16, kFlagPiecesShift = 8, kFlagPiecesMask = 7;  // (bits 8-10: log2 of the workgroups that share a row, SDDMM)
 inline int launch_flags(int xcd_contiguous_hint)
 {
     const Tuning& t = tuning();
@@ -126,7 +126,7 @@ inline int launch_flags(int xcd_contiguous_hint)
 //         product (0 = run-time loop, lhs row re-read instead of kept in registers)
 //   W   : waves per workgroup                                           R  : consecutive rows per workgroup
 struct SpmmShape { int vec, G, V, W, R, tile_major; };  // tile_major: column tiles one after the other (else row blocks)
-struct SddmmShape { int vec, G1, DS, W, R; };
+struct SddmmShape { int vec, G1, DS, W, R, pieces_lg; };  // pieces_lg: 2^pieces_lg workgroups share each row (sddmm_few_rows_pieces)
 struct FusedShape { int vec, G1, DS, G, V, W, R; };
 
 struct SpmmArgs {
@@ -212,6 +212,7 @@ hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const Slice
                               hipStream_t stream);
 
 SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even = false);
+void sddmm_few_rows_pieces(const DeviceInfo& dev, SddmmShape& s, int M, int nnz);  // a call without plan or memory: sets s.pieces_lg (and W = 4)
 hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t stream);
 hipError_t sddmm_flat_launch(const SddmmArgs& x, const SddmmShape& s, int chunk, hipStream_t stream);
 hipError_t sddmm_sliced_launch(const SddmmArgs& x, const SddmmShape& s, const SlicePlan& plan, void* workspace,

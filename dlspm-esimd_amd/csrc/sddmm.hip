@@ -83,8 +83,8 @@ __device__ __forceinline__ void sddmm_segment(int p, int q, int D, const int* __
 // Every result is one nonzero's own dot product, so which wave computes it changes no bit.
 // Measured (D = 128, in a graph, even split -> this): lognormal rows with a row plan, 2048 x 2048 8.6 -> 7.9 us, 16384 x 4096
 // 39.4 -> 32.9 us; 2048 x 512 with 51 per row 4.95 -> 4.16 us.
-template <int VEC, int G1, int DS, bool MASKED, int W>
-__device__ __forceinline__ void sddmm_row_interleaved(int p, int q, int w, int D, const int* __restrict__ col_indices,
+template <int VEC, int G1, int DS, bool MASKED>
+__device__ __forceinline__ void sddmm_row_interleaved(int p, int q, int w, int W, int D, const int* __restrict__ col_indices,
                                                       const float* __restrict__ lhs_row, const float* __restrict__ rhs,
                                                       SampledOut out, int lane, bool full_passes)
 {
@@ -129,12 +129,18 @@ __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __
                                             int flags = 0, const int* __restrict__ row_slots = nullptr, int slots = 0)
 {
     RowBlock<W, R, SLICED, PLANNED> blk;
-    blk.load(bid, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, lhs, rhs, out.at); }, flags,
+    const int lg = !SLICED && !PLANNED && R == 1 && W > 1 ? (flags >> kFlagPiecesShift) & kFlagPiecesMask : 0;
+    blk.load(bid >> lg, M, nnz, row_offsets, row_ends, row_ids, [&]() { fetch_args_now(col_indices, lhs, rhs, out.at); }, flags,
              row_slots, slots);
     if constexpr (R == 1 && W > 1) {
         const int first = blk.T0 + blk.shift(0);
-        sddmm_row_interleaved<VEC, G1, DS, MASKED, W>(first, first + blk.T, blk.w, D, col_indices, lhs + (size_t)blk.row0 * D, rhs,
-                                                      out, blk.lane, (flags & kFlagFullPasses) != 0);
+        int w = blk.w, waves = W;
+        if constexpr (!SLICED && !PLANNED) {  // 2^lg workgroups share the row: their waves take its passes in turn like one workgroup's
+            w += (bid & ((1 << lg) - 1)) * W;
+            waves = W << lg;
+        }
+        sddmm_row_interleaved<VEC, G1, DS, MASKED>(first, first + blk.T, w, waves, D, col_indices, lhs + (size_t)blk.row0 * D, rhs,
+                                                   out, blk.lane, (flags & kFlagFullPasses) != 0);
     } else {
         blk.for_each_segment([&](int r, int p, int q, int, int) {
             const float* lhs_row = lhs + (size_t)(blk.row0 + r) * D;
@@ -209,19 +215,22 @@ static int sddmm_flags(const SddmmArgs& x, long long entries)
 }
 
 template <int VEC, int G1, int DS, int W, int R>
-static hipError_t launch_one(const SddmmArgs& x, hipStream_t stream)
+static hipError_t launch_one(const SddmmArgs& x, int pieces_lg, hipStream_t stream)
 {
-    const int blocks = (int)ceil_div(x.M, R);
+    if (R != 1 || W == 1) pieces_lg = 0;
+    const int blocks = (int)ceil_div(x.M, R) << pieces_lg;
     if (blocks <= 0) return hipSuccess;
+    // (row pieces: the workgroups of a row must stay neighbours, so no XCD-contiguous runs of row blocks)
+    const int flags = pieces_lg > 0 ? (sddmm_flags(x, x.M) & ~kFlagXcdContiguous) | (pieces_lg << kFlagPiecesShift) : sddmm_flags(x, x.M);
     if constexpr (DS > 0) {
         if (x.D == G1 * VEC * DS && rule_on(kRuleExactWidthKernels)) {
             hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, false, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M,
-                               x.D, sddmm_flags(x, x.M), x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+                               x.D, flags, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
             return hipGetLastError();
         }
     }
     hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, true, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M, x.D,
-                       sddmm_flags(x, x.M), x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+                       flags, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     return hipGetLastError();
 }
 
@@ -249,13 +258,35 @@ SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
     return s;
 }
 
+// Few rows in a call without plan or memory: 2^lg four-wave workgroups share each row, so that the device gets two
+// workgroups per compute unit where one row per workgroup -- with eight waves -- leaves most of it idle. Their waves take the
+// row's passes in turn exactly as the waves of one workgroup do (sddmm_row_interleaved), every result is still one
+// nonzero's own dot product, and nothing else changes: no plan, no second kernel, the same bits. Up to three quarters of
+// a compute unit's count of rows, rows of 128 nonzeros and more on average, and a workgroup keeps at least 32 of a mean row.
+// Measured (us inside a graph, rule off / on / with a cut plan; Bernoulli rows, geometric means over five shapes of 300 ...
+// 1400 nonzeros per row): D = 128: 16 rows 3.75 / 2.59 / 2.62, 64 rows 3.84 / 3.01 / 3.04, 128 rows 3.90 / 3.53 / 3.53,
+// 192 rows 3.99 / 4.18 / 4.13; D = 256: 6.00 / 3.37 / 3.04, 7.13 / 4.00 / 4.41, 7.17 / 5.03 / 5.61, 7.18 / 6.12 / 7.37;
+// lognormal rows (sigma 0.8), D = 128: 6.03 / 2.81 / 2.64, 6.70 / 3.38 / 3.04, 6.74 / 4.47 / 3.58, 6.76 / 4.96 / 3.99
+// (a cut plan still cuts the longest rows finer); the reference's 128-row ResNet-50 layers (26 files): 3.80 / 3.28 / 3.31.
+void sddmm_few_rows_pieces(const DeviceInfo& dev, SddmmShape& s, int M, int nnz)
+{
+    s.pieces_lg = 0;
+    if (!rule_on(kRuleRowPiecesFewRows) || s.R != 1 || s.W == 1 || tuning().split_w > 0 || M <= 0) return;
+    if (4ll * M > 3ll * dev.cus || (long long)nnz < 128ll * M) return;
+    int lg = 0;
+    while (lg < kFlagPiecesMask && ((long long)M << lg) < 2ll * dev.cus && (long long)nnz >= (64ll << lg) * M) ++lg;
+    if (lg == 0) return;
+    s.pieces_lg = lg;
+    s.W = 4;
+}
+
 hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t stream)
 {
     return dispatch_layout(s, [&](auto l) {
         using L = decltype(l);
         return dispatch_split(s.W, s.R, [&](auto split) {
             using S = decltype(split);
-            return launch_one<L::VEC, L::G1, L::DS, S::W, S::R>(x, stream);
+            return launch_one<L::VEC, L::G1, L::DS, S::W, S::R>(x, s.pieces_lg, stream);
         });
     });
 }

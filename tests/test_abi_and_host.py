@@ -174,6 +174,29 @@ def test_finer_column_tiles_for_plain_spmm_calls(dl):
         dl.set_tuning()
 
 
+def test_row_pieces_for_plain_sddmm_calls_on_few_rows(dl):
+    """SDDMM without plan or memory on a mask of at most three quarters of the compute units' count of rows: 2^k four-wave
+    workgroups share each row, up to two workgroups per compute unit in all, each keeping 32 nonzeros of a mean row or
+    more; rows of 128 nonzeros and more on average only."""
+    pieces = lambda M, per_row, **kw: (lambda sh: (sh["W"], sh["col_tiles"]))(dl.describe_launch(dl.OP_SDDMM, M, 4608, 128, M * per_row, **kw))
+    assert pieces(128, 300) == (4, 4) and pieces(64, 300) == (4, 8) and pieces(32, 300) == (4, 8)   # (8: 37 per workgroup)
+    assert pieces(32, 600) == (4, 16) and pieces(1, 4608) == (4, 128) and pieces(192, 300) == (4, 4)
+    assert pieces(193, 300) == (8, 1)                      # more rows: eight waves per row as before
+    assert pieces(128, 127) == (8, 1) and pieces(128, 128) == (4, 4)
+    assert pieces(128, 300, rows_even=True) == (4, 4)      # the hint is about the lengths of the rows, not their number
+    assert pieces(128, 300, with_workspace=True) == (8, 1)
+    dl.set_tuning(rules_off=dl.RULES["row_pieces_few_rows"])
+    try:
+        assert pieces(128, 300) == (8, 1)
+    finally:
+        dl.set_tuning()
+    dl.set_tuning(split=(4, 1))                            # a forced split is taken as it is
+    try:
+        assert pieces(128, 300) == (4, 1)
+    finally:
+        dl.set_tuning()
+
+
 def test_column_tiles_narrow_with_the_height_of_the_dense_operand(dl):
     """Dense rows wider than 512 floats are covered by several column tiles, worked through one after the other: the
     widest tile whose K x tile slab of B fits 4 MiB."""

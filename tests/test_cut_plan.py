@@ -196,18 +196,22 @@ def test_cut_plan_sizes_and_advice(dl):
     assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 256, 52000, -1) == 1     # unknown rows: never a cut plan
     assert dl.row_plan_advice(dl.OP_SPMM, 2048, 512, 256, 105687, 312) == 1   # the headline matrix: below one share
     assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 256, 52000, 110) == 0    # even rows: no plan at all
-    # fewer rows than compute units (eight waves per row by the size rule): SDDMM takes a cut plan, whose pieces fill the
-    # device at no cost, and so does SpMM at widths where the pieces of a row share its columns (33 ... 512); the fused op and
-    # SpMM at the other widths, which would cut most rows and pay for adding the pieces, do not
-    assert dl.describe_launch(dl.OP_SDDMM, 128, 1152, 128, 29510)["W"] == 8
-    assert dl.row_plan_advice(dl.OP_SDDMM, 128, 1152, 128, 29510, 455) == 2
-    assert dl.row_plan_advice(dl.OP_SDDMM, 64, 576, 128, 31919, 547) == 2
+    # fewer rows than three quarters of the compute units: a call without plan spreads every row over several workgroups by
+    # itself (SDDMM: row pieces; SpMM: column tiles of B), so a cut plan is advised only where a row is still too long for
+    # one of them -- and never the plan over whole rows, which would undo the spread
+    sh = dl.describe_launch(dl.OP_SDDMM, 128, 1152, 128, 29510)
+    assert (sh["W"], sh["R"], sh["col_tiles"]) == (4, 1, 4)                    # ([7]: workgroups per row)
+    assert dl.row_plan_advice(dl.OP_SDDMM, 128, 1152, 128, 29510, 455) == 0    # a quarter of 455 is below one and a half shares (174)
+    assert dl.row_plan_advice(dl.OP_SDDMM, 128, 1152, 128, 29510, 1152) == 2
+    assert dl.row_plan_advice(dl.OP_SDDMM, 64, 576, 128, 31919, 547) == 0
     assert dl.row_plan_advice(dl.OP_SDDMM, 256, 2304, 128, 118041, 900) == 0   # 256 rows, longest below two shares: no
     assert dl.row_plan_advice(dl.OP_SDDMM, 256, 2304, 128, 53000, 800) == 2    # ... of nearly four shares: yes
-    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 256, 29510, 455) == 2
-    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 128, 29510, 455) == 2
-    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 64, 29510, 455) == 2
-    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 32, 29510, 455) in (0, 1)
+    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 256, 29510, 455) == 0
+    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 256, 29510, 1152) == 2
+    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 128, 29510, 455) == 0
+    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 64, 29510, 455) == 0
+    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 64, 29510, 1100) == 2
+    assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 32, 29510, 455) in (0, 1)  # (32 columns: nothing to tile)
     assert dl.row_plan_advice(dl.OP_SPMM, 512, 8192, 32, 52000, 3000) == 2     # (with partial rows: only from a large gain on
     assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 32, 52000, 700) == 1      # ... and two rows per compute unit)
     assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 256, 52000, 500) == 2

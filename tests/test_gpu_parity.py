@@ -482,6 +482,39 @@ def test_finer_column_tiles_of_plain_spmm_calls(torch_cuda, dl, oracle, M, K, N,
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
+@pytest.mark.parametrize("M,K,D,per_row,pieces", [
+    (128, 1152, 128, 230, 4), (16, 576, 64, 400, 8), (1, 700, 256, 700, 16), (64, 4608, 100, 1400, 8), (192, 2304, 32, 230, 4),
+    (7, 300, 16, 140, 4), (100, 512, 128, 60, 1), (193, 2304, 128, 230, 1)])
+@pytest.mark.parametrize("sigma", [0.0, 0.8])
+def test_row_pieces_of_plain_sddmm_calls_on_few_rows(torch_cuda, dl, oracle, M, K, D, per_row, pieces, sigma):
+    """Few rows: 2, 4, ... 16 workgroups share each row of a SDDMM call without plan or memory. Every result is still
+    one nonzero's own dot product: the bits of the same call with the rule switched off, and the oracle's values."""
+    torch = torch_cuda
+    if sigma == 0.0:
+        ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 181, M, K, per_row / K)
+    else:
+        ro, ci = dl.make_pattern(dl.PATTERN_LOGNORMAL_ROWS, 182, M, K, float(per_row), sigma)
+    nnz = ci.size
+    lhs = dl.fill("normal", 183, (M, D), 0.0, 1.0)
+    rhs = dl.fill("normal", 184, (K, D), 0.0, 1.0)
+    ro_d, ci_d, lhs_d, rhs_d = (dev(torch, x) for x in (ro, ci, lhs, rhs))
+    sh = dl.describe_launch(dl.OP_SDDMM, M, K, D, nnz)
+    if sigma == 0.0:
+        assert sh["col_tiles"] == pieces and (pieces == 1 or (sh["W"], sh["R"]) == (4, 1))
+    out = torch.full((nnz,), float("nan"), dtype=torch.float32, device="cuda")
+    dl.sddmm(ro_d, ci_d, lhs_d, rhs_d, out=out)
+    assert oracle.rel_frobenius(out.cpu().numpy(), oracle.sddmm(ro, ci, lhs, rhs, omp=True)) <= TOL
+    even = dl.sddmm(ro_d, ci_d, lhs_d, rhs_d, workspace=dl.ROWS_EVEN)
+    dl.set_tuning(rules_off=dl.RULES["row_pieces_few_rows"])
+    try:
+        assert dl.describe_launch(dl.OP_SDDMM, M, K, D, nnz)["col_tiles"] == 1
+        off = dl.sddmm(ro_d, ci_d, lhs_d, rhs_d)
+    finally:
+        dl.set_tuning()
+    assert torch.equal(out, off) and torch.equal(even, off)
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
 @pytest.mark.parametrize("sigma", [0.0, 1.0])
 def test_sliced_column_tiles_on_a_tall_wide_dense_operand(torch_cuda, dl, oracle, sigma):
     """B of 24576 x 392 floats (37 MiB; not even a tile of 128 columns fits twice the L2) under rows of ~130 nonzeros:
@@ -601,10 +634,13 @@ def test_row_plan_changes_the_order_of_the_rows_only(torch_cuda, dl, oracle):
         want = dl.spmm(ro_d, ci_d, va_d, B_d, K=K).clone()
         dl.set_tuning(split=(4, 1), rules_off=dl.RULES["finer_column_tiles"])   # (a planned launch takes the column tiles of the other calls)
         want_one_row = dl.spmm(ro_d, ci_d, va_d, B_d, K=K).clone()
+        dl.set_tuning(rules_off=dl.RULES["finer_column_tiles"])
+        # rows unknown: 1 exactly where the planned kernel runs (with the rule on, few rows are advised against a plan that would run)
+        planned_runs = dl.row_plan_advice(dl.OP_SPMM, M, K, N, ci.size, -1)
         dl.set_tuning()
         got = torch.full((M, N), float("nan"), device="cuda")
         dl.spmm(ro_d, ci_d, va_d, B_d, K=K, out=got, plan=plan)
-        if dl.row_plan_advice(dl.OP_SPMM, M, K, N, ci.size, -1):   # rows unknown: 1 exactly where the planned kernel runs
+        if planned_runs:
             assert torch.equal(got, want_one_row), (kind, shape)
             used += 1
             tiled += int(sh["col_tiles"] > 1)
