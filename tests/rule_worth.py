@@ -57,6 +57,9 @@ def cases(dl, quick):
     for (M, K, mean) in ((64, 576, 400.0), (128, 1152, 200.0), (256, 2304, 200.0), (512, 512, 50.0), (512, 2048, 100.0)):
         ro, ci = dl.make_pattern(dl.PATTERN_LOGNORMAL_ROWS, 9, M, K, mean, 0.5)
         out.append((f"layer {M}x{K} mean {mean:.0f} sigma 0.5 width 256/128/64", None, M, K, -1, ro, ci))
+    for (M, K, density) in ((16, 1152, 0.25), (64, 4608, 0.3), (128, 1152, 0.25)):
+        ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 12, M, K, density)
+        out.append((f"few rows {M}x{K} density {density} width 256/128/64", None, M, K, -1, ro, ci))
     for (M, K, mean, width) in ((128, 1152, 120.0, 784), (300, 1152, 115.0, 3136), (1000, 2048, 200.0, 640)):
         ro, ci = dl.make_pattern(dl.PATTERN_LOGNORMAL_ROWS, 10, M, K, mean, 0.5)
         out.append((f"wide dense rows {M}x{K} mean {mean:.0f} sigma 0.5 width {width}", dl.OP_SPMM, M, K, width, ro, ci))
