@@ -317,6 +317,7 @@ void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, co
 constexpr int kCutPlanAdviceMaxRows = 16384;     // the cut rule is one workgroup's work: 16 rounds of 1024 rows
 constexpr double kCutPlanMinGainNs = 2500.0;      // fused, SpMM with partial rows: the kernel that adds the pieces must be paid for
 constexpr double kCutPlanMinGainNsOneKernel = 300.0;  // SDDMM, and SpMM where the pieces share the columns: no second kernel
+constexpr int kCutPlanMinNnzSpmm = 5000;            // SpMM: no cut plan for fewer nonzeros
 constexpr double kCutPlanMinGainNsSddmmOneRowEach = 1000.0;  // ... one to two rows per compute unit: eight waves per row do nearly as well
 
 // longest row and number of rows without nonzeros (dlspm_csr_row_stats); stats[0] = max, stats[1] = empty rows
@@ -610,6 +611,10 @@ static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int n
     // shares are the exception and the kernel that adds their pieces has little to do (the reference's layers of 64 ...
     // 256 rows, where most rows would be cut: 0.85 ... 1.5 times the time of the plan over whole rows; 512 rows: 0.66 ... 1.0)
     if (second_kernel && M < 2 * cus) return false;
+    // SpMM on a handful of nonzeros is all start-up, and the cut plan's larger grid adds to it (the reference's data set at
+    // N = 256, cut plan / NULL: 1.10 below 2500 nonzeros (21 files), 1.00 below 5000 (23), 0.92 below 10 000 (49); SDDMM gains
+    // at every size: 0.89 / 0.91 / 0.88)
+    if (op == DLSPM_OP_SPMM && nnz < kCutPlanMinNnzSpmm) return false;
     const long long share = std::max<long long>(ceil_div(nnz, cus), 1);
     const long long longest_whole = (share * kCutAdvicePct + 99) / 100;
     const long long longest_unit = ceil_div(max_row_len, std::max(spread, 1));
