@@ -229,6 +229,8 @@ static bool looks_banded(const DeviceInfo& dev, int op, int width, const dlspm_m
            operand_bytes > (double)dev.l2_bytes;
 }
 
+constexpr int kClusteredEighthPermille = 1600;  // (1000: every eighth of the rows holds an eighth of the nonzeros)
+
 int dlspm_advise(int op, int N_or_D, const dlspm_matrix_info* info, dlspm_call_plan* plan)
 {
     if (!info || !plan || N_or_D < 0) return DLSPM_E_INVALID_ARG;
@@ -263,6 +265,10 @@ int dlspm_advise(int op, int N_or_D, const dlspm_matrix_info* info, dlspm_call_p
     const int passing = dlspm_workspace_advice(op, M, K, N_or_D, nnz, longest);
     if (passing == DLSPM_PASS_WORKSPACE) plan->bytes = dlspm_workspace_bytes(op, M, K, N_or_D, nnz);
     else if (passing == DLSPM_PASS_ROWS_EVEN) plan->hints = DLSPM_HINT_ROWS_EVEN;
+    // long rows that lie next to each other (one eighth of the rows holds 1.6 times its share, the longest row eight
+    // times the mean): the word that keeps the size rule from putting sixteen of them into one workgroup
+    else if (passing == DLSPM_PASS_NULL && info->eighths_nnz_permille >= kClusteredEighthPermille && (double)longest * M >= 8.0 * (double)nnz)
+        plan->hints = DLSPM_HINT_ROWS_SKEWED;
     return DLSPM_OK;
 }
 

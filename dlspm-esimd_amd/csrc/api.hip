@@ -255,8 +255,9 @@ SlicePlan slice_plan(const DeviceInfo& dev, int M, int K, int width, int nnz, in
     return p;
 }
 
-void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, const SplitRule& rule, bool rows_even, int& W, int& R)
+void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, const SplitRule& rule, int rows, int& W, int& R)
 {
+    const bool rows_even = rows == kRowsEven;
     if (tuning().split_w > 0 && split_is_built(tuning().split_w, tuning().split_r, rule.max_w)) {  // (else: ignored)
         W = tuning().split_w;
         R = tuning().split_r;
@@ -311,6 +312,13 @@ void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, co
         // operand takes a whole wave (from 256 columns on; rule.even_rows_avg): there the grouping pays from about a
         // hundred nonzeros per row (2048 x 512 with 102 per row: N = 392 14.9 -> 14.5 us, N = 256 9.7 -> 8.9 us).
         if (rows_even && R < 4 && avg >= rule.even_rows_avg && ceil_div(M, 4) * col_tiles >= 2 * cus) R = 4;
+        // Long rows known to lie next to each other (DLSPM_HINT_ROWS_SKEWED without a plan: dlspm_advise gives it where one
+        // eighth of the rows holds 1.6 times its share of the nonzeros): a workgroup of sixteen such rows has sixteen mean
+        // workgroups' work and four waves to do it with. Four rows at most, eight in the fused op (the reference's 33288 x 512
+        // embedding, 17.6 nonzeros per row, a run of rows of 300 at its start: SpMM N = 256 57.2 -> 27.8 us, SDDMM D = 128
+        // 35.5 -> 22.0 us, fused D = 64 34.8 -> 27.5 us with eight and 31.7 with four; with lengths independent of the position, sixteen rows lose nothing to four rows even at
+        // sigma 1.2, and short even rows need the sixteen: 65536 rows of 8, fused 30.8 against 44.5 us).
+        if (rows == kRowsSkewed && R > rule.skewed_rows_cap) R = rule.skewed_rows_cap;
     }
 }
 
@@ -492,7 +500,7 @@ int spmm_csr_f32(int M, int K, int N, int nnz, const int* row_offsets, const int
     // a banded matrix (DLSPM_HINT_BANDED) runs as row blocks whatever memory came with the call: column slices and
     // the flat schedule are answers to columns spread over all of K and to uneven rows
     const bool memory = !ws.rows_even && !ws.banded && ws.mem != nullptr;
-    const SpmmShape shape = spmm_choose(dev, M, K, N, nnz, vec4, ws.rows_even, !memory, ws.banded, !memory);
+    const SpmmShape shape = spmm_choose(dev, M, K, N, nnz, vec4, ws.rows_even ? kRowsEven : ws.skewed ? kRowsSkewed : kRowsUnknown, !memory, ws.banded, !memory);
     if (memory) {
         const SlicePlan sliced = spmm_slice_plan(dev, M, K, N, nnz, shape);
         const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(dev, M, nnz, N, shape.G);
@@ -724,7 +732,7 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
         }
         // sizes a planned launch is not built for run as with NULL
     }
-    const SddmmShape shape = sddmm_choose(dev, M, D, nnz, vec4, ws.rows_even);
+    const SddmmShape shape = sddmm_choose(dev, M, D, nnz, vec4, ws.rows_even ? kRowsEven : ws.skewed ? kRowsSkewed : kRowsUnknown);
     // the flat schedule needs no workspace here (nothing to combine), so the size rule alone decides; it has no
     // width condition for SDDMM (measured for D = 32 ... 256: equal on uniform rows, 15-33 % faster on skewed ones)
     if (ws.mem && !ws.rows_even && !ws.row_plan && !ws.cut_plan && !ws.banded) {
@@ -776,7 +784,7 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz, const int* row_offsets, c
                                                  : fused_launch(args, shape, st);
         return e == hipSuccess ? DLSPM_OK : fail_hip(e);
     }
-    const FusedShape shape = fused_choose(dev, M, D, nnz, vec4, ws.rows_even, K);
+    const FusedShape shape = fused_choose(dev, M, D, nnz, vec4, ws.rows_even ? kRowsEven : ws.skewed ? kRowsSkewed : kRowsUnknown, K);
     if (!ws.rows_even && !ws.banded && ws.mem) {
         const SlicePlan sliced = fused_slice_plan(dev, M, K, D, nnz, shape);
         const FlatPlan plan = sliced.slices > 0 ? FlatPlan{0, 0, 0} : flat_plan(dev, M, nnz, D, shape.G);
@@ -875,29 +883,30 @@ int dlspm_csr_row_stats(int M, const int* row_offsets, void* stream, int* max_ro
 int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int passing, int* shape)
 {
     const DeviceInfo& dev = device_info();
-    if (passing != DLSPM_PASS_NULL && passing != DLSPM_PASS_ROWS_EVEN && passing != DLSPM_PASS_WORKSPACE)
+    if (passing != DLSPM_PASS_NULL && passing != DLSPM_PASS_ROWS_EVEN && passing != DLSPM_PASS_WORKSPACE && passing != DLSPM_PASS_ROWS_SKEWED)
         return DLSPM_E_INVALID_ARG;
     const bool even = passing == DLSPM_PASS_ROWS_EVEN;
+    const int rows = even ? kRowsEven : passing == DLSPM_PASS_ROWS_SKEWED ? kRowsSkewed : kRowsUnknown;
     const bool memory = passing == DLSPM_PASS_WORKSPACE;
     if (!shape || M < 0 || N_or_D < 0 || nnz < 0) return DLSPM_E_INVALID_ARG;
     const int n = N_or_D;
     const bool vec4 = n >= 4;
     for (int i = 0; i < 10; ++i) shape[i] = 0;
     if (op == DLSPM_OP_SPMM) {
-        const SpmmShape s = spmm_choose(dev, M, K, n, nnz, vec4, even, !memory, false, !memory);
+        const SpmmShape s = spmm_choose(dev, M, K, n, nnz, vec4, rows, !memory, false, !memory);
         const int tw = s.G * s.vec * s.V;
         shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[5] = s.W; shape[6] = s.R; shape[7] = (int)ceil_div(n, tw);
         const FlatPlan fp = flat_plan(dev, M, nnz, n, s.G);
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_SDDMM) {
-        SddmmShape s = sddmm_choose(dev, M, n, nnz, vec4, even);
+        SddmmShape s = sddmm_choose(dev, M, n, nnz, vec4, rows);
         const FlatPlan fp = even ? FlatPlan{0, 0, 0} : sddmm_flat_plan(dev, M, nnz, n);  // as sddmm_csr_f32 decides
         if (!memory && fp.chunk == 0) sddmm_few_rows_pieces(dev, s, M, nnz);
         // ([7]: the workgroups that share a row -- SDDMM has no column tiles)
         shape[0] = s.vec; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R; shape[7] = 1 << s.pieces_lg;
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_FUSED) {
-        const FusedShape s = fused_choose(dev, M, n, nnz, vec4, even, K);
+        const FusedShape s = fused_choose(dev, M, n, nnz, vec4, rows, K);
         const int tw = s.G * s.vec * s.V;
         shape[0] = s.vec; shape[1] = s.G; shape[2] = s.V; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R;
         shape[7] = (int)ceil_div(n, tw);

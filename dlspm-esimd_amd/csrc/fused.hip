@@ -173,7 +173,7 @@ template <typename Launch> static hipError_t dispatch_layout(const FusedShape& s
 // the layouts the column-sliced and planned kernels are built for: 16 < D <= 512 in one column tile
 template <typename L> constexpr bool kOneTileLayout = L::VEC == 4 && L::G1 == 8 && L::DS >= 1;
 
-FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even, int K)
+FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, int rows, int K)
 {
     FusedShape s{};
     s.vec = vec4 ? 4 : 1;
@@ -201,7 +201,7 @@ FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
     // 486 -> 514, 545 -> 577 us), which is what a caller with such rows gets back several times over from a row plan or the
     // column slices. Within one L2 the same grouping gains 6 % on even rows and loses 7 % on uneven ones: only on the hint.
     const bool beyond_l2 = K > 0 && 2.0 * (double)K * (double)D * sizeof(float) > (double)dev.l2_bytes;
-    choose_split(dev, M, ceil_div(D, tw), nnz, SplitRule{3, tw >= 1024 ? 4 : 16, kWave / s.G, false, 96}, rows_even || beyond_l2, s.W,
+    choose_split(dev, M, ceil_div(D, tw), nnz, SplitRule{3, tw >= 1024 ? 4 : 16, kWave / s.G, false, 96, 128, 8}, rows == kRowsUnknown && beyond_l2 ? kRowsEven : rows, s.W,
                  s.R);
     return s;
 }

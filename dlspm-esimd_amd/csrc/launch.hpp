@@ -125,6 +125,9 @@ inline int launch_flags(int xcd_contiguous_hint)
 //   G1  : lanes covering one dot product (SDDMM / fused stage 1)        DS : accesses per lane per dot
 //         product (0 = run-time loop, lhs row re-read instead of kept in registers)
 //   W   : waves per workgroup                                           R  : consecutive rows per workgroup
+// what the caller said about the rows (`rows` of the *_choose functions): nothing, DLSPM_HINT_ROWS_EVEN, or DLSPM_HINT_ROWS_SKEWED
+// without a plan (long rows lie next to each other: fewer rows per workgroup)
+constexpr int kRowsUnknown = 0, kRowsEven = 1, kRowsSkewed = 2;
 struct SpmmShape { int vec, G, V, W, R, tile_major; };  // tile_major: column tiles one after the other (else row blocks)
 struct SddmmShape { int vec, G1, DS, W, R, pieces_lg; };  // pieces_lg: 2^pieces_lg workgroups share each row (sddmm_few_rows_pieces)
 struct FusedShape { int vec, G1, DS, G, V, W, R; };
@@ -195,7 +198,7 @@ hipError_t slice_bounds_launch(int M, int K, int slices, const int* row_offsets,
 hipError_t slice_sum_launch(long long count, int slices, const float* partial, float* out, hipStream_t stream);
 
 // narrow_tiles: the call passes no workspace memory (column tiles below 128 columns are then allowed)
-SpmmShape spmm_choose(const DeviceInfo& dev, int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles, bool banded = false,
+SpmmShape spmm_choose(const DeviceInfo& dev, int M, int K, int N, int nnz, bool vec4, int rows, bool narrow_tiles, bool banded = false,
                       bool plain = false);
 hipError_t spmm_launch(const SpmmArgs& x, const SpmmShape& s, hipStream_t stream);
 // Row plan (3 x M ints on the device: first nonzero, end and row number of the row that workgroup i works on): only for
@@ -211,7 +214,7 @@ hipError_t spmm_flat_launch(const SpmmArgs& x, const SpmmShape& s, const FlatPla
 hipError_t spmm_sliced_launch(const SpmmArgs& x, const SpmmShape& s, const SlicePlan& plan, void* workspace,
                               hipStream_t stream);
 
-SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even = false);
+SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, int rows = kRowsUnknown);
 void sddmm_few_rows_pieces(const DeviceInfo& dev, SddmmShape& s, int M, int nnz);  // a call without plan or memory: sets s.pieces_lg (and W = 4)
 hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t stream);
 hipError_t sddmm_flat_launch(const SddmmArgs& x, const SddmmShape& s, int chunk, hipStream_t stream);
@@ -219,7 +222,7 @@ hipError_t sddmm_sliced_launch(const SddmmArgs& x, const SddmmShape& s, const Sl
                                hipStream_t stream);
 
 // K > 0: the height of Kmat and V is known and may count (operands beyond one L2 group long rows as under the even-rows hint)
-FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even = false, int K = 0);
+FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, int rows = kRowsUnknown, int K = 0);
 hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t stream);
 hipError_t fused_flat_launch(const FusedArgs& x, const FusedShape& s, const FlatPlan& plan, float* partial,
                              hipStream_t stream);
@@ -237,8 +240,9 @@ struct SplitRule {
     bool more_waves_long_rows;
     int w8_few_rows_avg = 0;  // > 0: eight waves per row from this many nonzeros per row on where there are few rows
     int even_rows_avg = 128;  // rows known to be even are grouped four to a workgroup from this many nonzeros per row on
+    int skewed_rows_cap = 4;  // rows per workgroup at most where long rows are known to lie next to each other
 };
-void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, const SplitRule& rule, bool rows_even, int& W, int& R);
+void choose_split(const DeviceInfo& dev, int M, long long col_tiles, int nnz, const SplitRule& rule, int rows, int& W, int& R);
 
 // Row plan with cut rows ("cut plan"): rows longer than `longest_pct` per cent of a share (a share = the nonzeros of the
 // matrix over the compute units) are cut into pieces of at most `piece_pct` per cent of a share, and the plan hands out

@@ -240,7 +240,7 @@ template <typename Launch> static hipError_t dispatch_layout(const SddmmShape& s
     return dispatch<SddmmLayouts>([&](auto l) { return l.VEC == s.vec && l.G1 == s.G1 && l.DS == s.DS; }, launch);
 }
 
-SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, bool rows_even)
+SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4, int rows)
 {
     SddmmShape s{};
     s.vec = vec4 ? 4 : 1;
@@ -254,7 +254,7 @@ SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
         s.G1 = 4;
         s.DS = 1;
     }
-    choose_split(dev, M, 1, nnz, SplitRule{2, 16, kWave / s.G1, false, 96}, rows_even, s.W, s.R);
+    choose_split(dev, M, 1, nnz, SplitRule{2, 16, kWave / s.G1, false, 96}, rows, s.W, s.R);
     return s;
 }
 

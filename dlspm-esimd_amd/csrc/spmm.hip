@@ -334,7 +334,7 @@ static TileChoice spmm_tile_width(const DeviceInfo& dev, int M, int K, int N, in
 }
 
 // Chooses the lane layout from N (and the height of B) and the (W, R) split from the mean row length.
-SpmmShape spmm_choose(const DeviceInfo& dev, int M, int K, int N, int nnz, bool vec4, bool rows_even, bool narrow_tiles, bool banded,
+SpmmShape spmm_choose(const DeviceInfo& dev, int M, int K, int N, int nnz, bool vec4, int rows, bool narrow_tiles, bool banded,
                       bool plain)
 {
     SpmmShape s{};
@@ -359,7 +359,7 @@ SpmmShape spmm_choose(const DeviceInfo& dev, int M, int K, int N, int nnz, bool 
         s.V = 1;
     }
     const int tw = s.G * s.vec * s.V;
-    choose_split(dev, M, ceil_div(N, tw), nnz, SplitRule{8, 16, kWave / s.G, true, 0, s.G == kWave ? 96 : 128}, rows_even, s.W, s.R);
+    choose_split(dev, M, ceil_div(N, tw), nnz, SplitRule{8, 16, kWave / s.G, true, 0, s.G == kWave ? 96 : 128}, rows, s.W, s.R);
     return s;
 }
 

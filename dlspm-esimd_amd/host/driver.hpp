@@ -255,6 +255,7 @@ inline PreparedCall prepare_call(const Options& opt, int op, int M, int K, int w
                 : cp.bytes && slices > 0                    ? "dense operands beyond one L2, workspace passed (column-sliced schedule)"
                 : cp.bytes                                  ? "uneven, workspace passed (flat schedule)"
                 : (cp.hints & DLSPM_HINT_ROWS_EVEN)         ? "even, DLSPM_HINT_ROWS_EVEN passed"
+                : (cp.hints & DLSPM_HINT_ROWS_SKEWED)       ? "long rows next to each other, fewer rows per workgroup"
                                                             : "nothing passed",
                 (cp.hints & DLSPM_HINT_BANDED) && (cp.hints & DLSPM_HINT_ROWS_EVEN) ? " with DLSPM_HINT_ROWS_EVEN" : "",
                 (cp.hints & DLSPM_HINT_ROWS_SKEWED) ? " with DLSPM_HINT_ROWS_SKEWED" : "");

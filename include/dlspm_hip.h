@@ -53,6 +53,13 @@
  *         in column slices, 77 us with NULL, 74 us with this hint; the L2s fetch 33 MiB per launch instead of 145 MiB.
  *         A wrong hint costs time, never correctness: the bits are those of the call with NULL. May be combined with
  *         DLSPM_HINT_ROWS_EVEN; a row plan takes precedence. dlspm_advise detects bands from the matrix.
+ *       DLSPM_HINT_ROWS_SKEWED: with a row plan, the longest row is at least twenty times the mean (the planned SDDMM
+ *         and fused launches then run one row per workgroup at heights where they would keep rows grouped). With
+ *         workspace NULL: long rows lie next to each other in a tall matrix of short rows (an embedding whose frequent
+ *         tokens come first), and the launch groups at most four rows (fused: eight) into a workgroup instead of up to
+ *         sixteen -- 33288 x 512 with 17.6 nonzeros per row and a run of rows of 300: SpMM at N = 256 57 -> 28 us.
+ *         dlspm_advise gives it where one eighth of the rows holds 1.6 times its share of the nonzeros and the longest
+ *         row eight times the mean. Not together with DLSPM_HINT_ROWS_EVEN (DLSPM_E_INVALID_ARG). About speed only.
  * Calls on different streams may run concurrently from different host threads (each with its own
  * workspace). The library's only mutable state is per host thread (the tuning overrides of dlspm_set_tuning and the
  * last HIP error), a cache of the devices' properties, and the static scratch array of spmm_csr_f32_static.
@@ -189,7 +196,8 @@ int dlspm_csr_check(int M, int K, int nnz, const int* row_offsets, const int* co
  *                   pass NULL), what to build into it (`build`: nothing, dlspm_row_plan_build or
  *                   dlspm_row_plan_build_cut; nothing with bytes > 0: plain schedule memory, no initialisation), and
  *                   the hint bits to or into workspace_bytes (`hints`). A band is detected, not hinted; very uneven rows
- *                   in masks of 16 to 64 rows per compute unit get DLSPM_HINT_ROWS_SKEWED with their plan.
+ *                   in masks of 16 to 64 rows per compute unit get DLSPM_HINT_ROWS_SKEWED with their plan, and so do,
+ *                   without a plan, tall matrices of short rows whose long rows lie next to each other.
  * Use:  dlspm_matrix_info mi; dlspm_call_plan cp;
  *       dlspm_analyze(M, K, nnz, row_offsets, col_indices, stream, &mi);   dlspm_advise(DLSPM_OP_SPMM, N, &mi, &cp);
  *       void* ws = NULL; if (cp.bytes) hipMalloc(&ws, cp.bytes);
@@ -309,6 +317,7 @@ int dlspm_row_plan_build(int M, const int* row_offsets, void* plan, size_t plan_
 #define DLSPM_PASS_NULL       0
 #define DLSPM_PASS_ROWS_EVEN  1
 #define DLSPM_PASS_WORKSPACE  2
+#define DLSPM_PASS_ROWS_SKEWED 3  /* (dlspm_describe_launch_rows only: NULL with DLSPM_HINT_ROWS_SKEWED) */
 int dlspm_workspace_advice(int op, int M, int K, int N_or_D, int nnz, int max_row_len);
 
 /*

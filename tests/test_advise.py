@@ -57,7 +57,18 @@ def test_advise_branches(dl):
     cp = A(dl.OP_SPMM, 64, info(dl, 0, 0, 0, 0))
     assert (cp.build, cp.bytes, cp.hints) == (dl.BUILD_NOTHING, 0, 0)
     # arguments
+    # long rows next to each other in a tall matrix of short rows (one eighth of the rows holds 1.6 times its share, the
+    # longest row eight times the mean; too many rows and too short for a plan): the word that keeps the size rule from
+    # grouping sixteen rows into one workgroup
+    for op, width in ((dl.OP_SPMM, 256), (dl.OP_SDDMM, 128), (dl.OP_FUSED, 64)):
+        cp = A(op, width, info(dl, 33288, 512, 584680, 389, heaviest=2672))
+        assert (cp.build, cp.bytes, cp.hints) == (dl.BUILD_NOTHING, 0, dl.HINT_ROWS_SKEWED), (op, cp.build, cp.bytes, hex(cp.hints))
+        assert dl.describe_launch(op, 33288, 512, width, 584680)["R"] == 16
+        assert dl.describe_launch(op, 33288, 512, width, 584680, rows_skewed=True)["R"] == (8 if op == dl.OP_FUSED else 4)
+        assert not A(op, width, info(dl, 33288, 512, 584680, 389, heaviest=1500)).hints & dl.HINT_ROWS_SKEWED   # lengths independent of the position
+        assert not A(op, width, info(dl, 33288, 512, 584680, 100, heaviest=2672)).hints & dl.HINT_ROWS_SKEWED   # no row of eight times the mean
     L = dl.lib()
+    assert L.dlspm_describe_launch_rows(dl.OP_SPMM, 64, 64, 64, 64, 4, (ctypes.c_int * 10)()) == dl.E_INVALID_ARG
     mi, out = info(dl, 8, 8, 8, 1), dl.CallPlan()
     assert L.dlspm_advise(7, 64, ctypes.byref(mi), ctypes.byref(out)) == dl.E_INVALID_ARG
     assert L.dlspm_advise(dl.OP_SPMM, 64, None, ctypes.byref(out)) == dl.E_INVALID_ARG
@@ -201,6 +212,38 @@ def test_prepared_calls_follow_the_matrix(dl, oracle):
     # without the word the same plan is ignored at this height (the bits of the plain call)
     plain_plan = dl.row_plan(ro_d)
     assert torch.equal(dl.fused(ro_d, ci_d, Q_d, Km_d, V_d, 0.125, plan=plain_plan), dl.fused(ro_d, ci_d, Q_d, Km_d, V_d, 0.125))
+    # 3b. a tall matrix of short rows whose long rows lie next to each other (an embedding whose frequent tokens come
+    # first): no plan, no memory, DLSPM_HINT_ROWS_SKEWED -- four rows per workgroup instead of sixteen
+    M, K = 33288, 512
+    lens = rng.poisson(12, M)
+    lens[:1200] = rng.integers(150, 390, 1200)
+    lens = np.minimum(lens, K)
+    ro = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ci = np.concatenate([np.sort(rng.choice(K, n, replace=False)) for n in lens]).astype(np.int32)
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    mi = dl.analyze(ro_d, ci_d, K)
+    assert mi.eighths_nnz_permille >= 2000 and mi.max_row_len * M >= 8 * ci.size
+    va = rng.standard_normal(ci.size, dtype=np.float32)
+    for op, width in ((dl.OP_SPMM, 256), (dl.OP_SDDMM, 128), (dl.OP_FUSED, 64)):
+        prep = dl.prepare(ro_d, ci_d, K, op, width, info=mi)
+        assert prep.memory is None and prep.call_plan.hints == dl.HINT_ROWS_SKEWED
+        Q, Km, V = (rng.standard_normal(sh, dtype=np.float32) for sh in ((M, width), (K, width), (K, width)))
+        dl.set_tuning(split=(4, 8 if op == dl.OP_FUSED else 4))
+        if op == dl.OP_SPMM:
+            got, four = dl.spmm(ro_d, ci_d, dev(torch, va), dev(torch, Km), K=K, plan=prep), None
+            four = dl.spmm(ro_d, ci_d, dev(torch, va), dev(torch, Km), K=K)
+            want = oracle.spmm(ro, ci, va, Km, omp=True)
+        elif op == dl.OP_SDDMM:
+            got = dl.sddmm(ro_d, ci_d, dev(torch, Q), dev(torch, Km), plan=prep)
+            four = dl.sddmm(ro_d, ci_d, dev(torch, Q), dev(torch, Km))
+            want = oracle.sddmm(ro, ci, Q, Km, omp=True)
+        else:
+            got = dl.fused(ro_d, ci_d, dev(torch, Q), dev(torch, Km), dev(torch, V), 0.125, plan=prep)
+            four = dl.fused(ro_d, ci_d, dev(torch, Q), dev(torch, Km), dev(torch, V), 0.125)
+            want = oracle.fused(ro, ci, Q, Km, V, 0.125, omp=True)
+        dl.set_tuning()
+        assert torch.equal(got, four), op                     # the bits of four (fused: eight) rows per workgroup
+        assert oracle.rel_frobenius(got.cpu().numpy(), want) <= TOL
     # 4. even rows (the 1x1-convolution configuration): the even-rows hint, nothing to allocate
     c = dl.make_config(4)
     ro_d, ci_d = dev(torch, c["row_offsets"]), dev(torch, c["col_indices"])

@@ -58,7 +58,7 @@ def prepared_name(dl, prep):
         return "banded_hint"
     if cp.bytes:
         return "workspace"
-    return "rows_even_hint" if cp.hints & dl.HINT_ROWS_EVEN else "null"
+    return "rows_even_hint" if cp.hints & dl.HINT_ROWS_EVEN else "rows_skewed_hint" if cp.hints & dl.HINT_ROWS_SKEWED else "null"
 
 
 def schedules(dl, torch, op, M, K, N, nnz, ro_d, ci_d, every):
@@ -73,6 +73,7 @@ def schedules(dl, torch, op, M, K, N, nnz, ro_d, ci_d, every):
     if every:
         out.append(("null", None, None))
         out.append(("rows_even_hint", dl.ROWS_EVEN, None))
+        out.append(("rows_skewed_hint", dl.ROWS_SKEWED, None))
         if need:
             out.append(("workspace", memory(), None))
         if M > 0:
