@@ -27,6 +27,7 @@ int main()
         (void)dlspm_describe_launch(op, M, K, W, nnz, shape);
         (void)dlspm_describe_launch_rows(op, M, K, W, nnz, DLSPM_PASS_ROWS_EVEN, shape);
         (void)dlspm_describe_launch_rows(op, M, K, W, nnz, DLSPM_PASS_WORKSPACE, shape);
+        (void)dlspm_describe_launch_rows(op, M, K, W, nnz, DLSPM_PASS_ROWS_SKEWED, shape);
         volatile size_t pb = dlspm_row_plan_bytes(M);
         volatile size_t cb = dlspm_row_plan_bytes_for(op, M, W);
         // the one-look advice on a matrix description of these sizes (any figures: it must answer or refuse, never crash)
