@@ -422,7 +422,7 @@ int dlspm_set_tuning(const dlspm_tuning* t)
         return DLSPM_OK;
     }
     if (t->split_w < 0 || t->split_r < 0 || t->flat < -1 || t->flat > 1 || t->flat_chunk < 0 || t->slices < -1 ||
-        t->tile_major < -1 || t->tile_major > 1 || t->tile_width < 0 || t->plan_order < 0 || t->plan_order > 2 ||
+        t->tile_major < -1 || t->tile_major > 3 || t->tile_width < 0 || t->plan_order < 0 || t->plan_order > 2 ||
         t->xcd_contiguous < 0 || t->xcd_contiguous > 1 || t->stream_results < -1 || t->stream_results > 1 ||
         (t->cut_piece_pct != 0 && (t->cut_piece_pct < 10 || t->cut_piece_pct > 1000)) ||
         (t->cut_longest_pct != 0 && (t->cut_longest_pct < 10 || t->cut_longest_pct > 1000)) || t->rules_off < 0 || t->rules_off > 1023 ||

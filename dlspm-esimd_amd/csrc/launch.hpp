@@ -128,6 +128,7 @@ inline int launch_flags(int xcd_contiguous_hint)
 // what the caller said about the rows (`rows` of the *_choose functions): nothing, DLSPM_HINT_ROWS_EVEN, or DLSPM_HINT_ROWS_SKEWED
 // without a plan (long rows lie next to each other: fewer rows per workgroup)
 constexpr int kRowsUnknown = 0, kRowsEven = 1, kRowsSkewed = 2;
+constexpr int kTilesPerXcd = 2, kTilesPerXcdTileMajor = 3;  // SpmmShape::tile_major: 0 row-major, 1 tile-major, 2 / 3 each XCD on its own tiles (row- / tile-major within it)
 struct SpmmShape { int vec, G, V, W, R, tile_major; };  // tile_major: column tiles one after the other (else row blocks)
 struct SddmmShape { int vec, G1, DS, W, R, pieces_lg; };  // pieces_lg: 2^pieces_lg workgroups share each row (sddmm_few_rows_pieces)
 struct FusedShape { int vec, G1, DS, G, V, W, R; };

@@ -87,7 +87,37 @@ __device__ __forceinline__ void spmm_block(int bid, int M, int N, int col_tiles,
 {
     int ct = 0, rb = bid;
     if (col_tiles != 1) {
-        if (tile_major) {
+        if (tile_major >= kTilesPerXcd) {
+            // Each XCD works on its own run of column tiles (workgroup 8 j + x runs on XCD x, as the hardware deals them): the
+            // eight L2s then fetch B once between them, not once each. XCD x owns the q = T / 8 tiles from x q on; the T mod 8
+            // tiles left over come last and are shared by all XCDs like the tiles of the other orders, so every XCD gets
+            // the same number of workgroups. Inside an XCD's part (and in the shared part) the order is row-major or tile-major.
+            if constexpr (!PLANNED) row_blocks = (M - 1) / R + 1;
+            const int q = col_tiles >> 3, owned = 8 * q * row_blocks;
+            const bool tiles_first = tile_major == kTilesPerXcdTileMajor;
+            if (bid < owned) {
+                const int x = bid & 7, j = bid >> 3;
+                int local;
+                if (tiles_first) {
+                    local = j / row_blocks;
+                    rb = j - local * row_blocks;
+                } else {
+                    rb = j / q;
+                    local = j - rb * q;
+                }
+                ct = x * q + local;
+            } else {
+                const int rest = col_tiles - 8 * q, j = bid - owned;
+                if (tiles_first) {
+                    const int local = j / row_blocks;
+                    rb = j - local * row_blocks;
+                    ct = 8 * q + local;
+                } else {
+                    rb = j / rest;
+                    ct = 8 * q + j - rb * rest;
+                }
+            }
+        } else if (tile_major) {
             if constexpr (!PLANNED) row_blocks = (M - 1) / R + 1;  // (a plan has as many entries as its launch says)
             ct = bid / row_blocks;
             rb = bid - ct * row_blocks;
@@ -277,11 +307,16 @@ template <typename Launch> static hipError_t dispatch_layout(const SpmmShape& s,
 //  * N above 512 and up to eight rows per compute unit: row-major tiles of 256 instead of 512 (200 x 2304, N = 784:
 //    12.2 / 11.5 even, 42.1 / 19.7 lognormal; 1500 x 512, N = 600: 24.8 / 19.3 and 34.4 / 25.6; taller matrices lose:
 //    8192 x 512, N = 784: 57.4 / 62.0).
-//  * B beyond the L2 and N above 512: tile-major order from three pairs per compute unit on (instead of eight) for
-//    matrices of at least half a compute unit's count of rows, in tiles of 64: the finer the tile, the smaller the slab of B
-//    in use at a time and the more evenly long rows spread (256 x 2304, N = 3136: 86.8 / 39.8 even, 134 / 93 lognormal;
-//    1024 x 1152, N = 12544: 212 / 220 and 645 / 251; 2048 x 2304, N = 3136: 225 / 206 and 404 / 234; 4096 x 4096,
-//    N = 3136: 453 / 375 and 679 / 422; even rows lose at most 6 %, at K = 512).
+//  * B beyond the L2 and N above 512 (rows of 32 nonzeros and more): every XCD works on its own tiles of B (spmm_block), in
+//    tile-major order inside the XCD, in tiles of 128 where that gives each XCD two tiles and more, else of 64, and never
+//    wider than the slab that fits the L2. The eight L2s then fetch B once between them instead of once each, the finer
+//    tiles spread long rows, and the slab in use per XCD stays small. Against the widest fitting tile in one tile-major
+//    order for all XCDs (and row-major tiles of 512 on small grids), even / lognormal rows: 64 x 576, N = 3136: 10.4 -> 6.8 and
+//    14.3 -> 14.4; 64 x 147, N = 12544: 22.3 -> 12.7 and 19.3 -> 12.8; 256 x 2304, N = 3136: 86.8 -> ~40 and 134 -> ~90;
+//    1024 x 1152, N = 12544: 212 -> 197 and 645 -> 200; 2048 x 2304, N = 3136: 225 -> 200 and 404 -> 202; 4096 x 4096,
+//    N = 3136: 453 -> 350 and 679 -> 370; 8192 x 4096, N = 1024: 122 -> 120 and 134 -> 129 (tiles of 64).
+//    With tiles dealt to the XCDs in whole numbers only (49 tiles: 7 to one XCD, 6 to the others) the uneven load cost what
+//    the fetches saved (4096 x 4096: 394 us): hence the shared rest.
 //  Rows below 16 nonzeros pay the start of a row once more per tile: 256 x 64 with 3 ... 13 per row at N = 3136 lost 13-33 %
 //  to tiles of 256, 512 x 128 with 6 per row at N = 784 10-18 %.
 struct TileChoice { int width, major; };  // width 0: no tiles narrower than a wave covers (or than 512)
@@ -294,21 +329,28 @@ static TileChoice spmm_tile_width(const DeviceInfo& dev, int M, int K, int N, in
     const long long l2 = dev.l2_bytes;
     const int min_tile = narrow_tiles ? 32 : 128;
     if (N <= min_tile) return {0, 0};
+    const auto valid = [&](int t) { return (t == 512 || t == 256 || t == 128 || t == 64 || t == 32) && t >= min_tile; };
     const bool finer = plain && narrow_tiles && rule_on(kRuleFinerColumnTiles);
     const bool beyond_l2 = (double)K * (double)N * (double)sizeof(float) > (double)l2;
-    bool on = beyond_l2 && (long long)M * ceil_div(N, 512) >= (finer && N > 512 && 2ll * M >= dev.cus ? 3ll : 8ll) * dev.cus;
+    const int one = spmm_one_wave_tile(N);
+    const bool few_rows = finer && (long long)nnz >= 16ll * M && 4ll * M * ceil_div(N, one) <= 3ll * dev.cus;
+    // B beyond the L2 under dense rows wider than 512 floats, rows of 32 nonzeros and more: every XCD on its own tiles
+    const bool per_xcd = finer && !few_rows && beyond_l2 && N > 512 && (long long)nnz >= 32ll * M;
+    bool on = beyond_l2 && ((long long)M * ceil_div(N, 512) >= 8ll * dev.cus || per_xcd);
     if (tuning().tile_major >= 0) on = tuning().tile_major != 0;
+    if (tuning().tile_major >= kTilesPerXcd && plain)  // tuning: tiles of this width, each XCD on its own run of them (plain launches only)
+        return valid(tuning().tile_width) && tuning().tile_width < N ? TileChoice{tuning().tile_width, tuning().tile_major} : TileChoice{0, 0};
     if (!on) {
         const int t = tuning().tile_width;
         if (tuning().tile_major == 0)  // tuning: tiles of this width in row-major order
-            return (t == 512 || t == 256 || t == 128 || t == 64 || t == 32) && t >= min_tile && t < N ? TileChoice{t, 0} : TileChoice{0, 0};
+            return valid(t) && t < N ? TileChoice{t, 0} : TileChoice{0, 0};
         if (!finer || (long long)nnz < 16ll * M) return {0, 0};
-        const int one = spmm_one_wave_tile(N);
-        if (4ll * M * ceil_div(N, one) <= 3ll * dev.cus) {  // few rows
+        if (few_rows) {
             int tile = one;
             while (tile > 32 && (long long)M * ceil_div(N, tile) < 2ll * dev.cus) tile /= 2;
             if (2 * (N - (int)(ceil_div(N, tile) - 1) * tile) < tile) tile *= 2;  // a last tile less than half full: wider tiles
-            return tile < one && tile < N ? TileChoice{tile, 0} : TileChoice{0, 0};
+            if (tile >= one || tile >= N) return {0, 0};
+            return {tile, beyond_l2 && ceil_div(N, tile) >= 8 ? kTilesPerXcd : 0};
         }
         return N > 512 && M <= 8ll * dev.cus ? TileChoice{256, 0} : TileChoice{0, 0};
     }
@@ -324,13 +366,23 @@ static TileChoice spmm_tile_width(const DeviceInfo& dev, int M, int K, int N, in
     const bool sliced_too = !narrow_tiles && nnz >= kSlicedMinNnz && (long long)nnz >= 64ll * M && (long long)M >= kSlicedMinRowsPerCu * dev.cus;
     const bool narrow_ok =
         (long long)nnz >= 32ll * M && ((long long)K * tile * (long long)sizeof(float) <= 2 * l2 || sliced_too);
+    int major = 1;
     if (!narrow_ok) tile = 512;
-    else if (finer && tile > 64 && N > 512) tile = 64;
+    else if (per_xcd && tuning().tile_major < 0) {
+        int t = ceil_div(N, 128) >= 16 ? 128 : 64;  // two tiles of 128 per XCD and more, else tiles of 64
+        if (t > tile) t = tile;
+        if (ceil_div(N, t) >= 8) {
+            tile = t;
+            major = kTilesPerXcdTileMajor;
+        } else if (tile > 64) {
+            tile = 64;
+        }
+    }
     {
         const int t = tuning().tile_width;
-        if ((t == 512 || t == 256 || t == 128 || t == 64 || t == 32) && t >= min_tile) tile = t;
+        if (valid(t)) tile = t;
     }
-    return tile < N ? TileChoice{tile, 1} : TileChoice{0, 0};  // a single tile: nothing to order
+    return tile < N ? TileChoice{tile, major} : TileChoice{0, 0};  // a single tile: nothing to order
 }
 
 // Chooses the lane layout from N (and the height of B) and the (W, R) split from the mean row length.

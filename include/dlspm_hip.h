@@ -365,7 +365,8 @@ typedef struct dlspm_tuning {
     int flat;             /* flat schedule of a call with workspace: -1 the size rule, 0 never, 1 always            */
     int flat_chunk;       /* nonzeros per wave of the flat schedule (>= 64); 0 = the rule                           */
     int slices;           /* column-sliced schedule: -1 the size rule, 0 never, n >= 2 that many slices             */
-    int tile_major;       /* SpMM column tiles one after the other: -1 the rule, 0 no, 1 yes                        */
+    int tile_major;       /* SpMM column tiles: -1 the rule, 0 row-major, 1 one after the other (tile-major), 2 / 3 every */
+                          /* XCD on its own tiles, row- / tile-major within it (calls without memory, with tile_width)    */
     int tile_width;       /* SpMM column tile: 0 the rule, else 512, 256, 128, 64 or 32 (with tile_major = 0: tiles */
                           /* of this width in row-major order)                                                       */
     int plan_order;       /* dlspm_row_plan_build: 0 packed (the rule), 1 alternating groups, 2 longest first       */

@@ -154,12 +154,17 @@ def test_finer_column_tiles_for_plain_spmm_calls(dl):
     assert tile(2048, 512, 784, 100) == (256, 4)
     assert tile(2049, 512, 784, 100) == (512, 2)
     assert tile(1000, 512, 784, 15) == (512, 2)
-    assert tile(64, 576, 3136, 100) == (256, 13)     # 64 x 7 pairs: no longer "few rows"
-    # B beyond the L2 (K x N x 4 > 4 MiB): tile-major tiles of 64 from three pairs per compute unit on, 128 rows and more
-    assert tile(300, 1152, 3136, 100) == (64, 49)
-    assert tile(64, 1152, 12544, 100) == (256, 49)     # fewer rows than half the compute units: row-major tiles of 256
-    assert tile(4096, 4096, 3136, 100) == (64, 49)
+    assert tile(64, 256, 3136, 100) == (256, 13)     # 64 x 7 pairs: no longer "few rows"; B of 3.1 MiB fits the L2
+    # B beyond the L2 (K x N x 4 > 4 MiB) under N above 512: every XCD on its own tiles, of 128 columns where that gives
+    # each XCD two and more, else of 64; eight tiles at least
+    assert tile(64, 576, 3136, 100) == (128, 25)
+    assert tile(300, 1152, 3136, 100) == (128, 25)
+    assert tile(64, 1152, 12544, 100) == (128, 98)
+    assert tile(4096, 4096, 3136, 100) == (128, 25)
+    assert tile(256, 2304, 1536, 100) == (64, 24) and tile(1024, 4608, 784, 100) == (64, 13) and tile(1024, 4608, 640, 100) == (64, 10)
+    assert tile(8192, 16384, 3136, 100) == (64, 49)  # (the widest tile whose slab fits the L2 is narrower here)
     assert tile(4096, 4096, 3136, 20) == (512, 7)    # rows below 32 nonzeros keep the widest tile, as before
+    assert tile(32, 2304, 2048, 230) == (128, 16)    # few rows: two pairs per compute unit, the XCDs on their own tiles as well
     dl.set_tuning(rules_off=dl.RULES["finer_column_tiles"])
     try:
         assert tile(128, 1152, 256, 200) == (256, 1) and tile(1000, 512, 784, 100) == (512, 2)
@@ -208,9 +213,10 @@ def test_column_tiles_narrow_with_the_height_of_the_dense_operand(dl):
         finally:
             dl.set_tuning()
         assert sh["G"] * sh["vec"] * sh["V"] == tile and sh["col_tiles"] == -(-3136 // tile), (K, sh)
-        # a call without memory takes tiles of 64 at most (N above 512): long rows spread over more workgroups
+        # a call without memory takes tiles of 128 at most here (25 tiles: three to each XCD, one shared): every XCD
+        # works on its own tiles of B
         sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz)
-        assert sh["G"] * sh["vec"] * sh["V"] == min(tile, 64) and sh["col_tiles"] == -(-3136 // min(tile, 64)), (K, sh)
+        assert sh["G"] * sh["vec"] * sh["V"] == min(tile, 128) and sh["col_tiles"] == -(-3136 // min(tile, 128)), (K, sh)
         sh = dl.describe_launch(dl.OP_SPMM, 4096, K, 3136, nnz, with_workspace=True)
         assert sh["G"] * sh["vec"] * sh["V"] == (max(tile, 128) if K * 128 * 4 <= (8 << 20) else 512)
     # ... with memory and rows long enough for the column-sliced schedule (64 nonzeros per row, half a million in

@@ -447,11 +447,13 @@ def test_column_sliced_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
 
 @pytest.mark.parametrize("M,K,N,per_row,tile,tiles", [
     (128, 1152, 256, 200, 64, 4), (64, 576, 512, 100, 64, 8), (16, 576, 500, 100, 32, 16), (128, 1152, 196, 200, 128, 2),
-    (5, 300, 50, 40, 32, 2), (1000, 512, 784, 100, 256, 4), (300, 1152, 3140, 100, 64, 50), (130, 2304, 1030, 60, 256, 5)])
+    (5, 300, 50, 40, 32, 2), (1000, 512, 784, 100, 256, 4), (300, 1152, 3140, 100, 128, 25), (130, 2304, 1030, 60, 64, 17),
+    (32, 2304, 2048, 230, 128, 16), (700, 4608, 650, 100, 64, 11), (64, 147, 12548, 75, 128, 99)])
 @pytest.mark.parametrize("sigma", [0.0, 0.8])
 def test_finer_column_tiles_of_plain_spmm_calls(torch_cuda, dl, oracle, M, K, N, per_row, tile, tiles, sigma):
     """The column tiles a SpMM call without memory takes for few rows and for wide dense rows (row-major tiles of
-    32 ... 256 columns, tile-major tiles of 64 where B exceeds the L2; last tiles of 4, 5 and 6 columns among them):
+    32 ... 256 columns; where B exceeds the L2 every XCD on its own tiles of 64 or 128 columns, with 1 ... 3 tiles left
+    over that all XCDs share; last tiles of 4, 6 and 10 columns among them):
     NULL and the even-rows hint against the oracle, and against the same call with the rule switched off."""
     torch = torch_cuda
     if sigma == 0.0:

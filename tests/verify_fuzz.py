@@ -40,7 +40,7 @@ def random_tuning(rng):
     if rng.random() < 0.5:
         t["slices"] = pick([0, 2, 3, 4, 7, 16])
     if rng.random() < 0.5:
-        t["tile_major"] = pick([0, 1])
+        t["tile_major"] = pick([0, 1, 2, 3])
     if rng.random() < 0.5:
         t["tile_width"] = pick([512, 256, 128, 64, 32])
     if rng.random() < 0.5:
