@@ -2,7 +2,7 @@
 """Two rules for calls without memory or plan, each timed on and off where it applies (MI355X):
 
   * SpMM, finer column tiles of B (DLSPM_RULE_FINER_COLUMN_TILES): few rows at N = 64 ... 1024, and dense rows wider
-    than 512 floats on 200 ... 4096 rows;
+    than 512 floats on 64 ... 8192 rows (where B exceeds the L2: every XCD on its own tiles);
   * SDDMM, several workgroups per row of a mask of few rows (DLSPM_RULE_ROW_PIECES_FEW_ROWS), D = 32 ... 256, with the
     time of the same launch under a cut plan beside it.
 
@@ -108,7 +108,7 @@ def main():
                     spmm_case(f"{M} rows, N = {N}", kind, M, K, per_row, N)
     wide = ((200, 2304, 230, 784), (128, 1152, 290, 784), (1500, 512, 100, 600), (1000, 2048, 200, 640), (300, 1152, 115, 3136),
             (256, 2304, 230, 3136), (1024, 1152, 115, 12544), (2048, 2304, 230, 3136), (4096, 4096, 200, 3136), (2048, 512, 100, 784),
-            (256, 64, 13, 3136))
+            (256, 64, 13, 3136), (64, 576, 115, 3136), (64, 147, 75, 12544), (512, 4608, 460, 3136), (8192, 4096, 100, 1024))
     for kind in ("even", "logn"):
         for M, K, per_row, N in (wide[::3] if args.quick else wide):
             spmm_case("dense rows wider than 512", kind, M, K, per_row, N)
