@@ -650,6 +650,7 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
     const bool vec4 = N_or_D >= 4;
     bool second_kernel = op == DLSPM_OP_FUSED;  // a cut plan's pieces leave partial rows for a second kernel to add
     int spread = 1;  // workgroups over which a call without plan spreads each row by itself
+    int model_width = N_or_D;  // floats gathered per nonzero by one workgroup
     if (op == DLSPM_OP_SPMM) {
         SpmmShape shape = spmm_choose(dev, M, K, N_or_D, nnz, vec4, false, true);
         if (!spmm_plan_applies(dev, shape, M, N_or_D, nnz)) return 0;
@@ -658,6 +659,8 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
         const SpmmShape plain = spmm_choose(dev, M, K, N_or_D, nnz, vec4, false, true, false, true);
         const long long tiles = ceil_div(N_or_D, shape.G * shape.vec * shape.V), tiles_plain = ceil_div(N_or_D, plain.G * plain.vec * plain.V);
         if (!plain.tile_major && tiles_plain > tiles) spread = (int)(tiles_plain / tiles);
+        // dense rows in column tiles: a workgroup gathers one tile's width per nonzero, and that is what a cut would save
+        model_width = std::min(N_or_D, shape.G * shape.vec * shape.V);
     } else if (op == DLSPM_OP_SDDMM) {
         SddmmShape shape = sddmm_choose(dev, M, N_or_D, nnz, vec4);
         if (!sddmm_plan_applies(dev, shape, M, N_or_D, nnz, rows_are_skewed(M, nnz, max_row_len))) {
@@ -689,7 +692,11 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
     int slices = 0;
     (void)dlspm_describe_slices(op, M, K, N_or_D, nnz, &slices, nullptr);
     if (slices >= 3) return 0;
-    if (cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len, second_kernel, spread)) return 2;
+    // (dense rows in column tiles: the tiles already spread a long row over several workgroups, and the partial rows of a cut
+    // would be N floats wide: lognormal rows, sigma 1.2, cut plan / plan over whole rows: 512 x 2048, N = 1024: 23.6 / 16.0 us;
+    // 1024 x 1152, N = 12544: 229 / 203 us; 512 x 4608, N = 3136: 121 / 132 us)
+    const bool tiled = op == DLSPM_OP_SPMM && model_width < N_or_D;
+    if (!tiled && cut_plan_pays(dev, op, M, model_width, nnz, max_row_len, second_kernel, spread)) return 2;
     return spread > 1 ? 0 : 1;  // (a plan over whole rows would undo the spread)
 }
 

@@ -110,7 +110,7 @@ inline bool rule_on(int rule) { return (tuning().rules_off & rule) == 0; }
 // bit 3 = never take the row-aligned split (DLSPM_RULE_ROW_ALIGNED_SPLIT switched off); bit 4 (SDDMM, one row per
 // workgroup) = the waves of a row take whole passes of 64 nonzeros in turn (sddmm_row_interleaved).
 constexpr int kFlagXcdContiguous = 1, kFlagStreamShift = 1, kFlagStreamNever = 1, kFlagStreamAlways = 2, kFlagNoAlignedSplit = 8,
-              kFlagFullPasses = 16, kFlagPiecesShift = 8, kFlagPiecesMask = 7;  // (bits 8-10: log2 of the workgroups that share a row, SDDMM)
+              kFlagFullPasses = 16, kFlagPiecesShift = 8, kFlagPiecesMask = 7, kFlagTileOrderShift = 12;  // (bits 8-10: log2 of the workgroups that share a row, SDDMM; bits 12-13: SpmmShape::tile_major of a planned SpMM launch)
 inline int launch_flags(int xcd_contiguous_hint)
 {
     const Tuning& t = tuning();

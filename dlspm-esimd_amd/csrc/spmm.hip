@@ -165,6 +165,14 @@ __global__ __launch_bounds__(4 * 64) void spmm_sliced_kernel(int M, int N, int c
                                       bounds + (size_t)(sl + 1) * M, col_indices, values, B, partial + (size_t)sl * M * N);
 }
 
+// the order of the column tiles in a planned launch (launch flags, bits 12-13): tile after tile for all XCDs, or every
+// XCD on its own tiles (tile after tile inside it)
+__device__ __forceinline__ int planned_tile_order(int flags)
+{
+    const int order = (flags >> kFlagTileOrderShift) & 3;
+    return order >= kTilesPerXcd ? kTilesPerXcdTileMajor : 1;
+}
+
 // Row plan: workgroup i works on the whole row rows[i] = [starts[i], ends[i]) of the CSR matrix (one row per four-wave
 // workgroup); with column tiles the plan is gone through once per tile, tile after tile.
 template <int VEC, int G, int V, bool BUF>
@@ -175,8 +183,8 @@ __global__ __launch_bounds__(4 * 64) void spmm_planned_kernel(int M, int N, int 
                                                               const float* __restrict__ values,
                                                               const float* __restrict__ B, float* __restrict__ C)
 {
-    spmm_block<VEC, G, V, 4, 1, true, kPlanRows, BUF>((int)blockIdx.x, M, N, col_tiles, 1, starts, ends, col_indices, values,
-                                                      B, C, rows, nnz, flags, M);
+    spmm_block<VEC, G, V, 4, 1, true, kPlanRows, BUF>((int)blockIdx.x, M, N, col_tiles, planned_tile_order(flags), starts, ends,
+                                                      col_indices, values, B, C, rows, nnz, flags, M);
 }
 
 // Row plan with cut rows: `entries` workgroups per column tile, entry i = the nonzeros [starts[i], ends[i]) of row rows[i],
@@ -192,7 +200,7 @@ __global__ __launch_bounds__(4 * 64) void spmm_pieces_kernel(int M, int N, int n
                                                              const float* __restrict__ B, float* __restrict__ C,
                                                              float* __restrict__ pieces)
 {
-    spmm_block<VEC, G, V, 4, 1, true, kPlanPieces, BUF>((int)blockIdx.x, M, N, col_tiles, 1, starts, ends, col_indices, values,
+    spmm_block<VEC, G, V, 4, 1, true, kPlanPieces, BUF>((int)blockIdx.x, M, N, col_tiles, planned_tile_order(flags), starts, ends, col_indices, values,
                                                         B, C, rows, nnz, flags, entries, slot_of, pieces, slots);
 }
 
@@ -335,10 +343,11 @@ static TileChoice spmm_tile_width(const DeviceInfo& dev, int M, int K, int N, in
     const int one = spmm_one_wave_tile(N);
     const bool few_rows = finer && (long long)nnz >= 16ll * M && 4ll * M * ceil_div(N, one) <= 3ll * dev.cus;
     // B beyond the L2 under dense rows wider than 512 floats, rows of 32 nonzeros and more: every XCD on its own tiles
-    const bool per_xcd = finer && !few_rows && beyond_l2 && N > 512 && (long long)nnz >= 32ll * M;
+    // (calls without schedule memory: plain ones and planned ones alike, so that a plan keeps what the plain call has)
+    const bool per_xcd = narrow_tiles && rule_on(kRuleFinerColumnTiles) && !few_rows && beyond_l2 && N > 512 && (long long)nnz >= 32ll * M;
     bool on = beyond_l2 && ((long long)M * ceil_div(N, 512) >= 8ll * dev.cus || per_xcd);
     if (tuning().tile_major >= 0) on = tuning().tile_major != 0;
-    if (tuning().tile_major >= kTilesPerXcd && plain)  // tuning: tiles of this width, each XCD on its own run of them (plain launches only)
+    if (tuning().tile_major >= kTilesPerXcd && narrow_tiles)  // tuning: tiles of this width, each XCD on its own run of them (not with schedule memory)
         return valid(tuning().tile_width) && tuning().tile_width < N ? TileChoice{tuning().tile_width, tuning().tile_major} : TileChoice{0, 0};
     if (!on) {
         const int t = tuning().tile_width;
@@ -370,10 +379,22 @@ static TileChoice spmm_tile_width(const DeviceInfo& dev, int M, int K, int N, in
     if (!narrow_ok) tile = 512;
     else if (per_xcd && tuning().tile_major < 0) {
         int t = ceil_div(N, 128) >= 16 ? 128 : 64;  // two tiles of 128 per XCD and more, else tiles of 64
+        if (!plain && (long long)M >= 4ll * dev.cus) {
+            // a planned launch runs one row per workgroup whatever the rows' lengths (a plain one groups short rows): from four
+            // rows per compute unit on, the finest tile that still gives a workgroup 20 000 products of a mean row, 64 ... 256
+            // columns (lognormal rows, sigma 0.5, tiles of 256 / 128 / 64: 8192 x 4096 of 100 per row, N = 1024: 124 / 127 /
+            // 185 us; 2048 x 2304 of 230, N = 3136: 206 / 197 / 215 us; 4096 x 8192 of 400, N = 1024: 407 / 253 / 236 us;
+            // fewer rows want the finer tiles of the plain call, which shorten the tail: 300 x 1152 of 115: 23.5 / 19.7 / 24.0 us)
+            const long long avg = std::max<long long>(nnz / std::max(M, 1), 1);
+            const int by_work = avg * 64 >= 20000 ? 64 : avg * 128 >= 20000 ? 128 : 256;
+            if (by_work > t) t = by_work;
+        }
         if (t > tile) t = tile;
         if (ceil_div(N, t) >= 8) {
             tile = t;
             major = kTilesPerXcdTileMajor;
+        } else if (!plain) {
+            tile = t;  // fewer than eight tiles: one after the other for all XCDs
         } else if (tile > 64) {
             tile = 64;
         }
@@ -641,10 +662,10 @@ hipError_t spmm_planned_launch(const SpmmArgs& x, const SpmmShape& s, const int*
             if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
             if (dense_fits_buffer(x.K, x.N))
                 hipLaunchKernelGGL((spmm_planned_kernel<4, L::G, L::V, true>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M,
-                                   x.N, x.nnz, col_tiles, launch_flags(0), starts, ends, rows, x.col_indices, x.values, x.B, x.C);
+                                   x.N, x.nnz, col_tiles, launch_flags(0) | (s.tile_major << kFlagTileOrderShift), starts, ends, rows, x.col_indices, x.values, x.B, x.C);
             else
                 hipLaunchKernelGGL((spmm_planned_kernel<4, L::G, L::V, false>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M,
-                                   x.N, x.nnz, col_tiles, launch_flags(0), starts, ends, rows, x.col_indices, x.values, x.B, x.C);
+                                   x.N, x.nnz, col_tiles, launch_flags(0) | (s.tile_major << kFlagTileOrderShift), starts, ends, rows, x.col_indices, x.values, x.B, x.C);
             return hipGetLastError();
         }
     });
@@ -690,11 +711,11 @@ hipError_t spmm_pieces_launch(const SpmmArgs& x, const SpmmShape& s, const CutPl
             }
             if (dense_fits_buffer(x.K, x.N))
                 hipLaunchKernelGGL((spmm_pieces_kernel<4, L::G, L::V, true>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M,
-                                   x.N, x.nnz, col_tiles, launch_flags(0), cp.entries, cp.slots, starts, ends, rows, slot_of,
+                                   x.N, x.nnz, col_tiles, launch_flags(0) | (s.tile_major << kFlagTileOrderShift), cp.entries, cp.slots, starts, ends, rows, slot_of,
                                    x.col_indices, x.values, x.B, x.C, pieces);
             else
                 hipLaunchKernelGGL((spmm_pieces_kernel<4, L::G, L::V, false>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream, x.M,
-                                   x.N, x.nnz, col_tiles, launch_flags(0), cp.entries, cp.slots, starts, ends, rows, slot_of,
+                                   x.N, x.nnz, col_tiles, launch_flags(0) | (s.tile_major << kFlagTileOrderShift), cp.entries, cp.slots, starts, ends, rows, slot_of,
                                    x.col_indices, x.values, x.B, x.C, pieces);
             return hipGetLastError();
         }

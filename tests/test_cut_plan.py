@@ -198,7 +198,11 @@ def test_cut_plan_sizes_and_advice(dl):
     assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 256, 52000, 110) == 0    # even rows: no plan at all
     assert dl.row_plan_advice(dl.OP_SPMM, 2048, 512, 256, 4999, 100) == 1     # a handful of nonzeros: all start-up, no cut plan
     assert dl.row_plan_advice(dl.OP_SPMM, 2048, 512, 256, 5000, 100) == 2
-    assert dl.row_plan_advice(dl.OP_SDDMM, 2048, 512, 128, 2400, 200) == 2    # (SDDMM gains from a cut plan at every size)
+    assert dl.row_plan_advice(dl.OP_SDDMM, 2048, 512, 128, 2400, 200) == 2
+    # dense rows in column tiles (N above 512): the tiles spread a long row already, no cut plan
+    assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 1024, 52000, 2048) == 1
+    assert dl.row_plan_advice(dl.OP_SPMM, 1024, 1152, 12544, 119909, 1152) == 1
+    assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 512, 52000, 2048) == 2    # (SDDMM gains from a cut plan at every size)
     # fewer rows than three quarters of the compute units: a call without plan spreads every row over several workgroups by
     # itself (SDDMM: row pieces; SpMM: column tiles of B), so a cut plan is advised only where a row is still too long for
     # one of them -- and never the plan over whole rows, which would undo the spread
