@@ -342,9 +342,13 @@ static TileChoice spmm_tile_width(const DeviceInfo& dev, int M, int K, int N, in
     const bool beyond_l2 = (double)K * (double)N * (double)sizeof(float) > (double)l2;
     const int one = spmm_one_wave_tile(N);
     const bool few_rows = finer && (long long)nnz >= 16ll * M && 4ll * M * ceil_div(N, one) <= 3ll * dev.cus;
-    // B beyond the L2 under dense rows wider than 512 floats, rows of 32 nonzeros and more: every XCD on its own tiles
+    // B beyond the L2 under dense rows of eight tiles of 64 floats and more, rows of 32 nonzeros and more: every XCD on its own tiles
+    // (N = 512, tiles of 128 for all XCDs -> of 64, each XCD on its own: 2048 x 8192: 80.5 -> 64.0 us even, 137 -> 74.9 us lognormal; 8192 x
+    // 8192: 513 -> 505 and 631 -> 510 us; 1024 x 2304: 21.4 -> 20.7 and 64.1 -> 26.0 us; up to sixteen rows per compute unit: 8192 x
+    // 2304 of 100 per row lost 17 %; at N = 256 eight tiles of 32 lose up to 25 %)
     // (calls without schedule memory: plain ones and planned ones alike, so that a plan keeps what the plain call has)
-    const bool per_xcd = narrow_tiles && rule_on(kRuleFinerColumnTiles) && !few_rows && beyond_l2 && N > 512 && (long long)nnz >= 32ll * M;
+    const bool per_xcd = narrow_tiles && rule_on(kRuleFinerColumnTiles) && !few_rows && beyond_l2 && (long long)nnz >= 32ll * M &&
+                         (N > 512 || (N > 448 && M <= 16ll * dev.cus));
     bool on = beyond_l2 && ((long long)M * ceil_div(N, 512) >= 8ll * dev.cus || per_xcd);
     if (tuning().tile_major >= 0) on = tuning().tile_major != 0;
     if (tuning().tile_major >= kTilesPerXcd && narrow_tiles)  // tuning: tiles of this width, each XCD on its own run of them (not with schedule memory)

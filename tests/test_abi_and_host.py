@@ -163,6 +163,7 @@ def test_finer_column_tiles_for_plain_spmm_calls(dl):
     assert tile(4096, 4096, 3136, 100) == (128, 25)
     assert tile(256, 2304, 1536, 100) == (64, 24) and tile(1024, 4608, 784, 100) == (64, 13) and tile(1024, 4608, 640, 100) == (64, 10)
     assert tile(8192, 16384, 3136, 100) == (64, 49)  # (the widest tile whose slab fits the L2 is narrower here)
+    assert tile(2048, 8192, 512, 400) == (64, 8) and tile(2048, 8192, 448, 400) == (128, 4)   # from eight tiles of 64 on
     assert tile(4096, 4096, 3136, 20) == (512, 7)    # rows below 32 nonzeros keep the widest tile, as before
     assert tile(32, 2304, 2048, 230) == (128, 16)    # few rows: two pairs per compute unit, the XCDs on their own tiles as well
     dl.set_tuning(rules_off=dl.RULES["finer_column_tiles"])
@@ -245,8 +246,10 @@ def test_column_tiles_narrow_with_the_height_of_the_dense_operand(dl):
     assert dl.describe_launch(dl.OP_SPMM, 1 << 18, 32768, 128, (1 << 18) * 8)["col_tiles"] == 1
     assert dl.describe_launch(dl.OP_SPMM, 4096, 32768, 64, nnz)["col_tiles"] == 2
     assert dl.describe_launch(dl.OP_SPMM, 4096, 32768, 32, nnz)["col_tiles"] == 1   # 32 columns: the narrowest tile
-    sh = dl.describe_launch(dl.OP_SPMM, 4096, 4096, 512, nnz)
+    sh = dl.describe_launch(dl.OP_SPMM, 4097, 4096, 512, nnz)
     assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (256, 2)
+    sh = dl.describe_launch(dl.OP_SPMM, 4096, 4096, 512, nnz)         # up to sixteen rows per compute unit: the XCDs' own tiles of 64
+    assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (64, 8)
     assert dl.describe_launch(dl.OP_SPMM, 4096, 4096, 256, nnz)["col_tiles"] == 1   # 4 MiB: fits
     assert dl.describe_launch(dl.OP_SPMM, 1024, 8192, 256, nnz)["col_tiles"] == 1   # a grid the device holds at once
 

@@ -448,7 +448,7 @@ def test_column_sliced_schedule_at_its_own_sizes(torch_cuda, dl, oracle, sigma):
 @pytest.mark.parametrize("M,K,N,per_row,tile,tiles", [
     (128, 1152, 256, 200, 64, 4), (64, 576, 512, 100, 64, 8), (16, 576, 500, 100, 32, 16), (128, 1152, 196, 200, 128, 2),
     (5, 300, 50, 40, 32, 2), (1000, 512, 784, 100, 256, 4), (300, 1152, 3140, 100, 128, 25), (130, 2304, 1030, 60, 64, 17),
-    (32, 2304, 2048, 230, 128, 16), (700, 4608, 650, 100, 64, 11), (64, 147, 12548, 75, 128, 99)])
+    (32, 2304, 2048, 230, 128, 16), (700, 4608, 650, 100, 64, 11), (64, 147, 12548, 75, 128, 99), (300, 4608, 500, 300, 64, 8)])
 @pytest.mark.parametrize("sigma", [0.0, 0.8])
 def test_finer_column_tiles_of_plain_spmm_calls(torch_cuda, dl, oracle, M, K, N, per_row, tile, tiles, sigma):
     """The column tiles a SpMM call without memory takes for few rows and for wide dense rows (row-major tiles of
