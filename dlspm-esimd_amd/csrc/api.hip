@@ -618,7 +618,13 @@ static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int n
     // With a second kernel: only where a share holds at least two mean rows, so that the rows above one and a half
     // shares are the exception and the kernel that adds their pieces has little to do (the reference's layers of 64 ...
     // 256 rows, where most rows would be cut: 0.85 ... 1.5 times the time of the plan over whole rows; 512 rows: 0.66 ... 1.0)
-    if (second_kernel && M < 2 * cus) return false;
+    // The fused op on few rows is the exception: one row per compute unit, eight waves on it, most of the device idle, so a
+    // long row pays for the second kernel from a gain of 6 us by this model on (10 us below 32 rows, where a share is a
+    // handful of nonzeros), shares of 32 nonzeros and more (lognormal rows, sigma 0.8, NULL / cut plan: 64 x 2304 of 230
+    // per row, D = 128: 14.5 / 10.1 us; 32 x 4608 of 1380, D = 256: 82.6 / 16.8 us; even rows 64 x 4608, D = 128: 17.2 /
+    // 10.5 us; below the threshold the cut plan loses 5-60 %: the reference's layers of 128 ... 256 rows, D = 64: 1.2-1.5x).
+    const bool few_rows_fused = op == DLSPM_OP_FUSED && M < 2 * cus;
+    if (second_kernel && M < 2 * cus && !few_rows_fused) return false;
     // SpMM on a handful of nonzeros is all start-up, and the cut plan's larger grid adds to it (the reference's data set at
     // N = 256, cut plan / NULL: 1.10 below 2500 nonzeros (21 files), 1.00 below 5000 (23), 0.92 below 10 000 (49); SDDMM gains
     // at every size: 0.89 / 0.91 / 0.88)
@@ -629,6 +635,7 @@ static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int n
     if (longest_unit <= longest_whole) return false;
     const double bytes_per_nonzero = (op == DLSPM_OP_FUSED ? 2.0 : 1.0) * (double)std::min(width, 512) * sizeof(float);
     const double saved_ns = (double)(longest_unit - longest_whole) * bytes_per_nonzero / 115.0;
+    if (few_rows_fused) return share >= 32 && saved_ns >= (M < 32 ? 10000.0 : 6000.0);
     if (second_kernel) return saved_ns >= kCutPlanMinGainNs;
     // (SpMM, N = 256, the 302 files of the reference's data set with a row above one and a half shares, against the better
     // of NULL and the plan over whole rows: 0.99 of the time below 300 ns by this model, 0.96 / 0.91 / 0.84 / 0.81 from 300 /
@@ -674,7 +681,12 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
         }
     } else if (op == DLSPM_OP_FUSED) {
         FusedShape shape = fused_choose(dev, M, N_or_D, nnz, vec4);
-        if (!fused_plan_applies(dev, shape, M, N_or_D, nnz, rows_are_skewed(M, nnz, max_row_len))) return 0;
+        if (!fused_plan_applies(dev, shape, M, N_or_D, nnz, rows_are_skewed(M, nnz, max_row_len))) {
+            // fewer rows than two per compute unit (eight waves per row): only a cut plan helps, where a row is long enough
+            // to pay for the kernel that adds its pieces
+            FusedShape few = fused_choose(dev, M, N_or_D, nnz, vec4);
+            return fused_cut_plan_applies(dev, few, M, N_or_D, nnz) && cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len, true) ? 2 : 0;
+        }
     } else {
         return 0;
     }
@@ -782,7 +794,7 @@ int fused_sddmm_spmm_f32(int M, int K, int D, int nnz, const int* row_offsets, c
         const CutPlan cp = cut_plan_layout(M, D, dev.cus);
         if (cp.bytes == 0 || ws.bytes < cp.bytes) return DLSPM_E_WORKSPACE;
         FusedShape shape = fused_choose(dev, M, D, nnz, vec4);
-        e = fused_plan_applies(dev, shape, M, D, nnz) ? fused_pieces_launch(args, shape, cp, ws.mem, st) : fused_launch(args, shape, st);
+        e = fused_cut_plan_applies(dev, shape, M, D, nnz) ? fused_pieces_launch(args, shape, cp, ws.mem, st) : fused_launch(args, shape, st);
         return e == hipSuccess ? DLSPM_OK : fail_hip(e);
     }
     if (ws.row_plan && ws.mem) {

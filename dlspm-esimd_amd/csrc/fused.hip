@@ -380,6 +380,18 @@ bool fused_plan_applies(const DeviceInfo& dev, FusedShape& s, int M, int D, int 
     return true;
 }
 
+// A cut plan also serves masks of fewer rows than two per compute unit, which the size rule runs with eight waves per row:
+// cut, the pieces of the rows fill the device (four waves each), at the price of the kernel that adds the partial rows.
+bool fused_cut_plan_applies(const DeviceInfo& dev, FusedShape& s, int M, int D, int nnz)
+{
+    if (s.vec == 4 && s.G1 == 8 && s.DS >= 1 && s.G * s.vec * s.V >= D && s.W == 8 && M < 2 * dev.cus) {
+        s.W = 4;
+        s.R = 1;
+        return true;
+    }
+    return fused_plan_applies(dev, s, M, D, nnz);
+}
+
 template <int DS, int G, int V2>
 static hipError_t launch_planned(const FusedArgs& x, const int* plan, hipStream_t stream)
 {

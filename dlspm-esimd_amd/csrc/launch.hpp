@@ -283,6 +283,7 @@ bool sddmm_plan_applies(const DeviceInfo& dev, SddmmShape& s, int M, int D, int 
 bool sddmm_cut_plan_applies(const DeviceInfo& dev, SddmmShape& s, int M, int D, int nnz);  // also few rows of eight waves each
 hipError_t sddmm_planned_launch(const SddmmArgs& x, const SddmmShape& s, const int* plan, hipStream_t stream);
 bool fused_plan_applies(const DeviceInfo& dev, FusedShape& s, int M, int D, int nnz, bool skewed = false);
+bool fused_cut_plan_applies(const DeviceInfo& dev, FusedShape& s, int M, int D, int nnz);  // ... of a launch with a cut plan (also few rows)
 hipError_t fused_planned_launch(const FusedArgs& x, const FusedShape& s, const int* plan, hipStream_t stream);
 // with a cut plan: SDDMM needs neither partial rows nor a second kernel (every piece writes its own CSR slots)
 hipError_t sddmm_pieces_launch(const SddmmArgs& x, const SddmmShape& s, const CutPlan& cp, const void* plan, hipStream_t stream);

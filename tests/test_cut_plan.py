@@ -199,6 +199,15 @@ def test_cut_plan_sizes_and_advice(dl):
     assert dl.row_plan_advice(dl.OP_SPMM, 2048, 512, 256, 4999, 100) == 1     # a handful of nonzeros: all start-up, no cut plan
     assert dl.row_plan_advice(dl.OP_SPMM, 2048, 512, 256, 5000, 100) == 2
     assert dl.row_plan_advice(dl.OP_SDDMM, 2048, 512, 128, 2400, 200) == 2
+    # the fused op on fewer rows than two per compute unit (eight waves per row, nothing spreads a row): a cut plan where a
+    # row is long enough to pay for the kernel that adds its pieces, and a share holds 32 nonzeros
+    assert dl.row_plan_advice(dl.OP_FUSED, 64, 2304, 128, 16905, 1654) == 2
+    assert dl.row_plan_advice(dl.OP_FUSED, 64, 2304, 64, 16905, 1654) == 2
+    assert dl.row_plan_advice(dl.OP_FUSED, 64, 2304, 64, 16905, 1200) == 0
+    assert dl.row_plan_advice(dl.OP_FUSED, 8, 4608, 128, 10981, 1435) == 2
+    assert dl.row_plan_advice(dl.OP_FUSED, 8, 4608, 64, 10981, 1435) == 0      # below 32 rows: from 10 us on
+    assert dl.row_plan_advice(dl.OP_FUSED, 32, 512, 256, 3314, 512) == 0       # a share of 13 nonzeros
+    assert dl.row_plan_advice(dl.OP_FUSED, 128, 1152, 64, 29510, 455) == 0
     # dense rows in column tiles (N above 512): the tiles spread a long row already, no cut plan
     assert dl.row_plan_advice(dl.OP_SPMM, 512, 2048, 1024, 52000, 2048) == 1
     assert dl.row_plan_advice(dl.OP_SPMM, 1024, 1152, 12544, 119909, 1152) == 1
