@@ -315,7 +315,8 @@ template <typename Launch> static hipError_t dispatch_layout(const SpmmShape& s,
 //  * N above 512 and up to eight rows per compute unit: row-major tiles of 256 instead of 512 (200 x 2304, N = 784:
 //    12.2 / 11.5 even, 42.1 / 19.7 lognormal; 1500 x 512, N = 600: 24.8 / 19.3 and 34.4 / 25.6; taller matrices lose:
 //    8192 x 512, N = 784: 57.4 / 62.0).
-//  * B beyond the L2 and N above 512 (rows of 32 nonzeros and more): every XCD works on its own tiles of B (spmm_block), in
+//  * B beyond the L2 and N above 512 (rows of 32 nonzeros and more; planned launches too, and N from 449 on in matrices of up to
+//    sixteen rows per compute unit): every XCD works on its own tiles of B (spmm_block), in
 //    tile-major order inside the XCD, in tiles of 128 where that gives each XCD two tiles and more, else of 64, and never
 //    wider than the slab that fits the L2. The eight L2s then fetch B once between them instead of once each, the finer
 //    tiles spread long rows, and the slab in use per XCD stays small. Against the widest fitting tile in one tile-major
