@@ -326,7 +326,7 @@ constexpr int kCutPlanAdviceMaxRows = 16384;     // the cut rule is one workgrou
 constexpr double kCutPlanMinGainNs = 2500.0;      // fused, SpMM with partial rows: the kernel that adds the pieces must be paid for
 constexpr double kCutPlanMinGainNsOneKernel = 300.0;  // SDDMM, and SpMM where the pieces share the columns: no second kernel
 constexpr int kCutPlanMinNnzSpmm = 5000;            // SpMM: no cut plan for fewer nonzeros
-constexpr double kCutPlanMinGainNsSddmmOneRowEach = 1000.0;  // ... one to two rows per compute unit: eight waves per row do nearly as well
+constexpr double kCutPlanMinGainNsSddmmOneRowEach = 1000.0;  // ... one and a half to two rows per compute unit: eight waves per row do nearly as well
 
 // longest row and number of rows without nonzeros (dlspm_csr_row_stats); stats[0] = max, stats[1] = empty rows
 __global__ void row_stats_kernel(int M, const int* __restrict__ row_offsets, int* __restrict__ stats)
@@ -640,7 +640,7 @@ static bool cut_plan_pays(const DeviceInfo& dev, int op, int M, int width, int n
     // (SpMM, N = 256, the 302 files of the reference's data set with a row above one and a half shares, against the better
     // of NULL and the plan over whole rows: 0.99 of the time below 300 ns by this model, 0.96 / 0.91 / 0.84 / 0.81 from 300 /
     // 600 / 1000 / 2500 ns on, at every height from 64 to 2048 rows)
-    if (op == DLSPM_OP_SDDMM && M >= cus && M < 2 * cus) return saved_ns >= kCutPlanMinGainNsSddmmOneRowEach;
+    if (op == DLSPM_OP_SDDMM && 2 * M > 3 * cus && M < 2 * cus) return saved_ns >= kCutPlanMinGainNsSddmmOneRowEach;
     return saved_ns >= kCutPlanMinGainNsOneKernel;
 }
 
@@ -674,8 +674,12 @@ int dlspm_row_plan_advice(int op, int M, int K, int N_or_D, int nnz, int max_row
             // fewer rows than compute units: only a cut plan helps (its pieces fill the device)
             SddmmShape few = sddmm_choose(dev, M, N_or_D, nnz, vec4), plain = few;
             sddmm_few_rows_pieces(dev, plain, M, nnz);  // what a call without plan does by itself
+            // (from three quarters of a compute unit's count of rows on, its two workgroups per row fill the device no
+            // better than the rows themselves would: lognormal rows on 200 ... 384 rows, D = 64 ... 256, a cut plan against
+            // the call without: 0.95 of the time and less from 300 ns by the model of whole rows on, 0.5 ... 0.8 from 2000 ns)
+            const int spread = 4ll * M > 3ll * dev.cus ? 1 : 1 << plain.pieces_lg;
             return sddmm_cut_plan_applies(dev, few, M, N_or_D, nnz) &&
-                           cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len, false, 1 << plain.pieces_lg)
+                           cut_plan_pays(dev, op, M, N_or_D, nnz, max_row_len, false, spread)
                        ? 2
                        : 0;
         }

@@ -69,6 +69,14 @@ template <> struct Vec<4> {
         t.v.z = ov > 2 ? 0.f : t.v.z;
         return t;
     }
+    // zeroes the first `n` of the four elements (n >= 4: all of them), one select each and no branch
+    __device__ __forceinline__ void zero_first(int n)
+    {
+        v.x = n > 0 ? 0.f : v.x;
+        v.y = n > 1 ? 0.f : v.y;
+        v.z = n > 2 ? 0.f : v.z;
+        v.w = n > 3 ? 0.f : v.w;
+    }
     __device__ __forceinline__ void fma(float a, const Vec& b)
     {
         v.x = fmaf(a, b.v.x, v.x); v.y = fmaf(a, b.v.y, v.y); v.z = fmaf(a, b.v.z, v.z); v.w = fmaf(a, b.v.w, v.w);
@@ -97,6 +105,7 @@ template <> struct Vec<1> {
         else *p = v;
     }
     __device__ __forceinline__ static Vec gload_clip(const float* row, int d, int) { return Vec{row[d]}; }
+    __device__ __forceinline__ void zero_first(int n) { v = n > 0 ? 0.f : v; }
     __device__ __forceinline__ void fma(float a, const Vec& b) { v = fmaf(a, b.v, v); }
     __device__ __forceinline__ void add(const Vec& b) { v += b.v; }
     __device__ __forceinline__ float dot(const Vec& b, float acc) const { return fmaf(v, b.v, acc); }
@@ -748,20 +757,30 @@ template <int VEC, int G, int V> __device__ __forceinline__ void slots_sum(Vec<V
 // One round: the lane group handling nonzero `n` of the chunk (column index fetched from lane n) reads
 // that rhs row against the lhs row and returns the group's dot product in all of its lanes.
 // MASKED: D is not G1*VEC*DS; lanes past D read a safe in-row address and contribute 0, the lane that straddles D
-// reads the row's last VEC floats with the overlap zeroed.
+// reads the row's last VEC floats with the overlap zeroed. All DS loads are issued first and the zeroing follows as
+// selects (where and how many elements: the same in every round, so the compiler keeps it outside the loop): zeroing
+// under a condition right behind each load made every load wait for the one before (D = 192 took 1.7 times the time
+// of D = 256). An access that lies past D for the whole wave is issued all the same (it reads the row's first floats
+// again): leaving it out under a branch cost 5-45 % at D = 132 ... 320, the wait for all loads then comes before the
+// first product.
 template <int VEC, int G1, int DS, bool MASKED>
 __device__ __forceinline__ void sddmm_rounds_load(int D, int g, const float* __restrict__ rhs, int cn, Vec<VEC>* x)
 {
     const float* rrow = rhs + (size_t)cn * D;
+    if constexpr (MASKED) {
+        int gone[DS];  // leading elements of the access that are not the lane's to add
 #pragma unroll
-    for (int s = 0; s < DS; ++s) {
-        const int d = (s * G1 + g) * VEC;
-        if constexpr (MASKED) {
-            x[s] = Vec<VEC>::gload_clip(rrow, d < D ? d : 0, D);
-            if (d >= D) x[s] = Vec<VEC>::zero();  // not 0 * (whatever sits at column 0): that could be 0 * inf
-        } else {
-            x[s] = Vec<VEC>::gload(rrow + d);
+        for (int s = 0; s < DS; ++s) {
+            const int d = (s * G1 + g) * VEC;
+            const int from = d < D ? min(d, D - VEC) : 0;
+            gone[s] = d < D ? d - from : VEC;  // (not 0 * whatever sits at column 0: that could be 0 * inf)
+            x[s] = Vec<VEC>::gload(rrow + from);
         }
+#pragma unroll
+        for (int s = 0; s < DS; ++s) x[s].zero_first(gone[s]);
+    } else {
+#pragma unroll
+        for (int s = 0; s < DS; ++s) x[s] = Vec<VEC>::gload(rrow + (s * G1 + g) * VEC);
     }
 }
 

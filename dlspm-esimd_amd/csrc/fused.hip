@@ -181,8 +181,11 @@ FusedShape fused_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
         if (D <= 16) { s.G1 = 4; s.DS = 1; s.G = 8; s.V = 1; }
         else if (D <= 32) { s.G1 = 8; s.DS = 1; s.G = 8; s.V = 1; }
         else if (D <= 64) { s.G1 = 8; s.DS = 2; s.G = 16; s.V = 1; }
+        else if (D <= 96) { s.G1 = 8; s.DS = 3; s.G = 32; s.V = 1; }
         else if (D <= 128) { s.G1 = 8; s.DS = 4; s.G = 32; s.V = 1; }
+        else if (D <= 192) { s.G1 = 8; s.DS = 6; s.G = 64; s.V = 1; }
         else if (D <= 256) { s.G1 = 8; s.DS = 8; s.G = 64; s.V = 1; }
+        else if (D <= 384) { s.G1 = 8; s.DS = 12; s.G = 64; s.V = 2; }
         else if (D <= 512) { s.G1 = 8; s.DS = 16; s.G = 64; s.V = 2; }
         else { s.G1 = 8; s.DS = 0; s.G = 64; s.V = 4; }  // wider D: column tiles of 1024, scores recomputed per tile
     } else {  // D < 4: one float per lane

@@ -22,14 +22,16 @@ using SpmmLayouts = std::tuple<RowLanes<4, 64, 2>, RowLanes<4, 64, 1>, RowLanes<
                                RowLanes<1, 8, 1>>;
 // SDDMM: floats per lane and access, lanes per dot product, accesses per lane (0: a run-time loop)
 template <int VEC_, int G1_, int DS_> struct DotLanes { static constexpr int VEC = VEC_, G1 = G1_, DS = DS_; };
-using SddmmLayouts = std::tuple<DotLanes<4, 4, 1>, DotLanes<4, 8, 1>, DotLanes<4, 8, 2>, DotLanes<4, 8, 4>, DotLanes<4, 8, 8>,
-                                DotLanes<4, 8, 16>, DotLanes<4, 8, 0>, DotLanes<1, 4, 1>>;
+using SddmmLayouts = std::tuple<DotLanes<4, 4, 1>, DotLanes<4, 8, 1>, DotLanes<4, 8, 2>, DotLanes<4, 8, 3>, DotLanes<4, 8, 4>,
+                                DotLanes<4, 8, 6>, DotLanes<4, 8, 8>, DotLanes<4, 8, 12>, DotLanes<4, 8, 16>, DotLanes<4, 8, 0>,
+                                DotLanes<1, 4, 1>>;
 // fused: both stages
 template <int VEC_, int G1_, int DS_, int G_, int V_> struct FusedLanes {
     static constexpr int VEC = VEC_, G1 = G1_, DS = DS_, G = G_, V = V_;
 };
-using FusedLayouts = std::tuple<FusedLanes<4, 4, 1, 8, 1>, FusedLanes<4, 8, 1, 8, 1>, FusedLanes<4, 8, 2, 16, 1>, FusedLanes<4, 8, 4, 32, 1>,
-                                FusedLanes<4, 8, 8, 64, 1>, FusedLanes<4, 8, 16, 64, 2>, FusedLanes<4, 8, 0, 64, 4>, FusedLanes<1, 4, 1, 8, 1>>;
+using FusedLayouts = std::tuple<FusedLanes<4, 4, 1, 8, 1>, FusedLanes<4, 8, 1, 8, 1>, FusedLanes<4, 8, 2, 16, 1>, FusedLanes<4, 8, 3, 32, 1>,
+                                FusedLanes<4, 8, 4, 32, 1>, FusedLanes<4, 8, 6, 64, 1>, FusedLanes<4, 8, 8, 64, 1>, FusedLanes<4, 8, 12, 64, 2>,
+                                FusedLanes<4, 8, 16, 64, 2>, FusedLanes<4, 8, 0, 64, 4>, FusedLanes<1, 4, 1, 8, 1>>;
 
 // launch(entry) for the first entry of Table that `match` accepts; hipErrorInvalidValue if there is none
 template <typename Table, typename Match, typename Launch> hipError_t dispatch(Match&& match, Launch&& launch)

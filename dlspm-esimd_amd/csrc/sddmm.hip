@@ -150,9 +150,17 @@ __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __
     }
 }
 
+// Eight accesses per lane and row of rhs (D = 129 ... 256): the compiler, aiming at eight waves per SIMD and their 64
+// registers, would issue the accesses of a round two at a time and wait for each pair; told that four waves per SIMD are
+// enough here, it issues all eight before the first wait (78 registers, six waves per SIMD). In a graph, before -> after:
+// D = 256, Bernoulli rows 1024 x 2304 12.3 -> 10.7 us, 8192 x 2048 21.5 -> 20.5 us, lognormal rows 1024 x 2304 44.2 -> 26.0 us,
+// 4096 x 4096 120 -> 70 us; one row per workgroup on rows of 100 nonzeros loses 6-10 % (2048 x 512 under a row plan 9.5 ->
+// 10.4 us). Sixteen accesses (D = 257 ... 512) are left as they were: 4096 x 4096 of 200 per row lost 20 % there.
+#define DLSPM_SDDMM_WAVES_PER_SIMD(DS) __attribute__((amdgpu_waves_per_eu(1, (DS) > 4 && (DS) <= 8 ? 4 : (DS) >= 12 ? 3 : 8)))
+
 // MASKED = false: D == G1 * VEC * DS exactly, every access of every lane falls inside the row.
 template <int VEC, int G1, int DS, bool MASKED, int W, int R>
-__global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, int flags, const int* __restrict__ row_offsets,
+__global__ __launch_bounds__(W * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_kernel(int M, int D, int flags, const int* __restrict__ row_offsets,
                                                        const int* __restrict__ col_indices,
                                                        const float* __restrict__ lhs, const float* __restrict__ rhs,
                                                        SampledOut out)
@@ -165,7 +173,7 @@ __global__ __launch_bounds__(W * 64) void sddmm_kernel(int M, int D, int flags, 
 // the rows of rhs gathered at any time come from one slice. Every result still goes to its own CSR slot: no partial
 // rows, no second pass, and the same bits as under any other schedule.
 template <int VEC, int G1, int DS, bool MASKED, int R>
-__global__ __launch_bounds__(4 * 64) void sddmm_sliced_kernel(int M, int D, int slice_blocks,
+__global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_sliced_kernel(int M, int D, int slice_blocks,
                                                               const int* __restrict__ bounds,
                                                               const int* __restrict__ col_indices,
                                                               const float* __restrict__ lhs,
@@ -181,7 +189,7 @@ __global__ __launch_bounds__(4 * 64) void sddmm_sliced_kernel(int M, int D, int 
 
 // Row plan: workgroup i works on the whole row rows[i] = [starts[i], ends[i]) (one row per four-wave workgroup).
 template <int VEC, int G1, int DS, bool MASKED>
-__global__ __launch_bounds__(4 * 64) void sddmm_planned_kernel(int M, int D, int nnz, int flags, const int* __restrict__ starts,
+__global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_planned_kernel(int M, int D, int nnz, int flags, const int* __restrict__ starts,
                                                                const int* __restrict__ ends, const int* __restrict__ rows,
                                                                const int* __restrict__ col_indices,
                                                                const float* __restrict__ lhs, const float* __restrict__ rhs,
@@ -195,7 +203,7 @@ __global__ __launch_bounds__(4 * 64) void sddmm_planned_kernel(int M, int D, int
 // slot_of[i] says which piece of how many: that share of the row's nonzeros, whose results go to their own CSR slots like
 // any others -- or nothing (an empty range).
 template <int VEC, int G1, int DS, bool MASKED>
-__global__ __launch_bounds__(4 * 64) void sddmm_pieces_kernel(int M, int D, int nnz, int flags, int slots, const int* __restrict__ starts,
+__global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_pieces_kernel(int M, int D, int nnz, int flags, int slots, const int* __restrict__ starts,
                                                               const int* __restrict__ ends, const int* __restrict__ rows,
                                                               const int* __restrict__ slot_of,
                                                               const int* __restrict__ col_indices,
@@ -248,7 +256,9 @@ SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
         if (D <= 16) { s.G1 = 4; s.DS = 1; }
         else {
             s.G1 = 8;
-            s.DS = D <= 32 ? 1 : D <= 64 ? 2 : D <= 128 ? 4 : D <= 256 ? 8 : D <= 512 ? 16 : 0;
+            // accesses of 32 floats per dot product: powers of two and the steps half-way between them (an access
+            // that lies past D is issued like the others)
+            s.DS = D <= 32 ? 1 : D <= 64 ? 2 : D <= 96 ? 3 : D <= 128 ? 4 : D <= 192 ? 6 : D <= 256 ? 8 : D <= 384 ? 12 : D <= 512 ? 16 : 0;
         }
     } else {  // D < 4: one float per lane
         s.G1 = 4;
@@ -268,13 +278,17 @@ SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
 // 192 rows 3.99 / 4.18 / 4.13; D = 256: 6.00 / 3.37 / 3.04, 7.13 / 4.00 / 4.41, 7.17 / 5.03 / 5.61, 7.18 / 6.12 / 7.37;
 // lognormal rows (sigma 0.8), D = 128: 6.03 / 2.81 / 2.64, 6.70 / 3.38 / 3.04, 6.74 / 4.47 / 3.58, 6.76 / 4.96 / 3.99
 // (a cut plan still cuts the longest rows finer); the reference's 128-row ResNet-50 layers (26 files): 3.80 / 3.28 / 3.31.
+// Between three quarters and one and a half of a compute unit's count of rows two four-wave workgroups share a row, which
+// fills the device evenly where one eight-wave workgroup per row leaves the last compute units with one row and the
+// others with two (four workgroups per row lose 3 ... 23 % on Bernoulli rows there).
 void sddmm_few_rows_pieces(const DeviceInfo& dev, SddmmShape& s, int M, int nnz)
 {
     s.pieces_lg = 0;
     if (!rule_on(kRuleRowPiecesFewRows) || s.R != 1 || s.W == 1 || tuning().split_w > 0 || M <= 0) return;
-    if (4ll * M > 3ll * dev.cus || (long long)nnz < 128ll * M) return;
+    if (2ll * M > 3ll * dev.cus || (long long)nnz < 128ll * M) return;
     int lg = 0;
     while (lg < kFlagPiecesMask && ((long long)M << lg) < 2ll * dev.cus && (long long)nnz >= (64ll << lg) * M) ++lg;
+    if (4ll * M > 3ll * dev.cus) lg = 1;
     if (lg == 0) return;
     s.pieces_lg = lg;
     s.W = 4;
@@ -294,7 +308,7 @@ hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t str
 // ---- flat schedule: every wave owns `chunk` consecutive nonzeros of the mask, whatever rows they belong to ---------
 // (see spmm.hip; here every result goes to its own CSR slot, so there is nothing to combine and no workspace)
 template <int VEC, int G1, int DS, bool MASKED>
-__global__ __launch_bounds__(kFlatWaves * 64) void sddmm_flat_kernel(int M, int D, int nnz, int chunk,
+__global__ __launch_bounds__(kFlatWaves * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_flat_kernel(int M, int D, int nnz, int chunk,
                                                                       const int* __restrict__ row_offsets,
                                                                       const int* __restrict__ col_indices,
                                                                       const float* __restrict__ lhs,

@@ -399,7 +399,8 @@ typedef struct dlspm_tuning {
 #define DLSPM_RULE_FINER_COLUMN_TILES         256  /* SpMM without memory or plan: narrower column tiles of B for few rows,   */
                                                    /* and for N above 512 in matrices of up to eight rows per compute unit   */
 #define DLSPM_RULE_ROW_PIECES_FEW_ROWS        512  /* SDDMM without memory or plan: several workgroups share each row of a   */
-                                                   /* mask of fewer rows than three quarters of the compute units           */
+                                                   /* mask of fewer rows than three quarters of the compute units, two up to */
+                                                   /* one and a half times their number                                      */
 void dlspm_tuning_default(dlspm_tuning* t);   /* fills *t with "follow the rules" */
 int dlspm_set_tuning(const dlspm_tuning* t);  /* DLSPM_OK or DLSPM_E_INVALID_ARG (a field out of range) */
 int dlspm_get_tuning(dlspm_tuning* t);        /* what the calling thread's launches currently use */

@@ -3,8 +3,8 @@
 
   * SpMM, finer column tiles of B (DLSPM_RULE_FINER_COLUMN_TILES): few rows at N = 64 ... 1024, and dense rows wider
     than 512 floats on 64 ... 8192 rows (where B exceeds the L2: every XCD on its own tiles);
-  * SDDMM, several workgroups per row of a mask of few rows (DLSPM_RULE_ROW_PIECES_FEW_ROWS), D = 32 ... 256, with the
-    time of the same launch under a cut plan beside it.
+  * SDDMM, several workgroups per row of a mask of few rows (DLSPM_RULE_ROW_PIECES_FEW_ROWS), 16 ... 384 rows, D = 32 ... 256,
+    with the time of the same launch under a cut plan beside it.
 
     python tests/plain_call_rules_sweep.py [--quick] [--out table.txt]
 
@@ -73,7 +73,7 @@ def main():
             f"off {t_off:8.2f} on {t_on:8.2f} us  {t_on / t_off:.2f}")
         groups.setdefault((f"spmm {group}", kind), []).append((t_off, t_on))
 
-    def sddmm_case(group, kind, M, K, per_row, D):
+    def sddmm_case(group, kind, M, K, per_row, D, rule="row_pieces_few_rows"):
         ro_h, ci_h = pattern(kind, M, K, per_row)
         nnz = int(ci_h.size)
         ro, ci = torch.from_numpy(ro_h).cuda(), torch.from_numpy(ci_h).cuda()
@@ -83,19 +83,19 @@ def main():
         on = dl.describe_launch(dl.OP_SDDMM, M, K, D, nnz)
         call()
         with_rule = out.clone()
-        dl.set_tuning(rules_off=dl.RULES["row_pieces_few_rows"])
+        dl.set_tuning(rules_off=dl.RULES[rule])
         out.fill_(float("nan"))
         call()
         assert torch.equal(out, with_rule), (kind, M, K, D)
         dl.set_tuning()
         graph_us(torch, call)
         t_on = graph_us(torch, call)
-        dl.set_tuning(rules_off=dl.RULES["row_pieces_few_rows"])
+        dl.set_tuning(rules_off=dl.RULES[rule])
         t_off = graph_us(torch, call)
         dl.set_tuning()
         plan = dl.cut_plan(ro, dl.OP_SDDMM, D)
         t_cut = graph_us(torch, lambda: call(plan=plan))
-        say(f"sddmm {kind} {M:5d} x {K:5d} {nnz:8d} nnz longest {int(np.diff(ro_h).max()):5d} D {D:5d}: {on['col_tiles']:3d} workgroups per row   "
+        say(f"sddmm {kind} {M:5d} x {K:5d} {nnz:8d} nnz longest {int(np.diff(ro_h).max()):5d} D {D:5d}: {on['col_tiles']:3d} workgroups per row of {on['W']} waves   "
             f"off {t_off:8.2f} on {t_on:8.2f} us  {t_on / t_off:.2f}   cut plan {t_cut:8.2f}")
         groups.setdefault((f"sddmm {group}", kind), []).append((t_off, t_on, t_cut))
 
@@ -113,7 +113,7 @@ def main():
         for M, K, per_row, N in (wide[::3] if args.quick else wide):
             spmm_case("dense rows wider than 512", kind, M, K, per_row, N)
     for kind in ("even", "logn"):
-        for M in few:
+        for M in few + ((256, 384) if not args.quick else (384,)):
             for K, per_row in shapes:
                 for D in (32, 64, 128, 256):
                     sddmm_case(f"{M} rows, D = {D}", kind, M, K, per_row, D)

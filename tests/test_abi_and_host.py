@@ -104,7 +104,8 @@ def test_split_rule_for_small_matrices(dl):
         assert dl.describe_launch(op, 128, 512, width, 128 * 26)["W"] == 4
         assert dl.describe_launch(op, 64, 576, width, 64 * 58)["W"] == 4
         eight = 4 if op == dl.OP_SPMM else 8  # SpMM: only by the rule for very long rows
-        assert dl.describe_launch(op, 256, 2304, width, 256 * 208)["W"] == eight
+        sh = dl.describe_launch(op, 256, 2304, width, 256 * 208)
+        assert (sh["W"], sh["col_tiles"]) == ((4, 2) if op == dl.OP_SDDMM else (eight, 1))  # SDDMM: two four-wave workgroups per row
         assert dl.describe_launch(op, 511, 2304, width, 511 * 96)["W"] == eight
         assert dl.describe_launch(op, 512, 2304, width, 512 * 208)["W"] == 4
     assert dl.describe_launch(dl.OP_SPMM, 256, 2304, 196, 256 * 461)["W"] == 8
@@ -183,11 +184,13 @@ def test_finer_column_tiles_for_plain_spmm_calls(dl):
 def test_row_pieces_for_plain_sddmm_calls_on_few_rows(dl):
     """SDDMM without plan or memory on a mask of at most three quarters of the compute units' count of rows: 2^k four-wave
     workgroups share each row, up to two workgroups per compute unit in all, each keeping 32 nonzeros of a mean row or
-    more; rows of 128 nonzeros and more on average only."""
+    more; up to one and a half of that count: two workgroups per row; rows of 128 nonzeros and more on average only."""
     pieces = lambda M, per_row, **kw: (lambda sh: (sh["W"], sh["col_tiles"]))(dl.describe_launch(dl.OP_SDDMM, M, 4608, 128, M * per_row, **kw))
     assert pieces(128, 300) == (4, 4) and pieces(64, 300) == (4, 8) and pieces(32, 300) == (4, 8)   # (8: 37 per workgroup)
     assert pieces(32, 600) == (4, 16) and pieces(1, 4608) == (4, 128) and pieces(192, 300) == (4, 4)
-    assert pieces(193, 300) == (8, 1)                      # more rows: eight waves per row as before
+    # up to one and a half of the compute units' count of rows: two workgroups per row; beyond, eight or four waves as before
+    assert pieces(193, 300) == (4, 2) and pieces(256, 300) == (4, 2) and pieces(384, 300) == (4, 2) and pieces(385, 300) == (8, 1)
+    assert pieces(300, 127) == (8, 1) and pieces(512, 300) == (4, 1)
     assert pieces(128, 127) == (8, 1) and pieces(128, 128) == (4, 4)
     assert pieces(128, 300, rows_even=True) == (4, 4)      # the hint is about the lengths of the rows, not their number
     assert pieces(128, 300, with_workspace=True) == (8, 1)

@@ -220,8 +220,15 @@ def test_cut_plan_sizes_and_advice(dl):
     assert dl.row_plan_advice(dl.OP_SDDMM, 128, 1152, 128, 29510, 455) == 0    # a quarter of 455 is below one and a half shares (174)
     assert dl.row_plan_advice(dl.OP_SDDMM, 128, 1152, 128, 29510, 1152) == 2
     assert dl.row_plan_advice(dl.OP_SDDMM, 64, 576, 128, 31919, 547) == 0
-    assert dl.row_plan_advice(dl.OP_SDDMM, 256, 2304, 128, 118041, 900) == 0   # 256 rows, longest below two shares: no
-    assert dl.row_plan_advice(dl.OP_SDDMM, 256, 2304, 128, 53000, 800) == 2    # ... of nearly four shares: yes
+    # three quarters to one and a half of the compute units' count of rows (two workgroups per row without plan): judged as
+    # whole rows, from a longest row of little more than one and a half shares on; up to two rows per compute unit
+    # (eight waves per row) from about two and a half shares on
+    assert dl.row_plan_advice(dl.OP_SDDMM, 256, 2304, 128, 118041, 750) == 0
+    assert dl.row_plan_advice(dl.OP_SDDMM, 256, 2304, 128, 118041, 900) == 2
+    assert dl.row_plan_advice(dl.OP_SDDMM, 384, 2304, 128, 118041, 900) == 2
+    assert dl.row_plan_advice(dl.OP_SDDMM, 385, 2304, 128, 118041, 900) == 0
+    assert dl.row_plan_advice(dl.OP_SDDMM, 385, 2304, 128, 118041, 1200) == 2
+    assert dl.row_plan_advice(dl.OP_SDDMM, 256, 2304, 128, 53000, 800) == 2
     assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 256, 29510, 455) == 0
     assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 256, 29510, 1152) == 2
     assert dl.row_plan_advice(dl.OP_SPMM, 128, 1152, 128, 29510, 455) == 0

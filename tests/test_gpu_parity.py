@@ -149,6 +149,42 @@ def test_sddmm_matches_oracle(torch_cuda, dl, oracle, M, K, D, kind, density):
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
+@pytest.mark.parametrize("D", [20, 68, 80, 96, 100, 132, 160, 192, 200, 224, 300, 320, 384, 500])
+@pytest.mark.parametrize("op", ["sddmm", "fused"])
+def test_widths_between_the_powers_of_two(torch_cuda, dl, oracle, op, D):
+    """Dot products of D floats are gathered in accesses of 32 floats per nonzero: 1, 2, 3, 4, 6, 8, 12 or 16 of them, the last
+    ones past D for some or all lanes. Those lanes add nothing, whatever the floats they re-read are: with an infinity
+    at the start of some rows of rhs (where such lanes read) and finite floats everywhere else in those columns' products,
+    every result is the oracle's -- infinite where the oracle's is, never a NaN out of 0 * inf."""
+    torch = torch_cuda
+    rng = np.random.default_rng(977 + D)
+    M, K = 300, 400
+    ro, ci = random_csr(rng, M, K, "uniform", 0.2)
+    lhs = rng.normal(0, 1, (M, D)).astype(np.float32)
+    rhs = rng.normal(0, 1, (K, D)).astype(np.float32)
+    lhs[:, 0] = np.abs(lhs[:, 0]) + 0.5  # a positive first factor: inf * it is +inf, nothing cancels
+    hot = rng.random(K) < 0.1
+    ro_d, ci_d = dev(torch, ro), dev(torch, ci)
+    for poisoned in (False, True):
+        if poisoned:
+            rhs[hot, 0] = np.inf
+        if op == "sddmm":
+            sh = dl.describe_launch(dl.OP_SDDMM, M, K, D, ci.size)
+            assert sh["DS"] == (1 if D <= 32 else next(n for n in (2, 3, 4, 6, 8, 12, 16) if D <= 32 * n))
+            got = dl.sddmm(ro_d, ci_d, dev(torch, lhs), dev(torch, rhs)).cpu().numpy()
+            with np.errstate(invalid="ignore", over="ignore"):
+                ref = oracle.sddmm(ro, ci, lhs, rhs)
+            assert not np.isnan(got).any()
+            inf = np.isinf(ref)
+            assert inf.any() == poisoned and np.array_equal(np.isinf(got), inf) and np.array_equal(got[inf], ref[inf])
+            assert oracle.rel_frobenius(got[~inf], ref[~inf]) <= TOL
+        elif not poisoned:  # (the fused op would add inf * V rows of both signs: its oracle holds NaN there)
+            V = rng.normal(0, 1, (K, D)).astype(np.float32)
+            got = dl.fused(ro_d, ci_d, dev(torch, lhs), dev(torch, rhs), dev(torch, V), scale=0.1).cpu().numpy()
+            assert oracle.rel_frobenius(got, oracle.fused(ro, ci, lhs, rhs, V, scale=0.1)) <= TOL
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
 FUSED_CASES = [
     (1, 1, 4, "full", 1.0, 1.0),
     (9, 11, 8, "uniform", 0.5, 1.0),
@@ -486,10 +522,11 @@ def test_finer_column_tiles_of_plain_spmm_calls(torch_cuda, dl, oracle, M, K, N,
 
 @pytest.mark.parametrize("M,K,D,per_row,pieces", [
     (128, 1152, 128, 230, 4), (16, 576, 64, 400, 8), (1, 700, 256, 700, 16), (64, 4608, 100, 1400, 8), (192, 2304, 32, 230, 4),
-    (7, 300, 16, 140, 4), (100, 512, 128, 60, 1), (193, 2304, 128, 230, 1)])
+    (7, 300, 16, 140, 4), (100, 512, 128, 60, 1), (193, 2304, 128, 230, 2), (384, 576, 256, 300, 2), (385, 2304, 128, 230, 1)])
 @pytest.mark.parametrize("sigma", [0.0, 0.8])
 def test_row_pieces_of_plain_sddmm_calls_on_few_rows(torch_cuda, dl, oracle, M, K, D, per_row, pieces, sigma):
-    """Few rows: 2, 4, ... 16 workgroups share each row of a SDDMM call without plan or memory. Every result is still
+    """Few rows: 2, 4, ... 16 workgroups share each row of a SDDMM call without plan or memory (two from three quarters to
+    one and a half of the compute units' count of rows). Every result is still
     one nonzero's own dot product: the bits of the same call with the rule switched off, and the oracle's values."""
     torch = torch_cuda
     if sigma == 0.0:

@@ -80,7 +80,7 @@ def main():
     for case in range(args.cases):
         M = int(rng.choice([1, 2, 7, 63, 64, 65, 200, 700, 2047, 2500, 9000])) + int(rng.integers(0, 5))
         K = int(rng.choice([1, 3, 64, 130, 500, 1500, 2100, 4200, 20000])) + int(rng.integers(0, 5))
-        N = int(rng.choice([1, 2, 3, 5, 16, 33, 49, 64, 65, 100, 128, 129, 196, 256, 257, 392, 512, 513, 700, 1030]))
+        N = int(rng.choice([1, 2, 3, 5, 16, 33, 49, 64, 65, 96, 100, 128, 129, 192, 196, 256, 257, 384, 392, 512, 513, 700, 1030]))
         kind = str(rng.choice(["uniform", "skewed", "empty_rows", "full"]))
         density = float(rng.choice([0.005, 0.02, 0.1, 0.3]))
         if kind == "full" and M * K > 300000:
