@@ -150,12 +150,15 @@ __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __
     }
 }
 
-// Eight accesses per lane and row of rhs (D = 129 ... 256): the compiler, aiming at eight waves per SIMD and their 64
-// registers, would issue the accesses of a round two at a time and wait for each pair; told that four waves per SIMD are
-// enough here, it issues all eight before the first wait (78 registers, six waves per SIMD). In a graph, before -> after:
+// Five and more accesses per lane and row of rhs (D = 129 ... 512): the compiler, aiming at eight waves per SIMD and their 64
+// registers, would issue the accesses of a round two or three at a time and wait for each group; told that four waves
+// per SIMD are enough (three from twelve accesses on), it issues all of them before the first wait (D = 256: 78 registers,
+// six waves per SIMD; D = 384: 110; D = 512: four waves). In a graph, before -> after:
 // D = 256, Bernoulli rows 1024 x 2304 12.3 -> 10.7 us, 8192 x 2048 21.5 -> 20.5 us, lognormal rows 1024 x 2304 44.2 -> 26.0 us,
 // 4096 x 4096 120 -> 70 us; one row per workgroup on rows of 100 nonzeros loses 6-10 % (2048 x 512 under a row plan 9.5 ->
-// 10.4 us). Sixteen accesses (D = 257 ... 512) are left as they were: 4096 x 4096 of 200 per row lost 20 % there.
+// 10.4 us). D = 512: lognormal rows 0.58-1.03 of the time (0.84 in the mean), Bernoulli rows 0.92-1.12 (0.99; 4096 x 4096 of
+// 200 per row, rhs of twice the L2, 81 -> 91 us). D = 384 with twelve accesses at the compiler's own choice took longer
+// than D = 512 where rhs exceeds the L2 (512 x 4608 of 1380 per row: 69 against 57 us; with all twelve in flight 39 us).
 #define DLSPM_SDDMM_WAVES_PER_SIMD(DS) __attribute__((amdgpu_waves_per_eu(1, (DS) > 4 && (DS) <= 8 ? 4 : (DS) >= 12 ? 3 : 8)))
 
 // MASKED = false: D == G1 * VEC * DS exactly, every access of every lane falls inside the row.
@@ -273,14 +276,15 @@ SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
 // row's passes in turn exactly as the waves of one workgroup do (sddmm_row_interleaved), every result is still one
 // nonzero's own dot product, and nothing else changes: no plan, no second kernel, the same bits. Up to three quarters of
 // a compute unit's count of rows, rows of 128 nonzeros and more on average, and a workgroup keeps at least 32 of a mean row.
-// Measured (us inside a graph, rule off / on / with a cut plan; Bernoulli rows, geometric means over five shapes of 300 ...
-// 1400 nonzeros per row): D = 128: 16 rows 3.75 / 2.59 / 2.62, 64 rows 3.84 / 3.01 / 3.04, 128 rows 3.90 / 3.53 / 3.53,
-// 192 rows 3.99 / 4.18 / 4.13; D = 256: 6.00 / 3.37 / 3.04, 7.13 / 4.00 / 4.41, 7.17 / 5.03 / 5.61, 7.18 / 6.12 / 7.37;
-// lognormal rows (sigma 0.8), D = 128: 6.03 / 2.81 / 2.64, 6.70 / 3.38 / 3.04, 6.74 / 4.47 / 3.58, 6.76 / 4.96 / 3.99
+// Measured (us inside a graph, rule off / on / with a cut plan; Bernoulli rows, geometric means over four shapes of 230 ...
+// 1380 nonzeros per row): D = 128: 16 rows 4.04 / 2.60 / 2.63, 64 rows 4.14 / 3.09 / 3.08, 128 rows 4.22 / 3.69 / 3.65,
+// 192 rows 4.30 / 4.49 / 4.43; D = 256: 6.71 / 3.01 / 2.83, 8.29 / 3.89 / 4.04, 8.36 / 5.08 / 5.09, 8.33 / 6.49 / 6.64;
+// lognormal rows (sigma 0.8), D = 128: 6.36 / 2.84 / 2.64, 7.60 / 3.72 / 3.16, 8.05 / 4.84 / 3.72, 8.14 / 5.83 / 4.27
 // (a cut plan still cuts the longest rows finer); the reference's 128-row ResNet-50 layers (26 files): 3.80 / 3.28 / 3.31.
 // Between three quarters and one and a half of a compute unit's count of rows two four-wave workgroups share a row, which
 // fills the device evenly where one eight-wave workgroup per row leaves the last compute units with one row and the
-// others with two (four workgroups per row lose 3 ... 23 % on Bernoulli rows there).
+// others with two (four workgroups per row lose 3 ... 23 % on Bernoulli rows there): 256 rows, D = 128, 4.61 / 4.74 / 5.20 and
+// lognormal 8.76 / 7.82 / 4.94; 384 rows 6.54 / 5.95 / 6.17 and 11.37 / 9.06 / 6.09; D = 256: 0.84 ... 0.87 and 0.69 ... 0.71 of the time.
 void sddmm_few_rows_pieces(const DeviceInfo& dev, SddmmShape& s, int M, int nnz)
 {
     s.pieces_lg = 0;
