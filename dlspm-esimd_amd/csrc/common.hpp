@@ -111,6 +111,10 @@ template <> struct Vec<1> {
     __device__ __forceinline__ float dot(const Vec& b, float acc) const { return fmaf(v, b.v, acc); }
 };
 
+// arguments of amdgpu_waves_per_eu for a kernel of `waves` waves per workgroup (four SIMDs per compute unit)
+constexpr int waves_per_simd_least(int waves) { return waves > 4 ? (waves + 3) / 4 : 1; }
+constexpr int waves_per_simd_most(int waves, int wanted) { return wanted > waves_per_simd_least(waves) ? wanted : waves_per_simd_least(waves); }
+
 // ---- cross-lane ---------------------------------------------------------------------------------
 // value of `x` in lane `src` (any lane of the wave), through the LDS crossbar (ds_bpermute_b32)
 __device__ __forceinline__ int lane_get(int x, int src) { return __builtin_amdgcn_ds_bpermute(src << 2, x); }

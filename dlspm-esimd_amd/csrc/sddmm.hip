@@ -159,11 +159,15 @@ __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __
 // 10.4 us). D = 512: lognormal rows 0.58-1.03 of the time (0.84 in the mean), Bernoulli rows 0.92-1.12 (0.99; 4096 x 4096 of
 // 200 per row, rhs of twice the L2, 81 -> 91 us). D = 384 with twelve accesses at the compiler's own choice took longer
 // than D = 512 where rhs exceeds the L2 (512 x 4608 of 1380 per row: 69 against 57 us; with all twelve in flight 39 us).
-#define DLSPM_SDDMM_WAVES_PER_SIMD(DS) __attribute__((amdgpu_waves_per_eu(1, (DS) > 4 && (DS) <= 8 ? 4 : (DS) >= 12 ? 3 : 8)))
+// (W: waves per workgroup. The least number of waves per SIMD that the attribute names must not be below what one workgroup
+// puts there, or the compiler drops the attribute -- eight-wave workgroups, lognormal rows on 448 rows, D = 256 ... 512: 12-19 %
+// faster with it kept --; and the largest not below the least.)
+#define DLSPM_SDDMM_WAVES_PER_SIMD(DS, W) \
+    __attribute__((amdgpu_waves_per_eu(waves_per_simd_least(W), waves_per_simd_most(W, (DS) > 4 && (DS) <= 8 ? 4 : (DS) >= 12 ? 3 : 8))))
 
 // MASKED = false: D == G1 * VEC * DS exactly, every access of every lane falls inside the row.
 template <int VEC, int G1, int DS, bool MASKED, int W, int R>
-__global__ __launch_bounds__(W * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_kernel(int M, int D, int flags, const int* __restrict__ row_offsets,
+__global__ __launch_bounds__(W * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, W) void sddmm_kernel(int M, int D, int flags, const int* __restrict__ row_offsets,
                                                        const int* __restrict__ col_indices,
                                                        const float* __restrict__ lhs, const float* __restrict__ rhs,
                                                        SampledOut out)
@@ -176,7 +180,7 @@ __global__ __launch_bounds__(W * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_k
 // the rows of rhs gathered at any time come from one slice. Every result still goes to its own CSR slot: no partial
 // rows, no second pass, and the same bits as under any other schedule.
 template <int VEC, int G1, int DS, bool MASKED, int R>
-__global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_sliced_kernel(int M, int D, int slice_blocks,
+__global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, 4) void sddmm_sliced_kernel(int M, int D, int slice_blocks,
                                                               const int* __restrict__ bounds,
                                                               const int* __restrict__ col_indices,
                                                               const float* __restrict__ lhs,
@@ -192,7 +196,7 @@ __global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_s
 
 // Row plan: workgroup i works on the whole row rows[i] = [starts[i], ends[i]) (one row per four-wave workgroup).
 template <int VEC, int G1, int DS, bool MASKED>
-__global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_planned_kernel(int M, int D, int nnz, int flags, const int* __restrict__ starts,
+__global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, 4) void sddmm_planned_kernel(int M, int D, int nnz, int flags, const int* __restrict__ starts,
                                                                const int* __restrict__ ends, const int* __restrict__ rows,
                                                                const int* __restrict__ col_indices,
                                                                const float* __restrict__ lhs, const float* __restrict__ rhs,
@@ -206,7 +210,7 @@ __global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_p
 // slot_of[i] says which piece of how many: that share of the row's nonzeros, whose results go to their own CSR slots like
 // any others -- or nothing (an empty range).
 template <int VEC, int G1, int DS, bool MASKED>
-__global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_pieces_kernel(int M, int D, int nnz, int flags, int slots, const int* __restrict__ starts,
+__global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, 4) void sddmm_pieces_kernel(int M, int D, int nnz, int flags, int slots, const int* __restrict__ starts,
                                                               const int* __restrict__ ends, const int* __restrict__ rows,
                                                               const int* __restrict__ slot_of,
                                                               const int* __restrict__ col_indices,
@@ -278,13 +282,13 @@ SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
 // a compute unit's count of rows, rows of 128 nonzeros and more on average, and a workgroup keeps at least 32 of a mean row.
 // Measured (us inside a graph, rule off / on / with a cut plan; Bernoulli rows, geometric means over four shapes of 230 ...
 // 1380 nonzeros per row): D = 128: 16 rows 4.04 / 2.60 / 2.63, 64 rows 4.14 / 3.09 / 3.08, 128 rows 4.22 / 3.69 / 3.65,
-// 192 rows 4.30 / 4.49 / 4.43; D = 256: 6.71 / 3.01 / 2.83, 8.29 / 3.89 / 4.04, 8.36 / 5.08 / 5.09, 8.33 / 6.49 / 6.64;
+// 192 rows 4.30 / 4.49 / 4.43; D = 256: 5.81 / 3.00 / 2.83, 6.38 / 3.91 / 4.07, 6.45 / 5.05 / 5.07, 6.48 / 6.47 / 6.63;
 // lognormal rows (sigma 0.8), D = 128: 6.36 / 2.84 / 2.64, 7.60 / 3.72 / 3.16, 8.05 / 4.84 / 3.72, 8.14 / 5.83 / 4.27
 // (a cut plan still cuts the longest rows finer); the reference's 128-row ResNet-50 layers (26 files): 3.80 / 3.28 / 3.31.
 // Between three quarters and one and a half of a compute unit's count of rows two four-wave workgroups share a row, which
 // fills the device evenly where one eight-wave workgroup per row leaves the last compute units with one row and the
 // others with two (four workgroups per row lose 3 ... 23 % on Bernoulli rows there): 256 rows, D = 128, 4.61 / 4.74 / 5.20 and
-// lognormal 8.76 / 7.82 / 4.94; 384 rows 6.54 / 5.95 / 6.17 and 11.37 / 9.06 / 6.09; D = 256: 0.84 ... 0.87 and 0.69 ... 0.71 of the time.
+// lognormal 8.76 / 7.82 / 4.94; 384 rows 6.54 / 5.95 / 6.17 and 11.37 / 9.06 / 6.09; D = 256: 1.02 and 0.86 of the time, lognormal 0.86 and 0.78.
 void sddmm_few_rows_pieces(const DeviceInfo& dev, SddmmShape& s, int M, int nnz)
 {
     s.pieces_lg = 0;
@@ -312,7 +316,7 @@ hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t str
 // ---- flat schedule: every wave owns `chunk` consecutive nonzeros of the mask, whatever rows they belong to ---------
 // (see spmm.hip; here every result goes to its own CSR slot, so there is nothing to combine and no workspace)
 template <int VEC, int G1, int DS, bool MASKED>
-__global__ __launch_bounds__(kFlatWaves * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS) void sddmm_flat_kernel(int M, int D, int nnz, int chunk,
+__global__ __launch_bounds__(kFlatWaves * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, kFlatWaves) void sddmm_flat_kernel(int M, int D, int nnz, int chunk,
                                                                       const int* __restrict__ row_offsets,
                                                                       const int* __restrict__ col_indices,
                                                                       const float* __restrict__ lhs,
