@@ -425,7 +425,7 @@ int dlspm_set_tuning(const dlspm_tuning* t)
         t->tile_major < -1 || t->tile_major > 3 || t->tile_width < 0 || t->plan_order < 0 || t->plan_order > 2 ||
         t->xcd_contiguous < 0 || t->xcd_contiguous > 1 || t->stream_results < -1 || t->stream_results > 1 ||
         (t->cut_piece_pct != 0 && (t->cut_piece_pct < 10 || t->cut_piece_pct > 1000)) ||
-        (t->cut_longest_pct != 0 && (t->cut_longest_pct < 10 || t->cut_longest_pct > 1000)) || t->rules_off < 0 || t->rules_off > 1023 ||
+        (t->cut_longest_pct != 0 && (t->cut_longest_pct < 10 || t->cut_longest_pct > 1000)) || t->rules_off < 0 || t->rules_off > 2047 ||
         (t->compute_units != 0 && (t->compute_units < 8 || t->compute_units > 1024 || t->compute_units % 8 != 0)))
         return DLSPM_E_INVALID_ARG;
     t_tuning.split_w = t->split_w;

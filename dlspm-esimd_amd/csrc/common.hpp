@@ -767,11 +767,25 @@ template <int VEC, int G, int V> __device__ __forceinline__ void slots_sum(Vec<V
 // of D = 256). An access that lies past D for the whole wave is issued all the same (it reads the row's first floats
 // again): leaving it out under a branch cost 5-45 % at D = 132 ... 320, the wait for all loads then comes before the
 // first product.
-template <int VEC, int G1, int DS, bool MASKED>
+// MASKED == kMaskedByRange (D a multiple of four, rhs of at most 1 GiB and fewer than 2^24 rows: the host checks): rhs is
+// read as a raw buffer of 1 GiB, and a lane whose floats lie past D adds 3 GiB to its offset -- out of the buffer's
+// range, for which the load returns zeros without touching memory. No select, no second address, and 0 * 0 where the
+// other kind must keep 0 * (whatever it re-read) out of the sum.
+constexpr int kExactWidth = 0, kMaskedBySelect = 1, kMaskedByRange = 2;
+constexpr unsigned kRangeWindowBytes = 1u << 30, kRangeOutside = 3u << 30;
+template <int VEC, int G1, int DS, int MASKED>
 __device__ __forceinline__ void sddmm_rounds_load(int D, int g, const float* __restrict__ rhs, int cn, Vec<VEC>* x)
 {
     const float* rrow = rhs + (size_t)cn * D;
-    if constexpr (MASKED) {
+    if constexpr (MASKED == kMaskedByRange) {
+        const __amdgpu_buffer_rsrc_t window = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(rhs), 0, (int)kRangeWindowBytes, 0x00020000);
+        const unsigned row = __umul24((unsigned)cn, (unsigned)D * (unsigned)sizeof(float));
+#pragma unroll
+        for (int s = 0; s < DS; ++s) {
+            const int d = (s * G1 + g) * VEC;
+            x[s] = Vec<VEC>::bload(window, row + (d < D ? (unsigned)d * (unsigned)sizeof(float) : kRangeOutside), 0u);
+        }
+    } else if constexpr (MASKED) {
         int gone[DS];  // leading elements of the access that are not the lane's to add
 #pragma unroll
         for (int s = 0; s < DS; ++s) {
@@ -792,7 +806,7 @@ __device__ __forceinline__ void sddmm_rounds_load(int D, int g, const float* __r
 // (lanes past the chunk return an unspecified value that the caller must not store). `c` is the lane's
 // column index (0 past the chunk). `lq` holds the lhs row as laid out by the caller:
 // lq[s] = lhs_row[(s*G1 + g)*VEC ..] (Vec::gload_clip), zero past D. With DS = 0 the row is re-read from lhs_row.
-template <int VEC, int G1, int DS, bool MASKED>
+template <int VEC, int G1, int DS, int MASKED>
 __device__ __forceinline__ float sddmm_chunk(int D, int lane, int cnt, int c, const float* __restrict__ lhs_row,
                                              const Vec<VEC>* lq, const float* __restrict__ rhs)
 {

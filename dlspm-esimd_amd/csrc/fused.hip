@@ -20,7 +20,7 @@ namespace dlspm {
 
 // acc[v] = sum over the nonzeros [p, q) of one mask row (p < q, wave-uniform) of scale * <q_row, Kmat[column]> *
 // Vmat[column, colv[v] ..], summed over the wave's slots so that every lane ends with the total.
-template <int VEC, int G1, int DS, bool MASKED, int G, int V2>
+template <int VEC, int G1, int DS, int MASKED, int G, int V2>
 __device__ __forceinline__ void fused_segment(Vec<VEC>* acc, int p, int q, int D, float scale,
                                               const int* __restrict__ col_indices, const float* __restrict__ q_row,
                                               const float* __restrict__ Kmat, const float* __restrict__ Vmat,
@@ -57,7 +57,7 @@ __device__ __forceinline__ void fused_segment(Vec<VEC>* acc, int p, int q, int D
 // The work of workgroup `bid` (RowBlock in common.hpp explains SLICED and PLANNED: with PLANNED workgroup i works on row
 // row_ids[i] of Q, O and the mask). Column tiles (D > 1024) tile-major, as in spmm_block; no division in the usual
 // case of one tile.
-template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R, bool SLICED, int PLANNED = kPlanNone>
+template <int VEC, int G1, int DS, int MASKED, int G, int V2, int W, int R, bool SLICED, int PLANNED = kPlanNone>
 __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles, float scale,
                                             const int* __restrict__ row_offsets, const int* __restrict__ row_ends,
                                             const int* __restrict__ col_indices, const float* __restrict__ Q,
@@ -85,7 +85,7 @@ __device__ __forceinline__ void fused_block(int bid, int M, int D, int col_tiles
 // them in flight -- three waves per SIMD -- Bernoulli rows lost 6 % at D = 384 and up to 23 % at D = 512 (1024 x 2304 of 230 per
 // row: 47.5 -> 57.6 us), lognormal rows gained 0-11 %.)
 // MASKED = false: D == G1 * VEC * DS exactly, every stage-1 access of every lane falls inside the row.
-template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int W, int R>
+template <int VEC, int G1, int DS, int MASKED, int G, int V2, int W, int R>
 __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_tiles, int flags, float scale,
                                                        const int* __restrict__ row_offsets,
                                                        const int* __restrict__ col_indices,
@@ -98,7 +98,7 @@ __global__ __launch_bounds__(W * 64) void fused_kernel(int M, int D, int col_til
 
 // Column-sliced schedule (see spmm_sliced_kernel): the row blocks once per slice of columns, slice after slice, so
 // that the rows of Kmat and V gathered at any time come from one slice; partial[s][i][:] is row i's share of slice s.
-template <int VEC, int G1, int DS, bool MASKED, int G, int V2, int R>
+template <int VEC, int G1, int DS, int MASKED, int G, int V2, int R>
 __global__ __launch_bounds__(4 * 64) void fused_sliced_kernel(int M, int D, int col_tiles, int slice_blocks, float scale,
                                                               const int* __restrict__ bounds,
                                                               const int* __restrict__ col_indices,
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(4 * 64) void fused_sliced_kernel(int M, int D, int 
 
 // Row plan: workgroup i works on the whole row rows[i] = [starts[i], ends[i]) (one row per four-wave workgroup, one
 // column tile).
-template <int VEC, int G1, int DS, bool MASKED, int G, int V2>
+template <int VEC, int G1, int DS, int MASKED, int G, int V2>
 __global__ __launch_bounds__(4 * 64) void fused_planned_kernel(int M, int D, int nnz, int flags, float scale,
                                                                const int* __restrict__ starts, const int* __restrict__ ends,
                                                                const int* __restrict__ rows,
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(4 * 64) void fused_planned_kernel(int M, int D, int
 
 // Row plan with cut rows (see spmm_pieces_kernel): entry i is the whole row rows[i], a piece of it whose partial row of O
 // goes to pieces[slot_of[i]], or nothing.
-template <int VEC, int G1, int DS, bool MASKED, int G, int V2>
+template <int VEC, int G1, int DS, int MASKED, int G, int V2>
 __global__ __launch_bounds__(4 * 64) void fused_pieces_kernel(int M, int D, int nnz, int flags, int slots, float scale,
                                                               const int* __restrict__ starts, const int* __restrict__ ends,
                                                               const int* __restrict__ rows, const int* __restrict__ slot_of,
@@ -226,7 +226,7 @@ hipError_t fused_launch(const FusedArgs& x, const FusedShape& s, hipStream_t str
 }
 
 // ---- flat schedule (see spmm.hip): every wave owns `chunk` consecutive nonzeros of the mask ------------------------
-template <int VEC, int G1, int DS, bool MASKED, int G, int V2>
+template <int VEC, int G1, int DS, int MASKED, int G, int V2>
 __global__ __launch_bounds__(kFlatWaves * 64) void fused_flat_kernel(int M, int D, int nnz, int chunk, int col_tiles,
                                                                       float scale, const int* __restrict__ row_offsets,
                                                                       const int* __restrict__ col_indices,

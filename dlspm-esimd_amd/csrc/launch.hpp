@@ -101,7 +101,7 @@ struct Tuning {
 // (the values of DLSPM_RULE_* in the header)
 constexpr int kRuleEightWavesFewRows = 1, kRuleSixteenWavesTallLongRows = 2, kRuleMoreWavesFewLongRows = 4, kRuleGroupRows = 8,
               kRuleRowAlignedSplit = 16, kRulePlanUngroups = 32, kRuleExactWidthKernels = 64, kRuleCutRowsByColumns = 128,
-              kRuleFinerColumnTiles = 256, kRuleRowPiecesFewRows = 512;
+              kRuleFinerColumnTiles = 256, kRuleRowPiecesFewRows = 512, kRuleMaskByRange = 1024;
 
 const Tuning& tuning();
 inline bool rule_on(int rule) { return (tuning().rules_off & rule) == 0; }

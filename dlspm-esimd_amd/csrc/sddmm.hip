@@ -47,7 +47,7 @@ static inline SampledOut sampled_out(const SddmmArgs& x)
 }
 
 // out[j] = <lhs_row, rhs[col_indices[j]]> for the nonzeros j in [p, q) of one row (p < q, wave-uniform).
-template <int VEC, int G1, int DS, bool MASKED>
+template <int VEC, int G1, int DS, int MASKED>
 __device__ __forceinline__ void sddmm_segment(int p, int q, int D, const int* __restrict__ col_indices,
                                               const float* __restrict__ lhs_row, const float* __restrict__ rhs,
                                               SampledOut out, int lane)
@@ -83,7 +83,7 @@ __device__ __forceinline__ void sddmm_segment(int p, int q, int D, const int* __
 // Every result is one nonzero's own dot product, so which wave computes it changes no bit.
 // Measured (D = 128, in a graph, even split -> this): lognormal rows with a row plan, 2048 x 2048 8.6 -> 7.9 us, 16384 x 4096
 // 39.4 -> 32.9 us; 2048 x 512 with 51 per row 4.95 -> 4.16 us.
-template <int VEC, int G1, int DS, bool MASKED>
+template <int VEC, int G1, int DS, int MASKED>
 __device__ __forceinline__ void sddmm_row_interleaved(int p, int q, int w, int W, int D, const int* __restrict__ col_indices,
                                                       const float* __restrict__ lhs_row, const float* __restrict__ rhs,
                                                       SampledOut out, int lane, bool full_passes)
@@ -121,7 +121,7 @@ __device__ __forceinline__ void sddmm_row_interleaved(int p, int q, int w, int W
 // The work of workgroup `bid` (RowBlock in common.hpp explains SLICED and PLANNED; a segment's results go where its
 // nonzeros lie, so a sliced or planned launch writes the same slots as any other). This kernel has neither LDS nor a
 // barrier.
-template <int VEC, int G1, int DS, bool MASKED, int W, int R, bool SLICED, int PLANNED = kPlanNone>
+template <int VEC, int G1, int DS, int MASKED, int W, int R, bool SLICED, int PLANNED = kPlanNone>
 __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __restrict__ row_offsets,
                                             const int* __restrict__ row_ends, const int* __restrict__ col_indices,
                                             const float* __restrict__ lhs, const float* __restrict__ rhs,
@@ -166,7 +166,7 @@ __device__ __forceinline__ void sddmm_block(int bid, int M, int D, const int* __
     __attribute__((amdgpu_waves_per_eu(waves_per_simd_least(W), waves_per_simd_most(W, (DS) > 4 && (DS) <= 8 ? 4 : (DS) >= 12 ? 3 : 8))))
 
 // MASKED = false: D == G1 * VEC * DS exactly, every access of every lane falls inside the row.
-template <int VEC, int G1, int DS, bool MASKED, int W, int R>
+template <int VEC, int G1, int DS, int MASKED, int W, int R>
 __global__ __launch_bounds__(W * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, W) void sddmm_kernel(int M, int D, int flags, const int* __restrict__ row_offsets,
                                                        const int* __restrict__ col_indices,
                                                        const float* __restrict__ lhs, const float* __restrict__ rhs,
@@ -179,7 +179,7 @@ __global__ __launch_bounds__(W * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, W) void sddm
 // Column-sliced schedule (see spmm_sliced_kernel): the row blocks once per slice of columns, slice after slice, so that
 // the rows of rhs gathered at any time come from one slice. Every result still goes to its own CSR slot: no partial
 // rows, no second pass, and the same bits as under any other schedule.
-template <int VEC, int G1, int DS, bool MASKED, int R>
+template <int VEC, int G1, int DS, int MASKED, int R>
 __global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, 4) void sddmm_sliced_kernel(int M, int D, int slice_blocks,
                                                               const int* __restrict__ bounds,
                                                               const int* __restrict__ col_indices,
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, 4) void sddm
 // ---- host side --------------------------------------------------------------------------------------
 
 // Row plan: workgroup i works on the whole row rows[i] = [starts[i], ends[i]) (one row per four-wave workgroup).
-template <int VEC, int G1, int DS, bool MASKED>
+template <int VEC, int G1, int DS, int MASKED>
 __global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, 4) void sddmm_planned_kernel(int M, int D, int nnz, int flags, const int* __restrict__ starts,
                                                                const int* __restrict__ ends, const int* __restrict__ rows,
                                                                const int* __restrict__ col_indices,
@@ -209,7 +209,7 @@ __global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, 4) void sddm
 // Row plan with cut rows: entry i is a whole row (slot_of[i] == -1), a piece of one -- entered with its row's whole range,
 // slot_of[i] says which piece of how many: that share of the row's nonzeros, whose results go to their own CSR slots like
 // any others -- or nothing (an empty range).
-template <int VEC, int G1, int DS, bool MASKED>
+template <int VEC, int G1, int DS, int MASKED>
 __global__ __launch_bounds__(4 * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, 4) void sddmm_pieces_kernel(int M, int D, int nnz, int flags, int slots, const int* __restrict__ starts,
                                                               const int* __restrict__ ends, const int* __restrict__ rows,
                                                               const int* __restrict__ slot_of,
@@ -229,6 +229,19 @@ static int sddmm_flags(const SddmmArgs& x, long long entries)
     return launch_flags(x.xcd_contiguous) | (entries >= 2ll * x.cus ? kFlagFullPasses : 0);
 }
 
+// Whether the kernels that mask by the range of a buffer apply (sddmm_rounds_load): D a multiple of four, up to twelve
+// accesses per lane (D <= 384), rhs within the window. Against the kernels that mask by selects (Bernoulli / lognormal rows, 20
+// shapes of 128 ... 16384 rows, geometric means): D = 80 0.96 / 0.92 of the time, D = 100 0.89 / 0.80, D = 160 0.95 / 0.91, D = 224
+// 0.94 / 0.90, D = 320 0.90 / 0.88; with sixteen accesses (D = 448) 0.75 ... 1.5, which stay with the selects. The kernels of
+// the column-sliced and the flat schedule, and the fused op's, mask by selects at every width.
+template <int DS> static bool masked_by_range(int K, int D)
+{
+    return DS >= 1 && DS <= 12 && D % 4 == 0 && K < (1 << 24) &&
+           (long long)K * D * (long long)sizeof(float) <= (long long)kRangeWindowBytes && rule_on(kRuleMaskByRange);
+}
+// (the kind to instantiate: no range kernels where masked_by_range<DS> never says so)
+template <int DS> constexpr int masked_kind(bool by_range) { return by_range && DS >= 1 && DS <= 12 ? kMaskedByRange : kMaskedBySelect; }
+
 template <int VEC, int G1, int DS, int W, int R>
 static hipError_t launch_one(const SddmmArgs& x, int pieces_lg, hipStream_t stream)
 {
@@ -239,12 +252,19 @@ static hipError_t launch_one(const SddmmArgs& x, int pieces_lg, hipStream_t stre
     const int flags = pieces_lg > 0 ? (sddmm_flags(x, x.M) & ~kFlagXcdContiguous) | (pieces_lg << kFlagPiecesShift) : sddmm_flags(x, x.M);
     if constexpr (DS > 0) {
         if (x.D == G1 * VEC * DS && rule_on(kRuleExactWidthKernels)) {
-            hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, false, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M,
+            hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, kExactWidth, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M,
                                x.D, flags, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
             return hipGetLastError();
         }
     }
-    hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, true, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M, x.D,
+    if constexpr (VEC == 4 && G1 == 8 && DS >= 1 && DS <= 12) {
+        if (masked_by_range<DS>(x.K, x.D)) {
+            hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, kMaskedByRange, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M, x.D,
+                               flags, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, kMaskedBySelect, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M, x.D,
                        flags, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     return hipGetLastError();
 }
@@ -315,7 +335,7 @@ hipError_t sddmm_launch(const SddmmArgs& x, const SddmmShape& s, hipStream_t str
 
 // ---- flat schedule: every wave owns `chunk` consecutive nonzeros of the mask, whatever rows they belong to ---------
 // (see spmm.hip; here every result goes to its own CSR slot, so there is nothing to combine and no workspace)
-template <int VEC, int G1, int DS, bool MASKED>
+template <int VEC, int G1, int DS, int MASKED>
 __global__ __launch_bounds__(kFlatWaves * 64) DLSPM_SDDMM_WAVES_PER_SIMD(DS, kFlatWaves) void sddmm_flat_kernel(int M, int D, int nnz, int chunk,
                                                                       const int* __restrict__ row_offsets,
                                                                       const int* __restrict__ col_indices,
@@ -445,20 +465,27 @@ template <int DS>
 static hipError_t launch_planned(const SddmmArgs& x, const int* plan, int entries, int slots, hipStream_t stream)
 {
     const int *starts = plan, *ends = plan + entries, *rows = plan + 2 * (size_t)entries, *slot_of = plan + 3 * (size_t)entries;
+    const bool by_range = masked_by_range<DS>(x.K, x.D);
     if (slots > 0) {  // a cut plan
         if (x.D == 8 * 4 * DS)
-            hipLaunchKernelGGL((sddmm_pieces_kernel<4, 8, DS, false>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
+            hipLaunchKernelGGL((sddmm_pieces_kernel<4, 8, DS, kExactWidth>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
+                               x.nnz, sddmm_flags(x, x.M), slots, starts, ends, rows, slot_of, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+        else if (by_range)
+            hipLaunchKernelGGL((sddmm_pieces_kernel<4, 8, DS, masked_kind<DS>(true)>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
                                x.nnz, sddmm_flags(x, x.M), slots, starts, ends, rows, slot_of, x.col_indices, x.lhs, x.rhs, sampled_out(x));
         else
-            hipLaunchKernelGGL((sddmm_pieces_kernel<4, 8, DS, true>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
+            hipLaunchKernelGGL((sddmm_pieces_kernel<4, 8, DS, kMaskedBySelect>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
                                x.nnz, sddmm_flags(x, x.M), slots, starts, ends, rows, slot_of, x.col_indices, x.lhs, x.rhs, sampled_out(x));
         return hipGetLastError();
     }
     if (x.D == 8 * 4 * DS)
-        hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, false>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
+        hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, kExactWidth>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
+                           x.nnz, sddmm_flags(x, x.M), starts, ends, rows, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+    else if (by_range)
+        hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, masked_kind<DS>(true)>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
                            x.nnz, sddmm_flags(x, x.M), starts, ends, rows, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     else
-        hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, true>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
+        hipLaunchKernelGGL((sddmm_planned_kernel<4, 8, DS, kMaskedBySelect>), dim3((unsigned)entries), dim3(4 * 64), 0, stream, x.M, x.D,
                            x.nnz, sddmm_flags(x, x.M), starts, ends, rows, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     return hipGetLastError();
 }

@@ -90,7 +90,7 @@ class Tuning(ctypes.Structure):
 
 RULES = {"eight_waves_few_rows": 1, "sixteen_waves_tall_long_rows": 2, "more_waves_few_long_rows": 4, "group_rows": 8,
          "row_aligned_split": 16, "plan_ungroups": 32, "exact_width_kernels": 64, "cut_rows_by_columns": 128,
-         "finer_column_tiles": 256, "row_pieces_few_rows": 512}
+         "finer_column_tiles": 256, "row_pieces_few_rows": 512, "mask_by_range": 1024}
 
 
 class MatrixInfo(ctypes.Structure):

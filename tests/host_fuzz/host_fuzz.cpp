@@ -65,7 +65,7 @@ int main()
             tune.compute_units = units[rng() % 6];
             tune.cut_piece_pct = pcts[rng() % 6];
             tune.cut_longest_pct = pcts[rng() % 6];
-            tune.rules_off = (int)(rng() % 1024);
+            tune.rules_off = (int)(rng() % 2048);
             if (dlspm_set_tuning(&tune) != DLSPM_OK) return 1;
         }
         const int op = (int)(rng() % 3);

@@ -428,9 +428,14 @@ def test_tuning_overrides_go_through_one_call_and_the_environment_is_read_once(d
     assert (sh["G"] * sh["vec"] * sh["V"], sh["col_tiles"]) == (128, 4)
     dl.set_tuning()
     for bad in ({"flat": 2}, {"slices": -2}, {"plan_order": 3}, {"tile_major": 5}, {"split": (-1, 0)}, {"flat_chunk": -64},
-                {"xcd_contiguous": 2}, {"stream_results": 2}, {"stream_results": -2}):
+                {"xcd_contiguous": 2}, {"stream_results": 2}, {"stream_results": -2}, {"rules_off": -1},
+                {"rules_off": 2 * max(dl.RULES.values())}):
         with pytest.raises(dl.DlspmError):
             dl.set_tuning(**bad)
+    dl.set_tuning(rules_off=sum(dl.RULES.values()))   # every rule off at once is a valid setting
+    dl.set_tuning()
+    header = open(os.path.join(ROOT, "include", "dlspm_hip.h")).read()
+    assert sorted(dl.RULES.values()) == sorted(int(v) for v in re.findall(r"#define DLSPM_RULE_\w+\s+(\d+)", header))
     assert dl.get_tuning() == base
     assert dl.lib().dlspm_get_tuning(None) == dl.E_INVALID_ARG
     src = open(os.path.join(ROOT, "dlspm-esimd_amd", "csrc", "api.hip")).read()

@@ -178,11 +178,43 @@ def test_widths_between_the_powers_of_two(torch_cuda, dl, oracle, op, D):
             inf = np.isinf(ref)
             assert inf.any() == poisoned and np.array_equal(np.isinf(got), inf) and np.array_equal(got[inf], ref[inf])
             assert oracle.rel_frobenius(got[~inf], ref[~inf]) <= TOL
+            # the lanes past D are masked by the range of a buffer where D is a multiple of four below 385, by selects
+            # otherwise, under a plan like without: the same bits either way
+            kinds = [dl.sddmm(ro_d, ci_d, dev(torch, lhs), dev(torch, rhs), plan=p) for p in (dl.row_plan(ro_d), dl.cut_plan(ro_d, dl.OP_SDDMM, D))]
+            dl.set_tuning(rules_off=dl.RULES["mask_by_range"])
+            try:
+                kinds += [dl.sddmm(ro_d, ci_d, dev(torch, lhs), dev(torch, rhs), plan=p) for p in (None, dl.row_plan(ro_d), dl.cut_plan(ro_d, dl.OP_SDDMM, D))]
+            finally:
+                dl.set_tuning()
+            for other in kinds:
+                assert np.array_equal(other.cpu().numpy(), got, equal_nan=True)
         elif not poisoned:  # (the fused op would add inf * V rows of both signs: its oracle holds NaN there)
             V = rng.normal(0, 1, (K, D)).astype(np.float32)
             got = dl.fused(ro_d, ci_d, dev(torch, lhs), dev(torch, rhs), dev(torch, V), scale=0.1).cpu().numpy()
             assert oracle.rel_frobenius(got, oracle.fused(ro, ci, lhs, rhs, V, scale=0.1)) <= TOL
     check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
+def test_sddmm_rhs_beyond_the_window_of_the_range_masked_kernels(torch_cuda, dl, oracle):
+    """rhs of 3.4 million rows of 80 floats (1.09 GB) does not fit the 1 GiB buffer whose range check masks the lanes past D: the
+    call takes the kernels that mask by selects, with columns from the whole of rhs."""
+    torch = torch_cuda
+    M, K, D = 96, 3_400_000, 80
+    rng = np.random.default_rng(2718)
+    lens = rng.integers(40, 90, M)
+    ro = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ci = np.concatenate([np.sort(rng.choice(K, n, replace=False)) for n in lens]).astype(np.int32)
+    ci[-1] = K - 1  # the last row of rhs is read too
+    lhs = rng.normal(0, 1, (M, D)).astype(np.float32)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    rhs_d = torch.randn((K, D), dtype=torch.float32, device="cuda", generator=gen)
+    used, where = np.unique(ci, return_inverse=True)
+    rhs_used = rhs_d[torch.from_numpy(used.astype(np.int64)).cuda()].cpu().numpy()
+    ref = oracle.sddmm(ro, where.astype(np.int32), lhs, rhs_used)
+    got = dl.sddmm(dev(torch, ro), dev(torch, ci), dev(torch, lhs), rhs_d).cpu().numpy()
+    assert oracle.rel_frobenius(got, ref) <= TOL
+    del rhs_d
+    torch.cuda.empty_cache()
 
 
 FUSED_CASES = [

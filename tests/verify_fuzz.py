@@ -50,7 +50,7 @@ def random_tuning(rng):
     if rng.random() < 0.5:
         t["stream_results"] = pick([0, 1])
     if rng.random() < 0.5:
-        t["rules_off"] = int(rng.integers(0, 1024))
+        t["rules_off"] = int(rng.integers(0, 2048))
     if rng.random() < 0.3:
         t["cut_piece_pct"], t["cut_longest_pct"] = pick([(100, 150), (75, 100), (50, 75), (25, 30), (200, 150), (10, 10), (1000, 1000)])
     if rng.random() < 0.3:
