@@ -6,7 +6,7 @@ the same launches are timed again.
 
 Cases: the five benchmark configurations; the reference's 12-shape benchmark grid (SPMM/spmm-esimd-allbenchs.cpp:252-255)
 at density 0.1 with N = D = 32 and 128 (Bernoulli patterns); lognormal row lengths (sigma 1) on 2048 ... 16384 rows; layer
-shapes of 64 ... 512 rows as in the reference's dlmc/ tree, three of them under dense rows of 640 ... 3136 floats (SpMM); very long rows in a tall matrix (16384 x 8192 at density 0.2) and in
+widths between the powers of two (80, 160, 320; SDDMM and the fused op); layer shapes of 64 ... 512 rows as in the reference's dlmc/ tree, three of them under dense rows of 640 ... 3136 floats (SpMM); very long rows in a tall matrix (16384 x 8192 at density 0.2) and in
 few rows (256 ... 512 rows of 2048 ... 4096 nonzeros), which is where the rules that add waves per row apply; the three
 patterns of tests/golden/dlmc whose longest row holds four compute units' shares of the nonzeros (cut plans). Every case is launched as a driver would (dlspm_analyze ->
 dlspm_advise -> allocate -> build), inside a HIP graph of 20 launches (median of 7 double replays). With a rule off the
@@ -63,6 +63,13 @@ def cases(dl, quick):
     for (M, K, mean, width) in ((128, 1152, 120.0, 784), (300, 1152, 115.0, 3136), (1000, 2048, 200.0, 640)):
         ro, ci = dl.make_pattern(dl.PATTERN_LOGNORMAL_ROWS, 10, M, K, mean, 0.5)
         out.append((f"wide dense rows {M}x{K} mean {mean:.0f} sigma 0.5 width {width}", dl.OP_SPMM, M, K, width, ro, ci))
+    for (M, K, mean, sigma) in ((2048, 2048, 100.0, 0.0), (2048, 2048, 100.0, 0.8), (8192, 2048, 60.0, 0.0), (512, 2304, 230.0, 0.8)):
+        if sigma > 0:
+            ro, ci = dl.make_pattern(dl.PATTERN_LOGNORMAL_ROWS, 14, M, K, mean, sigma)
+        else:
+            ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 14, M, K, mean / K)
+        for width in (80, 160, 320):
+            out.append((f"between the powers of two {M}x{K} mean {mean:.0f} sigma {sigma} width {width}", "dots", M, K, width, ro, ci))
     if not quick:
         ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 11, 16384, 8192, 0.2)
         for width in (32, 128):
@@ -102,7 +109,10 @@ def main():
         ro_d, ci_d = torch.from_numpy(ro).cuda(), torch.from_numpy(ci).cuda()
         nnz = int(ci.size)
         for o in want:
-            if only_op is not None and ops[o] != only_op:
+            if only_op == "dots":
+                if o == "spmm":
+                    continue
+            elif only_op is not None and ops[o] != only_op:
                 continue
             w = width if width > 0 else {"spmm": 256, "sddmm": 128, "fused": 64}[o]
             if o == "spmm":
