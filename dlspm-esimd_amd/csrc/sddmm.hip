@@ -292,6 +292,19 @@ SddmmShape sddmm_choose(const DeviceInfo& dev, int M, int D, int nnz, bool vec4,
         s.DS = 1;
     }
     choose_split(dev, M, 1, nnz, SplitRule{2, 16, kWave / s.G1, false, 96}, rows, s.W, s.R);
+    // Rows of unknown lengths are grouped only where the launch is many times what the device holds at once: from 128
+    // rows per compute unit on, and from 64 at D <= 32. Below that one row per workgroup, whose four waves take the row's passes
+    // in turn, is the shorter way through the launch even where three of the four waves find nothing to do (rows per
+    // workgroup by the size rule against one, K = 2048, rows of 8 ... 128 nonzeros, D = 32 / 64 / 128 / 256, geometric means:
+    // Bernoulli rows 1.01 / 1.12 / 1.09 / 1.03 of the time, lognormal rows 1.21 / 1.21 / 1.13 / 1.05, up to 1.9; 2048 x 2048
+    // of 8 per row, D = 64: 3.42 -> 2.78 us; 8192 x 2048 of 16, lognormal, D = 64: 7.68 -> 4.76 us. At 32768 rows the groups
+    // win 5-30 % on Bernoulli rows and at D = 32, at 16384 rows at D = 32 only: 16384 x 2048 of 32 per row 6.4 against 8.7 us.)
+    // Rows known to be even keep their groups of four -- one whole row per wave -- where rows and dot products are long (128
+    // nonzeros, 128 floats: 0.91-1.03 of the time of one row per workgroup at 2048 ... 8192 rows), and lose the others
+    // (Bernoulli rows of 8 ... 64 nonzeros on 1024 ... 8192 rows, the hint's groups against none: 1.05-1.31 of the time).
+    const bool many_rows = (long long)M >= 128ll * dev.cus || ((long long)M >= 64ll * dev.cus && D <= 32);
+    const bool even_long_rows = rows == kRowsEven && (long long)nnz >= 128ll * M && D >= 128;
+    if (s.R > 1 && tuning().split_w == 0 && !many_rows && !even_long_rows) s.R = 1;
     return s;
 }
 

@@ -51,7 +51,9 @@ def test_split_rule_and_the_even_rows_hint(dl):
             a = dl.describe_launch(op, 8192, 4096, width, nnz)
             b = dl.describe_launch(op, 8192, 4096, width, nnz, rows_even=True)
             # (the fused op groups long rows by itself where Kmat and V together exceed one L2: 2 x 4096 x 256 floats)
-            assert (a["W"], a["R"]) == ((4, 4) if op == dl.OP_FUSED and width == 256 else (4, 1)) and (b["W"], b["R"]) == (4, 4)
+            # (SDDMM keeps the hint's groups of four only where the dot products are long too: from 128 floats on)
+            assert (a["W"], a["R"]) == ((4, 4) if op == dl.OP_FUSED and width == 256 else (4, 1))
+            assert (b["W"], b["R"]) == ((4, 1) if op == dl.OP_SDDMM and width == 32 else (4, 4))
             same = lambda d: {k: v for k, v in d.items() if k not in ("R", "flat_chunk", "flat_units")}
             assert same(a) == same(b)
             # SDDMM needs no memory for its flat schedule and takes it by the sizes alone -- except for rows known to be even
@@ -60,7 +62,7 @@ def test_split_rule_and_the_even_rows_hint(dl):
             else:
                 assert (a["flat_chunk"], a["flat_units"]) == (b["flat_chunk"], b["flat_units"])
             # too few rows for 512 workgroups of four rows: unchanged
-            assert dl.describe_launch(op, 2048, 4096, width, 2048 * 600, rows_even=True)["R"] == 4
+            assert dl.describe_launch(op, 2048, 4096, width, 2048 * 600, rows_even=True)["R"] == (1 if op == dl.OP_SDDMM and width == 32 else 4)
             assert dl.describe_launch(op, 1536, 4096, width, 1536 * 600, rows_even=True)["R"] == 1
         # short rows are grouped by the size rule already; the hint never makes the groups smaller
         a = dl.describe_launch(op, 65536, 1024, 64, 65536 * 20)
@@ -119,7 +121,16 @@ def test_split_rule_for_small_matrices(dl):
         dl.set_tuning()
     rows_per_workgroup = lambda op, M, avg: dl.describe_launch(op, M, 1024, 64, M * avg)["R"]
     assert [rows_per_workgroup(dl.OP_FUSED, M, 20) for M in (1024, 2048, 3072, 4096, 8192, 16384)] == [1, 2, 4, 4, 8, 16]
-    assert [rows_per_workgroup(dl.OP_SDDMM, M, 20) for M in (1024, 2048, 4096, 8192)] == [2, 4, 8, 16]
+    # SDDMM groups rows of unknown lengths only from 128 rows per compute unit on (from 64 at D <= 32)
+    assert [rows_per_workgroup(dl.OP_SDDMM, M, 20) for M in (1024, 2048, 4096, 8192, 16384, 32767, 32768)] == [1, 1, 1, 1, 1, 1, 16]
+    assert [dl.describe_launch(dl.OP_SDDMM, M, 1024, 32, M * 20)["R"] for M in (8192, 16383, 16384)] == [1, 1, 16]
+    assert dl.describe_launch(dl.OP_SDDMM, 8192, 1024, 64, 8192 * 20, rows_even=True)["R"] == 1      # short even rows: no groups either
+    assert dl.describe_launch(dl.OP_SDDMM, 8192, 1024, 128, 8192 * 128, rows_even=True)["R"] == 4    # long rows, long dot products
+    dl.set_tuning(rules_off=dl.RULES["group_rows"])
+    try:
+        assert rows_per_workgroup(dl.OP_SDDMM, 32768, 20) == 1
+    finally:
+        dl.set_tuning()
     assert [rows_per_workgroup(dl.OP_SPMM, M, 20) for M in (1024, 2048, 4096, 8192)] == [1, 1, 2, 4]
     M, K, nnz = 2048, 512, 2048 * 10
     assert dl.row_plan_advice(dl.OP_FUSED, M, K, 64, nnz, 23) == 1  # short rows: any unevenness
@@ -371,9 +382,13 @@ def test_row_plan_host_side(dl):
         assert not dl.row_plan_advice(op, 2048, 2048, 64, 2048 * 100, 120)     # even rows
         assert not dl.row_plan_advice(op, 2048, 2048, 16, 2048 * 100, 500)     # D <= 16
         assert not dl.row_plan_advice(op, 2048, 2048, 1024, 2048 * 100, 500)   # D > 512
-        assert not dl.row_plan_advice(op, 8192, 2048, 64, 8192 * 20, 200)      # short rows
-        assert dl.describe_launch(op, 16384, 2048, 128, 16384 * 60)["R"] == 8
-        assert not dl.row_plan_advice(op, 16384, 2048, 128, 16384 * 60, 600)   # tall mask, grouped rows: the grouping wins
+        # short rows in a tall mask: the fused op groups them, and its groups win; SDDMM runs one row per workgroup up
+        # to 128 rows per compute unit, and a plan over such rows only has to beat their given order
+        assert bool(dl.row_plan_advice(op, 8192, 2048, 64, 8192 * 20, 200)) == (op == dl.OP_SDDMM)
+        assert dl.describe_launch(op, 16384, 2048, 128, 16384 * 60)["R"] == (1 if op == dl.OP_SDDMM else 8)
+        assert bool(dl.row_plan_advice(op, 16384, 2048, 128, 16384 * 60, 600)) == (op == dl.OP_SDDMM)
+        assert dl.describe_launch(op, 32768, 2048, 128, 32768 * 60)["R"] == 8
+        assert not dl.row_plan_advice(op, 32768, 2048, 128, 32768 * 60, 600)   # grouped rows: the grouping wins
         assert dl.row_plan_advice(op, 16384, 4096, 128, 16384 * 400, 4000)     # ... rows the rule runs one per workgroup anyway
     assert not dl.row_plan_advice(dl.OP_FUSED, 8192, 8192, 128, 8192 * 800, 8000)   # Kmat and V of 8 MiB: the slices first
     assert not dl.row_plan_advice(7, 2048, 2048, 64, 2048 * 100, 500)

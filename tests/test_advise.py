@@ -43,8 +43,8 @@ def test_advise_branches(dl):
     for op, D in ((dl.OP_SDDMM, 128), (dl.OP_FUSED, 64)):
         cp = A(op, D, info(dl, 8192, 2048, 8192 * 60, 1500))
         assert (cp.build, cp.bytes, cp.hints) == (dl.BUILD_ROW_PLAN, dl.row_plan_bytes(8192), dl.HINT_ROW_PLAN | dl.HINT_ROWS_SKEWED)
-        cp = A(op, D, info(dl, 8192, 2048, 8192 * 60, 400))   # uneven, but not that uneven: grouped rows, no plan
-        assert cp.build == dl.BUILD_NOTHING
+        cp = A(op, D, info(dl, 8192, 2048, 8192 * 60, 400))   # uneven, but not that uneven: the fused op's grouped rows win
+        assert cp.build == (dl.BUILD_ROW_PLAN if op == dl.OP_SDDMM else dl.BUILD_NOTHING)  # (SDDMM does not group them)
     # even rows: the hint, no memory
     cp = A(dl.OP_SPMM, 392, info(dl, 2048, 512, 2048 * 102, 102))
     assert (cp.build, cp.bytes, cp.hints) == (dl.BUILD_NOTHING, 0, dl.HINT_ROWS_EVEN)
