@@ -188,10 +188,16 @@ FlatPlan flat_plan(const DeviceInfo& dev, int M, int nnz, int width, int G)
     return p;
 }
 
-static FlatPlan sddmm_flat_plan(const DeviceInfo& dev, int M, int nnz, int D)
+// Not by itself where rhs exceeds one L2 under rows of a thousand nonzeros and more: the four waves of a row-block workgroup,
+// and the workgroups of neighbouring rows, go through such rows' columns together and find each other's rows of rhs in
+// the L2, where the flat schedule's waves each start somewhere else (Bernoulli rows, flat / row-block: 8192 x 8192 of 1229
+// per row, D = 256 711 / 537 us, of 2458 per row 1388 / 789 us, D = 384 2704 / 1681 us; 4096 x 16384 of 3277, D = 192 811 /
+// 481 us; lognormal rows lose 0-7 % by it; rows of 819: 1.01-1.03 either way; rhs of exactly one L2: 1.02-1.11).
+static FlatPlan sddmm_flat_plan(const DeviceInfo& dev, int M, int K, int nnz, int D)
 {
     const int force = tuning().flat;
     if (force < 0 && (nnz < kFlatMinNnzSddmm || (long long)nnz < (long long)kFlatMinRowSddmm * M)) return FlatPlan{0, 0, 0};
+    if (force < 0 && (long long)K * D * (long long)sizeof(float) > dev.l2_bytes && (long long)nnz >= 1024ll * M) return FlatPlan{0, 0, 0};
     return flat_plan(dev, M, nnz, D, kWave);
 }
 
@@ -769,7 +775,7 @@ int sddmm_csr_f32(int M, int K, int D, int nnz, const int* row_offsets, const in
     }
     // (rows known to be even have nothing to gain from the flat schedule, which costs them 4 ... 12 % today: the reference's
     // grid at density 0.1, 12288 ... 32768 rows of 410 ... 819 nonzeros, D = 32 and 128)
-    const FlatPlan plan = ws.banded || ws.rows_even ? FlatPlan{0, 0, 0} : sddmm_flat_plan(dev, M, nnz, D);
+    const FlatPlan plan = ws.banded || ws.rows_even ? FlatPlan{0, 0, 0} : sddmm_flat_plan(dev, M, K, nnz, D);
     SddmmShape plain = shape;
     if (plan.chunk == 0) sddmm_few_rows_pieces(dev, plain, M, nnz);
     const hipError_t e = plan.chunk > 0 ? sddmm_flat_launch(args, shape, plan.chunk, st) : sddmm_launch(args, plain, st);
@@ -923,7 +929,7 @@ int dlspm_describe_launch_rows(int op, int M, int K, int N_or_D, int nnz, int pa
         shape[8] = fp.chunk; shape[9] = fp.units;
     } else if (op == DLSPM_OP_SDDMM) {
         SddmmShape s = sddmm_choose(dev, M, n, nnz, vec4, rows);
-        const FlatPlan fp = even ? FlatPlan{0, 0, 0} : sddmm_flat_plan(dev, M, nnz, n);  // as sddmm_csr_f32 decides
+        const FlatPlan fp = even ? FlatPlan{0, 0, 0} : sddmm_flat_plan(dev, M, K, nnz, n);  // as sddmm_csr_f32 decides
         if (!memory && fp.chunk == 0) sddmm_few_rows_pieces(dev, s, M, nnz);
         // ([7]: the workgroups that share a row -- SDDMM has no column tiles)
         shape[0] = s.vec; shape[3] = s.G1; shape[4] = s.DS; shape[5] = s.W; shape[6] = s.R; shape[7] = 1 << s.pieces_lg;

@@ -61,6 +61,10 @@ def test_split_rule_and_the_even_rows_hint(dl):
                 assert a["flat_chunk"] > 0 and b["flat_chunk"] == 0
             else:
                 assert (a["flat_chunk"], a["flat_units"]) == (b["flat_chunk"], b["flat_units"])
+            # ... nor where rhs exceeds one L2 under rows of a thousand nonzeros and more
+            if op == dl.OP_SDDMM:
+                flat = lambda K, D, per_row: dl.describe_launch(op, 8192, K, D, 8192 * per_row)["flat_chunk"] > 0
+                assert not flat(8192, 256, 2458) and not flat(16384, 128, 1024) and flat(8192, 128, 2458) and flat(8192, 256, 1023)
             # too few rows for 512 workgroups of four rows: unchanged
             assert dl.describe_launch(op, 2048, 4096, width, 2048 * 600, rows_even=True)["R"] == (1 if op == dl.OP_SDDMM and width == 32 else 4)
             assert dl.describe_launch(op, 1536, 4096, width, 1536 * 600, rows_even=True)["R"] == 1
