@@ -232,8 +232,8 @@ static int sddmm_flags(const SddmmArgs& x, long long entries)
 // Whether the kernels that mask by the range of a buffer apply (sddmm_rounds_load): D a multiple of four, up to twelve
 // accesses per lane (D <= 384), rhs within the window. Against the kernels that mask by selects (Bernoulli / lognormal rows, 20
 // shapes of 128 ... 16384 rows, geometric means): D = 80 0.96 / 0.92 of the time, D = 100 0.89 / 0.80, D = 160 0.95 / 0.91, D = 224
-// 0.94 / 0.90, D = 320 0.90 / 0.88; with sixteen accesses (D = 448) 0.75 ... 1.5, which stay with the selects. The kernels of
-// the column-sliced and the flat schedule, and the fused op's, mask by selects at every width.
+// 0.94 / 0.90, D = 320 0.90 / 0.88; with sixteen accesses (D = 448) 0.75 ... 1.5, which stay with the selects. The fused op's
+// kernels mask by selects at every width.
 template <int DS> static bool masked_by_range(int K, int D)
 {
     return DS >= 1 && DS <= 12 && D % 4 == 0 && K < (1 << 24) &&
@@ -387,12 +387,19 @@ static hipError_t launch_flat(const SddmmArgs& x, int chunk, hipStream_t stream)
     const unsigned blocks = (unsigned)((units + kFlatWaves - 1) / kFlatWaves);
     if constexpr (DS > 0) {
         if (x.D == G1 * VEC * DS && rule_on(kRuleExactWidthKernels)) {
-            hipLaunchKernelGGL((sddmm_flat_kernel<VEC, G1, DS, false>), dim3(blocks), dim3(kFlatWaves * 64), 0, stream, x.M,
+            hipLaunchKernelGGL((sddmm_flat_kernel<VEC, G1, DS, kExactWidth>), dim3(blocks), dim3(kFlatWaves * 64), 0, stream, x.M,
                                x.D, x.nnz, chunk, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
             return hipGetLastError();
         }
     }
-    hipLaunchKernelGGL((sddmm_flat_kernel<VEC, G1, DS, true>), dim3(blocks), dim3(kFlatWaves * 64), 0, stream, x.M, x.D,
+    if constexpr (VEC == 4 && G1 == 8 && DS >= 1 && DS <= 12) {
+        if (masked_by_range<DS>(x.K, x.D)) {
+            hipLaunchKernelGGL((sddmm_flat_kernel<VEC, G1, DS, kMaskedByRange>), dim3(blocks), dim3(kFlatWaves * 64), 0, stream, x.M,
+                               x.D, x.nnz, chunk, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((sddmm_flat_kernel<VEC, G1, DS, kMaskedBySelect>), dim3(blocks), dim3(kFlatWaves * 64), 0, stream, x.M, x.D,
                        x.nnz, chunk, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     return hipGetLastError();
 }
@@ -415,10 +422,13 @@ static hipError_t launch_sliced_r(const SddmmArgs& x, const SlicePlan& plan, con
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     if (x.D == G1 * VEC * DS)
-        hipLaunchKernelGGL((sddmm_sliced_kernel<VEC, G1, DS, false, R>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream,
+        hipLaunchKernelGGL((sddmm_sliced_kernel<VEC, G1, DS, kExactWidth, R>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream,
+                           x.M, x.D, (int)slice_blocks, bounds, x.col_indices, x.lhs, x.rhs, sampled_out(x));
+    else if (masked_by_range<DS>(x.K, x.D))
+        hipLaunchKernelGGL((sddmm_sliced_kernel<VEC, G1, DS, masked_kind<DS>(true), R>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream,
                            x.M, x.D, (int)slice_blocks, bounds, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     else
-        hipLaunchKernelGGL((sddmm_sliced_kernel<VEC, G1, DS, true, R>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream,
+        hipLaunchKernelGGL((sddmm_sliced_kernel<VEC, G1, DS, kMaskedBySelect, R>), dim3((unsigned)blocks), dim3(4 * 64), 0, stream,
                            x.M, x.D, (int)slice_blocks, bounds, x.col_indices, x.lhs, x.rhs, sampled_out(x));
     return hipGetLastError();
 }

@@ -195,6 +195,34 @@ def test_widths_between_the_powers_of_two(torch_cuda, dl, oracle, op, D):
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
+@pytest.mark.parametrize("schedule,M,K,D,density", [("flat", 4096, 8192, 80, 0.07), ("sliced", 2048, 16384, 160, 0.03)])
+def test_sddmm_flat_and_sliced_schedules_at_widths_between_the_powers_of_two(torch_cuda, dl, oracle, schedule, M, K, D, density):
+    """The kernels of SDDMM's flat schedule (taken by the sizes alone) and of its column-sliced schedule (with workspace)
+    mask the lanes past D by the range of a buffer too: the oracle's values, and the bits of the kernels that mask by selects."""
+    torch = torch_cuda
+    ro, ci = dl.make_pattern(dl.PATTERN_BERNOULLI, 201, M, K, density)
+    nnz = ci.size
+    lhs = dl.fill("normal", 202, (M, D), 0.0, 1.0)
+    rhs = dl.fill("normal", 203, (K, D), 0.0, 1.0)
+    ro_d, ci_d, lhs_d, rhs_d = (dev(torch, x) for x in (ro, ci, lhs, rhs))
+    if schedule == "flat":
+        assert dl.describe_launch(dl.OP_SDDMM, M, K, D, nnz)["flat_chunk"] > 0
+        run = lambda: dl.sddmm(ro_d, ci_d, lhs_d, rhs_d)
+    else:
+        assert dl.describe_slices(dl.OP_SDDMM, M, K, D, nnz)[0] > 1
+        ws = torch.empty(dl.workspace_bytes(dl.OP_SDDMM, M, K, D, nnz), dtype=torch.uint8, device="cuda")
+        run = lambda: dl.sddmm(ro_d, ci_d, lhs_d, rhs_d, workspace=ws)
+    got = run()
+    assert oracle.rel_frobenius(got.cpu().numpy(), oracle.sddmm(ro, ci, lhs, rhs, omp=True)) <= TOL
+    dl.set_tuning(rules_off=dl.RULES["mask_by_range"])
+    try:
+        by_selects = run()
+    finally:
+        dl.set_tuning()
+    assert torch.equal(got, by_selects)
+    check_csr_untouched(ro_d, ci_d, ro, ci)
+
+
 def test_sddmm_rhs_beyond_the_window_of_the_range_masked_kernels(torch_cuda, dl, oracle):
     """rhs of 3.4 million rows of 80 floats (1.09 GB) does not fit the 1 GiB buffer whose range check masks the lanes past D: the
     call takes the kernels that mask by selects, with columns from the whole of rhs."""
