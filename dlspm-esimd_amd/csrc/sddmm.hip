@@ -229,18 +229,19 @@ static int sddmm_flags(const SddmmArgs& x, long long entries)
     return launch_flags(x.xcd_contiguous) | (entries >= 2ll * x.cus ? kFlagFullPasses : 0);
 }
 
-// Whether the kernels that mask by the range of a buffer apply (sddmm_rounds_load): D a multiple of four, up to twelve
-// accesses per lane (D <= 384), rhs within the window. Against the kernels that mask by selects (Bernoulli / lognormal rows, 20
-// shapes of 128 ... 16384 rows, geometric means): D = 80 0.96 / 0.92 of the time, D = 100 0.89 / 0.80, D = 160 0.95 / 0.91, D = 224
-// 0.94 / 0.90, D = 320 0.90 / 0.88; with sixteen accesses (D = 448) 0.75 ... 1.5, which stay with the selects. The fused op's
-// kernels mask by selects at every width.
+// Whether the kernels that mask by the range of a buffer apply (sddmm_rounds_load): D a multiple of four, rhs within the
+// window. Against the kernels that mask by selects (Bernoulli / lognormal rows, 20 shapes of 128 ... 16384 rows, geometric
+// means): D = 80 0.96 / 0.92 of the time, D = 100 0.89 / 0.80, D = 160 0.95 / 0.91, D = 224 0.94 / 0.90, D = 320 0.90 / 0.88; with
+// sixteen accesses (D = 400 ... 496, twelve shapes, plain calls and planned ones) 0.78-0.82 and 0.75-0.77, 0.58 ... 1.13: the
+// select kernel needs 172 registers there, two waves per SIMD, the range kernel 122. The fused op's kernels mask by
+// selects at every width.
 template <int DS> static bool masked_by_range(int K, int D)
 {
-    return DS >= 1 && DS <= 12 && D % 4 == 0 && K < (1 << 24) &&
+    return DS >= 1 && DS <= 16 && D % 4 == 0 && K < (1 << 24) &&
            (long long)K * D * (long long)sizeof(float) <= (long long)kRangeWindowBytes && rule_on(kRuleMaskByRange);
 }
-// (the kind to instantiate: no range kernels where masked_by_range<DS> never says so)
-template <int DS> constexpr int masked_kind(bool by_range) { return by_range && DS >= 1 && DS <= 12 ? kMaskedByRange : kMaskedBySelect; }
+// (the kind to instantiate: no range kernels for the run-time loop of D > 512)
+template <int DS> constexpr int masked_kind(bool by_range) { return by_range && DS >= 1 && DS <= 16 ? kMaskedByRange : kMaskedBySelect; }
 
 template <int VEC, int G1, int DS, int W, int R>
 static hipError_t launch_one(const SddmmArgs& x, int pieces_lg, hipStream_t stream)
@@ -257,7 +258,7 @@ static hipError_t launch_one(const SddmmArgs& x, int pieces_lg, hipStream_t stre
             return hipGetLastError();
         }
     }
-    if constexpr (VEC == 4 && G1 == 8 && DS >= 1 && DS <= 12) {
+    if constexpr (VEC == 4 && G1 == 8 && DS >= 1 && DS <= 16) {
         if (masked_by_range<DS>(x.K, x.D)) {
             hipLaunchKernelGGL((sddmm_kernel<VEC, G1, DS, kMaskedByRange, W, R>), dim3(blocks), dim3(W * 64), 0, stream, x.M, x.D,
                                flags, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));
@@ -392,7 +393,7 @@ static hipError_t launch_flat(const SddmmArgs& x, int chunk, hipStream_t stream)
             return hipGetLastError();
         }
     }
-    if constexpr (VEC == 4 && G1 == 8 && DS >= 1 && DS <= 12) {
+    if constexpr (VEC == 4 && G1 == 8 && DS >= 1 && DS <= 16) {
         if (masked_by_range<DS>(x.K, x.D)) {
             hipLaunchKernelGGL((sddmm_flat_kernel<VEC, G1, DS, kMaskedByRange>), dim3(blocks), dim3(kFlatWaves * 64), 0, stream, x.M,
                                x.D, x.nnz, chunk, x.row_offsets, x.col_indices, x.lhs, x.rhs, sampled_out(x));

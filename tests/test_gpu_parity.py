@@ -178,8 +178,8 @@ def test_widths_between_the_powers_of_two(torch_cuda, dl, oracle, op, D):
             inf = np.isinf(ref)
             assert inf.any() == poisoned and np.array_equal(np.isinf(got), inf) and np.array_equal(got[inf], ref[inf])
             assert oracle.rel_frobenius(got[~inf], ref[~inf]) <= TOL
-            # the lanes past D are masked by the range of a buffer where D is a multiple of four below 385, by selects
-            # otherwise, under a plan like without: the same bits either way
+            # the lanes past D are masked by the range of a buffer where D is a multiple of four, by selects otherwise,
+            # under a plan like without: the same bits either way
             kinds = [dl.sddmm(ro_d, ci_d, dev(torch, lhs), dev(torch, rhs), plan=p) for p in (dl.row_plan(ro_d), dl.cut_plan(ro_d, dl.OP_SDDMM, D))]
             dl.set_tuning(rules_off=dl.RULES["mask_by_range"])
             try:
