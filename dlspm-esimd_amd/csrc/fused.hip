@@ -145,6 +145,17 @@ __global__ __launch_bounds__(4 * 64) void fused_pieces_kernel(int M, int D, int 
 
 // ---- host side --------------------------------------------------------------------------------------
 
+// Whether stage 1 masks the lanes past D by the range check of a buffer load (sddmm_rounds_load), in the row-block, planned and
+// cut-plan kernels of twelve stage-1 accesses (D = 257 ... 383, a multiple of four, Kmat within the window): 0.92-0.93 of the
+// time of the kernels that mask by selects over nine shapes (0.86 ... 0.97), the same bits. With sixteen accesses 0.99-1.00
+// (0.73 ... 1.14), and below 257 the masks are a few per cent of a kernel that stage 2 dominates: those keep the selects.
+template <int DS> static bool stage1_masked_by_range(int K, int D)
+{
+    return DS == 12 && D % 4 == 0 && K < (1 << 24) && (long long)K * D * (long long)sizeof(float) <= (long long)kRangeWindowBytes &&
+           rule_on(kRuleMaskByRange);
+}
+template <int DS> constexpr int stage1_masked_kind(bool by_range) { return by_range && DS == 12 ? kMaskedByRange : kMaskedBySelect; }
+
 template <int VEC, int G1, int DS, int G, int V2, int W, int R>
 static hipError_t launch_one(const FusedArgs& x, hipStream_t stream)
 {
@@ -161,7 +172,15 @@ static hipError_t launch_one(const FusedArgs& x, hipStream_t stream)
             return hipGetLastError();
         }
     }
-    hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, true, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream,
+    if constexpr (VEC == 4 && G1 == 8 && DS == 12) {
+        if (stage1_masked_by_range<DS>(x.K, x.D)) {
+            hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, kMaskedByRange, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream,
+                               x.M, x.D, col_tiles, launch_flags(x.xcd_contiguous), x.scale, x.row_offsets, x.col_indices, x.Q, x.Kmat,
+                               x.V, x.O);
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((fused_kernel<VEC, G1, DS, kMaskedBySelect, G, V2, W, R>), dim3((unsigned)blocks), dim3(W * 64), 0, stream,
                        x.M, x.D, col_tiles, launch_flags(x.xcd_contiguous), x.scale, x.row_offsets, x.col_indices, x.Q, x.Kmat, x.V,
                        x.O);
     return hipGetLastError();
@@ -405,8 +424,11 @@ static hipError_t launch_planned(const FusedArgs& x, const int* plan, hipStream_
     if (x.D == 8 * 4 * DS)
         hipLaunchKernelGGL((fused_planned_kernel<4, 8, DS, false, G, V2>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M,
                            x.D, x.nnz, launch_flags(0), x.scale, starts, ends, rows, x.col_indices, x.Q, x.Kmat, x.V, x.O);
+    else if (stage1_masked_by_range<DS>(x.K, x.D))
+        hipLaunchKernelGGL((fused_planned_kernel<4, 8, DS, stage1_masked_kind<DS>(true), G, V2>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M,
+                           x.D, x.nnz, launch_flags(0), x.scale, starts, ends, rows, x.col_indices, x.Q, x.Kmat, x.V, x.O);
     else
-        hipLaunchKernelGGL((fused_planned_kernel<4, 8, DS, true, G, V2>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M,
+        hipLaunchKernelGGL((fused_planned_kernel<4, 8, DS, kMaskedBySelect, G, V2>), dim3((unsigned)x.M), dim3(4 * 64), 0, stream, x.M,
                            x.D, x.nnz, launch_flags(0), x.scale, starts, ends, rows, x.col_indices, x.Q, x.Kmat, x.V, x.O);
     return hipGetLastError();
 }
@@ -422,8 +444,12 @@ static hipError_t launch_pieces(const FusedArgs& x, const CutPlan& cp, void* pla
         hipLaunchKernelGGL((fused_pieces_kernel<4, 8, DS, false, G, V2>), dim3((unsigned)cp.entries), dim3(4 * 64), 0, stream,
                            x.M, x.D, x.nnz, launch_flags(0), cp.slots, x.scale, starts, ends, rows, slot_of, x.col_indices, x.Q,
                            x.Kmat, x.V, x.O, pieces);
+    else if (stage1_masked_by_range<DS>(x.K, x.D))
+        hipLaunchKernelGGL((fused_pieces_kernel<4, 8, DS, stage1_masked_kind<DS>(true), G, V2>), dim3((unsigned)cp.entries), dim3(4 * 64), 0, stream,
+                           x.M, x.D, x.nnz, launch_flags(0), cp.slots, x.scale, starts, ends, rows, slot_of, x.col_indices, x.Q,
+                           x.Kmat, x.V, x.O, pieces);
     else
-        hipLaunchKernelGGL((fused_pieces_kernel<4, 8, DS, true, G, V2>), dim3((unsigned)cp.entries), dim3(4 * 64), 0, stream,
+        hipLaunchKernelGGL((fused_pieces_kernel<4, 8, DS, kMaskedBySelect, G, V2>), dim3((unsigned)cp.entries), dim3(4 * 64), 0, stream,
                            x.M, x.D, x.nnz, launch_flags(0), cp.slots, x.scale, starts, ends, rows, slot_of, x.col_indices, x.Q,
                            x.Kmat, x.V, x.O, pieces);
     const hipError_t e = hipGetLastError();

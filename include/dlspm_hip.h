@@ -403,7 +403,8 @@ typedef struct dlspm_tuning {
                                                    /* one and a half times their number                                      */
 #define DLSPM_RULE_MASK_BY_RANGE             1024  /* SDDMM, D a multiple of four up to 512 that no kernel is built for exactly */
                                                    /* (not 32, 64, 96, 128, 192, 256, 384, 512): rhs read as a buffer of 1 GiB    */
-                                                   /* whose range check zeroes the lanes past D, where rhs fits (else: by selects) */
+                                                   /* whose range check zeroes the lanes past D, where rhs fits (else: by selects); */
+                                                   /* the fused op's first stage likewise at D = 260 ... 380                      */
 void dlspm_tuning_default(dlspm_tuning* t);   /* fills *t with "follow the rules" */
 int dlspm_set_tuning(const dlspm_tuning* t);  /* DLSPM_OK or DLSPM_E_INVALID_ARG (a field out of range) */
 int dlspm_get_tuning(dlspm_tuning* t);        /* what the calling thread's launches currently use */

@@ -190,8 +190,19 @@ def test_widths_between_the_powers_of_two(torch_cuda, dl, oracle, op, D):
                 assert np.array_equal(other.cpu().numpy(), got, equal_nan=True)
         elif not poisoned:  # (the fused op would add inf * V rows of both signs: its oracle holds NaN there)
             V = rng.normal(0, 1, (K, D)).astype(np.float32)
-            got = dl.fused(ro_d, ci_d, dev(torch, lhs), dev(torch, rhs), dev(torch, V), scale=0.1).cpu().numpy()
-            assert oracle.rel_frobenius(got, oracle.fused(ro, ci, lhs, rhs, V, scale=0.1)) <= TOL
+            ops = (dev(torch, lhs), dev(torch, rhs), dev(torch, V))
+            got = dl.fused(ro_d, ci_d, *ops, scale=0.1)
+            assert oracle.rel_frobenius(got.cpu().numpy(), oracle.fused(ro, ci, lhs, rhs, V, scale=0.1)) <= TOL
+            # (D = 257 ... 383: the first stage masks by range too; the bits of the kernels that mask by selects, planned or not)
+            plans = (None, dl.row_plan(ro_d), dl.cut_plan(ro_d, dl.OP_FUSED, D))
+            with_rule = [got] + [dl.fused(ro_d, ci_d, *ops, scale=0.1, plan=p) for p in plans[1:]]
+            dl.set_tuning(rules_off=dl.RULES["mask_by_range"])
+            try:
+                without = [dl.fused(ro_d, ci_d, *ops, scale=0.1, plan=p) for p in plans]
+            finally:
+                dl.set_tuning()
+            for a, b in zip(with_rule, without):
+                assert torch.equal(a, b)
     check_csr_untouched(ro_d, ci_d, ro, ci)
 
 
